@@ -1,0 +1,781 @@
+// tf_oracle.cpp — CPU restatement of the reference's FP32 validation path.
+//
+// TEST INFRASTRUCTURE ONLY: see tf_oracle.h.  The product never links this file.
+// Build with -ffp-contract=off so that a*b+c is two roundings wherever the
+// reference writes two operations; fused operations are spelled fmaf().
+#include "tf_oracle.h"
+
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <limits>
+#include <unordered_set>
+#include <vector>
+
+namespace {
+
+inline uint32_t f32_bits(float f) { uint32_t u; std::memcpy(&u, &f, 4); return u; }
+inline float bits_f32(uint32_t u) { float f; std::memcpy(&f, &u, 4); return f; }
+
+inline uint16_t load_u16(const uint8_t *p) { return (uint16_t)(p[0] | (p[1] << 8)); }
+
+constexpr int G = TFO_GROUP_SIZE;
+constexpr float kGeluCoeff = 0.7978845608028654f;  // sqrt(2/pi)
+constexpr float kGeluCubic = 0.044715f;
+
+inline float gelu_tanh_ref(float xv) {                 // VS/Reference/MoE/Moe.swift:25-27
+    const float inner = kGeluCoeff * (xv + kGeluCubic * xv * xv * xv);
+    return 0.5f * xv * (1.0f + std::tanh(inner));
+}
+
+inline float gelu_tanh_kernel(float x) {               // M/MoE/moe.metal:53-60
+    const float x3 = x * x * x;
+    float inner = kGeluCoeff * (x + kGeluCubic * x3);
+    inner = std::min(std::max(inner, -20.0f), 20.0f);
+    return 0.5f * x * (1.0f + std::tanh(inner));
+}
+
+inline void dequant4_row(const uint8_t *packed, const uint16_t *scales, const uint16_t *biases, int n, float *out) {
+    const int groups = n / G;
+    for (int g = 0; g < groups; ++g) {
+        const float scale = tfo_bf16_to_float(scales[g]);
+        const float bias = tfo_bf16_to_float(biases[g]);
+        for (int k = 0; k < G; ++k) {
+            const uint8_t b = packed[g * (G / 2) + (k / 2)];
+            const int nibble = (k & 1) == 0 ? (b & 0x0F) : (b >> 4);
+            out[g * G + k] = (float)nibble * scale + bias;
+        }
+    }
+}
+
+inline void dequant8_row(const uint8_t *packed, const uint16_t *scales, const uint16_t *biases, int n, float *out) {
+    const int groups = n / G;
+    for (int g = 0; g < groups; ++g) {
+        const float scale = tfo_bf16_to_float(scales[g]);
+        const float bias = tfo_bf16_to_float(biases[g]);
+        for (int k = 0; k < G; ++k) out[g * G + k] = (float)packed[g * G + k] * scale + bias;
+    }
+}
+
+inline float dot_f32(const float *a, const float *b, int n) {   // stands in for vDSP_dotpr
+    float acc = 0.0f;
+    for (int i = 0; i < n; ++i) acc += a[i] * b[i];
+    return acc;
+}
+
+// One row of an int4 matrix living at byte offsets inside a blob (scales/biases may be 2-aligned only).
+inline float blob_row_dot(const uint8_t *blob, uint32_t w_off, uint32_t s_off, uint32_t b_off, int row, int n,
+                          const float *x, float *scratch) {
+    const int groups = n / G;
+    const uint8_t *w = blob + w_off + (int64_t)row * (n / 2);
+    const uint8_t *s = blob + s_off + (int64_t)row * groups * 2;
+    const uint8_t *b = blob + b_off + (int64_t)row * groups * 2;
+    for (int g = 0; g < groups; ++g) {
+        const float scale = tfo_bf16_to_float(load_u16(s + 2 * g));
+        const float bias = tfo_bf16_to_float(load_u16(b + 2 * g));
+        for (int k = 0; k < G; ++k) {
+            const uint8_t by = w[g * (G / 2) + (k / 2)];
+            const int nibble = (k & 1) == 0 ? (by & 0x0F) : (by >> 4);
+            scratch[g * G + k] = (float)nibble * scale + bias;
+        }
+    }
+    return dot_f32(scratch, x, n);
+}
+
+// The per-lane arithmetic shared by the reference's one-SIMD-per-row int4 kernels
+// (M/Quant/dequant_int4.metal:124-171 == M/MoE/moe.metal:203-247 == M/Sampling/logit.metal:646-690).
+// S/B given as byte pointers because blob-resident rows are only 2-byte aligned.
+float kernel_row_int4(const uint8_t *w_row, const uint8_t *s_row, const uint8_t *b_row, const uint16_t *x_f16, int n) {
+    const int groups = n / G;
+    const int full_blocks = groups / 4;
+    float lane_acc[32];
+    for (int lane = 0; lane < 32; ++lane) {
+        float acc = 0.0f;
+        for (int blk = 0; blk < full_blocks; ++blk) {
+            const int byte_base = blk * 128 + lane * 4;
+            const int g = blk * 4 + (lane >> 3);
+            const float s = tfo_bf16_to_float(load_u16(s_row + 2 * g));
+            const float b = tfo_bf16_to_float(load_u16(b_row + 2 * g));
+            const int elem = byte_base * 2;
+            float e[8];
+            for (int i = 0; i < 8; ++i) e[i] = tfo_f16_to_float(x_f16[elem + i]);
+            float dot = 0.0f;
+            for (int i = 0; i < 4; ++i) {
+                const uint8_t by = w_row[byte_base + i];
+                dot = fmaf((float)(by & 0x0F), e[2 * i], dot);
+                dot = fmaf((float)(by >> 4), e[2 * i + 1], dot);
+            }
+            const float sum = e[0] + e[1] + e[2] + e[3] + e[4] + e[5] + e[6] + e[7];
+            acc = fmaf(s, dot, acc);
+            acc = fmaf(b, sum, acc);
+        }
+        for (int g = full_blocks * 4; g < groups; ++g) {
+            const float s = tfo_bf16_to_float(load_u16(s_row + 2 * g));
+            const float b = tfo_bf16_to_float(load_u16(b_row + 2 * g));
+            const uint8_t by = w_row[g * (G / 2) + lane];
+            const float x0 = tfo_f16_to_float(x_f16[g * G + lane * 2]);
+            const float x1 = tfo_f16_to_float(x_f16[g * G + lane * 2 + 1]);
+            float dot = fmaf((float)(by & 0x0F), x0, 0.0f);
+            dot = fmaf((float)(by >> 4), x1, dot);
+            const float sum = x0 + x1;
+            acc = fmaf(s, dot, acc);
+            acc = fmaf(b, sum, acc);
+        }
+        lane_acc[lane] = acc;
+    }
+    float total = 0.0f;   // simd_sum: order unspecified by the reference; lanes taken in order here
+    for (int lane = 0; lane < 32; ++lane) total += lane_acc[lane];
+    return total;
+}
+
+}  // namespace
+
+extern "C" {
+
+// ---------------------------------------------------------------- codecs
+uint16_t tfo_bf16_bits(float x) {
+    const uint32_t bits = f32_bits(x);
+    const uint32_t lsb = (bits >> 16) & 1u;
+    const uint32_t rounding_bias = 0x7FFFu + lsb;
+    const uint32_t rounded = (bits + rounding_bias) >> 16;   // wraps like Swift's &+
+    return (uint16_t)rounded;
+}
+
+float tfo_bf16_to_float(uint16_t bits) { return bits_f32((uint32_t)bits << 16); }
+
+uint16_t tfo_f16_bits(float f) {
+    const uint32_t x = f32_bits(f);
+    const uint32_t sign = (x >> 16) & 0x8000u;
+    const uint32_t e = (x >> 23) & 0xFFu;
+    uint32_t m = x & 0x7FFFFFu;
+    if (e == 0xFFu) {
+        if (m == 0) return (uint16_t)(sign | 0x7C00u);
+        return (uint16_t)(sign | 0x7C00u | 0x0200u | (m >> 13));
+    }
+    const int32_t he = (int32_t)e - 112;
+    if (he >= 31) return (uint16_t)(sign | 0x7C00u);
+    if (he <= 0) {
+        if (he < -10) return (uint16_t)sign;
+        m |= 0x800000u;
+        const int shift = 14 - he;
+        uint32_t hm = m >> shift;
+        const uint32_t rem = m & ((1u << shift) - 1u);
+        const uint32_t halfway = 1u << (shift - 1);
+        if (rem > halfway || (rem == halfway && (hm & 1u))) hm++;
+        return (uint16_t)(sign | hm);
+    }
+    uint32_t h = sign | ((uint32_t)he << 10) | (m >> 13);
+    const uint32_t rem = m & 0x1FFFu;
+    if (rem > 0x1000u || (rem == 0x1000u && (h & 1u))) h++;
+    return (uint16_t)h;
+}
+
+float tfo_f16_to_float(uint16_t h) {
+    const uint32_t sign = ((uint32_t)h & 0x8000u) << 16;
+    const uint32_t e = (h >> 10) & 0x1Fu;
+    uint32_t m = h & 0x3FFu;
+    if (e == 0) {
+        if (m == 0) return bits_f32(sign);
+        int shift = 0;
+        while (!(m & 0x400u)) { m <<= 1; ++shift; }
+        m &= 0x3FFu;
+        return bits_f32(sign | ((uint32_t)(113 - shift) << 23) | (m << 13));
+    }
+    if (e == 31) return bits_f32(sign | 0x7F800000u | (m << 13));
+    return bits_f32(sign | ((e + 112u) << 23) | (m << 13));
+}
+
+// ---------------------------------------------------------------- seeded streams
+uint64_t tfo_splitmix64_next(uint64_t *state) {
+    *state += 0x9E3779B97F4A7C15ull;
+    uint64_t z = *state;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+
+float tfo_splitmix64_uniform(uint64_t *state, float lo, float hi) {
+    const float u = (float)(tfo_splitmix64_next(state) >> 40) / (float)(1 << 24);
+    return lo + (hi - lo) * u;
+}
+
+uint64_t tfo_seedtree_key(uint64_t root, const char *label) {
+    uint64_t h = 0xCBF29CE484222325ull;
+    for (const unsigned char *p = (const unsigned char *)label; *p; ++p) {
+        h ^= (uint64_t)*p;
+        h *= 0x100000001B3ull;
+    }
+    return root ^ h;
+}
+
+void tfo_fill_uniform(uint64_t *state, float lo, float hi, float *out, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) out[i] = tfo_splitmix64_uniform(state, lo, hi);
+}
+
+// ---------------------------------------------------------------- quantizer
+static void quantize_affine(const float *row, int n, int levels, bool nibbles, uint8_t *packed, uint16_t *scales,
+                            uint16_t *biases) {
+    const int groups = n / G;
+    if (nibbles) std::memset(packed, 0, (size_t)n / 2);
+    for (int g = 0; g < groups; ++g) {
+        float wmin = std::numeric_limits<float>::infinity();
+        float wmax = -std::numeric_limits<float>::infinity();
+        for (int k = 0; k < G; ++k) {
+            const float w = row[g * G + k];
+            if (w < wmin) wmin = w;
+            if (w > wmax) wmax = w;
+        }
+        float scale_f, bias_f;
+        if (wmax == wmin) { scale_f = 1.0f; bias_f = wmin; }
+        else { scale_f = (wmax - wmin) / (float)levels; bias_f = wmin; }
+        const uint16_t s_bits = tfo_bf16_bits(scale_f);
+        const uint16_t b_bits = tfo_bf16_bits(bias_f);
+        scales[g] = s_bits;
+        biases[g] = b_bits;
+        const float scale = tfo_bf16_to_float(s_bits);
+        const float bias = tfo_bf16_to_float(b_bits);
+        const float inv_scale = scale == 0.0f ? 0.0f : 1.0f / scale;
+        for (int k = 0; k < G; ++k) {
+            const float w = row[g * G + k];
+            int q = (int)std::round((w - bias) * inv_scale);   // Swift .rounded(): half away from zero
+            q = std::max(0, std::min(levels, q));
+            if (nibbles) {
+                const uint8_t nib = (uint8_t)q & 0x0F;
+                const int byte_idx = g * (G / 2) + (k / 2);
+                if ((k & 1) == 0) packed[byte_idx] = (uint8_t)((packed[byte_idx] & 0xF0) | nib);
+                else packed[byte_idx] = (uint8_t)((packed[byte_idx] & 0x0F) | (nib << 4));
+            } else {
+                packed[g * G + k] = (uint8_t)q;
+            }
+        }
+    }
+}
+
+void tfo_quantize_int4_affine(const float *row, int n, uint8_t *packed, uint16_t *scales, uint16_t *biases) {
+    quantize_affine(row, n, 15, true, packed, scales, biases);
+}
+void tfo_quantize_int8_affine(const float *row, int n, uint8_t *packed, uint16_t *scales, uint16_t *biases) {
+    quantize_affine(row, n, 255, false, packed, scales, biases);
+}
+void tfo_dequantize_int4_affine(const uint8_t *packed, const uint16_t *scales, const uint16_t *biases, int n, float *out) {
+    dequant4_row(packed, scales, biases, n, out);
+}
+void tfo_dequantize_int8_affine(const uint8_t *packed, const uint16_t *scales, const uint16_t *biases, int n, float *out) {
+    dequant8_row(packed, scales, biases, n, out);
+}
+
+void tfo_quantize_int4_matrix(const float *w, int m, int n, uint8_t *packed, uint16_t *scales, uint16_t *biases) {
+    const int groups = n / G;
+    for (int r = 0; r < m; ++r)
+        tfo_quantize_int4_affine(w + (int64_t)r * n, n, packed + (int64_t)r * (n / 2), scales + (int64_t)r * groups,
+                                 biases + (int64_t)r * groups);
+}
+void tfo_quantize_int8_matrix(const float *w, int m, int n, uint8_t *packed, uint16_t *scales, uint16_t *biases) {
+    const int groups = n / G;
+    for (int r = 0; r < m; ++r)
+        tfo_quantize_int8_affine(w + (int64_t)r * n, n, packed + (int64_t)r * n, scales + (int64_t)r * groups,
+                                 biases + (int64_t)r * groups);
+}
+void tfo_dequantize_int4_matrix(const uint8_t *packed, const uint16_t *scales, const uint16_t *biases, int m, int n, float *out) {
+    const int groups = n / G;
+    for (int r = 0; r < m; ++r)
+        dequant4_row(packed + (int64_t)r * (n / 2), scales + (int64_t)r * groups, biases + (int64_t)r * groups, n,
+                     out + (int64_t)r * n);
+}
+void tfo_dequantize_int8_matrix(const uint8_t *packed, const uint16_t *scales, const uint16_t *biases, int m, int n, float *out) {
+    const int groups = n / G;
+    for (int r = 0; r < m; ++r)
+        dequant8_row(packed + (int64_t)r * n, scales + (int64_t)r * groups, biases + (int64_t)r * groups, n,
+                     out + (int64_t)r * n);
+}
+
+// ---------------------------------------------------------------- error metrics
+float tfo_rel_error(const float *actual, const float *reference, int64_t n) {
+    float max_abs_diff = 0.0f, ref_norm = 0.0f;
+    for (int64_t i = 0; i < n; ++i) {
+        max_abs_diff = std::max(max_abs_diff, std::fabs(actual[i] - reference[i]));
+        ref_norm = std::max(ref_norm, std::fabs(reference[i]));
+    }
+    return max_abs_diff / std::max(ref_norm, 1e-6f);
+}
+float tfo_max_abs_diff(const float *a, const float *b, int64_t n) {
+    float m = 0.0f;
+    for (int64_t i = 0; i < n; ++i) m = std::max(m, std::fabs(a[i] - b[i]));
+    return m;
+}
+float tfo_bounded_rel(const float *actual, const float *reference, int64_t n, float abs_floor) {
+    float worst = 0.0f;
+    for (int64_t i = 0; i < n; ++i) {
+        const float diff = std::fabs(actual[i] - reference[i]);
+        const float denom = std::max(std::fabs(reference[i]), abs_floor);
+        worst = std::max(worst, diff / denom);
+    }
+    return worst;
+}
+
+// ---------------------------------------------------------------- GEMV references
+void tfo_int4_gemv_ref(const uint8_t *W, const uint16_t *S, const uint16_t *B, const float *x, float *y, int64_t m,
+                       int n, int threads) {
+    const int groups = n / G;
+#pragma omp parallel num_threads(threads > 1 ? threads : 1) if (threads > 1)
+    {
+        std::vector<float> w_row((size_t)n);
+#pragma omp for schedule(static)
+        for (int64_t row = 0; row < m; ++row) {
+            dequant4_row(W + row * (n / 2), S + row * groups, B + row * groups, n, w_row.data());
+            y[row] = dot_f32(w_row.data(), x, n);
+        }
+    }
+}
+
+void tfo_int8_gemv_ref(const uint8_t *W, const uint16_t *S, const uint16_t *B, const float *x, float *y, int64_t m,
+                       int n, int threads) {
+    const int groups = n / G;
+#pragma omp parallel num_threads(threads > 1 ? threads : 1) if (threads > 1)
+    {
+        std::vector<float> w_row((size_t)n);
+#pragma omp for schedule(static)
+        for (int64_t row = 0; row < m; ++row) {
+            dequant8_row(W + row * n, S + row * groups, B + row * groups, n, w_row.data());
+            y[row] = dot_f32(w_row.data(), x, n);
+        }
+    }
+}
+
+void tfo_int4_gemv_f64(const uint8_t *W, const uint16_t *S, const uint16_t *B, const float *x, double *y, int64_t m, int n) {
+    const int groups = n / G;
+    std::vector<float> w_row((size_t)n);
+    for (int64_t row = 0; row < m; ++row) {
+        dequant4_row(W + row * (n / 2), S + row * groups, B + row * groups, n, w_row.data());
+        double acc = 0.0;
+        for (int i = 0; i < n; ++i) acc += (double)w_row[i] * (double)x[i];
+        y[row] = acc;
+    }
+}
+
+void tfo_int8_gemv_f64(const uint8_t *W, const uint16_t *S, const uint16_t *B, const float *x, double *y, int64_t m, int n) {
+    const int groups = n / G;
+    std::vector<float> w_row((size_t)n);
+    for (int64_t row = 0; row < m; ++row) {
+        dequant8_row(W + row * n, S + row * groups, B + row * groups, n, w_row.data());
+        double acc = 0.0;
+        for (int i = 0; i < n; ++i) acc += (double)w_row[i] * (double)x[i];
+        y[row] = acc;
+    }
+}
+
+// ---------------------------------------------------------------- primitives
+void tfo_gelu_tanh(const float *x, float *y, int64_t n) {
+    for (int64_t i = 0; i < n; ++i) y[i] = gelu_tanh_ref(x[i]);
+}
+
+void tfo_rmsnorm_ref(const float *x, const float *weight, float eps, float *y, int d) {
+    float sum_sq = 0.0f;                       // vDSP_svesq
+    for (int i = 0; i < d; ++i) sum_sq += x[i] * x[i];
+    const float inv_rms = 1.0f / std::sqrt(sum_sq / (float)d + eps);
+    for (int i = 0; i < d; ++i) y[i] = (x[i] * weight[i]) * inv_rms;   // vDSP_vmul then vDSP_vsmul
+}
+
+// ---------------------------------------------------------------- MoE references
+void tfo_moe_run_ffn(const uint8_t *blob, const tfo_expert_offsets *off, const float *x, float *y, int d, int f) {
+    std::vector<float> scratch((size_t)std::max(d, f));
+    std::vector<float> act((size_t)f);
+    for (int r = 0; r < f; ++r) {
+        const float gate = blob_row_dot(blob, off->gate_W_off, off->gate_s_off, off->gate_b_off, r, d, x, scratch.data());
+        const float up = blob_row_dot(blob, off->up_W_off, off->up_s_off, off->up_b_off, r, d, x, scratch.data());
+        act[r] = gelu_tanh_ref(gate) * up;
+    }
+    for (int r = 0; r < d; ++r)
+        y[r] = blob_row_dot(blob, off->down_W_off, off->down_s_off, off->down_b_off, r, f, act.data(), scratch.data());
+}
+
+void tfo_moe_apply_streamed_routed(const uint8_t *const *blobs, const tfo_expert_offsets *off, const float *x,
+                                   const float *residual, const float *routing_w, int n_slots, float *y, int d, int f,
+                                   int threads) {
+    std::vector<float> outs((size_t)n_slots * d);
+#pragma omp parallel for num_threads(threads > 1 ? threads : 1) if (threads > 1) schedule(dynamic, 1)
+    for (int slot = 0; slot < n_slots; ++slot) tfo_moe_run_ffn(blobs[slot], off, x, outs.data() + (size_t)slot * d, d, f);
+    for (int i = 0; i < d; ++i) y[i] = residual[i];
+    for (int slot = 0; slot < n_slots; ++slot) {
+        const float w = routing_w[slot];
+        const float *out = outs.data() + (size_t)slot * d;
+        for (int i = 0; i < d; ++i) y[i] = y[i] + out[i] * w;   // vDSP_vsmul then vDSP_vadd
+    }
+}
+
+void tfo_router_reference(const uint8_t *W, const uint16_t *S, const uint16_t *B, const float *hidden,
+                          const float *effective_scale, const float *expert_scale, int num_experts, int d, int top_k,
+                          uint32_t *out_indices, float *out_weights, float *out_logits) {
+    std::vector<float> scaled((size_t)d), logits((size_t)num_experts);
+    for (int i = 0; i < d; ++i) scaled[i] = hidden[i] * effective_scale[i];
+    tfo_int8_gemv_ref(W, S, B, scaled.data(), logits.data(), num_experts, d, 1);
+    if (out_logits) std::memcpy(out_logits, logits.data(), sizeof(float) * (size_t)num_experts);
+    std::vector<uint32_t> order((size_t)num_experts);
+    for (int e = 0; e < num_experts; ++e) order[e] = (uint32_t)e;
+    std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) {
+        return logits[a] == logits[b] ? a < b : logits[a] > logits[b];
+    });
+    const int k = std::min(top_k, num_experts);
+    const float maximum = k > 0 ? logits[order[0]] : 0.0f;
+    std::vector<float> exps((size_t)k);
+    float sum = 0.0f;
+    for (int i = 0; i < k; ++i) { exps[i] = std::exp(logits[order[i]] - maximum); sum += exps[i]; }
+    for (int i = 0; i < k; ++i) {
+        out_indices[i] = order[i];
+        out_weights[i] = exps[i] / sum * expert_scale[order[i]];
+    }
+}
+
+void tfo_shared_expert_ref(const uint8_t *gW, const uint16_t *gS, const uint16_t *gB, const uint8_t *uW,
+                           const uint16_t *uS, const uint16_t *uB, const uint8_t *dW, const uint16_t *dS,
+                           const uint16_t *dB, const float *x, float *y, int d, int f, int threads) {
+    std::vector<float> gate((size_t)f), up((size_t)f), act((size_t)f);
+    tfo_int4_gemv_ref(gW, gS, gB, x, gate.data(), f, d, threads);
+    tfo_int4_gemv_ref(uW, uS, uB, x, up.data(), f, d, threads);
+    for (int i = 0; i < f; ++i) {
+        const float g = gate[i];
+        const float cube = g * g * g;
+        const double inner = 0.7978845608028654 * (double)(g + 0.044715f * cube);
+        const float gelu = (float)(0.5 * (double)g * (1.0 + std::tanh(inner)));
+        act[i] = tfo_f16_to_float(tfo_f16_bits(gelu * up[i]));
+    }
+    tfo_int4_gemv_ref(dW, dS, dB, act.data(), y, d, f, threads);
+}
+
+// ---------------------------------------------------------------- lm_head
+uint32_t tfo_lm_head_cpu_greedy(const uint16_t *hidden_f16, const uint16_t *norm_w_bf16, const uint8_t *W,
+                                const uint16_t *S, const uint16_t *B, int d, int64_t v, float eps, float *logits_out,
+                                int threads) {
+    std::vector<float> hidden((size_t)d), norm_w((size_t)d), normed((size_t)d);
+    for (int i = 0; i < d; ++i) { hidden[i] = tfo_f16_to_float(hidden_f16[i]); norm_w[i] = tfo_bf16_to_float(norm_w_bf16[i]); }
+    tfo_rmsnorm_ref(hidden.data(), norm_w.data(), eps, normed.data(), d);
+    for (int i = 0; i < d; ++i) normed[i] = tfo_f16_to_float(tfo_f16_bits(normed[i]));
+
+    std::vector<float> local;
+    float *logits = logits_out;
+    if (!logits) { local.resize((size_t)v); logits = local.data(); }
+    tfo_int4_gemv_ref(W, S, B, normed.data(), logits, v, d, threads);
+    float best_value = -std::numeric_limits<float>::infinity();
+    uint32_t best_index = 0;
+    for (int64_t row = 0; row < v; ++row) {
+        if (logits[row] > best_value) { best_value = logits[row]; best_index = (uint32_t)row; }
+    }
+    return best_index;
+}
+
+// ---------------------------------------------------------------- prefill
+void tfo_prefill_make_pairs(const uint32_t *indices, const uint16_t *weights_f16, int query_count, int top_k, tfo_pair *pairs) {
+    for (int token = 0; token < query_count; ++token)
+        for (int rank = 0; rank < top_k; ++rank) {
+            const int i = token * top_k + rank;
+            pairs[i] = tfo_pair{(uint32_t)token, indices[i], (uint32_t)rank, (uint32_t)weights_f16[i]};
+        }
+}
+
+int tfo_prefill_group_pairs(const tfo_pair *pairs, int64_t pair_count, int query_count, int top_k, int num_experts,
+                            int tile_expert_count, const uint64_t *expert_sort_keys, int sort_key_count,
+                            tfo_pair *sorted_pairs, uint32_t *per_expert_offsets, uint32_t *per_expert_counts,
+                            tfo_group *groups, int *n_groups, tfo_tile *tiles, int *n_tiles) {
+    if (query_count < 0) return TFO_GROUP_INVALID_QUERY_COUNT;
+    if (top_k <= 0) return TFO_GROUP_INVALID_TOP_K;
+    if (num_experts <= 0) return TFO_GROUP_INVALID_NUM_EXPERTS;
+    if (tile_expert_count < 1 || tile_expert_count > 16) return TFO_GROUP_INVALID_TILE_EXPERT_COUNT;
+    if (expert_sort_keys && sort_key_count != num_experts) return TFO_GROUP_SORT_KEY_COUNT_MISMATCH;
+    if (pair_count != (int64_t)query_count * top_k) return TFO_GROUP_PAIR_COUNT_MISMATCH;
+
+    std::unordered_set<uint64_t> seen;
+    seen.reserve((size_t)pair_count);
+    for (int64_t i = 0; i < pair_count; ++i) {
+        const tfo_pair &p = pairs[i];
+        if (!(p.token < (uint32_t)query_count)) return TFO_GROUP_TOKEN_OUT_OF_RANGE;
+        if (!(p.rank < (uint32_t)top_k)) return TFO_GROUP_RANK_OUT_OF_RANGE;
+        if (!(p.expert < (uint32_t)num_experts)) return TFO_GROUP_EXPERT_OUT_OF_RANGE;
+        const uint64_t key = ((uint64_t)p.token << 32) | (uint64_t)p.rank;
+        if (!seen.insert(key).second) return TFO_GROUP_DUPLICATE_TOKEN_RANK;
+    }
+
+    std::vector<tfo_pair> sorted(pairs, pairs + pair_count);
+    std::stable_sort(sorted.begin(), sorted.end(), [&](const tfo_pair &a, const tfo_pair &b) {
+        if (expert_sort_keys) {
+            const uint64_t ka = expert_sort_keys[a.expert], kb = expert_sort_keys[b.expert];
+            if (ka != kb) return ka < kb;
+        }
+        if (a.expert != b.expert) return a.expert < b.expert;
+        if (a.token != b.token) return a.token < b.token;
+        return a.rank < b.rank;
+    });
+    for (int e = 0; e < num_experts; ++e) { per_expert_offsets[e] = 0xFFFFFFFFu; per_expert_counts[e] = 0; }
+    int ng = 0;
+    int64_t i = 0;
+    while (i < pair_count) {
+        const uint32_t expert = sorted[(size_t)i].expert;
+        const int64_t start = i;
+        while (i < pair_count && sorted[(size_t)i].expert == expert) ++i;
+        per_expert_offsets[expert] = (uint32_t)start;
+        per_expert_counts[expert] = (uint32_t)(i - start);
+        groups[ng++] = tfo_group{expert, (uint32_t)start, (uint32_t)(i - start)};
+    }
+    int nt = 0;
+    int group_start = 0;
+    while (group_start < ng) {
+        const int group_end = std::min(ng, group_start + tile_expert_count);
+        const tfo_group &first = groups[group_start];
+        const tfo_group &last = groups[group_end - 1];
+        const uint32_t pair_end = last.pair_start + last.pair_count;
+        tiles[nt++] = tfo_tile{(uint32_t)group_start, (uint32_t)(group_end - group_start), first.pair_start,
+                               pair_end - first.pair_start};
+        group_start = group_end;
+    }
+    std::copy(sorted.begin(), sorted.end(), sorted_pairs);
+    *n_groups = ng;
+    *n_tiles = nt;
+    return TFO_GROUP_OK;
+}
+
+float tfo_prefill_cpu_int4_dot(const uint8_t *bytes, int64_t base, int64_t w_off, int64_t s_off, int64_t b_off, int row,
+                               int n, const float *x) {
+    const int groups = n / G;
+    const int row_bytes = n / 2;
+    const int64_t w_row = base + w_off + (int64_t)row * row_bytes;
+    const int64_t s_row = base + s_off + (int64_t)row * groups * 2;
+    const int64_t b_row = base + b_off + (int64_t)row * groups * 2;
+    float acc = 0.0f;
+    for (int group = 0; group < groups; ++group) {
+        const float scale = tfo_bf16_to_float(load_u16(bytes + s_row + group * 2));
+        const float bias = tfo_bf16_to_float(load_u16(bytes + b_row + group * 2));
+        for (int k = 0; k < G; ++k) {
+            const int col = group * G + k;
+            const uint8_t packed = bytes[w_row + col / 2];
+            const float q = (k & 1) == 0 ? (float)(packed & 0x0F) : (float)(packed >> 4);
+            acc += (q * scale + bias) * x[col];
+        }
+    }
+    return acc;
+}
+
+void tfo_prefill_route_partials(const tfo_pair *sorted_pairs, int64_t pair_count, int query_count,
+                                const uint16_t *hidden_f16, int hidden_stride, const uint8_t *pool, int64_t pool_stride,
+                                const tfo_expert_offsets *off, int top_k, int d, int f, uint16_t fill_f16,
+                                uint16_t *out_f16, int threads) {
+    const int64_t total = (int64_t)query_count * top_k * d;
+    for (int64_t i = 0; i < total; ++i) out_f16[i] = fill_f16;
+#pragma omp parallel for num_threads(threads > 1 ? threads : 1) if (threads > 1) schedule(dynamic, 4)
+    for (int64_t p = 0; p < pair_count; ++p) {
+        const tfo_pair &pair = sorted_pairs[p];
+        const int64_t expert_base = (int64_t)pair.expert * pool_stride;
+        const int64_t x_base = (int64_t)pair.token * hidden_stride;
+        std::vector<float> x((size_t)d), act((size_t)f);
+        for (int i = 0; i < d; ++i) x[i] = tfo_f16_to_float(hidden_f16[x_base + i]);
+        for (int row = 0; row < f; ++row) {
+            const float gate = tfo_prefill_cpu_int4_dot(pool, expert_base, off->gate_W_off, off->gate_s_off, off->gate_b_off, row, d, x.data());
+            const float up = tfo_prefill_cpu_int4_dot(pool, expert_base, off->up_W_off, off->up_s_off, off->up_b_off, row, d, x.data());
+            act[row] = tfo_f16_to_float(tfo_f16_bits(gelu_tanh_ref(gate) * up));
+        }
+        const int64_t out_base = ((int64_t)pair.token * top_k + pair.rank) * d;
+        for (int row = 0; row < d; ++row) {
+            const float value = tfo_prefill_cpu_int4_dot(pool, expert_base, off->down_W_off, off->down_s_off, off->down_b_off, row, f, act.data());
+            out_f16[out_base + row] = tfo_f16_bits(value);
+        }
+    }
+}
+
+void tfo_prefill_reduce_token_major(const uint16_t *partials_f16, const uint16_t *weights_f16, int rows, int top_k, int d,
+                                    uint16_t *out_f16) {
+    for (int token = 0; token < rows; ++token)
+        for (int column = 0; column < d; ++column) {
+            float accumulator = 0.0f;
+            for (int rank = 0; rank < top_k; ++rank) {
+                const int64_t partial_index = ((int64_t)token * top_k + rank) * d + column;
+                accumulator += tfo_f16_to_float(weights_f16[token * top_k + rank]) * tfo_f16_to_float(partials_f16[partial_index]);
+            }
+            out_f16[(int64_t)token * d + column] = tfo_f16_bits(accumulator);
+        }
+}
+
+void tfo_qmm_cpu_reference(const uint8_t *W, const uint16_t *S, const uint16_t *B, const uint16_t *x_f16, int m, int n,
+                           int k, float *out, int threads) {
+    const int groups = k / G;
+    const int row_bytes = k / 2;
+#pragma omp parallel for num_threads(threads > 1 ? threads : 1) if (threads > 1) schedule(static)
+    for (int token = 0; token < m; ++token) {
+        std::vector<float> xr((size_t)k);
+        for (int c = 0; c < k; ++c) xr[c] = tfo_f16_to_float(x_f16[(int64_t)token * k + c]);
+        for (int row = 0; row < n; ++row) {
+            float accumulator = 0.0f;
+            for (int group = 0; group < groups; ++group) {
+                const float scale = tfo_bf16_to_float(S[(int64_t)row * groups + group]);
+                const float bias = tfo_bf16_to_float(B[(int64_t)row * groups + group]);
+                for (int local_k = 0; local_k < G; ++local_k) {
+                    const int column = group * G + local_k;
+                    const uint8_t byte = W[(int64_t)row * row_bytes + column / 2];
+                    const uint8_t q = (column % 2 == 0) ? (byte & 0x0F) : (byte >> 4);
+                    const float weight = (float)q * scale + bias;
+                    accumulator = fmaf(weight, xr[column], accumulator);
+                }
+            }
+            out[(int64_t)token * n + row] = tfo_f16_to_float(tfo_f16_bits(accumulator));
+        }
+    }
+}
+
+// ---------------------------------------------------------------- kernel-order restatements
+void tfo_k_int4_gemv(const uint8_t *W, const uint16_t *S, const uint16_t *B, const uint16_t *x_f16, float *y_f32, int64_t m, int n) {
+    const int groups = n / G;
+    for (int64_t row = 0; row < m; ++row)
+        y_f32[row] = kernel_row_int4(W + row * (n / 2), (const uint8_t *)(S + row * groups), (const uint8_t *)(B + row * groups), x_f16, n);
+}
+
+void tfo_k_router_logits(const uint8_t *W, const uint16_t *S, const uint16_t *B, const uint16_t *hidden_f16,
+                         const uint16_t *eff_scale_bf16, float *logits, int num_experts, int d) {
+    const int groups = d / G;
+    for (int e = 0; e < num_experts; ++e) {
+        const uint8_t *w_row = W + (int64_t)e * d;
+        float total = 0.0f;
+        for (int lane = 0; lane < 32; ++lane) {
+            float acc = 0.0f;
+            for (int g = 0; g < groups; ++g) {
+                const float s = tfo_bf16_to_float(S[e * groups + g]);
+                const float b = tfo_bf16_to_float(B[e * groups + g]);
+                const int idx = g * G + lane * 2;
+                const float q0 = (float)w_row[idx], q1 = (float)w_row[idx + 1];
+                const float x0 = tfo_f16_to_float(hidden_f16[idx]) * tfo_bf16_to_float(eff_scale_bf16[idx]);
+                const float x1 = tfo_f16_to_float(hidden_f16[idx + 1]) * tfo_bf16_to_float(eff_scale_bf16[idx + 1]);
+                acc = fmaf(s, q0 * x0 + q1 * x1, acc);
+                acc = fmaf(b, x0 + x1, acc);
+            }
+            total += acc;
+        }
+        logits[e] = total;
+    }
+}
+
+void tfo_k_router_topk(const float *logits, const uint16_t *per_expert_scale_bf16, int num_experts, int top_k,
+                       uint32_t *out_indices, uint16_t *out_weights_f16) {
+    const int KK = std::min(top_k, 64);
+    uint32_t top_idx[64];
+    float top_score[64];
+    for (int i = 0; i < 64; ++i) { top_idx[i] = 0; top_score[i] = -std::numeric_limits<float>::infinity(); }
+    for (int e = 0; e < num_experts; ++e) {
+        const float s = logits[e];
+        if (KK > 0 && s <= top_score[KK - 1]) continue;
+        int pos = KK;
+        for (int i = 0; i < KK; ++i)
+            if (s > top_score[i] || (s == top_score[i] && (uint32_t)e < top_idx[i])) { pos = i; break; }
+        if (pos >= KK) continue;
+        for (int i = KK - 1; i > pos; --i) { top_idx[i] = top_idx[i - 1]; top_score[i] = top_score[i - 1]; }
+        top_idx[pos] = (uint32_t)e;
+        top_score[pos] = s;
+    }
+    const float max_s = top_score[0];
+    float sum_exp = 0.0f;
+    float exps[64];
+    for (int i = 0; i < KK; ++i) { exps[i] = std::exp(top_score[i] - max_s); sum_exp += exps[i]; }
+    for (int i = 0; i < KK; ++i) {
+        const uint32_t expert_idx = top_idx[i];
+        const float weight = exps[i] / sum_exp;
+        out_indices[i] = expert_idx;
+        out_weights_f16[i] = tfo_f16_bits(weight * tfo_bf16_to_float(per_expert_scale_bf16[expert_idx]));
+    }
+}
+
+void tfo_k_moe_phase1(const uint8_t *const *blobs, const tfo_expert_offsets *off, const uint16_t *x_f16,
+                      uint16_t *acts_f16, int d, int f, int top_k) {
+    const int groups = d / G;
+    for (int slot = 0; slot < top_k; ++slot) {
+        const uint8_t *base = blobs[slot];
+        for (int r = 0; r < f; ++r) {
+            const float g = kernel_row_int4(base + off->gate_W_off + (int64_t)r * (d / 2), base + off->gate_s_off + (int64_t)r * groups * 2,
+                                            base + off->gate_b_off + (int64_t)r * groups * 2, x_f16, d);
+            const float u = kernel_row_int4(base + off->up_W_off + (int64_t)r * (d / 2), base + off->up_s_off + (int64_t)r * groups * 2,
+                                            base + off->up_b_off + (int64_t)r * groups * 2, x_f16, d);
+            acts_f16[slot * f + r] = tfo_f16_bits(gelu_tanh_kernel(g) * u);
+        }
+    }
+}
+
+void tfo_k_moe_phase2(const uint8_t *const *blobs, const tfo_expert_offsets *off, const uint16_t *acts_f16,
+                      const uint16_t *routing_w_f16, const uint16_t *residual_f16, uint16_t *y_f16, int d, int f) {
+    const int groups = f / G;
+    for (int row = 0; row < d; ++row) {
+        float acc = tfo_f16_to_float(residual_f16[row]);
+        for (int s = 0; s < 8; ++s) {
+            const uint8_t *base = blobs[s];
+            const float value = kernel_row_int4(base + off->down_W_off + (int64_t)row * (f / 2), base + off->down_s_off + (int64_t)row * groups * 2,
+                                                base + off->down_b_off + (int64_t)row * groups * 2, acts_f16 + (int64_t)s * f, f);
+            acc += tfo_f16_to_float(routing_w_f16[s]) * value;
+        }
+        y_f16[row] = tfo_f16_bits(acc);
+    }
+}
+
+void tfo_k_gelu_mul_fp16(const uint16_t *gate_f16, const uint16_t *up_f16, uint16_t *out_f16, int n) {
+    for (int i = 0; i < n; ++i)
+        out_f16[i] = tfo_f16_bits(gelu_tanh_kernel(tfo_f16_to_float(gate_f16[i])) * tfo_f16_to_float(up_f16[i]));
+}
+
+void tfo_k_rmsnorm_bf16w(const uint16_t *x_f16, const uint16_t *w_bf16, float eps, uint16_t *out_f16, int d) {
+    float partial[256];
+    for (int lid = 0; lid < 256; ++lid) {
+        float acc = 0.0f;
+        for (int i = lid; i < d; i += 256) { const float v = tfo_f16_to_float(x_f16[i]); acc = fmaf(v, v, acc); }
+        partial[lid] = acc;
+    }
+    float total = 0.0f;
+    for (int sg = 0; sg < 8; ++sg) {
+        float s = 0.0f;
+        for (int lane = 0; lane < 32; ++lane) s += partial[sg * 32 + lane];
+        total += s;
+    }
+    const float inv = 1.0f / std::sqrt(total / (float)d + eps);
+    for (int i = 0; i < d; ++i)
+        out_f16[i] = tfo_f16_bits(tfo_f16_to_float(x_f16[i]) * inv * tfo_bf16_to_float(w_bf16[i]));
+}
+
+void tfo_k_prefill_router_logits(const uint8_t *W, const uint16_t *S, const uint16_t *B, const uint16_t *hidden_f16,
+                                 const uint16_t *eff_scale_bf16, float *logits, int num_experts, int d) {
+    const int groups = d / G;
+    for (int e = 0; e < num_experts; ++e) {
+        float acc = 0.0f;
+        for (int g = 0; g < groups; ++g) {
+            const float s = tfo_bf16_to_float(S[e * groups + g]);
+            const float b = tfo_bf16_to_float(B[e * groups + g]);
+            float dot_qx = 0.0f, sum_x = 0.0f;
+            for (int k = 0; k < G; ++k) {
+                const int idx = g * G + k;
+                const float q = (float)W[(int64_t)e * d + idx];
+                const float xv = tfo_f16_to_float(hidden_f16[idx]) * tfo_bf16_to_float(eff_scale_bf16[idx]);
+                dot_qx = fmaf(q, xv, dot_qx);
+                sum_x += xv;
+            }
+            acc = fmaf(s, dot_qx, acc);
+            acc = fmaf(b, sum_x, acc);
+        }
+        logits[e] = acc;
+    }
+}
+
+float tfo_k_prefill_int4_row(const uint8_t *W, const uint16_t *S, const uint16_t *B, const uint16_t *x_f16, int row, int n) {
+    const int groups = n / G;
+    const uint8_t *w_row = W + (int64_t)row * (n / 2);
+    const uint8_t *s_row = (const uint8_t *)S + (int64_t)row * groups * 2;
+    const uint8_t *b_row = (const uint8_t *)B + (int64_t)row * groups * 2;
+    float acc = 0.0f;
+    for (int g = 0; g < groups; ++g) {
+        const float scale = tfo_bf16_to_float(load_u16(s_row + 2 * g));
+        const float bias = tfo_bf16_to_float(load_u16(b_row + 2 * g));
+        float dot_qx = 0.0f, sum_x = 0.0f;
+        for (int k = 0; k < G / 2; ++k) {
+            const uint8_t packed = w_row[g * (G / 2) + k];
+            const float x0 = tfo_f16_to_float(x_f16[g * G + 2 * k]);
+            const float x1 = tfo_f16_to_float(x_f16[g * G + 2 * k + 1]);
+            dot_qx = fmaf((float)(packed & 0x0F), x0, dot_qx);
+            dot_qx = fmaf((float)(packed >> 4), x1, dot_qx);
+            sum_x += x0 + x1;
+        }
+        acc = fmaf(scale, dot_qx, acc);
+        acc = fmaf(bias, sum_x, acc);
+    }
+    return acc;
+}
+
+}  // extern "C"
