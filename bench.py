@@ -1,0 +1,365 @@
+#!/usr/bin/env python3
+"""Benchmark of the int4 MoE matmul path on one MI355X.
+
+A "step" is one token through one MoE layer of the reference model's shape: int8 router (128 x 2816) ->
+top-8 + softmax -> phase 1 (gate/up/GeGLU of the 8 selected experts, 704 x 2816 each) -> phase 2 (down 2816 x 704,
+weighted reduce).  Expert selection stays on the device.  Weights are synthetic (uniform nibbles, bf16 scale
+~U(0.005,0.02), bias ~U(-0.1,0.1)), resident in HBM before the timed region; consecutive steps walk through
+several layer replicas and different hidden states so that reads come from HBM, not from L2 / Infinity Cache.
+
+Prints ONE JSON line.  `value` = algorithmic bytes of the step / time per step.
+"""
+from __future__ import annotations
+
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+D, F_MOE, F_SHARED, E, TOPK, VOCAB = 2816, 704, 2112, 128, 8, 262144
+HBM_PEAK_GBPS = 8000.0   # MI355X HBM3E, published
+
+
+def int4_matrix_bytes(rows, cols):
+    return rows * cols // 2 + 2 * rows * (cols // 64) * 2
+
+
+# per-unit algorithmic bytes (what one launch must move at least once)
+ROUTER_BYTES = E * D + 2 * E * (D // 64) * 2 + D * 2 + D * 2 + E * 2 + TOPK * 4 + TOPK * 2   # W + s/b + hidden + eff + gains + outputs
+PHASE1_BYTES = TOPK * 2 * int4_matrix_bytes(F_MOE, D) + D * 2 + TOPK * F_MOE * 2             # gate+up of 8 experts + x + acts out
+PHASE2_BYTES = TOPK * int4_matrix_bytes(D, F_MOE) + TOPK * F_MOE * 2 + TOPK * 2 + D * 2 + D * 2   # down of 8 + acts in + w + residual + y
+STEP_BYTES = ROUTER_BYTES + PHASE1_BYTES + PHASE2_BYTES
+SHARED_BYTES = 2 * int4_matrix_bytes(F_SHARED, D) + int4_matrix_bytes(D, F_SHARED) + D * 2 + 4 * F_SHARED * 2 + D * 2
+LM_HEAD_BYTES = int4_matrix_bytes(VOCAB, D) + D * 2 + 4
+
+
+def expert_layout():
+    """Byte offsets of the nine sub-tensors in one routed-expert blob, in the reference's order
+    (gate W,S,B, up W,S,B, down W,S,B) with the stride rounded to 16 KiB."""
+    offs, pos = [], 0
+    for rows, cols in ((F_MOE, D), (F_MOE, D), (D, F_MOE)):
+        for nbytes in (rows * cols // 2, rows * (cols // 64) * 2, rows * (cols // 64) * 2):
+            offs.append(pos)
+            pos += nbytes
+    stride = (pos + 16383) // 16384 * 16384
+    return offs, pos, stride
+
+
+def bf16_bits_cuda(t):
+    import torch
+    return t.to(torch.bfloat16).view(torch.int16)
+
+
+def make_layer(torch, gen, offs, stride):
+    """One layer's resident weights on the device: expert pool [E, stride] + int8 router."""
+    pool = torch.randint(0, 256, (E, stride), dtype=torch.uint8, device="cuda", generator=gen)
+    shapes = ((F_MOE, D), (F_MOE, D), (D, F_MOE))
+    for p, (rows, cols) in enumerate(shapes):
+        n = rows * (cols // 64)
+        for j, (lo, hi) in ((1, (0.005, 0.02)), (2, (-0.1, 0.1))):
+            vals = torch.rand((E, n), device="cuda", generator=gen) * (hi - lo) + lo
+            o = offs[3 * p + j]
+            pool[:, o:o + 2 * n] = bf16_bits_cuda(vals).view(torch.uint8).view(E, 2 * n)
+    router = dict(
+        W=torch.randint(0, 256, (E, D), dtype=torch.uint8, device="cuda", generator=gen),
+        S=bf16_bits_cuda(torch.rand((E, D // 64), device="cuda", generator=gen) * 0.0006 + 0.0002),
+        B=bf16_bits_cuda(torch.rand((E, D // 64), device="cuda", generator=gen) * -0.1),
+        eff=bf16_bits_cuda((torch.rand(D, device="cuda", generator=gen) + 0.5) / (D ** 0.5)),
+        gain=bf16_bits_cuda(torch.rand(E, device="cuda", generator=gen) * 0.8 + 0.6),
+    )
+    return pool, router
+
+
+def make_int4(torch, gen, rows, cols):
+    W = torch.randint(0, 256, (rows, cols // 2), dtype=torch.uint8, device="cuda", generator=gen)
+    S = bf16_bits_cuda(torch.rand((rows, cols // 64), device="cuda", generator=gen) * 0.015 + 0.005)
+    B = bf16_bits_cuda(torch.rand((rows, cols // 64), device="cuda", generator=gen) * 0.2 - 0.1)
+    return W, S, B
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=640)
+    ap.add_argument("--warmup", type=int, default=64)
+    ap.add_argument("--layers", type=int, default=4, help="layer replicas the steps rotate through")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip lm_head / GEMV / shared-expert side measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    tfk = importlib.import_module("turbo-fieldfare_amd")
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    torch.cuda.set_device(0)
+    k = tfk.Context(0)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(0x7F1E1DFA)
+    offs, payload, stride = expert_layout()
+    off = tfk.ExpertOffsets(*offs)
+    layers = [make_layer(torch, gen, offs, stride) for _ in range(args.layers)]
+    n_hidden = 64
+    hidden = torch.randn((n_hidden, D), device="cuda", generator=gen).to(torch.float16)
+    idx = torch.zeros((n_hidden, TOPK), dtype=torch.int32, device="cuda")
+    wts = torch.zeros((n_hidden, TOPK), dtype=torch.float16, device="cuda")
+    acts = torch.zeros(TOPK * F_MOE, dtype=torch.float16, device="cuda")
+    residual = torch.zeros(D, dtype=torch.float16, device="cuda")
+    y = torch.zeros((n_hidden, D), dtype=torch.float16, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    lib, h = k.lib, k.handle
+    routed = [k.routed_from_pool(pool, stride, 0, E) for pool, _ in layers]
+
+    import ctypes as C
+
+    def step(i, ev=None):
+        li, hi = i % args.layers, i % n_hidden
+        pool, r = layers[li]
+        hp = hidden.data_ptr() + hi * D * 2
+        ip, wp = idx.data_ptr() + hi * TOPK * 4, wts.data_ptr() + hi * TOPK * 2
+        rb = routed[li]
+        rb.indices = ip
+        rc = lib.tf_router_gemma4(h, stream, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, hp,
+                                  r["eff"].data_ptr(), 0, r["gain"].data_ptr(), 0, ip, wp, E, D, TOPK)
+        if ev is not None:
+            ev[0].record()
+        rc |= lib.tf_moe_phase1_gate_up_act(h, stream, C.byref(rb), C.byref(off), hp, acts.data_ptr(), D, F_MOE, TOPK, tfk.TF_BF16)
+        if ev is not None:
+            ev[1].record()
+        rc |= lib.tf_moe_phase2_down_reduce(h, stream, C.byref(rb), C.byref(off), acts.data_ptr(), wp, residual.data_ptr(),
+                                            y.data_ptr() + hi * D * 2, D, F_MOE, TOPK, tfk.TF_BF16)
+        if ev is not None:
+            ev[2].record()
+        if rc != 0:
+            raise RuntimeError("kernel call failed: " + k.last_error())
+
+    def run_steps(first, count, ev=None):
+        for j in range(count):
+            step(first + j, None if ev is None else ev[j])
+
+    # ---- the decode loop is launch-bound on the host (3 short kernels per step), so the steps are captured once
+    # into HIP graphs and replayed: `graph_steps` steps per graph, plus one remainder graph, exactly `steps` in all.
+    graph_steps = min(64, args.steps)
+    n_full, rem = divmod(args.steps, graph_steps)
+    side = torch.cuda.Stream()            # default priority
+    graphs = {}
+    run_steps(0, args.warmup)             # untimed warm-up (eager)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(side):
+        for count in {graph_steps, rem} - {0}:
+            g = torch.cuda.CUDAGraph()
+            stream = torch.cuda.current_stream().cuda_stream
+            with torch.cuda.graph(g, stream=side):
+                stream = torch.cuda.current_stream().cuda_stream
+                run_steps(0, count)
+            graphs[count] = g
+        stream = torch.cuda.current_stream().cuda_stream
+        graphs[graph_steps].replay()      # one untimed replay
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n_full):
+            graphs[graph_steps].replay()
+        if rem:
+            graphs[rem].replay()
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+    stream = torch.cuda.current_stream().cuda_stream
+    ms_per_step = elapsed * 1e3 / args.steps
+    value = STEP_BYTES / (ms_per_step * 1e-3) / 1e9
+
+    # the same loop launched call by call (no graph): what a host that encodes every step itself would see
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    run_steps(args.warmup, args.steps)
+    torch.cuda.synchronize()
+    ms_per_step_eager = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # ---- per-kernel durations with HIP events on the launch stream.  A spin kernel is queued first so that the host
+    # finishes enqueueing before the GPU starts: the events then bracket back-to-back execution, not host gaps.
+    n_ev = min(args.steps, 128)
+    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(n_ev)]
+    torch.cuda._sleep(int(2.4e9 * 0.03))
+    for i in range(n_ev):
+        evs[i][3].record()
+        step(args.warmup + i, evs[i])
+    torch.cuda.synchronize()
+    t_router = float(np.mean([e[3].elapsed_time(e[0]) for e in evs])) * 1e3   # us
+    t_p1 = float(np.mean([e[0].elapsed_time(e[1]) for e in evs])) * 1e3
+    t_p2 = float(np.mean([e[1].elapsed_time(e[2]) for e in evs])) * 1e3
+    p1_gbps = PHASE1_BYTES / (t_p1 * 1e-6) / 1e9
+
+    out = {
+        "metric": "int4 MoE decode GEMV GB/s (% HBM peak) + batch-1 decode step/s; prefill tok/s",
+        "value": round(value, 2), "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int4 weights x fp16 activations, fp32 accumulate", "data": "synthetic",
+        "config": {"workload": "configs[1]: routed MoE FFN decode step, batch 1, hidden 2816, int8 router 128x2816 + top-8, "
+                               "8 of 128 int4 g64 experts (gate/up 704x2816, down 2816x704), GeGLU, weighted sum",
+                   "layer_replicas": args.layers, "resident_expert_bytes": args.layers * E * stride,
+                   "algorithmic_bytes_per_step": STEP_BYTES},
+        "roofline": {"bound": "hbm", "kernel": "phase1_long_kernel<2,3,bf16> (gate/up/GeGLU of 8 experts)",
+                     "achieved": round(p1_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(p1_gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "algorithmic_bytes_per_launch": PHASE1_BYTES, "avg_launch_us": round(t_p1, 3)},
+        "launch": f"HIP graph replay, {graph_steps} steps per graph",
+        "step_per_s": round(1e3 / ms_per_step, 1),
+        "ms_per_step_eager_launch": round(ms_per_step_eager, 6),
+        "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
+        "kernels_us": {"router": round(t_router, 3), "phase1": round(t_p1, 3), "phase2": round(t_p2, 3),
+                       "phase2_GBps": round(PHASE2_BYTES / (t_p2 * 1e-6) / 1e9, 1)},
+    }
+
+    if not args.no_extras:
+        out["extras"] = extras(torch, tfk, k, gen, lib, h, stream)
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(torch, layers, hidden, idx, wts, y, offs, stride, payload, args)
+    print(json.dumps(out))
+
+
+def time_loop(torch, fn, iters, warmup=3):
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for i in range(iters):
+        fn(warmup + i)
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / iters   # us per call
+
+
+def extras(torch, tfk, k, gen, lib, h, stream):
+    """Side measurements on the other single-GPU configurations (not the headline value)."""
+    res = {}
+    # configs[2]: int4 lm_head 262144 x 2816 -> greedy argmax; two replicas alternate (830 MB > Infinity Cache)
+    heads = [make_int4(torch, gen, VOCAB, D) for _ in range(2)]
+    hid = torch.randn((8, D), device="cuda", generator=gen).to(torch.float16)
+    norm_w = bf16_bits_cuda(torch.rand(D, device="cuda", generator=gen) + 0.5)
+    tok = torch.zeros(1, dtype=torch.int32, device="cuda")
+
+    def head(i):
+        W, S, B = heads[i % 2]
+        rc = lib.tf_lm_head_greedy_int4(h, stream, hid.data_ptr(), (i % 8) * D * 2, norm_w.data_ptr(), 0, W.data_ptr(), 0,
+                                        S.data_ptr(), 0, B.data_ptr(), 0, tok.data_ptr(), D, VOCAB, 1e-6, tfk.TF_BF16)
+        assert rc == 0, k.last_error()
+    us = time_loop(torch, head, 30)
+    res["lm_head_greedy"] = {"workload": "configs[2]: int4 lm_head 262144x2816 -> argmax (rmsnorm + rows + reduce)",
+                             "us_per_call": round(us, 2), "GBps": round(LM_HEAD_BYTES / (us * 1e-6) / 1e9, 1),
+                             "frac_hbm_peak": round(LM_HEAD_BYTES / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                             "algorithmic_bytes": LM_HEAD_BYTES}
+    logits = torch.zeros(VOCAB, dtype=torch.float32, device="cuda")
+
+    def head_logits(i):
+        W, S, B = heads[i % 2]
+        rc = lib.tf_lm_head_logits_int4(h, stream, hid.data_ptr(), (i % 8) * D * 2, norm_w.data_ptr(), 0, W.data_ptr(), 0,
+                                        S.data_ptr(), 0, B.data_ptr(), 0, logits.data_ptr(), 0, D, VOCAB, 1e-6, tfk.TF_BF16, tfk.TF_FP32)
+        assert rc == 0, k.last_error()
+    us = time_loop(torch, head_logits, 30)
+    nbytes = LM_HEAD_BYTES + VOCAB * 4
+    res["lm_head_logits_fp32"] = {"us_per_call": round(us, 2), "GBps": round(nbytes / (us * 1e-6) / 1e9, 1),
+                                  "frac_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
+    del heads
+
+    # configs[0]: int4 GEMV 2112 x 2816, rotating over 192 replicas (644 MB)
+    reps = 192
+    W, S, B = make_int4(torch, gen, reps * F_SHARED, D)
+    xs = torch.randn((8, D), device="cuda", generator=gen).to(torch.float16)
+    yv = torch.zeros(F_SHARED, dtype=torch.float16, device="cuda")
+    row_w, row_s = D // 2, (D // 64) * 2
+
+    def gemv(i):
+        r = (i % reps) * F_SHARED
+        rc = lib.tf_dequant_int4_gemv(h, stream, W.data_ptr(), r * row_w, S.data_ptr(), r * row_s, B.data_ptr(), r * row_s,
+                                      xs.data_ptr(), (i % 8) * D * 2, yv.data_ptr(), 0, F_SHARED, D, tfk.TF_BF16, tfk.TF_FP16)
+        assert rc == 0, k.last_error()
+    us = time_loop(torch, gemv, 400, warmup=20)
+    nbytes = int4_matrix_bytes(F_SHARED, D) + D * 2 + F_SHARED * 2
+    res["gemv_2112x2816"] = {"workload": "configs[0]: int4 g64 GEMV 2112x2816, batch 1", "us_per_call": round(us, 3),
+                             "GBps": round(nbytes / (us * 1e-6) / 1e9, 1), "algorithmic_bytes": nbytes}
+
+    # shared expert chain (gate/up 2112x2816 fused + GeGLU, down 2816x2112), rotating over 64 replicas of each matrix
+    sreps = 64
+    gu = W[: sreps * 2 * F_SHARED], S[: sreps * 2 * F_SHARED], B[: sreps * 2 * F_SHARED]
+    dW, dS, dB = make_int4(torch, gen, sreps * D, F_SHARED)
+    sg, su, sa = (torch.zeros(F_SHARED, dtype=torch.float16, device="cuda") for _ in range(3))
+    ys = torch.zeros(D, dtype=torch.float16, device="cuda")
+    import ctypes as C
+    drow_w, drow_s = F_SHARED // 2, (F_SHARED // 64) * 2
+
+    def shared(i):
+        r = (i % sreps) * 2 * F_SHARED
+        g = tfk.Projection(gu[0].data_ptr(), r * row_w, gu[1].data_ptr(), r * row_s, gu[2].data_ptr(), r * row_s, F_SHARED, D)
+        u = tfk.Projection(gu[0].data_ptr(), (r + F_SHARED) * row_w, gu[1].data_ptr(), (r + F_SHARED) * row_s, gu[2].data_ptr(),
+                           (r + F_SHARED) * row_s, F_SHARED, D)
+        dr = (i % sreps) * D
+        dn = tfk.Projection(dW.data_ptr(), dr * drow_w, dS.data_ptr(), dr * drow_s, dB.data_ptr(), dr * drow_s, D, F_SHARED)
+        rc = lib.tf_shared_expert_int4(h, stream, xs.data_ptr(), (i % 8) * D * 2, 8 * D * 2, C.byref(g), C.byref(u), C.byref(dn),
+                                       ys.data_ptr(), 0, D * 2, sg.data_ptr(), 0, F_SHARED * 2, su.data_ptr(), 0, F_SHARED * 2,
+                                       sa.data_ptr(), 0, F_SHARED * 2, 4, tfk.TF_BF16)
+        assert rc == 0, k.last_error()
+    us = time_loop(torch, shared, 300, warmup=20)
+    res["shared_expert_int4"] = {"us_per_call": round(us, 3), "GBps": round(SHARED_BYTES / (us * 1e-6) / 1e9, 1),
+                                 "algorithmic_bytes": SHARED_BYTES}
+    return res
+
+
+def cpu_baseline(torch, layers, hidden, idx, wts, y, offs, stride, payload, args):
+    """The CPU restatement of the reference's FP32 path (the oracle) timed on this host on a bounded sample of the same
+    steps; also checks the device results of those steps against it."""
+    from oracle import tfo
+    off = tfo.ExpertOffsets(*offs)
+    n_sample = 12
+    total_1, total_n, worst_rel, idx_match = 0.0, 0.0, 0.0, 0
+    cores = max(1, min(os.cpu_count() or 1, 16))
+    for sidx in range(n_sample):
+        i = args.warmup + sidx          # a step of the timed region
+        li, hi = i % args.layers, i % hidden.shape[0]
+        pool, r = layers[li]
+        hid_bits = hidden[hi].view(torch.int16).cpu().numpy().view(np.uint16)
+        x = tfo.from_f16_bits(hid_bits)
+        W, S, B = r["W"].cpu().numpy(), r["S"].cpu().numpy().view(np.uint16), r["B"].cpu().numpy().view(np.uint16)
+        eff = tfo.bf16_array_to_float(r["eff"].cpu().numpy().view(np.uint16))
+        gain = tfo.bf16_array_to_float(r["gain"].cpu().numpy().view(np.uint16))
+        gpu_idx = idx[hi].cpu().numpy().view(np.uint32)
+        blobs_all = {int(e): pool[int(e), :payload].cpu().numpy() for e in gpu_idx}
+        t0 = time.perf_counter()
+        ref_idx, ref_w, _ = tfo.router_reference(W, S, B, x, eff, gain)
+        t_router = time.perf_counter() - t0
+        for e in ref_idx:
+            if int(e) not in blobs_all:
+                blobs_all[int(e)] = pool[int(e), :payload].cpu().numpy()
+        blobs = [blobs_all[int(e)] for e in ref_idx]
+        zero = np.zeros(D, np.float32)
+        t0 = time.perf_counter()
+        ref_y = tfo.moe_apply_streamed_routed(blobs, off, x, zero, ref_w, D, F_MOE, threads=1)
+        total_1 += time.perf_counter() - t0 + t_router
+        t0 = time.perf_counter()
+        tfo.moe_apply_streamed_routed(blobs, off, x, zero, ref_w, D, F_MOE, threads=cores)
+        total_n += time.perf_counter() - t0 + t_router
+        if list(ref_idx) == list(gpu_idx):
+            idx_match += 1
+            got = y[hi].float().cpu().numpy()
+            worst_rel = max(worst_rel, tfo.rel_error(got, ref_y))
+    per_step_1 = total_1 / n_sample
+    return {"value": round(STEP_BYTES / per_step_1 / 1e9, 4), "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"{n_sample} of the timed decode steps (router + 8 experts), serial C++ restatement of the reference's "
+                      "bulk-dequantise-row-then-fp32-dot path",
+            "ms_per_step": round(per_step_1 * 1e3, 3),
+            "openmp": {"value": round(STEP_BYTES / (total_n / n_sample) / 1e9, 4), "cores": cores,
+                       "ms_per_step": round(total_n / n_sample * 1e3, 3)},
+            "parity_on_sample": {"steps_with_identical_expert_indices": idx_match, "of": n_sample,
+                                 "worst_rel_error_vs_cpu": round(worst_rel, 6)}}
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,43 @@
+"""The C-ABI library loads and exports exactly what include/tf_kernels.h declares (no GPU needed)."""
+import ctypes as C
+import importlib
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "tf_kernels.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(tf_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    tfk = importlib.import_module("turbo-fieldfare_amd")
+    lib = tfk.load()
+    names = declared_symbols()
+    assert len(names) >= 20
+    for name in names:
+        assert hasattr(lib, name), f"{name} declared in tf_kernels.h but not exported"
+    assert sorted(tfk.EXPORTS) == names, "python binding table and header disagree"
+    assert lib.tf_abi_version() == 1
+    assert lib.tf_status_string(0) == b"ok"
+    assert lib.tf_status_string(tfk.TF_ERR_UNAVAILABLE).startswith(b"unavailable")
+
+
+def test_pod_layouts_match_the_reference():
+    tfk = importlib.import_module("turbo-fieldfare_amd")
+    # MoE.swift:4-29 (9 x UInt32); PrefillRouterTests.swift:12-19 (16 bytes, offsets 0/4/8/12)
+    assert C.sizeof(tfk.ExpertOffsets) == 36
+    assert C.sizeof(tfk.PrefillPair) == 16
+    assert [getattr(tfk.PrefillPair, n).offset for n in ("token", "expert", "rank", "weight_bits_and_reserved")] == [0, 4, 8, 12]
+
+
+def test_product_does_not_reference_the_oracle():
+    pkg = os.path.join(ROOT, "turbo-fieldfare_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h", ".cpp")):
+                text = open(os.path.join(dirpath, f), errors="ignore").read()
+                assert "oracle" not in text.lower(), f"{f} mentions the oracle"

@@ -1,0 +1,244 @@
+"""GPU parity: router, routed experts (phase 1 / subset / phase 2), shared expert — through the C ABI, against the
+CPU oracle.  Cases restate RouterTopKTests, MoEFusedFFNTests and SharedExpertInt4Tests of the reference."""
+import numpy as np
+import pytest
+
+import refcases
+from gpu_helpers import ctx, dev, device_view, host, tfk, within_north_star, zeros_bytes
+from oracle import tfo
+
+pytestmark = pytest.mark.gpu
+
+
+def _router_tensors(weights, hidden, eff, escale, w_off=0):
+    W, S, B = tfo.quantize_int8(weights)
+    return W, S, B, dict(W=dev(W, w_off), S=dev(S), B=dev(B), h=dev(tfo.to_f16_bits(hidden)), eff=dev(tfo.bf16_bits_array(eff)),
+                         pes=dev(tfo.bf16_bits_array(escale)), idx=zeros_bytes(32), wts=zeros_bytes(16))
+
+
+def router_gpu(weights, hidden, eff, escale, w_off=0):
+    W, S, B, t = _router_tensors(weights, hidden, eff, escale, w_off)
+    e, d = W.shape
+    k = ctx()
+    k.check(k.lib.tf_router_gemma4(k.handle, None, t["W"].data_ptr(), w_off, t["S"].data_ptr(), 0, t["B"].data_ptr(), 0,
+                                   t["h"].data_ptr(), t["eff"].data_ptr(), 0, t["pes"].data_ptr(), 0, t["idx"].data_ptr(),
+                                   t["wts"].data_ptr(), e, d, 8))
+    import torch
+    torch.cuda.synchronize()
+    return (W, S, B), host(t["idx"], np.uint32, 8), tfo.from_f16_bits(host(t["wts"], np.uint16, 8))
+
+
+@pytest.mark.parametrize("w_off", [0, 1])
+def test_production_router_matches_reference(w_off):
+    weights, hidden, eff, escale = refcases.router_case_production()
+    (W, S, B), idx, wts = router_gpu(weights, hidden, eff, escale, w_off)
+    ref_idx, ref_w, _ = tfo.router_reference(W, S, B, hidden, eff, escale)
+    assert list(idx) == list(ref_idx)
+    assert np.max(np.abs(wts - ref_w)) < 5e-3
+
+
+def test_production_router_resolves_near_tie_like_reference():
+    weights, hidden, eff, escale = refcases.router_case_near_tie()
+    (W, S, B), idx, _ = router_gpu(weights, hidden, eff, escale)
+    assert list(idx) == [0, 1, 2, 3, 4, 5, 6, 8]
+    assert list(idx) == list(tfo.router_reference(W, S, B, hidden, eff, escale)[0])
+
+
+def test_router_at_production_shape_and_back_to_back_calls():
+    # 128 experts x 2816, the shape BASELINE config 1 routes with; two calls in a row check the ticket counter resets
+    rng = np.random.default_rng(0xA11)
+    W, S, B = refcases.synthetic_int8(128, 2816, 0xA11)
+    k = ctx()
+    for trial in range(2):
+        hidden_bits = refcases.normal_f16(2816, 0xA11 + trial)
+        eff = rng.uniform(0.5, 1.5, 2816).astype(np.float32) / np.float32(np.sqrt(2816.0))
+        escale = rng.uniform(0.6, 1.4, 128).astype(np.float32)
+        eff_bits, pes_bits = tfo.bf16_bits_array(eff), tfo.bf16_bits_array(escale)
+        idx, wts = zeros_bytes(32), zeros_bytes(16)
+        k.router_gemma4(dev(W), dev(S), dev(B), dev(hidden_bits), dev(eff_bits), dev(pes_bits), idx, wts, 128, 2816)
+        got_idx, got_w = host(idx, np.uint32, 8), tfo.from_f16_bits(host(wts, np.uint16, 8))
+        ref_idx, ref_w, ref_logits = tfo.router_reference(W, S, B, tfo.from_f16_bits(hidden_bits), tfo.bf16_array_to_float(eff_bits),
+                                                          tfo.bf16_array_to_float(pes_bits))
+        logits = device_view(k.router_logits_ptr(), 128, "<f4")
+        assert tfo.rel_error(logits, ref_logits) < 1e-4
+        srt = np.sort(ref_logits)[::-1]
+        if np.min(srt[:8] - srt[1:9]) > 1e-4 * np.max(np.abs(srt)):   # no near tie in the reference: order is pinned
+            assert list(got_idx) == list(ref_idx)
+            assert np.max(np.abs(got_w - ref_w)) < 5e-3
+        assert abs(float(got_w.sum() / np.sum(tfo.bf16_array_to_float(pes_bits)[got_idx] * ref_w / tfo.bf16_array_to_float(pes_bits)[ref_idx])) - 1) < 0.2
+
+
+def test_router_rejects_bad_contract():
+    weights, hidden, eff, escale = refcases.router_case_production()
+    W, S, B, t = _router_tensors(weights, hidden, eff, escale)
+    k = ctx()
+    def call(e, d, topk):
+        return k.lib.tf_router_gemma4(k.handle, None, t["W"].data_ptr(), 0, t["S"].data_ptr(), 0, t["B"].data_ptr(), 0, t["h"].data_ptr(),
+                                      t["eff"].data_ptr(), 0, t["pes"].data_ptr(), 0, t["idx"].data_ptr(), t["wts"].data_ptr(), e, d, topk)
+    assert call(16, 128, 4) == tfk.TF_ERR_INVALID_ARGUMENT      # topK must be 8 (MoE.swift:123)
+    assert call(257, 128, 8) == tfk.TF_ERR_INVALID_ARGUMENT     # numExperts <= 256 (MoE.swift:122)
+    assert call(16, 100, 8) == tfk.TF_ERR_INVALID_ARGUMENT      # d % 64 (MoE.swift:121)
+
+
+def _moe_buffers(c, blob_prefix=None):
+    blobs = [dev(b, 0 if blob_prefix is None else blob_prefix(i)) for i, b in enumerate(c["blobs"])]
+    ptrs = [t.data_ptr() + (0 if blob_prefix is None else blob_prefix(i)) for i, t in enumerate(blobs)]
+    off = tfk.ExpertOffsets(*c["off"].as_tuple())
+    return blobs, ptrs, off
+
+
+def run_moe(c, split=False, blob_prefix=None, pool_mode=False):
+    d, f = c["d"], c["f"]
+    k = ctx()
+    blobs, ptrs, off = _moe_buffers(c, blob_prefix)
+    x, res, rw = dev(c["x_bits"]), dev(c["residual_bits"]), dev(c["routing_w_bits"])
+    acts, y = zeros_bytes(8 * f * 2), zeros_bytes(d * 2 + 32, 0xEE)
+    if pool_mode:
+        stride = (c["blobs"][0].size + 63) // 64 * 64
+        pool_np = np.zeros(16 * stride, np.uint8)
+        perm = [5, 11, 2, 7, 0, 15, 9, 3]
+        for slot, e in enumerate(perm):
+            pool_np[e * stride:e * stride + c["blobs"][slot].size] = c["blobs"][slot]
+        pool = dev(pool_np)
+        routed = k.routed_from_pool(pool, stride, dev(np.array(perm, np.uint32)), 16)
+        keep = pool
+    else:
+        routed = k.routed_from_pointers(ptrs)
+        keep = blobs
+    if split:
+        for slots in ([0, 1, 2, 3], [4, 5, 6, 7]):
+            k.moe_phase1(routed, off, x, acts, d, f, active_slots=dev(np.array(slots, np.uint32)), active_count=4)
+    else:
+        k.moe_phase1(routed, off, x, acts, d, f)
+    k.moe_phase2(routed, off, acts, rw, res, y, d, f)
+    out = host(y, np.uint16, d)
+    assert np.all(host(y, np.uint8)[d * 2:] == 0xEE)
+    del keep
+    return out, host(acts, np.uint16, 8 * f)
+
+
+def test_production_routed_pipeline_and_hit_split_match_reference():
+    # MoEFusedFFNTests.swift:17-159
+    c = refcases.moe_fused_case()
+    d, f = c["d"], c["f"]
+    full, acts = run_moe(c)
+    split, acts_split = run_moe(c, split=True)
+    assert np.array_equal(full, split) and np.array_equal(acts, acts_split)     # bitwise
+    expected = tfo.moe_apply_streamed_routed(c["blobs"], c["off"], tfo.from_f16_bits(c["x_bits"]), tfo.from_f16_bits(c["residual_bits"]),
+                                             tfo.from_f16_bits(c["routing_w_bits"]), d, f)
+    got = tfo.from_f16_bits(full)
+    assert tfo.rel_error(got, expected) < tfo.Tolerance.fp16ChainedReduction
+    assert within_north_star(got, expected)
+    # against the kernel-order restatement the device may differ only by summation order: a couple of fp16 ulps
+    k_acts = tfo.k_moe_phase1(c["blobs"], c["off"], c["x_bits"], d, f)
+    assert np.max(np.abs(tfo.from_f16_bits(acts) - tfo.from_f16_bits(k_acts))) < 2e-3
+    k_y = tfo.from_f16_bits(tfo.k_moe_phase2(c["blobs"], c["off"], acts, c["routing_w_bits"], c["residual_bits"], d, f))
+    assert np.max(np.abs(got - k_y)) < 2e-3
+
+
+def test_routed_pipeline_pool_indirection_and_unaligned_blobs_agree():
+    c = refcases.moe_fused_case()
+    full, acts = run_moe(c)
+    pooled, acts_pool = run_moe(c, pool_mode=True)
+    assert np.array_equal(full, pooled) and np.array_equal(acts, acts_pool)
+    # blobs bound at 2-aligned, non-16-aligned bases take the 16-bit-load path: same sums up to order
+    odd, _ = run_moe(c, blob_prefix=lambda i: 2 + 4 * i)
+    assert np.max(np.abs(tfo.from_f16_bits(odd) - tfo.from_f16_bits(full))) < 2e-3
+
+
+@pytest.mark.parametrize("d,f", [(2816, 704), (2816, 64), (704, 128)])
+def test_routed_pipeline_production_shape(d, f):
+    # BASELINE config 1 expert shape (gate/up 704 x 2816, down 2816 x 704), synthetic nibbles/scales
+    rng = np.random.default_rng(d + f)
+    blobs, off = [], None
+    for e in range(8):
+        blob, off = tfo.make_blob(refcases.synthetic_int4(f, d, 0x100 + e, "gate"), refcases.synthetic_int4(f, d, 0x100 + e, "up"),
+                                  refcases.synthetic_int4(d, f, 0x100 + e, "down"))
+        blobs.append(blob)
+    c = dict(blobs=blobs, off=off, d=d, f=f, x_bits=refcases.normal_f16(d, 0x77),
+             residual_bits=np.zeros(d, np.uint16),
+             routing_w_bits=tfo.to_f16_bits(rng.dirichlet(np.ones(8)).astype(np.float32)))
+    full, acts = run_moe(c)
+    expected = tfo.moe_apply_streamed_routed(blobs, off, tfo.from_f16_bits(c["x_bits"]), np.zeros(d, np.float32),
+                                             tfo.from_f16_bits(c["routing_w_bits"]), d, f, threads=8)
+    got = tfo.from_f16_bits(full)
+    assert tfo.rel_error(got, expected) < tfo.Tolerance.fp16ChainedReduction
+    assert within_north_star(got, expected, abs_=1e-3 * max(1.0, float(np.max(np.abs(expected)))))
+    split, _ = run_moe(c, split=True)
+    assert np.array_equal(full, split)
+
+
+def test_moe_rejects_bad_contract():
+    c = refcases.moe_fused_case()
+    k = ctx()
+    blobs, ptrs, off = _moe_buffers(c)
+    x, acts = dev(c["x_bits"]), zeros_bytes(8 * 64 * 2, 0xEE)
+    routed = k.routed_from_pointers(ptrs)
+    assert k.moe_phase1(routed, off, x, acts, 128, 64, top_k=4, raise_on_error=False) == tfk.TF_ERR_INVALID_ARGUMENT   # MoE.swift:298
+    missing = k.routed_from_pointers(ptrs[:7])
+    assert k.moe_phase1(missing, off, x, acts, 128, 64, raise_on_error=False) == tfk.TF_ERR_INVALID_ARGUMENT          # MoE.swift:299
+    # activeCount == 0: nothing is enqueued (MoE.swift:231)
+    assert k.moe_phase1(routed, off, x, acts, 128, 64, active_slots=dev(np.zeros(1, np.uint32)), active_count=0) == tfk.TF_OK
+    assert np.all(host(acts, np.uint8) == 0xEE)
+
+
+def _proj(dW, dS, dB, rows, cols):
+    return tfk.projection(dW, dS, dB, rows, cols)
+
+
+def run_shared(c, scratch_halves=None, weight_bits=4):
+    d, f = c["d"], c["f"]
+    k = ctx()
+    t = {n: [dev(a) for a in c[n]] for n in ("gate", "up", "down")}
+    x, y = dev(c["x_bits"]), zeros_bytes(d * 2)
+    n_s = (scratch_halves if scratch_halves is not None else f) * 2
+    sg, su, sa = zeros_bytes(n_s), zeros_bytes(n_s), zeros_bytes(n_s)
+    rc = k.shared_expert_int4(x, _proj(*t["gate"], f, d), _proj(*t["up"], f, d), _proj(*t["down"], d, f), y, sg, su, sa,
+                              weight_bits=weight_bits, raise_on_error=False)
+    return rc, host(y, np.uint16, d), (host(sg, np.uint16), host(su, np.uint16), host(sa, np.uint16))
+
+
+def test_shared_expert_int4_matches_affine_reference():
+    # SharedExpertInt4Tests.swift:11-53
+    c = refcases.shared_expert_case()
+    rc, y, (sg, su, sa) = run_shared(c)
+    assert rc == tfk.TF_OK
+    ref = tfo.shared_expert_ref(c["gate"], c["up"], c["down"], tfo.from_f16_bits(c["x_bits"]))
+    assert tfo.rel_error(tfo.from_f16_bits(y), ref) < tfo.Tolerance.quantInt4 * 4
+    # stage boundaries: gate/up are fp16-rounded GEMV outputs, act = gelu_mul_fp16 of those
+    assert tfo.rel_error(tfo.from_f16_bits(sg), tfo.int4_gemv_ref(*c["gate"], tfo.from_f16_bits(c["x_bits"]))) < tfo.Tolerance.fp16Reduction
+    want_act = tfo.from_f16_bits(tfo.k_gelu_mul_fp16(sg, su))
+    assert np.max(np.abs(tfo.from_f16_bits(sa) - want_act)) <= 1e-3
+
+
+def test_shared_expert_production_shape_fused_gate_up():
+    # shared expert of the production model: gate/up 2112 x 2816, down 2816 x 2112
+    d, f = 2816, 2112
+    c = dict(d=d, f=f, x_bits=refcases.normal_f16(d, 0x5E), gate=refcases.synthetic_int4(f, d, 0x5E, "g"),
+             up=refcases.synthetic_int4(f, d, 0x5E, "u"), down=refcases.synthetic_int4(d, f, 0x5E, "d"))
+    rc, y, (sg, su, sa) = run_shared(c)
+    assert rc == tfk.TF_OK
+    x = tfo.from_f16_bits(c["x_bits"])
+    g_ref, u_ref = tfo.int4_gemv_ref(*c["gate"], x, threads=8), tfo.int4_gemv_ref(*c["up"], x, threads=8)
+    assert tfo.rel_error(tfo.from_f16_bits(sg), g_ref) < tfo.Tolerance.fp16Reduction
+    assert tfo.rel_error(tfo.from_f16_bits(su), u_ref) < tfo.Tolerance.fp16Reduction
+    want_act = tfo.from_f16_bits(tfo.k_gelu_mul_fp16(sg, su))
+    assert tfo.rel_error(tfo.from_f16_bits(sa), want_act) < 2e-3
+    y_ref = tfo.int4_gemv_ref(*c["down"], tfo.from_f16_bits(sa), threads=8)
+    assert tfo.rel_error(tfo.from_f16_bits(y), y_ref) < tfo.Tolerance.fp16Reduction
+    full_ref = tfo.shared_expert_ref(c["gate"], c["up"], c["down"], x, threads=8)
+    assert tfo.rel_error(tfo.from_f16_bits(y), full_ref) < tfo.Tolerance.fp16ChainedReduction
+
+
+def test_shared_expert_errors():
+    c = refcases.shared_expert_case()
+    assert run_shared(c, weight_bits=3)[0] == tfk.TF_ERR_UNSUPPORTED_BITS        # SharedExpertInt4.swift:110
+    assert run_shared(c, weight_bits=8)[0] == tfk.TF_ERR_UNSUPPORTED_BITS
+    assert run_shared(c, scratch_halves=c["f"] - 1)[0] == tfk.TF_ERR_SCRATCH_TOO_SMALL   # :46-50
+    bad = dict(c)
+    bad["down"] = c["gate"]
+    k = ctx()
+    t = {n: [dev(a) for a in c[n]] for n in ("gate", "up")}
+    x, y, s = dev(c["x_bits"]), zeros_bytes(256), zeros_bytes(128)
+    rc = k.shared_expert_int4(x, _proj(*t["gate"], 64, 128), _proj(*t["up"], 64, 128), _proj(*t["gate"], 64, 128), y, s, s, s, raise_on_error=False)
+    assert rc == tfk.TF_ERR_DIMENSION_MISMATCH                                    # :41-45

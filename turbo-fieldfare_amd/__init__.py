@@ -1,0 +1,253 @@
+"""ctypes binding of ``libtf_kernels.so`` — the C ABI declared in ``include/tf_kernels.h``.
+
+The product is the HIP library; this module only loads it and passes device pointers through.  PyTorch is used
+by callers for device memory and streams, never for arithmetic.  There is no CPU fallback: if the shared object is
+missing or cannot be loaded, importing :func:`load` raises.
+
+Load with ``importlib.import_module("turbo-fieldfare_amd")`` (the directory name is not a Python identifier).
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtf_kernels.so")
+
+TF_OK = 0
+TF_ERR_INVALID_ARGUMENT = -1
+TF_ERR_UNAVAILABLE = -2
+TF_ERR_DIMENSION_MISMATCH = -3
+TF_ERR_SCRATCH_TOO_SMALL = -4
+TF_ERR_UNSUPPORTED_BITS = -5
+TF_ERR_NO_DEVICE = -6
+TF_ERR_DEVICE = -7
+TF_ERR_OUT_OF_MEMORY = -8
+
+TF_BF16, TF_FP16, TF_FP32 = 0, 1, 2
+
+vp = C.c_void_p
+u64 = C.c_uint64
+u32 = C.c_uint32
+i32 = C.c_int32
+
+
+class ExpertOffsets(C.Structure):
+    """tf_expert_offsets (36 bytes)."""
+    _fields_ = [(n, C.c_uint32) for n in (
+        "gate_W_off", "gate_s_off", "gate_b_off", "up_W_off", "up_s_off", "up_b_off",
+        "down_W_off", "down_s_off", "down_b_off")]
+
+
+class Projection(C.Structure):
+    """tf_projection."""
+    _fields_ = [("weights", vp), ("weights_offset", u64), ("scales", vp), ("scales_offset", u64),
+                ("biases", vp), ("biases_offset", u64), ("rows", u32), ("cols", u32)]
+
+
+class RoutedBlobs(C.Structure):
+    """tf_routed_blobs."""
+    _fields_ = [("blobs", vp * 8), ("pool", vp), ("pool_stride", u64), ("indices", vp), ("num_experts", u32)]
+
+
+class PrefillPair(C.Structure):
+    """tf_prefill_pair (16 bytes)."""
+    _fields_ = [("token", u32), ("expert", u32), ("rank", u32), ("weight_bits_and_reserved", u32)]
+
+
+class TFError(RuntimeError):
+    def __init__(self, status: int, message: str):
+        super().__init__(f"tf_kernels status {status}: {message}")
+        self.status = status
+
+
+# every symbol include/tf_kernels.h declares; tests check that the library exports each one
+EXPORTS = {
+    "tf_ctx_create": (i32, [i32, C.POINTER(vp)]),
+    "tf_ctx_destroy": (None, [vp]),
+    "tf_stream_synchronize": (i32, [vp, vp]),
+    "tf_status_string": (C.c_char_p, [i32]),
+    "tf_last_error": (C.c_char_p, [vp]),
+    "tf_abi_version": (u32, []),
+    "tf_router_logits": (vp, [vp]),
+    "tf_dequantize_int4_affine": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32]),
+    "tf_dequantize_int8_affine": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32]),
+    "tf_dequant_int4_gemv": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32, i32]),
+    "tf_dequant_int8_gemv": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32, i32]),
+    "tf_gelu_mul_fp16": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32]),
+    "tf_rmsnorm_bf16w": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32, C.c_float]),
+    "tf_shared_expert_int4": (i32, [vp, vp, vp, u64, u64, C.POINTER(Projection), C.POINTER(Projection), C.POINTER(Projection),
+                                    vp, u64, u64, vp, u64, u64, vp, u64, u64, vp, u64, u64, u32, i32]),
+    "tf_router_gemma4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, vp, u64, vp, u64, vp, vp, u32, u32, u32]),
+    "tf_moe_phase1_gate_up_act": (i32, [vp, vp, C.POINTER(RoutedBlobs), C.POINTER(ExpertOffsets), vp, vp, u32, u32, u32, i32]),
+    "tf_moe_phase1_gate_up_act_subset": (i32, [vp, vp, C.POINTER(RoutedBlobs), C.POINTER(ExpertOffsets), vp, vp, vp, u32,
+                                               u32, u32, u32, i32]),
+    "tf_moe_phase2_down_reduce": (i32, [vp, vp, C.POINTER(RoutedBlobs), C.POINTER(ExpertOffsets), vp, vp, vp, vp, u32, u32,
+                                        u32, i32]),
+    "tf_moe_decode_step": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, vp, u64, vp, u64, vp, u64, u32, C.POINTER(ExpertOffsets),
+                                 vp, vp, vp, vp, vp, vp, u32, u32, u32, i32]),
+    "tf_lm_head_greedy_int4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u32, u32, C.c_float, i32]),
+    "tf_lm_head_logits_int4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, C.c_float,
+                                     i32, i32]),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the HIP library; raise if it has not been built (no fallback exists)."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python turbo-fieldfare_amd/build.py` (hipcc, gfx950). "
+            "There is no CPU fallback.")
+    try:
+        # callers allocate device memory and streams with PyTorch; loading it first makes both share one HIP runtime
+        # (the dynamic loader resolves libamdhip64.so.7 to whichever copy is already mapped)
+        import torch  # noqa: F401
+    except ImportError:
+        pass
+    lib = C.CDLL(LIB_PATH)
+    for name, (restype, argtypes) in EXPORTS.items():
+        fn = getattr(lib, name)      # AttributeError if the ABI and the library disagree
+        fn.restype = restype
+        fn.argtypes = argtypes
+    _lib = lib
+    return lib
+
+
+def _p(t):
+    """Device pointer of a torch tensor (or pass an int / None through)."""
+    if t is None:
+        return None
+    if isinstance(t, int):
+        return t
+    return t.data_ptr()
+
+
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+class Context:
+    """Owns a tf_ctx; methods mirror the C entry points one to one and raise TFError on a negative status."""
+
+    def __init__(self, device: int = 0):
+        self.lib = load()
+        h = vp()
+        rc = self.lib.tf_ctx_create(device, C.byref(h))
+        if rc != TF_OK:
+            raise TFError(rc, self.lib.tf_status_string(rc).decode())
+        self.handle = h
+
+    def close(self):
+        if getattr(self, "handle", None):
+            self.lib.tf_ctx_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    def check(self, rc: int) -> int:
+        if rc != TF_OK:
+            raise TFError(rc, self.lib.tf_last_error(self.handle).decode())
+        return rc
+
+    def last_error(self) -> str:
+        return self.lib.tf_last_error(self.handle).decode()
+
+    def synchronize(self, stream=None):
+        return self.check(self.lib.tf_stream_synchronize(self.handle, _stream() if stream is None else stream))
+
+    # ---- raw calls (return the status, do not raise) -----------------------------------------------------
+    def call(self, name: str, *args) -> int:
+        return getattr(self.lib, name)(self.handle, *args)
+
+    # ---- conveniences over torch tensors --------------------------------------------------------------------
+    def dequantize_int4(self, W, S, B, out, m, n, scale_dtype=TF_BF16, offsets=(0, 0, 0, 0), bits=4):
+        fn = self.lib.tf_dequantize_int4_affine if bits == 4 else self.lib.tf_dequantize_int8_affine
+        return self.check(fn(self.handle, _stream(), _p(W), offsets[0], _p(S), offsets[1], _p(B), offsets[2], _p(out),
+                             offsets[3], m, n, scale_dtype))
+
+    def dequant_int4_gemv(self, W, S, B, x, y, m, n, scale_dtype=TF_BF16, out_dtype=TF_FP16,
+                          offsets=(0, 0, 0, 0, 0), bits=4, raise_on_error=True):
+        fn = self.lib.tf_dequant_int4_gemv if bits == 4 else self.lib.tf_dequant_int8_gemv
+        rc = fn(self.handle, _stream(), _p(W), offsets[0], _p(S), offsets[1], _p(B), offsets[2], _p(x), offsets[3],
+                _p(y), offsets[4], m, n, scale_dtype, out_dtype)
+        return self.check(rc) if raise_on_error else rc
+
+    def gelu_mul_fp16(self, gate, up, out, count):
+        return self.check(self.lib.tf_gelu_mul_fp16(self.handle, _stream(), _p(gate), 0, _p(up), 0, _p(out), 0, count))
+
+    def rmsnorm_bf16w(self, x, w, out, d, eps, x_offset=0):
+        return self.check(self.lib.tf_rmsnorm_bf16w(self.handle, _stream(), _p(x), x_offset, _p(w), 0, _p(out), 0, d, eps))
+
+    def router_gemma4(self, W, S, B, hidden, eff, per_expert, out_idx, out_w, num_experts, d, top_k=8, raise_on_error=True):
+        rc = self.lib.tf_router_gemma4(self.handle, _stream(), _p(W), 0, _p(S), 0, _p(B), 0, _p(hidden), _p(eff), 0,
+                                       _p(per_expert), 0, _p(out_idx), _p(out_w), num_experts, d, top_k)
+        return self.check(rc) if raise_on_error else rc
+
+    def router_logits_ptr(self) -> int:
+        return int(self.lib.tf_router_logits(self.handle))
+
+    @staticmethod
+    def routed_from_pointers(ptrs) -> RoutedBlobs:
+        r = RoutedBlobs()
+        for i, p in enumerate(ptrs):
+            r.blobs[i] = p
+        return r
+
+    @staticmethod
+    def routed_from_pool(pool, stride: int, indices, num_experts: int) -> RoutedBlobs:
+        r = RoutedBlobs()
+        r.pool = _p(pool)
+        r.pool_stride = stride
+        r.indices = _p(indices)
+        r.num_experts = num_experts
+        return r
+
+    def moe_phase1(self, routed: RoutedBlobs, off: ExpertOffsets, x, acts, d, f, top_k=8, scale_dtype=TF_BF16,
+                   active_slots=None, active_count=0, raise_on_error=True):
+        if active_slots is None:
+            rc = self.lib.tf_moe_phase1_gate_up_act(self.handle, _stream(), C.byref(routed), C.byref(off), _p(x), _p(acts),
+                                                    d, f, top_k, scale_dtype)
+        else:
+            rc = self.lib.tf_moe_phase1_gate_up_act_subset(self.handle, _stream(), C.byref(routed), C.byref(off), _p(x),
+                                                           _p(acts), _p(active_slots), active_count, d, f, top_k, scale_dtype)
+        return self.check(rc) if raise_on_error else rc
+
+    def moe_phase2(self, routed: RoutedBlobs, off: ExpertOffsets, acts, routing_w, residual, y, d, f, top_k=8,
+                   scale_dtype=TF_BF16, raise_on_error=True):
+        rc = self.lib.tf_moe_phase2_down_reduce(self.handle, _stream(), C.byref(routed), C.byref(off), _p(acts), _p(routing_w),
+                                                _p(residual), _p(y), d, f, top_k, scale_dtype)
+        return self.check(rc) if raise_on_error else rc
+
+    def shared_expert_int4(self, x, gate: Projection, up: Projection, down: Projection, y, sg, su, sa, weight_bits=4,
+                           scale_dtype=TF_BF16, raise_on_error=True, lengths=None):
+        def nbytes(t):
+            return t.numel() * t.element_size()
+        ln = lengths or (nbytes(x), nbytes(y), nbytes(sg), nbytes(su), nbytes(sa))
+        rc = self.lib.tf_shared_expert_int4(self.handle, _stream(), _p(x), 0, ln[0], C.byref(gate), C.byref(up), C.byref(down),
+                                            _p(y), 0, ln[1], _p(sg), 0, ln[2], _p(su), 0, ln[3], _p(sa), 0, ln[4],
+                                            weight_bits, scale_dtype)
+        return self.check(rc) if raise_on_error else rc
+
+    def lm_head_greedy(self, hidden, norm_w, W, S, B, out_token, d, vocab, eps=1e-6, scale_dtype=TF_BF16,
+                       hidden_offset=0, weights_offset=0, raise_on_error=True):
+        rc = self.lib.tf_lm_head_greedy_int4(self.handle, _stream(), _p(hidden), hidden_offset, _p(norm_w), 0, _p(W),
+                                             weights_offset, _p(S), 0, _p(B), 0, _p(out_token), d, vocab, eps, scale_dtype)
+        return self.check(rc) if raise_on_error else rc
+
+    def lm_head_logits(self, hidden, norm_w, W, S, B, logits, d, vocab, eps=1e-6, scale_dtype=TF_BF16, out_dtype=TF_FP16):
+        return self.check(self.lib.tf_lm_head_logits_int4(self.handle, _stream(), _p(hidden), 0, _p(norm_w), 0, _p(W), 0,
+                                                          _p(S), 0, _p(B), 0, _p(logits), 0, d, vocab, eps, scale_dtype, out_dtype))
+
+
+def projection(W, S, B, rows: int, cols: int, offsets=(0, 0, 0)) -> Projection:
+    return Projection(_p(W), offsets[0], _p(S), offsets[1], _p(B), offsets[2], rows, cols)

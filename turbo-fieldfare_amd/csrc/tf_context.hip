@@ -1,0 +1,71 @@
+// Context lifetime, error strings and stream synchronisation of the C ABI.
+#include "tf_context.hpp"
+
+#include <new>
+
+using namespace tfk;
+
+extern "C" {
+
+uint32_t tf_abi_version(void) { return 1u; }
+
+const char *tf_status_string(int32_t status) {
+    switch (status) {
+        case TF_OK: return "ok";
+        case TF_ERR_INVALID_ARGUMENT: return "invalid argument";
+        case TF_ERR_UNAVAILABLE: return "unavailable for this shape or alignment";
+        case TF_ERR_DIMENSION_MISMATCH: return "dimension mismatch";
+        case TF_ERR_SCRATCH_TOO_SMALL: return "scratch too small";
+        case TF_ERR_UNSUPPORTED_BITS: return "unsupported weight bits";
+        case TF_ERR_NO_DEVICE: return "no device";
+        case TF_ERR_DEVICE: return "device error";
+        case TF_ERR_OUT_OF_MEMORY: return "out of device memory";
+        default: return "unknown status";
+    }
+}
+
+const char *tf_last_error(const tf_ctx *ctx) { return ctx ? ctx->last_error : "null context"; }
+
+int32_t tf_ctx_create(int32_t device, tf_ctx **out_ctx) {
+    if (!out_ctx) return TF_ERR_INVALID_ARGUMENT;
+    *out_ctx = nullptr;
+    int count = 0;
+    if (hipGetDeviceCount(&count) != hipSuccess || count <= 0 || device < 0 || device >= count) return TF_ERR_NO_DEVICE;
+    if (hipSetDevice(device) != hipSuccess) return TF_ERR_NO_DEVICE;
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, device) != hipSuccess) return TF_ERR_NO_DEVICE;
+    tf_ctx *ctx = new (std::nothrow) tf_ctx();
+    if (!ctx) return TF_ERR_OUT_OF_MEMORY;
+    ctx->device = device;
+    ctx->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    // 256 logits + one uint32 ticket counter (must start at 0; the router kernel leaves it at 0)
+    bool ok = hipMalloc(&ctx->router_logits, 264 * sizeof(float)) == hipSuccess;
+    ok = ok && hipMemset(ctx->router_logits, 0, 264 * sizeof(float)) == hipSuccess;
+    ok = ok && hipMalloc(&ctx->head_x_normed, kMaxHeadD * 2) == hipSuccess;
+    ok = ok && hipMalloc(&ctx->head_summaries, (size_t)kMaxHeadWaves * 2 * sizeof(float)) == hipSuccess;
+    if (!ok) {
+        tf_ctx_destroy(ctx);
+        return TF_ERR_OUT_OF_MEMORY;
+    }
+    *out_ctx = ctx;
+    return TF_OK;
+}
+
+void tf_ctx_destroy(tf_ctx *ctx) {
+    if (!ctx) return;
+    if (ctx->router_logits) (void)hipFree(ctx->router_logits);
+    if (ctx->head_x_normed) (void)hipFree(ctx->head_x_normed);
+    if (ctx->head_summaries) (void)hipFree(ctx->head_summaries);
+    if (ctx->head_logits) (void)hipFree(ctx->head_logits);
+    delete ctx;
+}
+
+int32_t tf_stream_synchronize(tf_ctx *ctx, tf_stream stream) {
+    const hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "stream synchronize: %s", hipGetErrorString(e));
+    return TF_OK;
+}
+
+const float *tf_router_logits(const tf_ctx *ctx) { return ctx ? ctx->router_logits : nullptr; }
+
+}  // extern "C"

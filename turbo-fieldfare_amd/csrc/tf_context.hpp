@@ -1,0 +1,54 @@
+// Host-side context shared by the C ABI entry points (not part of the public header).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdarg.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/tf_kernels.h"
+
+struct tf_ctx {
+    int device = 0;
+    int num_cus = 0;
+    // wrapper-owned scratch, as the reference's kernel classes own theirs
+    float *router_logits = nullptr;     // 256 floats (MoE.swift:92-99)
+    void *head_x_normed = nullptr;      // kMaxHeadD halves (LMHeadChainInt4.swift:38-51)
+    float *head_summaries = nullptr;    // kMaxHeadWaves x {value, index bits}
+    float *head_logits = nullptr;       // lazily sized fp32 logits for the unaligned lm_head path
+    size_t head_logits_count = 0;
+    char last_error[512] = {0};
+};
+
+namespace tfk {
+
+constexpr uint32_t kMaxHeadD = 16384;
+constexpr uint32_t kMaxHeadWaves = 16384;
+
+inline int32_t fail(tf_ctx *ctx, int32_t status, const char *fmt, ...) {
+    if (ctx) {
+        va_list ap;
+        va_start(ap, fmt);
+        vsnprintf(ctx->last_error, sizeof(ctx->last_error), fmt, ap);
+        va_end(ap);
+    }
+    return status;
+}
+
+inline int32_t check_launch(tf_ctx *ctx, const char *what) {
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "%s: %s", what, hipGetErrorString(e));
+    return TF_OK;
+}
+
+inline const uint8_t *at(const void *base, uint64_t off) { return static_cast<const uint8_t *>(base) + off; }
+inline uint8_t *at(void *base, uint64_t off) { return static_cast<uint8_t *>(base) + off; }
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline bool aligned(const void *p, unsigned a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1u)) == 0; }
+
+}  // namespace tfk
+
+#define TF_REQUIRE(ctx, cond, status, ...) \
+    do {                                    \
+        if (!(cond)) return tfk::fail((ctx), (status), __VA_ARGS__); \
+    } while (0)

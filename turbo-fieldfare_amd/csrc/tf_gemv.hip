@@ -1,0 +1,347 @@
+// Affine int4/int8 dequantization and GEMV for gfx950, plus the two small primitives on the same path
+// (gelu_mul_fp16, rmsnorm_bf16w).
+#include "tf_gemv_kernels.hpp"
+
+using namespace tfk;
+
+namespace {
+
+// ------------------------------------------------------------------------------------------------ dequantize
+// out[r, c] = float(q) * scale + bias, bit-exact with the CPU statement: the product q*scale is exact in fp32
+// (<= 8 bits x <= 11 bits), so a fused or an unfused multiply-add round identically.
+template <int BITS, int SD>
+__global__ __launch_bounds__(256) void dequantize_kernel(const uint8_t *w, const uint16_t *s, const uint16_t *b,
+                                                         float *out, uint32_t m, uint32_t n) {
+    const uint64_t total_pairs = (uint64_t)m * (n >> 1);
+    const uint32_t groups = n >> 6;
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total_pairs;
+         i += (uint64_t)gridDim.x * blockDim.x) {
+        const uint64_t r = i / (n >> 1);
+        const uint32_t c = (uint32_t)(i - r * (n >> 1)) * 2;
+        const float scale = sb_to_f32<SD>(s[r * groups + (c >> 6)]);
+        const float bias = sb_to_f32<SD>(b[r * groups + (c >> 6)]);
+        uint32_t q0, q1;
+        if constexpr (BITS == 4) {
+            const uint8_t byte = w[i];
+            q0 = byte & 0x0Fu;
+            q1 = byte >> 4;
+        } else {
+            q0 = w[r * n + c];
+            q1 = w[r * n + c + 1];
+        }
+        out[r * n + c] = (float)q0 * scale + bias;
+        out[r * n + c + 1] = (float)q1 * scale + bias;
+    }
+}
+
+template <typename OutT>
+__device__ __forceinline__ void store_out(OutT *y, long row, float v) {
+    y[row] = (OutT)v;
+}
+
+// ------------------------------------------------------------------------------------------------ GEMV kernels
+template <int RT, int NP, int SD, typename OutT>
+__global__ __launch_bounds__(256) void gemv4_long_kernel(const uint8_t *W, const uint16_t *S, const uint16_t *B,
+                                                         const half_t *x, OutT *y, long m, int k) {
+    const int lane = threadIdx.x & 63;
+    const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
+    const long ntiles = (m + RT - 1) / RT;
+    if (wave >= ntiles) return;
+    const int groups = k >> 6;
+    const size_t tile_bytes = (size_t)RT * (k >> 1);
+
+    LongRows<RT, NP> lr;
+    lr.init(x, k, lane);
+    typename LongRows<RT, NP>::Tile cur, nxt;
+    long tile = wave;
+    lr.load(cur, W + tile * tile_bytes, S + tile * RT * groups, B + tile * RT * groups, (int)min((long)RT, m - tile * RT), lane);
+    for (;;) {
+        const long next = tile + nwaves;
+        const bool has_next = next < ntiles;
+        if (has_next)
+            lr.load(nxt, W + next * tile_bytes, S + next * RT * groups, B + next * RT * groups,
+                    (int)min((long)RT, m - next * RT), lane);
+        float out[RT];
+        lr.template reduce<SD>(cur, out);
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < RT; ++r)
+                if (tile * RT + r < m) store_out(y, tile * RT + r, out[r]);
+        }
+        if (!has_next) break;
+        cur = nxt;
+        tile = next;
+    }
+}
+
+// K <= 1024: each wave covers 2 * NPASS consecutive rows, one row per half-wave per pass.
+template <int NPASS, int SD, typename OutT>
+__global__ __launch_bounds__(256) void gemv4_short_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B,
+                                                          const half_t *x, OutT *y, long m, int k) {
+    const int lane = threadIdx.x & 63;
+    const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const long row0 = wave * (2 * NPASS);
+    if (row0 >= m) return;
+    ShortRows sr;
+    sr.init(x, k, lane);
+    ShortRows::Pair t[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) sr.load(t[p], W, S, B, row0 + 2 * p, m, k);
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+        float lo, hi;
+        sr.template reduce<SD>(t[p], lo, hi);
+        if (lane == 0) {
+            if (row0 + 2 * p < m) store_out(y, row0 + 2 * p, lo);
+            if (row0 + 2 * p + 1 < m) store_out(y, row0 + 2 * p + 1, hi);
+        }
+    }
+}
+
+template <int BITS, int SD, typename OutT>
+__global__ __launch_bounds__(256) void gemv_generic_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B,
+                                                           const half_t *x, OutT *y, long m, int k) {
+    const int lane = threadIdx.x & 63;
+    const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
+    const int groups = k >> 6;
+    const size_t row_bytes = BITS == 4 ? (size_t)(k >> 1) : (size_t)k;
+    for (long row = wave; row < m; row += nwaves) {
+        float v;
+        if constexpr (BITS == 4)
+            v = generic_row_dot<SD>(W + row * row_bytes, S + (size_t)row * groups * 2, B + (size_t)row * groups * 2, x, k, lane);
+        else
+            v = generic_row_dot8<SD>(W + row * row_bytes, S + (size_t)row * groups * 2, B + (size_t)row * groups * 2, x, k, lane);
+        if (lane == 0) store_out(y, row, v);
+    }
+}
+
+// int8, 16-byte aligned rows and activations: lanes stride over 16-byte chunks (16 elements, a quarter group).
+template <int SD, typename OutT>
+__global__ __launch_bounds__(256) void gemv8_aligned_kernel(const uint8_t *W, const uint16_t *S, const uint16_t *B,
+                                                            const half_t *x, OutT *y, long m, int k) {
+    const int lane = threadIdx.x & 63;
+    const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
+    const int groups = k >> 6;
+    const int chunks = k >> 4;
+    for (long row = wave; row < m; row += nwaves) {
+        float acc = 0.0f;
+        for (int c = lane; c < chunks; c += kWave) {
+            const u32x4 w = load16(W + (size_t)row * k + (size_t)c * 16);
+            const u32x4 xa = load16(x + c * 16), xb = load16(x + c * 16 + 8);
+            const float s = sb_to_f32<SD>(S[(size_t)row * groups + (c >> 2)]);
+            const float b = sb_to_f32<SD>(B[(size_t)row * groups + (c >> 2)]);
+            float dot = 0.0f, sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t xw = i < 8 ? xa[i >> 1] : xb[(i - 8) >> 1];
+                const float xv = (float)__builtin_bit_cast(half_t, (uint16_t)((i & 1) ? (xw >> 16) : (xw & 0xFFFFu)));
+                const float q = (float)((w[i >> 2] >> (8 * (i & 3))) & 0xFFu);
+                dot = fmaf(q, xv, dot);
+                sum += xv;
+            }
+            acc = fmaf(s, dot, acc);
+            acc = fmaf(b, sum, acc);
+        }
+        const float v = wave_sum(acc);
+        if (lane == 0) store_out(y, row, v);
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ primitives
+__global__ __launch_bounds__(256) void gelu_mul_kernel(const half_t *gate, const half_t *up, half_t *out, uint32_t count) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= count) return;
+    out[i] = (half_t)(gelu_tanh((float)gate[i]) * (float)up[i]);
+}
+
+__global__ __launch_bounds__(256) void rmsnorm_bf16w_kernel(const half_t *x, const uint16_t *weight, half_t *out, uint32_t d, float eps) {
+    __shared__ float partial[4];
+    const float inv = block_rms_inv(x, d, eps, partial);
+    for (uint32_t i = threadIdx.x; i < d; i += blockDim.x)
+        out[i] = (half_t)((float)x[i] * inv * bf16_to_f32(weight[i]));
+}
+
+template <int BITS>
+int32_t dequantize_entry(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t wo, const void *scales, uint64_t so,
+                         const void *biases, uint64_t bo, void *out, uint64_t oo, uint32_t m, uint32_t n, tf_dtype sd) {
+    TF_REQUIRE(ctx, ctx && weights && scales && biases && out, TF_ERR_INVALID_ARGUMENT, "dequantize: null argument");
+    TF_REQUIRE(ctx, m > 0 && n > 0 && n % TF_GROUP_SIZE == 0, TF_ERR_INVALID_ARGUMENT, "dequantize: n=%u must be a positive multiple of 64", n);
+    TF_REQUIRE(ctx, so % 2 == 0 && bo % 2 == 0 && oo % 4 == 0, TF_ERR_INVALID_ARGUMENT, "dequantize: misaligned offset");
+    TF_REQUIRE(ctx, sd == TF_BF16 || sd == TF_FP16, TF_ERR_INVALID_ARGUMENT, "dequantize: scale dtype must be bf16 or fp16");
+    const uint8_t *w = at(weights, wo);
+    const uint16_t *s = reinterpret_cast<const uint16_t *>(at(scales, so));
+    const uint16_t *b = reinterpret_cast<const uint16_t *>(at(biases, bo));
+    TF_REQUIRE(ctx, aligned(s, 2) && aligned(b, 2) && aligned(at(out, oo), 4), TF_ERR_INVALID_ARGUMENT, "dequantize: misaligned pointer");
+    float *o = reinterpret_cast<float *>(at(out, oo));
+    const uint64_t pairs = (uint64_t)m * (n / 2);
+    const uint32_t grid = (uint32_t)std::min<uint64_t>((pairs + 255) / 256, (uint64_t)ctx->num_cus * 32);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (sd == TF_BF16) hipLaunchKernelGGL((dequantize_kernel<BITS, 0>), dim3(grid), dim3(256), 0, st, w, s, b, o, m, n);
+    else hipLaunchKernelGGL((dequantize_kernel<BITS, 1>), dim3(grid), dim3(256), 0, st, w, s, b, o, m, n);
+    return check_launch(ctx, "dequantize");
+}
+
+}  // namespace
+
+namespace tfk {
+
+// Shared by tf_dequant_int4_gemv, the shared expert and the logits head.
+template <int SD, typename OutT>
+static int32_t launch_gemv4_typed(tf_ctx *ctx, hipStream_t st, const uint8_t *w, const uint8_t *s, const uint8_t *b,
+                                  const half_t *x, OutT *y, uint32_t m, uint32_t n) {
+    const bool fast = aligned16(w) && aligned16(x);
+    if (fast && n <= 1024) {
+        constexpr int NPASS = 4;
+        const long waves = ((long)m + 2 * NPASS - 1) / (2 * NPASS);
+        const uint32_t grid = (uint32_t)((waves + 3) / 4);
+        hipLaunchKernelGGL((gemv4_short_kernel<NPASS, SD, OutT>), dim3(grid), dim3(256), 0, st, w, s, b, x, y, (long)m, (int)n);
+        return check_launch(ctx, "gemv4_short");
+    }
+    const LongPlan plan = plan_long_rows((int)n);
+    if (fast && plan.rt > 0) {
+        const long ntiles = ((long)m + plan.rt - 1) / plan.rt;
+        const long max_blocks = (long)ctx->num_cus * kLongBlocksPerCU;
+        const uint32_t grid = (uint32_t)std::max<long>(1, std::min<long>((ntiles + 3) / 4, max_blocks));
+        const uint16_t *s16 = reinterpret_cast<const uint16_t *>(s);
+        const uint16_t *b16 = reinterpret_cast<const uint16_t *>(b);
+#define TF_LONG_CASE(RT_, NP_)                                                                                          \
+    if (plan.rt == RT_ && plan.np == NP_) {                                                                             \
+        hipLaunchKernelGGL((gemv4_long_kernel<RT_, NP_, SD, OutT>), dim3(grid), dim3(256), 0, st, w, s16, b16, x, y,    \
+                           (long)m, (int)n);                                                                            \
+        return check_launch(ctx, "gemv4_long");                                                                         \
+    }
+        TF_LONG_CASE(1, 1) TF_LONG_CASE(1, 2) TF_LONG_CASE(1, 3) TF_LONG_CASE(1, 4)
+        TF_LONG_CASE(2, 1) TF_LONG_CASE(2, 2) TF_LONG_CASE(2, 3) TF_LONG_CASE(2, 4)
+        TF_LONG_CASE(4, 1) TF_LONG_CASE(4, 2) TF_LONG_CASE(4, 3) TF_LONG_CASE(4, 4)
+#undef TF_LONG_CASE
+    }
+    const uint32_t grid = (uint32_t)std::min<long>(((long)m + 3) / 4, (long)ctx->num_cus * 16);
+    hipLaunchKernelGGL((gemv_generic_kernel<4, SD, OutT>), dim3(grid), dim3(256), 0, st, w, s, b, x, y, (long)m, (int)n);
+    return check_launch(ctx, "gemv4_generic");
+}
+
+int32_t launch_gemv4(tf_ctx *ctx, hipStream_t st, const uint8_t *w, const uint8_t *s, const uint8_t *b, const void *x,
+                     void *y, uint32_t m, uint32_t n, tf_dtype sd, tf_dtype od) {
+    const half_t *xh = static_cast<const half_t *>(x);
+    if (sd == TF_BF16) {
+        if (od == TF_FP16) return launch_gemv4_typed<0, half_t>(ctx, st, w, s, b, xh, static_cast<half_t *>(y), m, n);
+        return launch_gemv4_typed<0, float>(ctx, st, w, s, b, xh, static_cast<float *>(y), m, n);
+    }
+    if (od == TF_FP16) return launch_gemv4_typed<1, half_t>(ctx, st, w, s, b, xh, static_cast<half_t *>(y), m, n);
+    return launch_gemv4_typed<1, float>(ctx, st, w, s, b, xh, static_cast<float *>(y), m, n);
+}
+
+int32_t launch_rmsnorm_bf16w(tf_ctx *ctx, hipStream_t st, const void *x, const void *w, void *out, uint32_t d, float eps) {
+    hipLaunchKernelGGL(rmsnorm_bf16w_kernel, dim3(1), dim3(256), 0, st, static_cast<const half_t *>(x),
+                       static_cast<const uint16_t *>(w), static_cast<half_t *>(out), d, eps);
+    return check_launch(ctx, "rmsnorm_bf16w");
+}
+
+int32_t launch_gelu_mul(tf_ctx *ctx, hipStream_t st, const void *gate, const void *up, void *out, uint32_t count) {
+    hipLaunchKernelGGL(gelu_mul_kernel, dim3((count + 255) / 256), dim3(256), 0, st, static_cast<const half_t *>(gate),
+                       static_cast<const half_t *>(up), static_cast<half_t *>(out), count);
+    return check_launch(ctx, "gelu_mul_fp16");
+}
+
+int32_t validate_gemv(tf_ctx *ctx, const char *who, const void *weights, uint64_t wo, const void *scales, uint64_t so,
+                      const void *biases, uint64_t bo, const void *x, uint64_t xo, const void *y, uint64_t yo,
+                      uint32_t m, uint32_t n, tf_dtype sd, tf_dtype od, unsigned weights_align) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "%s: null context", who);
+    TF_REQUIRE(ctx, weights && scales && biases && x && y, TF_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    TF_REQUIRE(ctx, m > 0, TF_ERR_INVALID_ARGUMENT, "%s: m must be positive", who);
+    TF_REQUIRE(ctx, n > 0 && n % TF_GROUP_SIZE == 0, TF_ERR_INVALID_ARGUMENT, "%s: N must be a multiple of 64, got %u", who, n);
+    TF_REQUIRE(ctx, aligned(at(weights, wo), weights_align), TF_ERR_INVALID_ARGUMENT, "%s needs a %u-aligned weightsOffset, got %llu", who,
+               weights_align, (unsigned long long)wo);
+    TF_REQUIRE(ctx, aligned(at(scales, so), 2) && aligned(at(biases, bo), 2) && aligned(at(x, xo), 2), TF_ERR_INVALID_ARGUMENT,
+               "%s: scales, biases and x must be 2-byte aligned", who);
+    TF_REQUIRE(ctx, sd == TF_BF16 || sd == TF_FP16, TF_ERR_INVALID_ARGUMENT, "%s: scale dtype must be bf16 or fp16", who);
+    TF_REQUIRE(ctx, od == TF_FP16 || od == TF_FP32, TF_ERR_INVALID_ARGUMENT, "%s: output dtype must be fp16 or fp32", who);
+    TF_REQUIRE(ctx, aligned(at(y, yo), od == TF_FP16 ? 2 : 4), TF_ERR_INVALID_ARGUMENT, "%s: misaligned output", who);
+    return TF_OK;
+}
+
+}  // namespace tfk
+
+extern "C" {
+
+int32_t tf_dequantize_int4_affine(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset,
+                                  const void *scales, uint64_t scales_offset, const void *biases, uint64_t biases_offset,
+                                  void *out_f32, uint64_t out_offset, uint32_t m, uint32_t n, tf_dtype scale_dtype) {
+    return dequantize_entry<4>(ctx, stream, weights, weights_offset, scales, scales_offset, biases, biases_offset, out_f32,
+                               out_offset, m, n, scale_dtype);
+}
+
+int32_t tf_dequantize_int8_affine(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset,
+                                  const void *scales, uint64_t scales_offset, const void *biases, uint64_t biases_offset,
+                                  void *out_f32, uint64_t out_offset, uint32_t m, uint32_t n, tf_dtype scale_dtype) {
+    return dequantize_entry<8>(ctx, stream, weights, weights_offset, scales, scales_offset, biases, biases_offset, out_f32,
+                               out_offset, m, n, scale_dtype);
+}
+
+int32_t tf_dequant_int4_gemv(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset, const void *scales,
+                             uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *x,
+                             uint64_t x_offset, void *y, uint64_t y_offset, uint32_t m, uint32_t n, tf_dtype scale_dtype,
+                             tf_dtype out_dtype) {
+    const int32_t rc = validate_gemv(ctx, "dequant_int4_gemv", weights, weights_offset, scales, scales_offset, biases,
+                                     biases_offset, x, x_offset, y, y_offset, m, n, scale_dtype, out_dtype, 2);
+    if (rc != TF_OK) return rc;
+    return launch_gemv4(ctx, static_cast<hipStream_t>(stream), at(weights, weights_offset), at(scales, scales_offset),
+                        at(biases, biases_offset), at(x, x_offset), at(y, y_offset), m, n, scale_dtype, out_dtype);
+}
+
+int32_t tf_dequant_int8_gemv(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset, const void *scales,
+                             uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *x,
+                             uint64_t x_offset, void *y, uint64_t y_offset, uint32_t m, uint32_t n, tf_dtype scale_dtype,
+                             tf_dtype out_dtype) {
+    const int32_t rc = validate_gemv(ctx, "dequant_int8_gemv", weights, weights_offset, scales, scales_offset, biases,
+                                     biases_offset, x, x_offset, y, y_offset, m, n, scale_dtype, out_dtype, 1);
+    if (rc != TF_OK) return rc;
+    const uint8_t *w = at(weights, weights_offset);
+    const uint8_t *s = at(scales, scales_offset);
+    const uint8_t *b = at(biases, biases_offset);
+    const half_t *xh = reinterpret_cast<const half_t *>(at(x, x_offset));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint32_t grid = (uint32_t)std::min<long>(((long)m + 3) / 4, (long)ctx->num_cus * 16);
+    const bool fast = aligned16(w) && aligned16(xh);
+#define TF_GEMV8(SD_, OUT_)                                                                                             \
+    do {                                                                                                                \
+        OUT_ *yo = reinterpret_cast<OUT_ *>(at(y, y_offset));                                                           \
+        if (fast)                                                                                                       \
+            hipLaunchKernelGGL((gemv8_aligned_kernel<SD_, OUT_>), dim3(grid), dim3(256), 0, st, w,                      \
+                               reinterpret_cast<const uint16_t *>(s), reinterpret_cast<const uint16_t *>(b), xh, yo,    \
+                               (long)m, (int)n);                                                                        \
+        else                                                                                                            \
+            hipLaunchKernelGGL((gemv_generic_kernel<8, SD_, OUT_>), dim3(grid), dim3(256), 0, st, w, s, b, xh, yo,      \
+                               (long)m, (int)n);                                                                        \
+    } while (0)
+    if (scale_dtype == TF_BF16) {
+        if (out_dtype == TF_FP16) TF_GEMV8(0, half_t); else TF_GEMV8(0, float);
+    } else {
+        if (out_dtype == TF_FP16) TF_GEMV8(1, half_t); else TF_GEMV8(1, float);
+    }
+#undef TF_GEMV8
+    return check_launch(ctx, "gemv8");
+}
+
+int32_t tf_gelu_mul_fp16(tf_ctx *ctx, tf_stream stream, const void *gate, uint64_t gate_offset, const void *up,
+                         uint64_t up_offset, void *out, uint64_t out_offset, uint32_t count) {
+    TF_REQUIRE(ctx, ctx && gate && up && out, TF_ERR_INVALID_ARGUMENT, "gelu_mul_fp16: null argument");
+    TF_REQUIRE(ctx, gate_offset % 2 == 0 && up_offset % 2 == 0 && out_offset % 2 == 0, TF_ERR_INVALID_ARGUMENT,
+               "gelu_mul_fp16: offsets must be 2-byte aligned");
+    if (count == 0) return TF_OK;
+    return launch_gelu_mul(ctx, static_cast<hipStream_t>(stream), at(gate, gate_offset), at(up, up_offset), at(out, out_offset), count);
+}
+
+int32_t tf_rmsnorm_bf16w(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, const void *weight,
+                         uint64_t weight_offset, void *out, uint64_t out_offset, uint32_t d, float eps) {
+    TF_REQUIRE(ctx, ctx && x && weight && out, TF_ERR_INVALID_ARGUMENT, "rmsnorm_bf16w: null argument");
+    TF_REQUIRE(ctx, d > 0, TF_ERR_INVALID_ARGUMENT, "rmsnorm_bf16w: d must be positive");
+    TF_REQUIRE(ctx, x_offset % 2 == 0 && weight_offset % 2 == 0 && out_offset % 2 == 0, TF_ERR_INVALID_ARGUMENT,
+               "rmsnorm_bf16w: offsets must be 2-byte aligned");
+    return launch_rmsnorm_bf16w(ctx, static_cast<hipStream_t>(stream), at(x, x_offset), at(weight, weight_offset), at(out, out_offset), d, eps);
+}
+
+}  // extern "C"

@@ -1,0 +1,214 @@
+// Tied int4 output head for gfx950: final RMSNorm -> vocab-sized int4 GEMV -> greedy argmax without materialising
+// logits, and the logits variant for samplers.
+#include "tf_gemv_kernels.hpp"
+
+using namespace tfk;
+
+namespace {
+
+struct Best {
+    float v;
+    uint32_t idx;
+};
+
+__device__ __forceinline__ void better(Best &b, float v, uint32_t idx) {
+    if (v > b.v || (v == b.v && idx < b.idx)) {
+        b.v = v;
+        b.idx = idx;
+    }
+}
+
+// Persistent row streamer: every wave walks tiles wave, wave + nwaves, ... of RT rows, keeps the best finite logit it
+// has seen (rows ascend within a wave, so a strict comparison keeps the lowest index among equals) and writes one
+// {value, index} summary.
+template <int RT, int NP, int SD>
+__global__ __launch_bounds__(256) void head_greedy_long_kernel(const uint8_t *W, const uint16_t *S, const uint16_t *B,
+                                                               const half_t *x, float *summaries, long v_rows, int k) {
+    const int lane = threadIdx.x & 63;
+    const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
+    const long ntiles = (v_rows + RT - 1) / RT;
+    if (wave >= ntiles) {
+        if (lane == 0) {
+            summaries[2 * wave] = -INFINITY;
+            summaries[2 * wave + 1] = __uint_as_float(0xFFFFFFFFu);
+        }
+        return;
+    }
+    const int groups = k >> 6;
+    const size_t tile_bytes = (size_t)RT * (k >> 1);
+    LongRows<RT, NP> lr;
+    typename LongRows<RT, NP>::Tile cur, nxt;
+    lr.init_map(k, lane);
+    long tile = wave;
+    lr.load(cur, W + tile * tile_bytes, S + tile * RT * groups, B + tile * RT * groups, (int)min((long)RT, v_rows - tile * RT), lane);
+    lr.init_x(x, lane);
+    Best best{-INFINITY, 0xFFFFFFFFu};
+    for (;;) {
+        const long next = tile + nwaves;
+        const bool has_next = next < ntiles;
+        if (has_next)
+            lr.load(nxt, W + next * tile_bytes, S + next * RT * groups, B + next * RT * groups,
+                    (int)min((long)RT, v_rows - next * RT), lane);
+        float out[RT];
+        lr.template reduce<SD>(cur, out);
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            const long row = tile * RT + r;
+            const float z = out[r];
+            if (row < v_rows && __builtin_isfinite(z) && z > best.v) {
+                best.v = z;
+                best.idx = (uint32_t)row;
+            }
+        }
+        if (!has_next) break;
+        cur = nxt;
+        tile = next;
+    }
+    if (lane == 0) {
+        summaries[2 * wave] = best.v;
+        summaries[2 * wave + 1] = __uint_as_float(best.idx);
+    }
+}
+
+// Fallback first stage: argmax summaries over an fp32 logits vector (one summary per block).
+__global__ __launch_bounds__(256) void logits_partial_argmax_kernel(const float *logits, float *summaries, long v_rows) {
+    __shared__ float sv[4];
+    __shared__ uint32_t si[4];
+    Best best{-INFINITY, 0xFFFFFFFFu};
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < v_rows; i += (long)gridDim.x * blockDim.x) {
+        const float z = logits[i];
+        if (__builtin_isfinite(z)) better(best, z, (uint32_t)i);
+    }
+    wave_best_pair(best.v, best.idx);
+    if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = best.v; si[threadIdx.x >> 6] = best.idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        Best b{sv[0], si[0]};
+        for (int w = 1; w < 4; ++w) better(b, sv[w], si[w]);
+        summaries[2 * blockIdx.x] = b.v;
+        summaries[2 * blockIdx.x + 1] = __uint_as_float(b.idx);
+    }
+}
+
+// Global argmax over the summaries: highest value, lowest index among equals, token 0 when nothing was finite
+// (lm_head_greedy_int4_rows_reduce, Metal/Sampling/logit.metal:740-787).
+__global__ __launch_bounds__(256) void head_reduce_kernel(const float *summaries, uint32_t *out_token, uint32_t count) {
+    __shared__ float sv[4];
+    __shared__ uint32_t si[4];
+    Best best{-INFINITY, 0xFFFFFFFFu};
+    for (uint32_t i = threadIdx.x; i < count; i += blockDim.x)
+        better(best, summaries[2 * i], __float_as_uint(summaries[2 * i + 1]));
+    wave_best_pair(best.v, best.idx);
+    if ((threadIdx.x & 63) == 0) { sv[threadIdx.x >> 6] = best.v; si[threadIdx.x >> 6] = best.idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        Best b{sv[0], si[0]};
+        for (int w = 1; w < 4; ++w) better(b, sv[w], si[w]);
+        out_token[0] = b.idx == 0xFFFFFFFFu ? 0u : b.idx;
+    }
+}
+
+int32_t validate_head(tf_ctx *ctx, const char *who, const void *hidden, uint64_t hidden_offset, const void *norm_weight,
+                      uint64_t norm_offset, const void *weights, uint64_t weights_offset, const void *scales,
+                      uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *out, uint32_t d,
+                      uint32_t vocab, tf_dtype sd) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "%s: null context", who);
+    TF_REQUIRE(ctx, hidden && norm_weight && weights && scales && biases && out, TF_ERR_INVALID_ARGUMENT, "%s: null buffer", who);
+    TF_REQUIRE(ctx, d > 0 && d <= kMaxHeadD, TF_ERR_INVALID_ARGUMENT, "%s: d=%u exceeds wrapper maxD=%u", who, d, kMaxHeadD);
+    TF_REQUIRE(ctx, vocab > 0, TF_ERR_INVALID_ARGUMENT, "%s: vocab must be positive", who);
+    TF_REQUIRE(ctx, d % TF_GROUP_SIZE == 0, TF_ERR_INVALID_ARGUMENT, "%s: d must be a multiple of 64", who);
+    TF_REQUIRE(ctx, aligned(at(weights, weights_offset), 2), TF_ERR_INVALID_ARGUMENT, "%s needs a 2-aligned weightsOffset", who);
+    TF_REQUIRE(ctx, aligned(at(hidden, hidden_offset), 2) && aligned(at(norm_weight, norm_offset), 2) &&
+                   aligned(at(scales, scales_offset), 2) && aligned(at(biases, biases_offset), 2),
+               TF_ERR_INVALID_ARGUMENT, "%s: misaligned operand", who);
+    TF_REQUIRE(ctx, sd == TF_BF16 || sd == TF_FP16, TF_ERR_INVALID_ARGUMENT, "%s: scale dtype must be bf16 or fp16", who);
+    return TF_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t tf_lm_head_greedy_int4(tf_ctx *ctx, tf_stream stream, const void *hidden, uint64_t hidden_offset, const void *norm_weight,
+                               uint64_t norm_offset, const void *weights, uint64_t weights_offset, const void *scales,
+                               uint64_t scales_offset, const void *biases, uint64_t biases_offset, void *out_token, uint32_t d,
+                               uint32_t vocab, float rms_eps, tf_dtype scale_dtype) {
+    int32_t rc = validate_head(ctx, "lm_head_greedy_int4", hidden, hidden_offset, norm_weight, norm_offset, weights, weights_offset,
+                               scales, scales_offset, biases, biases_offset, out_token, d, vocab, scale_dtype);
+    if (rc != TF_OK) return rc;
+    TF_REQUIRE(ctx, aligned(out_token, 4), TF_ERR_INVALID_ARGUMENT, "lm_head_greedy_int4: misaligned out_token");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    rc = launch_rmsnorm_bf16w(ctx, st, at(hidden, hidden_offset), at(norm_weight, norm_offset), ctx->head_x_normed, d, rms_eps);
+    if (rc != TF_OK) return rc;
+
+    const uint8_t *w = at(weights, weights_offset);
+    const uint8_t *s = at(scales, scales_offset);
+    const uint8_t *b = at(biases, biases_offset);
+    const half_t *xn = static_cast<const half_t *>(ctx->head_x_normed);
+    const LongPlan plan = plan_long_rows((int)d);
+    uint32_t n_summaries = 0;
+    if (aligned16(w) && d > 1024 && plan.rt > 0) {
+        const long ntiles = ((long)vocab + plan.rt - 1) / plan.rt;
+        const long max_blocks = std::min<long>((long)ctx->num_cus * kLongBlocksPerCU, kMaxHeadWaves / 4);
+        const uint32_t grid = (uint32_t)std::max<long>(1, std::min<long>((ntiles + 3) / 4, max_blocks));
+        n_summaries = grid * 4;
+        const uint16_t *s16 = reinterpret_cast<const uint16_t *>(s);
+        const uint16_t *b16 = reinterpret_cast<const uint16_t *>(b);
+        bool launched = false;
+#define TF_HEAD_CASE(RT_, NP_)                                                                                          \
+    if (!launched && plan.rt == RT_ && plan.np == NP_) {                                                                \
+        launched = true;                                                                                                \
+        if (scale_dtype == TF_BF16)                                                                                     \
+            hipLaunchKernelGGL((head_greedy_long_kernel<RT_, NP_, 0>), dim3(grid), dim3(256), 0, st, w, s16, b16, xn,   \
+                               ctx->head_summaries, (long)vocab, (int)d);                                               \
+        else                                                                                                            \
+            hipLaunchKernelGGL((head_greedy_long_kernel<RT_, NP_, 1>), dim3(grid), dim3(256), 0, st, w, s16, b16, xn,   \
+                               ctx->head_summaries, (long)vocab, (int)d);                                               \
+    }
+        TF_HEAD_CASE(1, 1) TF_HEAD_CASE(1, 2) TF_HEAD_CASE(1, 3) TF_HEAD_CASE(1, 4)
+        TF_HEAD_CASE(2, 1) TF_HEAD_CASE(2, 2) TF_HEAD_CASE(2, 3) TF_HEAD_CASE(2, 4)
+        TF_HEAD_CASE(4, 1) TF_HEAD_CASE(4, 2) TF_HEAD_CASE(4, 3) TF_HEAD_CASE(4, 4)
+#undef TF_HEAD_CASE
+        rc = check_launch(ctx, "lm_head_greedy rows");
+        if (rc != TF_OK) return rc;
+    } else {
+        // short or unaligned rows: fp32 logits into wrapper-owned scratch, then a two-stage argmax
+        if (ctx->head_logits_count < vocab) {
+            if (ctx->head_logits) (void)hipFree(ctx->head_logits);
+            ctx->head_logits = nullptr;
+            ctx->head_logits_count = 0;
+            if (hipMalloc(&ctx->head_logits, (size_t)vocab * sizeof(float)) != hipSuccess)
+                return fail(ctx, TF_ERR_OUT_OF_MEMORY, "lm_head_greedy_int4: cannot allocate %u logits", vocab);
+            ctx->head_logits_count = vocab;
+        }
+        rc = launch_gemv4(ctx, st, w, s, b, xn, ctx->head_logits, vocab, d, scale_dtype, TF_FP32);
+        if (rc != TF_OK) return rc;
+        const uint32_t grid = (uint32_t)std::min<long>(((long)vocab + 255) / 256, 1024);
+        n_summaries = grid;
+        hipLaunchKernelGGL(logits_partial_argmax_kernel, dim3(grid), dim3(256), 0, st, ctx->head_logits, ctx->head_summaries, (long)vocab);
+        rc = check_launch(ctx, "lm_head_greedy partial argmax");
+        if (rc != TF_OK) return rc;
+    }
+    hipLaunchKernelGGL(head_reduce_kernel, dim3(1), dim3(256), 0, st, ctx->head_summaries, static_cast<uint32_t *>(out_token), n_summaries);
+    return check_launch(ctx, "lm_head_greedy reduce");
+}
+
+int32_t tf_lm_head_logits_int4(tf_ctx *ctx, tf_stream stream, const void *hidden, uint64_t hidden_offset, const void *norm_weight,
+                               uint64_t norm_offset, const void *weights, uint64_t weights_offset, const void *scales,
+                               uint64_t scales_offset, const void *biases, uint64_t biases_offset, void *logits,
+                               uint64_t logits_offset, uint32_t d, uint32_t vocab, float rms_eps, tf_dtype scale_dtype,
+                               tf_dtype out_dtype) {
+    int32_t rc = validate_head(ctx, "lm_head_logits_int4", hidden, hidden_offset, norm_weight, norm_offset, weights, weights_offset,
+                               scales, scales_offset, biases, biases_offset, logits, d, vocab, scale_dtype);
+    if (rc != TF_OK) return rc;
+    TF_REQUIRE(ctx, out_dtype == TF_FP16 || out_dtype == TF_FP32, TF_ERR_INVALID_ARGUMENT, "lm_head_logits_int4: logits must be fp16 or fp32");
+    TF_REQUIRE(ctx, aligned(at(logits, logits_offset), out_dtype == TF_FP16 ? 2 : 4), TF_ERR_INVALID_ARGUMENT, "lm_head_logits_int4: misaligned logits");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    rc = launch_rmsnorm_bf16w(ctx, st, at(hidden, hidden_offset), at(norm_weight, norm_offset), ctx->head_x_normed, d, rms_eps);
+    if (rc != TF_OK) return rc;
+    return launch_gemv4(ctx, st, at(weights, weights_offset), at(scales, scales_offset), at(biases, biases_offset), ctx->head_x_normed,
+                        at(logits, logits_offset), vocab, d, scale_dtype, out_dtype);
+}
+
+}  // extern "C"

@@ -1,0 +1,599 @@
+// Router (int8 GEMV + top-8 + softmax), routed expert phases 1 and 2, and the int4 shared expert, for gfx950.
+#include "tf_gemv_kernels.hpp"
+
+using namespace tfk;
+
+namespace {
+
+struct RoutedArg {
+    const uint8_t *blob[TF_MAX_STREAMED_EXPERTS];
+    const uint8_t *pool;
+    uint64_t stride;
+    const uint32_t *indices;
+    uint32_t num_experts;
+};
+
+// Base pointer of the expert serving `slot`: a host-chosen pointer, or pool + stride * indices[slot] with the
+// index read on the device.
+__device__ __forceinline__ const uint8_t *blob_base(const RoutedArg &r, uint32_t slot) {
+    if (r.indices) {
+        uint32_t e = r.indices[slot];
+        e = e < r.num_experts ? e : r.num_experts - 1;
+        return r.pool + (uint64_t)e * r.stride;
+    }
+    return r.blob[slot];
+}
+
+// ------------------------------------------------------------------------------------------------ router
+// logits[e] = sum_g [ s * sum(q * x') + b * sum(x') ],  x' = float(hidden) * float(effective_scale).
+// One wave per expert row.  ALIGNED: 16-byte loads of 16 weights at a time; otherwise byte/halfword loads.
+template <int SD, bool ALIGNED>
+__device__ __forceinline__ float router_row(const uint8_t *w_row, const uint8_t *s_row, const uint8_t *b_row,
+                                            const half_t *hidden, const uint16_t *eff, int d, int lane) {
+    float acc = 0.0f;
+    if constexpr (ALIGNED) {
+        const int chunks = d >> 4;
+        for (int c = lane; c < chunks; c += kWave) {
+            const u32x4 w = load16(w_row + (size_t)c * 16);
+            const u32x4 ha = load16(hidden + c * 16), hb = load16(hidden + c * 16 + 8);
+            const u32x4 ea = load16(eff + c * 16), eb = load16(eff + c * 16 + 8);
+            const float s = sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(s_row + (c >> 2) * 2));
+            const float b = sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(b_row + (c >> 2) * 2));
+            float dot = 0.0f, sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const uint32_t hw = i < 8 ? ha[i >> 1] : hb[(i - 8) >> 1];
+                const uint32_t ew = i < 8 ? ea[i >> 1] : eb[(i - 8) >> 1];
+                const uint16_t hbits = (uint16_t)((i & 1) ? (hw >> 16) : (hw & 0xFFFFu));
+                const uint16_t ebits = (uint16_t)((i & 1) ? (ew >> 16) : (ew & 0xFFFFu));
+                const float xv = f16_to_f32(hbits) * bf16_to_f32(ebits);
+                const float q = (float)((w[i >> 2] >> (8 * (i & 3))) & 0xFFu);
+                dot = fmaf(q, xv, dot);
+                sum += xv;
+            }
+            acc = fmaf(s, dot, acc);
+            acc = fmaf(b, sum, acc);
+        }
+    } else {
+        const int words = d >> 2;
+        for (int wi = lane; wi < words; wi += kWave) {
+            const int g = wi >> 4;
+            const float s = sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(s_row + g * 2));
+            const float b = sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(b_row + g * 2));
+            float dot = 0.0f, sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float xv = (float)hidden[wi * 4 + i] * bf16_to_f32(eff[wi * 4 + i]);
+                dot = fmaf((float)w_row[wi * 4 + i], xv, dot);
+                sum += xv;
+            }
+            acc = fmaf(s, dot, acc);
+            acc = fmaf(b, sum, acc);
+        }
+    }
+    return wave_sum(acc);
+}
+
+// Top-k over <= 256 fp32 logits by one wave, then softmax over the selected and the per-expert gain.
+// Same ordering as the reference's serial insertion (moe.metal:152-171): score descending, ties to the lower index;
+// NaN and -inf are never selected; an unfilled position reads index 0 with score -inf.
+__device__ __forceinline__ void router_select(const float *logits, const uint16_t *per_expert_scale, uint32_t *out_indices,
+                                              half_t *out_weights, uint32_t num_experts, uint32_t top_k, int lane) {
+    float cand[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t e = lane + 64 * j;
+        const float v = e < num_experts ? __builtin_nontemporal_load(logits + e) : -INFINITY;
+        cand[j] = (v != v) ? -INFINITY : v;
+    }
+    float my_score = -INFINITY;   // lane i (< top_k) ends up holding the i-th selection
+    uint32_t my_idx = 0;
+    for (uint32_t i = 0; i < top_k; ++i) {
+        float bv = -INFINITY;
+        uint32_t bi = 0xFFFFFFFFu;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t e = lane + 64 * j;
+            if (cand[j] > bv) { bv = cand[j]; bi = e; }   // ascending e within the lane: strict > keeps the lower index
+        }
+        wave_best_pair(bv, bi);
+        const bool found = bi != 0xFFFFFFFFu;
+        if ((uint32_t)lane == i) { my_score = found ? bv : -INFINITY; my_idx = found ? bi : 0u; }
+        if (found && (bi & 63u) == (uint32_t)lane) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) if ((bi >> 6) == (uint32_t)j) cand[j] = -INFINITY;
+        }
+    }
+    const float max_s = __shfl(my_score, 0, kWave);
+    const float ex = (uint32_t)lane < top_k ? expf(my_score - max_s) : 0.0f;
+    float sum_exp = 0.0f;   // summed in selection order, like the reference
+    for (uint32_t i = 0; i < top_k; ++i) sum_exp += __shfl(ex, (int)i, kWave);
+    if ((uint32_t)lane < top_k) {
+        out_indices[lane] = my_idx;
+        out_weights[lane] = (half_t)((ex / sum_exp) * bf16_to_f32(per_expert_scale[my_idx]));
+    }
+}
+
+// One kernel for the whole router: every wave computes one logit; the wave that finishes last (an atomic ticket,
+// no waiting) performs the selection, so the indices are ready when the kernel ends and nothing returns to the host.
+template <int SD, bool ALIGNED>
+__global__ __launch_bounds__(256) void router_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *hidden,
+                                                     const uint16_t *eff, const uint16_t *per_expert_scale, float *logits,
+                                                     uint32_t *ticket, uint32_t *out_indices, half_t *out_weights,
+                                                     uint32_t num_experts, int d, uint32_t top_k) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t e = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    if (e >= num_experts) return;
+    const int groups = d >> 6;
+    const float v = router_row<SD, ALIGNED>(W + (size_t)e * d, S + (size_t)e * groups * 2, B + (size_t)e * groups * 2, hidden, eff, d, lane);
+    uint32_t t = 0;
+    if (lane == 0) {
+        __builtin_nontemporal_store(v, logits + e);
+        __threadfence();
+        t = atomicAdd(ticket, 1u);
+    }
+    t = (uint32_t)__shfl((int)t, 0, kWave);
+    if (t != num_experts - 1) return;
+    __threadfence();
+    if (lane == 0) *ticket = 0u;   // ready for the next call on this stream
+    router_select(logits, per_expert_scale, out_indices, out_weights, num_experts, top_k, lane);
+}
+
+// ------------------------------------------------------------------------------------------------ phase 1
+__device__ __forceinline__ void store_act(half_t *acts, uint32_t index, float gate, float up) {
+    acts[index] = (half_t)(gelu_tanh(gate) * up);
+}
+
+struct Phase1Geom {
+    uint32_t d, f, top_k;
+    uint32_t active_count;            // subset variant only
+    const uint32_t *active_slots;     // nullptr: all slots
+};
+
+__device__ __forceinline__ bool phase1_slot(const Phase1Geom &g, uint32_t unit, uint32_t units_per_slot, uint32_t &slot, uint32_t &tile) {
+    const uint32_t a = unit / units_per_slot;
+    tile = unit - a * units_per_slot;
+    if (g.active_slots) {
+        if (a >= g.active_count) return false;
+        slot = g.active_slots[a];
+    } else {
+        if (a >= g.top_k) return false;
+        slot = a;
+    }
+    return slot < g.top_k;
+}
+
+// D > 1024: one wave per RT-row tile of one slot; the gate tile and the up tile share the activations in registers.
+template <int RT, int NP, int SD>
+__global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_expert_offsets off, const half_t *x,
+                                                          half_t *acts, Phase1Geom g) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t unit = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint32_t tiles = (g.f + RT - 1) / RT;
+    uint32_t slot, tile;
+    if (!phase1_slot(g, unit, tiles, slot, tile)) return;
+    const uint8_t *base = blob_base(routed, slot);
+    const int groups = g.d >> 6;
+    const uint32_t row0 = tile * RT;
+    const int rows_left = (int)min((uint32_t)RT, g.f - row0);
+    const size_t w_byte = (size_t)row0 * (g.d >> 1);
+    const size_t sb_byte = (size_t)row0 * groups * 2;
+
+    LongRows<RT, NP> lr;
+    typename LongRows<RT, NP>::Tile tg, tu;
+    // weights do not depend on the activations: issue their loads first
+    lr.init_map(g.d, lane);
+    lr.load(tg, base + off.gate_W_off + w_byte, reinterpret_cast<const uint16_t *>(base + off.gate_s_off + sb_byte),
+            reinterpret_cast<const uint16_t *>(base + off.gate_b_off + sb_byte), rows_left, lane);
+    lr.load(tu, base + off.up_W_off + w_byte, reinterpret_cast<const uint16_t *>(base + off.up_s_off + sb_byte),
+            reinterpret_cast<const uint16_t *>(base + off.up_b_off + sb_byte), rows_left, lane);
+    lr.init_x(x, lane);
+    float gate[RT], up[RT];
+    lr.template reduce<SD>(tg, gate);
+    lr.template reduce<SD>(tu, up);
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < RT; ++r)
+            if (r < rows_left) store_act(acts, slot * g.f + row0 + r, gate[r], up[r]);
+    }
+}
+
+// D <= 1024: half-wave per row, NPASS passes: 2 * NPASS rows of gate and up per wave.
+template <int NPASS, int SD>
+__global__ __launch_bounds__(256) void phase1_short_kernel(RoutedArg routed, tf_expert_offsets off, const half_t *x,
+                                                           half_t *acts, Phase1Geom g) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t unit = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint32_t tiles = (g.f + 2 * NPASS - 1) / (2 * NPASS);
+    uint32_t slot, tile;
+    if (!phase1_slot(g, unit, tiles, slot, tile)) return;
+    const uint8_t *base = blob_base(routed, slot);
+    const long row0 = (long)tile * 2 * NPASS;
+    ShortRows sr;
+    sr.init(x, g.d, lane);
+    ShortRows::Pair tg[NPASS], tu[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+        sr.load(tg[p], base + off.gate_W_off, base + off.gate_s_off, base + off.gate_b_off, row0 + 2 * p, g.f, g.d);
+        sr.load(tu[p], base + off.up_W_off, base + off.up_s_off, base + off.up_b_off, row0 + 2 * p, g.f, g.d);
+    }
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+        float glo, ghi, ulo, uhi;
+        sr.template reduce<SD>(tg[p], glo, ghi);
+        sr.template reduce<SD>(tu[p], ulo, uhi);
+        if (lane == 0) {
+            const long r = row0 + 2 * p;
+            if (r < g.f) store_act(acts, slot * g.f + (uint32_t)r, glo, ulo);
+            if (r + 1 < g.f) store_act(acts, slot * g.f + (uint32_t)r + 1, ghi, uhi);
+        }
+    }
+}
+
+template <int SD>
+__global__ __launch_bounds__(256) void phase1_generic_kernel(RoutedArg routed, tf_expert_offsets off, const half_t *x,
+                                                             half_t *acts, Phase1Geom g) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t unit = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    uint32_t slot, r;
+    if (!phase1_slot(g, unit, g.f, slot, r)) return;
+    const uint8_t *base = blob_base(routed, slot);
+    const int groups = g.d >> 6;
+    const size_t w_byte = (size_t)r * (g.d >> 1), sb_byte = (size_t)r * groups * 2;
+    const float gate = generic_row_dot<SD>(base + off.gate_W_off + w_byte, base + off.gate_s_off + sb_byte, base + off.gate_b_off + sb_byte, x, g.d, lane);
+    const float up = generic_row_dot<SD>(base + off.up_W_off + w_byte, base + off.up_s_off + sb_byte, base + off.up_b_off + sb_byte, x, g.d, lane);
+    if (lane == 0) store_act(acts, slot * g.f + r, gate, up);
+}
+
+// ------------------------------------------------------------------------------------------------ phase 2
+// y[r] = half(residual[r] + sum_slot w[slot] * down_slot[r,:] . acts[slot,:]), slots added in order 0..7.
+// Block = 8 waves, wave s serves slot s; F <= 1024: 2 * NPASS rows per block.
+template <int NPASS, int SD>
+__global__ __launch_bounds__(512) void phase2_short_kernel(RoutedArg routed, tf_expert_offsets off, const half_t *acts,
+                                                           const half_t *routing_w, const half_t *residual, half_t *y,
+                                                           uint32_t d, uint32_t f) {
+    __shared__ float partial[8][2 * NPASS];
+    const int lane = threadIdx.x & 63;
+    const uint32_t slot = threadIdx.x >> 6;
+    const long row0 = (long)blockIdx.x * 2 * NPASS;
+    const uint8_t *base = blob_base(routed, slot);
+    ShortRows sr;
+    ShortRows::Pair t[NPASS];
+    sr.init_map(f, lane);
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p)
+        sr.load(t[p], base + off.down_W_off, base + off.down_s_off, base + off.down_b_off, row0 + 2 * p, d, f);
+    sr.init_x(acts + (size_t)slot * f);
+    const float w = (float)routing_w[slot];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+        float lo, hi;
+        sr.template reduce<SD>(t[p], lo, hi);
+        if (lane == 0) {
+            partial[slot][2 * p] = w * lo;
+            partial[slot][2 * p + 1] = w * hi;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < 2 * NPASS && row0 + threadIdx.x < d) {
+        float acc = (float)residual[row0 + threadIdx.x];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) acc += partial[s][threadIdx.x];
+        y[row0 + threadIdx.x] = (half_t)acc;
+    }
+}
+
+template <int SD>
+__global__ __launch_bounds__(512) void phase2_generic_kernel(RoutedArg routed, tf_expert_offsets off, const half_t *acts,
+                                                             const half_t *routing_w, const half_t *residual, half_t *y,
+                                                             uint32_t d, uint32_t f) {
+    __shared__ float partial[8];
+    const int lane = threadIdx.x & 63;
+    const uint32_t slot = threadIdx.x >> 6;
+    const uint32_t r = blockIdx.x;
+    const uint8_t *base = blob_base(routed, slot);
+    const int groups = f >> 6;
+    const float v = generic_row_dot<SD>(base + off.down_W_off + (size_t)r * (f >> 1), base + off.down_s_off + (size_t)r * groups * 2,
+                                        base + off.down_b_off + (size_t)r * groups * 2, acts + (size_t)slot * f, f, lane);
+    if (lane == 0) partial[slot] = (float)routing_w[slot] * v;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float acc = (float)residual[r];
+#pragma unroll
+        for (int s = 0; s < 8; ++s) acc += partial[s];
+        y[r] = (half_t)acc;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ shared expert
+// gate and up tiles share the activations; both sums are rounded to fp16 (the reference's two GEMVs write fp16)
+// before GeGLU (gelu_mul_fp16), and all three vectors land in the caller's scratch buffers.
+template <int RT, int NP, int SD>
+__global__ __launch_bounds__(256) void shared_gate_up_long_kernel(const uint8_t *gW, const uint16_t *gS, const uint16_t *gB,
+                                                                  const uint8_t *uW, const uint16_t *uS, const uint16_t *uB,
+                                                                  const half_t *x, half_t *gate_out, half_t *up_out,
+                                                                  half_t *act_out, uint32_t f, int d) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t tile = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint32_t row0 = tile * RT;
+    if (row0 >= f) return;
+    const int groups = d >> 6;
+    const int rows_left = (int)min((uint32_t)RT, f - row0);
+    LongRows<RT, NP> lr;
+    typename LongRows<RT, NP>::Tile tg, tu;
+    lr.init_map(d, lane);
+    lr.load(tg, gW + (size_t)row0 * (d >> 1), gS + (size_t)row0 * groups, gB + (size_t)row0 * groups, rows_left, lane);
+    lr.load(tu, uW + (size_t)row0 * (d >> 1), uS + (size_t)row0 * groups, uB + (size_t)row0 * groups, rows_left, lane);
+    lr.init_x(x, lane);
+    float gate[RT], up[RT];
+    lr.template reduce<SD>(tg, gate);
+    lr.template reduce<SD>(tu, up);
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            if (r >= rows_left) continue;
+            const half_t g16 = (half_t)gate[r], u16 = (half_t)up[r];
+            gate_out[row0 + r] = g16;
+            up_out[row0 + r] = u16;
+            act_out[row0 + r] = (half_t)(gelu_tanh((float)g16) * (float)u16);
+        }
+    }
+}
+
+bool routed_to_arg(const tf_routed_blobs *routed, uint32_t top_k, RoutedArg &arg, bool &all16) {
+    all16 = true;
+    arg.pool = nullptr;
+    arg.stride = 0;
+    arg.indices = nullptr;
+    arg.num_experts = 0;
+    for (uint32_t i = 0; i < TF_MAX_STREAMED_EXPERTS; ++i) arg.blob[i] = nullptr;
+    if (routed->indices) {
+        if (!routed->pool || routed->num_experts == 0) return false;
+        arg.pool = static_cast<const uint8_t *>(routed->pool);
+        arg.stride = routed->pool_stride;
+        arg.indices = routed->indices;
+        arg.num_experts = routed->num_experts;
+        all16 = aligned16(arg.pool) && (arg.stride % 16 == 0);
+        return true;
+    }
+    for (uint32_t i = 0; i < top_k; ++i) {
+        if (!routed->blobs[i]) return false;
+        arg.blob[i] = static_cast<const uint8_t *>(routed->blobs[i]);
+        all16 = all16 && aligned16(arg.blob[i]);
+    }
+    return true;
+}
+
+bool offsets_even(const tf_expert_offsets &o) {
+    return ((o.gate_W_off | o.gate_s_off | o.gate_b_off | o.up_W_off | o.up_s_off | o.up_b_off | o.down_W_off | o.down_s_off | o.down_b_off) & 1u) == 0;
+}
+
+int32_t phase1_entry(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *routed, const tf_expert_offsets *off, const void *x,
+                     void *acts, const uint32_t *active_slots, uint32_t active_count, bool subset, uint32_t d, uint32_t f,
+                     uint32_t top_k, tf_dtype sd) {
+    TF_REQUIRE(ctx, ctx && routed && off && x && acts, TF_ERR_INVALID_ARGUMENT, "moe_phase1: null argument");
+    TF_REQUIRE(ctx, top_k == TF_MAX_STREAMED_EXPERTS, TF_ERR_INVALID_ARGUMENT, "moe_phase1: topK must be 8, got %u", top_k);
+    TF_REQUIRE(ctx, d > 0 && d % TF_GROUP_SIZE == 0 && f > 0, TF_ERR_INVALID_ARGUMENT, "moe_phase1: d must be a multiple of 64 and f positive");
+    TF_REQUIRE(ctx, sd == TF_BF16 || sd == TF_FP16, TF_ERR_INVALID_ARGUMENT, "moe_phase1: scale dtype must be bf16 or fp16");
+    TF_REQUIRE(ctx, offsets_even(*off) && aligned(x, 2) && aligned(acts, 2), TF_ERR_INVALID_ARGUMENT, "moe_phase1: misaligned operand");
+    if (subset) {
+        if (active_count == 0) return TF_OK;
+        TF_REQUIRE(ctx, active_slots != nullptr && active_count <= top_k, TF_ERR_INVALID_ARGUMENT, "moe_phase1_subset: bad active slots");
+    }
+    RoutedArg arg;
+    bool all16;
+    TF_REQUIRE(ctx, routed_to_arg(routed, top_k, arg, all16), TF_ERR_INVALID_ARGUMENT, "moe_phase1: routed blobs incomplete");
+    Phase1Geom g{d, f, top_k, subset ? active_count : 0u, subset ? active_slots : nullptr};
+    const uint32_t n_slots = subset ? active_count : top_k;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const half_t *xh = static_cast<const half_t *>(x);
+    half_t *ah = static_cast<half_t *>(acts);
+    const bool fast = all16 && aligned16(x) && (off->gate_W_off % 16 == 0) && (off->up_W_off % 16 == 0);
+    const int SD = sd == TF_BF16 ? 0 : 1;
+    if (fast && d <= 1024) {
+        constexpr int NPASS = 2;
+        const uint32_t units = n_slots * ((f + 2 * NPASS - 1) / (2 * NPASS));
+        const dim3 grid((units + 3) / 4);
+        if (SD == 0) hipLaunchKernelGGL((phase1_short_kernel<NPASS, 0>), grid, dim3(256), 0, st, arg, *off, xh, ah, g);
+        else hipLaunchKernelGGL((phase1_short_kernel<NPASS, 1>), grid, dim3(256), 0, st, arg, *off, xh, ah, g);
+        return check_launch(ctx, "moe_phase1_short");
+    }
+    const LongPlan plan = plan_long_rows((int)d);
+    if (fast && plan.rt > 0) {
+        const uint32_t units = n_slots * ((f + plan.rt - 1) / plan.rt);
+        const dim3 grid((units + 3) / 4);
+#define TF_P1_CASE(RT_, NP_)                                                                                         \
+    if (plan.rt == RT_ && plan.np == NP_) {                                                                          \
+        if (SD == 0) hipLaunchKernelGGL((phase1_long_kernel<RT_, NP_, 0>), grid, dim3(256), 0, st, arg, *off, xh, ah, g); \
+        else hipLaunchKernelGGL((phase1_long_kernel<RT_, NP_, 1>), grid, dim3(256), 0, st, arg, *off, xh, ah, g);     \
+        return check_launch(ctx, "moe_phase1_long");                                                                 \
+    }
+        TF_P1_CASE(1, 1) TF_P1_CASE(1, 2) TF_P1_CASE(1, 3) TF_P1_CASE(1, 4)
+        TF_P1_CASE(2, 1) TF_P1_CASE(2, 2) TF_P1_CASE(2, 3) TF_P1_CASE(2, 4)
+        TF_P1_CASE(4, 1) TF_P1_CASE(4, 2) TF_P1_CASE(4, 3) TF_P1_CASE(4, 4)
+#undef TF_P1_CASE
+    }
+    const uint32_t units = n_slots * f;
+    const dim3 grid((units + 3) / 4);
+    if (SD == 0) hipLaunchKernelGGL((phase1_generic_kernel<0>), grid, dim3(256), 0, st, arg, *off, xh, ah, g);
+    else hipLaunchKernelGGL((phase1_generic_kernel<1>), grid, dim3(256), 0, st, arg, *off, xh, ah, g);
+    return check_launch(ctx, "moe_phase1_generic");
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t tf_router_gemma4(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset, const void *scales,
+                         uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *hidden,
+                         const void *effective_scale, uint64_t effective_scale_offset, const void *per_expert_scale,
+                         uint64_t per_expert_scale_offset, void *out_indices, void *out_weights, uint32_t num_experts,
+                         uint32_t d, uint32_t top_k) {
+    TF_REQUIRE(ctx, ctx && weights && scales && biases && hidden && effective_scale && per_expert_scale && out_indices && out_weights,
+               TF_ERR_INVALID_ARGUMENT, "router_gemma4: null argument");
+    TF_REQUIRE(ctx, d > 0 && d % TF_GROUP_SIZE == 0, TF_ERR_INVALID_ARGUMENT, "router_gemma4: d must be a multiple of 64, got %u", d);
+    TF_REQUIRE(ctx, num_experts > 0 && num_experts <= 256, TF_ERR_INVALID_ARGUMENT, "router_gemma4: numExperts must be in 1...256, got %u", num_experts);
+    TF_REQUIRE(ctx, top_k == TF_MAX_STREAMED_EXPERTS, TF_ERR_INVALID_ARGUMENT, "router_gemma4: topK must be 8, got %u", top_k);
+    const uint8_t *w = at(weights, weights_offset);
+    const uint8_t *s = at(scales, scales_offset);
+    const uint8_t *b = at(biases, biases_offset);
+    const uint8_t *eff = at(effective_scale, effective_scale_offset);
+    const uint8_t *pes = at(per_expert_scale, per_expert_scale_offset);
+    TF_REQUIRE(ctx, aligned(s, 2) && aligned(b, 2) && aligned(eff, 2) && aligned(pes, 2) && aligned(hidden, 2) &&
+                   aligned(out_indices, 4) && aligned(out_weights, 2),
+               TF_ERR_INVALID_ARGUMENT, "router_gemma4: misaligned operand");
+    const bool fast = aligned16(w) && aligned16(hidden) && aligned16(eff);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid((num_experts + 3) / 4);
+    uint32_t *ticket = reinterpret_cast<uint32_t *>(ctx->router_logits + 256);
+#define TF_ROUTER(AL_)                                                                                                        \
+    hipLaunchKernelGGL((router_kernel<0, AL_>), grid, dim3(256), 0, st, w, s, b, static_cast<const half_t *>(hidden),         \
+                       reinterpret_cast<const uint16_t *>(eff), reinterpret_cast<const uint16_t *>(pes), ctx->router_logits,  \
+                       ticket, static_cast<uint32_t *>(out_indices), static_cast<half_t *>(out_weights), num_experts, (int)d, top_k)
+    if (fast) TF_ROUTER(true); else TF_ROUTER(false);
+#undef TF_ROUTER
+    return check_launch(ctx, "router_gemma4");
+}
+
+int32_t tf_moe_phase1_gate_up_act(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *routed, const tf_expert_offsets *routed_offsets,
+                                  const void *x, void *acts, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype) {
+    return phase1_entry(ctx, stream, routed, routed_offsets, x, acts, nullptr, 0, false, d, f, top_k, scale_dtype);
+}
+
+int32_t tf_moe_phase1_gate_up_act_subset(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *routed, const tf_expert_offsets *routed_offsets,
+                                         const void *x, void *acts, const uint32_t *active_slots, uint32_t active_count,
+                                         uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype) {
+    return phase1_entry(ctx, stream, routed, routed_offsets, x, acts, active_slots, active_count, true, d, f, top_k, scale_dtype);
+}
+
+int32_t tf_moe_phase2_down_reduce(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *routed, const tf_expert_offsets *routed_offsets,
+                                  const void *acts, const void *routing_weights, const void *residual, void *y, uint32_t d,
+                                  uint32_t f, uint32_t top_k, tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx && routed && routed_offsets && acts && routing_weights && residual && y, TF_ERR_INVALID_ARGUMENT, "moe_phase2: null argument");
+    TF_REQUIRE(ctx, top_k == TF_MAX_STREAMED_EXPERTS, TF_ERR_INVALID_ARGUMENT, "moe_phase2: topK must be 8, got %u", top_k);
+    TF_REQUIRE(ctx, f > 0 && f % TF_GROUP_SIZE == 0 && d > 0, TF_ERR_INVALID_ARGUMENT, "moe_phase2: f must be a multiple of 64 and d positive");
+    TF_REQUIRE(ctx, scale_dtype == TF_BF16 || scale_dtype == TF_FP16, TF_ERR_INVALID_ARGUMENT, "moe_phase2: scale dtype must be bf16 or fp16");
+    TF_REQUIRE(ctx, offsets_even(*routed_offsets) && aligned(acts, 2) && aligned(routing_weights, 2) && aligned(residual, 2) && aligned(y, 2),
+               TF_ERR_INVALID_ARGUMENT, "moe_phase2: misaligned operand");
+    RoutedArg arg;
+    bool all16;
+    TF_REQUIRE(ctx, routed_to_arg(routed, top_k, arg, all16), TF_ERR_INVALID_ARGUMENT, "moe_phase2: routed blobs incomplete");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const half_t *ah = static_cast<const half_t *>(acts);
+    const half_t *wh = static_cast<const half_t *>(routing_weights);
+    const half_t *rh = static_cast<const half_t *>(residual);
+    half_t *yh = static_cast<half_t *>(y);
+    // acts rows start at slot * f halves: 16-byte aligned when f % 8 == 0, which f % 64 == 0 guarantees
+    const bool fast = all16 && aligned16(acts) && (routed_offsets->down_W_off % 16 == 0) && f <= 1024;
+    if (fast) {
+        constexpr int NPASS = 4;
+        const dim3 grid((d + 2 * NPASS - 1) / (2 * NPASS));
+        if (scale_dtype == TF_BF16) hipLaunchKernelGGL((phase2_short_kernel<NPASS, 0>), grid, dim3(512), 0, st, arg, *routed_offsets, ah, wh, rh, yh, d, f);
+        else hipLaunchKernelGGL((phase2_short_kernel<NPASS, 1>), grid, dim3(512), 0, st, arg, *routed_offsets, ah, wh, rh, yh, d, f);
+        return check_launch(ctx, "moe_phase2_short");
+    }
+    if (scale_dtype == TF_BF16) hipLaunchKernelGGL((phase2_generic_kernel<0>), dim3(d), dim3(512), 0, st, arg, *routed_offsets, ah, wh, rh, yh, d, f);
+    else hipLaunchKernelGGL((phase2_generic_kernel<1>), dim3(d), dim3(512), 0, st, arg, *routed_offsets, ah, wh, rh, yh, d, f);
+    return check_launch(ctx, "moe_phase2_generic");
+}
+
+int32_t tf_moe_decode_step(tf_ctx *ctx, tf_stream stream, const void *router_weights, uint64_t router_weights_offset,
+                           const void *router_scales, uint64_t router_scales_offset, const void *router_biases,
+                           uint64_t router_biases_offset, const void *router_x, const void *effective_scale,
+                           uint64_t effective_scale_offset, const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                           const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                           const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
+                           void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx && expert_pool && out_indices, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: null argument");
+    int32_t rc = tf_router_gemma4(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset,
+                                  router_biases, router_biases_offset, router_x, effective_scale, effective_scale_offset,
+                                  per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, d, top_k);
+    if (rc != TF_OK) return rc;
+    tf_routed_blobs routed = {};
+    routed.pool = expert_pool;
+    routed.pool_stride = expert_pool_stride;
+    routed.indices = static_cast<const uint32_t *>(out_indices);
+    routed.num_experts = num_experts;
+    rc = tf_moe_phase1_gate_up_act(ctx, stream, &routed, routed_offsets, x, acts, d, f, top_k, scale_dtype);
+    if (rc != TF_OK) return rc;
+    return tf_moe_phase2_down_reduce(ctx, stream, &routed, routed_offsets, acts, out_weights, residual, y, d, f, top_k, scale_dtype);
+}
+
+int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, uint64_t x_length,
+                              const tf_projection *gate, const tf_projection *up, const tf_projection *down, void *y,
+                              uint64_t y_offset, uint64_t y_length, void *scratch_gate, uint64_t scratch_gate_offset,
+                              uint64_t scratch_gate_length, void *scratch_up, uint64_t scratch_up_offset, uint64_t scratch_up_length,
+                              void *scratch_act, uint64_t scratch_act_offset, uint64_t scratch_act_length, uint32_t weight_bits,
+                              tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "shared_expert: null context");
+    TF_REQUIRE(ctx, weight_bits == 4, TF_ERR_UNSUPPORTED_BITS, "SharedExpert unsupported weight bits: %u", weight_bits);
+    TF_REQUIRE(ctx, x && gate && up && down && y && scratch_gate && scratch_up && scratch_act, TF_ERR_INVALID_ARGUMENT, "shared_expert: null argument");
+    TF_REQUIRE(ctx, gate->rows == up->rows && gate->cols == up->cols && down->rows == gate->cols && down->cols == gate->rows,
+               TF_ERR_DIMENSION_MISMATCH, "SharedExpert dimension mismatch: gate=(%u,%u) up=(%u,%u) down=(%u,%u)", gate->rows,
+               gate->cols, up->rows, up->cols, down->rows, down->cols);
+    const uint64_t required = (uint64_t)gate->rows * 2;
+    TF_REQUIRE(ctx, scratch_gate_offset + required <= scratch_gate_length && scratch_up_offset + required <= scratch_up_length &&
+                   scratch_act_offset + required <= scratch_act_length,
+               TF_ERR_SCRATCH_TOO_SMALL, "SharedExpert scratch too small: need %llu bytes per intermediate buffer", (unsigned long long)required);
+    TF_REQUIRE(ctx, x_offset + (uint64_t)gate->cols * 2 <= x_length, TF_ERR_SCRATCH_TOO_SMALL, "SharedExpert scratch too small: input range exceeds x buffer");
+    TF_REQUIRE(ctx, y_offset + (uint64_t)down->rows * 2 <= y_length, TF_ERR_SCRATCH_TOO_SMALL, "SharedExpert scratch too small: output range exceeds y buffer");
+    const tf_projection *proj[3] = {gate, up, down};
+    for (int i = 0; i < 3; ++i) {
+        TF_REQUIRE(ctx, proj[i]->weights && proj[i]->scales && proj[i]->biases, TF_ERR_INVALID_ARGUMENT, "shared_expert: null projection buffer");
+        TF_REQUIRE(ctx, proj[i]->cols % TF_GROUP_SIZE == 0 && proj[i]->cols > 0 && proj[i]->rows > 0, TF_ERR_INVALID_ARGUMENT,
+                   "shared_expert: N must be a multiple of 64");
+        TF_REQUIRE(ctx, aligned(at(proj[i]->weights, proj[i]->weights_offset), 2) && aligned(at(proj[i]->scales, proj[i]->scales_offset), 2) &&
+                       aligned(at(proj[i]->biases, proj[i]->biases_offset), 2),
+                   TF_ERR_INVALID_ARGUMENT, "shared_expert: projection offsets must be 2-byte aligned");
+    }
+    TF_REQUIRE(ctx, scale_dtype == TF_BF16 || scale_dtype == TF_FP16, TF_ERR_INVALID_ARGUMENT, "shared_expert: scale dtype must be bf16 or fp16");
+    TF_REQUIRE(ctx, x_offset % 2 == 0 && y_offset % 2 == 0 && scratch_gate_offset % 2 == 0 && scratch_up_offset % 2 == 0 && scratch_act_offset % 2 == 0,
+               TF_ERR_INVALID_ARGUMENT, "shared_expert: offsets must be 2-byte aligned");
+
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint8_t *xp = at(x, x_offset);
+    uint8_t *sg = at(scratch_gate, scratch_gate_offset), *su = at(scratch_up, scratch_up_offset), *sa = at(scratch_act, scratch_act_offset);
+    const uint8_t *gw = at(gate->weights, gate->weights_offset), *uw = at(up->weights, up->weights_offset);
+    const uint32_t f = gate->rows, d = gate->cols;
+    const LongPlan plan = plan_long_rows((int)d);
+    const bool fused = d > 1024 && plan.rt > 0 && aligned16(gw) && aligned16(uw) && aligned16(xp);
+    int32_t rc = TF_OK;
+    if (fused) {
+        const uint32_t tiles = (f + plan.rt - 1) / plan.rt;
+        const dim3 grid((tiles + 3) / 4);
+        const uint16_t *gs = reinterpret_cast<const uint16_t *>(at(gate->scales, gate->scales_offset));
+        const uint16_t *gb = reinterpret_cast<const uint16_t *>(at(gate->biases, gate->biases_offset));
+        const uint16_t *us = reinterpret_cast<const uint16_t *>(at(up->scales, up->scales_offset));
+        const uint16_t *ub = reinterpret_cast<const uint16_t *>(at(up->biases, up->biases_offset));
+        bool launched = false;
+#define TF_SH_CASE(RT_, NP_)                                                                                                    \
+    if (!launched && plan.rt == RT_ && plan.np == NP_) {                                                                        \
+        launched = true;                                                                                                        \
+        if (scale_dtype == TF_BF16)                                                                                             \
+            hipLaunchKernelGGL((shared_gate_up_long_kernel<RT_, NP_, 0>), grid, dim3(256), 0, st, gw, gs, gb, uw, us, ub,       \
+                               reinterpret_cast<const half_t *>(xp), reinterpret_cast<half_t *>(sg), reinterpret_cast<half_t *>(su), \
+                               reinterpret_cast<half_t *>(sa), f, (int)d);                                                      \
+        else                                                                                                                    \
+            hipLaunchKernelGGL((shared_gate_up_long_kernel<RT_, NP_, 1>), grid, dim3(256), 0, st, gw, gs, gb, uw, us, ub,       \
+                               reinterpret_cast<const half_t *>(xp), reinterpret_cast<half_t *>(sg), reinterpret_cast<half_t *>(su), \
+                               reinterpret_cast<half_t *>(sa), f, (int)d);                                                      \
+    }
+        TF_SH_CASE(1, 1) TF_SH_CASE(1, 2) TF_SH_CASE(1, 3) TF_SH_CASE(1, 4)
+        TF_SH_CASE(2, 1) TF_SH_CASE(2, 2) TF_SH_CASE(2, 3) TF_SH_CASE(2, 4)
+        TF_SH_CASE(4, 1) TF_SH_CASE(4, 2) TF_SH_CASE(4, 3) TF_SH_CASE(4, 4)
+#undef TF_SH_CASE
+        rc = check_launch(ctx, "shared_gate_up");
+        if (rc != TF_OK) return rc;
+    } else {
+        rc = launch_gemv4(ctx, st, gw, at(gate->scales, gate->scales_offset), at(gate->biases, gate->biases_offset), xp, sg, f, d, scale_dtype, TF_FP16);
+        if (rc != TF_OK) return rc;
+        rc = launch_gemv4(ctx, st, uw, at(up->scales, up->scales_offset), at(up->biases, up->biases_offset), xp, su, f, d, scale_dtype, TF_FP16);
+        if (rc != TF_OK) return rc;
+        rc = launch_gelu_mul(ctx, st, sg, su, sa, f);
+        if (rc != TF_OK) return rc;
+    }
+    return launch_gemv4(ctx, st, at(down->weights, down->weights_offset), at(down->scales, down->scales_offset),
+                        at(down->biases, down->biases_offset), sa, at(y, y_offset), down->rows, down->cols, scale_dtype, TF_FP16);
+}
+
+}  // extern "C"
