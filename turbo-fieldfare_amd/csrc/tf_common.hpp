@@ -63,6 +63,25 @@ __device__ __forceinline__ void half_wave_sums(float v, float &lo, float &hi) {
     hi = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+// Maximum over the 64 lanes (DPP, no LDS traffic); wave-uniform result.  NaNs must be filtered by the caller.
+template <int CTRL, int ROW_MASK = 0xF>
+__device__ __forceinline__ float dpp_f32_neg_inf(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp((int)0xFF800000u, __builtin_bit_cast(int, v), CTRL,
+                                                                 ROW_MASK, 0xF, false));
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_f32_neg_inf<0xB1>(v));
+    v = fmaxf(v, dpp_f32_neg_inf<0x4E>(v));
+    v = fmaxf(v, dpp_f32_neg_inf<0x141>(v));
+    v = fmaxf(v, dpp_f32_neg_inf<0x140>(v));
+    v = fmaxf(v, dpp_f32_neg_inf<0x142, 0xA>(v));
+    v = fmaxf(v, dpp_f32_neg_inf<0x143, 0xC>(v));
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+__device__ __forceinline__ float read_lane(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+
 // (value descending, index ascending) maximum across the wave; every lane ends with the winner.
 // Candidates that must never win carry value -inf and index 0xFFFFFFFF.
 __device__ __forceinline__ void wave_best_pair(float &v, uint32_t &idx) {

@@ -1,6 +1,8 @@
 // Context lifetime, error strings and stream synchronisation of the C ABI.
 #include "tf_context.hpp"
 
+#include <stdlib.h>
+
 #include <new>
 
 using namespace tfk;
@@ -38,11 +40,17 @@ int32_t tf_ctx_create(int32_t device, tf_ctx **out_ctx) {
     if (!ctx) return TF_ERR_OUT_OF_MEMORY;
     ctx->device = device;
     ctx->num_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-    // 256 logits + one uint32 ticket counter (must start at 0; the router kernel leaves it at 0)
-    bool ok = hipMalloc(&ctx->router_logits, 264 * sizeof(float)) == hipSuccess;
-    ok = ok && hipMemset(ctx->router_logits, 0, 264 * sizeof(float)) == hipSuccess;
+    bool ok = hipMalloc(&ctx->router_logits, 256 * sizeof(float)) == hipSuccess;
+    ok = ok && hipMemset(ctx->router_logits, 0, 256 * sizeof(float)) == hipSuccess;
     ok = ok && hipMalloc(&ctx->head_x_normed, kMaxHeadD * 2) == hipSuccess;
-    ok = ok && hipMalloc(&ctx->head_summaries, (size_t)kMaxHeadWaves * 2 * sizeof(float)) == hipSuccess;
+    // argmax summaries + 64 64-bit argmax cells behind them (start at 0; the decode kernel leaves them at 0)
+    const size_t summary_bytes = ((size_t)kMaxHeadWaves * 2 + 128) * sizeof(float);
+    ok = ok && hipMalloc(&ctx->head_summaries, summary_bytes) == hipSuccess;
+    ok = ok && hipMemset(ctx->head_summaries, 0, summary_bytes) == hipSuccess;
+    if (const char *env = getenv("TF_LONG_BLOCKS_PER_CU")) {
+        const int v = atoi(env);
+        if (v >= 1 && v <= 8) ctx->long_blocks_per_cu = v;
+    }
     if (!ok) {
         tf_ctx_destroy(ctx);
         return TF_ERR_OUT_OF_MEMORY;

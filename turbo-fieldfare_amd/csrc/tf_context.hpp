@@ -11,6 +11,7 @@
 struct tf_ctx {
     int device = 0;
     int num_cus = 0;
+    int long_blocks_per_cu = 4;         // 256-thread blocks per CU launched by the persistent row streamers
     // wrapper-owned scratch, as the reference's kernel classes own theirs
     float *router_logits = nullptr;     // 256 floats (MoE.swift:92-99)
     void *head_x_normed = nullptr;      // kMaxHeadD halves (LMHeadChainInt4.swift:38-51)

@@ -40,22 +40,35 @@ __device__ __forceinline__ void store_out(OutT *y, long row, float v) {
 }
 
 // ------------------------------------------------------------------------------------------------ GEMV kernels
-template <int RT, int NP, int SD, typename OutT>
-__global__ __launch_bounds__(256) void gemv4_long_kernel(const uint8_t *W, const uint16_t *S, const uint16_t *B,
-                                                         const half_t *x, OutT *y, long m, int k) {
+// Persistent: every wave walks tiles wave, wave + nwaves, ... of RT rows, requesting tile i+1 before reducing tile i.
+// FUSE_NORM: x is the raw hidden vector and the block normalises it itself (rmsnorm_bf16w with weight norm_w) into LDS.
+template <int RT, int NP, int SD, typename OutT, bool FUSE_NORM>
+__global__ __launch_bounds__(256, 4) void gemv4_long_kernel(const uint8_t *W, const uint16_t *S, const uint16_t *B,
+                                                            const half_t *x, const uint16_t *norm_w, float eps, OutT *y,
+                                                            long m, int k) {
     const int lane = threadIdx.x & 63;
     const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
     const long ntiles = (m + RT - 1) / RT;
-    if (wave >= ntiles) return;
+    const bool active = wave < ntiles;
     const int groups = k >> 6;
     const size_t tile_bytes = (size_t)RT * (k >> 1);
 
     LongRows<RT, NP> lr;
-    lr.init(x, k, lane);
     typename LongRows<RT, NP>::Tile cur, nxt;
+    lr.init_map(k, lane);
     long tile = wave;
-    lr.load(cur, W + tile * tile_bytes, S + tile * RT * groups, B + tile * RT * groups, (int)min((long)RT, m - tile * RT), lane);
+    if (active)
+        lr.load(cur, W + tile * tile_bytes, S + tile * RT * groups, B + tile * RT * groups, (int)min((long)RT, m - tile * RT), lane);
+    if constexpr (FUSE_NORM) {
+        __shared__ __align__(16) half_t xn_lds[kMaxFusedNormD];
+        __shared__ float partial[4];
+        block_rmsnorm_to_lds(x, norm_w, eps, k, xn_lds, partial);
+        if (active) lr.init_x(xn_lds, lane);
+    } else {
+        if (active) lr.init_x(x, lane);
+    }
+    if (!active) return;
     for (;;) {
         const long next = tile + nwaves;
         const bool has_next = next < ntiles;
@@ -164,6 +177,53 @@ __global__ __launch_bounds__(256) void rmsnorm_bf16w_kernel(const half_t *x, con
         out[i] = (half_t)((float)x[i] * inv * bf16_to_f32(weight[i]));
 }
 
+// 16-byte aligned operands, d % 8 == 0, d <= 2048 * PASSES: every thread requests all of its (at most PASSES) 8-element
+// chunks of x and of the weight up front, so the row costs one memory round trip instead of one per element.
+template <int PASSES>
+__global__ __launch_bounds__(256) void rmsnorm_bf16w_vec_kernel(const half_t *x, const uint16_t *weight, half_t *out, uint32_t d, float eps) {
+    __shared__ float partial[4];
+    u32x4 xr[PASSES], wr[PASSES];
+    float acc = 0.0f;
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+        const uint32_t i = (threadIdx.x + 256u * p) * 8u;
+        xr[p] = wr[p] = u32x4{0u, 0u, 0u, 0u};
+        if (i < d) {
+            xr[p] = load16(x + i);
+            wr[p] = load16(weight + i);
+        }
+    }
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const half2_t h = as_half2(xr[p][j]);
+            acc = fmaf((float)h[0], (float)h[0], acc);
+            acc = fmaf((float)h[1], (float)h[1], acc);
+        }
+    acc = wave_sum(acc);
+    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    const float inv = 1.0f / sqrtf((partial[0] + partial[1] + partial[2] + partial[3]) / (float)d + eps);
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+        const uint32_t i = (threadIdx.x + 256u * p) * 8u;
+        if (i < d) {
+            u32x4 o;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const half2_t h = as_half2(xr[p][j]);
+                const uint32_t wv = wr[p][j];
+                half2_t n;
+                n[0] = (half_t)((float)h[0] * inv * __uint_as_float(wv << 16));
+                n[1] = (half_t)((float)h[1] * inv * __uint_as_float(wv & 0xFFFF0000u));
+                o[j] = as_u32(n);
+            }
+            *reinterpret_cast<u32x4 *>(out + i) = o;
+        }
+    }
+}
+
 template <int BITS>
 int32_t dequantize_entry(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t wo, const void *scales, uint64_t so,
                          const void *biases, uint64_t bo, void *out, uint64_t oo, uint32_t m, uint32_t n, tf_dtype sd) {
@@ -191,7 +251,7 @@ namespace tfk {
 // Shared by tf_dequant_int4_gemv, the shared expert and the logits head.
 template <int SD, typename OutT>
 static int32_t launch_gemv4_typed(tf_ctx *ctx, hipStream_t st, const uint8_t *w, const uint8_t *s, const uint8_t *b,
-                                  const half_t *x, OutT *y, uint32_t m, uint32_t n) {
+                                  const half_t *x, OutT *y, uint32_t m, uint32_t n, const uint16_t *norm_w, float eps) {
     const bool fast = aligned16(w) && aligned16(x);
     if (fast && n <= 1024) {
         constexpr int NPASS = 4;
@@ -203,14 +263,18 @@ static int32_t launch_gemv4_typed(tf_ctx *ctx, hipStream_t st, const uint8_t *w,
     const LongPlan plan = plan_long_rows((int)n);
     if (fast && plan.rt > 0) {
         const long ntiles = ((long)m + plan.rt - 1) / plan.rt;
-        const long max_blocks = (long)ctx->num_cus * kLongBlocksPerCU;
+        const long max_blocks = (long)ctx->num_cus * ctx->long_blocks_per_cu;
         const uint32_t grid = (uint32_t)std::max<long>(1, std::min<long>((ntiles + 3) / 4, max_blocks));
         const uint16_t *s16 = reinterpret_cast<const uint16_t *>(s);
         const uint16_t *b16 = reinterpret_cast<const uint16_t *>(b);
 #define TF_LONG_CASE(RT_, NP_)                                                                                          \
     if (plan.rt == RT_ && plan.np == NP_) {                                                                             \
-        hipLaunchKernelGGL((gemv4_long_kernel<RT_, NP_, SD, OutT>), dim3(grid), dim3(256), 0, st, w, s16, b16, x, y,    \
-                           (long)m, (int)n);                                                                            \
+        if (norm_w)                                                                                                     \
+            hipLaunchKernelGGL((gemv4_long_kernel<RT_, NP_, SD, OutT, true>), dim3(grid), dim3(256), 0, st, w, s16,     \
+                               b16, x, norm_w, eps, y, (long)m, (int)n);                                                \
+        else                                                                                                            \
+            hipLaunchKernelGGL((gemv4_long_kernel<RT_, NP_, SD, OutT, false>), dim3(grid), dim3(256), 0, st, w, s16,    \
+                               b16, x, norm_w, eps, y, (long)m, (int)n);                                                \
         return check_launch(ctx, "gemv4_long");                                                                         \
     }
         TF_LONG_CASE(1, 1) TF_LONG_CASE(1, 2) TF_LONG_CASE(1, 3) TF_LONG_CASE(1, 4)
@@ -223,20 +287,33 @@ static int32_t launch_gemv4_typed(tf_ctx *ctx, hipStream_t st, const uint8_t *w,
     return check_launch(ctx, "gemv4_generic");
 }
 
+bool gemv4_can_fuse_norm(const uint8_t *w, const void *x, const void *norm_w, uint32_t n) {
+    return aligned16(w) && aligned16(x) && aligned16(norm_w) && n > 1024 && n <= (uint32_t)kMaxFusedNormD && plan_long_rows((int)n).rt > 0;
+}
+
+// norm_w != nullptr: x is the raw hidden vector, normalised inside the kernel; only legal when gemv4_can_fuse_norm().
 int32_t launch_gemv4(tf_ctx *ctx, hipStream_t st, const uint8_t *w, const uint8_t *s, const uint8_t *b, const void *x,
-                     void *y, uint32_t m, uint32_t n, tf_dtype sd, tf_dtype od) {
+                     void *y, uint32_t m, uint32_t n, tf_dtype sd, tf_dtype od, const void *norm_w, float eps) {
     const half_t *xh = static_cast<const half_t *>(x);
+    const uint16_t *nw = static_cast<const uint16_t *>(norm_w);
     if (sd == TF_BF16) {
-        if (od == TF_FP16) return launch_gemv4_typed<0, half_t>(ctx, st, w, s, b, xh, static_cast<half_t *>(y), m, n);
-        return launch_gemv4_typed<0, float>(ctx, st, w, s, b, xh, static_cast<float *>(y), m, n);
+        if (od == TF_FP16) return launch_gemv4_typed<0, half_t>(ctx, st, w, s, b, xh, static_cast<half_t *>(y), m, n, nw, eps);
+        return launch_gemv4_typed<0, float>(ctx, st, w, s, b, xh, static_cast<float *>(y), m, n, nw, eps);
     }
-    if (od == TF_FP16) return launch_gemv4_typed<1, half_t>(ctx, st, w, s, b, xh, static_cast<half_t *>(y), m, n);
-    return launch_gemv4_typed<1, float>(ctx, st, w, s, b, xh, static_cast<float *>(y), m, n);
+    if (od == TF_FP16) return launch_gemv4_typed<1, half_t>(ctx, st, w, s, b, xh, static_cast<half_t *>(y), m, n, nw, eps);
+    return launch_gemv4_typed<1, float>(ctx, st, w, s, b, xh, static_cast<float *>(y), m, n, nw, eps);
 }
 
 int32_t launch_rmsnorm_bf16w(tf_ctx *ctx, hipStream_t st, const void *x, const void *w, void *out, uint32_t d, float eps) {
-    hipLaunchKernelGGL(rmsnorm_bf16w_kernel, dim3(1), dim3(256), 0, st, static_cast<const half_t *>(x),
-                       static_cast<const uint16_t *>(w), static_cast<half_t *>(out), d, eps);
+    const half_t *xh = static_cast<const half_t *>(x);
+    const uint16_t *wh = static_cast<const uint16_t *>(w);
+    half_t *oh = static_cast<half_t *>(out);
+    const bool vec = aligned16(x) && aligned16(w) && aligned16(out) && d % 8 == 0 && d <= 16384;
+    if (vec && d <= 2048) hipLaunchKernelGGL(rmsnorm_bf16w_vec_kernel<1>, dim3(1), dim3(256), 0, st, xh, wh, oh, d, eps);
+    else if (vec && d <= 4096) hipLaunchKernelGGL(rmsnorm_bf16w_vec_kernel<2>, dim3(1), dim3(256), 0, st, xh, wh, oh, d, eps);
+    else if (vec && d <= 8192) hipLaunchKernelGGL(rmsnorm_bf16w_vec_kernel<4>, dim3(1), dim3(256), 0, st, xh, wh, oh, d, eps);
+    else if (vec) hipLaunchKernelGGL(rmsnorm_bf16w_vec_kernel<8>, dim3(1), dim3(256), 0, st, xh, wh, oh, d, eps);
+    else hipLaunchKernelGGL(rmsnorm_bf16w_kernel, dim3(1), dim3(256), 0, st, xh, wh, oh, d, eps);
     return check_launch(ctx, "rmsnorm_bf16w");
 }
 

@@ -18,57 +18,95 @@ __device__ __forceinline__ void better(Best &b, float v, uint32_t idx) {
     }
 }
 
-// Persistent row streamer: every wave walks tiles wave, wave + nwaves, ... of RT rows, keeps the best finite logit it
-// has seen (rows ascend within a wave, so a strict comparison keeps the lowest index among equals) and writes one
-// {value, index} summary.
-template <int RT, int NP, int SD>
-__global__ __launch_bounds__(256) void head_greedy_long_kernel(const uint8_t *W, const uint16_t *S, const uint16_t *B,
-                                                               const half_t *x, float *summaries, long v_rows, int k) {
+// Persistent row streamer: every wave walks tiles wave, wave + nwaves, ... of RT rows and keeps the best finite logit it
+// has seen (rows ascend within a wave, so a strict comparison keeps the lowest index among equals).  With FUSE_NORM each
+// block normalises the hidden vector itself (rmsnorm_bf16w needs no kernel of its own).  Each block folds its best
+// {value, index} into one of kHeadCells 64-bit cells with a single atomic max on the key
+// (orderable(value) << 32 | ~index): larger value wins, equal values resolve to the lower index, 0 means "nothing finite".
+// No fences, no waiting; head_decode_kernel turns the cells into the token.
+constexpr uint32_t kHeadCells = 64;
+
+__device__ __forceinline__ unsigned long long best_key(float v, uint32_t idx) {
+    if (idx == 0xFFFFFFFFu) return 0ull;
+    uint32_t u = __float_as_uint(v);
+    u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);   // monotone map of finite floats onto unsigned integers
+    return ((unsigned long long)u << 32) | (unsigned long long)(0xFFFFFFFFu - idx);
+}
+
+template <int RT, int NP, int SD, bool FUSE_NORM>
+__global__ __launch_bounds__(256, 4) void head_greedy_long_kernel(const uint8_t *W, const uint16_t *S, const uint16_t *B,
+                                                               const half_t *x, const uint16_t *norm_w, float eps,
+                                                               unsigned long long *cells, long v_rows, int k) {
+    __shared__ float sv[4];
+    __shared__ uint32_t si[4];
     const int lane = threadIdx.x & 63;
+    const int wib = threadIdx.x >> 6;
     const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
     const long ntiles = (v_rows + RT - 1) / RT;
-    if (wave >= ntiles) {
-        if (lane == 0) {
-            summaries[2 * wave] = -INFINITY;
-            summaries[2 * wave + 1] = __uint_as_float(0xFFFFFFFFu);
-        }
-        return;
-    }
+    Best best{-INFINITY, 0xFFFFFFFFu};
+    const bool active = wave < ntiles;
     const int groups = k >> 6;
     const size_t tile_bytes = (size_t)RT * (k >> 1);
     LongRows<RT, NP> lr;
     typename LongRows<RT, NP>::Tile cur, nxt;
     lr.init_map(k, lane);
     long tile = wave;
-    lr.load(cur, W + tile * tile_bytes, S + tile * RT * groups, B + tile * RT * groups, (int)min((long)RT, v_rows - tile * RT), lane);
-    lr.init_x(x, lane);
-    Best best{-INFINITY, 0xFFFFFFFFu};
-    for (;;) {
-        const long next = tile + nwaves;
-        const bool has_next = next < ntiles;
-        if (has_next)
-            lr.load(nxt, W + next * tile_bytes, S + next * RT * groups, B + next * RT * groups,
-                    (int)min((long)RT, v_rows - next * RT), lane);
-        float out[RT];
-        lr.template reduce<SD>(cur, out);
+    // the first tile does not depend on the activations: request it before normalising them
+    if (active)
+        lr.load(cur, W + tile * tile_bytes, S + tile * RT * groups, B + tile * RT * groups, (int)min((long)RT, v_rows - tile * RT), lane);
+    if constexpr (FUSE_NORM) {
+        __shared__ __align__(16) half_t xn_lds[kMaxFusedNormD];
+        __shared__ float partial[4];
+        block_rmsnorm_to_lds(x, norm_w, eps, k, xn_lds, partial);
+        if (active) lr.init_x(xn_lds, lane);
+    } else {
+        if (active) lr.init_x(x, lane);
+    }
+    if (active) {
+        for (;;) {
+            const long next = tile + nwaves;
+            const bool has_next = next < ntiles;
+            if (has_next)
+                lr.load(nxt, W + next * tile_bytes, S + next * RT * groups, B + next * RT * groups,
+                        (int)min((long)RT, v_rows - next * RT), lane);
+            float out[RT];
+            lr.template reduce<SD>(cur, out);
 #pragma unroll
-        for (int r = 0; r < RT; ++r) {
-            const long row = tile * RT + r;
-            const float z = out[r];
-            if (row < v_rows && __builtin_isfinite(z) && z > best.v) {
-                best.v = z;
-                best.idx = (uint32_t)row;
+            for (int r = 0; r < RT; ++r) {
+                const long row = tile * RT + r;
+                const float z = out[r];
+                if (row < v_rows && __builtin_isfinite(z) && z > best.v) {
+                    best.v = z;
+                    best.idx = (uint32_t)row;
+                }
             }
+            if (!has_next) break;
+            cur = nxt;
+            tile = next;
         }
-        if (!has_next) break;
-        cur = nxt;
-        tile = next;
     }
-    if (lane == 0) {
-        summaries[2 * wave] = best.v;
-        summaries[2 * wave + 1] = __uint_as_float(best.idx);
+    if (lane == 0) { sv[wib] = best.v; si[wib] = best.idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        Best b{sv[0], si[0]};
+        for (int w = 1; w < 4; ++w) better(b, sv[w], si[w]);
+        const unsigned long long key = best_key(b.v, b.idx);
+        if (key) atomicMax(cells + (blockIdx.x % kHeadCells), key);
     }
+}
+
+// One wave: the largest key among the cells is the answer; the cells are cleared for the next call.
+__global__ __launch_bounds__(64) void head_decode_kernel(unsigned long long *cells, uint32_t *out_token) {
+    const int lane = threadIdx.x;
+    unsigned long long key = cells[lane];
+    cells[lane] = 0ull;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const unsigned long long other = __shfl_xor(key, off, kWave);
+        key = other > key ? other : key;
+    }
+    if (lane == 0) out_token[0] = key ? 0xFFFFFFFFu - (uint32_t)(key & 0xFFFFFFFFull) : 0u;
 }
 
 // Fallback first stage: argmax summaries over an fp32 logits vector (one summary per block).
@@ -139,39 +177,46 @@ int32_t tf_lm_head_greedy_int4(tf_ctx *ctx, tf_stream stream, const void *hidden
     if (rc != TF_OK) return rc;
     TF_REQUIRE(ctx, aligned(out_token, 4), TF_ERR_INVALID_ARGUMENT, "lm_head_greedy_int4: misaligned out_token");
     hipStream_t st = static_cast<hipStream_t>(stream);
-    rc = launch_rmsnorm_bf16w(ctx, st, at(hidden, hidden_offset), at(norm_weight, norm_offset), ctx->head_x_normed, d, rms_eps);
-    if (rc != TF_OK) return rc;
-
     const uint8_t *w = at(weights, weights_offset);
     const uint8_t *s = at(scales, scales_offset);
     const uint8_t *b = at(biases, biases_offset);
+    const half_t *hid = reinterpret_cast<const half_t *>(at(hidden, hidden_offset));
+    const uint16_t *nw = reinterpret_cast<const uint16_t *>(at(norm_weight, norm_offset));
     const half_t *xn = static_cast<const half_t *>(ctx->head_x_normed);
     const LongPlan plan = plan_long_rows((int)d);
+    const bool rows_fast = aligned16(w) && d > 1024 && plan.rt > 0;
+    const bool fuse_norm = rows_fast && aligned16(hid) && aligned16(nw) && d <= (uint32_t)kMaxFusedNormD;
+    if (!fuse_norm) {
+        rc = launch_rmsnorm_bf16w(ctx, st, hid, nw, ctx->head_x_normed, d, rms_eps);
+        if (rc != TF_OK) return rc;
+    }
     uint32_t n_summaries = 0;
-    if (aligned16(w) && d > 1024 && plan.rt > 0) {
+    if (rows_fast) {
         const long ntiles = ((long)vocab + plan.rt - 1) / plan.rt;
-        const long max_blocks = std::min<long>((long)ctx->num_cus * kLongBlocksPerCU, kMaxHeadWaves / 4);
+        const long max_blocks = std::min<long>((long)ctx->num_cus * ctx->long_blocks_per_cu, 1024);
         const uint32_t grid = (uint32_t)std::max<long>(1, std::min<long>((ntiles + 3) / 4, max_blocks));
-        n_summaries = grid * 4;
         const uint16_t *s16 = reinterpret_cast<const uint16_t *>(s);
         const uint16_t *b16 = reinterpret_cast<const uint16_t *>(b);
+        unsigned long long *cells = reinterpret_cast<unsigned long long *>(ctx->head_summaries + 2 * kMaxHeadWaves);
         bool launched = false;
+#define TF_HEAD_LAUNCH(RT_, NP_, SD_, FN_)                                                                              \
+    hipLaunchKernelGGL((head_greedy_long_kernel<RT_, NP_, SD_, FN_>), dim3(grid), dim3(256), 0, st, w, s16, b16,        \
+                       FN_ ? hid : xn, nw, rms_eps, cells, (long)vocab, (int)d)
 #define TF_HEAD_CASE(RT_, NP_)                                                                                          \
     if (!launched && plan.rt == RT_ && plan.np == NP_) {                                                                \
         launched = true;                                                                                                \
-        if (scale_dtype == TF_BF16)                                                                                     \
-            hipLaunchKernelGGL((head_greedy_long_kernel<RT_, NP_, 0>), dim3(grid), dim3(256), 0, st, w, s16, b16, xn,   \
-                               ctx->head_summaries, (long)vocab, (int)d);                                               \
-        else                                                                                                            \
-            hipLaunchKernelGGL((head_greedy_long_kernel<RT_, NP_, 1>), dim3(grid), dim3(256), 0, st, w, s16, b16, xn,   \
-                               ctx->head_summaries, (long)vocab, (int)d);                                               \
+        if (scale_dtype == TF_BF16) { if (fuse_norm) TF_HEAD_LAUNCH(RT_, NP_, 0, true); else TF_HEAD_LAUNCH(RT_, NP_, 0, false); } \
+        else { if (fuse_norm) TF_HEAD_LAUNCH(RT_, NP_, 1, true); else TF_HEAD_LAUNCH(RT_, NP_, 1, false); }             \
     }
         TF_HEAD_CASE(1, 1) TF_HEAD_CASE(1, 2) TF_HEAD_CASE(1, 3) TF_HEAD_CASE(1, 4)
         TF_HEAD_CASE(2, 1) TF_HEAD_CASE(2, 2) TF_HEAD_CASE(2, 3) TF_HEAD_CASE(2, 4)
         TF_HEAD_CASE(4, 1) TF_HEAD_CASE(4, 2) TF_HEAD_CASE(4, 3) TF_HEAD_CASE(4, 4)
 #undef TF_HEAD_CASE
+#undef TF_HEAD_LAUNCH
         rc = check_launch(ctx, "lm_head_greedy rows");
         if (rc != TF_OK) return rc;
+        hipLaunchKernelGGL(head_decode_kernel, dim3(1), dim3(64), 0, st, cells, static_cast<uint32_t *>(out_token));
+        return check_launch(ctx, "lm_head_greedy decode");
     } else {
         // short or unaligned rows: fp32 logits into wrapper-owned scratch, then a two-stage argmax
         if (ctx->head_logits_count < vocab) {
@@ -205,9 +250,13 @@ int32_t tf_lm_head_logits_int4(tf_ctx *ctx, tf_stream stream, const void *hidden
     TF_REQUIRE(ctx, out_dtype == TF_FP16 || out_dtype == TF_FP32, TF_ERR_INVALID_ARGUMENT, "lm_head_logits_int4: logits must be fp16 or fp32");
     TF_REQUIRE(ctx, aligned(at(logits, logits_offset), out_dtype == TF_FP16 ? 2 : 4), TF_ERR_INVALID_ARGUMENT, "lm_head_logits_int4: misaligned logits");
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint8_t *w = at(weights, weights_offset);
+    if (gemv4_can_fuse_norm(w, at(hidden, hidden_offset), at(norm_weight, norm_offset), d))
+        return launch_gemv4(ctx, st, w, at(scales, scales_offset), at(biases, biases_offset), at(hidden, hidden_offset),
+                            at(logits, logits_offset), vocab, d, scale_dtype, out_dtype, at(norm_weight, norm_offset), rms_eps);
     rc = launch_rmsnorm_bf16w(ctx, st, at(hidden, hidden_offset), at(norm_weight, norm_offset), ctx->head_x_normed, d, rms_eps);
     if (rc != TF_OK) return rc;
-    return launch_gemv4(ctx, st, at(weights, weights_offset), at(scales, scales_offset), at(biases, biases_offset), ctx->head_x_normed,
+    return launch_gemv4(ctx, st, w, at(scales, scales_offset), at(biases, biases_offset), ctx->head_x_normed,
                         at(logits, logits_offset), vocab, d, scale_dtype, out_dtype);
 }
 

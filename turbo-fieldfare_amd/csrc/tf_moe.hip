@@ -26,34 +26,53 @@ __device__ __forceinline__ const uint8_t *blob_base(const RoutedArg &r, uint32_t
 
 // ------------------------------------------------------------------------------------------------ router
 // logits[e] = sum_g [ s * sum(q * x') + b * sum(x') ],  x' = float(hidden) * float(effective_scale).
-// One wave per expert row.  ALIGNED: 16-byte loads of 16 weights at a time; otherwise byte/halfword loads.
-template <int SD, bool ALIGNED>
+// One wave per expert row.  NPASS > 0: every operand 16-byte aligned and d <= 1024 * NPASS; the lane's <= NPASS chunks of
+// 16 weights are all requested before the first is used, so the row costs one memory round trip.  NPASS == 0: any
+// alignment and size, byte/halfword loads in a loop.
+__device__ __forceinline__ void router_chunk(const u32x4 w, const u32x4 ha, const u32x4 hb, const u32x4 ea, const u32x4 eb,
+                                             float s, float b, float &acc) {
+    float dot = 0.0f, sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t hw = i < 8 ? ha[i >> 1] : hb[(i - 8) >> 1];
+        const uint32_t ew = i < 8 ? ea[i >> 1] : eb[(i - 8) >> 1];
+        const uint16_t hbits = (uint16_t)((i & 1) ? (hw >> 16) : (hw & 0xFFFFu));
+        const float ev = (i & 1) ? __uint_as_float(ew & 0xFFFF0000u) : __uint_as_float(ew << 16);
+        const float xv = f16_to_f32(hbits) * ev;
+        const float q = (float)((w[i >> 2] >> (8 * (i & 3))) & 0xFFu);
+        dot = fmaf(q, xv, dot);
+        sum += xv;
+    }
+    acc = fmaf(s, dot, acc);
+    acc = fmaf(b, sum, acc);
+}
+
+template <int SD, int NPASS>
 __device__ __forceinline__ float router_row(const uint8_t *w_row, const uint8_t *s_row, const uint8_t *b_row,
                                             const half_t *hidden, const uint16_t *eff, int d, int lane) {
     float acc = 0.0f;
-    if constexpr (ALIGNED) {
+    if constexpr (NPASS > 0) {
         const int chunks = d >> 4;
-        for (int c = lane; c < chunks; c += kWave) {
-            const u32x4 w = load16(w_row + (size_t)c * 16);
-            const u32x4 ha = load16(hidden + c * 16), hb = load16(hidden + c * 16 + 8);
-            const u32x4 ea = load16(eff + c * 16), eb = load16(eff + c * 16 + 8);
-            const float s = sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(s_row + (c >> 2) * 2));
-            const float b = sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(b_row + (c >> 2) * 2));
-            float dot = 0.0f, sum = 0.0f;
+        u32x4 w[NPASS], ha[NPASS], hb[NPASS], ea[NPASS], eb[NPASS];
+        uint16_t sv[NPASS], bv[NPASS];
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const uint32_t hw = i < 8 ? ha[i >> 1] : hb[(i - 8) >> 1];
-                const uint32_t ew = i < 8 ? ea[i >> 1] : eb[(i - 8) >> 1];
-                const uint16_t hbits = (uint16_t)((i & 1) ? (hw >> 16) : (hw & 0xFFFFu));
-                const uint16_t ebits = (uint16_t)((i & 1) ? (ew >> 16) : (ew & 0xFFFFu));
-                const float xv = f16_to_f32(hbits) * bf16_to_f32(ebits);
-                const float q = (float)((w[i >> 2] >> (8 * (i & 3))) & 0xFFu);
-                dot = fmaf(q, xv, dot);
-                sum += xv;
+        for (int p = 0; p < NPASS; ++p) {
+            const int c = lane + 64 * p;
+            w[p] = ha[p] = hb[p] = ea[p] = eb[p] = u32x4{0u, 0u, 0u, 0u};
+            sv[p] = bv[p] = 0;
+            if (c < chunks) {
+                w[p] = load16(w_row + (size_t)c * 16);
+                ha[p] = load16(hidden + c * 16);
+                hb[p] = load16(hidden + c * 16 + 8);
+                ea[p] = load16(eff + c * 16);
+                eb[p] = load16(eff + c * 16 + 8);
+                sv[p] = *reinterpret_cast<const uint16_t *>(s_row + (c >> 2) * 2);
+                bv[p] = *reinterpret_cast<const uint16_t *>(b_row + (c >> 2) * 2);
             }
-            acc = fmaf(s, dot, acc);
-            acc = fmaf(b, sum, acc);
         }
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p)
+            router_chunk(w[p], ha[p], hb[p], ea[p], eb[p], sb_to_f32<SD>(sv[p]), sb_to_f32<SD>(bv[p]), acc);
     } else {
         const int words = d >> 2;
         for (int wi = lane; wi < words; wi += kWave) {
@@ -77,66 +96,79 @@ __device__ __forceinline__ float router_row(const uint8_t *w_row, const uint8_t 
 // Top-k over <= 256 fp32 logits by one wave, then softmax over the selected and the per-expert gain.
 // Same ordering as the reference's serial insertion (moe.metal:152-171): score descending, ties to the lower index;
 // NaN and -inf are never selected; an unfilled position reads index 0 with score -inf.
-__device__ __forceinline__ void router_select(const float *logits, const uint16_t *per_expert_scale, uint32_t *out_indices,
+// Lane l holds candidates l, l+64, l+128, l+192 and their gains; each round takes the wave maximum with DPP and finds
+// its lowest expert index with ballots, so a round is a few dozen ALU instructions and no memory traffic.
+__device__ __forceinline__ void router_select(const float *logits, const float gain[4], uint32_t *out_indices,
                                               half_t *out_weights, uint32_t num_experts, uint32_t top_k, int lane) {
     float cand[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
         const uint32_t e = lane + 64 * j;
-        const float v = e < num_experts ? __builtin_nontemporal_load(logits + e) : -INFINITY;
+        const float v = e < num_experts ? logits[e] : -INFINITY;
         cand[j] = (v != v) ? -INFINITY : v;
     }
-    float my_score = -INFINITY;   // lane i (< top_k) ends up holding the i-th selection
+    float my_score = -INFINITY, my_gain = 0.0f;   // lane i (< top_k) ends up holding the i-th selection
     uint32_t my_idx = 0;
     for (uint32_t i = 0; i < top_k; ++i) {
-        float bv = -INFINITY;
-        uint32_t bi = 0xFFFFFFFFu;
+        const float m = fmaxf(fmaxf(cand[0], cand[1]), fmaxf(cand[2], cand[3]));
+        const float wm = wave_max(m);
+        const bool found = wm > -INFINITY;
+        int sel_j = 4, sel_lane = 0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t e = lane + 64 * j;
-            if (cand[j] > bv) { bv = cand[j]; bi = e; }   // ascending e within the lane: strict > keeps the lower index
+        for (int j = 3; j >= 0; --j) {
+            const uint64_t mask = __ballot(cand[j] == wm);
+            if (mask) { sel_j = j; sel_lane = __builtin_ctzll(mask); }
         }
-        wave_best_pair(bv, bi);
-        const bool found = bi != 0xFFFFFFFFu;
-        if ((uint32_t)lane == i) { my_score = found ? bv : -INFINITY; my_idx = found ? bi : 0u; }
-        if (found && (bi & 63u) == (uint32_t)lane) {
+        float g = 0.0f;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) if ((bi >> 6) == (uint32_t)j) cand[j] = -INFINITY;
+        for (int j = 0; j < 4; ++j)
+            if (sel_j == j) g = read_lane(gain[j], sel_lane);
+        if ((uint32_t)lane == i) {
+            my_score = found ? wm : -INFINITY;
+            my_idx = found ? (uint32_t)(sel_lane + 64 * sel_j) : 0u;
+            my_gain = found ? g : read_lane(gain[0], 0);
+        }
+        if (found && lane == sel_lane) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (sel_j == j) cand[j] = -INFINITY;
         }
     }
-    const float max_s = __shfl(my_score, 0, kWave);
+    const float max_s = read_lane(my_score, 0);
     const float ex = (uint32_t)lane < top_k ? expf(my_score - max_s) : 0.0f;
     float sum_exp = 0.0f;   // summed in selection order, like the reference
-    for (uint32_t i = 0; i < top_k; ++i) sum_exp += __shfl(ex, (int)i, kWave);
+    for (uint32_t i = 0; i < top_k; ++i) sum_exp += read_lane(ex, (int)i);
     if ((uint32_t)lane < top_k) {
         out_indices[lane] = my_idx;
-        out_weights[lane] = (half_t)((ex / sum_exp) * bf16_to_f32(per_expert_scale[my_idx]));
+        out_weights[lane] = (half_t)((ex / sum_exp) * my_gain);
     }
 }
 
-// One kernel for the whole router: every wave computes one logit; the wave that finishes last (an atomic ticket,
-// no waiting) performs the selection, so the indices are ready when the kernel ends and nothing returns to the host.
-template <int SD, bool ALIGNED>
-__global__ __launch_bounds__(256) void router_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *hidden,
-                                                     const uint16_t *eff, const uint16_t *per_expert_scale, float *logits,
-                                                     uint32_t *ticket, uint32_t *out_indices, half_t *out_weights,
-                                                     uint32_t num_experts, int d, uint32_t top_k) {
+// Two launches, as in the reference (router_gemv_gemma4_r4 then router_topk_select_k8): one wave per expert row writes
+// its logit; a single wave then selects.  Both stay on the device; nothing returns to the host.
+template <int SD, int NPASS>
+__global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B,
+                                                            const half_t *hidden, const uint16_t *eff, float *logits,
+                                                            uint32_t num_experts, int d) {
     const int lane = threadIdx.x & 63;
     const uint32_t e = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
     if (e >= num_experts) return;
     const int groups = d >> 6;
-    const float v = router_row<SD, ALIGNED>(W + (size_t)e * d, S + (size_t)e * groups * 2, B + (size_t)e * groups * 2, hidden, eff, d, lane);
-    uint32_t t = 0;
-    if (lane == 0) {
-        __builtin_nontemporal_store(v, logits + e);
-        __threadfence();
-        t = atomicAdd(ticket, 1u);
+    const float v = router_row<SD, NPASS>(W + (size_t)e * d, S + (size_t)e * groups * 2, B + (size_t)e * groups * 2, hidden, eff, d, lane);
+    if (lane == 0) logits[e] = v;
+}
+
+__global__ __launch_bounds__(64) void router_select_kernel(const float *logits, const uint16_t *per_expert_scale,
+                                                           uint32_t *out_indices, half_t *out_weights, uint32_t num_experts,
+                                                           uint32_t top_k) {
+    const int lane = threadIdx.x;
+    float gain[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t c = lane + 64 * j;
+        gain[j] = c < num_experts ? bf16_to_f32(per_expert_scale[c]) : 0.0f;
     }
-    t = (uint32_t)__shfl((int)t, 0, kWave);
-    if (t != num_experts - 1) return;
-    __threadfence();
-    if (lane == 0) *ticket = 0u;   // ready for the next call on this stream
-    router_select(logits, per_expert_scale, out_indices, out_weights, num_experts, top_k, lane);
+    router_select(logits, gain, out_indices, out_weights, num_experts, top_k, lane);
 }
 
 // ------------------------------------------------------------------------------------------------ phase 1
@@ -442,17 +474,26 @@ int32_t tf_router_gemma4(tf_ctx *ctx, tf_stream stream, const void *weights, uin
     TF_REQUIRE(ctx, aligned(s, 2) && aligned(b, 2) && aligned(eff, 2) && aligned(pes, 2) && aligned(hidden, 2) &&
                    aligned(out_indices, 4) && aligned(out_weights, 2),
                TF_ERR_INVALID_ARGUMENT, "router_gemma4: misaligned operand");
-    const bool fast = aligned16(w) && aligned16(hidden) && aligned16(eff);
+    const bool fast = aligned16(w) && aligned16(hidden) && aligned16(eff) && d <= 4096;
+    const int npass = fast ? (int)((d / 16 + 63) / 64) : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 grid((num_experts + 3) / 4);
-    uint32_t *ticket = reinterpret_cast<uint32_t *>(ctx->router_logits + 256);
-#define TF_ROUTER(AL_)                                                                                                        \
-    hipLaunchKernelGGL((router_kernel<0, AL_>), grid, dim3(256), 0, st, w, s, b, static_cast<const half_t *>(hidden),         \
-                       reinterpret_cast<const uint16_t *>(eff), reinterpret_cast<const uint16_t *>(pes), ctx->router_logits,  \
-                       ticket, static_cast<uint32_t *>(out_indices), static_cast<half_t *>(out_weights), num_experts, (int)d, top_k)
-    if (fast) TF_ROUTER(true); else TF_ROUTER(false);
+#define TF_ROUTER(NP_)                                                                                                        \
+    hipLaunchKernelGGL((router_logits_kernel<0, NP_>), grid, dim3(256), 0, st, w, s, b, static_cast<const half_t *>(hidden),  \
+                       reinterpret_cast<const uint16_t *>(eff), ctx->router_logits, num_experts, (int)d)
+    switch (npass) {
+        case 1: TF_ROUTER(1); break;
+        case 2: TF_ROUTER(2); break;
+        case 3: TF_ROUTER(3); break;
+        case 4: TF_ROUTER(4); break;
+        default: TF_ROUTER(0); break;
+    }
 #undef TF_ROUTER
-    return check_launch(ctx, "router_gemma4");
+    const int32_t rc = check_launch(ctx, "router_gemma4 logits");
+    if (rc != TF_OK) return rc;
+    hipLaunchKernelGGL(router_select_kernel, dim3(1), dim3(64), 0, st, ctx->router_logits, reinterpret_cast<const uint16_t *>(pes),
+                       static_cast<uint32_t *>(out_indices), static_cast<half_t *>(out_weights), num_experts, top_k);
+    return check_launch(ctx, "router_gemma4 select");
 }
 
 int32_t tf_moe_phase1_gate_up_act(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *routed, const tf_expert_offsets *routed_offsets,
