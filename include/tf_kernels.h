@@ -249,6 +249,130 @@ int32_t tf_lm_head_logits_int4(tf_ctx *ctx, tf_stream stream,
                                void *logits, uint64_t logits_offset,
                                uint32_t d, uint32_t vocab, float rms_eps, tf_dtype scale_dtype, tf_dtype out_dtype);
 
+/* ---- prefill / multi-token path --------------------------------------------------------------------------------------- */
+/* PrefillTokenExpertPair (Kernels/Prefill/MoE/PrefillRouter.swift:5-28): 16 bytes, fields at 0/4/8/12; the low 16 bits of
+ * weight_bits_and_reserved hold the fp16 routing weight. */
+typedef struct tf_prefill_pair { uint32_t token, expert, rank, weight_bits_and_reserved; } tf_prefill_pair;
+/* PrefillMoEGroup / PrefillMoETile (Kernels/Prefill/MoE/PrefillMoEGrouping.swift:4-29). */
+typedef struct tf_prefill_group { uint32_t expert, pair_start, pair_count; } tf_prefill_group;
+typedef struct tf_prefill_tile { uint32_t group_start, group_count, pair_start, pair_count; } tf_prefill_tile;
+/* PrefillGroupedRoutedMoEStreamedParams (Kernels/Prefill/MoE/PrefillGroupedRoutedMoE.swift:104-183): 128 bytes, field
+ * offsets 0,4,...,24, local_expert[0] at 28, local_expert[15] at 88, gate_W_off at 92, down_b_off at 124.  Unused
+ * local_expert slots hold 0xFFFFFFFF. */
+typedef struct tf_prefill_streamed_params {
+    uint32_t pair_start, pair_count, d, routed_intermediate, top_k, hidden_stride_elements, live_expert_count;
+    uint32_t local_expert[TF_MAX_TILE_EXPERTS];
+    uint32_t gate_W_off, gate_s_off, gate_b_off, up_W_off, up_s_off, up_b_off, down_W_off, down_s_off, down_b_off;
+} tf_prefill_streamed_params;
+
+/* PrefillMoEGroupingError (PrefillMoEGrouping.swift:52-63), as negative statuses of the grouping call. */
+#define TF_ERR_GROUP_INVALID_QUERY_COUNT (-101)
+#define TF_ERR_GROUP_INVALID_TOP_K (-102)
+#define TF_ERR_GROUP_INVALID_NUM_EXPERTS (-103)
+#define TF_ERR_GROUP_INVALID_TILE_EXPERT_COUNT (-104)
+#define TF_ERR_GROUP_PAIR_COUNT_MISMATCH (-105)
+#define TF_ERR_GROUP_TOKEN_OUT_OF_RANGE (-106)
+#define TF_ERR_GROUP_RANK_OUT_OF_RANGE (-107)
+#define TF_ERR_GROUP_EXPERT_OUT_OF_RANGE (-108)
+#define TF_ERR_GROUP_DUPLICATE_TOKEN_RANK (-109)
+#define TF_ERR_GROUP_SORT_KEY_COUNT_MISMATCH (-110)
+
+/* PrefillRouter.encodeGemma4Block (PrefillRouter.swift:37-89) -> prefill_router_gemma4_block (Metal/Prefill/prefill.metal:
+ * 478-573): per token row t, logits over num_experts, top_k (1...64) by (score desc, index asc), softmax over the selected,
+ * times per_expert_scale.  hidden rows are hidden_stride_elements apart.  out_indices uint32[T, top_k], out_weights
+ * fp16[T, top_k].  query_count > 0, num_experts <= 256, d % 64 == 0, hidden_stride_elements >= d. */
+int32_t tf_prefill_router_gemma4_block(tf_ctx *ctx, tf_stream stream,
+                                       const void *weights, uint64_t weights_offset,
+                                       const void *scales, uint64_t scales_offset,
+                                       const void *biases, uint64_t biases_offset,
+                                       const void *hidden, uint64_t hidden_offset,
+                                       const void *effective_scale, uint64_t effective_scale_offset,
+                                       const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                                       void *out_indices, uint64_t out_indices_offset,
+                                       void *out_weights, uint64_t out_weights_offset,
+                                       uint32_t query_count, uint32_t num_experts, uint32_t d, uint32_t top_k,
+                                       uint32_t hidden_stride_elements);
+
+/* PrefillRouter.makeTokenExpertPairs (PrefillRouter.swift:91-111).  HOST arrays; pure CPU. */
+int32_t tf_prefill_make_token_expert_pairs(const uint32_t *indices, const uint16_t *weights_f16, int32_t query_count,
+                                           int32_t top_k, tf_prefill_pair *pairs);
+/* PrefillMoEGrouping.groupTokenExpertPairs (PrefillMoEGrouping.swift:90-193).  HOST arrays; pure CPU.  Validates, sorts by
+ * (sort key?, expert, token, rank), run-length groups, tiles of <= tile_expert_count experts.  expert_sort_keys may be NULL.
+ * per_expert_offsets/per_expert_counts: num_experts entries (offset 0xFFFFFFFF = expert unused); groups/tiles: capacity
+ * min(num_experts, pair_count) each.  Returns TF_OK or one of TF_ERR_GROUP_*. */
+int32_t tf_prefill_group_token_expert_pairs(const tf_prefill_pair *pairs, uint64_t pair_count, int32_t query_count,
+                                            int32_t top_k, int32_t num_experts, int32_t tile_expert_count,
+                                            const uint64_t *expert_sort_keys, uint64_t expert_sort_key_count,
+                                            tf_prefill_pair *sorted_pairs, uint32_t *per_expert_offsets,
+                                            uint32_t *per_expert_counts, tf_prefill_group *groups, uint32_t *group_count,
+                                            tf_prefill_tile *tiles, uint32_t *tile_count);
+/* The same grouping (no sort keys) done on the DEVICE straight from the router's outputs, so a resident-expert pipeline
+ * needs no host round trip: sorted_pairs[T*top_k] ordered by (expert, token, rank), per_expert_offsets / per_expert_counts
+ * [num_experts], and a work list `chunks` (runs of <= 64 sorted pairs sharing one expert) with its length in chunk_count[0].
+ * chunks capacity: num_experts + T*top_k/64 entries.  Expert ids are clamped to num_experts - 1
+ * (RealForwardRunner.swift:955); the experts of one token must be distinct (the router guarantees it). */
+int32_t tf_prefill_group_pairs_device(tf_ctx *ctx, tf_stream stream, const void *indices, const void *weights,
+                                      uint32_t query_count, uint32_t top_k, uint32_t num_experts,
+                                      void *sorted_pairs, void *per_expert_offsets, void *per_expert_counts,
+                                      void *chunks, void *chunk_count);
+
+/* PrefillGroupedRoutedMoE.encodeStreamedBatched (PrefillGroupedRoutedMoE.swift:386-461) -> prefill_grouped_routed_moe_
+ * batched_phase1 / _down (prefill.metal:598-670): for the sorted pairs [pair_start, pair_start + pair_count) of one tile,
+ * route_partials[(token*top_k + rank)*d + c] = half(down_c . half(gelu(gate . x) * (up . x))), unweighted.  `blobs`: HOST array
+ * of live_expert_count device pointers bound to params->local_expert[i].  `tile_groups`: HOST array, the groups of this tile
+ * (PrefillMoEGroupedRoutes.groups[tile.groupStart ..< tile.groupStart + tile.groupCount]).  Pairs are processed in
+ * micro-batches of pair_microbatch_rows (reference default 32) so that gate_up_act_scratch needs 3 * rows * F halves and
+ * down_scratch rows * d halves, as in the reference; *out_microbatches (may be NULL) receives the micro-batch count.
+ * Pairs whose expert is not bound are skipped. */
+int32_t tf_prefill_grouped_routed_moe_streamed(tf_ctx *ctx, tf_stream stream,
+                                               const void *hidden, uint64_t hidden_offset,
+                                               const void *sorted_pairs, uint64_t sorted_pairs_offset,
+                                               void *route_partials, uint64_t route_partials_offset,
+                                               void *gate_up_act_scratch, uint64_t gate_up_act_scratch_offset,
+                                               void *down_scratch, uint64_t down_scratch_offset,
+                                               const void *const *blobs, const tf_prefill_streamed_params *params,
+                                               const tf_prefill_group *tile_groups, uint32_t tile_group_count,
+                                               int32_t pair_microbatch_rows, int32_t *out_microbatches, tf_dtype scale_dtype);
+/* Resident-pool form of the same computation over ALL sorted pairs of a chunk of tokens in one go: experts are
+ * pool + expert * pool_stride, the work list comes from tf_prefill_group_pairs_device, nothing is read by the host.  Groups
+ * of a few pairs stream each expert row once and apply it to every routed token (weight-read bound, the small-M regime);
+ * large groups run as a grouped GEMM on the matrix cores (weights expanded to fp16 in LDS, fp32 accumulation).
+ * acts_scratch: pair_count * f halves.  max_chunks: capacity of `chunks`. */
+int32_t tf_prefill_grouped_routed_moe_resident(tf_ctx *ctx, tf_stream stream,
+                                               const void *hidden, uint64_t hidden_offset, uint32_t hidden_stride_elements,
+                                               const void *sorted_pairs, const void *chunks, const void *chunk_count,
+                                               uint32_t max_chunks, uint32_t pair_count,
+                                               const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                               const tf_expert_offsets *routed_offsets,
+                                               void *acts_scratch, void *route_partials,
+                                               uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype);
+/* PrefillMoE.encodeReduceTokenMajor (Kernels/Prefill/MoE/PrefillMoE.swift:11-38) -> prefill_moe_reduce_token_major
+ * (prefill.metal:575-596): h2[t, c] = half(sum_r float(w[t, r]) * float(partial[t, r, c])), r ascending, fused multiply-adds. */
+int32_t tf_prefill_moe_reduce_token_major(tf_ctx *ctx, tf_stream stream,
+                                          const void *route_partials, uint64_t route_partials_offset,
+                                          const void *route_weights, uint64_t route_weights_offset,
+                                          void *h2, uint64_t h2_offset, uint32_t query_count, uint32_t top_k, uint32_t d);
+
+/* MPPPrefillInt4QMM.encode (Kernels/TensorCore/MPPPrefillInt4QMM.swift:34-77) -> mpp_prefill_affine_threadgroup_f16
+ * (Metal/TensorCore/tensorops.metal:13-105): y[m, n] fp16 [M, N] = x[M, K] . W[N, K]^T, weights expanded to fp16
+ * half(q*s+b) per K group, fp32 accumulation on the matrix cores.  Returns TF_ERR_UNAVAILABLE (the reference's
+ * Path.unavailable) when m, n, k <= 0, k % 64 != 0 or an operand is not 16-byte aligned; nothing is enqueued then. */
+int32_t tf_int4_qmm(tf_ctx *ctx, tf_stream stream,
+                    const void *weights, uint64_t weights_offset,
+                    const void *scales, uint64_t scales_offset,
+                    const void *biases, uint64_t biases_offset,
+                    const void *x, uint64_t x_offset, void *y, uint64_t y_offset,
+                    int32_t m, int32_t n, int32_t k, tf_dtype scale_dtype);
+/* PrefillInt4QMM.encode (Kernels/Prefill/Primitives/PrefillPrimitives.swift:73-109) -> prefill_dequant_int4_qmm_f16_block
+ * (prefill.metal:672-709): the same product with fp32 weights q*s+b (no fp16 rounding of the weight): every token row
+ * goes through the GEMV arithmetic, so QMM == repeated GEMV.  Any 2-byte alignment. */
+int32_t tf_prefill_int4_qmm(tf_ctx *ctx, tf_stream stream,
+                            const void *weights, uint64_t weights_offset,
+                            const void *scales, uint64_t scales_offset,
+                            const void *biases, uint64_t biases_offset,
+                            const void *x, uint64_t x_offset, void *y, uint64_t y_offset,
+                            int32_t t, int32_t n, int32_t k, tf_dtype scale_dtype);
+
 #ifdef __cplusplus
 }
 #endif

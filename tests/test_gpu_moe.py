@@ -99,15 +99,16 @@ def run_moe(c, split=False, blob_prefix=None, pool_mode=False):
         perm = [5, 11, 2, 7, 0, 15, 9, 3]
         for slot, e in enumerate(perm):
             pool_np[e * stride:e * stride + c["blobs"][slot].size] = c["blobs"][slot]
-        pool = dev(pool_np)
-        routed = k.routed_from_pool(pool, stride, dev(np.array(perm, np.uint32)), 16)
-        keep = pool
+        pool, d_perm = dev(pool_np), dev(np.array(perm, np.uint32))
+        routed = k.routed_from_pool(pool, stride, d_perm, 16)
+        keep = (pool, d_perm)
     else:
         routed = k.routed_from_pointers(ptrs)
         keep = blobs
     if split:
         for slots in ([0, 1, 2, 3], [4, 5, 6, 7]):
-            k.moe_phase1(routed, off, x, acts, d, f, active_slots=dev(np.array(slots, np.uint32)), active_count=4)
+            d_slots = dev(np.array(slots, np.uint32))
+            k.moe_phase1(routed, off, x, acts, d, f, active_slots=d_slots, active_count=4)
     else:
         k.moe_phase1(routed, off, x, acts, d, f)
     k.moe_phase2(routed, off, acts, rw, res, y, d, f)

@@ -1,0 +1,318 @@
+"""GPU parity of the prefill / multi-token path through the C ABI: per-token router, device grouping, grouped routed experts
+(reference-shaped streamed tile and resident pool; row-streaming and matrix-core variants), token-major reduce, int4 QMM.
+Cases restate PrefillRouterTests, PrefillGroupedRoutedMoETests+Execution, PrefillMoETests, MPPPrefillInt4QMMTests."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import refcases
+from gpu_helpers import ctx, dev, host, tfk, within_north_star, zeros_bytes
+from oracle import tfo
+
+pytestmark = pytest.mark.gpu
+
+
+def prefill_router(W, S, B, hidden_bits, stride, eff_bits, pes_bits, rows, top_k=8, hidden_off=0):
+    e, d = W.shape
+    k = ctx()
+    hid = dev(hidden_bits, hidden_off)
+    before = host(hid, np.uint8).copy()
+    idx, wts = zeros_bytes(rows * top_k * 4), zeros_bytes(rows * top_k * 2)
+    dW, dS, dB, dE, dP = dev(W), dev(S), dev(B), dev(eff_bits), dev(pes_bits)   # keep the tensors alive across the call
+    k.check(k.lib.tf_prefill_router_gemma4_block(k.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0,
+                                                 hid.data_ptr(), hidden_off, dE.data_ptr(), 0, dP.data_ptr(), 0,
+                                                 idx.data_ptr(), 0, wts.data_ptr(), 0, rows, e, d, top_k, stride))
+    torch.cuda.synchronize()
+    assert np.array_equal(host(hid, np.uint8), before), "router wrote into the hidden block"
+    return host(idx, np.uint32, rows * top_k).reshape(rows, top_k), tfo.from_f16_bits(host(wts, np.uint16, rows * top_k)).reshape(rows, top_k)
+
+
+def decode_router(W, S, B, hidden_bits, eff_bits, pes_bits):
+    e, d = W.shape
+    idx, wts = zeros_bytes(32), zeros_bytes(16)
+    ctx().router_gemma4(dev(W), dev(S), dev(B), dev(hidden_bits), dev(eff_bits), dev(pes_bits), idx, wts, e, d)
+    return host(idx, np.uint32, 8), tfo.from_f16_bits(host(wts, np.uint16, 8))
+
+
+@pytest.mark.parametrize("stride_pad,hidden_off", [(13, 0), (16, 0), (0, 32)])
+def test_block_router_matches_repeated_scalar_rows(stride_pad, hidden_off):
+    # PrefillRouterTests.swift:33-103
+    experts, d, rows = 16, 128, 3
+    rng = tfo.SplitMix64(0x9A7E2026)
+    weights = np.stack([rng.uniform_array(-0.04, 0.04, d) + np.float32(e) * np.float32(0.015) for e in range(experts)])
+    stride = d + stride_pad
+    hidden = np.full(rows * stride, tfo.f16_bits(-31.0), np.uint16)
+    for r in range(rows):
+        hidden[r * stride:r * stride + d] = tfo.to_f16_bits(rng.uniform_array(-1.0, 1.0, d))
+    eff = tfo.bf16_bits_array(rng.uniform_array(0.5, 1.5, d) / np.sqrt(np.float32(d)))
+    pes = tfo.bf16_bits_array(rng.uniform_array(0.6, 1.4, experts))
+    W, S, B = tfo.quantize_int8(weights)
+    got_idx, got_w = prefill_router(W, S, B, hidden, stride, eff, pes, rows, hidden_off=hidden_off)
+    for r in range(rows):
+        row_bits = hidden[r * stride:r * stride + d]
+        d_idx, d_w = decode_router(W, S, B, row_bits, eff, pes)
+        assert list(got_idx[r]) == list(d_idx)
+        assert np.max(np.abs(got_w[r] - d_w)) <= 5e-3
+        ref_idx, ref_w, _ = tfo.router_reference(W, S, B, tfo.from_f16_bits(row_bits), tfo.bf16_array_to_float(eff), tfo.bf16_array_to_float(pes))
+        assert list(got_idx[r]) == list(ref_idx) and np.max(np.abs(got_w[r] - ref_w)) <= 5e-3
+
+
+def test_block_router_near_tie_and_generic_topk():
+    # PrefillRouterTests.swift:105-146: same near-tie winner as the scalar path
+    experts, d = 16, 128
+    gains = [1.0 - e * 0.05 for e in range(7)] + [0.5, 0.5 * (1 + 1e-4)] + [0.4 - (e - 9) * 0.02 for e in range(9, 16)]
+    pattern = (np.float32(0.25) + ((np.arange(d) * 37 + 11) % 97).astype(np.float32) / np.float32(97.0))
+    weights = np.array(gains, np.float32)[:, None] * pattern[None, :]
+    W, S, B = tfo.quantize_int8(weights.astype(np.float32))
+    hid = tfo.to_f16_bits(np.ones(d, np.float32))
+    eff, pes = tfo.bf16_bits_array(np.ones(d, np.float32)), tfo.bf16_bits_array(np.ones(experts, np.float32))
+    got_idx, _ = prefill_router(W, S, B, hid, d, eff, pes, 1)
+    assert list(got_idx[0]) == list(decode_router(W, S, B, hid, eff, pes)[0]) == [0, 1, 2, 3, 4, 5, 6, 8]
+    # generic top_k (PrefillRouter.swift:62: 1...64): top-3 is the prefix of top-8, weights are a softmax over three
+    idx3, w3 = prefill_router(W, S, B, hid, d, eff, pes, 1, top_k=3)
+    assert list(idx3[0]) == [0, 1, 2] and abs(float(w3.sum()) - 1.0) < 2e-3
+    k = ctx()
+    z = zeros_bytes(64)
+    bad = k.lib.tf_prefill_router_gemma4_block(k.handle, None, z.data_ptr(), 0, z.data_ptr(), 0, z.data_ptr(), 0, z.data_ptr(), 0, z.data_ptr(), 0,
+                                               z.data_ptr(), 0, z.data_ptr(), 0, z.data_ptr(), 0, 1, 16, 128, 65, 128)
+    assert bad == tfk.TF_ERR_INVALID_ARGUMENT
+
+
+def device_grouping(idx, wts_bits, T, top_k, E):
+    k = ctx()
+    n = T * top_k
+    cap = E + n // 64 + 1
+    sp, offs, cnts = zeros_bytes(n * 16), zeros_bytes(E * 4), zeros_bytes(E * 4)
+    chunks, nch = zeros_bytes(cap * 12), zeros_bytes(4)
+    d_idx, d_w = dev(np.ascontiguousarray(idx, np.uint32)), dev(np.ascontiguousarray(wts_bits, np.uint16))
+    k.check(k.lib.tf_prefill_group_pairs_device(k.handle, None, d_idx.data_ptr(), d_w.data_ptr(), T, top_k, E, sp.data_ptr(),
+                                                offs.data_ptr(), cnts.data_ptr(), chunks.data_ptr(), nch.data_ptr()))
+    return dict(sorted_pairs=sp, offsets=offs, counts=cnts, chunks=chunks, n_chunks=nch, cap=cap, keep=(d_idx, d_w))
+
+
+@pytest.mark.parametrize("T,top_k,E", [(4, 3, 6), (32, 8, 128), (300, 8, 128), (2048, 8, 128), (16, 8, 16)])
+def test_device_grouping_equals_host_grouping(T, top_k, E):
+    rng = np.random.default_rng(T + E)
+    p = 1.0 / np.arange(1, E + 1) ** 1.1
+    p /= p.sum()
+    idx = np.stack([rng.choice(E, size=top_k, replace=False, p=p) for _ in range(T)]).astype(np.uint32)
+    w = rng.integers(1, 0x3C00, (T, top_k)).astype(np.uint16)
+    g = device_grouping(idx, w, T, top_k, E)
+    pairs = tfk.make_token_expert_pairs(idx.ravel(), w.ravel(), T, top_k)
+    ref = tfk.group_token_expert_pairs([(q.token, q.expert, q.rank, q.weight_bits_and_reserved) for q in pairs[:T * top_k]], T, top_k, E)
+    got = host(g["sorted_pairs"], np.uint32, T * top_k * 4).reshape(-1, 4)
+    assert [tuple(int(v) for v in r) for r in got] == ref["sorted_pairs"]
+    assert list(host(g["offsets"], np.uint32, E)) == ref["per_expert_offsets"]
+    assert list(host(g["counts"], np.uint32, E)) == ref["per_expert_counts"]
+    nch = int(host(g["n_chunks"], np.uint32, 1)[0])
+    chunks = host(g["chunks"], np.uint32, nch * 3).reshape(nch, 3)
+    covered = []
+    for e, s, c in chunks:
+        assert 1 <= c <= 64 and all(int(x) == int(e) for x in got[s:s + c, 1])
+        covered.extend(range(int(s), int(s + c)))
+    assert covered == list(range(T * top_k)) and nch <= g["cap"]
+
+
+def test_streamed_batched_matches_reference_across_partial_microbatch():
+    # PrefillGroupedRoutedMoETests+Execution.swift:8-103
+    d = f = 64
+    rows, top_k = 3, 2
+    rank_w = lambda r: tfo.f16_bits(0.125 + r * 0.0625)
+    raw = [(0, 2, 0), (0, 0, 1), (1, 1, 0), (1, 2, 1), (2, 0, 0), (2, 1, 1)]
+    routes = tfk.group_token_expert_pairs([(t, e, r, rank_w(r)) for t, e, r in raw], rows, top_k, 16, 16)
+    pool, off, stride = refcases.synthetic_expert_pool(16, d, f)
+    hidden = tfo.to_f16_bits(((np.arange(rows * d) % 17) - 8).astype(np.float32) * np.float32(0.01))
+    sp_np = np.array(routes["sorted_pairs"], np.uint32)
+    expected = tfo.prefill_route_partials(np.array([tuple(r) for r in sp_np], tfo.PAIR_DTYPE), rows, hidden, d, pool, stride, off,
+                                          top_k, d, f, fill_bits=tfo.f16_bits(-77.0))
+    k = ctx()
+    # every expert lives in its own allocation at a non-zero offset (64 + 16 * index), as in the reference test
+    blob_t, ptrs = [], (C.c_void_p * 16)()
+    for i in range(16):
+        prefix = 64 + i * 16
+        t = dev(pool[i * stride:(i + 1) * stride], prefix)
+        blob_t.append(t)
+        ptrs[i] = t.data_ptr() + prefix
+    params = tfk.StreamedParams()
+    params.pair_start, params.pair_count, params.d, params.routed_intermediate = 0, len(raw), d, f
+    params.top_k, params.hidden_stride_elements, params.live_expert_count = top_k, d, 16
+    for i in range(16):
+        params.local_expert[i] = i
+    for name, v in zip([n for n, _ in tfo.ExpertOffsets._fields_], off.as_tuple()):
+        setattr(params, name, v)
+    groups = (tfk.PrefillGroup * len(routes["groups"]))(*[tfk.PrefillGroup(*g) for g in routes["groups"]])
+    out = dev(np.full(rows * top_k * d, tfo.f16_bits(-77.0), np.uint16))
+    scratch_act, scratch_down = zeros_bytes(3 * 4 * f * 2), zeros_bytes(4 * d * 2)
+    nmb = C.c_int32(0)
+    d_hidden, d_sp = dev(hidden), dev(sp_np)
+    rc = k.lib.tf_prefill_grouped_routed_moe_streamed(k.handle, None, d_hidden.data_ptr(), 0, d_sp.data_ptr(), 0, out.data_ptr(), 0,
+                                                      scratch_act.data_ptr(), 0, scratch_down.data_ptr(), 0, C.cast(ptrs, C.c_void_p), C.byref(params),
+                                                      C.cast(groups, C.c_void_p), len(routes["groups"]), 4, C.byref(nmb), tfk.TF_BF16)
+    assert rc == tfk.TF_OK, k.last_error()
+    got = tfo.from_f16_bits(host(out, np.uint16, rows * top_k * d))
+    assert nmb.value == 2
+    assert np.max(np.abs(got - tfo.from_f16_bits(expected))) <= 0.0015
+    del blob_t
+
+
+def resident_pipeline(T, E, d, f, top_k, seed, zipf=False, from_router=True):
+    """router block -> device grouping -> grouped experts (resident pool) -> token-major reduce; returns everything needed to check."""
+    rng = np.random.default_rng(seed)
+    blobs, off = [], None
+    for e in range(E):
+        blob, off = tfo.make_blob(refcases.synthetic_int4(f, d, seed + e, "g"), refcases.synthetic_int4(f, d, seed + e, "u"),
+                                  refcases.synthetic_int4(d, f, seed + e, "d"))
+        blobs.append(blob)
+    stride = (blobs[0].size + 255) // 256 * 256
+    pool_np = np.zeros((E, stride), np.uint8)
+    for e, b in enumerate(blobs):
+        pool_np[e, :b.size] = b
+    hidden = rng.standard_normal((T, d)).astype(np.float16).view(np.uint16)
+    k = ctx()
+    if from_router:
+        rW, rS, rB = refcases.synthetic_int8(E, d, seed)
+        eff = tfo.bf16_bits_array((rng.uniform(0.5, 1.5, d) / np.sqrt(d)).astype(np.float32))
+        pes = tfo.bf16_bits_array(rng.uniform(0.6, 1.4, E).astype(np.float32))
+        idx, w = prefill_router(rW, rS, rB, hidden.ravel(), d, eff, pes, T, top_k=top_k)
+        w_bits = tfo.to_f16_bits(w)
+    else:
+        p = 1.0 / np.arange(1, E + 1) ** 1.1
+        p /= p.sum()
+        idx = np.stack([rng.choice(E, size=top_k, replace=False, p=p if zipf else None) for _ in range(T)]).astype(np.uint32)
+        w_bits = tfo.to_f16_bits(rng.dirichlet(np.ones(top_k), T).astype(np.float32))
+    g = device_grouping(idx, w_bits, T, top_k, E)
+    n = T * top_k
+    acts, partials, h2 = zeros_bytes(n * f * 2), zeros_bytes(n * d * 2), zeros_bytes(T * d * 2)
+    koff = tfk.ExpertOffsets(*off.as_tuple())
+    d_pool, d_hidden, d_w = dev(pool_np), dev(hidden), dev(np.ascontiguousarray(w_bits, np.uint16))
+    k.check(k.lib.tf_prefill_grouped_routed_moe_resident(k.handle, None, d_hidden.data_ptr(), 0, d, g["sorted_pairs"].data_ptr(),
+                                                         g["chunks"].data_ptr(), g["n_chunks"].data_ptr(), g["cap"], n, d_pool.data_ptr(),
+                                                         stride, E, C.byref(koff), acts.data_ptr(), partials.data_ptr(), d, f, top_k, tfk.TF_BF16))
+    k.check(k.lib.tf_prefill_moe_reduce_token_major(k.handle, None, partials.data_ptr(), 0, d_w.data_ptr(), 0, h2.data_ptr(), 0, T, top_k, d))
+    sp = host(g["sorted_pairs"], np.uint32, n * 4).reshape(n, 4)
+    return dict(blobs=blobs, off=off, pool=pool_np.ravel(), stride=stride, hidden=hidden, idx=np.asarray(idx), w_bits=np.asarray(w_bits).reshape(T, top_k),
+                sorted_pairs=np.array([tuple(r) for r in sp], tfo.PAIR_DTYPE), partials=host(partials, np.uint16, n * d),
+                h2=tfo.from_f16_bits(host(h2, np.uint16, T * d)).reshape(T, d))
+
+
+def check_against_oracle(r, T, d, f, top_k, abs_tol, rel_tol=1e-2):
+    want_partials = tfo.prefill_route_partials(r["sorted_pairs"], T, r["hidden"].ravel(), d, r["pool"], r["stride"], r["off"], top_k, d, f,
+                                               fill_bits=0, threads=8)
+    got, want = tfo.from_f16_bits(r["partials"]), tfo.from_f16_bits(want_partials)
+    assert within_north_star(got, want, rel=rel_tol, abs_=abs_tol)
+    want_h2 = tfo.from_f16_bits(tfo.prefill_reduce_token_major(want_partials, r["w_bits"].ravel(), T, top_k, d)).reshape(T, d)
+    assert within_north_star(r["h2"], want_h2, rel=rel_tol, abs_=abs_tol)
+    # and against the all-fp32 reference the decode path is judged by (Moe.swift:60-89)
+    for t in range(min(T, 3)):
+        ref = tfo.moe_apply_streamed_routed([r["blobs"][int(e)] for e in r["idx"][t]], r["off"], tfo.from_f16_bits(r["hidden"][t]),
+                                            np.zeros(d, np.float32), tfo.from_f16_bits(r["w_bits"][t]), d, f, threads=8)
+        assert tfo.rel_error(r["h2"][t], ref) < tfo.Tolerance.fp16ChainedReduction
+
+
+@pytest.mark.parametrize("M", [2, 4, 8, 16])
+def test_small_m_resident_pipeline_matches_oracle(M):
+    # BASELINE config 3: M tokens, top-8 over the production expert shape; small groups take the row-streaming kernels
+    E, d, f, top_k = 32, 2816, 704, 8
+    r = resident_pipeline(M, E, d, f, top_k, 0x300 + M)
+    scale = float(np.max(np.abs(tfo.from_f16_bits(r["partials"]))))
+    check_against_oracle(r, M, d, f, top_k, abs_tol=1e-3 * max(1.0, scale))
+
+
+def test_small_m_equals_decode_step_per_token():
+    # the multi-token pipeline and the batch-1 decode kernels must agree token by token (same arithmetic up to fp16 rounding of partials)
+    E, d, f, top_k, M = 16, 2816, 704, 8, 4
+    r = resident_pipeline(M, E, d, f, top_k, 0x3AA)
+    k = ctx()
+    koff = tfk.ExpertOffsets(*r["off"].as_tuple())
+    d_pool = dev(r["pool"])
+    for t in range(M):
+        d_idx, d_x, d_w, d_res = dev(r["idx"][t].astype(np.uint32)), dev(r["hidden"][t]), dev(r["w_bits"][t]), zeros_bytes(d * 2)
+        routed = k.routed_from_pool(d_pool, r["stride"], d_idx, E)
+        acts, y = zeros_bytes(8 * f * 2), zeros_bytes(d * 2)
+        k.moe_phase1(routed, koff, d_x, acts, d, f)
+        k.moe_phase2(routed, koff, acts, d_w, d_res, y, d, f)
+        dec = tfo.from_f16_bits(host(y, np.uint16, d))
+        assert np.max(np.abs(dec - r["h2"][t])) <= 4e-3 * max(1.0, float(np.max(np.abs(dec))))
+
+
+@pytest.mark.parametrize("T,E,d,f,zipf", [(64, 16, 2816, 704, True), (96, 8, 512, 128, False), (200, 16, 256, 192, True)])
+def test_grouped_gemm_on_matrix_cores_matches_oracle(T, E, d, f, zipf):
+    # BASELINE config 4 in miniature: enough pairs per expert for the MFMA path (pairs >= 8 * experts), Zipf-skewed routing
+    top_k = 8
+    r = resident_pipeline(T, E, d, f, top_k, 0x400 + T, zipf=zipf, from_router=False)
+    scale = float(np.max(np.abs(tfo.from_f16_bits(r["partials"]))))
+    check_against_oracle(r, T, d, f, top_k, abs_tol=2e-3 * max(1.0, scale))
+
+
+def test_token_major_reduce_matches_cpu_reference():
+    # PrefillMoETests.swift:11-44
+    rows, top_k, d = 3, 8, 64
+    rng = tfo.SplitMix64(0x4D0E2026)
+    partials = tfo.to_f16_bits(rng.uniform_array(-2.0, 2.0, rows * top_k * d))
+    weights = tfo.to_f16_bits(rng.uniform_array(-1.0, 1.0, rows * top_k))
+    h2 = dev(np.full(rows * d, tfo.f16_bits(-19.0), np.uint16))
+    k = ctx()
+    d_p, d_w = dev(partials), dev(weights)
+    k.check(k.lib.tf_prefill_moe_reduce_token_major(k.handle, None, d_p.data_ptr(), 0, d_w.data_ptr(), 0, h2.data_ptr(), 0, rows, top_k, d))
+    got = tfo.from_f16_bits(host(h2, np.uint16, rows * d))
+    want = tfo.from_f16_bits(tfo.prefill_reduce_token_major(partials, weights, rows, top_k, d))
+    assert np.max(np.abs(got - want)) <= 2e-3
+    assert k.lib.tf_prefill_moe_reduce_token_major(k.handle, None, h2.data_ptr(), 0, h2.data_ptr(), 0, h2.data_ptr(), 0, 0, 8, 64) == tfk.TF_ERR_INVALID_ARGUMENT
+
+
+def mpp_inputs(m, n, k, adversarial=False):
+    # MPPPrefillInt4QMMTests.swift:19-60
+    groups = k // 64
+    W = ((np.arange(n * k // 2, dtype=np.uint64) * 37 + 0x29) & 0xFF).astype(np.uint8).reshape(n, k // 2)
+    r, g = np.arange(n)[:, None], np.arange(groups)[None, :]
+    if adversarial:
+        sc = np.array([tfo.bf16_bits(0.001), tfo.bf16_bits(-0.0015), 0x0001, 0x8001], np.uint16)
+        bi = np.array([tfo.bf16_bits(-0.01), tfo.bf16_bits(0.006), 0x0001, 0x8001], np.uint16)
+        S, B = sc[(r + g) % 4], bi[(r * 3 + g) % 4]
+    else:
+        S = tfo.bf16_bits_array(np.float32(0.001) + ((r + g) % 5).astype(np.float32) * np.float32(0.00025)).reshape(n, groups)
+        B = tfo.bf16_bits_array(np.float32(-0.01) + ((r * 3 + g) % 7).astype(np.float32) * np.float32(0.002)).reshape(n, groups)
+    x = tfo.to_f16_bits(((np.arange(m * k) * 11) % 29 - 14).astype(np.float32) / np.float32(64.0))
+    return W, np.ascontiguousarray(S), np.ascontiguousarray(B), x
+
+
+@pytest.mark.parametrize("m,n,k,adv", [(64, 32, 64, False), (128, 64, 128, False), (33, 70, 192, True), (5, 40, 128, False),
+                                       (32, 2112, 2816, False), (32, 2816, 2112, False), (100, 704, 2816, True), (32, 2816, 704, False)])
+def test_int4_qmm_on_matrix_cores(m, n, k, adv):
+    # MPPPrefillInt4QMMTests.swift:183-200 (rel <= 1e-3 vs the fp32-fma CPU reference rounded to fp16) + production shapes
+    W, S, B, x = mpp_inputs(m, n, k, adv)
+    kk = ctx()
+    y = zeros_bytes(m * n * 2 + 64, 0xEE)
+    dW, dS, dB, dx = dev(W), dev(S), dev(B), dev(x)
+    rc = kk.lib.tf_int4_qmm(kk.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dx.data_ptr(), 0,
+                            y.data_ptr(), 0, m, n, k, tfk.TF_BF16)
+    assert rc == tfk.TF_OK, kk.last_error()
+    got = tfo.from_f16_bits(host(y, np.uint16, m * n)).reshape(m, n)
+    assert np.all(host(y, np.uint8)[m * n * 2:] == 0xEE)
+    want = tfo.qmm_cpu_reference(W, S, B, x, m, n, k, threads=8)
+    assert tfo.rel_error(got, want) <= 1e-3
+    assert within_north_star(got, want)
+
+
+def test_int4_qmm_unavailable_and_exact_variant():
+    W, S, B, x = mpp_inputs(8, 64, 128)
+    kk = ctx()
+    y = zeros_bytes(8 * 64 * 2, 0xEE)
+    dW, dS, dB, dx = dev(W, 2), dev(S), dev(B), dev(x)
+    # k not a multiple of 64 / misaligned weights: Path.unavailable, nothing enqueued (MPPPrefillInt4QMM.swift:40-56)
+    assert kk.lib.tf_int4_qmm(kk.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dx.data_ptr(), 0, y.data_ptr(), 0, 8, 64, 96, tfk.TF_BF16) == tfk.TF_ERR_UNAVAILABLE
+    assert kk.lib.tf_int4_qmm(kk.handle, None, dW.data_ptr(), 2, dS.data_ptr(), 0, dB.data_ptr(), 0, dx.data_ptr(), 0, y.data_ptr(), 0, 8, 64, 128, tfk.TF_BF16) == tfk.TF_ERR_UNAVAILABLE
+    assert kk.lib.tf_int4_qmm(kk.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dx.data_ptr(), 0, y.data_ptr(), 0, 0, 64, 128, tfk.TF_BF16) == tfk.TF_ERR_UNAVAILABLE
+    torch.cuda.synchronize()
+    assert np.all(host(y, np.uint8) == 0xEE)
+    # the exact (fp32 weight) QMM equals repeated GEMV bit for bit, at the +2 weight offset too (PrefillAffineTests.swift:176-231)
+    kk.check(kk.lib.tf_prefill_int4_qmm(kk.handle, None, dW.data_ptr(), 2, dS.data_ptr(), 0, dB.data_ptr(), 0, dx.data_ptr(), 0, y.data_ptr(), 0, 8, 64, 128, tfk.TF_BF16))
+    got = host(y, np.uint16, 8 * 64).reshape(8, 64)
+    for t in range(8):
+        yr = zeros_bytes(64 * 2)
+        kk.dequant_int4_gemv(dW, dS, dB, dev(x[t * 128:(t + 1) * 128]), yr, 64, 128, offsets=(2, 0, 0, 0, 0))
+        assert np.array_equal(host(yr, np.uint16, 64), got[t])
+    ref = tfo.qmm_cpu_reference(W, S, B, x, 8, 64, 128)
+    assert np.max(np.abs(tfo.from_f16_bits(got.ravel()).reshape(8, 64) - ref)) <= 2e-4 + 5e-4 * np.max(np.abs(ref))

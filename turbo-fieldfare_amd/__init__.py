@@ -55,6 +55,30 @@ class PrefillPair(C.Structure):
     _fields_ = [("token", u32), ("expert", u32), ("rank", u32), ("weight_bits_and_reserved", u32)]
 
 
+class PrefillGroup(C.Structure):
+    """tf_prefill_group."""
+    _fields_ = [("expert", u32), ("pair_start", u32), ("pair_count", u32)]
+
+
+class PrefillTile(C.Structure):
+    """tf_prefill_tile."""
+    _fields_ = [("group_start", u32), ("group_count", u32), ("pair_start", u32), ("pair_count", u32)]
+
+
+class StreamedParams(C.Structure):
+    """tf_prefill_streamed_params (128 bytes)."""
+    _fields_ = ([(n, u32) for n in ("pair_start", "pair_count", "d", "routed_intermediate", "top_k", "hidden_stride_elements",
+                                    "live_expert_count")]
+                + [("local_expert", u32 * 16)]
+                + [(n, u32) for n in ("gate_W_off", "gate_s_off", "gate_b_off", "up_W_off", "up_s_off", "up_b_off",
+                                      "down_W_off", "down_s_off", "down_b_off")])
+
+
+GROUP_ERRORS = {-101: "invalidQueryCount", -102: "invalidTopK", -103: "invalidNumExperts", -104: "invalidTileExpertCount",
+                -105: "pairCountMismatch", -106: "tokenOutOfRange", -107: "rankOutOfRange", -108: "expertOutOfRange",
+                -109: "duplicateTokenRank", -110: "expertSortKeyCountMismatch"}
+
+
 class TFError(RuntimeError):
     def __init__(self, status: int, message: str):
         super().__init__(f"tf_kernels status {status}: {message}")
@@ -86,6 +110,18 @@ EXPORTS = {
                                         u32, i32]),
     "tf_moe_decode_step": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, vp, u64, vp, u64, vp, u64, u32, C.POINTER(ExpertOffsets),
                                  vp, vp, vp, vp, vp, vp, u32, u32, u32, i32]),
+    "tf_prefill_router_gemma4_block": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64,
+                                             u32, u32, u32, u32, u32]),
+    "tf_prefill_make_token_expert_pairs": (i32, [vp, vp, i32, i32, vp]),
+    "tf_prefill_group_token_expert_pairs": (i32, [vp, u64, i32, i32, i32, i32, vp, u64, vp, vp, vp, vp, vp, vp, vp]),
+    "tf_prefill_group_pairs_device": (i32, [vp, vp, vp, vp, u32, u32, u32, vp, vp, vp, vp, vp]),
+    "tf_prefill_grouped_routed_moe_streamed": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp,
+                                                     C.POINTER(StreamedParams), vp, u32, i32, C.POINTER(i32), i32]),
+    "tf_prefill_grouped_routed_moe_resident": (i32, [vp, vp, vp, u64, u32, vp, vp, vp, u32, u32, vp, u64, u32,
+                                                     C.POINTER(ExpertOffsets), vp, vp, u32, u32, u32, i32]),
+    "tf_prefill_moe_reduce_token_major": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32, u32, u32]),
+    "tf_int4_qmm": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, i32, i32, i32, i32]),
+    "tf_prefill_int4_qmm": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, i32, i32, i32, i32]),
     "tf_lm_head_greedy_int4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u32, u32, C.c_float, i32]),
     "tf_lm_head_logits_int4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, C.c_float,
                                      i32, i32]),
@@ -251,3 +287,52 @@ class Context:
 
 def projection(W, S, B, rows: int, cols: int, offsets=(0, 0, 0)) -> Projection:
     return Projection(_p(W), offsets[0], _p(S), offsets[1], _p(B), offsets[2], rows, cols)
+
+
+# ---- host-side grouping (pure CPU functions of the library) ----------------------------------------------------------
+def make_token_expert_pairs(indices, weights_f16_bits, query_count: int, top_k: int):
+    """PrefillRouter.makeTokenExpertPairs over numpy arrays -> (PrefillPair * n)."""
+    import numpy as np
+    lib = load()
+    idx = np.ascontiguousarray(indices, np.uint32)
+    w = np.ascontiguousarray(weights_f16_bits, np.uint16)
+    pairs = (PrefillPair * max(1, query_count * top_k))()
+    rc = lib.tf_prefill_make_token_expert_pairs(idx.ctypes.data, w.ctypes.data, query_count, top_k, C.cast(pairs, vp))
+    if rc != TF_OK:
+        raise TFError(rc, "make_token_expert_pairs")
+    return pairs
+
+
+def group_token_expert_pairs(pairs, query_count: int, top_k: int, num_experts: int, tile_expert_count: int = 16,
+                             expert_sort_keys=None):
+    """PrefillMoEGrouping.groupTokenExpertPairs.  `pairs`: sequence of (token, expert, rank, weight_bits) or PrefillPair array.
+    Returns a dict of python lists; raises TFError whose .status is one of the TF_ERR_GROUP_* codes."""
+    lib = load()
+    if not isinstance(pairs, C.Array):
+        arr = (PrefillPair * max(1, len(pairs)))()
+        for i, p in enumerate(pairs):
+            arr[i] = PrefillPair(*p)
+        n = len(pairs)
+    else:
+        arr, n = pairs, len(pairs)
+    ne = max(num_experts, 1)
+    cap = max(1, min(ne, max(n, 1)))
+    sorted_pairs = (PrefillPair * max(1, n))()
+    offs, cnts = (u32 * ne)(), (u32 * ne)()
+    groups, tiles = (PrefillGroup * cap)(), (PrefillTile * cap)()
+    ng, nt = u32(0), u32(0)
+    keys, nkeys = None, 0
+    if expert_sort_keys is not None:
+        keys_arr = (u64 * len(expert_sort_keys))(*expert_sort_keys)
+        keys, nkeys = C.cast(keys_arr, vp), len(expert_sort_keys)
+    rc = lib.tf_prefill_group_token_expert_pairs(C.cast(arr, vp), n, query_count, top_k, num_experts, tile_expert_count, keys, nkeys,
+                                                 C.cast(sorted_pairs, vp), C.cast(offs, vp), C.cast(cnts, vp), C.cast(groups, vp),
+                                                 C.byref(ng), C.cast(tiles, vp), C.byref(nt))
+    if rc != TF_OK:
+        raise TFError(rc, GROUP_ERRORS.get(rc, "grouping failed"))
+    return dict(
+        sorted_pairs=[(p.token, p.expert, p.rank, p.weight_bits_and_reserved) for p in sorted_pairs[:n]],
+        sorted_pairs_raw=sorted_pairs, n_pairs=n,
+        per_expert_offsets=list(offs[:num_experts]), per_expert_counts=list(cnts[:num_experts]),
+        groups=[(g.expert, g.pair_start, g.pair_count) for g in groups[:ng.value]], groups_raw=groups,
+        tiles=[(t.group_start, t.group_count, t.pair_start, t.pair_count) for t in tiles[:nt.value]])

@@ -1,0 +1,604 @@
+// Prefill / multi-token path: per-token router, (token, expert) pair grouping on the host and on the device, the grouped
+// routed-expert computation (row-streaming for small groups, matrix cores for large ones), token-major weighted reduce.
+#include <algorithm>
+#include <unordered_set>
+#include <vector>
+
+#include "tf_prefill_kernels.hpp"
+#include "tf_router.hpp"
+
+using namespace tfk;
+
+namespace tfk {
+bool qmm_operands_ok(const void *w, const void *x, long ldx_halves, int k);
+int32_t launch_grouped_phase1_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off,
+                                   const ChunkList &cl, uint32_t n_chunks_upper, const tf_prefill_pair *pairs,
+                                   const half_t *hidden, long hidden_stride, half_t *acts, uint32_t acts_pair_base, int d, int f,
+                                   tf_dtype sd);
+int32_t launch_grouped_down_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off,
+                                 const ChunkList &cl, uint32_t n_chunks_upper, const tf_prefill_pair *pairs, const half_t *acts,
+                                 uint32_t acts_pair_base, half_t *route_partials, int d, int f, int top_k, tf_dtype sd);
+}  // namespace tfk
+
+namespace {
+
+// ------------------------------------------------------------------------------------------------ router block
+// One 256-thread block per token row: the four waves share the experts (wave w takes e = w, w+4, ...), the logits meet in
+// LDS, wave 0 selects.
+template <int NPASS>
+__global__ __launch_bounds__(256) void prefill_router_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B,
+                                                             const half_t *hidden, long hidden_stride, const uint16_t *eff,
+                                                             const uint16_t *per_expert_scale, uint32_t *out_indices,
+                                                             half_t *out_weights, uint32_t num_experts, int d, uint32_t top_k) {
+    __shared__ float logits[256];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t t = blockIdx.x;
+    const half_t *row = hidden + (size_t)t * hidden_stride;
+    const int groups = d >> 6;
+    for (uint32_t e = wave; e < num_experts; e += 4) {
+        const float v = router_row<0, NPASS>(W + (size_t)e * d, S + (size_t)e * groups * 2, B + (size_t)e * groups * 2, row, eff, d, lane);
+        if (lane == 0) logits[e] = v;
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float gain[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t c = lane + 64 * j;
+        gain[j] = c < num_experts ? bf16_to_f32(per_expert_scale[c]) : 0.0f;
+    }
+    router_select(logits, gain, out_indices + (size_t)t * top_k, out_weights + (size_t)t * top_k, num_experts, top_k, lane);
+}
+
+// ------------------------------------------------------------------------------------------------ device grouping
+// One 1024-thread block.  (1) histogram of experts in LDS, (2) exclusive scan -> per-expert offsets, (3) one wave per
+// expert walks the tokens in order, 64 at a time, and places that expert's pairs by ballot + popcount (stable: sorted by
+// token, then rank), (4) the work list of <= 64-pair chunks.
+__global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *indices, const uint16_t *weights, uint32_t query_count,
+                                                           uint32_t top_k, uint32_t num_experts, tf_prefill_pair *sorted_pairs,
+                                                           uint32_t *per_expert_offsets, uint32_t *per_expert_counts,
+                                                           tf_prefill_group *chunks, uint32_t *chunk_count) {
+    __shared__ uint32_t cnt[256], start[256], chunk_start[256];
+    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const uint32_t n_pairs = query_count * top_k;
+    if (tid < 256) cnt[tid] = 0;
+    __syncthreads();
+    for (uint32_t i = tid; i < n_pairs; i += blockDim.x) {
+        uint32_t e = indices[i];
+        e = e < num_experts ? e : num_experts - 1;
+        atomicAdd(&cnt[e], 1u);
+    }
+    __syncthreads();
+    if (tid == 0) {
+        uint32_t run = 0, cr = 0;
+        for (uint32_t e = 0; e < num_experts; ++e) {
+            start[e] = run;
+            chunk_start[e] = cr;
+            run += cnt[e];
+            cr += (cnt[e] + kChunkPairs - 1) / kChunkPairs;
+        }
+        chunk_count[0] = cr;
+    }
+    __syncthreads();
+    if (tid < num_experts) {
+        per_expert_offsets[tid] = cnt[tid] ? start[tid] : 0xFFFFFFFFu;
+        per_expert_counts[tid] = cnt[tid];
+        const uint32_t nch = (cnt[tid] + kChunkPairs - 1) / kChunkPairs;
+        for (uint32_t c = 0; c < nch; ++c) {
+            tf_prefill_group g;
+            g.expert = tid;
+            g.pair_start = start[tid] + c * kChunkPairs;
+            g.pair_count = min(kChunkPairs, cnt[tid] - c * kChunkPairs);
+            chunks[chunk_start[tid] + c] = g;
+        }
+    }
+    for (uint32_t e = wave; e < num_experts; e += blockDim.x >> 6) {
+        if (cnt[e] == 0) continue;
+        uint32_t base = start[e];
+        for (uint32_t t0 = 0; t0 < query_count; t0 += 64) {
+            const uint32_t t = t0 + lane;
+            int rank = -1;
+            if (t < query_count) {
+                for (uint32_t r = 0; r < top_k; ++r) {
+                    uint32_t x = indices[(size_t)t * top_k + r];
+                    x = x < num_experts ? x : num_experts - 1;
+                    if (x == e && rank < 0) rank = (int)r;
+                }
+            }
+            const uint64_t mask = __ballot(rank >= 0);
+            if (rank >= 0) {
+                const uint32_t pos = base + __builtin_popcountll(mask & ((1ull << lane) - 1ull));
+                tf_prefill_pair p;
+                p.token = t;
+                p.expert = e;
+                p.rank = (uint32_t)rank;
+                p.weight_bits_and_reserved = (uint32_t)weights[(size_t)t * top_k + rank];
+                sorted_pairs[pos] = p;
+            }
+            base += (uint32_t)__builtin_popcountll(mask);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ grouped, row-streaming
+// Small groups: a wave loads one tile of gate rows and the same tile of up rows ONCE and applies it to every pair of the
+// chunk, so each touched expert is read once however many tokens chose it.
+__device__ __forceinline__ void store_act(half_t *acts, size_t index, float gate, float up) {
+    acts[index] = (half_t)(gelu_tanh(gate) * up);
+}
+
+template <int RT, int NP, int SD>
+__global__ __launch_bounds__(256) void grouped_phase1_long_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl,
+                                                                  const tf_prefill_pair *pairs, const half_t *hidden,
+                                                                  long hidden_stride, half_t *acts, uint32_t acts_pair_base,
+                                                                  int d, int f) {
+    tf_prefill_group ch;
+    if (!get_chunk(cl, blockIdx.y, ch)) return;
+    const uint8_t *base = expert_base(tab, ch.expert);
+    if (!base) return;
+    const int lane = threadIdx.x & 63;
+    const int tile = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int row0 = tile * RT;
+    if (row0 >= f) return;
+    const int groups = d >> 6;
+    const int rows_left = min(RT, f - row0);
+    const size_t w_byte = (size_t)row0 * (d >> 1), sb_byte = (size_t)row0 * groups * 2;
+    LongRows<RT, NP> lr;
+    typename LongRows<RT, NP>::Tile tg, tu;
+    lr.init_map(d, lane);
+    lr.load(tg, base + off.gate_W_off + w_byte, reinterpret_cast<const uint16_t *>(base + off.gate_s_off + sb_byte),
+            reinterpret_cast<const uint16_t *>(base + off.gate_b_off + sb_byte), rows_left, lane);
+    lr.load(tu, base + off.up_W_off + w_byte, reinterpret_cast<const uint16_t *>(base + off.up_s_off + sb_byte),
+            reinterpret_cast<const uint16_t *>(base + off.up_b_off + sb_byte), rows_left, lane);
+    for (uint32_t j = 0; j < ch.pair_count; ++j) {
+        const uint32_t pi = ch.pair_start + j;
+        lr.init_x(hidden + (size_t)pairs[pi].token * hidden_stride, lane);
+        float gate[RT], up[RT];
+        lr.template reduce<SD>(tg, gate);
+        lr.template reduce<SD>(tu, up);
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < RT; ++r)
+                if (r < rows_left) store_act(acts, (size_t)(pi - acts_pair_base) * f + row0 + r, gate[r], up[r]);
+        }
+    }
+}
+
+template <int SD>
+__global__ __launch_bounds__(256) void grouped_phase1_generic_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl,
+                                                                     const tf_prefill_pair *pairs, const half_t *hidden,
+                                                                     long hidden_stride, half_t *acts, uint32_t acts_pair_base,
+                                                                     int d, int f) {
+    tf_prefill_group ch;
+    if (!get_chunk(cl, blockIdx.y, ch)) return;
+    const uint8_t *base = expert_base(tab, ch.expert);
+    if (!base) return;
+    const int lane = threadIdx.x & 63;
+    const int r = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    if (r >= f) return;
+    const int groups = d >> 6;
+    const size_t w_byte = (size_t)r * (d >> 1), sb_byte = (size_t)r * groups * 2;
+    for (uint32_t j = 0; j < ch.pair_count; ++j) {
+        const uint32_t pi = ch.pair_start + j;
+        const half_t *x = hidden + (size_t)pairs[pi].token * hidden_stride;
+        const float gate = generic_row_dot<SD>(base + off.gate_W_off + w_byte, base + off.gate_s_off + sb_byte, base + off.gate_b_off + sb_byte, x, d, lane);
+        const float up = generic_row_dot<SD>(base + off.up_W_off + w_byte, base + off.up_s_off + sb_byte, base + off.up_b_off + sb_byte, x, d, lane);
+        if (lane == 0) store_act(acts, (size_t)(pi - acts_pair_base) * f + r, gate, up);
+    }
+}
+
+// down rows, F <= 1024: half-wave per row, 2 * NPASS rows per wave, loaded once, applied to every pair of the chunk
+template <int NPASS, int SD>
+__global__ __launch_bounds__(256) void grouped_down_short_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl,
+                                                                 const tf_prefill_pair *pairs, const half_t *acts,
+                                                                 uint32_t acts_pair_base, half_t *route_partials, int d, int f,
+                                                                 int top_k) {
+    tf_prefill_group ch;
+    if (!get_chunk(cl, blockIdx.y, ch)) return;
+    const uint8_t *base = expert_base(tab, ch.expert);
+    if (!base) return;
+    const int lane = threadIdx.x & 63;
+    const long row0 = (long)((blockIdx.x * blockDim.x + threadIdx.x) >> 6) * 2 * NPASS;
+    if (row0 >= d) return;
+    ShortRows sr;
+    ShortRows::Pair t[NPASS];
+    sr.init_map(f, lane);
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p)
+        sr.load(t[p], base + off.down_W_off, base + off.down_s_off, base + off.down_b_off, row0 + 2 * p, d, f);
+    for (uint32_t j = 0; j < ch.pair_count; ++j) {
+        const tf_prefill_pair pr = pairs[ch.pair_start + j];
+        sr.init_x(acts + (size_t)(ch.pair_start + j - acts_pair_base) * f);
+        half_t *out = route_partials + ((size_t)pr.token * top_k + pr.rank) * d;
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p) {
+            float lo, hi;
+            sr.template reduce<SD>(t[p], lo, hi);
+            if (lane == 0) {
+                if (row0 + 2 * p < d) out[row0 + 2 * p] = (half_t)lo;
+                if (row0 + 2 * p + 1 < d) out[row0 + 2 * p + 1] = (half_t)hi;
+            }
+        }
+    }
+}
+
+template <int SD>
+__global__ __launch_bounds__(256) void grouped_down_generic_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl,
+                                                                   const tf_prefill_pair *pairs, const half_t *acts,
+                                                                   uint32_t acts_pair_base, half_t *route_partials, int d, int f,
+                                                                   int top_k) {
+    tf_prefill_group ch;
+    if (!get_chunk(cl, blockIdx.y, ch)) return;
+    const uint8_t *base = expert_base(tab, ch.expert);
+    if (!base) return;
+    const int lane = threadIdx.x & 63;
+    const int r = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    if (r >= d) return;
+    const int groups = f >> 6;
+    for (uint32_t j = 0; j < ch.pair_count; ++j) {
+        const tf_prefill_pair pr = pairs[ch.pair_start + j];
+        const float v = generic_row_dot<SD>(base + off.down_W_off + (size_t)r * (f >> 1), base + off.down_s_off + (size_t)r * groups * 2,
+                                            base + off.down_b_off + (size_t)r * groups * 2,
+                                            acts + (size_t)(ch.pair_start + j - acts_pair_base) * f, f, lane);
+        if (lane == 0) route_partials[((size_t)pr.token * top_k + pr.rank) * d + r] = (half_t)v;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ reduce
+__global__ __launch_bounds__(256) void reduce_token_major_kernel(const half_t *partials, const half_t *weights, half_t *h2,
+                                                                 uint32_t T, uint32_t top_k, uint32_t D) {
+    const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t t = blockIdx.y;
+    if (c >= D || t >= T) return;
+    float acc = 0.0f;
+    for (uint32_t r = 0; r < top_k; ++r)
+        acc = fmaf((float)weights[t * top_k + r], (float)partials[((size_t)t * top_k + r) * D + c], acc);
+    h2[(size_t)t * D + c] = (half_t)acc;
+}
+
+// ------------------------------------------------------------------------------------------------ launch helpers
+struct GroupedGeom {
+    const tf_prefill_pair *pairs;
+    const half_t *hidden;
+    long hidden_stride;
+    half_t *acts;
+    uint32_t acts_pair_base;
+    half_t *route_partials;
+    int d, f, top_k;
+};
+
+bool table_aligned(const ExpertTable &t) {
+    if (t.pool) return aligned16(t.pool) && t.stride % 16 == 0;
+    for (uint32_t i = 0; i < t.live; ++i)
+        if (!aligned16(t.blob[i])) return false;
+    return true;
+}
+
+// use_mfma: the chunks are large enough for the matrix cores to pay
+int32_t run_grouped(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off, const ChunkList &cl,
+                    uint32_t n_chunks_upper, const GroupedGeom &g, tf_dtype sd, bool use_mfma) {
+    if (n_chunks_upper == 0) return TF_OK;
+    const bool blobs16 = table_aligned(tab);
+    const bool hidden16 = aligned16(g.hidden) && g.hidden_stride % 8 == 0;
+    const bool acts16 = aligned16(g.acts);
+    const bool p1_fast = blobs16 && hidden16 && off.gate_W_off % 16 == 0 && off.up_W_off % 16 == 0;
+    const bool dn_fast = blobs16 && acts16 && off.down_W_off % 16 == 0;
+    int32_t rc;
+    // ---- phase 1
+    if (use_mfma && p1_fast && acts16) {
+        rc = launch_grouped_phase1_mfma(ctx, st, tab, off, cl, n_chunks_upper, g.pairs, g.hidden, g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f, sd);
+    } else {
+        const LongPlan plan = plan_long_rows(g.d);
+        bool launched = false;
+        if (p1_fast && g.d > 1024 && plan.rt > 0) {
+            const dim3 grid(((g.f + plan.rt - 1) / plan.rt + 3) / 4, n_chunks_upper);
+#define TF_GP1(RT_, NP_)                                                                                                   \
+    if (!launched && plan.rt == RT_ && plan.np == NP_) {                                                                   \
+        launched = true;                                                                                                   \
+        if (sd == TF_BF16)                                                                                                 \
+            hipLaunchKernelGGL((grouped_phase1_long_kernel<RT_, NP_, 0>), grid, dim3(256), 0, st, tab, off, cl, g.pairs,   \
+                               g.hidden, g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f);                             \
+        else                                                                                                               \
+            hipLaunchKernelGGL((grouped_phase1_long_kernel<RT_, NP_, 1>), grid, dim3(256), 0, st, tab, off, cl, g.pairs,   \
+                               g.hidden, g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f);                             \
+    }
+            TF_GP1(1, 1) TF_GP1(1, 2) TF_GP1(1, 3) TF_GP1(1, 4) TF_GP1(2, 1) TF_GP1(2, 2) TF_GP1(2, 3) TF_GP1(2, 4)
+            TF_GP1(4, 1) TF_GP1(4, 2) TF_GP1(4, 3) TF_GP1(4, 4)
+#undef TF_GP1
+        }
+        if (!launched) {
+            const dim3 grid((g.f + 3) / 4, n_chunks_upper);
+            if (sd == TF_BF16)
+                hipLaunchKernelGGL(grouped_phase1_generic_kernel<0>, grid, dim3(256), 0, st, tab, off, cl, g.pairs, g.hidden, g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f);
+            else
+                hipLaunchKernelGGL(grouped_phase1_generic_kernel<1>, grid, dim3(256), 0, st, tab, off, cl, g.pairs, g.hidden, g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f);
+        }
+        rc = check_launch(ctx, "grouped phase 1");
+    }
+    if (rc != TF_OK) return rc;
+    // ---- down
+    if (use_mfma && dn_fast) {
+        return launch_grouped_down_mfma(ctx, st, tab, off, cl, n_chunks_upper, g.pairs, g.acts, g.acts_pair_base, g.route_partials, g.d, g.f, g.top_k, sd);
+    }
+    if (dn_fast && g.f <= 1024) {
+        constexpr int NPASS = 4;
+        const dim3 grid(((g.d + 2 * NPASS - 1) / (2 * NPASS) + 3) / 4, n_chunks_upper);
+        if (sd == TF_BF16)
+            hipLaunchKernelGGL((grouped_down_short_kernel<NPASS, 0>), grid, dim3(256), 0, st, tab, off, cl, g.pairs, g.acts, g.acts_pair_base, g.route_partials, g.d, g.f, g.top_k);
+        else
+            hipLaunchKernelGGL((grouped_down_short_kernel<NPASS, 1>), grid, dim3(256), 0, st, tab, off, cl, g.pairs, g.acts, g.acts_pair_base, g.route_partials, g.d, g.f, g.top_k);
+    } else {
+        const dim3 grid((g.d + 3) / 4, n_chunks_upper);
+        if (sd == TF_BF16)
+            hipLaunchKernelGGL(grouped_down_generic_kernel<0>, grid, dim3(256), 0, st, tab, off, cl, g.pairs, g.acts, g.acts_pair_base, g.route_partials, g.d, g.f, g.top_k);
+        else
+            hipLaunchKernelGGL(grouped_down_generic_kernel<1>, grid, dim3(256), 0, st, tab, off, cl, g.pairs, g.acts, g.acts_pair_base, g.route_partials, g.d, g.f, g.top_k);
+    }
+    return check_launch(ctx, "grouped down");
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t tf_prefill_router_gemma4_block(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset,
+                                       const void *scales, uint64_t scales_offset, const void *biases, uint64_t biases_offset,
+                                       const void *hidden, uint64_t hidden_offset, const void *effective_scale,
+                                       uint64_t effective_scale_offset, const void *per_expert_scale,
+                                       uint64_t per_expert_scale_offset, void *out_indices, uint64_t out_indices_offset,
+                                       void *out_weights, uint64_t out_weights_offset, uint32_t query_count, uint32_t num_experts,
+                                       uint32_t d, uint32_t top_k, uint32_t hidden_stride_elements) {
+    TF_REQUIRE(ctx, ctx && weights && scales && biases && hidden && effective_scale && per_expert_scale && out_indices && out_weights,
+               TF_ERR_INVALID_ARGUMENT, "prefill_router: null argument");
+    TF_REQUIRE(ctx, query_count > 0, TF_ERR_INVALID_ARGUMENT, "prefill_router: queryCount must be positive");
+    TF_REQUIRE(ctx, num_experts > 0 && num_experts <= 256, TF_ERR_INVALID_ARGUMENT, "prefill_router: numExperts > 256 is not supported");
+    TF_REQUIRE(ctx, top_k > 0 && top_k <= 64, TF_ERR_INVALID_ARGUMENT, "prefill_router: topK must be in 1...64");
+    TF_REQUIRE(ctx, d > 0 && d % TF_GROUP_SIZE == 0, TF_ERR_INVALID_ARGUMENT, "prefill_router: D must be a multiple of 64");
+    TF_REQUIRE(ctx, hidden_stride_elements >= d, TF_ERR_INVALID_ARGUMENT, "prefill_router: hidden stride is too small");
+    const uint8_t *w = at(weights, weights_offset);
+    const uint8_t *s = at(scales, scales_offset), *b = at(biases, biases_offset);
+    const half_t *h = reinterpret_cast<const half_t *>(at(hidden, hidden_offset));
+    const uint16_t *eff = reinterpret_cast<const uint16_t *>(at(effective_scale, effective_scale_offset));
+    const uint16_t *pes = reinterpret_cast<const uint16_t *>(at(per_expert_scale, per_expert_scale_offset));
+    uint32_t *oi = reinterpret_cast<uint32_t *>(at(out_indices, out_indices_offset));
+    half_t *ow = reinterpret_cast<half_t *>(at(out_weights, out_weights_offset));
+    TF_REQUIRE(ctx, aligned(s, 2) && aligned(b, 2) && aligned(h, 2) && aligned(eff, 2) && aligned(pes, 2) && aligned(oi, 4) && aligned(ow, 2),
+               TF_ERR_INVALID_ARGUMENT, "prefill_router: misaligned operand");
+    const bool fast = aligned16(w) && aligned16(h) && aligned16(eff) && hidden_stride_elements % 8 == 0 && d <= 4096;
+    const int npass = fast ? (int)((d / 16 + 63) / 64) : 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define TF_PR(NP_)                                                                                                           \
+    hipLaunchKernelGGL(prefill_router_kernel<NP_>, dim3(query_count), dim3(256), 0, st, w, s, b, h, (long)hidden_stride_elements, \
+                       eff, pes, oi, ow, num_experts, (int)d, top_k)
+    switch (npass) {
+        case 1: TF_PR(1); break;
+        case 2: TF_PR(2); break;
+        case 3: TF_PR(3); break;
+        case 4: TF_PR(4); break;
+        default: TF_PR(0); break;
+    }
+#undef TF_PR
+    return check_launch(ctx, "prefill_router_gemma4_block");
+}
+
+int32_t tf_prefill_make_token_expert_pairs(const uint32_t *indices, const uint16_t *weights_f16, int32_t query_count, int32_t top_k,
+                                           tf_prefill_pair *pairs) {
+    if (query_count < 0 || top_k < 0) return TF_ERR_INVALID_ARGUMENT;
+    if ((int64_t)query_count * top_k > 0 && (!indices || !weights_f16 || !pairs)) return TF_ERR_INVALID_ARGUMENT;
+    for (int32_t token = 0; token < query_count; ++token)
+        for (int32_t rank = 0; rank < top_k; ++rank) {
+            const int64_t i = (int64_t)token * top_k + rank;
+            pairs[i].token = (uint32_t)token;
+            pairs[i].expert = indices[i];
+            pairs[i].rank = (uint32_t)rank;
+            pairs[i].weight_bits_and_reserved = (uint32_t)weights_f16[i];
+        }
+    return TF_OK;
+}
+
+int32_t tf_prefill_group_token_expert_pairs(const tf_prefill_pair *pairs, uint64_t pair_count, int32_t query_count, int32_t top_k,
+                                            int32_t num_experts, int32_t tile_expert_count, const uint64_t *expert_sort_keys,
+                                            uint64_t expert_sort_key_count, tf_prefill_pair *sorted_pairs,
+                                            uint32_t *per_expert_offsets, uint32_t *per_expert_counts, tf_prefill_group *groups,
+                                            uint32_t *group_count, tf_prefill_tile *tiles, uint32_t *tile_count) {
+    if (query_count < 0) return TF_ERR_GROUP_INVALID_QUERY_COUNT;
+    if (top_k <= 0) return TF_ERR_GROUP_INVALID_TOP_K;
+    if (num_experts <= 0) return TF_ERR_GROUP_INVALID_NUM_EXPERTS;
+    if (tile_expert_count < 1 || tile_expert_count > (int32_t)TF_MAX_TILE_EXPERTS) return TF_ERR_GROUP_INVALID_TILE_EXPERT_COUNT;
+    if (expert_sort_keys && expert_sort_key_count != (uint64_t)num_experts) return TF_ERR_GROUP_SORT_KEY_COUNT_MISMATCH;
+    if (pair_count != (uint64_t)query_count * (uint64_t)top_k) return TF_ERR_GROUP_PAIR_COUNT_MISMATCH;
+    if (!per_expert_offsets || !per_expert_counts || !group_count || !tile_count) return TF_ERR_INVALID_ARGUMENT;
+    if (pair_count && (!pairs || !sorted_pairs || !groups || !tiles)) return TF_ERR_INVALID_ARGUMENT;
+
+    std::unordered_set<uint64_t> seen;
+    seen.reserve((size_t)pair_count);
+    for (uint64_t i = 0; i < pair_count; ++i) {
+        if (pairs[i].token >= (uint32_t)query_count) return TF_ERR_GROUP_TOKEN_OUT_OF_RANGE;
+        if (pairs[i].rank >= (uint32_t)top_k) return TF_ERR_GROUP_RANK_OUT_OF_RANGE;
+        if (pairs[i].expert >= (uint32_t)num_experts) return TF_ERR_GROUP_EXPERT_OUT_OF_RANGE;
+        if (!seen.insert(((uint64_t)pairs[i].token << 32) | pairs[i].rank).second) return TF_ERR_GROUP_DUPLICATE_TOKEN_RANK;
+    }
+    std::vector<uint32_t> order((size_t)pair_count);
+    for (uint64_t i = 0; i < pair_count; ++i) order[(size_t)i] = (uint32_t)i;
+    std::sort(order.begin(), order.end(), [&](uint32_t ia, uint32_t ib) {
+        const tf_prefill_pair &a = pairs[ia], &b = pairs[ib];
+        if (expert_sort_keys && expert_sort_keys[a.expert] != expert_sort_keys[b.expert])
+            return expert_sort_keys[a.expert] < expert_sort_keys[b.expert];
+        if (a.expert != b.expert) return a.expert < b.expert;
+        if (a.token != b.token) return a.token < b.token;
+        return a.rank < b.rank;
+    });
+    for (int32_t e = 0; e < num_experts; ++e) {
+        per_expert_offsets[e] = 0xFFFFFFFFu;
+        per_expert_counts[e] = 0;
+    }
+    uint32_t ng = 0;
+    for (uint64_t i = 0; i < pair_count;) {
+        const uint32_t expert = pairs[order[(size_t)i]].expert;
+        const uint64_t first = i;
+        while (i < pair_count && pairs[order[(size_t)i]].expert == expert) {
+            sorted_pairs[i] = pairs[order[(size_t)i]];
+            ++i;
+        }
+        per_expert_offsets[expert] = (uint32_t)first;
+        per_expert_counts[expert] = (uint32_t)(i - first);
+        groups[ng].expert = expert;
+        groups[ng].pair_start = (uint32_t)first;
+        groups[ng].pair_count = (uint32_t)(i - first);
+        ++ng;
+    }
+    uint32_t nt = 0;
+    for (uint32_t gs = 0; gs < ng; gs += (uint32_t)tile_expert_count) {
+        const uint32_t ge = std::min(ng, gs + (uint32_t)tile_expert_count);
+        tiles[nt].group_start = gs;
+        tiles[nt].group_count = ge - gs;
+        tiles[nt].pair_start = groups[gs].pair_start;
+        tiles[nt].pair_count = groups[ge - 1].pair_start + groups[ge - 1].pair_count - groups[gs].pair_start;
+        ++nt;
+    }
+    *group_count = ng;
+    *tile_count = nt;
+    return TF_OK;
+}
+
+int32_t tf_prefill_group_pairs_device(tf_ctx *ctx, tf_stream stream, const void *indices, const void *weights, uint32_t query_count,
+                                      uint32_t top_k, uint32_t num_experts, void *sorted_pairs, void *per_expert_offsets,
+                                      void *per_expert_counts, void *chunks, void *chunk_count) {
+    TF_REQUIRE(ctx, ctx && indices && weights && sorted_pairs && per_expert_offsets && per_expert_counts && chunks && chunk_count,
+               TF_ERR_INVALID_ARGUMENT, "group_pairs_device: null argument");
+    TF_REQUIRE(ctx, query_count > 0 && top_k > 0 && num_experts > 0 && num_experts <= 256, TF_ERR_INVALID_ARGUMENT,
+               "group_pairs_device: need queryCount > 0, topK > 0, 1 <= numExperts <= 256");
+    TF_REQUIRE(ctx, aligned(indices, 4) && aligned(weights, 2) && aligned(sorted_pairs, 4) && aligned(chunks, 4), TF_ERR_INVALID_ARGUMENT,
+               "group_pairs_device: misaligned operand");
+    hipLaunchKernelGGL(group_pairs_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint32_t *>(indices), static_cast<const uint16_t *>(weights), query_count, top_k, num_experts,
+                       static_cast<tf_prefill_pair *>(sorted_pairs), static_cast<uint32_t *>(per_expert_offsets),
+                       static_cast<uint32_t *>(per_expert_counts), static_cast<tf_prefill_group *>(chunks),
+                       static_cast<uint32_t *>(chunk_count));
+    return check_launch(ctx, "group_pairs_device");
+}
+
+int32_t tf_prefill_grouped_routed_moe_streamed(tf_ctx *ctx, tf_stream stream, const void *hidden, uint64_t hidden_offset,
+                                               const void *sorted_pairs, uint64_t sorted_pairs_offset, void *route_partials,
+                                               uint64_t route_partials_offset, void *gate_up_act_scratch,
+                                               uint64_t gate_up_act_scratch_offset, void *down_scratch, uint64_t down_scratch_offset,
+                                               const void *const *blobs, const tf_prefill_streamed_params *params,
+                                               const tf_prefill_group *tile_groups, uint32_t tile_group_count,
+                                               int32_t pair_microbatch_rows, int32_t *out_microbatches, tf_dtype scale_dtype) {
+    if (out_microbatches) *out_microbatches = 0;
+    TF_REQUIRE(ctx, ctx && params, TF_ERR_INVALID_ARGUMENT, "grouped_routed_moe: null argument");
+    // encodeStreamedBatched's guard (PrefillGroupedRoutedMoE.swift:401-403): nothing to do, zero micro-batches
+    if (params->pair_count == 0 || pair_microbatch_rows <= 0) return TF_OK;
+    TF_REQUIRE(ctx, hidden && sorted_pairs && route_partials && gate_up_act_scratch && down_scratch && blobs && tile_groups,
+               TF_ERR_INVALID_ARGUMENT, "grouped_routed_moe: null argument");
+    TF_REQUIRE(ctx, params->live_expert_count >= 1 && params->live_expert_count <= TF_MAX_TILE_EXPERTS, TF_ERR_INVALID_ARGUMENT,
+               "invalid streamed tile binding: tile has %u live experts; expected 1...16", params->live_expert_count);
+    TF_REQUIRE(ctx, params->d % TF_GROUP_SIZE == 0 && params->routed_intermediate % TF_GROUP_SIZE == 0 && params->d > 0 &&
+                   params->routed_intermediate > 0 && params->top_k > 0 && params->hidden_stride_elements >= params->d,
+               TF_ERR_INVALID_ARGUMENT, "grouped_routed_moe: bad dimensions");
+    TF_REQUIRE(ctx, scale_dtype == TF_BF16 || scale_dtype == TF_FP16, TF_ERR_INVALID_ARGUMENT, "grouped_routed_moe: scale dtype must be bf16 or fp16");
+    ExpertTable tab = {};
+    tab.live = params->live_expert_count;
+    for (uint32_t i = 0; i < tab.live; ++i) {
+        TF_REQUIRE(ctx, blobs[i] != nullptr, TF_ERR_INVALID_ARGUMENT, "invalid streamed tile binding: expert %u has no blob", i);
+        tab.blob[i] = static_cast<const uint8_t *>(blobs[i]);
+        tab.local_id[i] = params->local_expert[i];
+    }
+    const tf_expert_offsets off = {params->gate_W_off, params->gate_s_off, params->gate_b_off, params->up_W_off, params->up_s_off,
+                                   params->up_b_off, params->down_W_off, params->down_s_off, params->down_b_off};
+    const tf_prefill_pair *pairs = reinterpret_cast<const tf_prefill_pair *>(at(sorted_pairs, sorted_pairs_offset));
+    const uint32_t f = params->routed_intermediate;
+    // the activation plane is the third of the reference's [gate | up | act] scratch planes of `rows` pairs each
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint32_t begin = params->pair_start, end = params->pair_start + params->pair_count;
+    int32_t microbatches = 0;
+    for (uint32_t mb_start = begin; mb_start < end; mb_start += (uint32_t)pair_microbatch_rows) {
+        const uint32_t mb_end = std::min(end, mb_start + (uint32_t)pair_microbatch_rows);
+        const uint32_t rows = mb_end - mb_start;
+        half_t *acts = reinterpret_cast<half_t *>(at(gate_up_act_scratch, gate_up_act_scratch_offset)) + (size_t)2 * rows * f;
+        // cut the micro-batch into runs of one expert (<= kChunkPairs pairs) using the host's group table
+        std::vector<tf_prefill_group> runs;
+        for (uint32_t gi = 0; gi < tile_group_count; ++gi) {
+            const uint32_t gs = std::max(tile_groups[gi].pair_start, mb_start);
+            const uint32_t ge = std::min(tile_groups[gi].pair_start + tile_groups[gi].pair_count, mb_end);
+            for (uint32_t s0 = gs; s0 < ge; s0 += kChunkPairs) runs.push_back(tf_prefill_group{tile_groups[gi].expert, s0, std::min(kChunkPairs, ge - s0)});
+        }
+        for (size_t r0 = 0; r0 < runs.size(); r0 += kInlineChunks) {
+            ChunkList cl = {};
+            cl.n = (uint32_t)std::min<size_t>(kInlineChunks, runs.size() - r0);
+            for (uint32_t i = 0; i < cl.n; ++i) cl.inline_chunks[i] = runs[r0 + i];
+            GroupedGeom g{pairs, reinterpret_cast<const half_t *>(at(hidden, hidden_offset)), (long)params->hidden_stride_elements, acts,
+                          mb_start, reinterpret_cast<half_t *>(at(route_partials, route_partials_offset)), (int)params->d, (int)f,
+                          (int)params->top_k};
+            const int32_t rc = run_grouped(ctx, st, tab, off, cl, cl.n, g, scale_dtype, false);
+            if (rc != TF_OK) return rc;
+        }
+        ++microbatches;
+    }
+    (void)down_scratch;   // the down outputs go straight to route_partials; the reference's second copy is not needed
+    if (out_microbatches) *out_microbatches = microbatches;
+    return TF_OK;
+}
+
+int32_t tf_prefill_grouped_routed_moe_resident(tf_ctx *ctx, tf_stream stream, const void *hidden, uint64_t hidden_offset,
+                                               uint32_t hidden_stride_elements, const void *sorted_pairs, const void *chunks,
+                                               const void *chunk_count, uint32_t max_chunks, uint32_t pair_count,
+                                               const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                               const tf_expert_offsets *routed_offsets, void *acts_scratch, void *route_partials,
+                                               uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx && hidden && sorted_pairs && chunks && chunk_count && expert_pool && routed_offsets && acts_scratch && route_partials,
+               TF_ERR_INVALID_ARGUMENT, "grouped_routed_moe_resident: null argument");
+    TF_REQUIRE(ctx, d > 0 && d % TF_GROUP_SIZE == 0 && f > 0 && f % TF_GROUP_SIZE == 0 && top_k > 0 && num_experts > 0 &&
+                   hidden_stride_elements >= d,
+               TF_ERR_INVALID_ARGUMENT, "grouped_routed_moe_resident: bad dimensions");
+    TF_REQUIRE(ctx, scale_dtype == TF_BF16 || scale_dtype == TF_FP16, TF_ERR_INVALID_ARGUMENT, "grouped_routed_moe_resident: scale dtype must be bf16 or fp16");
+    if (pair_count == 0 || max_chunks == 0) return TF_OK;
+    ExpertTable tab = {};
+    tab.pool = static_cast<const uint8_t *>(expert_pool);
+    tab.stride = expert_pool_stride;
+    tab.num_experts = num_experts;
+    ChunkList cl = {};
+    cl.dev = static_cast<const tf_prefill_group *>(chunks);
+    cl.dev_n = static_cast<const uint32_t *>(chunk_count);
+    GroupedGeom g{static_cast<const tf_prefill_pair *>(sorted_pairs), reinterpret_cast<const half_t *>(at(hidden, hidden_offset)),
+                  (long)hidden_stride_elements, static_cast<half_t *>(acts_scratch), 0u, static_cast<half_t *>(route_partials), (int)d,
+                  (int)f, (int)top_k};
+    // the host only knows the average group size: matrix cores once experts see 8 or more tokens on average
+    const bool use_mfma = (uint64_t)pair_count >= (uint64_t)num_experts * 8;
+    return run_grouped(ctx, static_cast<hipStream_t>(stream), tab, *routed_offsets, cl, max_chunks, g, scale_dtype, use_mfma);
+}
+
+int32_t tf_prefill_moe_reduce_token_major(tf_ctx *ctx, tf_stream stream, const void *route_partials, uint64_t route_partials_offset,
+                                          const void *route_weights, uint64_t route_weights_offset, void *h2, uint64_t h2_offset,
+                                          uint32_t query_count, uint32_t top_k, uint32_t d) {
+    TF_REQUIRE(ctx, ctx && route_partials && route_weights && h2, TF_ERR_INVALID_ARGUMENT, "moe_reduce_token_major: null argument");
+    TF_REQUIRE(ctx, query_count > 0, TF_ERR_INVALID_ARGUMENT, "moe_reduce_token_major: queryCount must be positive");
+    TF_REQUIRE(ctx, top_k > 0, TF_ERR_INVALID_ARGUMENT, "moe_reduce_token_major: topK must be positive");
+    TF_REQUIRE(ctx, d > 0, TF_ERR_INVALID_ARGUMENT, "moe_reduce_token_major: D must be positive");
+    TF_REQUIRE(ctx, route_partials_offset % 2 == 0 && route_weights_offset % 2 == 0 && h2_offset % 2 == 0, TF_ERR_INVALID_ARGUMENT,
+               "moe_reduce_token_major: offsets must be 2-byte aligned");
+    const dim3 grid((d + 255) / 256, query_count);
+    hipLaunchKernelGGL(reduce_token_major_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
+                       reinterpret_cast<const half_t *>(at(route_partials, route_partials_offset)),
+                       reinterpret_cast<const half_t *>(at(route_weights, route_weights_offset)),
+                       reinterpret_cast<half_t *>(at(h2, h2_offset)), query_count, top_k, d);
+    return check_launch(ctx, "moe_reduce_token_major");
+}
+
+int32_t tf_prefill_int4_qmm(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset, const void *scales,
+                            uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *x, uint64_t x_offset,
+                            void *y, uint64_t y_offset, int32_t t, int32_t n, int32_t k, tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "prefill_int4_qmm: null context");
+    TF_REQUIRE(ctx, t > 0 && n > 0, TF_ERR_INVALID_ARGUMENT, "prefill_int4_qmm: t and n must be positive");
+    TF_REQUIRE(ctx, k > 0 && k % (int32_t)TF_GROUP_SIZE == 0, TF_ERR_INVALID_ARGUMENT, "prefill_int4_qmm: K must be a multiple of 64");
+    // every token row takes the GEMV path: Y[t, :] = gemv(W, X[t, :]); identical arithmetic, hence QMM == repeated GEMV
+    for (int32_t row = 0; row < t; ++row) {
+        const int32_t rc = tf_dequant_int4_gemv(ctx, stream, weights, weights_offset, scales, scales_offset, biases, biases_offset, x,
+                                                x_offset + (uint64_t)row * k * 2, y, y_offset + (uint64_t)row * n * 2, (uint32_t)n,
+                                                (uint32_t)k, scale_dtype, TF_FP16);
+        if (rc != TF_OK) return rc;
+    }
+    return TF_OK;
+}
+
+}  // extern "C"

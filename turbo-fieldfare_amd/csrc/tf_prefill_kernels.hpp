@@ -1,0 +1,53 @@
+// Shared pieces of the prefill / multi-token path: POD layouts, expert lookup, work lists.
+#pragma once
+
+#include "tf_gemv_kernels.hpp"
+#include "tf_qmm.hpp"
+
+namespace tfk {
+
+// Where the expert blobs live: a table of up to 16 (id, pointer) bindings — the reference's streamed tile
+// (PrefillGroupedRoutedMoE.swift:185-216) — or a resident pool indexed by expert id.
+struct ExpertTable {
+    const uint8_t *blob[TF_MAX_TILE_EXPERTS];
+    uint32_t local_id[TF_MAX_TILE_EXPERTS];
+    uint32_t live;
+    const uint8_t *pool;
+    uint64_t stride;
+    uint32_t num_experts;
+};
+
+// nullptr when the expert is not bound in the tile (the reference's kernels skip such pairs, prefill.metal:611-618).
+__device__ __forceinline__ const uint8_t *expert_base(const ExpertTable &t, uint32_t expert) {
+    if (t.pool) {
+        const uint32_t e = expert < t.num_experts ? expert : t.num_experts - 1;
+        return t.pool + (uint64_t)e * t.stride;
+    }
+    for (uint32_t s = 0; s < t.live; ++s)
+        if (t.local_id[s] == expert) return t.blob[s];
+    return nullptr;
+}
+
+// Work list: runs of sorted pairs that share one expert, each at most kChunkPairs long.  Either a short list passed with
+// the kernel arguments or a device array written by the grouping kernel (with its length in device memory).
+constexpr uint32_t kChunkPairs = 64;
+constexpr uint32_t kInlineChunks = 48;
+struct ChunkList {
+    uint32_t n;
+    tf_prefill_group inline_chunks[kInlineChunks];
+    const tf_prefill_group *dev;
+    const uint32_t *dev_n;
+};
+
+__device__ __forceinline__ bool get_chunk(const ChunkList &cl, uint32_t i, tf_prefill_group &out) {
+    if (cl.dev) {
+        if (i >= *cl.dev_n) return false;
+        out = cl.dev[i];
+        return true;
+    }
+    if (i >= cl.n) return false;
+    out = cl.inline_chunks[i];
+    return true;
+}
+
+}  // namespace tfk

@@ -1,0 +1,128 @@
+// Router arithmetic shared by the decode router and the per-token prefill router.
+#pragma once
+
+#include "tf_common.hpp"
+
+namespace tfk {
+
+// logits[e] = sum_g [ s * sum(q * x') + b * sum(x') ],  x' = float(hidden) * float(effective_scale).
+// One wave per expert row.  NPASS > 0: every operand 16-byte aligned and d <= 1024 * NPASS; the lane's <= NPASS chunks of
+// 16 weights are all requested before the first is used, so the row costs one memory round trip.  NPASS == 0: any
+// alignment and size, byte/halfword loads in a loop.
+__device__ __forceinline__ void router_chunk(const u32x4 w, const u32x4 ha, const u32x4 hb, const u32x4 ea, const u32x4 eb,
+                                             float s, float b, float &acc) {
+    float dot = 0.0f, sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t hw = i < 8 ? ha[i >> 1] : hb[(i - 8) >> 1];
+        const uint32_t ew = i < 8 ? ea[i >> 1] : eb[(i - 8) >> 1];
+        const uint16_t hbits = (uint16_t)((i & 1) ? (hw >> 16) : (hw & 0xFFFFu));
+        const float ev = (i & 1) ? __uint_as_float(ew & 0xFFFF0000u) : __uint_as_float(ew << 16);
+        const float xv = f16_to_f32(hbits) * ev;
+        const float q = (float)((w[i >> 2] >> (8 * (i & 3))) & 0xFFu);
+        dot = fmaf(q, xv, dot);
+        sum += xv;
+    }
+    acc = fmaf(s, dot, acc);
+    acc = fmaf(b, sum, acc);
+}
+
+template <int SD, int NPASS>
+__device__ __forceinline__ float router_row(const uint8_t *w_row, const uint8_t *s_row, const uint8_t *b_row,
+                                            const half_t *hidden, const uint16_t *eff, int d, int lane) {
+    float acc = 0.0f;
+    if constexpr (NPASS > 0) {
+        const int chunks = d >> 4;
+        u32x4 w[NPASS], ha[NPASS], hb[NPASS], ea[NPASS], eb[NPASS];
+        uint16_t sv[NPASS], bv[NPASS];
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p) {
+            const int c = lane + 64 * p;
+            w[p] = ha[p] = hb[p] = ea[p] = eb[p] = u32x4{0u, 0u, 0u, 0u};
+            sv[p] = bv[p] = 0;
+            if (c < chunks) {
+                w[p] = load16(w_row + (size_t)c * 16);
+                ha[p] = load16(hidden + c * 16);
+                hb[p] = load16(hidden + c * 16 + 8);
+                ea[p] = load16(eff + c * 16);
+                eb[p] = load16(eff + c * 16 + 8);
+                sv[p] = *reinterpret_cast<const uint16_t *>(s_row + (c >> 2) * 2);
+                bv[p] = *reinterpret_cast<const uint16_t *>(b_row + (c >> 2) * 2);
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p)
+            router_chunk(w[p], ha[p], hb[p], ea[p], eb[p], sb_to_f32<SD>(sv[p]), sb_to_f32<SD>(bv[p]), acc);
+    } else {
+        const int words = d >> 2;
+        for (int wi = lane; wi < words; wi += kWave) {
+            const int g = wi >> 4;
+            const float s = sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(s_row + g * 2));
+            const float b = sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(b_row + g * 2));
+            float dot = 0.0f, sum = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const float xv = (float)hidden[wi * 4 + i] * bf16_to_f32(eff[wi * 4 + i]);
+                dot = fmaf((float)w_row[wi * 4 + i], xv, dot);
+                sum += xv;
+            }
+            acc = fmaf(s, dot, acc);
+            acc = fmaf(b, sum, acc);
+        }
+    }
+    return wave_sum(acc);
+}
+
+// Top-k over <= 256 fp32 logits by one wave, then softmax over the selected and the per-expert gain.
+// Same ordering as the reference's serial insertion (moe.metal:152-171): score descending, ties to the lower index;
+// NaN and -inf are never selected; an unfilled position reads index 0 with score -inf.
+// Lane l holds candidates l, l+64, l+128, l+192 and their gains; each round takes the wave maximum with DPP and finds
+// its lowest expert index with ballots, so a round is a few dozen ALU instructions and no memory traffic.
+__device__ __forceinline__ void router_select(const float *logits, const float gain[4], uint32_t *out_indices,
+                                              half_t *out_weights, uint32_t num_experts, uint32_t top_k, int lane) {
+    float cand[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const uint32_t e = lane + 64 * j;
+        const float v = e < num_experts ? logits[e] : -INFINITY;
+        cand[j] = (v != v) ? -INFINITY : v;
+    }
+    float my_score = -INFINITY, my_gain = 0.0f;   // lane i (< top_k) ends up holding the i-th selection
+    uint32_t my_idx = 0;
+    for (uint32_t i = 0; i < top_k; ++i) {
+        const float m = fmaxf(fmaxf(cand[0], cand[1]), fmaxf(cand[2], cand[3]));
+        const float wm = wave_max(m);
+        const bool found = wm > -INFINITY;
+        int sel_j = 4, sel_lane = 0;
+#pragma unroll
+        for (int j = 3; j >= 0; --j) {
+            const uint64_t mask = __ballot(cand[j] == wm);
+            if (mask) { sel_j = j; sel_lane = __builtin_ctzll(mask); }
+        }
+        float g = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (sel_j == j) g = read_lane(gain[j], sel_lane);
+        if ((uint32_t)lane == i) {
+            my_score = found ? wm : -INFINITY;
+            my_idx = found ? (uint32_t)(sel_lane + 64 * sel_j) : 0u;
+            my_gain = found ? g : read_lane(gain[0], 0);
+        }
+        if (found && lane == sel_lane) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (sel_j == j) cand[j] = -INFINITY;
+        }
+    }
+    const float max_s = read_lane(my_score, 0);
+    const float ex = (uint32_t)lane < top_k ? expf(my_score - max_s) : 0.0f;
+    float sum_exp = 0.0f;   // summed in selection order, like the reference
+    for (uint32_t i = 0; i < top_k; ++i) sum_exp += read_lane(ex, (int)i);
+    if ((uint32_t)lane < top_k) {
+        out_indices[lane] = my_idx;
+        out_weights[lane] = (half_t)((ex / sum_exp) * my_gain);
+    }
+}
+
+
+}  // namespace tfk
