@@ -33,6 +33,9 @@ def int4_matrix_bytes(rows, cols):
 
 # per-unit algorithmic bytes (what one launch must move at least once)
 ROUTER_BYTES = E * D + 2 * E * (D // 64) * 2 + D * 2 + D * 2 + E * 2 + TOPK * 4 + TOPK * 2   # W + s/b + hidden + eff + gains + outputs
+# HBM bytes one phase-1 launch moves, from hardware counters (profiles/bench_hbm_traffic_counters.txt): FETCH_SIZE 8875.6 KiB
+# x 2.0 (the factor a plain 1 GiB copy calibrates) + WRITE_SIZE 22.0 KiB x 1.0.
+PHASE1_TRAFFIC_BYTES = int(8875.6 * 1024 * 1.9999 + 22.0 * 1024)
 PHASE1_BYTES = TOPK * 2 * int4_matrix_bytes(F_MOE, D) + D * 2 + TOPK * F_MOE * 2             # gate+up of 8 experts + x + acts out
 PHASE2_BYTES = TOPK * int4_matrix_bytes(D, F_MOE) + TOPK * F_MOE * 2 + TOPK * 2 + D * 2 + D * 2   # down of 8 + acts in + w + residual + y
 STEP_BYTES = ROUTER_BYTES + PHASE1_BYTES + PHASE2_BYTES
@@ -92,6 +95,8 @@ def main():
     ap.add_argument("--layers", type=int, default=4, help="layer replicas the steps rotate through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip lm_head / GEMV / shared-expert side measurements")
+    ap.add_argument("--calibration-copy", action="store_true",
+                    help="also run one plain 1 GiB device copy (a known-size reference for hardware byte counters)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -207,7 +212,7 @@ def main():
                    "algorithmic_bytes_per_step": STEP_BYTES},
         "roofline": {"bound": "hbm", "kernel": "phase1_long_kernel<2,3,bf16> (gate/up/GeGLU of 8 experts)",
                      "achieved": round(p1_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(p1_gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "frac": round(p1_gbps / HBM_PEAK_GBPS, 4), "traffic": PHASE1_TRAFFIC_BYTES,
                      "algorithmic_bytes_per_launch": PHASE1_BYTES, "avg_launch_us": round(t_p1, 3)},
         "launch": f"HIP graph replay, {graph_steps} steps per graph",
         "step_per_s": round(1e3 / ms_per_step, 1),
@@ -217,8 +222,15 @@ def main():
                        "phase2_GBps": round(PHASE2_BYTES / (t_p2 * 1e-6) / 1e9, 1)},
     }
 
+    if args.calibration_copy:
+        src = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     if not args.no_extras:
         out["extras"] = extras(torch, tfk, k, gen, lib, h, stream)
+        out["extras"].update(multi_token_extras(torch, tfk, k, gen, lib, h, stream, layers[0], offs, stride))
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, layers, hidden, idx, wts, y, offs, stride, payload, args)
@@ -310,6 +322,94 @@ def extras(torch, tfk, k, gen, lib, h, stream):
     us = time_loop(torch, shared, 300, warmup=20)
     res["shared_expert_int4"] = {"us_per_call": round(us, 3), "GBps": round(SHARED_BYTES / (us * 1e-6) / 1e9, 1),
                                  "algorithmic_bytes": SHARED_BYTES}
+    return res
+
+
+def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride):
+    """configs[3] (small-M verification, M in {2,4,8,16}) and configs[4] (2048-token prefill, Zipf(1.1) routing) over one
+    resident layer: router block -> device grouping -> grouped experts -> token-major reduce, no host round trip."""
+    import ctypes as C
+    pool, r = layer
+    off = tfk.ExpertOffsets(*offs)
+    expert_bytes = 3 * int4_matrix_bytes(F_MOE, D)
+    res = {}
+
+    def run(T, idx_dev=None, wts_dev=None, iters=20, with_router=True):
+        n = T * TOPK
+        cap = E + n // 64 + 1
+        hid = torch.randn((T, D), device="cuda", generator=gen).to(torch.float16)
+        idx = torch.zeros((T, TOPK), dtype=torch.int32, device="cuda") if idx_dev is None else idx_dev
+        wts = torch.zeros((T, TOPK), dtype=torch.float16, device="cuda") if wts_dev is None else wts_dev
+        sp = torch.zeros(n * 4, dtype=torch.int32, device="cuda")
+        offs_d, cnts_d = torch.zeros(E, dtype=torch.int32, device="cuda"), torch.zeros(E, dtype=torch.int32, device="cuda")
+        chunks, nch = torch.zeros(cap * 3, dtype=torch.int32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+        acts = torch.zeros(n * F_MOE, dtype=torch.float16, device="cuda")
+        partials = torch.zeros(n * D, dtype=torch.float16, device="cuda")
+        h2 = torch.zeros(T * D, dtype=torch.float16, device="cuda")
+
+        def fn(i):
+            rc = 0
+            if with_router:
+                rc |= lib.tf_prefill_router_gemma4_block(h, stream, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0,
+                                                         hid.data_ptr(), 0, r["eff"].data_ptr(), 0, r["gain"].data_ptr(), 0,
+                                                         idx.data_ptr(), 0, wts.data_ptr(), 0, T, E, D, TOPK, D)
+            rc |= lib.tf_prefill_group_pairs_device(h, stream, idx.data_ptr(), wts.data_ptr(), T, TOPK, E, sp.data_ptr(),
+                                                    offs_d.data_ptr(), cnts_d.data_ptr(), chunks.data_ptr(), nch.data_ptr())
+            rc |= lib.tf_prefill_grouped_routed_moe_resident(h, stream, hid.data_ptr(), 0, D, sp.data_ptr(), chunks.data_ptr(), nch.data_ptr(),
+                                                             cap, n, pool.data_ptr(), stride, E, C.byref(off), acts.data_ptr(),
+                                                             partials.data_ptr(), D, F_MOE, TOPK, tfk.TF_BF16)
+            rc |= lib.tf_prefill_moe_reduce_token_major(h, stream, partials.data_ptr(), 0, wts.data_ptr(), 0, h2.data_ptr(), 0, T, TOPK, D)
+            assert rc == 0, k.last_error()
+        us = time_loop(torch, fn, iters, warmup=2)
+        unique = int((cnts_d > 0).sum().item())
+        return us, unique
+
+    small = {}
+    for M in (2, 4, 8, 16):
+        us, unique = run(M, iters=50)
+        nbytes = unique * expert_bytes + E * D + M * (2 * D * 2 + TOPK * F_MOE * 2 * 2 + TOPK * D * 2 * 2)
+        small[str(M)] = {"us": round(us, 2), "unique_experts": unique, "GBps_on_unique_expert_bytes": round(nbytes / (us * 1e-6) / 1e9, 1),
+                         "tokens_per_s": round(M / (us * 1e-6), 1)}
+    res["small_m"] = {"workload": "configs[3]: M tokens x top-8 over 128 resident experts (router block + grouping + grouped experts + reduce)",
+                      "per_M": small}
+
+    # configs[4]: 2048 tokens, Zipf(1.1) expert popularity, 8 distinct experts per token
+    T = 2048
+    rng = np.random.default_rng(0x21BF)
+    p = 1.0 / np.arange(1, E + 1) ** 1.1
+    p /= p.sum()
+    idx_np = np.stack([rng.choice(E, size=TOPK, replace=False, p=p) for _ in range(T)]).astype(np.int32)
+    idx_dev = torch.from_numpy(idx_np).cuda()
+    wts_dev = torch.softmax(torch.randn((T, TOPK), device="cuda", generator=gen), dim=1).to(torch.float16)
+    us, unique = run(T, idx_dev, wts_dev, iters=5, with_router=False)
+    routed_flop = T * TOPK * 2 * 3 * F_MOE * D
+    res["prefill_routed_2048"] = {"workload": "configs[4] routed part: 2048 tokens, Zipf(1.1) top-8 over 128 int4 experts, grouped GEMM on MFMA",
+                                  "ms": round(us / 1e3, 3), "tokens_per_s": round(T / (us * 1e-6), 1), "unique_experts": unique,
+                                  "TFLOPs": round(routed_flop / (us * 1e-6) / 1e12, 2),
+                                  "frac_mfma_fp16_peak": round(routed_flop / (us * 1e-6) / 2.5e15, 4)}
+    # shared expert over all tokens: gate, up (2112 x 2816), GeGLU, down (2816 x 2112) as dense int4 QMMs
+    gW, gS, gB = make_int4(torch, gen, F_SHARED, D)
+    uW, uS, uB = make_int4(torch, gen, F_SHARED, D)
+    dW, dS, dB = make_int4(torch, gen, D, F_SHARED)
+    x = torch.randn((T, D), device="cuda", generator=gen).to(torch.float16)
+    g_out = torch.zeros((T, F_SHARED), dtype=torch.float16, device="cuda")
+    u_out = torch.zeros((T, F_SHARED), dtype=torch.float16, device="cuda")
+    a_out = torch.zeros((T, F_SHARED), dtype=torch.float16, device="cuda")
+    y_out = torch.zeros((T, D), dtype=torch.float16, device="cuda")
+
+    def shared(i):
+        rc = lib.tf_int4_qmm(h, stream, gW.data_ptr(), 0, gS.data_ptr(), 0, gB.data_ptr(), 0, x.data_ptr(), 0, g_out.data_ptr(), 0, T, F_SHARED, D, tfk.TF_BF16)
+        rc |= lib.tf_int4_qmm(h, stream, uW.data_ptr(), 0, uS.data_ptr(), 0, uB.data_ptr(), 0, x.data_ptr(), 0, u_out.data_ptr(), 0, T, F_SHARED, D, tfk.TF_BF16)
+        rc |= lib.tf_gelu_mul_fp16(h, stream, g_out.data_ptr(), 0, u_out.data_ptr(), 0, a_out.data_ptr(), 0, T * F_SHARED)
+        rc |= lib.tf_int4_qmm(h, stream, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, a_out.data_ptr(), 0, y_out.data_ptr(), 0, T, D, F_SHARED, tfk.TF_BF16)
+        assert rc == 0, k.last_error()
+    us_s = time_loop(torch, shared, 5, warmup=2)
+    shared_flop = T * 2 * 3 * F_SHARED * D
+    res["prefill_shared_2048"] = {"workload": "configs[4] shared expert: 2048 tokens through int4 2112x2816 (x2) and 2816x2112 dense QMMs on MFMA",
+                                  "ms": round(us_s / 1e3, 3), "TFLOPs": round(shared_flop / (us_s * 1e-6) / 1e12, 2),
+                                  "frac_mfma_fp16_peak": round(shared_flop / (us_s * 1e-6) / 2.5e15, 4)}
+    res["prefill_2048_total"] = {"ms": round((us + us_s) / 1e3, 3), "tokens_per_s": round(T / ((us + us_s) * 1e-6), 1),
+                                 "GFLOP": round((routed_flop + shared_flop) / 1e9, 1)}
     return res
 
 

@@ -1,0 +1,299 @@
+// C++ mirror of the reference's Swift kernel wrappers (Sources/TurboFieldfare/Kernels/**) over the C ABI.
+// Class and method names follow the Swift ones; a "buffer" is a device pointer, the "command buffer" is the context's
+// stream.  Contract violations that trap in Swift (`precondition`) and errors that `throw` there surface as tf::Error.
+#pragma once
+
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/tf_kernels.h"
+
+namespace tf {
+
+struct Error : std::runtime_error {
+    int32_t status;
+    Error(int32_t s, const std::string &what) : std::runtime_error(what), status(s) {}
+};
+
+// MetalContext (Infrastructure/Metal/MetalContext.swift:51-214): device + one in-order queue.
+class Context {
+public:
+    explicit Context(int32_t device = 0, tf_stream stream = nullptr) : stream_(stream) {
+        const int32_t rc = tf_ctx_create(device, &ctx_);
+        if (rc != TF_OK) throw Error(rc, tf_status_string(rc));
+    }
+    ~Context() { tf_ctx_destroy(ctx_); }
+    Context(const Context &) = delete;
+    Context &operator=(const Context &) = delete;
+    tf_ctx *raw() const { return ctx_; }
+    tf_stream stream() const { return stream_; }
+    void check(int32_t rc) const {
+        if (rc != TF_OK) throw Error(rc, tf_last_error(ctx_));
+    }
+    // commandBuffer.commit + waitUntilCompleted + checkCommandBufferError (MetalContext.swift:22-26)
+    void waitUntilCompleted() const { check(tf_stream_synchronize(ctx_, stream_)); }
+
+private:
+    tf_ctx *ctx_ = nullptr;
+    tf_stream stream_ = nullptr;
+};
+
+// DequantInt4GEMV (Kernels/Quant/DequantInt4GEMV.swift)
+class DequantInt4GEMV {
+public:
+    explicit DequantInt4GEMV(const Context &context) : c_(context) {}
+    void encode(const void *weights, uint64_t weightsOffset, const void *scales, uint64_t scalesOffset, const void *biases,
+                uint64_t biasesOffset, const void *x, uint64_t xOffset, void *y, uint64_t yOffset, uint32_t m, uint32_t n) const {
+        c_.check(tf_dequant_int4_gemv(c_.raw(), c_.stream(), weights, weightsOffset, scales, scalesOffset, biases, biasesOffset, x,
+                                      xOffset, y, yOffset, m, n, TF_BF16, TF_FP16));
+    }
+
+private:
+    const Context &c_;
+};
+
+// DequantInt8GEMV (Kernels/Quant/DequantInt8GEMV.swift)
+class DequantInt8GEMV {
+public:
+    explicit DequantInt8GEMV(const Context &context) : c_(context) {}
+    void encode(const void *weights, uint64_t weightsOffset, const void *scales, uint64_t scalesOffset, const void *biases,
+                uint64_t biasesOffset, const void *x, uint64_t xOffset, void *y, uint64_t yOffset, uint32_t m, uint32_t n) const {
+        c_.check(tf_dequant_int8_gemv(c_.raw(), c_.stream(), weights, weightsOffset, scales, scalesOffset, biases, biasesOffset, x,
+                                      xOffset, y, yOffset, m, n, TF_BF16, TF_FP16));
+    }
+
+private:
+    const Context &c_;
+};
+
+using MoEExpertOffsets = tf_expert_offsets;   // Kernels/MoE/MoE.swift:4-29
+
+// MoE (Kernels/MoE/MoE.swift:31-313)
+class MoE {
+public:
+    static constexpr uint32_t maxStreamedExperts = TF_MAX_STREAMED_EXPERTS;
+    explicit MoE(const Context &context) : c_(context) {}
+
+    void encodeRouterGemma4(const void *weights, uint64_t weightsOffset, const void *scales, uint64_t scalesOffset,
+                            const void *biases, uint64_t biasesOffset, const void *hidden, const void *effectiveScale,
+                            uint64_t effectiveScaleOffset, const void *perExpertScale, uint64_t perExpertScaleOffset,
+                            void *outIndices, void *outWeights, uint32_t numExperts, uint32_t d, uint32_t topK) const {
+        c_.check(tf_router_gemma4(c_.raw(), c_.stream(), weights, weightsOffset, scales, scalesOffset, biases, biasesOffset, hidden,
+                                  effectiveScale, effectiveScaleOffset, perExpertScale, perExpertScaleOffset, outIndices, outWeights,
+                                  numExperts, d, topK));
+    }
+    // makeRoutedArgumentBuffer (MoE.swift:161-171): eight host-chosen blobs
+    tf_routed_blobs makeRoutedArgumentBuffer(const std::vector<const void *> &routedBlobs, uint32_t topK) const {
+        if (topK != maxStreamedExperts || routedBlobs.size() != topK) throw Error(TF_ERR_INVALID_ARGUMENT, "routedBlobs.count must equal topK == 8");
+        tf_routed_blobs r = {};
+        for (uint32_t i = 0; i < topK; ++i) r.blobs[i] = routedBlobs[i];
+        return r;
+    }
+    // resident experts: the indices the router wrote are read by the kernels themselves
+    static tf_routed_blobs residentPool(const void *pool, uint64_t stride, const uint32_t *deviceIndices, uint32_t numExperts) {
+        tf_routed_blobs r = {};
+        r.pool = pool;
+        r.pool_stride = stride;
+        r.indices = deviceIndices;
+        r.num_experts = numExperts;
+        return r;
+    }
+    void encodeRoutedPersistentPhase1U16Load(const tf_routed_blobs &routed, const MoEExpertOffsets &routedOffsets, const void *x,
+                                             void *acts, uint32_t d, uint32_t f, uint32_t topK) const {
+        c_.check(tf_moe_phase1_gate_up_act(c_.raw(), c_.stream(), &routed, &routedOffsets, x, acts, d, f, topK, TF_BF16));
+    }
+    void encodeRoutedPersistentPhase1SubsetU16Load(const tf_routed_blobs &routed, const MoEExpertOffsets &routedOffsets, const void *x,
+                                                   void *acts, const uint32_t *activeSlots, uint32_t activeCount, uint32_t d,
+                                                   uint32_t f, uint32_t topK) const {
+        c_.check(tf_moe_phase1_gate_up_act_subset(c_.raw(), c_.stream(), &routed, &routedOffsets, x, acts, activeSlots, activeCount, d,
+                                                  f, topK, TF_BF16));
+    }
+    void encodeRoutedPersistentPhase2Reduce(const tf_routed_blobs &routed, const MoEExpertOffsets &routedOffsets, const void *acts,
+                                            const void *routingWeights, const void *residual, void *y, uint32_t d, uint32_t f,
+                                            uint32_t topK) const {
+        c_.check(tf_moe_phase2_down_reduce(c_.raw(), c_.stream(), &routed, &routedOffsets, acts, routingWeights, residual, y, d, f, topK,
+                                           TF_BF16));
+    }
+
+private:
+    const Context &c_;
+};
+
+using SharedExpertProjection = tf_projection;   // Kernels/MoE/SharedExpertInt8.swift:9-31
+
+// SharedExpertRuntime / SharedExpertInt4 (Kernels/MoE/SharedExpertInt4.swift)
+class SharedExpertRuntime {
+public:
+    SharedExpertRuntime(const Context &context, int weightBits) : c_(context), weightBits_(weightBits) {
+        if (weightBits != 4) throw Error(TF_ERR_UNSUPPORTED_BITS, "SharedExpert unsupported weight bits: " + std::to_string(weightBits));
+    }
+    struct Buffer {   // an MTLBuffer's (contents, length)
+        void *ptr;
+        uint64_t length;
+    };
+    void encode(Buffer x, uint64_t xOffset, const SharedExpertProjection &gate, const SharedExpertProjection &up,
+                const SharedExpertProjection &down, Buffer y, uint64_t yOffset, Buffer scratchGate, uint64_t scratchGateOffset,
+                Buffer scratchUp, uint64_t scratchUpOffset, Buffer scratchAct, uint64_t scratchActOffset) const {
+        c_.check(tf_shared_expert_int4(c_.raw(), c_.stream(), x.ptr, xOffset, x.length, &gate, &up, &down, y.ptr, yOffset, y.length,
+                                       scratchGate.ptr, scratchGateOffset, scratchGate.length, scratchUp.ptr, scratchUpOffset,
+                                       scratchUp.length, scratchAct.ptr, scratchActOffset, scratchAct.length, (uint32_t)weightBits_,
+                                       TF_BF16));
+    }
+
+private:
+    const Context &c_;
+    int weightBits_;
+};
+
+// SharedExpertInt4 (Kernels/MoE/SharedExpertInt4.swift:6-100) is the 4-bit instance of the runtime.
+struct SharedExpertInt4 : SharedExpertRuntime {
+    explicit SharedExpertInt4(const Context &context) : SharedExpertRuntime(context, 4) {}
+};
+
+// LMHeadChainInt4 (Kernels/Fusions/LMHeadChainInt4.swift)
+class LMHeadChainInt4 {
+public:
+    explicit LMHeadChainInt4(const Context &context) : c_(context) {}
+    void encodeGreedyDecode(const void *hidden, uint64_t hiddenOffset, const void *normWeight, uint64_t normOffset,
+                            const void *weights, uint64_t weightsOffset, const void *scales, uint64_t scalesOffset,
+                            const void *biases, uint64_t biasesOffset, void *outToken, uint32_t d, uint32_t vocab,
+                            float rmsEps = 1e-6f) const {
+        c_.check(tf_lm_head_greedy_int4(c_.raw(), c_.stream(), hidden, hiddenOffset, normWeight, normOffset, weights, weightsOffset,
+                                        scales, scalesOffset, biases, biasesOffset, outToken, d, vocab, rmsEps, TF_BF16));
+    }
+
+private:
+    const Context &c_;
+};
+
+using PrefillTokenExpertPair = tf_prefill_pair;   // Kernels/Prefill/MoE/PrefillRouter.swift:5-28
+using PrefillMoEGroup = tf_prefill_group;         // Kernels/Prefill/MoE/PrefillMoEGrouping.swift:4-14
+using PrefillMoETile = tf_prefill_tile;           // :17-29
+
+// PrefillRouter (Kernels/Prefill/MoE/PrefillRouter.swift:30-112)
+class PrefillRouter {
+public:
+    explicit PrefillRouter(const Context &context) : c_(context) {}
+    void encodeGemma4Block(const void *weights, uint64_t weightsOffset, const void *scales, uint64_t scalesOffset, const void *biases,
+                           uint64_t biasesOffset, const void *hidden, uint64_t hiddenOffset, const void *effectiveScale,
+                           uint64_t effectiveScaleOffset, const void *perExpertScale, uint64_t perExpertScaleOffset,
+                           void *outIndices, uint64_t outIndicesOffset, void *outWeights, uint64_t outWeightsOffset,
+                           uint32_t queryCount, uint32_t numExperts, uint32_t d, uint32_t topK, uint32_t hiddenStrideElements) const {
+        c_.check(tf_prefill_router_gemma4_block(c_.raw(), c_.stream(), weights, weightsOffset, scales, scalesOffset, biases,
+                                                biasesOffset, hidden, hiddenOffset, effectiveScale, effectiveScaleOffset, perExpertScale,
+                                                perExpertScaleOffset, outIndices, outIndicesOffset, outWeights, outWeightsOffset,
+                                                queryCount, numExperts, d, topK, hiddenStrideElements));
+    }
+    static std::vector<PrefillTokenExpertPair> makeTokenExpertPairs(const std::vector<uint32_t> &indices,
+                                                                    const std::vector<uint16_t> &weightsF16, int queryCount, int topK) {
+        if (queryCount < 0 || topK < 0 || indices.size() != (size_t)queryCount * topK || weightsF16.size() != indices.size())
+            throw Error(TF_ERR_INVALID_ARGUMENT, "indices/weights count mismatch");
+        std::vector<PrefillTokenExpertPair> pairs(indices.size());
+        const int32_t rc = tf_prefill_make_token_expert_pairs(indices.data(), weightsF16.data(), queryCount, topK, pairs.data());
+        if (rc != TF_OK) throw Error(rc, "makeTokenExpertPairs");
+        return pairs;
+    }
+
+private:
+    const Context &c_;
+};
+
+// PrefillMoEGroupedRoutes + PrefillMoEGrouping.groupTokenExpertPairs (Kernels/Prefill/MoE/PrefillMoEGrouping.swift:31-193)
+struct PrefillMoEGroupedRoutes {
+    std::vector<PrefillTokenExpertPair> sortedPairs;
+    std::vector<uint32_t> perExpertOffsets, perExpertCounts;
+    std::vector<PrefillMoEGroup> groups;
+    std::vector<PrefillMoETile> tiles;
+    int queryCount = 0;
+    int maxPairsPerExpert() const { uint32_t m = 0; for (const auto &g : groups) m = g.pair_count > m ? g.pair_count : m; return (int)m; }
+    int maxPairsPerTile() const { uint32_t m = 0; for (const auto &t : tiles) m = t.pair_count > m ? t.pair_count : m; return (int)m; }
+    int maxLiveExpertsPerTile() const { uint32_t m = 0; for (const auto &t : tiles) m = t.group_count > m ? t.group_count : m; return (int)m; }
+};
+
+struct PrefillMoEGrouping {
+    static PrefillMoEGroupedRoutes groupTokenExpertPairs(const std::vector<PrefillTokenExpertPair> &pairs, int queryCount, int topK,
+                                                         int numExperts, int tileExpertCount = 16,
+                                                         const std::vector<uint64_t> *expertSortKeys = nullptr) {
+        PrefillMoEGroupedRoutes r;
+        r.queryCount = queryCount;
+        const size_t ne = numExperts > 0 ? (size_t)numExperts : 1;
+        r.sortedPairs.resize(pairs.size());
+        r.perExpertOffsets.resize(ne);
+        r.perExpertCounts.resize(ne);
+        r.groups.resize(pairs.size() < ne ? pairs.size() + 1 : ne);
+        r.tiles.resize(r.groups.size());
+        uint32_t ng = 0, nt = 0;
+        const int32_t rc = tf_prefill_group_token_expert_pairs(
+            pairs.data(), pairs.size(), queryCount, topK, numExperts, tileExpertCount, expertSortKeys ? expertSortKeys->data() : nullptr,
+            expertSortKeys ? expertSortKeys->size() : 0, r.sortedPairs.data(), r.perExpertOffsets.data(), r.perExpertCounts.data(),
+            r.groups.data(), &ng, r.tiles.data(), &nt);
+        if (rc != TF_OK) throw Error(rc, "PrefillMoEGroupingError " + std::to_string(rc));
+        r.groups.resize(ng);
+        r.tiles.resize(nt);
+        if (numExperts > 0) { r.perExpertOffsets.resize((size_t)numExperts); r.perExpertCounts.resize((size_t)numExperts); }
+        return r;
+    }
+};
+
+using PrefillGroupedRoutedMoEStreamedParams = tf_prefill_streamed_params;   // PrefillGroupedRoutedMoE.swift:104-183
+
+// PrefillGroupedRoutedMoE (Kernels/Prefill/MoE/PrefillGroupedRoutedMoE.swift:338-463)
+class PrefillGroupedRoutedMoE {
+public:
+    explicit PrefillGroupedRoutedMoE(const Context &context) : c_(context) {}
+    // returns the micro-batch count, like the Swift method
+    int encodeStreamedBatched(const void *hidden, uint64_t hiddenOffset, const void *sortedPairs, uint64_t sortedPairsOffset,
+                              void *routePartials, uint64_t routePartialsOffset, void *gateUpActScratch, uint64_t gateUpActScratchOffset,
+                              void *downScratch, uint64_t downScratchOffset, const std::vector<const void *> &bindingViews,
+                              const PrefillGroupedRoutedMoEStreamedParams &params, const PrefillMoEGroup *tileGroups,
+                              uint32_t tileGroupCount, int pairMicrobatchRows = 32) const {
+        int32_t microbatches = 0;
+        if (params.live_expert_count != bindingViews.size()) return 0;   // the Swift guard (:401-403)
+        c_.check(tf_prefill_grouped_routed_moe_streamed(c_.raw(), c_.stream(), hidden, hiddenOffset, sortedPairs, sortedPairsOffset,
+                                                        routePartials, routePartialsOffset, gateUpActScratch, gateUpActScratchOffset,
+                                                        downScratch, downScratchOffset, bindingViews.data(), &params, tileGroups,
+                                                        tileGroupCount, pairMicrobatchRows, &microbatches, TF_BF16));
+        return microbatches;
+    }
+
+private:
+    const Context &c_;
+};
+
+// PrefillMoE (Kernels/Prefill/MoE/PrefillMoE.swift)
+class PrefillMoE {
+public:
+    explicit PrefillMoE(const Context &context) : c_(context) {}
+    void encodeReduceTokenMajor(const void *routePartials, uint64_t routePartialsOffset, const void *routeWeights,
+                                uint64_t routeWeightsOffset, void *h2, uint64_t h2Offset, uint32_t queryCount, uint32_t topK,
+                                uint32_t d) const {
+        c_.check(tf_prefill_moe_reduce_token_major(c_.raw(), c_.stream(), routePartials, routePartialsOffset, routeWeights,
+                                                   routeWeightsOffset, h2, h2Offset, queryCount, topK, d));
+    }
+
+private:
+    const Context &c_;
+};
+
+// MPPPrefillInt4QMM (Kernels/TensorCore/MPPPrefillInt4QMM.swift)
+class MPPPrefillInt4QMM {
+public:
+    enum class Path { affineThreadgroupF16, unavailable };
+    static constexpr int tileK = TF_GROUP_SIZE;
+    explicit MPPPrefillInt4QMM(const Context &context) : c_(context) {}
+    bool isAvailable() const { return true; }
+    Path encode(const void *weights, uint64_t weightsOffset, const void *scales, uint64_t scalesOffset, const void *biases,
+                uint64_t biasesOffset, const void *x, uint64_t xOffset, void *y, uint64_t yOffset, int m, int n, int k) const {
+        const int32_t rc = tf_int4_qmm(c_.raw(), c_.stream(), weights, weightsOffset, scales, scalesOffset, biases, biasesOffset, x, xOffset,
+                                       y, yOffset, m, n, k, TF_BF16);
+        if (rc == TF_ERR_UNAVAILABLE) return Path::unavailable;
+        c_.check(rc);
+        return Path::affineThreadgroupF16;
+    }
+
+private:
+    const Context &c_;
+};
+
+}  // namespace tf
