@@ -121,34 +121,25 @@ def main():
     y = torch.zeros((n_hidden, D), dtype=torch.float16, device="cuda")
     stream = torch.cuda.current_stream().cuda_stream
     lib, h = k.lib, k.handle
-    routed = [k.routed_from_pool(pool, stride, 0, E) for pool, _ in layers]
 
     import ctypes as C
 
-    def step(i, ev=None):
+    def step(i):
         li, hi = i % args.layers, i % n_hidden
         pool, r = layers[li]
         hp = hidden.data_ptr() + hi * D * 2
         ip, wp = idx.data_ptr() + hi * TOPK * 4, wts.data_ptr() + hi * TOPK * 2
-        rb = routed[li]
-        rb.indices = ip
-        rc = lib.tf_router_gemma4(h, stream, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, hp,
-                                  r["eff"].data_ptr(), 0, r["gain"].data_ptr(), 0, ip, wp, E, D, TOPK)
-        if ev is not None:
-            ev[0].record()
-        rc |= lib.tf_moe_phase1_gate_up_act(h, stream, C.byref(rb), C.byref(off), hp, acts.data_ptr(), D, F_MOE, TOPK, tfk.TF_BF16)
-        if ev is not None:
-            ev[1].record()
-        rc |= lib.tf_moe_phase2_down_reduce(h, stream, C.byref(rb), C.byref(off), acts.data_ptr(), wp, residual.data_ptr(),
-                                            y.data_ptr() + hi * D * 2, D, F_MOE, TOPK, tfk.TF_BF16)
-        if ev is not None:
-            ev[2].record()
+        # one call = router logits -> (top-8 + gate/up/GeGLU of the 8 chosen experts) -> down + weighted sum + residual
+        rc = lib.tf_moe_decode_step(h, stream, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, hp,
+                                    r["eff"].data_ptr(), 0, r["gain"].data_ptr(), 0, pool.data_ptr(), stride, E, C.byref(off),
+                                    hp, acts.data_ptr(), residual.data_ptr(), y.data_ptr() + hi * D * 2, ip, wp, D, F_MOE, TOPK,
+                                    tfk.TF_BF16)
         if rc != 0:
             raise RuntimeError("kernel call failed: " + k.last_error())
 
-    def run_steps(first, count, ev=None):
+    def run_steps(first, count):
         for j in range(count):
-            step(first + j, None if ev is None else ev[j])
+            step(first + j)
 
     # ---- the decode loop is launch-bound on the host (3 short kernels per step), so the steps are captured once
     # into HIP graphs and replayed: `graph_steps` steps per graph, plus one remainder graph, exactly `steps` in all.
@@ -187,18 +178,27 @@ def main():
     torch.cuda.synchronize()
     ms_per_step_eager = (time.perf_counter() - t0) * 1e3 / args.steps
 
-    # ---- per-kernel durations with HIP events on the launch stream.  A spin kernel is queued first so that the host
-    # finishes enqueueing before the GPU starts: the events then bracket back-to-back execution, not host gaps.
+    # ---- per-kernel durations: the library brackets the step's three launches with HIP events on the launch stream
+    # (eager launches; a spin kernel is queued first so that the host is ahead of the GPU and the events bracket
+    # back-to-back execution, not host gaps).
     n_ev = min(args.steps, 128)
-    evs = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(n_ev)]
-    torch.cuda._sleep(int(2.4e9 * 0.03))
-    for i in range(n_ev):
-        evs[i][3].record()
-        step(args.warmup + i, evs[i])
-    torch.cuda.synchronize()
-    t_router = float(np.mean([e[3].elapsed_time(e[0]) for e in evs])) * 1e3   # us
-    t_p1 = float(np.mean([e[0].elapsed_time(e[1]) for e in evs])) * 1e3
-    t_p2 = float(np.mean([e[1].elapsed_time(e[2]) for e in evs])) * 1e3
+    k.set_step_timing(True)
+    times = []
+    for i0 in range(0, n_ev, 8):
+        torch.cuda._sleep(int(2.4e9 * 0.002))
+        for i in range(i0, min(i0 + 8, n_ev)):
+            step(args.warmup + i)
+            times.append(None)
+        times[-1] = k.last_step_timing()      # only the last step of a burst keeps its events
+    k.set_step_timing(False)
+    burst_last = [t for t in times if t is not None]
+    raw = [float(np.mean([t[j] for t in burst_last])) for j in range(3)]
+    t_empty = float(np.median([t[3] for t in burst_last]))     # an empty bracket, for reference
+    # Every bracket carries the same constant cost of its event packets.  The three kernels of a step depend on one
+    # another and so run back to back: in the timed region (no events) their durations add up to the step time, which
+    # fixes that constant.
+    per_bracket = max((sum(raw) - ms_per_step * 1e3) / 3.0, 0.0)
+    t_router, t_p1, t_p2 = (max(t - per_bracket, 1e-3) for t in raw)
     p1_gbps = PHASE1_BYTES / (t_p1 * 1e-6) / 1e9
 
     out = {
@@ -210,7 +210,7 @@ def main():
                                "8 of 128 int4 g64 experts (gate/up 704x2816, down 2816x704), GeGLU, weighted sum",
                    "layer_replicas": args.layers, "resident_expert_bytes": args.layers * E * stride,
                    "algorithmic_bytes_per_step": STEP_BYTES},
-        "roofline": {"bound": "hbm", "kernel": "phase1_long_kernel<2,3,bf16> (gate/up/GeGLU of 8 experts)",
+        "roofline": {"bound": "hbm", "kernel": "phase1_long_kernel<2,3,bf16,fused top-8> (expert selection + gate/up/GeGLU of 8 experts)",
                      "achieved": round(p1_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(p1_gbps / HBM_PEAK_GBPS, 4), "traffic": PHASE1_TRAFFIC_BYTES,
                      "algorithmic_bytes_per_launch": PHASE1_BYTES, "avg_launch_us": round(t_p1, 3)},
@@ -219,6 +219,8 @@ def main():
         "ms_per_step_eager_launch": round(ms_per_step_eager, 6),
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "kernels_us": {"router": round(t_router, 3), "phase1": round(t_p1, 3), "phase2": round(t_p2, 3),
+                       "event_bracket_overhead_subtracted": round(per_bracket, 3), "empty_bracket": round(t_empty, 3),
+                       "raw_brackets": [round(t, 3) for t in raw],
                        "phase2_GBps": round(PHASE2_BYTES / (t_p2 * 1e-6) / 1e9, 1)},
     }
 

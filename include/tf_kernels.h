@@ -104,6 +104,14 @@ int32_t tf_stream_synchronize(tf_ctx *ctx, tf_stream stream);
 const char *tf_status_string(int32_t status);
 const char *tf_last_error(const tf_ctx *ctx);
 uint32_t tf_abi_version(void);
+/* The runner's hand-rolled phase counters (totalCb1Nanos / totalCb2Nanos ..., RealForwardRunner.swift:408-419, surfaced by
+ * DecodeRunnerDiagnostics), as device time: while enabled, tf_moe_decode_step brackets its router, phase-1 and phase-2
+ * launches with HIP events on the call's stream, and tf_ctx_last_step_timing waits for the most recent step and returns,
+ * in microseconds, out_us[0..2] = the three brackets and out_us[3] = an empty bracket (two events with nothing between
+ * them: what the event packets themselves cost, to be subtracted from each of the others).  Leave it disabled while a
+ * stream is being captured into a graph. */
+int32_t tf_ctx_set_step_timing(tf_ctx *ctx, int32_t enabled);
+int32_t tf_ctx_last_step_timing(tf_ctx *ctx, float out_us[4]);
 
 /* ---- dequantization (bit-exact) --------------------------------------------------------------------- */
 /* Quantization.dequantizeInt4Affine / dequantizeInt8Affine (Infrastructure/ModelIO/Quantization.swift:105-119,

@@ -243,3 +243,72 @@ def test_shared_expert_errors():
     x, y, s = dev(c["x_bits"]), zeros_bytes(256), zeros_bytes(128)
     rc = k.shared_expert_int4(x, _proj(*t["gate"], 64, 128), _proj(*t["up"], 64, 128), _proj(*t["gate"], 64, 128), y, s, s, s, raise_on_error=False)
     assert rc == tfk.TF_ERR_DIMENSION_MISMATCH                                    # :41-45
+
+
+# ---------------------------------------------------------------------------------------------------- decode step
+def _decode_step_case(d, f, num_experts, seed):
+    rng = np.random.default_rng(seed)
+    blobs, off = [], None
+    for e in range(num_experts):
+        blob, off = tfo.make_blob(refcases.synthetic_int4(f, d, seed + e, "gate"), refcases.synthetic_int4(f, d, seed + e, "up"),
+                                  refcases.synthetic_int4(d, f, seed + e, "down"))
+        blobs.append(blob)
+    stride = (blobs[0].size + 63) // 64 * 64
+    pool = np.zeros(num_experts * stride, np.uint8)
+    for e, blob in enumerate(blobs):
+        pool[e * stride:e * stride + blob.size] = blob
+    rW, rS, rB = refcases.synthetic_int8(num_experts, d, seed)
+    eff = rng.uniform(0.5, 1.5, d).astype(np.float32) / np.float32(np.sqrt(d))
+    gain = rng.uniform(0.6, 1.4, num_experts).astype(np.float32)
+    return dict(blobs=blobs, off=off, stride=stride, pool=pool, rW=rW, rS=rS, rB=rB, eff_bits=tfo.bf16_bits_array(eff),
+                gain_bits=tfo.bf16_bits_array(gain), x_bits=refcases.normal_f16(d, seed + 7),
+                residual_bits=refcases.normal_f16(d, seed + 9))
+
+
+@pytest.mark.parametrize("d,f,num_experts", [(2816, 704, 16), (2816, 128, 128), (704, 128, 16)])
+def test_decode_step_equals_router_then_phases_and_the_reference(d, f, num_experts):
+    # one call (selection repeated inside phase 1 when the vector path applies) against the three wrapper calls of the
+    # reference runner (RealForwardRunner.swift:1462-1685): bitwise the same indices, weights, activations and output
+    import torch
+    c = _decode_step_case(d, f, num_experts, 0x5EED + d + f)
+    k = ctx()
+    off = tfk.ExpertOffsets(*c["off"].as_tuple())
+    pool, rW, rS, rB = dev(c["pool"]), dev(c["rW"]), dev(c["rS"]), dev(c["rB"])
+    eff, gain, x, res = dev(c["eff_bits"]), dev(c["gain_bits"]), dev(c["x_bits"]), dev(c["residual_bits"])
+    outs = []
+    for fused in (True, False):
+        idx, wts, acts, y = zeros_bytes(32), zeros_bytes(16), zeros_bytes(8 * f * 2), zeros_bytes(d * 2)
+        if fused:
+            k.set_step_timing(True)
+            k.check(k.lib.tf_moe_decode_step(k.handle, None, rW.data_ptr(), 0, rS.data_ptr(), 0, rB.data_ptr(), 0, x.data_ptr(),
+                                             eff.data_ptr(), 0, gain.data_ptr(), 0, pool.data_ptr(), c["stride"], num_experts,
+                                             off, x.data_ptr(), acts.data_ptr(), res.data_ptr(), y.data_ptr(), idx.data_ptr(),
+                                             wts.data_ptr(), d, f, 8, tfk.TF_BF16))
+            times = k.last_step_timing()
+            k.set_step_timing(False)
+            assert len(times) == 4 and all(0.0 <= t < 5e4 for t in times) and min(times[:3]) > 0.0
+        else:
+            k.router_gemma4(rW, rS, rB, x, eff, gain, idx, wts, num_experts, d)
+            routed = k.routed_from_pool(pool, c["stride"], idx, num_experts)
+            k.moe_phase1(routed, off, x, acts, d, f)
+            k.moe_phase2(routed, off, acts, wts, res, y, d, f)
+        torch.cuda.synchronize()
+        outs.append((host(idx, np.uint32, 8), host(wts, np.uint16, 8), host(acts, np.uint16, 8 * f), host(y, np.uint16, d)))
+    for a, b in zip(outs[0], outs[1]):
+        assert np.array_equal(a, b)
+    got_idx, got_w_bits, _, got_y = outs[0]
+    ref_idx, ref_w, _ = tfo.router_reference(c["rW"], c["rS"], c["rB"], tfo.from_f16_bits(c["x_bits"]),
+                                             tfo.bf16_array_to_float(c["eff_bits"]), tfo.bf16_array_to_float(c["gain_bits"]))
+    assert sorted(got_idx) == sorted(ref_idx)
+    expected = tfo.moe_apply_streamed_routed([c["blobs"][e] for e in got_idx], c["off"], tfo.from_f16_bits(c["x_bits"]),
+                                             tfo.from_f16_bits(c["residual_bits"]), tfo.from_f16_bits(got_w_bits), d, f, threads=8)
+    assert within_north_star(tfo.from_f16_bits(got_y), expected, abs_=1e-3 * max(1.0, float(np.max(np.abs(expected)))))
+
+
+def test_step_timing_needs_a_recorded_step():
+    k = ctx()
+    k.set_step_timing(True)
+    import ctypes as C
+    out = (C.c_float * 4)()
+    assert k.lib.tf_ctx_last_step_timing(k.handle, out) == tfk.TF_ERR_UNAVAILABLE
+    k.set_step_timing(False)

@@ -93,6 +93,8 @@ EXPORTS = {
     "tf_status_string": (C.c_char_p, [i32]),
     "tf_last_error": (C.c_char_p, [vp]),
     "tf_abi_version": (u32, []),
+    "tf_ctx_set_step_timing": (i32, [vp, i32]),
+    "tf_ctx_last_step_timing": (i32, [vp, C.POINTER(C.c_float)]),
     "tf_router_logits": (vp, [vp]),
     "tf_dequantize_int4_affine": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32]),
     "tf_dequantize_int8_affine": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32]),
@@ -200,6 +202,15 @@ class Context:
 
     def synchronize(self, stream=None):
         return self.check(self.lib.tf_stream_synchronize(self.handle, _stream() if stream is None else stream))
+
+    def set_step_timing(self, enabled: bool):
+        return self.check(self.lib.tf_ctx_set_step_timing(self.handle, 1 if enabled else 0))
+
+    def last_step_timing(self):
+        """(router_us, phase1_us, phase2_us, empty_bracket_us) of the most recent tf_moe_decode_step; waits for it."""
+        out = (C.c_float * 4)()
+        self.check(self.lib.tf_ctx_last_step_timing(self.handle, out))
+        return tuple(out)
 
     # ---- raw calls (return the status, do not raise) -----------------------------------------------------
     def call(self, name: str, *args) -> int:

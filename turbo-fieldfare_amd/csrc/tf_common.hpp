@@ -98,39 +98,58 @@ __device__ __forceinline__ void wave_best_pair(float &v, uint32_t &idx) {
 // --- int4 chunk arithmetic -------------------------------------------------------------------------
 // A "chunk" is 16 consecutive bytes of a packed row: 32 nibbles = half a quantization group.
 // Word d of the chunk holds elements 8d..8d+7, nibble i of the word = element 8d+i.
-// Masking a word with 0x000F000F leaves nibbles (i, i+4) in the low mantissa bits of two fp16 values: read as
-// fp16 subnormals they are exactly q * 2^-24, which v_dot2_f32_f16 multiplies without flushing (fp16 denormals are
-// enabled in the kernels' float mode).  The 0x00F000F0 mask leaves nibbles (i+1, i+5) as 16 q * 2^-24; those products
-// go to a second accumulator.  Both accumulators are rescaled once per chunk.  Every product q*x (4 bits x 11 bits)
-// is exact in fp32, so unpacking costs one AND per pair and no conversion instruction.
 //
-// xq[16] holds the chunk's 32 activations arranged to match: xq[4d+j] = (x[8d+j], x[8d+j+4]).
+// Unpacking costs one AND per element pair and no conversion: masking a word with 0x000F000F leaves nibbles (i, i+4)
+// in the low mantissa bits of two fp16 values, which read as fp16 subnormals are exactly q * 2^-24; the 0x00F000F0 mask
+// leaves nibbles (i+1, i+5) as 16 q * 2^-24, and their activations are stored pre-multiplied by 1/16 (exact for
+// |x| >= 2^-10, otherwise off by at most 2^-25).  fp16 denormals are not flushed by the matrix pipe.
+//
+// The multiply-accumulate runs on the matrix pipe, which is otherwise idle in these kernels: v_mfma_f32_4x4x4_16b_f16
+// computes, for each group of four lanes, the 4x4 products of the lanes' A rows with the lanes' B columns over K = 4.
+// With A = this lane's four weights and B = this lane's four activations, the diagonal element of the group's 4x4
+// result, which lands in result register (lane & 3) of this lane, is the lane's own 4-element dot product; the
+// off-diagonal elements are discarded.  Eight such instructions cover the chunk and accumulate in fp32; every product
+// q*x (4 bits x 11 bits) is exact.  The instruction ignores the execution mask, so chunk_dot() must be called from
+// wave-uniform control flow.
+//
+// xq[16] holds the chunk's 32 activations arranged to match: xq[4d+0] = (x[8d], x[8d+4]), xq[4d+1] = (x[8d+1], x[8d+5]) / 16,
+// xq[4d+2] = (x[8d+2], x[8d+6]), xq[4d+3] = (x[8d+3], x[8d+7]) / 16.
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ int lane_index() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
+
 __device__ __forceinline__ float chunk_dot(const u32x4 w, const half2_t *xq) {
-    float lo = 0.0f, hi = 0.0f;
+    const int sel = lane_index() & 3;
+    f32x4 c = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
         const uint32_t v = w[d];
         const uint32_t v8 = v >> 8;
-        lo = __builtin_amdgcn_fdot2(as_half2(v & 0x000F000Fu), xq[4 * d + 0], lo, false);   // (e0, e4)
-        hi = __builtin_amdgcn_fdot2(as_half2(v & 0x00F000F0u), xq[4 * d + 1], hi, false);   // 16 (e1, e5)
-        lo = __builtin_amdgcn_fdot2(as_half2(v8 & 0x000F000Fu), xq[4 * d + 2], lo, false);  // (e2, e6)
-        hi = __builtin_amdgcn_fdot2(as_half2(v8 & 0x00F000F0u), xq[4 * d + 3], hi, false);  // 16 (e3, e7)
+        const u32x2 a0 = {v & 0x000F000Fu, v & 0x00F000F0u};     // (e0, e4), 16 (e1, e5)
+        const u32x2 a1 = {v8 & 0x000F000Fu, v8 & 0x00F000F0u};   // (e2, e6), 16 (e3, e7)
+        const half4_t b0 = __builtin_shufflevector(xq[4 * d + 0], xq[4 * d + 1], 0, 1, 2, 3);
+        const half4_t b1 = __builtin_shufflevector(xq[4 * d + 2], xq[4 * d + 3], 0, 1, 2, 3);
+        c = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, a0), b0, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, a1), b1, c, 0, 0, 0);
     }
-    return fmaf(hi, 1048576.0f, lo * 16777216.0f);   // hi * 2^20 + lo * 2^24
+    const float c01 = (sel & 1) ? c[1] : c[0];
+    const float c23 = (sel & 1) ? c[3] : c[2];
+    return ((sel & 2) ? c23 : c01) * 16777216.0f;   // subnormal units -> integers
 }
 
 // Arrange 32 consecutive activations (four 16-byte loads, xr[d] = elements 8d..8d+7 as 4 packed pairs)
 // into the order chunk_dot() consumes, and return their fp32 sum.
 __device__ __forceinline__ float arrange_x(const u32x4 *xr, half2_t *xq) {
     float sum = 0.0f;
+    const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
         const uint32_t p01 = xr[d][0], p23 = xr[d][1], p45 = xr[d][2], p67 = xr[d][3];
-        // (e0,e4) (e1,e5) (e2,e6) (e3,e7)
-        xq[4 * d + 0] = as_half2((p01 & 0xFFFFu) | (p45 << 16));
-        xq[4 * d + 1] = as_half2((p01 >> 16) | (p45 & 0xFFFF0000u));
-        xq[4 * d + 2] = as_half2((p23 & 0xFFFFu) | (p67 << 16));
-        xq[4 * d + 3] = as_half2((p23 >> 16) | (p67 & 0xFFFF0000u));
+        xq[4 * d + 0] = as_half2((p01 & 0xFFFFu) | (p45 << 16));                     // (e0, e4)
+        xq[4 * d + 1] = as_half2((p01 >> 16) | (p45 & 0xFFFF0000u)) * sixteenth;     // (e1, e5) / 16
+        xq[4 * d + 2] = as_half2((p23 & 0xFFFFu) | (p67 << 16));                     // (e2, e6)
+        xq[4 * d + 3] = as_half2((p23 >> 16) | (p67 & 0xFFFF0000u)) * sixteenth;     // (e3, e7) / 16
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const half2_t h = as_half2(xr[d][j]);

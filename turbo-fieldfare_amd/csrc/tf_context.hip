@@ -43,13 +43,14 @@ int32_t tf_ctx_create(int32_t device, tf_ctx **out_ctx) {
     bool ok = hipMalloc(&ctx->router_logits, 256 * sizeof(float)) == hipSuccess;
     ok = ok && hipMemset(ctx->router_logits, 0, 256 * sizeof(float)) == hipSuccess;
     ok = ok && hipMalloc(&ctx->head_x_normed, kMaxHeadD * 2) == hipSuccess;
-    // argmax summaries + 64 64-bit argmax cells behind them (start at 0; the decode kernel leaves them at 0)
-    const size_t summary_bytes = ((size_t)kMaxHeadWaves * 2 + 128) * sizeof(float);
+    // argmax summaries + 64 64-bit argmax cells and a ticket counter behind them (start at 0; every call leaves them at 0)
+    const size_t summary_bytes = ((size_t)kMaxHeadWaves * 2 + 128 + 4) * sizeof(float);
     ok = ok && hipMalloc(&ctx->head_summaries, summary_bytes) == hipSuccess;
     ok = ok && hipMemset(ctx->head_summaries, 0, summary_bytes) == hipSuccess;
-    if (const char *env = getenv("TF_LONG_BLOCKS_PER_CU")) {
+    ok = ok && hipMalloc(&ctx->group_scratch, (size_t)kGroupSegments * 256 * sizeof(uint32_t)) == hipSuccess;
+    if (const char *env = getenv("TF_STREAM_BLOCKS_PER_CU")) {
         const int v = atoi(env);
-        if (v >= 1 && v <= 8) ctx->long_blocks_per_cu = v;
+        if (v >= 1 && v <= 8) ctx->stream_blocks_per_cu = v;
     }
     if (!ok) {
         tf_ctx_destroy(ctx);
@@ -65,12 +66,43 @@ void tf_ctx_destroy(tf_ctx *ctx) {
     if (ctx->head_x_normed) (void)hipFree(ctx->head_x_normed);
     if (ctx->head_summaries) (void)hipFree(ctx->head_summaries);
     if (ctx->head_logits) (void)hipFree(ctx->head_logits);
+    if (ctx->group_scratch) (void)hipFree(ctx->group_scratch);
+    if (ctx->prefill_logits) (void)hipFree(ctx->prefill_logits);
+    for (hipEvent_t e : ctx->step_events)
+        if (e) (void)hipEventDestroy(e);
     delete ctx;
 }
 
 int32_t tf_stream_synchronize(tf_ctx *ctx, tf_stream stream) {
     const hipError_t e = hipStreamSynchronize(static_cast<hipStream_t>(stream));
     if (e != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "stream synchronize: %s", hipGetErrorString(e));
+    return TF_OK;
+}
+
+int32_t tf_ctx_set_step_timing(tf_ctx *ctx, int32_t enabled) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "step timing: null context");
+    if (enabled) {
+        for (hipEvent_t &e : ctx->step_events) {
+            if (e) continue;
+            const hipError_t err = hipEventCreate(&e);
+            if (err != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "step timing: %s", hipGetErrorString(err));
+        }
+    }
+    ctx->step_timing = enabled != 0;
+    ctx->step_timed = false;
+    return TF_OK;
+}
+
+int32_t tf_ctx_last_step_timing(tf_ctx *ctx, float out_us[4]) {
+    TF_REQUIRE(ctx, ctx && out_us, TF_ERR_INVALID_ARGUMENT, "step timing: null argument");
+    TF_REQUIRE(ctx, ctx->step_timing && ctx->step_timed, TF_ERR_UNAVAILABLE, "step timing: no decode step recorded while timing was enabled");
+    hipError_t err = hipEventSynchronize(ctx->step_events[4]);
+    for (int i = 0; i < 4 && err == hipSuccess; ++i) {
+        float ms = 0.0f;
+        err = hipEventElapsedTime(&ms, ctx->step_events[i], ctx->step_events[i + 1]);
+        out_us[i] = ms * 1e3f;
+    }
+    if (err != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "step timing: %s", hipGetErrorString(err));
     return TF_OK;
 }
 

@@ -11,13 +11,20 @@
 struct tf_ctx {
     int device = 0;
     int num_cus = 0;
-    int long_blocks_per_cu = 4;         // 256-thread blocks per CU launched by the persistent row streamers
+    int stream_blocks_per_cu = 2;       // 256-thread blocks per CU launched by the persistent row streamers
     // wrapper-owned scratch, as the reference's kernel classes own theirs
     float *router_logits = nullptr;     // 256 floats (MoE.swift:92-99)
     void *head_x_normed = nullptr;      // kMaxHeadD halves (LMHeadChainInt4.swift:38-51)
     float *head_summaries = nullptr;    // kMaxHeadWaves x {value, index bits}
     float *head_logits = nullptr;       // lazily sized fp32 logits for the unaligned lm_head path
     size_t head_logits_count = 0;
+    uint32_t *group_scratch = nullptr;  // kGroupSegments x 256 per-segment expert counts of the device pair grouping
+    float *prefill_logits = nullptr;    // lazily sized [tokens, experts] router logits of the multi-token router
+    size_t prefill_logits_count = 0;
+    // optional device-time bracketing of the decode step's three launches
+    bool step_timing = false;
+    bool step_timed = false;            // a step has been recorded since timing was enabled
+    hipEvent_t step_events[5] = {nullptr, nullptr, nullptr, nullptr, nullptr};
     char last_error[512] = {0};
 };
 
@@ -25,6 +32,7 @@ namespace tfk {
 
 constexpr uint32_t kMaxHeadD = 16384;
 constexpr uint32_t kMaxHeadWaves = 16384;
+constexpr uint32_t kGroupSegments = 64;   // token segments the device pair grouping counts and places independently
 
 inline int32_t fail(tf_ctx *ctx, int32_t status, const char *fmt, ...) {
     if (ctx) {

@@ -40,50 +40,55 @@ __device__ __forceinline__ void store_out(OutT *y, long row, float v) {
 }
 
 // ------------------------------------------------------------------------------------------------ GEMV kernels
-// Persistent: every wave walks tiles wave, wave + nwaves, ... of RT rows, requesting tile i+1 before reducing tile i.
+// Persistent: every wave walks tiles wave, wave + nwaves, ... of RT rows, requesting tile i+1 before reducing tile i
+// (two tile buffers used alternately, so nothing is copied).
 // FUSE_NORM: x is the raw hidden vector and the block normalises it itself (rmsnorm_bf16w with weight norm_w) into LDS.
 template <int RT, int NP, int SD, typename OutT, bool FUSE_NORM>
-__global__ __launch_bounds__(256, 4) void gemv4_long_kernel(const uint8_t *W, const uint16_t *S, const uint16_t *B,
+__global__ __launch_bounds__(256, 4) void gemv4_long_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B,
                                                             const half_t *x, const uint16_t *norm_w, float eps, OutT *y,
                                                             long m, int k) {
     const int lane = threadIdx.x & 63;
-    const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const long wave = uniform_int((int)(((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6));
     const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
     const long ntiles = (m + RT - 1) / RT;
     const bool active = wave < ntiles;
-    const int groups = k >> 6;
     const size_t tile_bytes = (size_t)RT * (k >> 1);
+    const size_t sb_bytes = (size_t)RT * (k >> 6) * 2;
 
-    LongRows<RT, NP> lr;
-    typename LongRows<RT, NP>::Tile cur, nxt;
-    lr.init_map(k, lane);
+    RowStream<RT, NP> rs;
+    typename RowStream<RT, NP>::Tile ta, tb;
+    rs.init_map(k, lane);
     long tile = wave;
-    if (active)
-        lr.load(cur, W + tile * tile_bytes, S + tile * RT * groups, B + tile * RT * groups, (int)min((long)RT, m - tile * RT), lane);
+    // the first tile does not depend on the activations: request it before anything else
+    if (active) rs.load(ta, W + tile * tile_bytes, S + tile * sb_bytes, B + tile * sb_bytes, m - tile * RT);
     if constexpr (FUSE_NORM) {
         __shared__ __align__(16) half_t xn_lds[kMaxFusedNormD];
         __shared__ float partial[4];
         block_rmsnorm_to_lds(x, norm_w, eps, k, xn_lds, partial);
-        if (active) lr.init_x(xn_lds, lane);
+        if (active) rs.init_x(xn_lds);
     } else {
-        if (active) lr.init_x(x, lane);
+        if (active) rs.init_x(x);
     }
     if (!active) return;
-    for (;;) {
-        const long next = tile + nwaves;
-        const bool has_next = next < ntiles;
-        if (has_next)
-            lr.load(nxt, W + next * tile_bytes, S + next * RT * groups, B + next * RT * groups,
-                    (int)min((long)RT, m - next * RT), lane);
+    auto emit = [&](const typename RowStream<RT, NP>::Tile &t, long at) {
         float out[RT];
-        lr.template reduce<SD>(cur, out);
+        rs.template reduce<SD>(t, out);
         if (lane == 0) {
 #pragma unroll
             for (int r = 0; r < RT; ++r)
-                if (tile * RT + r < m) store_out(y, tile * RT + r, out[r]);
+                if (at * RT + r < m) store_out(y, at * RT + r, out[r]);
         }
-        if (!has_next) break;
-        cur = nxt;
+    };
+    for (;;) {
+        long next = tile + nwaves;
+        if (next < ntiles) rs.load(tb, W + next * tile_bytes, S + next * sb_bytes, B + next * sb_bytes, m - next * RT);
+        emit(ta, tile);
+        if (next >= ntiles) break;
+        tile = next;
+        next = tile + nwaves;
+        if (next < ntiles) rs.load(ta, W + next * tile_bytes, S + next * sb_bytes, B + next * sb_bytes, m - next * RT);
+        emit(tb, tile);
+        if (next >= ntiles) break;
         tile = next;
     }
 }
@@ -263,18 +268,16 @@ static int32_t launch_gemv4_typed(tf_ctx *ctx, hipStream_t st, const uint8_t *w,
     const LongPlan plan = plan_long_rows((int)n);
     if (fast && plan.rt > 0) {
         const long ntiles = ((long)m + plan.rt - 1) / plan.rt;
-        const long max_blocks = (long)ctx->num_cus * ctx->long_blocks_per_cu;
+        const long max_blocks = (long)ctx->num_cus * ctx->stream_blocks_per_cu;
         const uint32_t grid = (uint32_t)std::max<long>(1, std::min<long>((ntiles + 3) / 4, max_blocks));
-        const uint16_t *s16 = reinterpret_cast<const uint16_t *>(s);
-        const uint16_t *b16 = reinterpret_cast<const uint16_t *>(b);
 #define TF_LONG_CASE(RT_, NP_)                                                                                          \
     if (plan.rt == RT_ && plan.np == NP_) {                                                                             \
         if (norm_w)                                                                                                     \
-            hipLaunchKernelGGL((gemv4_long_kernel<RT_, NP_, SD, OutT, true>), dim3(grid), dim3(256), 0, st, w, s16,     \
-                               b16, x, norm_w, eps, y, (long)m, (int)n);                                                \
+            hipLaunchKernelGGL((gemv4_long_kernel<RT_, NP_, SD, OutT, true>), dim3(grid), dim3(256), 0, st, w, s,       \
+                               b, x, norm_w, eps, y, (long)m, (int)n);                                                  \
         else                                                                                                            \
-            hipLaunchKernelGGL((gemv4_long_kernel<RT_, NP_, SD, OutT, false>), dim3(grid), dim3(256), 0, st, w, s16,    \
-                               b16, x, norm_w, eps, y, (long)m, (int)n);                                                \
+            hipLaunchKernelGGL((gemv4_long_kernel<RT_, NP_, SD, OutT, false>), dim3(grid), dim3(256), 0, st, w, s,      \
+                               b, x, norm_w, eps, y, (long)m, (int)n);                                                  \
         return check_launch(ctx, "gemv4_long");                                                                         \
     }
         TF_LONG_CASE(1, 1) TF_LONG_CASE(1, 2) TF_LONG_CASE(1, 3) TF_LONG_CASE(1, 4)

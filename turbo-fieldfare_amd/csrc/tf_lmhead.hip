@@ -23,7 +23,7 @@ __device__ __forceinline__ void better(Best &b, float v, uint32_t idx) {
 // block normalises the hidden vector itself (rmsnorm_bf16w needs no kernel of its own).  Each block folds its best
 // {value, index} into one of kHeadCells 64-bit cells with a single atomic max on the key
 // (orderable(value) << 32 | ~index): larger value wins, equal values resolve to the lower index, 0 means "nothing finite".
-// No fences, no waiting; head_decode_kernel turns the cells into the token.
+// The block that finishes last turns the cells into the token and clears them for the next call.
 constexpr uint32_t kHeadCells = 64;
 
 __device__ __forceinline__ unsigned long long best_key(float v, uint32_t idx) {
@@ -34,79 +34,95 @@ __device__ __forceinline__ unsigned long long best_key(float v, uint32_t idx) {
 }
 
 template <int RT, int NP, int SD, bool FUSE_NORM>
-__global__ __launch_bounds__(256, 4) void head_greedy_long_kernel(const uint8_t *W, const uint16_t *S, const uint16_t *B,
+__global__ __launch_bounds__(256, 4) void head_greedy_long_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B,
                                                                const half_t *x, const uint16_t *norm_w, float eps,
-                                                               unsigned long long *cells, long v_rows, int k) {
+                                                               unsigned long long *cells, uint32_t *out_token, long v_rows,
+                                                               int k) {
     __shared__ float sv[4];
     __shared__ uint32_t si[4];
     const int lane = threadIdx.x & 63;
     const int wib = threadIdx.x >> 6;
-    const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const long wave = uniform_int((int)(((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6));
     const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
     const long ntiles = (v_rows + RT - 1) / RT;
     Best best{-INFINITY, 0xFFFFFFFFu};
     const bool active = wave < ntiles;
-    const int groups = k >> 6;
     const size_t tile_bytes = (size_t)RT * (k >> 1);
-    LongRows<RT, NP> lr;
-    typename LongRows<RT, NP>::Tile cur, nxt;
-    lr.init_map(k, lane);
+    const size_t sb_bytes = (size_t)RT * (k >> 6) * 2;
+    RowStream<RT, NP> rs;
+    typename RowStream<RT, NP>::Tile ta, tb;
+    rs.init_map(k, lane);
     long tile = wave;
     // the first tile does not depend on the activations: request it before normalising them
-    if (active)
-        lr.load(cur, W + tile * tile_bytes, S + tile * RT * groups, B + tile * RT * groups, (int)min((long)RT, v_rows - tile * RT), lane);
+    if (active) rs.load(ta, W + tile * tile_bytes, S + tile * sb_bytes, B + tile * sb_bytes, v_rows - tile * RT);
     if constexpr (FUSE_NORM) {
         __shared__ __align__(16) half_t xn_lds[kMaxFusedNormD];
         __shared__ float partial[4];
         block_rmsnorm_to_lds(x, norm_w, eps, k, xn_lds, partial);
-        if (active) lr.init_x(xn_lds, lane);
+        if (active) rs.init_x(xn_lds);
     } else {
-        if (active) lr.init_x(x, lane);
+        if (active) rs.init_x(x);
     }
+    // rows ascend within a wave, so a strict comparison keeps the lowest index among equals
+    auto consider = [&](const typename RowStream<RT, NP>::Tile &t, long at) {
+        float out[RT];
+        rs.template reduce<SD>(t, out);
+#pragma unroll
+        for (int r = 0; r < RT; ++r) {
+            const long row = at * RT + r;
+            const float z = out[r];
+            if (row < v_rows && __builtin_isfinite(z) && z > best.v) {
+                best.v = z;
+                best.idx = (uint32_t)row;
+            }
+        }
+    };
     if (active) {
         for (;;) {
-            const long next = tile + nwaves;
-            const bool has_next = next < ntiles;
-            if (has_next)
-                lr.load(nxt, W + next * tile_bytes, S + next * RT * groups, B + next * RT * groups,
-                        (int)min((long)RT, v_rows - next * RT), lane);
-            float out[RT];
-            lr.template reduce<SD>(cur, out);
-#pragma unroll
-            for (int r = 0; r < RT; ++r) {
-                const long row = tile * RT + r;
-                const float z = out[r];
-                if (row < v_rows && __builtin_isfinite(z) && z > best.v) {
-                    best.v = z;
-                    best.idx = (uint32_t)row;
-                }
-            }
-            if (!has_next) break;
-            cur = nxt;
+            long next = tile + nwaves;
+            if (next < ntiles) rs.load(tb, W + next * tile_bytes, S + next * sb_bytes, B + next * sb_bytes, v_rows - next * RT);
+            consider(ta, tile);
+            if (next >= ntiles) break;
+            tile = next;
+            next = tile + nwaves;
+            if (next < ntiles) rs.load(ta, W + next * tile_bytes, S + next * sb_bytes, B + next * sb_bytes, v_rows - next * RT);
+            consider(tb, tile);
+            if (next >= ntiles) break;
             tile = next;
         }
     }
     if (lane == 0) { sv[wib] = best.v; si[wib] = best.idx; }
     __syncthreads();
+    // Fold the block's best into a cell, then take a ticket.  Both are device-scope atomics performed at the memory
+    // side, and the ticket is only requested after the fold has returned, so the block that draws the last ticket
+    // finds every fold in the cells (read with atomics as well) without any cache write-back or invalidate.
+    __shared__ uint32_t is_last;
     if (threadIdx.x == 0) {
         Best b{sv[0], si[0]};
         for (int w = 1; w < 4; ++w) better(b, sv[w], si[w]);
         const unsigned long long key = best_key(b.v, b.idx);
-        if (key) atomicMax(cells + (blockIdx.x % kHeadCells), key);
+        unsigned long long seen = 0ull;
+        if (key) seen = atomicMax(cells + (blockIdx.x % kHeadCells), key);
+        // the ticket increment depends on the value the fold returned
+        uint32_t one = 1u;
+        const uint32_t seen_lo = (uint32_t)seen;
+        asm volatile("" : "+v"(one) : "v"(seen_lo));
+        unsigned int *ticket = reinterpret_cast<unsigned int *>(cells + kHeadCells);
+        is_last = atomicAdd(ticket, one) == gridDim.x - 1 ? 1u : 0u;
     }
-}
-
-// One wave: the largest key among the cells is the answer; the cells are cleared for the next call.
-__global__ __launch_bounds__(64) void head_decode_kernel(unsigned long long *cells, uint32_t *out_token) {
-    const int lane = threadIdx.x;
-    unsigned long long key = cells[lane];
-    cells[lane] = 0ull;
+    __syncthreads();
+    if (is_last && wib == 0) {
+        unsigned long long key = __hip_atomic_exchange(cells + lane, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        const unsigned long long other = __shfl_xor(key, off, kWave);
-        key = other > key ? other : key;
+        for (int off = 32; off >= 1; off >>= 1) {
+            const unsigned long long other = __shfl_xor(key, off, kWave);
+            key = other > key ? other : key;
+        }
+        if (lane == 0) {
+            out_token[0] = key ? 0xFFFFFFFFu - (uint32_t)(key & 0xFFFFFFFFull) : 0u;
+            __hip_atomic_store(reinterpret_cast<unsigned int *>(cells + kHeadCells), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
     }
-    if (lane == 0) out_token[0] = key ? 0xFFFFFFFFu - (uint32_t)(key & 0xFFFFFFFFull) : 0u;
 }
 
 // Fallback first stage: argmax summaries over an fp32 logits vector (one summary per block).
@@ -193,15 +209,13 @@ int32_t tf_lm_head_greedy_int4(tf_ctx *ctx, tf_stream stream, const void *hidden
     uint32_t n_summaries = 0;
     if (rows_fast) {
         const long ntiles = ((long)vocab + plan.rt - 1) / plan.rt;
-        const long max_blocks = std::min<long>((long)ctx->num_cus * ctx->long_blocks_per_cu, 1024);
+        const long max_blocks = (long)ctx->num_cus * ctx->stream_blocks_per_cu;
         const uint32_t grid = (uint32_t)std::max<long>(1, std::min<long>((ntiles + 3) / 4, max_blocks));
-        const uint16_t *s16 = reinterpret_cast<const uint16_t *>(s);
-        const uint16_t *b16 = reinterpret_cast<const uint16_t *>(b);
         unsigned long long *cells = reinterpret_cast<unsigned long long *>(ctx->head_summaries + 2 * kMaxHeadWaves);
         bool launched = false;
 #define TF_HEAD_LAUNCH(RT_, NP_, SD_, FN_)                                                                              \
-    hipLaunchKernelGGL((head_greedy_long_kernel<RT_, NP_, SD_, FN_>), dim3(grid), dim3(256), 0, st, w, s16, b16,        \
-                       FN_ ? hid : xn, nw, rms_eps, cells, (long)vocab, (int)d)
+    hipLaunchKernelGGL((head_greedy_long_kernel<RT_, NP_, SD_, FN_>), dim3(grid), dim3(256), 0, st, w, s, b,            \
+                       FN_ ? hid : xn, nw, rms_eps, cells, static_cast<uint32_t *>(out_token), (long)vocab, (int)d)
 #define TF_HEAD_CASE(RT_, NP_)                                                                                          \
     if (!launched && plan.rt == RT_ && plan.np == NP_) {                                                                \
         launched = true;                                                                                                \
@@ -213,10 +227,7 @@ int32_t tf_lm_head_greedy_int4(tf_ctx *ctx, tf_stream stream, const void *hidden
         TF_HEAD_CASE(4, 1) TF_HEAD_CASE(4, 2) TF_HEAD_CASE(4, 3) TF_HEAD_CASE(4, 4)
 #undef TF_HEAD_CASE
 #undef TF_HEAD_LAUNCH
-        rc = check_launch(ctx, "lm_head_greedy rows");
-        if (rc != TF_OK) return rc;
-        hipLaunchKernelGGL(head_decode_kernel, dim3(1), dim3(64), 0, st, cells, static_cast<uint32_t *>(out_token));
-        return check_launch(ctx, "lm_head_greedy decode");
+        return check_launch(ctx, "lm_head_greedy rows");
     } else {
         // short or unaligned rows: fp32 logits into wrapper-owned scratch, then a two-stage argmax
         if (ctx->head_logits_count < vocab) {

@@ -43,14 +43,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t *W, co
 __global__ __launch_bounds__(64) void router_select_kernel(const float *logits, const uint16_t *per_expert_scale,
                                                            uint32_t *out_indices, half_t *out_weights, uint32_t num_experts,
                                                            uint32_t top_k) {
-    const int lane = threadIdx.x;
-    float gain[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t c = lane + 64 * j;
-        gain[j] = c < num_experts ? bf16_to_f32(per_expert_scale[c]) : 0.0f;
-    }
-    router_select(logits, gain, out_indices, out_weights, num_experts, top_k, lane);
+    router_select(logits, per_expert_scale, out_indices, out_weights, num_experts, top_k, threadIdx.x);
 }
 
 // ------------------------------------------------------------------------------------------------ phase 1
@@ -77,38 +70,70 @@ __device__ __forceinline__ bool phase1_slot(const Phase1Geom &g, uint32_t unit, 
     return slot < g.top_k;
 }
 
-// D > 1024: one wave per RT-row tile of one slot; the gate tile and the up tile share the activations in registers.
-template <int RT, int NP, int SD>
-__global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_expert_offsets off, const half_t *x,
-                                                          half_t *acts, Phase1Geom g) {
-    const int lane = threadIdx.x & 63;
-    const uint32_t unit = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
-    const uint32_t tiles = (g.f + RT - 1) / RT;
-    uint32_t slot, tile;
-    if (!phase1_slot(g, unit, tiles, slot, tile)) return;
-    const uint8_t *base = blob_base(routed, slot);
-    const int groups = g.d >> 6;
-    const uint32_t row0 = tile * RT;
-    const int rows_left = (int)min((uint32_t)RT, g.f - row0);
-    const size_t w_byte = (size_t)row0 * (g.d >> 1);
-    const size_t sb_byte = (size_t)row0 * groups * 2;
+// Selection fused into phase 1 (the decode step): wave 0 of every block repeats the top-k over the router's logits
+// while the block's activation loads are in flight, instead of the grid waiting for a selection kernel and then for its
+// indices; block 0 publishes indices and weights for phase 2 and for the caller.
+struct FusedSelect {
+    const float *logits;
+    const uint16_t *per_expert_scale;
+    uint32_t *out_indices;
+    half_t *out_weights;
+    uint32_t num_experts;
+};
 
-    LongRows<RT, NP> lr;
-    typename LongRows<RT, NP>::Tile tg, tu;
-    // weights do not depend on the activations: issue their loads first
-    lr.init_map(g.d, lane);
-    lr.load(tg, base + off.gate_W_off + w_byte, reinterpret_cast<const uint16_t *>(base + off.gate_s_off + sb_byte),
-            reinterpret_cast<const uint16_t *>(base + off.gate_b_off + sb_byte), rows_left, lane);
-    lr.load(tu, base + off.up_W_off + w_byte, reinterpret_cast<const uint16_t *>(base + off.up_s_off + sb_byte),
-            reinterpret_cast<const uint16_t *>(base + off.up_b_off + sb_byte), rows_left, lane);
-    lr.init_x(x, lane);
+// D > 1024: one wave per RT-row tile of one slot; the gate tile and the up tile share the activations, which the block
+// stages once in LDS.  Order of requests: activations, expert lookup, weights; the activations are arranged while the
+// weights are in flight (with the fused selection the weights are requested right after the block's barrier).
+template <int RT, int NP, int SD, bool FUSED>
+__global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_expert_offsets off, const half_t *x,
+                                                          half_t *acts, Phase1Geom g, FusedSelect fs) {
+    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
+    __shared__ float xsum[XStage::kMaxK / 32];
+    __shared__ uint32_t chosen[TF_MAX_STREAMED_EXPERTS];
+    const int lane = threadIdx.x & 63;
+    const uint32_t unit = uniform_u32((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
+    const uint32_t tiles = (g.f + RT - 1) / RT;
+    XStage stage;
+    stage.request(x, (int)g.d);
+    uint32_t slot = 0, tile = 0;
+    const bool live = phase1_slot(g, unit, tiles, slot, tile);
+    const uint32_t row0 = tile * RT;
+    const size_t w_byte = (size_t)row0 * (g.d >> 1);
+    const size_t sb_byte = (size_t)row0 * (g.d >> 6) * 2;
+    RowStream<RT, NP> rs;
+    typename RowStream<RT, NP>::Tile tg, tu;
+    rs.init_map((int)g.d, lane);
+    auto request_weights = [&](const uint8_t *base) {
+        rs.load(tg, base + off.gate_W_off + w_byte, base + off.gate_s_off + sb_byte, base + off.gate_b_off + sb_byte, g.f - row0);
+        rs.load(tu, base + off.up_W_off + w_byte, base + off.up_s_off + sb_byte, base + off.up_b_off + sb_byte, g.f - row0);
+    };
+    if constexpr (FUSED) {
+        if (uniform_u32(threadIdx.x >> 6) == 0) {
+            uint32_t idx;
+            half_t weight;
+            router_select_lanes(fs.logits, fs.per_expert_scale, fs.num_experts, g.top_k, lane, idx, weight);
+            if ((uint32_t)lane < g.top_k) {
+                chosen[lane] = idx < fs.num_experts ? idx : fs.num_experts - 1;
+                if (blockIdx.x == 0) {
+                    fs.out_indices[lane] = idx;
+                    fs.out_weights[lane] = weight;
+                }
+            }
+        }
+    } else {
+        if (live) request_weights(uniform_ptr(blob_base(routed, slot)));
+    }
+    stage.publish((int)g.d, xa, xsum);
+    if (!live) return;
+    if constexpr (FUSED) request_weights(routed.pool + (uint64_t)uniform_u32(chosen[slot]) * routed.stride);
+    rs.init_x_lds(xa, xsum, (int)g.d);
     float gate[RT], up[RT];
-    lr.template reduce<SD>(tg, gate);
-    lr.template reduce<SD>(tu, up);
+    rs.template reduce<SD>(tg, gate);
+    rs.template reduce<SD>(tu, up);
     if (lane == 0) {
 #pragma unroll
         for (int r = 0; r < RT; ++r)
-            if (r < rows_left) store_act(acts, slot * g.f + row0 + r, gate[r], up[r]);
+            if (row0 + r < g.f) store_act(acts, slot * g.f + row0 + r, gate[r], up[r]);
     }
 }
 
@@ -223,29 +248,37 @@ __global__ __launch_bounds__(512) void phase2_generic_kernel(RoutedArg routed, t
 // gate and up tiles share the activations; both sums are rounded to fp16 (the reference's two GEMVs write fp16)
 // before GeGLU (gelu_mul_fp16), and all three vectors land in the caller's scratch buffers.
 template <int RT, int NP, int SD>
-__global__ __launch_bounds__(256) void shared_gate_up_long_kernel(const uint8_t *gW, const uint16_t *gS, const uint16_t *gB,
-                                                                  const uint8_t *uW, const uint16_t *uS, const uint16_t *uB,
+__global__ __launch_bounds__(256) void shared_gate_up_long_kernel(const uint8_t *gW, const uint8_t *gS, const uint8_t *gB,
+                                                                  const uint8_t *uW, const uint8_t *uS, const uint8_t *uB,
                                                                   const half_t *x, half_t *gate_out, half_t *up_out,
                                                                   half_t *act_out, uint32_t f, int d) {
+    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
+    __shared__ float xsum[XStage::kMaxK / 32];
     const int lane = threadIdx.x & 63;
-    const uint32_t tile = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint32_t tile = uniform_u32((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
     const uint32_t row0 = tile * RT;
-    if (row0 >= f) return;
-    const int groups = d >> 6;
-    const int rows_left = (int)min((uint32_t)RT, f - row0);
-    LongRows<RT, NP> lr;
-    typename LongRows<RT, NP>::Tile tg, tu;
-    lr.init_map(d, lane);
-    lr.load(tg, gW + (size_t)row0 * (d >> 1), gS + (size_t)row0 * groups, gB + (size_t)row0 * groups, rows_left, lane);
-    lr.load(tu, uW + (size_t)row0 * (d >> 1), uS + (size_t)row0 * groups, uB + (size_t)row0 * groups, rows_left, lane);
-    lr.init_x(x, lane);
+    const bool live = row0 < f;
+    XStage stage;
+    stage.request(x, d);
+    RowStream<RT, NP> rs;
+    typename RowStream<RT, NP>::Tile tg, tu;
+    rs.init_map(d, lane);
+    if (live) {
+        const size_t w_byte = (size_t)row0 * (d >> 1);
+        const size_t sb_byte = (size_t)row0 * (d >> 6) * 2;
+        rs.load(tg, gW + w_byte, gS + sb_byte, gB + sb_byte, f - row0);
+        rs.load(tu, uW + w_byte, uS + sb_byte, uB + sb_byte, f - row0);
+    }
+    stage.publish(d, xa, xsum);
+    if (!live) return;
+    rs.init_x_lds(xa, xsum, d);
     float gate[RT], up[RT];
-    lr.template reduce<SD>(tg, gate);
-    lr.template reduce<SD>(tu, up);
+    rs.template reduce<SD>(tg, gate);
+    rs.template reduce<SD>(tu, up);
     if (lane == 0) {
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
-            if (r >= rows_left) continue;
+            if (row0 + r >= f) continue;
             const half_t g16 = (half_t)gate[r], u16 = (half_t)up[r];
             gate_out[row0 + r] = g16;
             up_out[row0 + r] = u16;
@@ -282,9 +315,11 @@ bool offsets_even(const tf_expert_offsets &o) {
     return ((o.gate_W_off | o.gate_s_off | o.gate_b_off | o.up_W_off | o.up_s_off | o.up_b_off | o.down_W_off | o.down_s_off | o.down_b_off) & 1u) == 0;
 }
 
+// fused != nullptr (decode step): the expert indices are not read from routed->indices but selected inside the
+// kernel from fused->logits; returns TF_ERR_UNAVAILABLE when the operands do not allow the fused kernel.
 int32_t phase1_entry(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *routed, const tf_expert_offsets *off, const void *x,
                      void *acts, const uint32_t *active_slots, uint32_t active_count, bool subset, uint32_t d, uint32_t f,
-                     uint32_t top_k, tf_dtype sd) {
+                     uint32_t top_k, tf_dtype sd, const FusedSelect *fused = nullptr, int mark_event = -1) {
     TF_REQUIRE(ctx, ctx && routed && off && x && acts, TF_ERR_INVALID_ARGUMENT, "moe_phase1: null argument");
     TF_REQUIRE(ctx, top_k == TF_MAX_STREAMED_EXPERTS, TF_ERR_INVALID_ARGUMENT, "moe_phase1: topK must be 8, got %u", top_k);
     TF_REQUIRE(ctx, d > 0 && d % TF_GROUP_SIZE == 0 && f > 0, TF_ERR_INVALID_ARGUMENT, "moe_phase1: d must be a multiple of 64 and f positive");
@@ -304,6 +339,7 @@ int32_t phase1_entry(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *route
     half_t *ah = static_cast<half_t *>(acts);
     const bool fast = all16 && aligned16(x) && (off->gate_W_off % 16 == 0) && (off->up_W_off % 16 == 0);
     const int SD = sd == TF_BF16 ? 0 : 1;
+    if (fused && !(fast && d > 1024 && d <= (uint32_t)XStage::kMaxK && plan_long_rows((int)d).rt > 0)) return TF_ERR_UNAVAILABLE;
     if (fast && d <= 1024) {
         constexpr int NPASS = 2;
         const uint32_t units = n_slots * ((f + 2 * NPASS - 1) / (2 * NPASS));
@@ -313,19 +349,27 @@ int32_t phase1_entry(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *route
         return check_launch(ctx, "moe_phase1_short");
     }
     const LongPlan plan = plan_long_rows((int)d);
-    if (fast && plan.rt > 0) {
+    const FusedSelect no_select = {nullptr, nullptr, nullptr, nullptr, 0};
+    if (fast && d > 1024 && plan.rt > 0) {
         const uint32_t units = n_slots * ((f + plan.rt - 1) / plan.rt);
         const dim3 grid((units + 3) / 4);
+        if (fused && mark_event >= 0 && ctx->step_timing) (void)hipEventRecord(ctx->step_events[mark_event], st);
+#define TF_P1_LAUNCH(RT_, NP_, SD_)                                                                                  \
+    do {                                                                                                             \
+        if (fused) hipLaunchKernelGGL((phase1_long_kernel<RT_, NP_, SD_, true>), grid, dim3(256), 0, st, arg, *off, xh, ah, g, *fused); \
+        else hipLaunchKernelGGL((phase1_long_kernel<RT_, NP_, SD_, false>), grid, dim3(256), 0, st, arg, *off, xh, ah, g, no_select);    \
+    } while (0)
 #define TF_P1_CASE(RT_, NP_)                                                                                         \
     if (plan.rt == RT_ && plan.np == NP_) {                                                                          \
-        if (SD == 0) hipLaunchKernelGGL((phase1_long_kernel<RT_, NP_, 0>), grid, dim3(256), 0, st, arg, *off, xh, ah, g); \
-        else hipLaunchKernelGGL((phase1_long_kernel<RT_, NP_, 1>), grid, dim3(256), 0, st, arg, *off, xh, ah, g);     \
+        if (SD == 0) TF_P1_LAUNCH(RT_, NP_, 0);                                                                      \
+        else TF_P1_LAUNCH(RT_, NP_, 1);                                                                              \
         return check_launch(ctx, "moe_phase1_long");                                                                 \
     }
         TF_P1_CASE(1, 1) TF_P1_CASE(1, 2) TF_P1_CASE(1, 3) TF_P1_CASE(1, 4)
         TF_P1_CASE(2, 1) TF_P1_CASE(2, 2) TF_P1_CASE(2, 3) TF_P1_CASE(2, 4)
         TF_P1_CASE(4, 1) TF_P1_CASE(4, 2) TF_P1_CASE(4, 3) TF_P1_CASE(4, 4)
 #undef TF_P1_CASE
+#undef TF_P1_LAUNCH
     }
     const uint32_t units = n_slots * f;
     const dim3 grid((units + 3) / 4);
@@ -334,15 +378,12 @@ int32_t phase1_entry(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *route
     return check_launch(ctx, "moe_phase1_generic");
 }
 
-}  // namespace
-
-extern "C" {
-
-int32_t tf_router_gemma4(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset, const void *scales,
-                         uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *hidden,
-                         const void *effective_scale, uint64_t effective_scale_offset, const void *per_expert_scale,
-                         uint64_t per_expert_scale_offset, void *out_indices, void *out_weights, uint32_t num_experts,
-                         uint32_t d, uint32_t top_k) {
+// Router stage 1: validates the whole router call and writes the logits into the context's scratch.
+int32_t router_logits_entry(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset, const void *scales,
+                            uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *hidden,
+                            const void *effective_scale, uint64_t effective_scale_offset, const void *per_expert_scale,
+                            uint64_t per_expert_scale_offset, void *out_indices, void *out_weights, uint32_t num_experts,
+                            uint32_t d, uint32_t top_k) {
     TF_REQUIRE(ctx, ctx && weights && scales && biases && hidden && effective_scale && per_expert_scale && out_indices && out_weights,
                TF_ERR_INVALID_ARGUMENT, "router_gemma4: null argument");
     TF_REQUIRE(ctx, d > 0 && d % TF_GROUP_SIZE == 0, TF_ERR_INVALID_ARGUMENT, "router_gemma4: d must be a multiple of 64, got %u", d);
@@ -371,11 +412,32 @@ int32_t tf_router_gemma4(tf_ctx *ctx, tf_stream stream, const void *weights, uin
         default: TF_ROUTER(0); break;
     }
 #undef TF_ROUTER
-    const int32_t rc = check_launch(ctx, "router_gemma4 logits");
-    if (rc != TF_OK) return rc;
-    hipLaunchKernelGGL(router_select_kernel, dim3(1), dim3(64), 0, st, ctx->router_logits, reinterpret_cast<const uint16_t *>(pes),
+    return check_launch(ctx, "router_gemma4 logits");
+}
+
+// Router stage 2: one wave selects from the logits.
+int32_t router_select_entry(tf_ctx *ctx, tf_stream stream, const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                            void *out_indices, void *out_weights, uint32_t num_experts, uint32_t top_k) {
+    hipLaunchKernelGGL(router_select_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), ctx->router_logits,
+                       reinterpret_cast<const uint16_t *>(at(per_expert_scale, per_expert_scale_offset)),
                        static_cast<uint32_t *>(out_indices), static_cast<half_t *>(out_weights), num_experts, top_k);
     return check_launch(ctx, "router_gemma4 select");
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t tf_router_gemma4(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset, const void *scales,
+                         uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *hidden,
+                         const void *effective_scale, uint64_t effective_scale_offset, const void *per_expert_scale,
+                         uint64_t per_expert_scale_offset, void *out_indices, void *out_weights, uint32_t num_experts,
+                         uint32_t d, uint32_t top_k) {
+    int32_t rc = router_logits_entry(ctx, stream, weights, weights_offset, scales, scales_offset, biases, biases_offset, hidden,
+                                     effective_scale, effective_scale_offset, per_expert_scale, per_expert_scale_offset,
+                                     out_indices, out_weights, num_experts, d, top_k);
+    if (rc != TF_OK) return rc;
+    return router_select_entry(ctx, stream, per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, top_k);
 }
 
 int32_t tf_moe_phase1_gate_up_act(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *routed, const tf_expert_offsets *routed_offsets,
@@ -428,18 +490,38 @@ int32_t tf_moe_decode_step(tf_ctx *ctx, tf_stream stream, const void *router_wei
                            const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
                            void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype) {
     TF_REQUIRE(ctx, ctx && expert_pool && out_indices, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: null argument");
-    int32_t rc = tf_router_gemma4(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset,
-                                  router_biases, router_biases_offset, router_x, effective_scale, effective_scale_offset,
-                                  per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, d, top_k);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool timed = ctx->step_timing;
+    auto mark = [&](int i) {
+        if (timed) (void)hipEventRecord(ctx->step_events[i], st);
+    };
+    mark(0);
+    int32_t rc = router_logits_entry(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset,
+                                     router_biases, router_biases_offset, router_x, effective_scale, effective_scale_offset,
+                                     per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, d, top_k);
     if (rc != TF_OK) return rc;
     tf_routed_blobs routed = {};
     routed.pool = expert_pool;
     routed.pool_stride = expert_pool_stride;
     routed.indices = static_cast<const uint32_t *>(out_indices);
     routed.num_experts = num_experts;
-    rc = tf_moe_phase1_gate_up_act(ctx, stream, &routed, routed_offsets, x, acts, d, f, top_k, scale_dtype);
+    // Three launches when the vector path applies: logits, phase 1 with the selection repeated by every wave, phase 2.
+    const FusedSelect fused = {ctx->router_logits, reinterpret_cast<const uint16_t *>(at(per_expert_scale, per_expert_scale_offset)),
+                               static_cast<uint32_t *>(out_indices), static_cast<half_t *>(out_weights), num_experts};
+    rc = phase1_entry(ctx, stream, &routed, routed_offsets, x, acts, nullptr, 0, false, d, f, top_k, scale_dtype, &fused, 1);
+    if (rc == TF_ERR_UNAVAILABLE) {
+        rc = router_select_entry(ctx, stream, per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, top_k);
+        if (rc != TF_OK) return rc;
+        mark(1);
+        rc = phase1_entry(ctx, stream, &routed, routed_offsets, x, acts, nullptr, 0, false, d, f, top_k, scale_dtype);
+    }
     if (rc != TF_OK) return rc;
-    return tf_moe_phase2_down_reduce(ctx, stream, &routed, routed_offsets, acts, out_weights, residual, y, d, f, top_k, scale_dtype);
+    mark(2);
+    rc = tf_moe_phase2_down_reduce(ctx, stream, &routed, routed_offsets, acts, out_weights, residual, y, d, f, top_k, scale_dtype);
+    mark(3);
+    mark(4);
+    if (timed && rc == TF_OK) ctx->step_timed = true;
+    return rc;
 }
 
 int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, uint64_t x_length,
@@ -484,10 +566,8 @@ int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream, const void *x, uint
     if (fused) {
         const uint32_t tiles = (f + plan.rt - 1) / plan.rt;
         const dim3 grid((tiles + 3) / 4);
-        const uint16_t *gs = reinterpret_cast<const uint16_t *>(at(gate->scales, gate->scales_offset));
-        const uint16_t *gb = reinterpret_cast<const uint16_t *>(at(gate->biases, gate->biases_offset));
-        const uint16_t *us = reinterpret_cast<const uint16_t *>(at(up->scales, up->scales_offset));
-        const uint16_t *ub = reinterpret_cast<const uint16_t *>(at(up->biases, up->biases_offset));
+        const uint8_t *gs = at(gate->scales, gate->scales_offset), *gb = at(gate->biases, gate->biases_offset);
+        const uint8_t *us = at(up->scales, up->scales_offset), *ub = at(up->biases, up->biases_offset);
         bool launched = false;
 #define TF_SH_CASE(RT_, NP_)                                                                                                    \
     if (!launched && plan.rt == RT_ && plan.np == NP_) {                                                                        \

@@ -22,6 +22,8 @@ int32_t launch_grouped_down_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTable 
 
 namespace {
 
+constexpr uint32_t kFewTokens = 64;   // up to here the router runs one wave per (token, expert)
+
 // ------------------------------------------------------------------------------------------------ router block
 // One 256-thread block per token row: the four waves share the experts (wave w takes e = w, w+4, ...), the logits meet in
 // LDS, wave 0 selects.
@@ -41,81 +43,129 @@ __global__ __launch_bounds__(256) void prefill_router_kernel(const uint8_t *W, c
     }
     __syncthreads();
     if (wave != 0) return;
-    float gain[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t c = lane + 64 * j;
-        gain[j] = c < num_experts ? bf16_to_f32(per_expert_scale[c]) : 0.0f;
-    }
-    router_select(logits, gain, out_indices + (size_t)t * top_k, out_weights + (size_t)t * top_k, num_experts, top_k, lane);
+    router_select(logits, per_expert_scale, out_indices + (size_t)t * top_k, out_weights + (size_t)t * top_k, num_experts, top_k, lane);
+}
+
+// Few tokens (multi-token verification): one wave per (token, expert) logit, then one wave per token selects, so the
+// latency is that of a single row however many experts there are.
+template <int NPASS>
+__global__ __launch_bounds__(256) void prefill_logits_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B,
+                                                             const half_t *hidden, long hidden_stride, const uint16_t *eff,
+                                                             float *logits, uint32_t num_experts, int d) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t e = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const uint32_t t = blockIdx.y;
+    if (e >= num_experts) return;
+    const int groups = d >> 6;
+    const float v = router_row<0, NPASS>(W + (size_t)e * d, S + (size_t)e * groups * 2, B + (size_t)e * groups * 2,
+                                         hidden + (size_t)t * hidden_stride, eff, d, lane);
+    if (lane == 0) logits[(size_t)t * num_experts + e] = v;
+}
+
+__global__ __launch_bounds__(64) void prefill_select_kernel(const float *logits, const uint16_t *per_expert_scale,
+                                                            uint32_t *out_indices, half_t *out_weights, uint32_t num_experts,
+                                                            uint32_t top_k) {
+    const uint32_t t = blockIdx.x;
+    router_select(logits + (size_t)t * num_experts, per_expert_scale, out_indices + (size_t)t * top_k, out_weights + (size_t)t * top_k,
+                  num_experts, top_k, threadIdx.x);
 }
 
 // ------------------------------------------------------------------------------------------------ device grouping
-// One 1024-thread block.  (1) histogram of experts in LDS, (2) exclusive scan -> per-expert offsets, (3) one wave per
-// expert walks the tokens in order, 64 at a time, and places that expert's pairs by ballot + popcount (stable: sorted by
-// token, then rank), (4) the work list of <= 64-pair chunks.
-__global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *indices, const uint16_t *weights, uint32_t query_count,
-                                                           uint32_t top_k, uint32_t num_experts, tf_prefill_pair *sorted_pairs,
-                                                           uint32_t *per_expert_offsets, uint32_t *per_expert_counts,
-                                                           tf_prefill_group *chunks, uint32_t *chunk_count) {
-    __shared__ uint32_t cnt[256], start[256], chunk_start[256];
-    const uint32_t tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const uint32_t n_pairs = query_count * top_k;
-    if (tid < 256) cnt[tid] = 0;
+// A stable counting sort of the (token, rank) pairs by expert in three short launches.  The tokens are cut into at most
+// kGroupSegments segments.  (1) one wave per segment counts its pairs per expert; (2) one block turns the
+// [segment, expert] counts into start positions (expert-major, segments in order), per-expert offsets / counts and the
+// work list of <= 64-pair chunks; (3) one wave per segment places its pairs, 64 at a time in (token, rank) order, each
+// lane ranking itself among the lanes of the same expert with ballots.  Deterministic: no order depends on timing.
+__device__ __forceinline__ uint32_t clamp_expert(uint32_t e, uint32_t num_experts) { return e < num_experts ? e : num_experts - 1; }
+
+__global__ __launch_bounds__(64) void group_count_kernel(const uint32_t *indices, uint32_t n_pairs, uint32_t seg_pairs,
+                                                         uint32_t num_experts, uint32_t *seg_counts) {
+    __shared__ uint32_t cnt[256];
+    const uint32_t lane = threadIdx.x;
+    for (uint32_t e = lane; e < 256; e += 64) cnt[e] = 0;
     __syncthreads();
-    for (uint32_t i = tid; i < n_pairs; i += blockDim.x) {
-        uint32_t e = indices[i];
-        e = e < num_experts ? e : num_experts - 1;
-        atomicAdd(&cnt[e], 1u);
-    }
+    const uint32_t first = blockIdx.x * seg_pairs, last = min(first + seg_pairs, n_pairs);
+    for (uint32_t i = first + lane; i < last; i += 64) atomicAdd(&cnt[clamp_expert(indices[i], num_experts)], 1u);
     __syncthreads();
-    if (tid == 0) {
-        uint32_t run = 0, cr = 0;
-        for (uint32_t e = 0; e < num_experts; ++e) {
-            start[e] = run;
-            chunk_start[e] = cr;
-            run += cnt[e];
-            cr += (cnt[e] + kChunkPairs - 1) / kChunkPairs;
-        }
-        chunk_count[0] = cr;
-    }
-    __syncthreads();
-    if (tid < num_experts) {
-        per_expert_offsets[tid] = cnt[tid] ? start[tid] : 0xFFFFFFFFu;
-        per_expert_counts[tid] = cnt[tid];
-        const uint32_t nch = (cnt[tid] + kChunkPairs - 1) / kChunkPairs;
-        for (uint32_t c = 0; c < nch; ++c) {
-            tf_prefill_group g;
-            g.expert = tid;
-            g.pair_start = start[tid] + c * kChunkPairs;
-            g.pair_count = min(kChunkPairs, cnt[tid] - c * kChunkPairs);
-            chunks[chunk_start[tid] + c] = g;
+    for (uint32_t e = lane; e < 256; e += 64) seg_counts[blockIdx.x * 256 + e] = cnt[e];
+}
+
+// 256 threads, thread e owns expert e.  seg_counts[s][e] becomes the position of segment s's first pair of expert e.
+__global__ __launch_bounds__(256) void group_scan_kernel(uint32_t *seg_counts, uint32_t n_segments, uint32_t num_experts,
+                                                         uint32_t *per_expert_offsets, uint32_t *per_expert_counts,
+                                                         tf_prefill_group *chunks, uint32_t *chunk_count) {
+    __shared__ uint32_t scan_pairs[256], scan_chunks[256];
+    const uint32_t e = threadIdx.x;
+    uint32_t total = 0;
+    for (uint32_t s0 = 0; s0 < n_segments; s0 += 8) {
+        uint32_t v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = s0 + j < n_segments ? seg_counts[(s0 + j) * 256 + e] : 0u;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            if (s0 + j < n_segments) seg_counts[(s0 + j) * 256 + e] = total;   // exclusive prefix inside expert e
+            total += v[j];
         }
     }
-    for (uint32_t e = wave; e < num_experts; e += blockDim.x >> 6) {
-        if (cnt[e] == 0) continue;
-        uint32_t base = start[e];
-        for (uint32_t t0 = 0; t0 < query_count; t0 += 64) {
-            const uint32_t t = t0 + lane;
-            int rank = -1;
-            if (t < query_count) {
-                for (uint32_t r = 0; r < top_k; ++r) {
-                    uint32_t x = indices[(size_t)t * top_k + r];
-                    x = x < num_experts ? x : num_experts - 1;
-                    if (x == e && rank < 0) rank = (int)r;
-                }
-            }
-            const uint64_t mask = __ballot(rank >= 0);
-            if (rank >= 0) {
-                const uint32_t pos = base + __builtin_popcountll(mask & ((1ull << lane) - 1ull));
-                tf_prefill_pair p;
-                p.token = t;
-                p.expert = e;
-                p.rank = (uint32_t)rank;
-                p.weight_bits_and_reserved = (uint32_t)weights[(size_t)t * top_k + rank];
-                sorted_pairs[pos] = p;
-            }
-            base += (uint32_t)__builtin_popcountll(mask);
+    const uint32_t nch = (total + kChunkPairs - 1) / kChunkPairs;
+    scan_pairs[e] = total;
+    scan_chunks[e] = nch;
+    __syncthreads();
+    for (uint32_t step = 1; step < 256; step <<= 1) {   // inclusive scans over the experts
+        const uint32_t a = e >= step ? scan_pairs[e - step] : 0u, c = e >= step ? scan_chunks[e - step] : 0u;
+        __syncthreads();
+        scan_pairs[e] += a;
+        scan_chunks[e] += c;
+        __syncthreads();
+    }
+    const uint32_t start = scan_pairs[e] - total, chunk_start = scan_chunks[e] - nch;
+    if (e == 255) chunk_count[0] = scan_chunks[255];
+    if (e < num_experts) {
+        per_expert_offsets[e] = total ? start : 0xFFFFFFFFu;
+        per_expert_counts[e] = total;
+    }
+    for (uint32_t s = 0; s < n_segments; ++s) seg_counts[s * 256 + e] += start;   // the read-modify-writes are independent
+    for (uint32_t c = 0; c < nch; ++c) {
+        tf_prefill_group g;
+        g.expert = e;
+        g.pair_start = start + c * kChunkPairs;
+        g.pair_count = min(kChunkPairs, total - c * kChunkPairs);
+        chunks[chunk_start + c] = g;
+    }
+}
+
+__global__ __launch_bounds__(64) void group_place_kernel(const uint32_t *indices, const uint16_t *weights, uint32_t n_pairs,
+                                                         uint32_t seg_pairs, uint32_t top_k, uint32_t num_experts,
+                                                         const uint32_t *seg_starts, tf_prefill_pair *sorted_pairs) {
+    __shared__ uint32_t next[256];
+    const uint32_t lane = threadIdx.x;
+    for (uint32_t e = lane; e < 256; e += 64) next[e] = seg_starts[blockIdx.x * 256 + e];
+    __syncthreads();
+    const uint32_t first = blockIdx.x * seg_pairs, last = min(first + seg_pairs, n_pairs);
+    const uint64_t below = (1ull << lane) - 1ull;
+    for (uint32_t i0 = first; i0 < last; i0 += 64) {
+        const uint32_t i = i0 + lane;
+        const bool valid = i < last;
+        const uint32_t e = valid ? clamp_expert(indices[i], num_experts) : 0xFFFFFFFFu;
+        const uint16_t wbits = valid ? weights[i] : (uint16_t)0;
+        uint64_t remaining = __ballot(valid);
+        uint32_t pos = 0;
+        while (remaining) {   // one round per distinct expert among the 64 pairs
+            const int leader = __builtin_ctzll(remaining);
+            const uint32_t v = (uint32_t)__builtin_amdgcn_readlane((int)e, leader);
+            const uint64_t same = __ballot(e == v);
+            const uint32_t at = next[v];
+            if (e == v) pos = at + (uint32_t)__builtin_popcountll(same & below);
+            if ((int)lane == leader) next[v] = at + (uint32_t)__builtin_popcountll(same);
+            remaining &= ~same;
+        }
+        if (valid) {
+            tf_prefill_pair p;
+            p.token = i / top_k;
+            p.expert = e;
+            p.rank = i - p.token * top_k;
+            p.weight_bits_and_reserved = (uint32_t)wbits;
+            sorted_pairs[pos] = p;
         }
     }
 }
@@ -134,32 +184,28 @@ __global__ __launch_bounds__(256) void grouped_phase1_long_kernel(ExpertTable ta
                                                                   int d, int f) {
     tf_prefill_group ch;
     if (!get_chunk(cl, blockIdx.y, ch)) return;
-    const uint8_t *base = expert_base(tab, ch.expert);
+    const uint8_t *base = uniform_ptr(expert_base(tab, ch.expert));
     if (!base) return;
     const int lane = threadIdx.x & 63;
-    const int tile = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int tile = uniform_int((int)((blockIdx.x * blockDim.x + threadIdx.x) >> 6));
     const int row0 = tile * RT;
     if (row0 >= f) return;
-    const int groups = d >> 6;
-    const int rows_left = min(RT, f - row0);
-    const size_t w_byte = (size_t)row0 * (d >> 1), sb_byte = (size_t)row0 * groups * 2;
-    LongRows<RT, NP> lr;
-    typename LongRows<RT, NP>::Tile tg, tu;
-    lr.init_map(d, lane);
-    lr.load(tg, base + off.gate_W_off + w_byte, reinterpret_cast<const uint16_t *>(base + off.gate_s_off + sb_byte),
-            reinterpret_cast<const uint16_t *>(base + off.gate_b_off + sb_byte), rows_left, lane);
-    lr.load(tu, base + off.up_W_off + w_byte, reinterpret_cast<const uint16_t *>(base + off.up_s_off + sb_byte),
-            reinterpret_cast<const uint16_t *>(base + off.up_b_off + sb_byte), rows_left, lane);
+    const size_t w_byte = (size_t)row0 * (d >> 1), sb_byte = (size_t)row0 * (d >> 6) * 2;
+    RowStream<RT, NP> rs;
+    typename RowStream<RT, NP>::Tile tg, tu;
+    rs.init_map(d, lane);
+    rs.load(tg, base + off.gate_W_off + w_byte, base + off.gate_s_off + sb_byte, base + off.gate_b_off + sb_byte, f - row0);
+    rs.load(tu, base + off.up_W_off + w_byte, base + off.up_s_off + sb_byte, base + off.up_b_off + sb_byte, f - row0);
     for (uint32_t j = 0; j < ch.pair_count; ++j) {
         const uint32_t pi = ch.pair_start + j;
-        lr.init_x(hidden + (size_t)pairs[pi].token * hidden_stride, lane);
+        rs.init_x(hidden + (size_t)pairs[pi].token * hidden_stride);
         float gate[RT], up[RT];
-        lr.template reduce<SD>(tg, gate);
-        lr.template reduce<SD>(tu, up);
+        rs.template reduce<SD>(tg, gate);
+        rs.template reduce<SD>(tu, up);
         if (lane == 0) {
 #pragma unroll
             for (int r = 0; r < RT; ++r)
-                if (r < rows_left) store_act(acts, (size_t)(pi - acts_pair_base) * f + row0 + r, gate[r], up[r]);
+                if (row0 + r < f) store_act(acts, (size_t)(pi - acts_pair_base) * f + row0 + r, gate[r], up[r]);
         }
     }
 }
@@ -367,6 +413,33 @@ int32_t tf_prefill_router_gemma4_block(tf_ctx *ctx, tf_stream stream, const void
     const bool fast = aligned16(w) && aligned16(h) && aligned16(eff) && hidden_stride_elements % 8 == 0 && d <= 4096;
     const int npass = fast ? (int)((d / 16 + 63) / 64) : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (query_count <= kFewTokens) {
+        const size_t need = (size_t)kFewTokens * 256;
+        if (ctx->prefill_logits_count < need) {
+            if (ctx->prefill_logits) (void)hipFree(ctx->prefill_logits);
+            ctx->prefill_logits = nullptr;
+            ctx->prefill_logits_count = 0;
+            if (hipMalloc(&ctx->prefill_logits, need * sizeof(float)) != hipSuccess)
+                return fail(ctx, TF_ERR_OUT_OF_MEMORY, "prefill_router: cannot allocate the logits scratch");
+            ctx->prefill_logits_count = need;
+        }
+        const dim3 grid((num_experts + 3) / 4, query_count);
+#define TF_PL(NP_)                                                                                                           \
+    hipLaunchKernelGGL(prefill_logits_kernel<NP_>, grid, dim3(256), 0, st, w, s, b, h, (long)hidden_stride_elements, eff,    \
+                       ctx->prefill_logits, num_experts, (int)d)
+        switch (npass) {
+            case 1: TF_PL(1); break;
+            case 2: TF_PL(2); break;
+            case 3: TF_PL(3); break;
+            case 4: TF_PL(4); break;
+            default: TF_PL(0); break;
+        }
+#undef TF_PL
+        const int32_t rc = check_launch(ctx, "prefill_router logits");
+        if (rc != TF_OK) return rc;
+        hipLaunchKernelGGL(prefill_select_kernel, dim3(query_count), dim3(64), 0, st, ctx->prefill_logits, pes, oi, ow, num_experts, top_k);
+        return check_launch(ctx, "prefill_router select");
+    }
 #define TF_PR(NP_)                                                                                                           \
     hipLaunchKernelGGL(prefill_router_kernel<NP_>, dim3(query_count), dim3(256), 0, st, w, s, b, h, (long)hidden_stride_elements, \
                        eff, pes, oi, ow, num_experts, (int)d, top_k)
@@ -470,11 +543,19 @@ int32_t tf_prefill_group_pairs_device(tf_ctx *ctx, tf_stream stream, const void 
                "group_pairs_device: need queryCount > 0, topK > 0, 1 <= numExperts <= 256");
     TF_REQUIRE(ctx, aligned(indices, 4) && aligned(weights, 2) && aligned(sorted_pairs, 4) && aligned(chunks, 4), TF_ERR_INVALID_ARGUMENT,
                "group_pairs_device: misaligned operand");
-    hipLaunchKernelGGL(group_pairs_kernel, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const uint32_t *>(indices), static_cast<const uint16_t *>(weights), query_count, top_k, num_experts,
-                       static_cast<tf_prefill_pair *>(sorted_pairs), static_cast<uint32_t *>(per_expert_offsets),
-                       static_cast<uint32_t *>(per_expert_counts), static_cast<tf_prefill_group *>(chunks),
-                       static_cast<uint32_t *>(chunk_count));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint32_t n_pairs = query_count * top_k;
+    // whole tokens per segment, at least 32 of them, at most kGroupSegments segments
+    const uint32_t seg_tokens = std::max<uint32_t>(32u, (query_count + kGroupSegments - 1) / kGroupSegments);
+    const uint32_t n_segments = (query_count + seg_tokens - 1) / seg_tokens;
+    const uint32_t seg_pairs = seg_tokens * top_k;
+    const uint32_t *idx = static_cast<const uint32_t *>(indices);
+    hipLaunchKernelGGL(group_count_kernel, dim3(n_segments), dim3(64), 0, st, idx, n_pairs, seg_pairs, num_experts, ctx->group_scratch);
+    hipLaunchKernelGGL(group_scan_kernel, dim3(1), dim3(256), 0, st, ctx->group_scratch, n_segments, num_experts,
+                       static_cast<uint32_t *>(per_expert_offsets), static_cast<uint32_t *>(per_expert_counts),
+                       static_cast<tf_prefill_group *>(chunks), static_cast<uint32_t *>(chunk_count));
+    hipLaunchKernelGGL(group_place_kernel, dim3(n_segments), dim3(64), 0, st, idx, static_cast<const uint16_t *>(weights), n_pairs,
+                       seg_pairs, top_k, num_experts, ctx->group_scratch, static_cast<tf_prefill_pair *>(sorted_pairs));
     return check_launch(ctx, "group_pairs_device");
 }
 

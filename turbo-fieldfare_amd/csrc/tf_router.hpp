@@ -78,30 +78,36 @@ __device__ __forceinline__ float router_row(const uint8_t *w_row, const uint8_t 
 // NaN and -inf are never selected; an unfilled position reads index 0 with score -inf.
 // Lane l holds candidates l, l+64, l+128, l+192 and their gains; each round takes the wave maximum with DPP and finds
 // its lowest expert index with ballots, so a round is a few dozen ALU instructions and no memory traffic.
-__device__ __forceinline__ void router_select(const float *logits, const float gain[4], uint32_t *out_indices,
-                                              half_t *out_weights, uint32_t num_experts, uint32_t top_k, int lane) {
-    float cand[4];
+// router_select_lanes leaves selection i in lane i (i < top_k): its expert index and its routing weight.
+// NC = candidates per lane: 2 serves up to 128 experts, 4 up to 256.
+template <int NC>
+__device__ __forceinline__ void router_select_lanes(const float *logits, const uint16_t *per_expert_scale, uint32_t num_experts,
+                                                    uint32_t top_k, int lane, uint32_t &sel_index, half_t &sel_weight) {
+    float cand[NC], gain[NC];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < NC; ++j) {
         const uint32_t e = lane + 64 * j;
         const float v = e < num_experts ? logits[e] : -INFINITY;
+        gain[j] = e < num_experts ? bf16_to_f32(per_expert_scale[e]) : 0.0f;
         cand[j] = (v != v) ? -INFINITY : v;
     }
     float my_score = -INFINITY, my_gain = 0.0f;   // lane i (< top_k) ends up holding the i-th selection
     uint32_t my_idx = 0;
     for (uint32_t i = 0; i < top_k; ++i) {
-        const float m = fmaxf(fmaxf(cand[0], cand[1]), fmaxf(cand[2], cand[3]));
+        float m = cand[0];
+#pragma unroll
+        for (int j = 1; j < NC; ++j) m = fmaxf(m, cand[j]);
         const float wm = wave_max(m);
         const bool found = wm > -INFINITY;
-        int sel_j = 4, sel_lane = 0;
+        int sel_j = NC, sel_lane = 0;
 #pragma unroll
-        for (int j = 3; j >= 0; --j) {
+        for (int j = NC - 1; j >= 0; --j) {
             const uint64_t mask = __ballot(cand[j] == wm);
             if (mask) { sel_j = j; sel_lane = __builtin_ctzll(mask); }
         }
         float g = 0.0f;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int j = 0; j < NC; ++j)
             if (sel_j == j) g = read_lane(gain[j], sel_lane);
         if ((uint32_t)lane == i) {
             my_score = found ? wm : -INFINITY;
@@ -110,7 +116,7 @@ __device__ __forceinline__ void router_select(const float *logits, const float g
         }
         if (found && lane == sel_lane) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j)
+            for (int j = 0; j < NC; ++j)
                 if (sel_j == j) cand[j] = -INFINITY;
         }
     }
@@ -118,9 +124,24 @@ __device__ __forceinline__ void router_select(const float *logits, const float g
     const float ex = (uint32_t)lane < top_k ? expf(my_score - max_s) : 0.0f;
     float sum_exp = 0.0f;   // summed in selection order, like the reference
     for (uint32_t i = 0; i < top_k; ++i) sum_exp += read_lane(ex, (int)i);
+    sel_index = my_idx;
+    sel_weight = (half_t)((ex / sum_exp) * my_gain);
+}
+
+__device__ __forceinline__ void router_select_lanes(const float *logits, const uint16_t *per_expert_scale, uint32_t num_experts,
+                                                    uint32_t top_k, int lane, uint32_t &sel_index, half_t &sel_weight) {
+    if (num_experts <= 128) router_select_lanes<2>(logits, per_expert_scale, num_experts, top_k, lane, sel_index, sel_weight);
+    else router_select_lanes<4>(logits, per_expert_scale, num_experts, top_k, lane, sel_index, sel_weight);
+}
+
+__device__ __forceinline__ void router_select(const float *logits, const uint16_t *per_expert_scale, uint32_t *out_indices,
+                                              half_t *out_weights, uint32_t num_experts, uint32_t top_k, int lane) {
+    uint32_t idx;
+    half_t weight;
+    router_select_lanes(logits, per_expert_scale, num_experts, top_k, lane, idx, weight);
     if ((uint32_t)lane < top_k) {
-        out_indices[lane] = my_idx;
-        out_weights[lane] = (half_t)((ex / sum_exp) * my_gain);
+        out_indices[lane] = idx;
+        out_weights[lane] = weight;
     }
 }
 

@@ -2,7 +2,7 @@
 //
 // Three shapes of the same arithmetic  y = sum_g [ s_g * sum_k q_k x_k + b_g * sum_k x_k ]:
 //
-//   LongRows<RT, NP>  a wave owns RT consecutive rows (RT * K/2 contiguous bytes) and reads them as one flat
+//   RowStream<RT, NP> a wave owns RT consecutive rows (RT * K/2 contiguous bytes) and reads them as one flat
 //                     stream of 16-byte chunks: pass p, lane l reads chunk 64p + l, so every load instruction
 //                     of the wave covers 1024 contiguous bytes.  The chunk -> (row, column) map is the same for
 //                     every tile, so each lane keeps the activations of its <= NP column positions in registers
@@ -19,47 +19,92 @@
 
 namespace tfk {
 
-// ------------------------------------------------------------------------------------------------ long rows
+// ------------------------------------------------------------------------------------------------ row stream
+// A value that is the same in every lane, told to the compiler: arithmetic on it runs on the scalar unit.
+template <typename T>
+__device__ __forceinline__ T *uniform_ptr(T *p) {
+    const uint64_t v = (uint64_t)p;
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v);
+    const uint32_t hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return (T *)(((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ int uniform_int(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ uint32_t uniform_u32(uint32_t v) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)v); }
+
+// Every load is a bounds-checked buffer load: the tile base is wave-uniform and lives in a buffer descriptor (scalar
+// registers), each lane keeps constant byte offsets, so a tile costs no address arithmetic on the vector unit and no
+// branches.  The descriptor ends where the tile (or the matrix) ends: lanes without a chunk in the last pass and rows
+// past the end of the matrix read zeros and contribute nothing.
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+__device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+
 template <int RT, int NP>
-struct LongRows {
-    // per-lane constants
-    int row[NP];    // row within the tile served by this lane in pass p (-1: lane idle in that pass)
-    int col[NP];    // chunk column inside that row
-    int sb[NP];     // row * groups + group: index of the (scale, bias) pair inside the tile's scale block
+struct RowStream {
+    uint32_t woff[NP];   // byte offset of this lane's chunk inside the tile's weights
+    uint32_t sboff[NP];  // byte offset of its (scale, bias) inside the tile's scale / bias block
+    int row[NP];         // tile row served in pass p, -1 when idle
+    int col[NP];         // chunk column inside that row
     half2_t xq[NP][16];
     float xs[NP];
+    uint32_t row_bytes, sb_row_bytes;   // wave-uniform
 
     // chunk -> (row, column) map of this lane; independent of the data
     __device__ __forceinline__ void init_map(int k, int lane) {
         const int nch = k >> 5;  // 16-byte chunks per row
         const int groups = k >> 6;
         const int tot = RT * nch;
+        row_bytes = (uint32_t)k >> 1;
+        sb_row_bytes = (uint32_t)groups * 2u;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
             const int c = lane + 64 * p;
             const bool valid = c < tot;
-            const int cc = valid ? c : 0;
-            const int r = cc / nch;
-            col[p] = cc - r * nch;
+            const int r = c / nch;
+            const int cc = c - r * nch;
+            col[p] = valid ? cc : 0;
             row[p] = valid ? r : -1;
-            sb[p] = r * groups + (col[p] >> 1);
+            woff[p] = (uint32_t)c * 16u;                                   // past the tile when !valid: reads zeros
+            sboff[p] = valid ? (uint32_t)(r * groups + (cc >> 1)) * 2u : 0xFFFFFFF0u;
         }
     }
 
-    // activations of this lane's column positions, kept in registers; x must be 16-byte aligned
-    __device__ __forceinline__ void init_x(const half_t *x, int /*lane*/) {
+    // The activations of this lane's column positions, requested (load_x) and later arranged into registers
+    // (arrange): a caller can put other loads between the two.  x must be 16-byte aligned.
+    struct XRaw {
+        u32x4 r[NP][4];
+    };
+    __device__ __forceinline__ void load_x(XRaw &raw, const half_t *x) const {
+#pragma unroll
+        for (int p = 0; p < NP; ++p)
+#pragma unroll
+            for (int d = 0; d < 4; ++d) raw.r[p][d] = load16(x + col[p] * 32 + d * 8);
+    }
+    __device__ __forceinline__ void arrange(const XRaw &raw) {
+#pragma unroll
+        for (int p = 0; p < NP; ++p) xs[p] = arrange_x(raw.r[p], xq[p]);
+    }
+    __device__ __forceinline__ void init_x(const half_t *x) {
+        XRaw raw;
+        load_x(raw, x);
+        arrange(raw);
+    }
+
+    // The same from a block-wide LDS image written by XStage (below): xa[d * nch + c] holds word d of chunk column c
+    // already in chunk_dot order, xsum[c] the column's sum.
+    __device__ __forceinline__ void init_x_lds(const u32x4 *xa, const float *xsum, int k) {
+        const int nch = k >> 5;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
-            u32x4 xr[4];
 #pragma unroll
-            for (int d = 0; d < 4; ++d) xr[d] = load16(x + col[p] * 32 + d * 8);
-            xs[p] = arrange_x(xr, xq[p]);
+            for (int d = 0; d < 4; ++d) {
+                const u32x4 v = xa[d * nch + col[p]];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) xq[p][4 * d + j] = as_half2(v[j]);
+            }
+            xs[p] = xsum[col[p]];
         }
-    }
-
-    __device__ __forceinline__ void init(const half_t *x, int k, int lane) {
-        init_map(k, lane);
-        init_x(x, lane);
     }
 
     struct Tile {
@@ -67,32 +112,29 @@ struct LongRows {
         uint16_t s[NP], b[NP];
     };
 
-    // rows_left: rows of the matrix from the tile's first row on (>= 1); rows beyond it are not touched.
-    __device__ __forceinline__ void load(Tile &t, const uint8_t *w_tile, const uint16_t *s_tile, const uint16_t *b_tile,
-                                         int rows_left, int lane) const {
+    // w_tile / s_tile / b_tile: wave-uniform bases of the tile; rows: rows of the matrix from the tile's first row on
+    // (wave-uniform, >= 1).
+    __device__ __forceinline__ void load(Tile &t, const uint8_t *w_tile, const uint8_t *s_tile, const uint8_t *b_tile,
+                                         long rows) const {
+        const uint32_t nr = rows < RT ? (uint32_t)rows : (uint32_t)RT;
+        const rsrc_t rw = make_rsrc(w_tile, nr * row_bytes);
+        const rsrc_t rs = make_rsrc(s_tile, nr * sb_row_bytes);
+        const rsrc_t rb = make_rsrc(b_tile, nr * sb_row_bytes);
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
-            t.w[p] = u32x4{0u, 0u, 0u, 0u};
-            t.s[p] = 0;
-            t.b[p] = 0;
-            if (row[p] >= 0 && row[p] < rows_left) {
-                t.w[p] = load16(w_tile + (size_t)(lane + 64 * p) * 16);
-                t.s[p] = s_tile[sb[p]];
-                t.b[p] = b_tile[sb[p]];
-            }
+            t.w[p] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, woff[p], 0, 0));
+            t.s[p] = __builtin_amdgcn_raw_buffer_load_b16(rs, sboff[p], 0, 0);
+            t.b[p] = __builtin_amdgcn_raw_buffer_load_b16(rb, sboff[p], 0, 0);
         }
     }
 
-    // out[r]: the dot product of tile row r, wave-uniform
+    // out[r]: the dot product of tile row r, wave-uniform.  Wave-uniform control flow only (see chunk_dot).
     template <int SD>
     __device__ __forceinline__ void reduce(const Tile &t, float *out) const {
         float part[NP];
 #pragma unroll
-        for (int p = 0; p < NP; ++p) {
-            const float s = sb_to_f32<SD>(t.s[p]);
-            const float b = sb_to_f32<SD>(t.b[p]);
-            part[p] = fmaf(s, chunk_dot(t.w[p], xq[p]), b * xs[p]);   // idle lanes loaded zeros: contributes 0
-        }
+        for (int p = 0; p < NP; ++p)
+            part[p] = fmaf(sb_to_f32<SD>(t.s[p]), chunk_dot(t.w[p], xq[p]), sb_to_f32<SD>(t.b[p]) * xs[p]);
 #pragma unroll
         for (int r = 0; r < RT; ++r) {
             float v = 0.0f;
@@ -100,6 +142,52 @@ struct LongRows {
             for (int p = 0; p < NP; ++p) v += (row[p] == r) ? part[p] : 0.0f;
             out[r] = wave_sum(v);
         }
+    }
+};
+
+// Block-wide staging of an activation vector into LDS in chunk_dot order, shared by all waves of a 256-thread block:
+// request() issues the global loads (k <= 8192, x 16-byte aligned), publish() arranges them, writes the image and
+// ends with a barrier; a caller puts its weight loads between the two.  Every thread of the block must call both.
+struct XStage {
+    static constexpr int kMaxK = 8192;
+    u32x4 r[4];
+    __device__ __forceinline__ void request(const half_t *x, int k) {
+        const int pieces = k >> 3;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int piece = threadIdx.x + 256 * i;
+            r[i] = u32x4{0u, 0u, 0u, 0u};
+            if (piece < pieces) r[i] = load16(x + piece * 8);
+        }
+    }
+    __device__ __forceinline__ void publish(int k, u32x4 *xa, float *xsum) const {
+        const int pieces = k >> 3;
+        const int nch = k >> 5;
+        const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int piece = threadIdx.x + 256 * i;   // word d = piece & 3 of chunk column c = piece >> 2
+            const uint32_t p01 = r[i][0], p23 = r[i][1], p45 = r[i][2], p67 = r[i][3];
+            u32x4 o;
+            o[0] = (p01 & 0xFFFFu) | (p45 << 16);
+            o[1] = as_u32(as_half2((p01 >> 16) | (p45 & 0xFFFF0000u)) * sixteenth);
+            o[2] = (p23 & 0xFFFFu) | (p67 << 16);
+            o[3] = as_u32(as_half2((p23 >> 16) | (p67 & 0xFFFF0000u)) * sixteenth);
+            float sum = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const half2_t h = as_half2(r[i][j]);
+                sum += (float)h[0];
+                sum += (float)h[1];
+            }
+            sum += dpp_f32<0xB1>(sum);   // the four pieces of a column sit in one aligned quad of lanes
+            sum += dpp_f32<0x4E>(sum);
+            if (piece < pieces) {
+                xa[(piece & 3) * nch + (piece >> 2)] = o;
+                if ((piece & 3) == 0) xsum[piece >> 2] = sum;
+            }
+        }
+        __syncthreads();
     }
 };
 
@@ -207,7 +295,7 @@ __device__ __forceinline__ float generic_row_dot8(const uint8_t *w_row, const ui
     return wave_sum(acc);
 }
 
-// Picks the rows-per-tile and pass count of LongRows for a given K: best lane utilisation with NP <= 4.
+// Picks the rows-per-tile and pass count of RowStream for a given K: best lane utilisation with NP <= 4.
 struct LongPlan {
     int rt, np;
 };
