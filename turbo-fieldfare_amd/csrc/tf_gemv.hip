@@ -40,36 +40,47 @@ __device__ __forceinline__ void store_out(OutT *y, long row, float v) {
 }
 
 // ------------------------------------------------------------------------------------------------ GEMV kernels
-// Persistent: every wave walks tiles wave, wave + nwaves, ... of RT rows, requesting tile i+1 before reducing tile i
-// (two tile buffers used alternately, so nothing is copied).
-// FUSE_NORM: x is the raw hidden vector and the block normalises it itself (rmsnorm_bf16w with weight norm_w) into LDS.
+// Persistent: every wave walks tiles wave, wave + nwaves, ... of RT rows through two tile buffers used alternately: a
+// buffer is refilled as soon as it has been reduced, so one tile is always in flight while the other is reduced.
+// The activations are requested first, then the first two tiles, and are staged in LDS (in chunk order, once per block)
+// while the tiles are in flight.  FUSE_NORM: x is the raw hidden vector and the block normalises it on the way
+// (rmsnorm_bf16w with weight norm_w).  k <= XStage::kMaxK.
 template <int RT, int NP, int SD, typename OutT, bool FUSE_NORM>
 __global__ __launch_bounds__(256, 4) void gemv4_long_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B,
                                                             const half_t *x, const uint16_t *norm_w, float eps, OutT *y,
                                                             long m, int k) {
+    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
+    __shared__ float xsum[XStage::kMaxK / 32];
+    __shared__ float partial[4];
     const int lane = threadIdx.x & 63;
     const long wave = uniform_int((int)(((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6));
     const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
     const long ntiles = (m + RT - 1) / RT;
-    const bool active = wave < ntiles;
     const size_t tile_bytes = (size_t)RT * (k >> 1);
     const size_t sb_bytes = (size_t)RT * (k >> 6) * 2;
 
     RowStream<RT, NP> rs;
     typename RowStream<RT, NP>::Tile ta, tb;
     rs.init_map(k, lane);
-    long tile = wave;
-    // the first tile does not depend on the activations: request it before anything else
-    if (active) rs.load(ta, W + tile * tile_bytes, S + tile * sb_bytes, B + tile * sb_bytes, m - tile * RT);
+    auto request = [&](typename RowStream<RT, NP>::Tile &t, long at) {
+        rs.load(t, W + at * tile_bytes, S + at * sb_bytes, B + at * sb_bytes, m - at * RT);
+    };
+    long t0 = wave, t1 = wave + nwaves;
     if constexpr (FUSE_NORM) {
-        __shared__ __align__(16) half_t xn_lds[kMaxFusedNormD];
-        __shared__ float partial[4];
-        block_rmsnorm_to_lds(x, norm_w, eps, k, xn_lds, partial);
-        if (active) rs.init_x(xn_lds);
+        XNormStage stage;
+        stage.request(x, norm_w, k);
+        if (t0 < ntiles) request(ta, t0);
+        if (t1 < ntiles) request(tb, t1);
+        stage.publish(eps, k, xa, xsum, partial);
     } else {
-        if (active) rs.init_x(x);
+        XStage stage;
+        stage.request(x, k);
+        if (t0 < ntiles) request(ta, t0);
+        if (t1 < ntiles) request(tb, t1);
+        stage.publish(k, xa, xsum);
     }
-    if (!active) return;
+    if (t0 >= ntiles) return;
+    rs.init_x_lds(xa, xsum, k);
     auto emit = [&](const typename RowStream<RT, NP>::Tile &t, long at) {
         float out[RT];
         rs.template reduce<SD>(t, out);
@@ -80,16 +91,14 @@ __global__ __launch_bounds__(256, 4) void gemv4_long_kernel(const uint8_t *W, co
         }
     };
     for (;;) {
-        long next = tile + nwaves;
-        if (next < ntiles) rs.load(tb, W + next * tile_bytes, S + next * sb_bytes, B + next * sb_bytes, m - next * RT);
-        emit(ta, tile);
-        if (next >= ntiles) break;
-        tile = next;
-        next = tile + nwaves;
-        if (next < ntiles) rs.load(ta, W + next * tile_bytes, S + next * sb_bytes, B + next * sb_bytes, m - next * RT);
-        emit(tb, tile);
-        if (next >= ntiles) break;
-        tile = next;
+        emit(ta, t0);
+        t0 += 2 * nwaves;
+        if (t0 < ntiles) request(ta, t0);
+        if (t1 >= ntiles) break;
+        emit(tb, t1);
+        t1 += 2 * nwaves;
+        if (t1 < ntiles) request(tb, t1);
+        if (t0 >= ntiles) break;
     }
 }
 

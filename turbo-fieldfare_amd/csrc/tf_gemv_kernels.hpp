@@ -24,54 +24,8 @@ __device__ __forceinline__ float block_rms_inv(const half_t *x, uint32_t d, floa
     return 1.0f / sqrtf(total / (float)d + eps);
 }
 
-// rmsnorm_bf16w computed by one 256-thread block straight into LDS: xn[i] = half(x[i] * inv * w[i]).
-// k % 8 == 0, k <= 8192, x and w 16-byte aligned.  Every thread requests its (at most four) 8-element chunks of both
-// operands before using any.  Ends with a barrier: xn is readable by the whole block on return.
-constexpr int kMaxFusedNormD = 8192;
-__device__ __forceinline__ void block_rmsnorm_to_lds(const half_t *x, const uint16_t *w_bf16, float eps, int k, half_t *xn,
-                                                     float *partial) {
-    const int nchunks = k >> 3;
-    u32x4 xr[4], wr[4];
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const int c = threadIdx.x + 256 * p;
-        xr[p] = wr[p] = u32x4{0u, 0u, 0u, 0u};
-        if (c < nchunks) {
-            xr[p] = load16(x + c * 8);
-            wr[p] = load16(w_bf16 + c * 8);
-        }
-    }
-    float acc = 0.0f;
-#pragma unroll
-    for (int p = 0; p < 4; ++p)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const half2_t h = as_half2(xr[p][j]);
-            acc = fmaf((float)h[0], (float)h[0], acc);
-            acc = fmaf((float)h[1], (float)h[1], acc);
-        }
-    acc = wave_sum(acc);
-    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = acc;
-    __syncthreads();
-    const float inv = 1.0f / sqrtf((partial[0] + partial[1] + partial[2] + partial[3]) / (float)k + eps);
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const int c = threadIdx.x + 256 * p;
-        if (c < nchunks) {
-            u32x4 o;
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const half2_t h = as_half2(xr[p][j]);
-                half2_t n;
-                n[0] = (half_t)((float)h[0] * inv * __uint_as_float(wr[p][j] << 16));
-                n[1] = (half_t)((float)h[1] * inv * __uint_as_float(wr[p][j] & 0xFFFF0000u));
-                o[j] = as_u32(n);
-            }
-            *reinterpret_cast<u32x4 *>(xn + c * 8) = o;
-        }
-    }
-    __syncthreads();
-}
+// largest hidden size the row streamers normalise and stage themselves (XNormStage)
+constexpr int kMaxFusedNormD = XStage::kMaxK;
 
 int32_t launch_gemv4(tf_ctx *ctx, hipStream_t st, const uint8_t *w, const uint8_t *s, const uint8_t *b, const void *x,
                      void *y, uint32_t m, uint32_t n, tf_dtype sd, tf_dtype od, const void *norm_w = nullptr, float eps = 0.0f);

@@ -40,28 +40,38 @@ __global__ __launch_bounds__(256, 4) void head_greedy_long_kernel(const uint8_t 
                                                                int k) {
     __shared__ float sv[4];
     __shared__ uint32_t si[4];
+    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
+    __shared__ float xsum[XStage::kMaxK / 32];
+    __shared__ float partial[4];
     const int lane = threadIdx.x & 63;
     const int wib = threadIdx.x >> 6;
     const long wave = uniform_int((int)(((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6));
     const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
     const long ntiles = (v_rows + RT - 1) / RT;
     Best best{-INFINITY, 0xFFFFFFFFu};
-    const bool active = wave < ntiles;
     const size_t tile_bytes = (size_t)RT * (k >> 1);
     const size_t sb_bytes = (size_t)RT * (k >> 6) * 2;
     RowStream<RT, NP> rs;
     typename RowStream<RT, NP>::Tile ta, tb;
     rs.init_map(k, lane);
-    long tile = wave;
-    // the first tile does not depend on the activations: request it before normalising them
-    if (active) rs.load(ta, W + tile * tile_bytes, S + tile * sb_bytes, B + tile * sb_bytes, v_rows - tile * RT);
+    auto request = [&](typename RowStream<RT, NP>::Tile &t, long at) {
+        rs.load(t, W + at * tile_bytes, S + at * sb_bytes, B + at * sb_bytes, v_rows - at * RT);
+    };
+    // requests in this order: the activations, then the first two tiles; the activations are normalised and staged in
+    // LDS while the tiles are in flight
+    long t0 = wave, t1 = wave + nwaves;
     if constexpr (FUSE_NORM) {
-        __shared__ __align__(16) half_t xn_lds[kMaxFusedNormD];
-        __shared__ float partial[4];
-        block_rmsnorm_to_lds(x, norm_w, eps, k, xn_lds, partial);
-        if (active) rs.init_x(xn_lds);
+        XNormStage stage;
+        stage.request(x, norm_w, k);
+        if (t0 < ntiles) request(ta, t0);
+        if (t1 < ntiles) request(tb, t1);
+        stage.publish(eps, k, xa, xsum, partial);
     } else {
-        if (active) rs.init_x(x);
+        XStage stage;
+        stage.request(x, k);
+        if (t0 < ntiles) request(ta, t0);
+        if (t1 < ntiles) request(tb, t1);
+        stage.publish(k, xa, xsum);
     }
     // rows ascend within a wave, so a strict comparison keeps the lowest index among equals
     auto consider = [&](const typename RowStream<RT, NP>::Tile &t, long at) {
@@ -77,18 +87,17 @@ __global__ __launch_bounds__(256, 4) void head_greedy_long_kernel(const uint8_t 
             }
         }
     };
-    if (active) {
+    if (t0 < ntiles) {
+        rs.init_x_lds(xa, xsum, k);
         for (;;) {
-            long next = tile + nwaves;
-            if (next < ntiles) rs.load(tb, W + next * tile_bytes, S + next * sb_bytes, B + next * sb_bytes, v_rows - next * RT);
-            consider(ta, tile);
-            if (next >= ntiles) break;
-            tile = next;
-            next = tile + nwaves;
-            if (next < ntiles) rs.load(ta, W + next * tile_bytes, S + next * sb_bytes, B + next * sb_bytes, v_rows - next * RT);
-            consider(tb, tile);
-            if (next >= ntiles) break;
-            tile = next;
+            consider(ta, t0);
+            t0 += 2 * nwaves;
+            if (t0 < ntiles) request(ta, t0);
+            if (t1 >= ntiles) break;
+            consider(tb, t1);
+            t1 += 2 * nwaves;
+            if (t1 < ntiles) request(tb, t1);
+            if (t0 >= ntiles) break;
         }
     }
     if (lane == 0) { sv[wib] = best.v; si[wib] = best.idx; }

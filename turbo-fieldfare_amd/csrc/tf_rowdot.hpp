@@ -148,9 +148,12 @@ struct RowStream {
 // Block-wide staging of an activation vector into LDS in chunk_dot order, shared by all waves of a 256-thread block:
 // request() issues the global loads (k <= 8192, x 16-byte aligned), publish() arranges them, writes the image and
 // ends with a barrier; a caller puts its weight loads between the two.  Every thread of the block must call both.
+// With a norm weight (request_norm / publish_norm) the vector is first normalised as rmsnorm_bf16w does:
+// half(x * rsqrt(mean(x^2) + eps) * w).
 struct XStage {
     static constexpr int kMaxK = 8192;
     u32x4 r[4];
+
     __device__ __forceinline__ void request(const half_t *x, int k) {
         const int pieces = k >> 3;
 #pragma unroll
@@ -160,32 +163,81 @@ struct XStage {
             if (piece < pieces) r[i] = load16(x + piece * 8);
         }
     }
-    __device__ __forceinline__ void publish(int k, u32x4 *xa, float *xsum) const {
-        const int pieces = k >> 3;
-        const int nch = k >> 5;
+
+    // piece = 8 consecutive activations = word (piece & 3) of chunk column (piece >> 2)
+    static __device__ __forceinline__ void publish_piece(const u32x4 raw, int piece, int pieces, int nch, u32x4 *xa, float *xsum) {
         const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
+        const uint32_t p01 = raw[0], p23 = raw[1], p45 = raw[2], p67 = raw[3];
+        u32x4 o;
+        o[0] = (p01 & 0xFFFFu) | (p45 << 16);
+        o[1] = as_u32(as_half2((p01 >> 16) | (p45 & 0xFFFF0000u)) * sixteenth);
+        o[2] = (p23 & 0xFFFFu) | (p67 << 16);
+        o[3] = as_u32(as_half2((p23 >> 16) | (p67 & 0xFFFF0000u)) * sixteenth);
+        float sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const half2_t h = as_half2(raw[j]);
+            sum += (float)h[0];
+            sum += (float)h[1];
+        }
+        sum += dpp_f32<0xB1>(sum);   // the four pieces of a column sit in one aligned quad of lanes
+        sum += dpp_f32<0x4E>(sum);
+        if (piece < pieces) {
+            xa[(piece & 3) * nch + (piece >> 2)] = o;
+            if ((piece & 3) == 0) xsum[piece >> 2] = sum;
+        }
+    }
+
+    __device__ __forceinline__ void publish(int k, u32x4 *xa, float *xsum) const {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) publish_piece(r[i], threadIdx.x + 256 * i, k >> 3, k >> 5, xa, xsum);
+        __syncthreads();
+    }
+};
+
+struct XNormStage {
+    u32x4 xr[4], wr[4];
+
+    __device__ __forceinline__ void request(const half_t *x, const uint16_t *w_bf16, int k) {
+        const int pieces = k >> 3;
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int piece = threadIdx.x + 256 * i;   // word d = piece & 3 of chunk column c = piece >> 2
-            const uint32_t p01 = r[i][0], p23 = r[i][1], p45 = r[i][2], p67 = r[i][3];
-            u32x4 o;
-            o[0] = (p01 & 0xFFFFu) | (p45 << 16);
-            o[1] = as_u32(as_half2((p01 >> 16) | (p45 & 0xFFFF0000u)) * sixteenth);
-            o[2] = (p23 & 0xFFFFu) | (p67 << 16);
-            o[3] = as_u32(as_half2((p23 >> 16) | (p67 & 0xFFFF0000u)) * sixteenth);
-            float sum = 0.0f;
+            const int piece = threadIdx.x + 256 * i;
+            xr[i] = wr[i] = u32x4{0u, 0u, 0u, 0u};
+            if (piece < pieces) {
+                xr[i] = load16(x + piece * 8);
+                wr[i] = load16(w_bf16 + piece * 8);
+            }
+        }
+    }
+
+    // partial: 4 floats of LDS
+    __device__ __forceinline__ void publish(float eps, int k, u32x4 *xa, float *xsum, float *partial) const {
+        float acc = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const half2_t h = as_half2(r[i][j]);
-                sum += (float)h[0];
-                sum += (float)h[1];
+                const half2_t h = as_half2(xr[i][j]);
+                acc = fmaf((float)h[0], (float)h[0], acc);
+                acc = fmaf((float)h[1], (float)h[1], acc);
             }
-            sum += dpp_f32<0xB1>(sum);   // the four pieces of a column sit in one aligned quad of lanes
-            sum += dpp_f32<0x4E>(sum);
-            if (piece < pieces) {
-                xa[(piece & 3) * nch + (piece >> 2)] = o;
-                if ((piece & 3) == 0) xsum[piece >> 2] = sum;
+        acc = wave_sum(acc);
+        if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = acc;
+        __syncthreads();
+        const float inv = 1.0f / sqrtf((partial[0] + partial[1] + partial[2] + partial[3]) / (float)k + eps);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            u32x4 o;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const half2_t h = as_half2(xr[i][j]);
+                half2_t n;
+                n[0] = (half_t)((float)h[0] * inv * __uint_as_float(wr[i][j] << 16));
+                n[1] = (half_t)((float)h[1] * inv * __uint_as_float(wr[i][j] & 0xFFFF0000u));
+                o[j] = as_u32(n);
             }
+            XStage::publish_piece(o, threadIdx.x + 256 * i, k >> 3, k >> 5, xa, xsum);
         }
         __syncthreads();
     }
