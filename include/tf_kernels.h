@@ -316,8 +316,8 @@ int32_t tf_prefill_group_token_expert_pairs(const tf_prefill_pair *pairs, uint64
                                             tf_prefill_tile *tiles, uint32_t *tile_count);
 /* The same grouping (no sort keys) done on the DEVICE straight from the router's outputs, so a resident-expert pipeline
  * needs no host round trip: sorted_pairs[T*top_k] ordered by (expert, token, rank), per_expert_offsets / per_expert_counts
- * [num_experts], and a work list `chunks` (runs of <= 64 sorted pairs sharing one expert) with its length in chunk_count[0].
- * chunks capacity: num_experts + T*top_k/64 entries.  Expert ids are clamped to num_experts - 1
+ * [num_experts], and a work list `chunks` (runs of <= 128 sorted pairs sharing one expert) with its length in chunk_count[0].
+ * chunks capacity: num_experts + T*top_k/128 entries.  Expert ids are clamped to num_experts - 1
  * (RealForwardRunner.swift:955); the experts of one token must be distinct (the router guarantees it). */
 int32_t tf_prefill_group_pairs_device(tf_ctx *ctx, tf_stream stream, const void *indices, const void *weights,
                                       uint32_t query_count, uint32_t top_k, uint32_t num_experts,

@@ -110,7 +110,7 @@ def test_device_grouping_equals_host_grouping(T, top_k, E):
     chunks = host(g["chunks"], np.uint32, nch * 3).reshape(nch, 3)
     covered = []
     for e, s, c in chunks:
-        assert 1 <= c <= 64 and all(int(x) == int(e) for x in got[s:s + c, 1])
+        assert 1 <= c <= 128 and all(int(x) == int(e) for x in got[s:s + c, 1])
         covered.extend(range(int(s), int(s + c)))
     assert covered == list(range(T * top_k)) and nch <= g["cap"]
 

@@ -74,7 +74,7 @@ __global__ __launch_bounds__(64) void prefill_select_kernel(const float *logits,
 // A stable counting sort of the (token, rank) pairs by expert in three short launches.  The tokens are cut into at most
 // kGroupSegments segments.  (1) one wave per segment counts its pairs per expert; (2) one block turns the
 // [segment, expert] counts into start positions (expert-major, segments in order), per-expert offsets / counts and the
-// work list of <= 64-pair chunks; (3) one wave per segment places its pairs, 64 at a time in (token, rank) order, each
+// work list of <= 128-pair chunks; (3) one wave per segment places its pairs, 64 at a time in (token, rank) order, each
 // lane ranking itself among the lanes of the same expert with ballots.  Deterministic: no order depends on timing.
 __device__ __forceinline__ uint32_t clamp_expert(uint32_t e, uint32_t num_experts) { return e < num_experts ? e : num_experts - 1; }
 

@@ -30,7 +30,7 @@ __device__ __forceinline__ const uint8_t *expert_base(const ExpertTable &t, uint
 
 // Work list: runs of sorted pairs that share one expert, each at most kChunkPairs long.  Either a short list passed with
 // the kernel arguments or a device array written by the grouping kernel (with its length in device memory).
-constexpr uint32_t kChunkPairs = 64;
+constexpr uint32_t kChunkPairs = 128;
 constexpr uint32_t kInlineChunks = 48;
 struct ChunkList {
     uint32_t n;

@@ -6,218 +6,151 @@ using namespace tfk;
 
 namespace {
 
+// The lane's weight rows for the wave's two column tiles: tile j covers rows row0[j] + (lane & 31) of a matrix that
+// starts at w / s / b and has `limit[j]` rows.
+__device__ __forceinline__ QmmBRows make_b_rows(const uint8_t *const w[2], const uint8_t *const s[2], const uint8_t *const b[2],
+                                                const int row0[2], const int limit[2], int row_bytes, int groups, int lane) {
+    QmmBRows rows;
+    const int i = lane & 31, kb = lane >> 5;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int n = min(row0[j] + i, limit[j] - 1);
+        rows.w[j] = w[j] + (size_t)n * row_bytes + kb * 16;
+        rows.s[j] = s[j] + (size_t)n * groups * 2;
+        rows.b[j] = b[j] + (size_t)n * groups * 2;
+    }
+    return rows;
+}
+
+__device__ __forceinline__ void zero_acc(float16_t acc[4][2]) {
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[mt][j][r] = 0.0f;
+}
+
 // ------------------------------------------------------------------------------------------------ dense
 template <int SD>
-__global__ __launch_bounds__(256) void qmm_dense_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *X,
-                                                        long ldx, half_t *Y, long ldy, int M, int N, int K) {
-    __shared__ __align__(16) QmmSmem sm;
+__global__ __launch_bounds__(256, 2) void qmm_dense_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *X,
+                                                           long ldx, half_t *Y, long ldy, int M, int N, int K) {
+    __shared__ __align__(16) u32x4 lds[2 * kQmmBM * 8];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n0 = blockIdx.x * kQmmBN, m0 = blockIdx.y * kQmmBM;
-    const int groups = K >> 6, row_bytes = K >> 1, kt_count = K >> 6;
-    const half_t *arow[2];
+    const int n0 = blockIdx.x * kQmmBN + wave * kQmmWaveN, m0 = blockIdx.y * kQmmBM;
+    const half_t *arow[kQmmAChunks];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const int r = (threadIdx.x + 256 * i) >> 3;
-        arow[i] = (m0 + r < M) ? X + (size_t)(m0 + r) * ldx : nullptr;
+    for (int q = 0; q < kQmmAChunks; ++q) {
+        const int r = (threadIdx.x + 256 * q) >> 3;
+        arow[q] = X + (size_t)min(m0 + r, M - 1) * ldx;
     }
-    const int n_left = min(kQmmBN, N - n0);
-    const uint8_t *w_rows = W + (size_t)n0 * row_bytes;
-    const uint8_t *s_rows = S + (size_t)n0 * groups * 2;
-    const uint8_t *b_rows = B + (size_t)n0 * groups * 2;
-
-    AStage ast;
-    WStage wst;
-    a_stage_load(ast, arow, 0);
-    w_stage_load(wst, w_rows, s_rows, b_rows, n_left, row_bytes, groups, 0);
-    a_stage_store(ast, sm.a[0]);
-    w_stage_store<SD>(wst, sm.b[0]);
-    __syncthreads();
-    float16_t acc[2];
+    const uint8_t *w[2] = {W, W}, *s[2] = {S, S}, *b[2] = {B, B};
+    const int row0[2] = {n0, n0 + 32}, limit[2] = {N, N};
+    const QmmBRows rows = make_b_rows(w, s, b, row0, limit, K >> 1, K >> 6, lane);
+    const int row_tiles = min(4, (M - m0 + 31) >> 5);
+    float16_t acc[4][2];
+    zero_acc(acc);
+    qmm_k_loop<SD>(K >> 6, arow, rows, lds, lane, row_tiles, acc);
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+    for (int j = 0; j < 2; ++j) {
+        const int n = n0 + j * 32 + acc_col(lane);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) acc[mb][r] = 0.0f;
-    for (int kt = 0; kt < kt_count; ++kt) {
-        const bool more = kt + 1 < kt_count;
-        if (more) {
-            a_stage_load(ast, arow, kt + 1);
-            w_stage_load(wst, w_rows, s_rows, b_rows, n_left, row_bytes, groups, kt + 1);
-        }
-        mfma_group(sm.a[kt & 1], sm.b[kt & 1], wave, lane, acc);
-        if (more) {
-            a_stage_store(ast, sm.a[(kt + 1) & 1]);
-            w_stage_store<SD>(wst, sm.b[(kt + 1) & 1]);
-        }
-        __syncthreads();
+        for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int m = m0 + mt * 32 + acc_row(r, lane);
+                if (m < M && n < N) Y[(size_t)m * ldy + n] = (half_t)acc[mt][j][r];
+            }
     }
-    const int n = n0 + wave * 32 + acc_col(lane);
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int m = m0 + mb * 32 + acc_row(r, lane);
-            if (m < M && n < N) Y[(size_t)m * ldy + n] = (half_t)acc[mb][r];
-        }
 }
 
 // ------------------------------------------------------------------------------------------------ grouped phase 1
-// Block = one chunk (<= 64 sorted pairs of one expert) x 64 intermediate columns.  Wave w owns rows (w/2)*32.. and columns
-// (w%2)*32.. for BOTH the gate and the up matrix, so GeGLU is applied to the fp32 accumulators in registers.
-constexpr int kP1BN = 64;
+// Block = one chunk (<= 128 sorted pairs of one expert) x 128 intermediate columns.  A wave's first column tile is 32
+// rows of the gate matrix, its second the same 32 rows of the up matrix, so GeGLU is applied to the fp32 accumulators
+// in registers.
+constexpr int kP1BN = 128;
 
 template <int SD>
-__global__ __launch_bounds__(256) void grouped_phase1_mfma_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl,
-                                                                  const tf_prefill_pair *pairs, const half_t *hidden,
-                                                                  long hidden_stride, half_t *acts, uint32_t acts_pair_base,
-                                                                  int D, int F) {
-    __shared__ __align__(16) half_t sa[2][kQmmBM * kQmmLDK];
-    __shared__ __align__(16) half_t sb[2][2][kP1BN * kQmmLDK];
+__global__ __launch_bounds__(256, 2) void grouped_phase1_mfma_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl,
+                                                                     const tf_prefill_pair *pairs, const half_t *hidden,
+                                                                     long hidden_stride, half_t *acts, uint32_t acts_pair_base,
+                                                                     int D, int F) {
+    __shared__ __align__(16) u32x4 lds[2 * kQmmBM * 8];
     tf_prefill_group ch;
     if (!get_chunk(cl, blockIdx.y, ch)) return;
     const uint8_t *base = expert_base(tab, ch.expert);
     if (!base) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n0 = blockIdx.x * kP1BN;
-    const int groups = D >> 6, row_bytes = D >> 1, kt_count = D >> 6;
-    const half_t *arow[2];
+    const int n0 = blockIdx.x * kP1BN + wave * 32;
+    const half_t *arow[kQmmAChunks];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const uint32_t r = (threadIdx.x + 256 * i) >> 3;
-        arow[i] = r < ch.pair_count ? hidden + (size_t)pairs[ch.pair_start + r].token * hidden_stride : nullptr;
+    for (int q = 0; q < kQmmAChunks; ++q) {
+        const uint32_t r = (threadIdx.x + 256 * q) >> 3;
+        arow[q] = hidden + (size_t)pairs[ch.pair_start + min(r, ch.pair_count - 1)].token * hidden_stride;
     }
-    // 64 rows x 32 bytes per matrix and K step = 128 16-byte chunks: threads 0..127 stage gate, 128..255 stage up
-    const int which = threadIdx.x >> 7, tt = threadIdx.x & 127;
-    const int wr = tt >> 1, hc = tt & 1;
-    const int n_left = min(kP1BN, F - n0);
-    const uint32_t w_off = which ? off.up_W_off : off.gate_W_off;
-    const uint32_t s_off = which ? off.up_s_off : off.gate_s_off;
-    const uint32_t b_off = which ? off.up_b_off : off.gate_b_off;
-    const uint8_t *w_row = base + w_off + (size_t)(n0 + wr) * row_bytes + hc * 16;
-    const uint8_t *s_row = base + s_off + (size_t)(n0 + wr) * groups * 2;
-    const uint8_t *b_row = base + b_off + (size_t)(n0 + wr) * groups * 2;
-    const bool w_valid = wr < n_left;
-
-    AStage ast;
-    WStage wst;
-    auto load_w = [&](int kt) {
-        wst.w = u32x4{0u, 0u, 0u, 0u};
-        wst.s = 0;
-        wst.b = 0;
-        if (w_valid) {
-            wst.w = load16(w_row + kt * 32);
-            wst.s = *reinterpret_cast<const uint16_t *>(s_row + kt * 2);
-            wst.b = *reinterpret_cast<const uint16_t *>(b_row + kt * 2);
-        }
-    };
-    auto store_w = [&](int buf) {
-        const half2_t s2 = sb_to_half2<SD>(wst.s), b2 = sb_to_half2<SD>(wst.b);
-        half_t *dst = sb[buf][which] + wr * kQmmLDK + hc * 32;
+    const uint8_t *w[2] = {base + off.gate_W_off, base + off.up_W_off};
+    const uint8_t *s[2] = {base + off.gate_s_off, base + off.up_s_off};
+    const uint8_t *b[2] = {base + off.gate_b_off, base + off.up_b_off};
+    const int row0[2] = {n0, n0}, limit[2] = {F, F};
+    const QmmBRows rows = make_b_rows(w, s, b, row0, limit, D >> 1, D >> 6, lane);
+    const int row_tiles = (int)((ch.pair_count + 31) >> 5);
+    float16_t acc[4][2];
+    zero_acc(acc);
+    qmm_k_loop<SD>(D >> 6, arow, rows, lds, lane, row_tiles, acc);
+    const int n = n0 + acc_col(lane);
 #pragma unroll
-        for (int d = 0; d < 4; ++d) *reinterpret_cast<u32x4 *>(dst + d * 8) = dequant_word(wst.w[d], s2, b2);
-    };
-    a_stage_load(ast, arow, 0);
-    load_w(0);
-    a_stage_store(ast, sa[0]);
-    store_w(0);
-    __syncthreads();
-    float16_t ag, au;
+    for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) { ag[r] = 0.0f; au[r] = 0.0f; }
-    const int mb = wave >> 1, nb = wave & 1;
-    const int i = lane & 31, kb = lane >> 5;
-    for (int kt = 0; kt < kt_count; ++kt) {
-        const bool more = kt + 1 < kt_count;
-        if (more) {
-            a_stage_load(ast, arow, kt + 1);
-            load_w(kt + 1);
+        for (int r = 0; r < 16; ++r) {
+            const uint32_t m = mt * 32 + acc_row(r, lane);
+            if (m < ch.pair_count && n < F)
+                acts[(size_t)(ch.pair_start + m - acts_pair_base) * F + n] = (half_t)(gelu_tanh(acc[mt][0][r]) * acc[mt][1][r]);
         }
-        const half_t *as = sa[kt & 1] + (mb * 32 + i) * kQmmLDK + kb * 8;
-        const half_t *gs = sb[kt & 1][0] + (nb * 32 + i) * kQmmLDK + kb * 8;
-        const half_t *us = sb[kt & 1][1] + (nb * 32 + i) * kQmmLDK + kb * 8;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-            const half8_t af = *reinterpret_cast<const half8_t *>(as + ks * 16);
-            const half8_t gf = *reinterpret_cast<const half8_t *>(gs + ks * 16);
-            const half8_t uf = *reinterpret_cast<const half8_t *>(us + ks * 16);
-            ag = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, gf, ag, 0, 0, 0);
-            au = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, uf, au, 0, 0, 0);
-        }
-        if (more) {
-            a_stage_store(ast, sa[(kt + 1) & 1]);
-            store_w((kt + 1) & 1);
-        }
-        __syncthreads();
-    }
-    const int n = n0 + nb * 32 + acc_col(lane);
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const uint32_t m = mb * 32 + acc_row(r, lane);
-        if (m < ch.pair_count && n < F)
-            acts[(size_t)(ch.pair_start + m - acts_pair_base) * F + n] = (half_t)(gelu_tanh(ag[r]) * au[r]);
-    }
 }
 
 // ------------------------------------------------------------------------------------------------ grouped down
-// Block = one chunk x 128 output columns: A rows are the chunk's activation rows, C rows scatter to
+// Block = one chunk x 256 output columns: X rows are the chunk's activation rows, Y rows scatter to
 // route_partials[(token * top_k + rank) * D + c].
 template <int SD>
-__global__ __launch_bounds__(256) void grouped_down_mfma_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl,
-                                                                const tf_prefill_pair *pairs, const half_t *acts,
-                                                                uint32_t acts_pair_base, half_t *route_partials, int D, int F,
-                                                                int top_k) {
-    __shared__ __align__(16) QmmSmem sm;
+__global__ __launch_bounds__(256, 2) void grouped_down_mfma_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl,
+                                                                   const tf_prefill_pair *pairs, const half_t *acts,
+                                                                   uint32_t acts_pair_base, half_t *route_partials, int D, int F,
+                                                                   int top_k) {
+    __shared__ __align__(16) u32x4 lds[2 * kQmmBM * 8];
     tf_prefill_group ch;
     if (!get_chunk(cl, blockIdx.y, ch)) return;
     const uint8_t *base = expert_base(tab, ch.expert);
     if (!base) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n0 = blockIdx.x * kQmmBN;
-    const int groups = F >> 6, row_bytes = F >> 1, kt_count = F >> 6;
-    const half_t *arow[2];
+    const int n0 = blockIdx.x * kQmmBN + wave * kQmmWaveN;
+    const half_t *arow[kQmmAChunks];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-        const uint32_t r = (threadIdx.x + 256 * i) >> 3;
-        arow[i] = r < ch.pair_count ? acts + (size_t)(ch.pair_start + r - acts_pair_base) * F : nullptr;
+    for (int q = 0; q < kQmmAChunks; ++q) {
+        const uint32_t r = (threadIdx.x + 256 * q) >> 3;
+        arow[q] = acts + (size_t)(ch.pair_start + min(r, ch.pair_count - 1) - acts_pair_base) * F;
     }
-    const int n_left = min(kQmmBN, D - n0);
-    const uint8_t *w_rows = base + off.down_W_off + (size_t)n0 * row_bytes;
-    const uint8_t *s_rows = base + off.down_s_off + (size_t)n0 * groups * 2;
-    const uint8_t *b_rows = base + off.down_b_off + (size_t)n0 * groups * 2;
-
-    AStage ast;
-    WStage wst;
-    a_stage_load(ast, arow, 0);
-    w_stage_load(wst, w_rows, s_rows, b_rows, n_left, row_bytes, groups, 0);
-    a_stage_store(ast, sm.a[0]);
-    w_stage_store<SD>(wst, sm.b[0]);
-    __syncthreads();
-    float16_t acc[2];
+    const uint8_t *w[2] = {base + off.down_W_off, base + off.down_W_off};
+    const uint8_t *s[2] = {base + off.down_s_off, base + off.down_s_off};
+    const uint8_t *b[2] = {base + off.down_b_off, base + off.down_b_off};
+    const int row0[2] = {n0, n0 + 32}, limit[2] = {D, D};
+    const QmmBRows rows = make_b_rows(w, s, b, row0, limit, F >> 1, F >> 6, lane);
+    const int row_tiles = (int)((ch.pair_count + 31) >> 5);
+    float16_t acc[4][2];
+    zero_acc(acc);
+    qmm_k_loop<SD>(F >> 6, arow, rows, lds, lane, row_tiles, acc);
 #pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[mb][r] = 0.0f;
-    for (int kt = 0; kt < kt_count; ++kt) {
-        const bool more = kt + 1 < kt_count;
-        if (more) {
-            a_stage_load(ast, arow, kt + 1);
-            w_stage_load(wst, w_rows, s_rows, b_rows, n_left, row_bytes, groups, kt + 1);
-        }
-        mfma_group(sm.a[kt & 1], sm.b[kt & 1], wave, lane, acc);
-        if (more) {
-            a_stage_store(ast, sm.a[(kt + 1) & 1]);
-            w_stage_store<SD>(wst, sm.b[(kt + 1) & 1]);
-        }
-        __syncthreads();
-    }
-    const int n = n0 + wave * 32 + acc_col(lane);
-#pragma unroll
-    for (int mb = 0; mb < 2; ++mb)
+    for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const uint32_t m = mb * 32 + acc_row(r, lane);
-            if (m < ch.pair_count && n < D) {
+            const uint32_t m = mt * 32 + acc_row(r, lane);
+            if (m < ch.pair_count) {
                 const tf_prefill_pair p = pairs[ch.pair_start + m];
-                route_partials[((size_t)p.token * top_k + p.rank) * D + n] = (half_t)acc[mb][r];
+                half_t *out = route_partials + ((size_t)p.token * top_k + p.rank) * D;
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int n = n0 + j * 32 + acc_col(lane);
+                    if (n < D) out[n] = (half_t)acc[mt][j][r];
+                }
             }
         }
 }
