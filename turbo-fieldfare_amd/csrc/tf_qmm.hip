@@ -1,23 +1,26 @@
 // Matrix-core (MFMA) kernels: dense int4 QMM, and the grouped expert GEMMs of batched prefill
 // (gate/up + GeGLU, then down) driven by a work list of (expert, pair range) chunks.
 #include "tf_prefill_kernels.hpp"
+#include "tf_rowdot.hpp"
 
 using namespace tfk;
 
 namespace {
 
-// The lane's weight rows for the wave's two column tiles: tile j covers rows row0[j] + (lane & 31) of a matrix that
-// starts at w / s / b and has `limit[j]` rows.
+// The lane's weight rows for the wave's two column tiles: tile j covers rows row0[j] + (lane & 31) of a matrix of
+// `limit[j]` rows that starts at w / s / b.
 __device__ __forceinline__ QmmBRows make_b_rows(const uint8_t *const w[2], const uint8_t *const s[2], const uint8_t *const b[2],
                                                 const int row0[2], const int limit[2], int row_bytes, int groups, int lane) {
     QmmBRows rows;
     const int i = lane & 31, kb = lane >> 5;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const int n = min(row0[j] + i, limit[j] - 1);
-        rows.w[j] = w[j] + (size_t)n * row_bytes + kb * 16;
-        rows.s[j] = s[j] + (size_t)n * groups * 2;
-        rows.b[j] = b[j] + (size_t)n * groups * 2;
+        rows.w[j] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w[j]), 0, limit[j] * row_bytes, 0x00020000);
+        rows.s[j] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(s[j]), 0, limit[j] * groups * 2, 0x00020000);
+        rows.b[j] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(b[j]), 0, limit[j] * groups * 2, 0x00020000);
+        const uint32_t n = (uint32_t)(row0[j] + i);
+        rows.w_off[j] = n * (uint32_t)row_bytes + (uint32_t)kb * 16u;
+        rows.sb_off[j] = n * (uint32_t)groups * 2u;
     }
     return rows;
 }
@@ -35,22 +38,20 @@ __device__ __forceinline__ void zero_acc(float16_t acc[4][2]) {
 template <int SD>
 __global__ __launch_bounds__(256, 2) void qmm_dense_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *X,
                                                            long ldx, half_t *Y, long ldy, int M, int N, int K) {
-    __shared__ __align__(16) u32x4 lds[2 * kQmmBM * 8];
+    __shared__ __align__(128) uint8_t lds[kQmmLdsBytes];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = blockIdx.x * kQmmBN + wave * kQmmWaveN, m0 = blockIdx.y * kQmmBM;
-    const half_t *arow[kQmmAChunks];
+    QmmARows arow;
+    arow.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(X), 0, (int)0xFFFFFFFFu, 0x00020000);
 #pragma unroll
-    for (int q = 0; q < kQmmAChunks; ++q) {
-        const int r = (threadIdx.x + 256 * q) >> 3;
-        arow[q] = X + (size_t)min(m0 + r, M - 1) * ldx;
-    }
+    for (int q = 0; q < kQmmAChunks; ++q) qmm_a_rows_set(arow, q, (uint64_t)min(m0 + qmm_a_row_of(q), M - 1) * (uint64_t)ldx * 2u);
     const uint8_t *w[2] = {W, W}, *s[2] = {S, S}, *b[2] = {B, B};
     const int row0[2] = {n0, n0 + 32}, limit[2] = {N, N};
     const QmmBRows rows = make_b_rows(w, s, b, row0, limit, K >> 1, K >> 6, lane);
     const int row_tiles = min(4, (M - m0 + 31) >> 5);
     float16_t acc[4][2];
     zero_acc(acc);
-    qmm_k_loop<SD>(K >> 6, arow, rows, lds, lane, row_tiles, acc);
+    qmm_k_loop<SD>(K >> 6, arow, rows, (uint32_t)(uintptr_t)lds, lane, row_tiles, acc);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int n = n0 + j * 32 + acc_col(lane);
@@ -75,18 +76,26 @@ __global__ __launch_bounds__(256, 2) void grouped_phase1_mfma_kernel(ExpertTable
                                                                      const tf_prefill_pair *pairs, const half_t *hidden,
                                                                      long hidden_stride, half_t *acts, uint32_t acts_pair_base,
                                                                      int D, int F) {
-    __shared__ __align__(16) u32x4 lds[2 * kQmmBM * 8];
+    __shared__ __align__(128) uint8_t lds[kQmmLdsBytes];
     tf_prefill_group ch;
     if (!get_chunk(cl, blockIdx.y, ch)) return;
-    const uint8_t *base = expert_base(tab, ch.expert);
+    // everything taken from the work list is the same in all lanes: say so, the descriptors built from it live in
+    // scalar registers
+    ch.expert = uniform_u32(ch.expert);
+    ch.pair_start = uniform_u32(ch.pair_start);
+    ch.pair_count = uniform_u32(ch.pair_count);
+    const uint8_t *base = uniform_ptr(expert_base(tab, ch.expert));
     if (!base) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = blockIdx.x * kP1BN + wave * 32;
-    const half_t *arow[kQmmAChunks];
+    // the pairs of a chunk ascend by token: offsets are taken from the first pair's row
+    const uint32_t token0 = uniform_u32(pairs[ch.pair_start].token);
+    QmmARows arow;
+    arow.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(hidden + (size_t)token0 * hidden_stride), 0, (int)0xFFFFFFFFu, 0x00020000);
 #pragma unroll
     for (int q = 0; q < kQmmAChunks; ++q) {
-        const uint32_t r = (threadIdx.x + 256 * q) >> 3;
-        arow[q] = hidden + (size_t)pairs[ch.pair_start + min(r, ch.pair_count - 1)].token * hidden_stride;
+        const uint32_t r = min((uint32_t)qmm_a_row_of(q), ch.pair_count - 1);
+        qmm_a_rows_set(arow, q, (uint64_t)(pairs[ch.pair_start + r].token - token0) * (uint64_t)hidden_stride * 2u);
     }
     const uint8_t *w[2] = {base + off.gate_W_off, base + off.up_W_off};
     const uint8_t *s[2] = {base + off.gate_s_off, base + off.up_s_off};
@@ -96,7 +105,7 @@ __global__ __launch_bounds__(256, 2) void grouped_phase1_mfma_kernel(ExpertTable
     const int row_tiles = (int)((ch.pair_count + 31) >> 5);
     float16_t acc[4][2];
     zero_acc(acc);
-    qmm_k_loop<SD>(D >> 6, arow, rows, lds, lane, row_tiles, acc);
+    qmm_k_loop<SD>(D >> 6, arow, rows, (uint32_t)(uintptr_t)lds, lane, row_tiles, acc);
     const int n = n0 + acc_col(lane);
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt)
@@ -116,18 +125,24 @@ __global__ __launch_bounds__(256, 2) void grouped_down_mfma_kernel(ExpertTable t
                                                                    const tf_prefill_pair *pairs, const half_t *acts,
                                                                    uint32_t acts_pair_base, half_t *route_partials, int D, int F,
                                                                    int top_k) {
-    __shared__ __align__(16) u32x4 lds[2 * kQmmBM * 8];
+    __shared__ __align__(128) uint8_t lds[kQmmLdsBytes];
     tf_prefill_group ch;
     if (!get_chunk(cl, blockIdx.y, ch)) return;
-    const uint8_t *base = expert_base(tab, ch.expert);
+    // everything taken from the work list is the same in all lanes: say so, the descriptors built from it live in
+    // scalar registers
+    ch.expert = uniform_u32(ch.expert);
+    ch.pair_start = uniform_u32(ch.pair_start);
+    ch.pair_count = uniform_u32(ch.pair_count);
+    const uint8_t *base = uniform_ptr(expert_base(tab, ch.expert));
     if (!base) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = blockIdx.x * kQmmBN + wave * kQmmWaveN;
-    const half_t *arow[kQmmAChunks];
+    QmmARows arow;
+    arow.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(acts + (size_t)(ch.pair_start - acts_pair_base) * F), 0, (int)0xFFFFFFFFu, 0x00020000);
 #pragma unroll
     for (int q = 0; q < kQmmAChunks; ++q) {
-        const uint32_t r = (threadIdx.x + 256 * q) >> 3;
-        arow[q] = acts + (size_t)(ch.pair_start + min(r, ch.pair_count - 1) - acts_pair_base) * F;
+        const uint32_t r = min((uint32_t)qmm_a_row_of(q), ch.pair_count - 1);
+        qmm_a_rows_set(arow, q, (uint64_t)r * (uint64_t)F * 2u);
     }
     const uint8_t *w[2] = {base + off.down_W_off, base + off.down_W_off};
     const uint8_t *s[2] = {base + off.down_s_off, base + off.down_s_off};
@@ -137,7 +152,7 @@ __global__ __launch_bounds__(256, 2) void grouped_down_mfma_kernel(ExpertTable t
     const int row_tiles = (int)((ch.pair_count + 31) >> 5);
     float16_t acc[4][2];
     zero_acc(acc);
-    qmm_k_loop<SD>(F >> 6, arow, rows, lds, lane, row_tiles, acc);
+    qmm_k_loop<SD>(F >> 6, arow, rows, (uint32_t)(uintptr_t)lds, lane, row_tiles, acc);
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt)
 #pragma unroll

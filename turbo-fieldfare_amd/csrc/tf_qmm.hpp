@@ -3,15 +3,17 @@
 // quantization group (64) at a time:
 //
 //   W   never touches LDS.  In v_mfma_f32_32x32x16_f16 lane (i, kb) supplies, for output column i, the 8 weights of
-//       k-slots 8 kb .. 8 kb + 7.  The lane loads 16 packed bytes of "its" row (32 nibbles: the kb-th half of the group)
-//       and expands one 32-bit word (8 nibbles) per MFMA straight into the operand registers as half(q * s + b), the
-//       rounding point of the reference's staged-affine path (tensorops.metal:57-94).  MFMA number d of the group then
-//       covers k = {8d .. 8d+7} u {32+8d .. 32+8d+7}.
-//   X   goes through LDS once per block and K step, shared by the four waves: 16-byte chunks, the 8 elements of a chunk
-//       stored in the order (0,4,1,5,2,6,3,7) that the nibble masks produce for W, chunk positions XOR-swizzled so that
-//       both the row-major stores and the fragment reads are free of bank conflicts.
-//   global loads are requested kQmmDepth K steps ahead of their use (a ring of staging registers): one K step of MFMAs
-//       is far shorter than a trip to L2 or HBM.
+//       k-slots 8 kb .. 8 kb + 7.  The lane loads 16 packed bytes of "its" row (32 nibbles: the kb-th half of the group),
+//       two K steps ahead of their use, and expands one 32-bit word (8 nibbles) per MFMA straight into the operand
+//       registers as half(q * s + b), the rounding point of the reference's staged-affine path (tensorops.metal:57-94).
+//       MFMA number d of the group then covers k = {8d .. 8d+7} u {32+8d .. 32+8d+7}.
+//   X   is copied by the load unit from global memory straight into LDS (global_load_lds_dwordx4: no staging registers,
+//       no vector instructions), two K steps ahead, into a ring of three stages shared by the four waves.  A stage is
+//       128 rows x 8 chunks of 16 bytes; chunk c of row r sits at position c ^ ((r >> 1) & 7) of its row, which keeps
+//       the fragment reads free of bank conflicts although the copies land contiguously.
+//   The fragment reads are software-pipelined by hand (the fragments of MFMA group d + 1 are requested before group d
+//   is multiplied) and written as inline assembly with explicit waits: the compiler would otherwise make every LDS read
+//   wait for all outstanding copies, the prefetched ones included.
 //
 // Row indirection makes the same loop serve the grouped expert GEMMs: X rows can be gathered through a row table
 // (tokens routed to one expert) and Y rows scattered through another; row tiles beyond the rows present are skipped.
@@ -27,33 +29,24 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 constexpr int kQmmBM = 128;      // rows per block tile (4 MFMA row tiles)
 constexpr int kQmmWaveN = 64;    // columns per wave (2 MFMA column tiles)
 constexpr int kQmmBN = 256;      // columns per block tile (4 waves)
-constexpr int kQmmDepth = 2;     // K steps between a global request and its use
-constexpr int kQmmAChunks = kQmmBM * 8 / 256;   // 16-byte X chunks staged per thread and K step
+constexpr int kQmmAChunks = kQmmBM * 8 / 256;    // 16-byte X chunks copied per thread and K step
+constexpr int kQmmStageBytes = kQmmBM * 8 * 16;  // one X stage
+constexpr int kQmmLdsBytes = 3 * kQmmStageBytes; // the ring
 
-// (0,1)(2,3)(4,5)(6,7) -> (0,4)(1,5)(2,6)(3,7)
-__device__ __forceinline__ u32x4 permute_k8(const u32x4 v) {
-    u32x4 o;
-    o[0] = (v[0] & 0xFFFFu) | (v[2] << 16);
-    o[1] = (v[0] >> 16) | (v[2] & 0xFFFF0000u);
-    o[2] = (v[1] & 0xFFFFu) | (v[3] << 16);
-    o[3] = (v[1] >> 16) | (v[3] & 0xFFFF0000u);
-    return o;
-}
-
-// 8 nibbles of one word -> 8 fp16 weights half(q * s + b) in the order (0,4)(1,5)(2,6)(3,7).
-// q is formed exactly in fp16: the low nibble of each half as 1024 + q (0x6400 | q), the next one in place as 64 + q
-// (0x5400 | q << 4), each minus its offset; q * s + b is then one fp16 fused multiply-add on fp16 copies of s and b.
+// 8 nibbles of one word -> 8 fp16 weights half(q * s + b) in element order.  A byte holds two neighbouring elements:
+// v_perm_b32 copies it into both halves of a register, one mask leaves the low nibble in the low half as 1024 + q
+// (0x6400 | q) and the high nibble in place in the high half as 64 + q (0x5400 | q << 4); both offsets are removed
+// exactly, and q * s + b is one fp16 fused multiply-add on fp16 copies of s and b.
 __device__ __forceinline__ half8_t dequant_word(uint32_t v, half2_t s2, half2_t b2) {
-    const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
-    const half2_t k64 = {(half_t)64.0f, (half_t)64.0f};
-    const uint32_t v8 = v >> 8;
-    const half2_t q0 = as_half2((v & 0x000F000Fu) | 0x64006400u) - k1024;    // (e0, e4)
-    const half2_t q1 = as_half2((v & 0x00F000F0u) | 0x54005400u) - k64;      // (e1, e5)
-    const half2_t q2 = as_half2((v8 & 0x000F000Fu) | 0x64006400u) - k1024;   // (e2, e6)
-    const half2_t q3 = as_half2((v8 & 0x00F000F0u) | 0x54005400u) - k64;     // (e3, e7)
-    const half2_t w0 = __builtin_elementwise_fma(q0, s2, b2), w1 = __builtin_elementwise_fma(q1, s2, b2);
-    const half2_t w2 = __builtin_elementwise_fma(q2, s2, b2), w3 = __builtin_elementwise_fma(q3, s2, b2);
-    return half8_t{w0[0], w0[1], w1[0], w1[1], w2[0], w2[1], w3[0], w3[1]};
+    const half2_t offs = {(half_t)1024.0f, (half_t)64.0f};
+    half2_t w[4];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const uint32_t both = __builtin_amdgcn_perm(0u, v, 0x0c000c00u | ((uint32_t)p << 16) | (uint32_t)p);
+        const half2_t q = as_half2((both & 0x00F0000Fu) | 0x54006400u) - offs;
+        w[p] = __builtin_elementwise_fma(q, s2, b2);
+    }
+    return half8_t{w[0][0], w[0][1], w[1][0], w[1][1], w[2][0], w[2][1], w[3][0], w[3][1]};
 }
 
 template <int SD>
@@ -62,115 +55,190 @@ __device__ __forceinline__ half2_t sb_to_half2(uint16_t v) {
     return half2_t{h, h};
 }
 
-// 16-byte slot of X chunk (row r, chunk c of 8) inside one LDS stage of kQmmBM x 64 halves
+// 16-byte slot of X chunk (row r, chunk c of 8) inside one stage
 __device__ __forceinline__ int a_slot(int r, int c) { return r * 8 + (c ^ ((r >> 1) & 7)); }
 
-// Staging registers of one K step: this thread's X chunks, and for each of the wave's two column tiles the lane's 16
-// packed bytes and the row's scale / bias for the group.
-struct QmmStage {
-    u32x4 a[kQmmAChunks];
-    u32x4 w[2];
-    uint16_t s[2], b[2];
+// What a thread needs to know about the X chunks it copies: slot 256 q + threadIdx.x of every stage receives the chunk
+// at byte offset off[q] + 128 kt of the tensor the descriptor covers (rows beyond the tile repeat a valid row; nobody
+// reads what they produce).  32-bit offsets: the rows of one tile must lie within 4 GiB of the descriptor's base.
+typedef __amdgpu_buffer_rsrc_t qmm_rsrc_t;
+struct QmmARows {
+    qmm_rsrc_t rsrc;
+    uint32_t off[kQmmAChunks];
 };
+__device__ __forceinline__ int qmm_a_row_of(int q) { return (256 * q + (int)threadIdx.x) >> 3; }
+// row_byte_offset: where the row of slot group q starts, relative to the descriptor's base
+__device__ __forceinline__ void qmm_a_rows_set(QmmARows &a, int q, uint64_t row_byte_offset) {
+    const int p = 256 * q + (int)threadIdx.x, r = p >> 3;
+    a.off[q] = (uint32_t)row_byte_offset + (uint32_t)(((p & 7) ^ ((r >> 1) & 7)) * 16);
+}
 
-// What a lane needs to know about its two weight rows (one per column tile).  Columns beyond the matrix and rows
-// beyond the tile are served by a clamped, valid row: every load is unconditional, and what such lanes compute is
-// never stored.
+// The lane's two weight rows (one per column tile), as buffer descriptors over the whole matrices (scalar registers)
+// plus per-lane byte offsets: a step's loads then need only a scalar offset.  Columns beyond the matrix read zeros
+// (the descriptor ends with the matrix); what such lanes compute is never stored.
 struct QmmBRows {
-    const uint8_t *w[2];   // row start + kb * 16
-    const uint8_t *s[2];   // scales of the row
-    const uint8_t *b[2];
+    qmm_rsrc_t w[2], s[2], b[2];
+    uint32_t w_off[2];    // row * K/2 + kb * 16
+    uint32_t sb_off[2];   // row * K/64 * 2
 };
-
-__device__ __forceinline__ void qmm_stage_load(QmmStage &st, const half_t *const a_row[kQmmAChunks], const QmmBRows &rows, int kt) {
-#pragma unroll
-    for (int q = 0; q < kQmmAChunks; ++q) {
-        const int kc = (threadIdx.x + 256 * q) & 7;
-        st.a[q] = load16(a_row[q] + kt * 64 + kc * 8);
-    }
+struct QmmBStage {
+    u32x4 w[2];
+    uint16_t s[2], b[2];   // kept as loaded: touching them here would make the step wait for its own requests
+};
+__device__ __forceinline__ void qmm_b_load(QmmBStage &st, const QmmBRows &rows, int kt) {
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        st.w[j] = load16(rows.w[j] + kt * 32);
-        st.s[j] = *reinterpret_cast<const uint16_t *>(rows.s[j] + kt * 2);
-        st.b[j] = *reinterpret_cast<const uint16_t *>(rows.b[j] + kt * 2);
+        st.w[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rows.w[j], rows.w_off[j], kt * 32, 0));
+        st.s[j] = __builtin_amdgcn_raw_buffer_load_b16(rows.s[j], rows.sb_off[j], kt * 2, 0);
+        st.b[j] = __builtin_amdgcn_raw_buffer_load_b16(rows.b[j], rows.sb_off[j], kt * 2, 0);
     }
 }
 
-__device__ __forceinline__ void qmm_stage_store_a(const QmmStage &st, u32x4 *as) {
+// X tile of step kt -> LDS stage at byte address `stage` (wave-uniform); four copies of 64 x 16 bytes per wave
+__device__ __forceinline__ void qmm_a_copy(const QmmARows &a, int kt, uint32_t stage) {
+    const uint32_t wave_base = stage + (threadIdx.x >> 6) * 1024u;
 #pragma unroll
-    for (int q = 0; q < kQmmAChunks; ++q) {
-        const int c = threadIdx.x + 256 * q;
-        as[a_slot(c >> 3, c & 7)] = permute_k8(st.a[q]);
-    }
+    for (int q = 0; q < kQmmAChunks; ++q)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(a.rsrc, (__attribute__((address_space(3))) void *)(uintptr_t)(wave_base + q * 4096u), 16,
+                                                 a.off[q], kt * 128, 0, 0);
 }
 
-// One K group for this wave: acc[mt][j] += X[mt*32.., group] . W_j[.., group]^T for the row tiles mt < RT.
-template <int SD, int RT>
-__device__ __forceinline__ void qmm_group(const QmmStage &st, const u32x4 *as, int lane, float16_t acc[4][2]) {
-    const int i = lane & 31, kb = lane >> 5;
+// ds_read_b128 at addr + OFFSET, invisible to the compiler's memory tracking (see the header comment)
+template <int OFFSET>
+__device__ __forceinline__ u32x4 lds_read16(uint32_t addr) {
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+
+// One K group for this wave: acc[mt][j] += X[mt*32.., group] . W_j[.., group]^T for the row tiles mt < RT, out of LDS
+// stage STAGE.  frag[d]: LDS byte address of this lane's fragment for MFMA d in row tile 0 of stage 0.
+// The fragments of MFMA group d + 1 are requested before group d is multiplied, and the weights of group d + 1 are
+// expanded between the MFMAs of group d.
+template <int SD, int RT, int STAGE>
+__device__ __forceinline__ void qmm_group(const QmmBStage &st, const uint32_t frag[4], float16_t acc[4][2]) {
     half2_t s2[2], b2[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         s2[j] = sb_to_half2<SD>(st.s[j]);
         b2[j] = sb_to_half2<SD>(st.b[j]);
     }
+    constexpr int base = STAGE * kQmmStageBytes;
+    half8_t bf0 = dequant_word(st.w[0][0], s2[0], b2[0]);
+    half8_t bf1 = dequant_word(st.w[1][0], s2[1], b2[1]);
+    u32x4 af[2][4];
+    af[0][0] = lds_read16<base>(frag[0]);
+    if constexpr (RT > 1) af[0][1] = lds_read16<base + 4096>(frag[0]);
+    if constexpr (RT > 2) af[0][2] = lds_read16<base + 8192>(frag[0]);
+    if constexpr (RT > 3) af[0][3] = lds_read16<base + 12288>(frag[0]);
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-        const half8_t bf0 = dequant_word(st.w[0][d], s2[0], b2[0]);
-        const half8_t bf1 = dequant_word(st.w[1][d], s2[1], b2[1]);
+        // fragments of the next MFMA group first: they arrive while this group is multiplied
+        if (d < 3) {
+            af[(d + 1) & 1][0] = lds_read16<base>(frag[d + 1]);
+            if constexpr (RT > 1) af[(d + 1) & 1][1] = lds_read16<base + 4096>(frag[d + 1]);
+            if constexpr (RT > 2) af[(d + 1) & 1][2] = lds_read16<base + 8192>(frag[d + 1]);
+            if constexpr (RT > 3) af[(d + 1) & 1][3] = lds_read16<base + 12288>(frag[d + 1]);
+        }
+        // this group's RT reads are older than the RT just requested
+        constexpr int newer = RT;
+        if (d < 3) {
+            if constexpr (newer == 1) asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(af[d & 1][0]));
+            if constexpr (newer == 2) asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(af[d & 1][0]), "+v"(af[d & 1][1]));
+            if constexpr (newer == 3) asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(af[d & 1][0]), "+v"(af[d & 1][1]), "+v"(af[d & 1][2]));
+            if constexpr (newer == 4) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(af[d & 1][0]), "+v"(af[d & 1][1]), "+v"(af[d & 1][2]), "+v"(af[d & 1][3]));
+        } else {
+            if constexpr (RT == 1) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[d & 1][0]));
+            if constexpr (RT == 2) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[d & 1][0]), "+v"(af[d & 1][1]));
+            if constexpr (RT == 3) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[d & 1][0]), "+v"(af[d & 1][1]), "+v"(af[d & 1][2]));
+            if constexpr (RT == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[d & 1][0]), "+v"(af[d & 1][1]), "+v"(af[d & 1][2]), "+v"(af[d & 1][3]));
+        }
+        half8_t nf0 = bf0, nf1 = bf1;
 #pragma unroll
         for (int mt = 0; mt < RT; ++mt) {
-            const half8_t af = __builtin_bit_cast(half8_t, as[a_slot(mt * 32 + i, kb * 4 + d)]);
-            acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf0, acc[mt][0], 0, 0, 0);
-            acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, bf1, acc[mt][1], 0, 0, 0);
+            const half8_t a8 = __builtin_bit_cast(half8_t, af[d & 1][mt]);
+            acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a8, bf0, acc[mt][0], 0, 0, 0);
+            acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a8, bf1, acc[mt][1], 0, 0, 0);
+            // the next group's weights are expanded between the MFMAs
+            if (d < 3 && mt == 0) nf0 = dequant_word(st.w[0][d + 1], s2[0], b2[0]);
+            if (d < 3 && mt == (RT > 1 ? 1 : 0)) nf1 = dequant_word(st.w[1][d + 1], s2[1], b2[1]);
         }
+        bf0 = nf0;
+        bf1 = nf1;
     }
 }
 
-// The K loop.  Step kt lives in staging slot kt % kQmmDepth; its X tile is in LDS stage kt & 1 when it is multiplied.
-// While step kt is multiplied, the X tile of step kt + 1 goes to the other LDS stage and the slot of step kt is
-// refilled with step kt + kQmmDepth.  Requests and stores are unconditional (past the end they repeat the last step,
-// which nobody reads): a load under a branch would make every later wait for memory a wait for all of it.
+// The K loop.  The X tile of step kt lives in LDS stage kt % 3, the W registers of step kt in slot kt % 2.
+// Per step, in this order: meet at the barrier (every wave has waited for its X copies of this step); request the X tile
+// of step kt + 2 into the stage read two steps ago; multiply; request the W registers of step kt + 2 into the slot just
+// consumed; wait until the X copies of the next step have landed (the 6 W loads, 4 copies and 6 W loads issued after
+// them stay in flight).  Requests are unconditional: past the end they repeat the last step, which nobody reads, so
+// that the number of requests in flight is the same at every wait.
 template <int SD, int RT>
-__device__ __forceinline__ void qmm_k_loop_rt(int kt_count, const half_t *const a_row[kQmmAChunks], const QmmBRows &rows,
-                                              u32x4 *lds /* 2 stages of kQmmBM * 8 */, int lane, float16_t acc[4][2]) {
-    QmmStage st[kQmmDepth];
-    const int last = kt_count - 1;
-#pragma unroll
-    for (int u = 0; u < kQmmDepth; ++u) qmm_stage_load(st[u], a_row, rows, min(u, last));
-    qmm_stage_store_a(st[0], lds);
-    __syncthreads();
-    int kt0 = 0;
-    for (; kt0 + kQmmDepth <= kt_count; kt0 += kQmmDepth) {
-#pragma unroll
-        for (int u = 0; u < kQmmDepth; ++u) {
-            const int kt = kt0 + u;
-            qmm_group<SD, RT>(st[u], lds + (kt & 1) * (kQmmBM * 8), lane, acc);
-            qmm_stage_store_a(st[(u + 1) % kQmmDepth], lds + ((kt + 1) & 1) * (kQmmBM * 8));
-            qmm_stage_load(st[u], a_row, rows, min(kt + kQmmDepth, last));
-            __syncthreads();
-        }
+struct QmmLoop {
+    const QmmARows &a;
+    const QmmBRows &rows;
+    uint32_t lds;
+    uint32_t frag[4];
+    int last;
+    QmmBStage st[2];
+
+    template <int U3, int U2>
+    __device__ __forceinline__ void step(int kt, float16_t acc[4][2]) {
+        __builtin_amdgcn_s_barrier();
+        qmm_a_copy(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
+        qmm_group<SD, RT, U3>(st[U2], frag, acc);
+        qmm_b_load(st[U2], rows, min(kt + 2, last));
+        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
     }
+
+    __device__ __forceinline__ void run(int kt_count, int lane, float16_t acc[4][2]) {
+        last = kt_count - 1;
+        const int i = lane & 31, kb = lane >> 5;
+        const uint32_t frag0 = lds + (uint32_t)i * 128u + ((((uint32_t)kb * 4u) ^ (uint32_t)((i >> 1) & 7)) << 4);
 #pragma unroll
-    for (int u = 0; u < kQmmDepth - 1; ++u) {   // the kt_count % kQmmDepth steps left
-        const int kt = kt0 + u;
-        if (kt < kt_count) {
-            qmm_group<SD, RT>(st[u], lds + (kt & 1) * (kQmmBM * 8), lane, acc);
-            qmm_stage_store_a(st[(u + 1) % kQmmDepth], lds + ((kt + 1) & 1) * (kQmmBM * 8));
-            __syncthreads();
+        for (int d = 0; d < 4; ++d) frag[d] = frag0 ^ ((uint32_t)d << 4);   // lds is 128-byte aligned
+        qmm_a_copy(a, 0, lds);
+        qmm_a_copy(a, min(1, last), lds + kQmmStageBytes);
+        qmm_b_load(st[0], rows, 0);
+        qmm_b_load(st[1], rows, min(1, last));
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        int kt0 = 0;
+        for (; kt0 + 6 <= kt_count; kt0 += 6) {
+            step<0, 0>(kt0, acc);
+            step<1, 1>(kt0 + 1, acc);
+            step<2, 0>(kt0 + 2, acc);
+            step<0, 1>(kt0 + 3, acc);
+            step<1, 0>(kt0 + 4, acc);
+            step<2, 1>(kt0 + 5, acc);
         }
+        if (kt0 < kt_count) step<0, 0>(kt0, acc);
+        if (kt0 + 1 < kt_count) step<1, 1>(kt0 + 1, acc);
+        if (kt0 + 2 < kt_count) step<2, 0>(kt0 + 2, acc);
+        if (kt0 + 3 < kt_count) step<0, 1>(kt0 + 3, acc);
+        if (kt0 + 4 < kt_count) step<1, 0>(kt0 + 4, acc);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be landing in LDS when the block moves on
+        __builtin_amdgcn_s_barrier();
     }
+};
+
+template <int SD, int RT>
+__device__ __forceinline__ void qmm_k_loop_rt(int kt_count, const QmmARows &a, const QmmBRows &rows, uint32_t lds, int lane,
+                                              float16_t acc[4][2]) {
+    QmmLoop<SD, RT> loop{a, rows, lds};
+    loop.run(kt_count, lane, acc);
 }
 
 // row_tiles (1..4, block-uniform): 32-row tiles that hold rows; the others are not multiplied.
+// lds: byte address of kQmmLdsBytes of LDS, 128-byte aligned.
 template <int SD>
-__device__ __forceinline__ void qmm_k_loop(int kt_count, const half_t *const a_row[kQmmAChunks], const QmmBRows &rows, u32x4 *lds,
-                                           int lane, int row_tiles, float16_t acc[4][2]) {
+__device__ __forceinline__ void qmm_k_loop(int kt_count, const QmmARows &a, const QmmBRows &rows, uint32_t lds, int lane,
+                                           int row_tiles, float16_t acc[4][2]) {
     switch (row_tiles) {
-        case 1: qmm_k_loop_rt<SD, 1>(kt_count, a_row, rows, lds, lane, acc); break;
-        case 2: qmm_k_loop_rt<SD, 2>(kt_count, a_row, rows, lds, lane, acc); break;
-        case 3: qmm_k_loop_rt<SD, 3>(kt_count, a_row, rows, lds, lane, acc); break;
-        default: qmm_k_loop_rt<SD, 4>(kt_count, a_row, rows, lds, lane, acc); break;
+        case 1: qmm_k_loop_rt<SD, 1>(kt_count, a, rows, lds, lane, acc); break;
+        case 2: qmm_k_loop_rt<SD, 2>(kt_count, a, rows, lds, lane, acc); break;
+        case 3: qmm_k_loop_rt<SD, 3>(kt_count, a, rows, lds, lane, acc); break;
+        default: qmm_k_loop_rt<SD, 4>(kt_count, a, rows, lds, lane, acc); break;
     }
 }
 
