@@ -7,20 +7,23 @@ using namespace tfk;
 
 namespace {
 
-// The lane's weight rows for the wave's two column tiles: tile j covers rows row0[j] + (lane & 31) of a matrix of
-// `limit[j]` rows that starts at w / s / b.
+// The wave's weight rows: column tile j covers rows row0[j] .. row0[j] + 31 of a matrix of `limit[j]` rows that starts
+// at w / s / b.
 __device__ __forceinline__ QmmBRows make_b_rows(const uint8_t *const w[2], const uint8_t *const s[2], const uint8_t *const b[2],
                                                 const int row0[2], const int limit[2], int row_bytes, int groups, int lane) {
     QmmBRows rows;
-    const int i = lane & 31, kb = lane >> 5;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         rows.w[j] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w[j]), 0, limit[j] * row_bytes, 0x00020000);
         rows.s[j] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(s[j]), 0, limit[j] * groups * 2, 0x00020000);
         rows.b[j] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(b[j]), 0, limit[j] * groups * 2, 0x00020000);
-        const uint32_t n = (uint32_t)(row0[j] + i);
-        rows.w_off[j] = n * (uint32_t)row_bytes + (uint32_t)kb * 16u;
-        rows.sb_off[j] = n * (uint32_t)groups * 2u;
+        rows.sb_off[j] = (uint32_t)(row0[j] + (lane & 31)) * (uint32_t)groups * 2u;
+    }
+#pragma unroll
+    for (int t = 0; t < 4; ++t) {
+        const int r = 16 * (t & 1) + (lane >> 2);                    // row inside the column tile
+        const int piece = (lane & 3) ^ ((r >> 2) & 3);
+        rows.copy_off[t] = (uint32_t)(row0[t >> 1] + r) * (uint32_t)row_bytes + (uint32_t)piece * 16u;
     }
     return rows;
 }

@@ -2,11 +2,14 @@
 // int4 layout.  A 256-thread block owns a 128 x 256 output tile (four waves, each 128 rows x 64 columns) and walks K one
 // quantization group (64) at a time:
 //
-//   W   never touches LDS.  In v_mfma_f32_32x32x16_f16 lane (i, kb) supplies, for output column i, the 8 weights of
-//       k-slots 8 kb .. 8 kb + 7.  The lane loads 16 packed bytes of "its" row (32 nibbles: the kb-th half of the group),
-//       two K steps ahead of their use, and expands one 32-bit word (8 nibbles) per MFMA straight into the operand
-//       registers as half(q * s + b), the rounding point of the reference's staged-affine path (tensorops.metal:57-94).
-//       MFMA number d of the group then covers k = {8d .. 8d+7} u {32+8d .. 32+8d+7}.
+//   W   In v_mfma_f32_32x32x16_f16 lane (i, kb) supplies, for output column i, the 8 weights of k-slots 8 kb .. 8 kb + 7.
+//       The lane reads 16 packed bytes of "its" row (32 nibbles: the kb-th half of the group) and expands one 32-bit
+//       word (8 nibbles) per MFMA straight into the operand registers as half(q * s + b), the rounding point of the
+//       reference's staged-affine path (tensorops.metal:57-94).  MFMA number d of the group then covers
+//       k = {8d .. 8d+7} u {32+8d .. 32+8d+7}.  Reading "its" row straight from global memory would touch 32 cache
+//       lines per load instruction; instead the load unit copies the packed rows into a wave-private LDS area two K
+//       steps at a time (64 contiguous bytes per row, four lanes per row), and the lanes pick their 16 bytes there.
+//       Scales and biases are loaded two groups at a time (one 32-bit load per row and array).
 //   X   is copied by the load unit from global memory straight into LDS (global_load_lds_dwordx4: no staging registers,
 //       no vector instructions), two K steps ahead, into a ring of three stages shared by the four waves.  A stage is
 //       128 rows x 8 chunks of 16 bytes; chunk c of row r sits at position c ^ ((r >> 1) & 7) of its row, which keeps
@@ -31,7 +34,8 @@ constexpr int kQmmWaveN = 64;    // columns per wave (2 MFMA column tiles)
 constexpr int kQmmBN = 256;      // columns per block tile (4 waves)
 constexpr int kQmmAChunks = kQmmBM * 8 / 256;    // 16-byte X chunks copied per thread and K step
 constexpr int kQmmStageBytes = kQmmBM * 8 * 16;  // one X stage
-constexpr int kQmmLdsBytes = 3 * kQmmStageBytes; // the ring
+constexpr int kQmmWBytes = 64 * 64;               // packed W rows of one wave for two K steps: 64 rows x 64 bytes
+constexpr int kQmmLdsBytes = 3 * kQmmStageBytes + 4 * 2 * kQmmWBytes;   // X ring + two W buffers per wave
 
 // 8 nibbles of one word -> 8 fp16 weights half(q * s + b) in element order.  A byte holds two neighbouring elements:
 // v_perm_b32 copies it into both halves of a register, one mask leaves the low nibble in the low half as 1024 + q
@@ -73,25 +77,45 @@ __device__ __forceinline__ void qmm_a_rows_set(QmmARows &a, int q, uint64_t row_
     a.off[q] = (uint32_t)row_byte_offset + (uint32_t)(((p & 7) ^ ((r >> 1) & 7)) * 16);
 }
 
-// The lane's two weight rows (one per column tile), as buffer descriptors over the whole matrices (scalar registers)
-// plus per-lane byte offsets: a step's loads then need only a scalar offset.  Columns beyond the matrix read zeros
-// (the descriptor ends with the matrix); what such lanes compute is never stored.
+// The wave's weight rows (32 per column tile), as buffer descriptors over the whole matrices (scalar registers) plus
+// per-lane byte offsets.  Columns beyond the matrix read zeros (the descriptor ends with the matrix); what such lanes
+// compute is never stored.
+//   copy_off[t]: where copy number t of a two-step block starts for this lane: row 16 (t & 1) + lane / 4 of column
+//                tile t / 2, 16-byte piece (lane & 3) ^ ((row / 4) & 3) of the row's 64 bytes (the XOR keeps the later
+//                reads free of bank conflicts);
+//   sb_off[j]:   the lane's own row (lane & 31) of tile j in the scale / bias arrays.
 struct QmmBRows {
     qmm_rsrc_t w[2], s[2], b[2];
-    uint32_t w_off[2];    // row * K/2 + kb * 16
-    uint32_t sb_off[2];   // row * K/64 * 2
+    uint32_t copy_off[4];
+    uint32_t sb_off[2];
 };
-struct QmmBStage {
-    u32x4 w[2];
-    uint16_t s[2], b[2];   // kept as loaded: touching them here would make the step wait for its own requests
+// scales and biases of the lane's rows for two consecutive groups (low half: even group)
+struct QmmSB {
+    uint32_t s[2], b[2];
 };
-__device__ __forceinline__ void qmm_b_load(QmmBStage &st, const QmmBRows &rows, int kt) {
+// single (wave-uniform): the pair has only its first group (the last pair of an odd number of groups); a 32-bit load
+// would run past the end of the last row.  Both arms issue the same number of loads.
+__device__ __forceinline__ void qmm_sb_load(QmmSB &sb, const QmmBRows &rows, int pair, bool single) {
+    if (single) {
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        st.w[j] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rows.w[j], rows.w_off[j], kt * 32, 0));
-        st.s[j] = __builtin_amdgcn_raw_buffer_load_b16(rows.s[j], rows.sb_off[j], kt * 2, 0);
-        st.b[j] = __builtin_amdgcn_raw_buffer_load_b16(rows.b[j], rows.sb_off[j], kt * 2, 0);
+        for (int j = 0; j < 2; ++j) {
+            sb.s[j] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rows.s[j], rows.sb_off[j], pair * 4, 0);
+            sb.b[j] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rows.b[j], rows.sb_off[j], pair * 4, 0);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            sb.s[j] = __builtin_amdgcn_raw_buffer_load_b32(rows.s[j], rows.sb_off[j], pair * 4, 0);
+            sb.b[j] = __builtin_amdgcn_raw_buffer_load_b32(rows.b[j], rows.sb_off[j], pair * 4, 0);
+        }
     }
+}
+// packed W rows of K steps 2 pair, 2 pair + 1 -> the wave's LDS buffer at byte address `dst` (wave-uniform)
+__device__ __forceinline__ void qmm_w_copy(const QmmBRows &rows, int pair, uint32_t dst) {
+#pragma unroll
+    for (int t = 0; t < 4; ++t)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rows.w[t >> 1], (__attribute__((address_space(3))) void *)(uintptr_t)(dst + t * 1024u), 16,
+                                                 rows.copy_off[t], pair * 64, 0, 0);
 }
 
 // X tile of step kt -> LDS stage at byte address `stage` (wave-uniform); four copies of 64 x 16 bytes per wave
@@ -115,17 +139,17 @@ __device__ __forceinline__ u32x4 lds_read16(uint32_t addr) {
 // stage STAGE.  frag[d]: LDS byte address of this lane's fragment for MFMA d in row tile 0 of stage 0.
 // The fragments of MFMA group d + 1 are requested before group d is multiplied, and the weights of group d + 1 are
 // expanded between the MFMAs of group d.
-template <int SD, int RT, int STAGE>
-__device__ __forceinline__ void qmm_group(const QmmBStage &st, const uint32_t frag[4], float16_t acc[4][2]) {
+template <int SD, int RT, int STAGE, int HALF>
+__device__ __forceinline__ void qmm_group(const u32x4 w[2], const QmmSB &sb, const uint32_t frag[4], float16_t acc[4][2]) {
     half2_t s2[2], b2[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        s2[j] = sb_to_half2<SD>(st.s[j]);
-        b2[j] = sb_to_half2<SD>(st.b[j]);
+        s2[j] = sb_to_half2<SD>((uint16_t)(HALF ? sb.s[j] >> 16 : sb.s[j] & 0xFFFFu));
+        b2[j] = sb_to_half2<SD>((uint16_t)(HALF ? sb.b[j] >> 16 : sb.b[j] & 0xFFFFu));
     }
     constexpr int base = STAGE * kQmmStageBytes;
-    half8_t bf0 = dequant_word(st.w[0][0], s2[0], b2[0]);
-    half8_t bf1 = dequant_word(st.w[1][0], s2[1], b2[1]);
+    half8_t bf0 = dequant_word(w[0][0], s2[0], b2[0]);
+    half8_t bf1 = dequant_word(w[1][0], s2[1], b2[1]);
     u32x4 af[2][4];
     af[0][0] = lds_read16<base>(frag[0]);
     if constexpr (RT > 1) af[0][1] = lds_read16<base + 4096>(frag[0]);
@@ -160,63 +184,99 @@ __device__ __forceinline__ void qmm_group(const QmmBStage &st, const uint32_t fr
             acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a8, bf0, acc[mt][0], 0, 0, 0);
             acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a8, bf1, acc[mt][1], 0, 0, 0);
             // the next group's weights are expanded between the MFMAs
-            if (d < 3 && mt == 0) nf0 = dequant_word(st.w[0][d + 1], s2[0], b2[0]);
-            if (d < 3 && mt == (RT > 1 ? 1 : 0)) nf1 = dequant_word(st.w[1][d + 1], s2[1], b2[1]);
+            if (d < 3 && mt == 0) nf0 = dequant_word(w[0][d + 1], s2[0], b2[0]);
+            if (d < 3 && mt == (RT > 1 ? 1 : 0)) nf1 = dequant_word(w[1][d + 1], s2[1], b2[1]);
         }
         bf0 = nf0;
         bf1 = nf1;
     }
 }
 
-// The K loop.  The X tile of step kt lives in LDS stage kt % 3, the W registers of step kt in slot kt % 2.
-// Per step, in this order: meet at the barrier (every wave has waited for its X copies of this step); request the X tile
-// of step kt + 2 into the stage read two steps ago; multiply; request the W registers of step kt + 2 into the slot just
-// consumed; wait until the X copies of the next step have landed (the 6 W loads, 4 copies and 6 W loads issued after
-// them stay in flight).  Requests are unconditional: past the end they repeat the last step, which nobody reads, so
-// that the number of requests in flight is the same at every wait.
+// The K loop.  The X tile of step kt lives in LDS stage kt % 3; the packed W rows of steps 2p, 2p + 1 in the wave's
+// buffer p & 1, the scales / biases of those two groups in register slot p & 1.
+// Even step kt = 2p:  barrier; request X(kt + 2), W(p + 1); multiply with the W words read from LDS at the end of the
+//                     previous step; request the scales of pair p + 1; wait for X(kt + 1) (12 newer requests stay in
+//                     flight).
+// Odd step:           barrier; request X(kt + 2); multiply; wait for X(kt + 1), W(p + 1) and the scales (4 newer
+//                     requests stay in flight); read the W words of both steps of pair p + 1 from LDS, switch to
+//                     its scales.
+// Requests are unconditional: past the end they repeat the last step or pair, which nobody reads, so that the number
+// of requests in flight is the same at every wait.
 template <int SD, int RT>
 struct QmmLoop {
     const QmmARows &a;
     const QmmBRows &rows;
     uint32_t lds;
     uint32_t frag[4];
-    int last;
-    QmmBStage st[2];
+    uint32_t wread;      // this lane's 16 bytes of column tile 0, first step of a pair, in the wave's W buffer 0
+    uint32_t wbuf;       // the wave's W buffer 0
+    int last, last_pair;
+    bool odd_count;      // an odd number of K steps: the last pair has one group
+    u32x4 w[2][2];       // [step of the pair][column tile]
+    QmmSB sb, sb_next;
+    uint32_t pb;         // (current pair & 1) * kQmmWBytes: which W buffer holds the current pair
 
-    template <int U3, int U2>
-    __device__ __forceinline__ void step(int kt, float16_t acc[4][2]) {
+    __device__ __forceinline__ void read_w(uint32_t at) {
+        w[0][0] = lds_read16<0>(at);
+        w[0][1] = lds_read16<2048>(at);
+        w[1][0] = lds_read16<0>(at ^ 32u);
+        w[1][1] = lds_read16<2048>(at ^ 32u);
+        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]));
+    }
+
+    template <int U3>
+    __device__ __forceinline__ void even_step(int kt, float16_t acc[4][2]) {
+        const int pair = kt >> 1;
         __builtin_amdgcn_s_barrier();
         qmm_a_copy(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
-        qmm_group<SD, RT, U3>(st[U2], frag, acc);
-        qmm_b_load(st[U2], rows, min(kt + 2, last));
-        asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+        qmm_w_copy(rows, min(pair + 1, last_pair), wbuf + (pb ^ kQmmWBytes));
+        qmm_group<SD, RT, U3, 0>(w[0], sb, frag, acc);
+        const int next_pair = min(pair + 1, last_pair);
+        qmm_sb_load(sb_next, rows, next_pair, odd_count && next_pair == last_pair);
+        asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+    }
+    template <int U3>
+    __device__ __forceinline__ void odd_step(int kt, float16_t acc[4][2]) {
+        __builtin_amdgcn_s_barrier();
+        qmm_a_copy(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
+        qmm_group<SD, RT, U3, 1>(w[1], sb, frag, acc);
+        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        pb ^= kQmmWBytes;
+        read_w(wread + pb);
+        sb = sb_next;
     }
 
     __device__ __forceinline__ void run(int kt_count, int lane, float16_t acc[4][2]) {
         last = kt_count - 1;
+        last_pair = last >> 1;
+        odd_count = (kt_count & 1) != 0;
         const int i = lane & 31, kb = lane >> 5;
         const uint32_t frag0 = lds + (uint32_t)i * 128u + ((((uint32_t)kb * 4u) ^ (uint32_t)((i >> 1) & 7)) << 4);
 #pragma unroll
         for (int d = 0; d < 4; ++d) frag[d] = frag0 ^ ((uint32_t)d << 4);   // lds is 128-byte aligned
+        wbuf = lds + 3 * kQmmStageBytes + (threadIdx.x >> 6) * (2 * kQmmWBytes);
+        wread = wbuf + (uint32_t)i * 64u + ((((uint32_t)kb) ^ (uint32_t)((i >> 2) & 3)) << 4);
+        pb = 0;
         qmm_a_copy(a, 0, lds);
         qmm_a_copy(a, min(1, last), lds + kQmmStageBytes);
-        qmm_b_load(st[0], rows, 0);
-        qmm_b_load(st[1], rows, min(1, last));
+        qmm_w_copy(rows, 0, wbuf);
+        qmm_sb_load(sb, rows, 0, odd_count && last_pair == 0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        read_w(wread);
         int kt0 = 0;
         for (; kt0 + 6 <= kt_count; kt0 += 6) {
-            step<0, 0>(kt0, acc);
-            step<1, 1>(kt0 + 1, acc);
-            step<2, 0>(kt0 + 2, acc);
-            step<0, 1>(kt0 + 3, acc);
-            step<1, 0>(kt0 + 4, acc);
-            step<2, 1>(kt0 + 5, acc);
+            even_step<0>(kt0, acc);
+            odd_step<1>(kt0 + 1, acc);
+            even_step<2>(kt0 + 2, acc);
+            odd_step<0>(kt0 + 3, acc);
+            even_step<1>(kt0 + 4, acc);
+            odd_step<2>(kt0 + 5, acc);
         }
-        if (kt0 < kt_count) step<0, 0>(kt0, acc);
-        if (kt0 + 1 < kt_count) step<1, 1>(kt0 + 1, acc);
-        if (kt0 + 2 < kt_count) step<2, 0>(kt0 + 2, acc);
-        if (kt0 + 3 < kt_count) step<0, 1>(kt0 + 3, acc);
-        if (kt0 + 4 < kt_count) step<1, 0>(kt0 + 4, acc);
+        if (kt0 < kt_count) even_step<0>(kt0, acc);
+        if (kt0 + 1 < kt_count) odd_step<1>(kt0 + 1, acc);
+        if (kt0 + 2 < kt_count) even_step<2>(kt0 + 2, acc);
+        if (kt0 + 3 < kt_count) odd_step<0>(kt0 + 3, acc);
+        if (kt0 + 4 < kt_count) even_step<1>(kt0 + 4, acc);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be landing in LDS when the block moves on
         __builtin_amdgcn_s_barrier();
     }
