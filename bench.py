@@ -389,6 +389,18 @@ def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride):
                                   "ms": round(us / 1e3, 3), "tokens_per_s": round(T / (us * 1e-6), 1), "unique_experts": unique,
                                   "TFLOPs": round(routed_flop / (us * 1e-6) / 1e12, 2),
                                   "frac_mfma_fp16_peak": round(routed_flop / (us * 1e-6) / 2.5e15, 4)}
+    # the router block for the same 2048 tokens (8-bit projection on the matrix cores + one selection wave per token)
+    hid_r = torch.randn((T, D), device="cuda", generator=gen).to(torch.float16)
+    idx_r = torch.zeros((T, TOPK), dtype=torch.int32, device="cuda")
+    wts_r = torch.zeros((T, TOPK), dtype=torch.float16, device="cuda")
+
+    def router_fn(i):
+        rc = lib.tf_prefill_router_gemma4_block(h, stream, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0,
+                                                hid_r.data_ptr(), 0, r["eff"].data_ptr(), 0, r["gain"].data_ptr(), 0,
+                                                idx_r.data_ptr(), 0, wts_r.data_ptr(), 0, T, E, D, TOPK, D)
+        assert rc == 0, k.last_error()
+    us_router = time_loop(torch, router_fn, 20, warmup=2)
+    res["prefill_router_2048"] = {"us": round(us_router, 2), "tokens_per_s": round(T / (us_router * 1e-6), 1)}
     # shared expert over all tokens: gate, up (2112 x 2816), GeGLU, down (2816 x 2112) as dense int4 QMMs
     gW, gS, gB = make_int4(torch, gen, F_SHARED, D)
     uW, uS, uB = make_int4(torch, gen, F_SHARED, D)

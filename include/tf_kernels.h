@@ -193,6 +193,9 @@ int32_t tf_router_gemma4(tf_ctx *ctx, tf_stream stream,
 /* The fp32 logits of the last tf_router_gemma4 call on this ctx (the wrapper-owned `routerLogits`, MoE.swift:92-99).
  * Device pointer to 256 floats; valid until the ctx is destroyed. */
 const float *tf_router_logits(const tf_ctx *ctx);
+/* The same for the block router: [query_count, num_experts] fp32 logits of the most recent
+ * tf_prefill_router_gemma4_block call on this context (NULL before the first call). */
+const float *tf_prefill_router_logits(const tf_ctx *ctx);
 
 /* ---- routed experts ------------------------------------------------------------------------------------------------- */
 /* MoE.encodeRoutedPersistentPhase1U16Load (MoE.swift:180-213) -> moe_phase1_gate_up_act_u16load (moe.metal:407-423):

@@ -8,7 +8,7 @@ import pytest
 import torch
 
 import refcases
-from gpu_helpers import ctx, dev, host, tfk, within_north_star, zeros_bytes
+from gpu_helpers import device_view, ctx, dev, host, tfk, within_north_star, zeros_bytes
 from oracle import tfo
 
 pytestmark = pytest.mark.gpu
@@ -78,6 +78,31 @@ def test_block_router_near_tie_and_generic_topk():
     bad = k.lib.tf_prefill_router_gemma4_block(k.handle, None, z.data_ptr(), 0, z.data_ptr(), 0, z.data_ptr(), 0, z.data_ptr(), 0, z.data_ptr(), 0,
                                                z.data_ptr(), 0, z.data_ptr(), 0, z.data_ptr(), 0, 1, 16, 128, 65, 128)
     assert bad == tfk.TF_ERR_INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("rows,experts,d", [(200, 128, 2816), (97, 48, 704), (65, 128, 128)])
+def test_block_router_many_tokens_on_matrix_cores(rows, experts, d):
+    # more than 64 tokens take the matrix-core projection: same logits (to 1e-4) and, away from near ties, the same
+    # experts in the same order as the reference's scalar arithmetic
+    rng = np.random.default_rng(rows * 7 + experts)
+    W, S, B = refcases.synthetic_int8(experts, d, 0xB10C + rows)
+    hidden = np.concatenate([refcases.normal_f16(d, 0x500 + r) for r in range(rows)])
+    eff_f = rng.uniform(0.5, 1.5, d).astype(np.float32) / np.float32(np.sqrt(d))
+    pes_f = rng.uniform(0.6, 1.4, experts).astype(np.float32)
+    eff, pes = tfo.bf16_bits_array(eff_f), tfo.bf16_bits_array(pes_f)
+    got_idx, got_w = prefill_router(W, S, B, hidden, d, eff, pes, rows)
+    logits = device_view(ctx().lib.tf_prefill_router_logits(ctx().handle), rows * experts, "<f4").reshape(rows, experts)
+    pinned = 0
+    for r in range(rows):
+        ref_idx, ref_w, ref_logits = tfo.router_reference(W, S, B, tfo.from_f16_bits(hidden[r * d:(r + 1) * d]), tfo.bf16_array_to_float(eff),
+                                                          tfo.bf16_array_to_float(pes))
+        assert tfo.rel_error(logits[r], ref_logits) < 1e-4
+        srt = np.sort(ref_logits)[::-1]
+        if np.min(srt[:8] - srt[1:9]) > 1e-4 * np.max(np.abs(srt)):
+            pinned += 1
+            assert list(got_idx[r]) == list(ref_idx)
+            assert np.max(np.abs(got_w[r] - ref_w)) < 5e-3
+    assert pinned > rows // 2
 
 
 def device_grouping(idx, wts_bits, T, top_k, E):

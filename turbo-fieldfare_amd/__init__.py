@@ -96,6 +96,7 @@ EXPORTS = {
     "tf_ctx_set_step_timing": (i32, [vp, i32]),
     "tf_ctx_last_step_timing": (i32, [vp, C.POINTER(C.c_float)]),
     "tf_router_logits": (vp, [vp]),
+    "tf_prefill_router_logits": (vp, [vp]),
     "tf_dequantize_int4_affine": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32]),
     "tf_dequantize_int8_affine": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32]),
     "tf_dequant_int4_gemv": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32, i32]),

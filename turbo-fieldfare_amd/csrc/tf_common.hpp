@@ -160,6 +160,14 @@ __device__ __forceinline__ float arrange_x(const u32x4 *xr, half2_t *xq) {
     return sum;
 }
 
+// Block barrier that orders LDS traffic only: unlike __syncthreads() it does not wait for global loads that are still in
+// flight, so requests issued ahead of their use stay ahead across the barrier.
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
 __device__ __forceinline__ u32x4 load16(const void *p) { return *reinterpret_cast<const u32x4 *>(p); }
 
 // GELU, tanh approximation, as the reference kernels compute it (Metal/MoE/moe.metal:53-60):

@@ -107,5 +107,6 @@ int32_t tf_ctx_last_step_timing(tf_ctx *ctx, float out_us[4]) {
 }
 
 const float *tf_router_logits(const tf_ctx *ctx) { return ctx ? ctx->router_logits : nullptr; }
+const float *tf_prefill_router_logits(const tf_ctx *ctx) { return ctx ? ctx->prefill_logits : nullptr; }
 
 }  // extern "C"

@@ -70,6 +70,163 @@ __global__ __launch_bounds__(64) void prefill_select_kernel(const float *logits,
                   num_experts, top_k, threadIdx.x);
 }
 
+// Many tokens: the router projection as a matrix product on the matrix cores.  A block takes 32 tokens and up to 128
+// experts (wave w: experts 32 w ..), one quantization group of 64 at a time:
+//   - the 256 threads form x' = float(hidden) * float(effective_scale) for the block's 32 tokens x 64 columns once,
+//     split it into two fp16 parts (x' * 16 = hi + lo, so that nothing of its 24 bits is lost) and put both in LDS,
+//     together with the fp32 column sums of x' that the bias term needs;
+//   - every wave multiplies its 32 experts' 8-bit weights (exact in fp16) with both parts: the products are exact and
+//     accumulate in fp32, per group, and the group's scale is applied to the accumulator, as in the reference's
+//     arithmetic (s * sum(q x') + b * sum(x'));
+//   - the bias term sum_g b[e,g] * sum(x')[t,g] is one more small product over the groups at the end.
+// The selection runs afterwards, one wave per token, on the logits this kernel leaves in scratch.
+template <int SD>
+__global__ __launch_bounds__(256) void prefill_logits_mfma_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B,
+                                                                  const half_t *hidden, long hidden_stride, const uint16_t *eff,
+                                                                  float *logits, uint32_t query_count, uint32_t num_experts, int d) {
+    __shared__ __align__(16) u32x4 x_hi[2][256], x_lo[2][256];   // [stage][a_slot(token, chunk)]
+    __shared__ float xsum[32][65];                                // [token][group], padded
+    __shared__ __align__(16) u32x4 g_hi[256], g_lo[256];         // the sums as fp16 parts, a_slot(token, chunk of 8 groups)
+    __shared__ __align__(16) half_t bias_h[128][64];              // [expert of the block][group] biases as fp16, 0 beyond
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int i = lane & 31, kb = lane >> 5;
+    const int groups = d >> 6;
+    const uint32_t t0 = blockIdx.x * 32;
+    // producer role: token p_tok, 8 columns p_chunk * 8 .. of every group
+    const int p_tok = threadIdx.x >> 3, p_chunk = threadIdx.x & 7;
+    const half_t *p_row = hidden + (size_t)min(t0 + (uint32_t)p_tok, query_count - 1) * hidden_stride + p_chunk * 8;
+    const uint16_t *p_eff = eff + p_chunk * 8;
+    const int p_slot = a_slot(p_tok, p_chunk);
+    // consumer role: expert row e_row (clamped), the kb-th 32 columns of every group
+    const uint32_t e_lane = (uint32_t)wave * 32u + (uint32_t)i;
+    const uint32_t e_row = min(e_lane, num_experts - 1);
+    const uint8_t *w_row = W + (size_t)e_row * d + kb * 32;
+    const uint8_t *s_row = S + (size_t)e_row * groups * 2;
+    const uint8_t *b_row = B + (size_t)e_row * groups * 2;
+    const bool wave_live = (uint32_t)wave * 32u < num_experts;
+
+    auto produce = [&](const u32x4 hraw, const u32x4 eraw, int stage, int g) {
+        float xv[8], sum = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const half2_t h2 = as_half2(hraw[j]);
+            xv[2 * j] = (float)h2[0] * __uint_as_float(eraw[j] << 16);
+            xv[2 * j + 1] = (float)h2[1] * __uint_as_float(eraw[j] & 0xFFFF0000u);
+            sum += xv[2 * j];
+            sum += xv[2 * j + 1];
+        }
+        u32x4 hi, lo;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            half2_t a, b;
+            a[0] = (half_t)(xv[2 * j] * 16.0f);
+            a[1] = (half_t)(xv[2 * j + 1] * 16.0f);
+            b[0] = (half_t)(xv[2 * j] * 16.0f - (float)a[0]);
+            b[1] = (half_t)(xv[2 * j + 1] * 16.0f - (float)a[1]);
+            hi[j] = as_u32(a);
+            lo[j] = as_u32(b);
+        }
+        x_hi[stage][p_slot] = hi;
+        x_lo[stage][p_slot] = lo;
+        sum += dpp_f32<0xB1>(sum);    // the 8 chunks of a token sit in 8 neighbouring lanes
+        sum += dpp_f32<0x4E>(sum);
+        sum += dpp_f32<0x141>(sum);
+        if (p_chunk == 0) xsum[p_tok][g] = sum;
+    };
+    // 8 bytes (two words) -> 8 fp16 weights in element order, exact
+    auto expand8 = [&](uint32_t w0, uint32_t w1) {
+        const half2_t k1024 = {(half_t)1024.0f, (half_t)1024.0f};
+        const half2_t q0 = as_half2(__builtin_amdgcn_perm(0u, w0, 0x0c010c00u) | 0x64006400u) - k1024;
+        const half2_t q1 = as_half2(__builtin_amdgcn_perm(0u, w0, 0x0c030c02u) | 0x64006400u) - k1024;
+        const half2_t q2 = as_half2(__builtin_amdgcn_perm(0u, w1, 0x0c010c00u) | 0x64006400u) - k1024;
+        const half2_t q3 = as_half2(__builtin_amdgcn_perm(0u, w1, 0x0c030c02u) | 0x64006400u) - k1024;
+        return half8_t{q0[0], q0[1], q1[0], q1[1], q2[0], q2[1], q3[0], q3[1]};
+    };
+
+    for (int z = threadIdx.x; z < 128 * 64 / 8; z += 256) reinterpret_cast<u32x4 *>(&bias_h[0][0])[z] = u32x4{0u, 0u, 0u, 0u};
+    // requests run two groups ahead of their use: one group of MFMAs is much shorter than a trip to L2
+    const int g1 = min(1, groups - 1);
+    u32x4 hraw = load16(p_row), eraw = load16(p_eff);
+    u32x4 wq0 = load16(w_row), wq1 = load16(w_row + 16);
+    uint16_t sg = *reinterpret_cast<const uint16_t *>(s_row), bg = *reinterpret_cast<const uint16_t *>(b_row);
+    u32x4 h1 = load16(p_row + g1 * 64), e1 = load16(p_eff + g1 * 64);
+    u32x4 w10 = load16(w_row + g1 * 64), w11 = load16(w_row + g1 * 64 + 16);
+    uint16_t s1 = *reinterpret_cast<const uint16_t *>(s_row + g1 * 2), b1 = *reinterpret_cast<const uint16_t *>(b_row + g1 * 2);
+    produce(hraw, eraw, 0, 0);
+    lds_barrier();
+    float16_t acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.0f;
+    for (int g = 0; g < groups; ++g) {
+        const int g2 = min(g + 2, groups - 1);
+        const u32x4 h2 = load16(p_row + g2 * 64), e2 = load16(p_eff + g2 * 64);
+        const u32x4 w20 = load16(w_row + g2 * 64), w21 = load16(w_row + g2 * 64 + 16);
+        const uint16_t s2 = *reinterpret_cast<const uint16_t *>(s_row + g2 * 2), b2 = *reinterpret_cast<const uint16_t *>(b_row + g2 * 2);
+        if (kb == 0) bias_h[wave * 32 + i][g] = (half_t)sb_to_f32<SD>(bg);
+        if (wave_live) {
+            const int stage = g & 1;
+            float16_t cg, cl;   // two chains: consecutive MFMAs do not wait for each other
+#pragma unroll
+            for (int r = 0; r < 16; ++r) { cg[r] = 0.0f; cl[r] = 0.0f; }
+#pragma unroll
+            for (int dd = 0; dd < 4; ++dd) {
+                const u32x4 wsrc = dd < 2 ? wq0 : wq1;
+                const half8_t bf = expand8(wsrc[(dd & 1) * 2], wsrc[(dd & 1) * 2 + 1]);
+                const int slot = a_slot(i, kb * 4 + dd);
+                const half8_t ah = __builtin_bit_cast(half8_t, x_hi[stage][slot]);
+                const half8_t al = __builtin_bit_cast(half8_t, x_lo[stage][slot]);
+                cg = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, bf, cg, 0, 0, 0);
+                cl = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, bf, cl, 0, 0, 0);
+            }
+            const float sc = sb_to_f32<SD>(sg) * 0.0625f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[r] = fmaf(sc, cg[r] + cl[r], acc[r]);
+        }
+        if (g + 1 < groups) produce(h1, e1, (g + 1) & 1, g + 1);
+        wq0 = w10; wq1 = w11; sg = s1; bg = b1;
+        h1 = h2; e1 = e2; w10 = w20; w11 = w21; s1 = s2; b1 = b2;
+        lds_barrier();
+    }
+    // bias term: the sums as two fp16 parts (scaled by 16 like x'), the biases as fp16
+    {
+        float v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int g = p_chunk * 8 + j;
+            v[j] = g < groups ? xsum[p_tok][g] * 16.0f : 0.0f;
+        }
+        u32x4 hi, lo;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            half2_t a, b;
+            a[0] = (half_t)v[2 * j];
+            a[1] = (half_t)v[2 * j + 1];
+            b[0] = (half_t)(v[2 * j] - (float)a[0]);
+            b[1] = (half_t)(v[2 * j + 1] - (float)a[1]);
+            hi[j] = as_u32(a);
+            lo[j] = as_u32(b);
+        }
+        g_hi[p_slot] = hi;
+        g_lo[p_slot] = lo;
+    }
+    __syncthreads();
+    if (!wave_live) return;
+    float16_t cb;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) cb[r] = 0.0f;
+    for (int m = 0; m * 16 < groups; ++m) {
+        const half8_t bf = *reinterpret_cast<const half8_t *>(&bias_h[wave * 32 + i][m * 16 + kb * 8]);
+        const int slot = a_slot(i, m * 2 + kb);
+        cb = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, g_hi[slot]), bf, cb, 0, 0, 0);
+        cb = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, g_lo[slot]), bf, cb, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+        const uint32_t t = t0 + (uint32_t)acc_row(r, lane);
+        if (t < query_count && e_lane < num_experts) logits[(size_t)t * num_experts + e_lane] = acc[r] + cb[r] * 0.0625f;
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ device grouping
 // A stable counting sort of the (token, rank) pairs by expert in three short launches.  The tokens are cut into at most
 // kGroupSegments segments.  (1) one wave per segment counts its pairs per expert; (2) one block turns the
@@ -413,8 +570,9 @@ int32_t tf_prefill_router_gemma4_block(tf_ctx *ctx, tf_stream stream, const void
     const bool fast = aligned16(w) && aligned16(h) && aligned16(eff) && hidden_stride_elements % 8 == 0 && d <= 4096;
     const int npass = fast ? (int)((d / 16 + 63) / 64) : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (query_count <= kFewTokens) {
-        const size_t need = (size_t)kFewTokens * 256;
+    const bool mfma_ok = fast && num_experts <= 128 && d <= 4096 && aligned16(w) && d % 64 == 0;
+    if (query_count <= kFewTokens || mfma_ok) {
+        const size_t need = std::max<size_t>((size_t)kFewTokens * 256, (size_t)query_count * num_experts);
         if (ctx->prefill_logits_count < need) {
             if (ctx->prefill_logits) (void)hipFree(ctx->prefill_logits);
             ctx->prefill_logits = nullptr;
@@ -423,18 +581,23 @@ int32_t tf_prefill_router_gemma4_block(tf_ctx *ctx, tf_stream stream, const void
                 return fail(ctx, TF_ERR_OUT_OF_MEMORY, "prefill_router: cannot allocate the logits scratch");
             ctx->prefill_logits_count = need;
         }
-        const dim3 grid((num_experts + 3) / 4, query_count);
+        if (query_count > kFewTokens) {
+            hipLaunchKernelGGL(prefill_logits_mfma_kernel<0>, dim3((query_count + 31) / 32), dim3(256), 0, st, w, s, b, h,
+                               (long)hidden_stride_elements, eff, ctx->prefill_logits, query_count, num_experts, (int)d);
+        } else {
+            const dim3 grid((num_experts + 3) / 4, query_count);
 #define TF_PL(NP_)                                                                                                           \
     hipLaunchKernelGGL(prefill_logits_kernel<NP_>, grid, dim3(256), 0, st, w, s, b, h, (long)hidden_stride_elements, eff,    \
                        ctx->prefill_logits, num_experts, (int)d)
-        switch (npass) {
-            case 1: TF_PL(1); break;
-            case 2: TF_PL(2); break;
-            case 3: TF_PL(3); break;
-            case 4: TF_PL(4); break;
-            default: TF_PL(0); break;
-        }
+            switch (npass) {
+                case 1: TF_PL(1); break;
+                case 2: TF_PL(2); break;
+                case 3: TF_PL(3); break;
+                case 4: TF_PL(4); break;
+                default: TF_PL(0); break;
+            }
 #undef TF_PL
+        }
         const int32_t rc = check_launch(ctx, "prefill_router logits");
         if (rc != TF_OK) return rc;
         hipLaunchKernelGGL(prefill_select_kernel, dim3(query_count), dim3(64), 0, st, ctx->prefill_logits, pes, oi, ow, num_experts, top_k);
