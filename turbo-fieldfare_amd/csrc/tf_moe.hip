@@ -193,17 +193,23 @@ __global__ __launch_bounds__(512) void phase2_short_kernel(RoutedArg routed, tf_
                                                            uint32_t d, uint32_t f) {
     __shared__ float partial[8][2 * NPASS];
     const int lane = threadIdx.x & 63;
-    const uint32_t slot = threadIdx.x >> 6;
+    const uint32_t slot = uniform_u32(threadIdx.x >> 6);
     const long row0 = (long)blockIdx.x * 2 * NPASS;
-    const uint8_t *base = blob_base(routed, slot);
     ShortRows sr;
     ShortRows::Pair t[NPASS];
     sr.init_map(f, lane);
+    // requests in this order: what does not depend on the expert lookup (activations, routing weight), the lookup,
+    // then the weights
+    u32x4 xr[4];
+#pragma unroll
+    for (int dd = 0; dd < 4; ++dd) xr[dd] = load16(acts + (size_t)slot * f + (sr.col < 0 ? 0 : sr.col) * 32 + dd * 8);
+    const half_t w16 = routing_w[slot];
+    const uint8_t *base = uniform_ptr(blob_base(routed, slot));
 #pragma unroll
     for (int p = 0; p < NPASS; ++p)
         sr.load(t[p], base + off.down_W_off, base + off.down_s_off, base + off.down_b_off, row0 + 2 * p, d, f);
-    sr.init_x(acts + (size_t)slot * f);
-    const float w = (float)routing_w[slot];
+    sr.xs = arrange_x(xr, sr.xq);
+    const float w = (float)w16;
 #pragma unroll
     for (int p = 0; p < NPASS; ++p) {
         float lo, hi;

@@ -327,6 +327,74 @@ __global__ __launch_bounds__(64) void group_place_kernel(const uint32_t *indices
     }
 }
 
+// A single segment (at most 32 tokens, the multi-token verification case): the three steps in one 256-thread block.
+__global__ __launch_bounds__(256) void group_small_kernel(const uint32_t *indices, const uint16_t *weights, uint32_t n_pairs,
+                                                          uint32_t top_k, uint32_t num_experts, tf_prefill_pair *sorted_pairs,
+                                                          uint32_t *per_expert_offsets, uint32_t *per_expert_counts,
+                                                          tf_prefill_group *chunks, uint32_t *chunk_count) {
+    __shared__ uint32_t cnt[256], scan_pairs[256], scan_chunks[256], next[256];
+    const uint32_t e = threadIdx.x;
+    cnt[e] = 0;
+    __syncthreads();
+    for (uint32_t i = e; i < n_pairs; i += 256) atomicAdd(&cnt[clamp_expert(indices[i], num_experts)], 1u);
+    __syncthreads();
+    const uint32_t total = cnt[e];
+    const uint32_t nch = (total + kChunkPairs - 1) / kChunkPairs;
+    scan_pairs[e] = total;
+    scan_chunks[e] = nch;
+    __syncthreads();
+    for (uint32_t step = 1; step < 256; step <<= 1) {
+        const uint32_t a = e >= step ? scan_pairs[e - step] : 0u, c = e >= step ? scan_chunks[e - step] : 0u;
+        __syncthreads();
+        scan_pairs[e] += a;
+        scan_chunks[e] += c;
+        __syncthreads();
+    }
+    const uint32_t start = scan_pairs[e] - total, chunk_start = scan_chunks[e] - nch;
+    if (e == 255) chunk_count[0] = scan_chunks[255];
+    if (e < num_experts) {
+        per_expert_offsets[e] = total ? start : 0xFFFFFFFFu;
+        per_expert_counts[e] = total;
+    }
+    for (uint32_t c = 0; c < nch; ++c) {
+        tf_prefill_group g;
+        g.expert = e;
+        g.pair_start = start + c * kChunkPairs;
+        g.pair_count = min(kChunkPairs, total - c * kChunkPairs);
+        chunks[chunk_start + c] = g;
+    }
+    next[e] = start;
+    __syncthreads();
+    if (threadIdx.x >= 64) return;
+    const uint32_t lane = threadIdx.x;
+    const uint64_t below = (1ull << lane) - 1ull;
+    for (uint32_t i0 = 0; i0 < n_pairs; i0 += 64) {
+        const uint32_t i = i0 + lane;
+        const bool valid = i < n_pairs;
+        const uint32_t x = valid ? clamp_expert(indices[i], num_experts) : 0xFFFFFFFFu;
+        const uint16_t wbits = valid ? weights[i] : (uint16_t)0;
+        uint64_t remaining = __ballot(valid);
+        uint32_t pos = 0;
+        while (remaining) {
+            const int leader = __builtin_ctzll(remaining);
+            const uint32_t v = (uint32_t)__builtin_amdgcn_readlane((int)x, leader);
+            const uint64_t same = __ballot(x == v);
+            const uint32_t at = next[v];
+            if (x == v) pos = at + (uint32_t)__builtin_popcountll(same & below);
+            if ((int)lane == leader) next[v] = at + (uint32_t)__builtin_popcountll(same);
+            remaining &= ~same;
+        }
+        if (valid) {
+            tf_prefill_pair p;
+            p.token = i / top_k;
+            p.expert = x;
+            p.rank = i - p.token * top_k;
+            p.weight_bits_and_reserved = (uint32_t)wbits;
+            sorted_pairs[pos] = p;
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------ grouped, row-streaming
 // Small groups: a wave loads one tile of gate rows and the same tile of up rows ONCE and applies it to every pair of the
 // chunk, so each touched expert is read once however many tokens chose it.
@@ -713,6 +781,13 @@ int32_t tf_prefill_group_pairs_device(tf_ctx *ctx, tf_stream stream, const void 
     const uint32_t n_segments = (query_count + seg_tokens - 1) / seg_tokens;
     const uint32_t seg_pairs = seg_tokens * top_k;
     const uint32_t *idx = static_cast<const uint32_t *>(indices);
+    if (n_segments == 1) {
+        hipLaunchKernelGGL(group_small_kernel, dim3(1), dim3(256), 0, st, idx, static_cast<const uint16_t *>(weights), n_pairs, top_k,
+                           num_experts, static_cast<tf_prefill_pair *>(sorted_pairs), static_cast<uint32_t *>(per_expert_offsets),
+                           static_cast<uint32_t *>(per_expert_counts), static_cast<tf_prefill_group *>(chunks),
+                           static_cast<uint32_t *>(chunk_count));
+        return check_launch(ctx, "group_pairs_device");
+    }
     hipLaunchKernelGGL(group_count_kernel, dim3(n_segments), dim3(64), 0, st, idx, n_pairs, seg_pairs, num_experts, ctx->group_scratch);
     hipLaunchKernelGGL(group_scan_kernel, dim3(1), dim3(256), 0, st, ctx->group_scratch, n_segments, num_experts,
                        static_cast<uint32_t *>(per_expert_offsets), static_cast<uint32_t *>(per_expert_counts),
