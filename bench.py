@@ -33,9 +33,9 @@ def int4_matrix_bytes(rows, cols):
 
 # per-unit algorithmic bytes (what one launch must move at least once)
 ROUTER_BYTES = E * D + 2 * E * (D // 64) * 2 + D * 2 + D * 2 + E * 2 + TOPK * 4 + TOPK * 2   # W + s/b + hidden + eff + gains + outputs
-# HBM bytes one phase-1 launch moves, from hardware counters (profiles/bench_hbm_traffic_counters.txt): FETCH_SIZE 8875.6 KiB
-# x 2.0 (the factor a plain 1 GiB copy calibrates) + WRITE_SIZE 22.0 KiB x 1.0.
-PHASE1_TRAFFIC_BYTES = int(8875.6 * 1024 * 1.9999 + 22.0 * 1024)
+# HBM bytes one phase-1 launch moves, from hardware counters (profiles/bench_hbm_traffic_counters.txt): FETCH_SIZE 8895.6 KiB
+# x 2.0 (the factor a plain 1 GiB copy calibrates) + WRITE_SIZE 22.1 KiB x 1.0.
+PHASE1_TRAFFIC_BYTES = int(8895.6 * 1024 * 1.9999 + 22.1 * 1024)
 PHASE1_BYTES = TOPK * 2 * int4_matrix_bytes(F_MOE, D) + D * 2 + TOPK * F_MOE * 2             # gate+up of 8 experts + x + acts out
 PHASE2_BYTES = TOPK * int4_matrix_bytes(D, F_MOE) + TOPK * F_MOE * 2 + TOPK * 2 + D * 2 + D * 2   # down of 8 + acts in + w + residual + y
 STEP_BYTES = ROUTER_BYTES + PHASE1_BYTES + PHASE2_BYTES
