@@ -161,6 +161,42 @@ int32_t tf_rmsnorm_bf16w(tf_ctx *ctx, tf_stream stream,
                          const void *x, uint64_t x_offset, const void *weight, uint64_t weight_offset,
                          void *out, uint64_t out_offset, uint32_t d, float eps);
 
+/* ---- the stages either side of the MoE block ------------------------------------------------------------------- */
+/* FusedPostAttentionSetup.encode (Kernels/Fusions/FusedPostAttentionSetup.swift:19-56) -> fused_post_attn_setup
+ * (Metal/Fusions/fused.metal:190-269).  All activations fp16[d], weights bf16[d], d <= 4096:
+ *   hidden   <- half(hidden + half(attn * rsqrt(mean(attn^2) + eps) * post_attention_weight))      (in place)
+ *   h         = hidden * rsqrt(mean(hidden^2) + eps)
+ *   dense_x   = half(h * pre_ffn_weight),  routed_x = half(h * pre_ffn2_weight),  router_x = half(h). */
+int32_t tf_fused_post_attn_setup(tf_ctx *ctx, tf_stream stream, void *hidden, const void *attn, void *dense_x, void *routed_x,
+                                 void *router_x, const void *post_attention_weight, uint64_t post_attention_weight_offset,
+                                 const void *pre_ffn_weight, uint64_t pre_ffn_weight_offset, const void *pre_ffn2_weight,
+                                 uint64_t pre_ffn2_weight_offset, uint32_t d, float eps);
+/* PrefillPostAttentionSetup.encode (Kernels/Prefill/Epilogues/PrefillPostAttentionSetup.swift:11-74) ->
+ * prefill_post_attn_setup_block (Metal/Prefill/prefill.metal:178-253): the same for query_count rows, row r of each
+ * operand at r * its stride (in elements, >= d); bytes between rows are left untouched. */
+int32_t tf_prefill_post_attn_setup_block(tf_ctx *ctx, tf_stream stream, void *hidden, uint64_t hidden_offset, const void *attn,
+                                         uint64_t attn_offset, void *dense_x, uint64_t dense_x_offset, void *routed_x,
+                                         uint64_t routed_x_offset, void *router_x, uint64_t router_x_offset,
+                                         const void *post_attention_weight, uint64_t post_attention_weight_offset,
+                                         const void *pre_ffn_weight, uint64_t pre_ffn_weight_offset, const void *pre_ffn2_weight,
+                                         uint64_t pre_ffn2_weight_offset, uint32_t query_count, uint32_t d,
+                                         uint32_t hidden_stride_elements, uint32_t attn_stride_elements,
+                                         uint32_t dense_stride_elements, uint32_t routed_stride_elements,
+                                         uint32_t router_stride_elements, float eps);
+/* FusedLayerTail.encode (Kernels/Fusions/FusedLayerTail.swift:19-52) -> fused_layer_tail (Metal/Fusions/fused.metal:271-375):
+ *   h12     = half(h1 + half(h2 * rsqrt(mean(h2^2) + eps) * post_ffn2_weight))
+ *   hidden <- half(half(hidden + half(h12 * rsqrt(mean(h12^2) + eps) * post_ffn_weight)) * half(layer_scalar))   (in place) */
+int32_t tf_fused_layer_tail(tf_ctx *ctx, tf_stream stream, const void *h2, const void *h1, void *hidden, const void *post_ffn2_weight,
+                            uint64_t post_ffn2_weight_offset, const void *post_ffn_weight, uint64_t post_ffn_weight_offset, uint32_t d,
+                            float eps, float layer_scalar);
+/* PrefillLayerTail.encode (Kernels/Prefill/Epilogues/PrefillLayerTail.swift:11-60) -> prefill_layer_tail_block
+ * (Metal/Prefill/prefill.metal:255-334): the same for query_count strided rows. */
+int32_t tf_prefill_layer_tail_block(tf_ctx *ctx, tf_stream stream, const void *h2, uint64_t h2_offset, const void *h1,
+                                    uint64_t h1_offset, void *hidden, uint64_t hidden_offset, const void *post_ffn2_weight,
+                                    uint64_t post_ffn2_weight_offset, const void *post_ffn_weight, uint64_t post_ffn_weight_offset,
+                                    uint32_t query_count, uint32_t d, uint32_t h2_stride_elements, uint32_t h1_stride_elements,
+                                    uint32_t hidden_stride_elements, float eps, float layer_scalar);
+
 /* ---- shared expert ------------------------------------------------------------------------------------------- */
 /* SharedExpertInt4.encode (Kernels/MoE/SharedExpertInt4.swift:31-99): gate GEMV, up GEMV (fp16 out),
  * gelu_mul_fp16, down GEMV.  Scratch sizes are in BYTES (the MTLBuffer.length checks at :46-58); each must hold

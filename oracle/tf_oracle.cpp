@@ -731,6 +731,82 @@ void tfo_k_rmsnorm_bf16w(const uint16_t *x_f16, const uint16_t *w_bf16, float ep
         out_f16[i] = tfo_f16_bits(tfo_f16_to_float(x_f16[i]) * inv * tfo_bf16_to_float(w_bf16[i]));
 }
 
+// Sum of squares of d fp16 values in the order of the reference's 256-thread, 32-lane two-stage reduction
+// (M/Fusions/fused.metal:217-235): strided per-thread fma chains, lane sums, then the per-group partials.
+static float k_block_sum_squares(const uint16_t *x_f16, int d) {
+    float partial[256];
+    for (int lid = 0; lid < 256; ++lid) {
+        float acc = 0.0f;
+        for (int i = lid; i < d; i += 256) { const float v = tfo_f16_to_float(x_f16[i]); acc = fmaf(v, v, acc); }
+        partial[lid] = acc;
+    }
+    float total = 0.0f;
+    for (int sg = 0; sg < 8; ++sg) {
+        float s = 0.0f;
+        for (int lane = 0; lane < 32; ++lane) s += partial[sg * 32 + lane];
+        total += s;
+    }
+    return total;
+}
+
+// M/Fusions/fused.metal:190-269 (fused_post_attn_setup) and its per-row twin M/Prefill/prefill.metal:178-253:
+// hidden += rmsnorm(attn, w_post_attn) rounded to fp16 at each stage; then the three views of rmsnorm(hidden).
+void tfo_k_post_attn_setup(uint16_t *hidden_f16, const uint16_t *attn_f16, const uint16_t *w_post_attn_bf16,
+                           const uint16_t *w_pre_ffn_bf16, const uint16_t *w_pre_ffn2_bf16, float eps, uint16_t *dense_f16,
+                           uint16_t *routed_f16, uint16_t *router_f16, int d) {
+    const float attn_inv = 1.0f / std::sqrt(k_block_sum_squares(attn_f16, d) / (float)d + eps);
+    for (int i = 0; i < d; ++i) {
+        const uint16_t an = tfo_f16_bits(tfo_f16_to_float(attn_f16[i]) * attn_inv * tfo_bf16_to_float(w_post_attn_bf16[i]));
+        hidden_f16[i] = tfo_f16_bits(tfo_f16_to_float(hidden_f16[i]) + tfo_f16_to_float(an));
+    }
+    const float hidden_inv = 1.0f / std::sqrt(k_block_sum_squares(hidden_f16, d) / (float)d + eps);
+    for (int i = 0; i < d; ++i) {
+        const float h = tfo_f16_to_float(hidden_f16[i]) * hidden_inv;
+        dense_f16[i] = tfo_f16_bits(h * tfo_bf16_to_float(w_pre_ffn_bf16[i]));
+        routed_f16[i] = tfo_f16_bits(h * tfo_bf16_to_float(w_pre_ffn2_bf16[i]));
+        router_f16[i] = tfo_f16_bits(h);
+    }
+}
+
+// M/Fusions/fused.metal:271-375 (fused_layer_tail) and M/Prefill/prefill.metal:255-334:
+// hidden = half(half(hidden + rmsnorm(h1 + rmsnorm(h2, w_postffn2), w_postffn)) * half(layer_scalar)), fp16 at every stage.
+void tfo_k_layer_tail(const uint16_t *h2_f16, const uint16_t *h1_f16, uint16_t *hidden_f16, const uint16_t *w_postffn2_bf16,
+                      const uint16_t *w_postffn_bf16, float eps, float layer_scalar, int d) {
+    std::vector<uint16_t> h12(d);
+    const float inv_h2 = 1.0f / std::sqrt(k_block_sum_squares(h2_f16, d) / (float)d + eps);
+    for (int i = 0; i < d; ++i) {
+        const uint16_t t = tfo_f16_bits(tfo_f16_to_float(h2_f16[i]) * inv_h2 * tfo_bf16_to_float(w_postffn2_bf16[i]));
+        h12[i] = tfo_f16_bits(tfo_f16_to_float(h1_f16[i]) + tfo_f16_to_float(t));
+    }
+    const float inv_h12 = 1.0f / std::sqrt(k_block_sum_squares(h12.data(), d) / (float)d + eps);
+    const float scale = tfo_f16_to_float(tfo_f16_bits(layer_scalar));
+    for (int i = 0; i < d; ++i) {
+        const uint16_t t = tfo_f16_bits(tfo_f16_to_float(h12[i]) * inv_h12 * tfo_bf16_to_float(w_postffn_bf16[i]));
+        const uint16_t sum = tfo_f16_bits(tfo_f16_to_float(hidden_f16[i]) + tfo_f16_to_float(t));
+        hidden_f16[i] = tfo_f16_bits(tfo_f16_to_float(sum) * scale);
+    }
+}
+
+// T/Core/Kernels/Fusions/FusedLayerTailTests.swift:76-92 (cpuReference): the same chain through the fp32 RmsNorm reference.
+void tfo_layer_tail_ref(const uint16_t *h2_f16, const uint16_t *h1_f16, const uint16_t *hidden_f16, const uint16_t *w_postffn2_bf16,
+                        const uint16_t *w_postffn_bf16, float eps, float layer_scalar, float *out, int d) {
+    std::vector<float> x(d), w2(d), w(d), n(d), h12(d);
+    for (int i = 0; i < d; ++i) {
+        x[i] = tfo_f16_to_float(h2_f16[i]);
+        w2[i] = tfo_bf16_to_float(w_postffn2_bf16[i]);
+        w[i] = tfo_bf16_to_float(w_postffn_bf16[i]);
+    }
+    tfo_rmsnorm_ref(x.data(), w2.data(), eps, n.data(), d);
+    for (int i = 0; i < d; ++i)
+        h12[i] = tfo_f16_to_float(tfo_f16_bits(tfo_f16_to_float(h1_f16[i]) + tfo_f16_to_float(tfo_f16_bits(n[i]))));
+    tfo_rmsnorm_ref(h12.data(), w.data(), eps, n.data(), d);
+    const float scale = tfo_f16_to_float(tfo_f16_bits(layer_scalar));
+    for (int i = 0; i < d; ++i) {
+        const float sum = tfo_f16_to_float(tfo_f16_bits(tfo_f16_to_float(hidden_f16[i]) + tfo_f16_to_float(tfo_f16_bits(n[i]))));
+        out[i] = tfo_f16_to_float(tfo_f16_bits(sum * scale));
+    }
+}
+
 void tfo_k_prefill_router_logits(const uint8_t *W, const uint16_t *S, const uint16_t *B, const uint16_t *hidden_f16,
                                  const uint16_t *eff_scale_bf16, float *logits, int num_experts, int d) {
     const int groups = d / G;

@@ -178,6 +178,13 @@ void tfo_k_moe_phase2(const uint8_t *const *blobs, const tfo_expert_offsets *off
                       const uint16_t *routing_w_f16, const uint16_t *residual_f16, uint16_t *y_f16,
                       int d, int f);                                            /* M/MoE/moe.metal:446-482 */
 void tfo_k_gelu_mul_fp16(const uint16_t *gate_f16, const uint16_t *up_f16, uint16_t *out_f16, int n); /* M/Primitives/utility.metal:6-18 */
+void tfo_k_post_attn_setup(uint16_t *hidden_f16, const uint16_t *attn_f16, const uint16_t *w_post_attn_bf16,
+                           const uint16_t *w_pre_ffn_bf16, const uint16_t *w_pre_ffn2_bf16, float eps, uint16_t *dense_f16,
+                           uint16_t *routed_f16, uint16_t *router_f16, int d); /* M/Fusions/fused.metal:190-269 */
+void tfo_k_layer_tail(const uint16_t *h2_f16, const uint16_t *h1_f16, uint16_t *hidden_f16, const uint16_t *w_postffn2_bf16,
+                      const uint16_t *w_postffn_bf16, float eps, float layer_scalar, int d); /* M/Fusions/fused.metal:271-375 */
+void tfo_layer_tail_ref(const uint16_t *h2_f16, const uint16_t *h1_f16, const uint16_t *hidden_f16, const uint16_t *w_postffn2_bf16,
+                        const uint16_t *w_postffn_bf16, float eps, float layer_scalar, float *out, int d); /* T/Core/Kernels/Fusions/FusedLayerTailTests.swift:76-92 */
 void tfo_k_rmsnorm_bf16w(const uint16_t *x_f16, const uint16_t *w_bf16, float eps, uint16_t *out_f16, int d); /* M/Primitives/rmsnorm.metal:32-93 */
 void tfo_k_prefill_router_logits(const uint8_t *W, const uint16_t *S, const uint16_t *B, const uint16_t *hidden_f16,
                                  const uint16_t *eff_scale_bf16, float *logits, int num_experts, int d); /* M/Prefill/prefill.metal:503-525 */

@@ -307,6 +307,38 @@ def k_rmsnorm_bf16w(x_bits, w_bits, eps: float) -> np.ndarray:
     return out
 
 
+_sig("tfo_k_post_attn_setup", None, u16p, u16p, u16p, u16p, u16p, C.c_float, u16p, u16p, u16p, i32)
+_sig("tfo_k_layer_tail", None, u16p, u16p, u16p, u16p, u16p, C.c_float, C.c_float, i32)
+_sig("tfo_layer_tail_ref", None, u16p, u16p, u16p, u16p, u16p, C.c_float, C.c_float, f32p, i32)
+
+
+def _u16(a):
+    return np.ascontiguousarray(a, np.uint16)
+
+
+def k_post_attn_setup(hidden_bits, attn_bits, w_post_bits, w_pre_bits, w_pre2_bits, eps: float):
+    """-> (hidden', dense_x, routed_x, router_x) as fp16 bit arrays (fused.metal:190-269)."""
+    hidden = _u16(hidden_bits).copy()
+    dense, routed, router = np.empty_like(hidden), np.empty_like(hidden), np.empty_like(hidden)
+    lib.tfo_k_post_attn_setup(hidden, _u16(attn_bits), _u16(w_post_bits), _u16(w_pre_bits), _u16(w_pre2_bits), eps, dense, routed,
+                              router, hidden.size)
+    return hidden, dense, routed, router
+
+
+def k_layer_tail(h2_bits, h1_bits, hidden_bits, w_postffn2_bits, w_postffn_bits, eps: float, layer_scalar: float) -> np.ndarray:
+    hidden = _u16(hidden_bits).copy()
+    lib.tfo_k_layer_tail(_u16(h2_bits), _u16(h1_bits), hidden, _u16(w_postffn2_bits), _u16(w_postffn_bits), eps, layer_scalar, hidden.size)
+    return hidden
+
+
+def layer_tail_ref(h2_bits, h1_bits, hidden_bits, w_postffn2_bits, w_postffn_bits, eps: float, layer_scalar: float) -> np.ndarray:
+    hidden = _u16(hidden_bits)
+    out = np.empty(hidden.size, np.float32)
+    lib.tfo_layer_tail_ref(_u16(h2_bits), _u16(h1_bits), hidden, _u16(w_postffn2_bits), _u16(w_postffn_bits), eps, layer_scalar, out,
+                           hidden.size)
+    return out
+
+
 # ---- MoE ---------------------------------------------------------------------------------
 _pp = C.POINTER(C.c_void_p)
 _sig("tfo_moe_run_ffn", None, C.c_void_p, C.POINTER(ExpertOffsets), f32p, f32p, i32, i32)

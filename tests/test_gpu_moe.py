@@ -265,35 +265,60 @@ def _decode_step_case(d, f, num_experts, seed):
                 residual_bits=refcases.normal_f16(d, seed + 9))
 
 
-@pytest.mark.parametrize("d,f,num_experts", [(2816, 704, 16), (2816, 128, 128), (704, 128, 16)])
-def test_decode_step_equals_router_then_phases_and_the_reference(d, f, num_experts):
+def _decode_step_call(k, t, c, d, f, num_experts, outs):
+    idx, wts, acts, y = outs
+    off = tfk.ExpertOffsets(*c["off"].as_tuple())
+    return k.lib.tf_moe_decode_step(k.handle, None, t["rW"].data_ptr(), 0, t["rS"].data_ptr(), 0, t["rB"].data_ptr(), 0, t["x"].data_ptr(),
+                                    t["eff"].data_ptr(), 0, t["gain"].data_ptr(), 0, t["pool"].data_ptr(), c["stride"], num_experts,
+                                    off, t["x"].data_ptr(), acts.data_ptr(), t["res"].data_ptr(), y.data_ptr(), idx.data_ptr(),
+                                    wts.data_ptr(), d, f, 8, tfk.TF_BF16)
+
+
+def _decode_step_tensors(c):
+    return dict(pool=dev(c["pool"]), rW=dev(c["rW"]), rS=dev(c["rS"]), rB=dev(c["rB"]), eff=dev(c["eff_bits"]), gain=dev(c["gain_bits"]),
+                x=dev(c["x_bits"]), res=dev(c["residual_bits"]))
+
+
+def _fresh_outs(d, f):
+    return zeros_bytes(32), zeros_bytes(16), zeros_bytes(8 * f * 2), zeros_bytes(d * 2)
+
+
+def _read_outs(outs, d, f):
+    idx, wts, acts, y = outs
+    return host(idx, np.uint32, 8), host(wts, np.uint16, 8), host(acts, np.uint16, 8 * f), host(y, np.uint16, d)
+
+
+# (2816, 704, 128) is the production shape
+@pytest.mark.parametrize("d,f,num_experts", [(2816, 704, 128), (2816, 704, 16), (3072, 128, 200), (2816, 128, 128), (704, 128, 16)])
+@pytest.mark.parametrize("mode", ["default", "timed"])
+def test_decode_step_equals_router_then_phases_and_the_reference(d, f, num_experts, mode):
     # one call (selection repeated inside phase 1 when the vector path applies) against the three wrapper calls of the
-    # reference runner (RealForwardRunner.swift:1462-1685): bitwise the same indices, weights, activations and output
+    # reference runner (RealForwardRunner.swift:1462-1685): bitwise the same indices, weights, activations and output;
+    # "timed" also brackets the three launches with events
     import torch
     c = _decode_step_case(d, f, num_experts, 0x5EED + d + f)
     k = ctx()
     off = tfk.ExpertOffsets(*c["off"].as_tuple())
-    pool, rW, rS, rB = dev(c["pool"]), dev(c["rW"]), dev(c["rS"]), dev(c["rB"])
-    eff, gain, x, res = dev(c["eff_bits"]), dev(c["gain_bits"]), dev(c["x_bits"]), dev(c["residual_bits"])
+    t = _decode_step_tensors(c)
     outs = []
     for fused in (True, False):
-        idx, wts, acts, y = zeros_bytes(32), zeros_bytes(16), zeros_bytes(8 * f * 2), zeros_bytes(d * 2)
+        o = _fresh_outs(d, f)
+        idx, wts, acts, y = o
         if fused:
-            k.set_step_timing(True)
-            k.check(k.lib.tf_moe_decode_step(k.handle, None, rW.data_ptr(), 0, rS.data_ptr(), 0, rB.data_ptr(), 0, x.data_ptr(),
-                                             eff.data_ptr(), 0, gain.data_ptr(), 0, pool.data_ptr(), c["stride"], num_experts,
-                                             off, x.data_ptr(), acts.data_ptr(), res.data_ptr(), y.data_ptr(), idx.data_ptr(),
-                                             wts.data_ptr(), d, f, 8, tfk.TF_BF16))
-            times = k.last_step_timing()
+            k.set_step_timing(mode == "timed")
+            k.check(_decode_step_call(k, t, c, d, f, num_experts, o))
+            if mode == "timed":
+                times = k.last_step_timing()
+                assert len(times) == 4 and all(0.0 <= v < 5e4 for v in times) and min(times[:3]) > 0.0
             k.set_step_timing(False)
-            assert len(times) == 4 and all(0.0 <= t < 5e4 for t in times) and min(times[:3]) > 0.0
+            k.synchronize()
         else:
-            k.router_gemma4(rW, rS, rB, x, eff, gain, idx, wts, num_experts, d)
-            routed = k.routed_from_pool(pool, c["stride"], idx, num_experts)
-            k.moe_phase1(routed, off, x, acts, d, f)
-            k.moe_phase2(routed, off, acts, wts, res, y, d, f)
+            k.router_gemma4(t["rW"], t["rS"], t["rB"], t["x"], t["eff"], t["gain"], idx, wts, num_experts, d)
+            routed = k.routed_from_pool(t["pool"], c["stride"], idx, num_experts)
+            k.moe_phase1(routed, off, t["x"], acts, d, f)
+            k.moe_phase2(routed, off, acts, wts, t["res"], y, d, f)
         torch.cuda.synchronize()
-        outs.append((host(idx, np.uint32, 8), host(wts, np.uint16, 8), host(acts, np.uint16, 8 * f), host(y, np.uint16, d)))
+        outs.append(_read_outs(o, d, f))
     for a, b in zip(outs[0], outs[1]):
         assert np.array_equal(a, b)
     got_idx, got_w_bits, _, got_y = outs[0]
@@ -303,6 +328,70 @@ def test_decode_step_equals_router_then_phases_and_the_reference(d, f, num_exper
     expected = tfo.moe_apply_streamed_routed([c["blobs"][e] for e in got_idx], c["off"], tfo.from_f16_bits(c["x_bits"]),
                                              tfo.from_f16_bits(c["residual_bits"]), tfo.from_f16_bits(got_w_bits), d, f, threads=8)
     assert within_north_star(tfo.from_f16_bits(got_y), expected, abs_=1e-3 * max(1.0, float(np.max(np.abs(expected)))))
+    logits = device_view(k.router_logits_ptr(), num_experts, "<f4")
+    assert tfo.rel_error(logits, tfo.router_reference(c["rW"], c["rS"], c["rB"], tfo.from_f16_bits(c["x_bits"]),
+                                                      tfo.bf16_array_to_float(c["eff_bits"]), tfo.bf16_array_to_float(c["gain_bits"]))[2]) < 1e-4
+
+
+def test_decode_steps_back_to_back_and_replayed_from_a_graph():
+    # many steps in a row on one stream with changing activations and no host wait in between: every step must see its own
+    # router result (logits and indices pass through device memory); then the same from a captured graph, replayed
+    import torch
+    d, f, num_experts, steps = 2816, 704, 128, 12
+    c = _decode_step_case(d, f, num_experts, 0xBEE5)
+    k = ctx()
+    t = _decode_step_tensors(c)
+    rng = np.random.default_rng(0xBEE5)
+    xs = [dev(rng.standard_normal(d).astype(np.float16).view(np.uint16)) for _ in range(steps)]
+    want = []
+    off = tfk.ExpertOffsets(*c["off"].as_tuple())
+    for i in range(steps):          # expected: the three wrapper calls, one step at a time
+        o = _fresh_outs(d, f)
+        idx, wts, acts, y = o
+        k.router_gemma4(t["rW"], t["rS"], t["rB"], xs[i], t["eff"], t["gain"], idx, wts, num_experts, d)
+        routed = k.routed_from_pool(t["pool"], c["stride"], idx, num_experts)
+        k.moe_phase1(routed, off, xs[i], acts, d, f)
+        k.moe_phase2(routed, off, acts, wts, t["res"], y, d, f)
+        want.append(_read_outs(o, d, f))
+    outs = [_fresh_outs(d, f) for _ in range(steps)]
+    for i in range(steps):
+        t["x"] = xs[i]
+        k.check(_decode_step_call(k, t, c, d, f, num_experts, outs[i]))
+    k.synchronize()
+    for i in range(steps):
+        for a, b in zip(_read_outs(outs[i], d, f), want[i]):
+            assert np.array_equal(a, b), i
+    assert len({tuple(w[0]) for w in want}) > 1      # the steps really chose different experts
+    # graph: capture 4 steps on a side stream, replay three times with eager work between the replays
+    side = torch.cuda.Stream()
+    gouts = [_fresh_outs(d, f) for _ in range(4)]
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            for i in range(4):
+                t["x"] = xs[i]
+                idx, wts, acts, y = gouts[i]
+                off = tfk.ExpertOffsets(*c["off"].as_tuple())
+                k.check(k.lib.tf_moe_decode_step(k.handle, side.cuda_stream, t["rW"].data_ptr(), 0, t["rS"].data_ptr(), 0, t["rB"].data_ptr(), 0,
+                                                 t["x"].data_ptr(), t["eff"].data_ptr(), 0, t["gain"].data_ptr(), 0, t["pool"].data_ptr(),
+                                                 c["stride"], num_experts, off, t["x"].data_ptr(), acts.data_ptr(), t["res"].data_ptr(),
+                                                 y.data_ptr(), idx.data_ptr(), wts.data_ptr(), d, f, 8, tfk.TF_BF16))
+    for replay in range(3):
+        for o in gouts:
+            for buf in o:
+                buf.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for i in range(4):
+            for a, b in zip(_read_outs(gouts[i], d, f), want[i]):
+                assert np.array_equal(a, b), (replay, i)
+        t["x"] = xs[5 + replay]                       # an eager step between the replays
+        o = _fresh_outs(d, f)
+        k.check(_decode_step_call(k, t, c, d, f, num_experts, o))
+        k.synchronize()
+        for a, b in zip(_read_outs(o, d, f), want[5 + replay]):
+            assert np.array_equal(a, b)
 
 
 def test_step_timing_needs_a_recorded_step():

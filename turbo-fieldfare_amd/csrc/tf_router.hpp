@@ -80,17 +80,11 @@ __device__ __forceinline__ float router_row(const uint8_t *w_row, const uint8_t 
 // its lowest expert index with ballots, so a round is a few dozen ALU instructions and no memory traffic.
 // router_select_lanes leaves selection i in lane i (i < top_k): its expert index and its routing weight.
 // NC = candidates per lane: 2 serves up to 128 experts, 4 up to 256.
+// router_select_core: the same on candidates already in registers (cand[j] = logit of expert lane + 64 j, -inf where
+// there is no such expert or the logit is NaN; gain[j] its per-expert gain).  cand is consumed.
 template <int NC>
-__device__ __forceinline__ void router_select_lanes(const float *logits, const uint16_t *per_expert_scale, uint32_t num_experts,
-                                                    uint32_t top_k, int lane, uint32_t &sel_index, half_t &sel_weight) {
-    float cand[NC], gain[NC];
-#pragma unroll
-    for (int j = 0; j < NC; ++j) {
-        const uint32_t e = lane + 64 * j;
-        const float v = e < num_experts ? logits[e] : -INFINITY;
-        gain[j] = e < num_experts ? bf16_to_f32(per_expert_scale[e]) : 0.0f;
-        cand[j] = (v != v) ? -INFINITY : v;
-    }
+__device__ __forceinline__ void router_select_core(float (&cand)[NC], const float (&gain)[NC], uint32_t top_k, int lane,
+                                                   uint32_t &sel_index, half_t &sel_weight) {
     float my_score = -INFINITY, my_gain = 0.0f;   // lane i (< top_k) ends up holding the i-th selection
     uint32_t my_idx = 0;
     for (uint32_t i = 0; i < top_k; ++i) {
@@ -126,6 +120,20 @@ __device__ __forceinline__ void router_select_lanes(const float *logits, const u
     for (uint32_t i = 0; i < top_k; ++i) sum_exp += read_lane(ex, (int)i);
     sel_index = my_idx;
     sel_weight = (half_t)((ex / sum_exp) * my_gain);
+}
+
+template <int NC>
+__device__ __forceinline__ void router_select_lanes(const float *logits, const uint16_t *per_expert_scale, uint32_t num_experts,
+                                                    uint32_t top_k, int lane, uint32_t &sel_index, half_t &sel_weight) {
+    float cand[NC], gain[NC];
+#pragma unroll
+    for (int j = 0; j < NC; ++j) {
+        const uint32_t e = lane + 64 * j;
+        const float v = e < num_experts ? logits[e] : -INFINITY;
+        gain[j] = e < num_experts ? bf16_to_f32(per_expert_scale[e]) : 0.0f;
+        cand[j] = (v != v) ? -INFINITY : v;
+    }
+    router_select_core<NC>(cand, gain, top_k, lane, sel_index, sel_weight);
 }
 
 __device__ __forceinline__ void router_select_lanes(const float *logits, const uint16_t *per_expert_scale, uint32_t num_experts,

@@ -276,6 +276,75 @@ private:
     const Context &c_;
 };
 
+
+// FusedPostAttentionSetup (Kernels/Fusions/FusedPostAttentionSetup.swift)
+class FusedPostAttentionSetup {
+public:
+    explicit FusedPostAttentionSetup(const Context &context) : c_(context) {}
+    void encode(void *hidden, const void *attn, void *denseX, void *routedX, void *routerX, const void *postAttentionWeight,
+                uint64_t postAttentionWeightOffset, const void *preFFNWeight, uint64_t preFFNWeightOffset, const void *preFFN2Weight,
+                uint64_t preFFN2WeightOffset, uint32_t d, float eps) const {
+        c_.check(tf_fused_post_attn_setup(c_.raw(), c_.stream(), hidden, attn, denseX, routedX, routerX, postAttentionWeight,
+                                          postAttentionWeightOffset, preFFNWeight, preFFNWeightOffset, preFFN2Weight, preFFN2WeightOffset,
+                                          d, eps));
+    }
+
+private:
+    const Context &c_;
+};
+
+// FusedLayerTail (Kernels/Fusions/FusedLayerTail.swift)
+class FusedLayerTail {
+public:
+    explicit FusedLayerTail(const Context &context) : c_(context) {}
+    void encode(const void *h2, const void *h1, void *hidden, const void *postFFN2Weight, uint64_t postFFN2WeightOffset,
+                const void *postFFNWeight, uint64_t postFFNWeightOffset, uint32_t d, float eps, float layerScalar) const {
+        c_.check(tf_fused_layer_tail(c_.raw(), c_.stream(), h2, h1, hidden, postFFN2Weight, postFFN2WeightOffset, postFFNWeight,
+                                     postFFNWeightOffset, d, eps, layerScalar));
+    }
+
+private:
+    const Context &c_;
+};
+
+// PrefillPostAttentionSetup (Kernels/Prefill/Epilogues/PrefillPostAttentionSetup.swift)
+class PrefillPostAttentionSetup {
+public:
+    explicit PrefillPostAttentionSetup(const Context &context) : c_(context) {}
+    void encode(void *hidden, uint64_t hiddenOffset, const void *attn, uint64_t attnOffset, void *denseX, uint64_t denseXOffset,
+                void *routedX, uint64_t routedXOffset, void *routerX, uint64_t routerXOffset, const void *postAttentionWeight,
+                uint64_t postAttentionWeightOffset, const void *preFFNWeight, uint64_t preFFNWeightOffset, const void *preFFN2Weight,
+                uint64_t preFFN2WeightOffset, uint32_t queryCount, uint32_t d, uint32_t hiddenStrideElements,
+                uint32_t attnStrideElements, uint32_t denseStrideElements, uint32_t routedStrideElements,
+                uint32_t routerStrideElements, float eps) const {
+        c_.check(tf_prefill_post_attn_setup_block(c_.raw(), c_.stream(), hidden, hiddenOffset, attn, attnOffset, denseX, denseXOffset,
+                                                  routedX, routedXOffset, routerX, routerXOffset, postAttentionWeight,
+                                                  postAttentionWeightOffset, preFFNWeight, preFFNWeightOffset, preFFN2Weight,
+                                                  preFFN2WeightOffset, queryCount, d, hiddenStrideElements, attnStrideElements,
+                                                  denseStrideElements, routedStrideElements, routerStrideElements, eps));
+    }
+
+private:
+    const Context &c_;
+};
+
+// PrefillLayerTail (Kernels/Prefill/Epilogues/PrefillLayerTail.swift)
+class PrefillLayerTail {
+public:
+    explicit PrefillLayerTail(const Context &context) : c_(context) {}
+    void encode(const void *h2, uint64_t h2Offset, const void *h1, uint64_t h1Offset, void *hidden, uint64_t hiddenOffset,
+                const void *postFFN2Weight, uint64_t postFFN2WeightOffset, const void *postFFNWeight, uint64_t postFFNWeightOffset,
+                uint32_t queryCount, uint32_t d, uint32_t h2StrideElements, uint32_t h1StrideElements, uint32_t hiddenStrideElements,
+                float eps, float layerScalar) const {
+        c_.check(tf_prefill_layer_tail_block(c_.raw(), c_.stream(), h2, h2Offset, h1, h1Offset, hidden, hiddenOffset, postFFN2Weight,
+                                             postFFN2WeightOffset, postFFNWeight, postFFNWeightOffset, queryCount, d, h2StrideElements,
+                                             h1StrideElements, hiddenStrideElements, eps, layerScalar));
+    }
+
+private:
+    const Context &c_;
+};
+
 // MPPPrefillInt4QMM (Kernels/TensorCore/MPPPrefillInt4QMM.swift)
 class MPPPrefillInt4QMM {
 public:
