@@ -420,6 +420,39 @@ int32_t tf_prefill_int4_qmm(tf_ctx *ctx, tf_stream stream,
                             const void *x, uint64_t x_offset, void *y, uint64_t y_offset,
                             int32_t t, int32_t n, int32_t k, tf_dtype scale_dtype);
 
+/* ---- neighbours of the output head --------------------------------------------------------------------------- */
+/* EmbedLookupInt4.encode (Kernels/Quant/EmbedLookupInt4.swift:11-41) -> embed_lookup_int4
+ * (Metal/Quant/dequant_int4.metal:63-83): out[i] = half((q_i * s + b) * out_scale) for row token_id of the tied int4
+ * table [table_rows, d/2], scales/biases bf16 [table_rows, d/64]; d % 64 == 0.  table_rows has no counterpart in the
+ * Metal wrapper (which cannot check the token): a token outside the table is rejected here instead of read. */
+int32_t tf_embed_lookup_int4(tf_ctx *ctx, tf_stream stream, const void *table, uint64_t table_offset, const void *scales,
+                             uint64_t scales_offset, const void *biases, uint64_t biases_offset, void *out, uint64_t out_offset,
+                             uint32_t token_id, uint32_t d, float out_scale, uint32_t table_rows);
+/* PrefillEmbedLookupInt4.encode (Kernels/Prefill/Primitives/PrefillPrimitives.swift:11-38) -> prefill_embed_lookup_int4_block
+ * (Metal/Prefill/prefill.metal:26-52): the same for t tokens read from the DEVICE array tokens[t] (uint32), out [t, d].
+ * A token >= table_rows reads the last row. */
+int32_t tf_prefill_embed_lookup_int4_block(tf_ctx *ctx, tf_stream stream, const void *table, uint64_t table_offset, const void *scales,
+                                           uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *tokens,
+                                           uint64_t tokens_offset, void *out, uint64_t out_offset, uint32_t t, uint32_t d, float out_scale,
+                                           uint32_t table_rows);
+/* LogitSoftcapSoftmax.encode (Kernels/Sampling/LogitOutput.swift:11-30) -> logit_softcap_softmax
+ * (Metal/Sampling/logit.metal:52-124): probs[i] = half(softmax_i(softcap * tanh(logits / softcap))), probs fp16[v].
+ * logits_dtype: TF_FP16 (the reference's) or TF_FP32 (what tf_lm_head_logits_int4 can write). */
+int32_t tf_logit_softcap_softmax(tf_ctx *ctx, tf_stream stream, const void *logits, void *probs, uint32_t v, float softcap,
+                                 tf_dtype logits_dtype);
+/* Sample.encode (Kernels/Sampling/LogitOutput.swift:40-71) -> sample (Metal/Sampling/logit.metal:183-447).
+ * probs fp16[v] -> out_token uint32[1].  temperature <= 0: argmax (lowest index on ties).  top_k == 0 and top_p outside
+ * (0, 1): Gumbel-max draw from p^(1/T) with counter-based noise keyed by (seed, position, index).  Otherwise: the
+ * min(top_k or v, 256) most probable, cut where their cumulative mass reaches top_p, reweighted by p^(1/T), one
+ * inverse-CDF draw with xorshift64* seeded by `seed` (which must be non-zero). */
+int32_t tf_sample(tf_ctx *ctx, tf_stream stream, const void *probs, void *out_token, uint32_t v, float temperature, uint32_t top_k,
+                  float top_p, uint64_t seed, uint32_t position);
+/* SampleTopK64.encode (Kernels/Sampling/LogitOutput.swift:150-206) -> sample_topk64_stage1 / _reduce / _final
+ * (Metal/Sampling/logit.metal:449-606): the top-64 sampler through sorted 1024-entry tiles; same token as
+ * tf_sample(..., top_k = 64, ...).  vocab in 1...262144 (SampleTopK64Error.unsupportedVocabulary otherwise). */
+int32_t tf_sample_topk64(tf_ctx *ctx, tf_stream stream, const void *probs, void *out_token, uint32_t vocab, float temperature, float top_p,
+                         uint64_t seed);
+
 #ifdef __cplusplus
 }
 #endif

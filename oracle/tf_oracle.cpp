@@ -731,6 +731,149 @@ void tfo_k_rmsnorm_bf16w(const uint16_t *x_f16, const uint16_t *w_bf16, float ep
         out_f16[i] = tfo_f16_bits(tfo_f16_to_float(x_f16[i]) * inv * tfo_bf16_to_float(w_bf16[i]));
 }
 
+// ---- neighbours of the output head ---------------------------------------------------------------------------------
+// VS/Reference/Quant/EmbedLookup.swift:41-68 (applyInt4): one row of the tied int4 table, dequantized and scaled.
+void tfo_embed_lookup_int4(const uint8_t *table, const uint16_t *S, const uint16_t *B, uint32_t token, int d, float out_scale, float *out) {
+    const int groups = d / G;
+    const uint8_t *row = table + (size_t)token * (d / 2);
+    for (int i = 0; i < d; ++i) {
+        const uint8_t byte = row[i >> 1];
+        const int q = (i & 1) == 0 ? (byte & 0x0F) : (byte >> 4);
+        const float s = tfo_bf16_to_float(S[(size_t)token * groups + i / G]);
+        const float b = tfo_bf16_to_float(B[(size_t)token * groups + i / G]);
+        out[i] = ((float)q * s + b) * out_scale;
+    }
+}
+
+// VS/Reference/Sampling/LogitSoftcapSoftmax.swift:12-48: softcap * tanh(x / softcap), then a two-pass safe softmax.
+void tfo_logit_softcap_softmax_ref(const float *x, int v, float softcap, float *out) {
+    const float inv_c = 1.0f / softcap;
+    float mx = -INFINITY;
+    for (int i = 0; i < v; ++i) {
+        out[i] = softcap * std::tanh(x[i] * inv_c);
+        mx = out[i] > mx ? out[i] : mx;
+    }
+    float sum = 0.0f;
+    for (int i = 0; i < v; ++i) {
+        out[i] = std::exp(out[i] - mx);
+        sum += out[i];
+    }
+    const float inv_sum = 1.0f / sum;
+    for (int i = 0; i < v; ++i) out[i] *= inv_sum;
+}
+
+// M/Sampling/logit.metal:148-181: the sampler's two generators.
+static uint64_t sampler_xorshift64(uint64_t &s) {
+    s ^= s << 13;
+    s ^= s >> 7;
+    s ^= s << 17;
+    return s * 2685821657736338717ULL;
+}
+static float sampler_uniform01(uint64_t &s) { return (float)(uint32_t)(sampler_xorshift64(s) >> 40) * (1.0f / 16777216.0f); }
+uint64_t tfo_sampler_xorshift64(uint64_t *state) { return sampler_xorshift64(*state); }
+float tfo_sampler_gumbel(uint64_t seed, uint32_t position, uint32_t row) {
+    uint64_t x = seed ^ ((uint64_t)position * 0xD2B74407B1CE6E93ull) ^ (uint64_t)row;
+    x = x + 0x9E3779B97F4A7C15ull;
+    x = (x ^ (x >> 30)) * 0xBF58476D1CE4E5B9ull;
+    x = (x ^ (x >> 27)) * 0x94D049BB133111EBull;
+    x = x ^ (x >> 31);
+    const float u = ((float)(uint32_t)(x >> 40) + 0.5f) * (1.0f / 16777216.0f);
+    return -std::log(-std::log(u));
+}
+
+// Tail of the truncating sampler, shared by `sample` (M/Sampling/logit.metal:381-447) and `sample_topk64_final` (:566-606):
+// values/indices = the k best (probability descending, index ascending).  Returns the token.
+static uint32_t sampler_finish(std::vector<float> &values, const std::vector<uint32_t> &indices, uint32_t v, float temperature,
+                               float top_p, uint64_t seed) {
+    uint32_t kept = 0;
+    while (kept < values.size() && indices[kept] < v && std::isfinite(values[kept])) ++kept;
+    if (top_p > 0.0f && top_p < 1.0f) {
+        float cum = 0.0f;
+        uint32_t cut = kept;
+        for (uint32_t i = 0; i < kept; ++i) {
+            cum += values[i];
+            if (cum >= top_p) { cut = i + 1; break; }
+        }
+        kept = cut;
+    }
+    const float inv_temp = 1.0f / temperature;
+    if (temperature != 1.0f)
+        for (uint32_t i = 0; i < kept; ++i) values[i] = std::pow(values[i], inv_temp);
+    float surviving = 0.0f;
+    for (uint32_t i = 0; i < kept; ++i) surviving += values[i];
+    uint64_t rng = seed;
+    (void)sampler_xorshift64(rng);
+    const float u = sampler_uniform01(rng) * surviving;
+    float run = 0.0f;
+    uint32_t picked = indices.empty() ? 0u : indices[0];
+    for (uint32_t i = 0; i < kept; ++i) {
+        run += values[i];
+        if (u <= run) { picked = indices[i]; break; }
+    }
+    return picked;
+}
+
+static void sampler_top(const uint16_t *probs_f16, uint32_t v, uint32_t k, std::vector<float> &values, std::vector<uint32_t> &indices) {
+    // k rounds of "largest not yet taken, lowest index on ties" == the first k of a stable sort by descending value;
+    // NaN never compares greater, so it is never taken (the slot then holds -inf / 0xFFFFFFFF, as in the kernel)
+    std::vector<uint32_t> order;
+    order.reserve(v);
+    for (uint32_t i = 0; i < v; ++i) {
+        const float p = tfo_f16_to_float(probs_f16[i]);
+        if (p > -INFINITY) order.push_back(i);
+    }
+    std::stable_sort(order.begin(), order.end(), [&](uint32_t a, uint32_t b) { return tfo_f16_to_float(probs_f16[a]) > tfo_f16_to_float(probs_f16[b]); });
+    values.assign(k, -INFINITY);
+    indices.assign(k, 0xFFFFFFFFu);
+    for (uint32_t i = 0; i < k && i < order.size(); ++i) {
+        values[i] = tfo_f16_to_float(probs_f16[order[i]]);
+        indices[i] = order[i];
+    }
+}
+
+// M/Sampling/logit.metal:183-447 (`sample`): greedy, Gumbel-max, or top-k / top-p / temperature / inverse CDF.
+uint32_t tfo_sample(const uint16_t *probs_f16, uint32_t v, float temperature, uint32_t top_k, float top_p, uint64_t seed, uint32_t position) {
+    if (temperature <= 0.0f) {
+        float best = -INFINITY;
+        uint32_t idx = 0u;   // nothing above -inf: every thread of the kernel keeps its initial index 0
+        for (uint32_t i = 0; i < v; ++i) {
+            const float p = tfo_f16_to_float(probs_f16[i]);
+            if (p > best) { best = p; idx = i; }
+        }
+        return idx;
+    }
+    if (top_k == 0u && (top_p <= 0.0f || top_p >= 1.0f)) {
+        const float inv_t = 1.0f / temperature;
+        float best = -INFINITY;
+        uint32_t idx = 0xFFFFFFFFu;
+        for (uint32_t i = 0; i < v; ++i) {
+            const float p = tfo_f16_to_float(probs_f16[i]);
+            if (!(p > 0.0f)) continue;
+            const float sc = inv_t * std::log(p) + tfo_sampler_gumbel(seed, position, i);
+            if (sc > best) { best = sc; idx = i; }
+        }
+        return idx == 0xFFFFFFFFu ? 0u : idx;
+    }
+    uint32_t k = top_k == 0u ? v : top_k;
+    k = k < 256u ? k : 256u;
+    k = k < v ? k : v;
+    std::vector<float> values;
+    std::vector<uint32_t> indices;
+    sampler_top(probs_f16, v, k, values, indices);
+    return sampler_finish(values, indices, v, temperature, top_p, seed);
+}
+
+// M/Sampling/logit.metal:449-606 + Kernels/Sampling/LogitOutput.swift:88-206 (SampleTopK64): the 64 best through sorted
+// 1024-entry tiles, then the same tail.  Tile sorting keeps exactly the 64 best by (value descending, index ascending).
+uint32_t tfo_sample_topk64(const uint16_t *probs_f16, uint32_t v, float temperature, float top_p, uint64_t seed) {
+    std::vector<float> values;
+    std::vector<uint32_t> indices;
+    sampler_top(probs_f16, v, 64u < v ? 64u : v, values, indices);
+    values.resize(64, -INFINITY);
+    indices.resize(64, 0xFFFFFFFFu);
+    return sampler_finish(values, indices, 0xFFFFFFFFu, temperature, top_p, seed);
+}
+
 // Sum of squares of d fp16 values in the order of the reference's 256-thread, 32-lane two-stage reduction
 // (M/Fusions/fused.metal:217-235): strided per-thread fma chains, lane sums, then the per-group partials.
 static float k_block_sum_squares(const uint16_t *x_f16, int d) {

@@ -178,6 +178,12 @@ void tfo_k_moe_phase2(const uint8_t *const *blobs, const tfo_expert_offsets *off
                       const uint16_t *routing_w_f16, const uint16_t *residual_f16, uint16_t *y_f16,
                       int d, int f);                                            /* M/MoE/moe.metal:446-482 */
 void tfo_k_gelu_mul_fp16(const uint16_t *gate_f16, const uint16_t *up_f16, uint16_t *out_f16, int n); /* M/Primitives/utility.metal:6-18 */
+void tfo_embed_lookup_int4(const uint8_t *table, const uint16_t *S, const uint16_t *B, uint32_t token, int d, float out_scale, float *out); /* VS/Reference/Quant/EmbedLookup.swift:41-68 */
+void tfo_logit_softcap_softmax_ref(const float *x, int v, float softcap, float *out); /* VS/Reference/Sampling/LogitSoftcapSoftmax.swift:12-48 */
+uint64_t tfo_sampler_xorshift64(uint64_t *state);                                      /* M/Sampling/logit.metal:148-153 */
+float tfo_sampler_gumbel(uint64_t seed, uint32_t position, uint32_t row);              /* M/Sampling/logit.metal:165-181 */
+uint32_t tfo_sample(const uint16_t *probs_f16, uint32_t v, float temperature, uint32_t top_k, float top_p, uint64_t seed, uint32_t position); /* M/Sampling/logit.metal:183-447 */
+uint32_t tfo_sample_topk64(const uint16_t *probs_f16, uint32_t v, float temperature, float top_p, uint64_t seed); /* M/Sampling/logit.metal:449-606 */
 void tfo_k_post_attn_setup(uint16_t *hidden_f16, const uint16_t *attn_f16, const uint16_t *w_post_attn_bf16,
                            const uint16_t *w_pre_ffn_bf16, const uint16_t *w_pre_ffn2_bf16, float eps, uint16_t *dense_f16,
                            uint16_t *routed_f16, uint16_t *router_f16, int d); /* M/Fusions/fused.metal:190-269 */

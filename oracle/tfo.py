@@ -339,6 +339,51 @@ def layer_tail_ref(h2_bits, h1_bits, hidden_bits, w_postffn2_bits, w_postffn_bit
     return out
 
 
+# ---- neighbours of the output head --------------------------------------------------------
+_sig("tfo_embed_lookup_int4", None, u8p, u16p, u16p, C.c_uint32, i32, C.c_float, f32p)
+_sig("tfo_logit_softcap_softmax_ref", None, f32p, i32, C.c_float, f32p)
+_sig("tfo_sampler_xorshift64", C.c_uint64, C.POINTER(C.c_uint64))
+_sig("tfo_sampler_gumbel", C.c_float, C.c_uint64, C.c_uint32, C.c_uint32)
+_sig("tfo_sample", C.c_uint32, u16p, C.c_uint32, C.c_float, C.c_uint32, C.c_float, C.c_uint64, C.c_uint32)
+_sig("tfo_sample_topk64", C.c_uint32, u16p, C.c_uint32, C.c_float, C.c_float, C.c_uint64)
+
+
+def embed_lookup_int4(W, S, B, token: int, out_scale: float) -> np.ndarray:
+    W, S, B = _wsb(W, S, B)
+    d = W.shape[1] * 2
+    out = np.empty(d, np.float32)
+    lib.tfo_embed_lookup_int4(W, S, B, token, d, out_scale, out)
+    return out
+
+
+def logit_softcap_softmax_ref(x, softcap: float) -> np.ndarray:
+    x = _flat32(x)
+    out = np.empty_like(x)
+    lib.tfo_logit_softcap_softmax_ref(x, x.size, softcap, out)
+    return out
+
+
+def sampler_xorshift64(state: int):
+    """-> (output, new state)"""
+    s = C.c_uint64(state)
+    out = lib.tfo_sampler_xorshift64(C.byref(s))
+    return int(out), int(s.value)
+
+
+def sampler_gumbel(seed: int, position: int, row: int) -> float:
+    return float(lib.tfo_sampler_gumbel(seed, position, row))
+
+
+def sample(probs_bits, temperature: float, top_k: int, top_p: float, seed: int, position: int = 0) -> int:
+    p = np.ascontiguousarray(probs_bits, np.uint16)
+    return int(lib.tfo_sample(p, p.size, temperature, top_k, top_p, seed, position))
+
+
+def sample_topk64(probs_bits, temperature: float, top_p: float, seed: int) -> int:
+    p = np.ascontiguousarray(probs_bits, np.uint16)
+    return int(lib.tfo_sample_topk64(p, p.size, temperature, top_p, seed))
+
+
 # ---- MoE ---------------------------------------------------------------------------------
 _pp = C.POINTER(C.c_void_p)
 _sig("tfo_moe_run_ffn", None, C.c_void_p, C.POINTER(ExpertOffsets), f32p, f32p, i32, i32)

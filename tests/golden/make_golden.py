@@ -159,9 +159,51 @@ def qmm():
     return dict(W=W, S=S, B=B, x_bits=x_bits, y_ref=np.asarray(tfo.qmm_cpu_reference(W, S, B, x_bits, m, n, k), np.float32).reshape(m, n))
 
 
+def layer_glue():
+    """Tests/.../Kernels/Fusions/FusedLayerTailTests.swift:11-20 and FusedPostAttentionSetupTests.swift:11-17 at D = 2816."""
+    d, eps = 2816, 1e-6
+    rng = tfo.SplitMix64(0xC0DE7A11)
+    half = lambda r: tfo.to_f16_bits(r.uniform_array(-1.0, 1.0, d))
+    weight = lambda r: tfo.bf16_bits_array(r.uniform_array(0.5, 1.5, d))
+    h2, h1, hidden = half(rng), half(rng), half(rng)
+    w2, w = weight(rng), weight(rng)
+    scalar = rng.uniform(0.75, 1.25)
+    out = dict(tail_h2=h2, tail_h1=h1, tail_hidden=hidden, tail_w_postffn2=w2, tail_w_postffn=w, tail_scalar=np.array([scalar], np.float32),
+               tail_hidden_out=tfo.k_layer_tail(h2, h1, hidden, w2, w, eps, scalar), tail_ref=tfo.layer_tail_ref(h2, h1, hidden, w2, w, eps, scalar))
+    rng = tfo.SplitMix64(0x9057A77E)
+    hidden, attn = half(rng), half(rng)
+    w_post, w_pre, w_pre2 = weight(rng), weight(rng), weight(rng)
+    h_out, dense, routed, router = tfo.k_post_attn_setup(hidden, attn, w_post, w_pre, w_pre2, eps)
+    out.update(setup_hidden=hidden, setup_attn=attn, setup_w_post=w_post, setup_w_pre=w_pre, setup_w_pre2=w_pre2, setup_hidden_out=h_out,
+               setup_dense=dense, setup_routed=routed, setup_router=router)
+    return out
+
+
+def head_neighbours():
+    """EmbedLookupTests.swift:16-77 (V=16, D=128), LogitSoftcapSoftmaxTests.swift:34-54 (2048 logits in +-50), and sampler draws
+    on a 1003-entry distribution (SampleTopK64Tests.swift:101-131 shapes) with the tokens the restated sampler returns."""
+    rng = tfo.SeedTree(0x131).key("embed-lookup-int4-table")
+    W, S, B = tfo.quantize_int4(rng.uniform_array(-1.0, 1.0, 16 * 128).reshape(16, 128))
+    scale = float(np.sqrt(np.float32(128)))
+    out = dict(embed_W=W, embed_S=S, embed_B=B, embed_scale=np.array([scale], np.float32),
+               embed_row9=tfo.embed_lookup_int4(W, S, B, 9, scale))
+    rng = tfo.SeedTree(0x131).key("softcap-softmax-random")
+    logits = tfo.to_f16_bits(rng.uniform_array(-50.0, 50.0, 2048))
+    out.update(softmax_logits=logits, softmax_probs=tfo.logit_softcap_softmax_ref(tfo.from_f16_bits(logits), 30.0))
+    p = np.random.default_rng(1003).random(1003).astype(np.float32)
+    probs = tfo.to_f16_bits(p / p.sum())
+    seeds = np.array([1, 2, 3, 0x123456789ABCDEF0, 0xFFFFFFFFFFFFFFFF], np.uint64)
+    out.update(sample_probs=probs, sample_seeds=seeds,
+               sample_greedy=np.array([tfo.sample(probs, 0.0, 0, 1.0, 1)], np.uint32),
+               sample_top4=np.array([tfo.sample(probs, 1.0, 4, 1.0, int(s)) for s in seeds], np.uint32),
+               sample_top64_p95_t085=np.array([tfo.sample_topk64(probs, 0.85, 0.95, int(s)) for s in seeds], np.uint32),
+               sample_nucleus_p30=np.array([tfo.sample(probs, 1.3, 0, 0.3, int(s)) for s in seeds], np.uint32))
+    return out
+
+
 CASES = dict(prng_streams=prng_streams, gemv_int4_m64_k128=gemv_int4, gemv_int8_m16_k128=gemv_int8, router_e16_d128=router,
              moe_d128_f64_top8=moe, shared_expert_d128_f64=shared_expert, lm_head_d64_v1024=lm_head, rmsnorm_gelu_256=rmsnorm_gelu,
-             prefill_grouped_e6_d128_f64=prefill, int4_qmm_m8_n64_k128=qmm)
+             prefill_grouped_e6_d128_f64=prefill, int4_qmm_m8_n64_k128=qmm, layer_glue_d2816=layer_glue, head_neighbours=head_neighbours)
 
 
 def generate(name):

@@ -151,3 +151,48 @@ def test_int4_qmm_fixture():
                                       m, n, kk, tfk.TF_BF16))
         got = f16(host(y, np.uint16, m * n)).reshape(m, n)
         assert within_north_star(got, z["y_ref"]), entry
+
+
+def test_layer_glue_fixture():
+    z = load("layer_glue_d2816")
+    k = ctx()
+    d = 2816
+    t = {n: dev(z[n]) for n in z if z[n].dtype == np.uint16 and z[n].size == d}       # keeps every operand alive until the results are read
+    k.check(k.lib.tf_fused_layer_tail(k.handle, None, t["tail_h2"].data_ptr(), t["tail_h1"].data_ptr(), t["tail_hidden"].data_ptr(),
+                                      t["tail_w_postffn2"].data_ptr(), 0, t["tail_w_postffn"].data_ptr(), 0, d, 1e-6, float(z["tail_scalar"][0])))
+    got = host(t["tail_hidden"], np.uint16, d)
+    assert np.count_nonzero(got != z["tail_hidden_out"]) <= 14 and np.max(np.abs(f16(got) - f16(z["tail_hidden_out"]))) <= 2.0 ** -9
+    assert np.max(np.abs(f16(got) - z["tail_ref"])) / float(np.max(np.abs(z["tail_ref"]))) < 4e-3       # FusedLayerTailTests.swift:72
+    dense, routed, router = zeros_bytes(d * 2), zeros_bytes(d * 2), zeros_bytes(d * 2)
+    k.check(k.lib.tf_fused_post_attn_setup(k.handle, None, t["setup_hidden"].data_ptr(), t["setup_attn"].data_ptr(), dense.data_ptr(), routed.data_ptr(),
+                                           router.data_ptr(), t["setup_w_post"].data_ptr(), 0, t["setup_w_pre"].data_ptr(), 0,
+                                           t["setup_w_pre2"].data_ptr(), 0, d, 1e-6))
+    for buf, name in ((t["setup_hidden"], "setup_hidden_out"), (dense, "setup_dense"), (routed, "setup_routed"), (router, "setup_router")):
+        got = host(buf, np.uint16, d)
+        assert np.count_nonzero(got != z[name]) <= 14 and np.max(np.abs(f16(got) - f16(z[name]))) <= 2.0 ** -9, name
+
+
+def test_head_neighbours_fixture():
+    z = load("head_neighbours")
+    k = ctx()
+    out = zeros_bytes(128 * 2)
+    eW, eS, eB, logits = dev(z["embed_W"]), dev(z["embed_S"]), dev(z["embed_B"]), dev(z["softmax_logits"])
+    k.check(k.lib.tf_embed_lookup_int4(k.handle, None, eW.data_ptr(), 0, eS.data_ptr(), 0, eB.data_ptr(), 0,
+                                       out.data_ptr(), 0, 9, 128, float(z["embed_scale"][0]), 16))
+    assert np.array_equal(host(out, np.uint16, 128), z["embed_row9"].astype(np.float16).view(np.uint16))
+    probs = zeros_bytes(2048 * 2)
+    k.check(k.lib.tf_logit_softcap_softmax(k.handle, None, logits.data_ptr(), probs.data_ptr(), 2048, 30.0, tfk.TF_FP16))
+    got, ref = f16(host(probs, np.uint16, 2048)), z["softmax_probs"]
+    assert np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-4)) < 5e-3        # LogitSoftcapSoftmaxTests.swift:46-49
+    d_probs, tok = dev(z["sample_probs"]), zeros_bytes(4)
+
+    def draw(*args, topk64=False):
+        fn = k.lib.tf_sample_topk64 if topk64 else k.lib.tf_sample
+        k.check(fn(k.handle, None, d_probs.data_ptr(), tok.data_ptr(), 1003, *args))
+        return int(host(tok, np.uint32, 1)[0])
+
+    assert draw(0.0, 0, 1.0, 1, 0) == int(z["sample_greedy"][0])
+    for i, seed in enumerate(int(s) for s in z["sample_seeds"]):
+        assert draw(1.0, 4, 1.0, seed, 0) == int(z["sample_top4"][i])
+        assert draw(0.85, 0.95, seed, topk64=True) == int(z["sample_top64_p95_t085"][i])
+        assert draw(1.3, 0, 0.3, seed, 0) == int(z["sample_nucleus_p30"][i])

@@ -131,6 +131,11 @@ EXPORTS = {
     "tf_prefill_moe_reduce_token_major": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32, u32, u32]),
     "tf_int4_qmm": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, i32, i32, i32, i32]),
     "tf_prefill_int4_qmm": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, i32, i32, i32, i32]),
+    "tf_embed_lookup_int4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, C.c_float, u32]),
+    "tf_prefill_embed_lookup_int4_block": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, C.c_float, u32]),
+    "tf_logit_softcap_softmax": (i32, [vp, vp, vp, vp, u32, C.c_float, i32]),
+    "tf_sample": (i32, [vp, vp, vp, vp, u32, C.c_float, u32, C.c_float, u64, u32]),
+    "tf_sample_topk64": (i32, [vp, vp, vp, vp, u32, C.c_float, C.c_float, u64]),
     "tf_lm_head_greedy_int4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u32, u32, C.c_float, i32]),
     "tf_lm_head_logits_int4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, C.c_float,
                                      i32, i32]),

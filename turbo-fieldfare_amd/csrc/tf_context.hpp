@@ -21,6 +21,8 @@ struct tf_ctx {
     uint32_t *group_scratch = nullptr;  // kGroupSegments x 256 per-segment expert counts of the device pair grouping
     float *prefill_logits = nullptr;    // lazily sized [tokens, experts] router logits of the multi-token router
     size_t prefill_logits_count = 0;
+    void *sample_scratch = nullptr;     // lazily sized: argmax cells, softmax partials, top-k pair buffers of the samplers
+    size_t sample_scratch_bytes = 0;
     // optional device-time bracketing of the decode step's three launches
     bool step_timing = false;
     bool step_timed = false;            // a step has been recorded since timing was enabled

@@ -1,22 +1,11 @@
 // Tied int4 output head for gfx950: final RMSNorm -> vocab-sized int4 GEMV -> greedy argmax without materialising
 // logits, and the logits variant for samplers.
+#include "tf_argmax.hpp"
 #include "tf_gemv_kernels.hpp"
 
 using namespace tfk;
 
 namespace {
-
-struct Best {
-    float v;
-    uint32_t idx;
-};
-
-__device__ __forceinline__ void better(Best &b, float v, uint32_t idx) {
-    if (v > b.v || (v == b.v && idx < b.idx)) {
-        b.v = v;
-        b.idx = idx;
-    }
-}
 
 // Persistent row streamer: every wave walks tiles wave, wave + nwaves, ... of RT rows and keeps the best finite logit it
 // has seen (rows ascend within a wave, so a strict comparison keeps the lowest index among equals).  With FUSE_NORM each
@@ -24,15 +13,6 @@ __device__ __forceinline__ void better(Best &b, float v, uint32_t idx) {
 // {value, index} into one of kHeadCells 64-bit cells with a single atomic max on the key
 // (orderable(value) << 32 | ~index): larger value wins, equal values resolve to the lower index, 0 means "nothing finite".
 // The block that finishes last turns the cells into the token and clears them for the next call.
-constexpr uint32_t kHeadCells = 64;
-
-__device__ __forceinline__ unsigned long long best_key(float v, uint32_t idx) {
-    if (idx == 0xFFFFFFFFu) return 0ull;
-    uint32_t u = __float_as_uint(v);
-    u = (u & 0x80000000u) ? ~u : (u | 0x80000000u);   // monotone map of finite floats onto unsigned integers
-    return ((unsigned long long)u << 32) | (unsigned long long)(0xFFFFFFFFu - idx);
-}
-
 template <int RT, int NP, int SD, bool FUSE_NORM>
 __global__ __launch_bounds__(256, 4) void head_greedy_long_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B,
                                                                const half_t *x, const uint16_t *norm_w, float eps,
@@ -101,37 +81,7 @@ __global__ __launch_bounds__(256, 4) void head_greedy_long_kernel(const uint8_t 
         }
     }
     if (lane == 0) { sv[wib] = best.v; si[wib] = best.idx; }
-    __syncthreads();
-    // Fold the block's best into a cell, then take a ticket.  Both are device-scope atomics performed at the memory
-    // side, and the ticket is only requested after the fold has returned, so the block that draws the last ticket
-    // finds every fold in the cells (read with atomics as well) without any cache write-back or invalidate.
-    __shared__ uint32_t is_last;
-    if (threadIdx.x == 0) {
-        Best b{sv[0], si[0]};
-        for (int w = 1; w < 4; ++w) better(b, sv[w], si[w]);
-        const unsigned long long key = best_key(b.v, b.idx);
-        unsigned long long seen = 0ull;
-        if (key) seen = atomicMax(cells + (blockIdx.x % kHeadCells), key);
-        // the ticket increment depends on the value the fold returned
-        uint32_t one = 1u;
-        const uint32_t seen_lo = (uint32_t)seen;
-        asm volatile("" : "+v"(one) : "v"(seen_lo));
-        unsigned int *ticket = reinterpret_cast<unsigned int *>(cells + kHeadCells);
-        is_last = atomicAdd(ticket, one) == gridDim.x - 1 ? 1u : 0u;
-    }
-    __syncthreads();
-    if (is_last && wib == 0) {
-        unsigned long long key = __hip_atomic_exchange(cells + lane, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#pragma unroll
-        for (int off = 32; off >= 1; off >>= 1) {
-            const unsigned long long other = __shfl_xor(key, off, kWave);
-            key = other > key ? other : key;
-        }
-        if (lane == 0) {
-            out_token[0] = key ? 0xFFFFFFFFu - (uint32_t)(key & 0xFFFFFFFFull) : 0u;
-            __hip_atomic_store(reinterpret_cast<unsigned int *>(cells + kHeadCells), 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
-    }
+    fold_block_best(sv, si, cells, out_token);
 }
 
 // Fallback first stage: argmax summaries over an fp32 logits vector (one summary per block).

@@ -345,6 +345,75 @@ private:
     const Context &c_;
 };
 
+
+// EmbedLookupInt4 (Kernels/Quant/EmbedLookupInt4.swift); tableRows bounds the token (see tf_embed_lookup_int4)
+class EmbedLookupInt4 {
+public:
+    explicit EmbedLookupInt4(const Context &context) : c_(context) {}
+    void encode(const void *table, uint64_t tableOffset, const void *scales, uint64_t scalesOffset, const void *biases,
+                uint64_t biasesOffset, void *out, uint64_t outOffset, uint32_t tokenId, uint32_t d, float outScale,
+                uint32_t tableRows) const {
+        c_.check(tf_embed_lookup_int4(c_.raw(), c_.stream(), table, tableOffset, scales, scalesOffset, biases, biasesOffset, out, outOffset,
+                                      tokenId, d, outScale, tableRows));
+    }
+
+private:
+    const Context &c_;
+};
+
+// PrefillEmbedLookupInt4 (Kernels/Prefill/Primitives/PrefillPrimitives.swift:4-39)
+class PrefillEmbedLookupInt4 {
+public:
+    explicit PrefillEmbedLookupInt4(const Context &context) : c_(context) {}
+    void encode(const void *table, uint64_t tableOffset, const void *scales, uint64_t scalesOffset, const void *biases,
+                uint64_t biasesOffset, const void *tokens, uint64_t tokensOffset, void *out, uint64_t outOffset, uint32_t t, uint32_t d,
+                float outScale, uint32_t tableRows) const {
+        c_.check(tf_prefill_embed_lookup_int4_block(c_.raw(), c_.stream(), table, tableOffset, scales, scalesOffset, biases, biasesOffset,
+                                                    tokens, tokensOffset, out, outOffset, t, d, outScale, tableRows));
+    }
+
+private:
+    const Context &c_;
+};
+
+// LogitSoftcapSoftmax, Sample, SampleTopK64 (Kernels/Sampling/LogitOutput.swift)
+class LogitSoftcapSoftmax {
+public:
+    explicit LogitSoftcapSoftmax(const Context &context) : c_(context) {}
+    void encode(const void *logits, void *probs, uint32_t v, float softcap = 30.0f) const {
+        c_.check(tf_logit_softcap_softmax(c_.raw(), c_.stream(), logits, probs, v, softcap, TF_FP16));
+    }
+
+private:
+    const Context &c_;
+};
+
+class Sample {
+public:
+    explicit Sample(const Context &context) : c_(context) {}
+    void encode(const void *probs, void *outToken, uint32_t v, float temperature, uint32_t topK, float topP, uint64_t seed,
+                uint32_t position = 0) const {
+        c_.check(tf_sample(c_.raw(), c_.stream(), probs, outToken, v, temperature, topK, topP, seed, position));
+    }
+
+private:
+    const Context &c_;
+};
+
+class SampleTopK64 {
+public:
+    SampleTopK64(const Context &context, uint32_t vocab) : c_(context), vocab_(vocab) {
+        if (vocab == 0 || vocab > 262144) throw Error(TF_ERR_INVALID_ARGUMENT, "unsupportedVocabulary");
+    }
+    void encode(const void *probs, void *outToken, float temperature, float topP, uint64_t seed) const {
+        c_.check(tf_sample_topk64(c_.raw(), c_.stream(), probs, outToken, vocab_, temperature, topP, seed));
+    }
+
+private:
+    const Context &c_;
+    uint32_t vocab_;
+};
+
 // MPPPrefillInt4QMM (Kernels/TensorCore/MPPPrefillInt4QMM.swift)
 class MPPPrefillInt4QMM {
 public:
