@@ -301,6 +301,25 @@ def extras(torch, tfk, k, gen, lib, h, stream):
     res["gemv_2112x2816"] = {"workload": "configs[0]: int4 g64 GEMV 2112x2816, batch 1", "us_per_call": round(us, 3),
                              "GBps": round(nbytes / (us * 1e-6) / 1e9, 1), "algorithmic_bytes": nbytes}
 
+    # q / k / v projections of one token in one launch (4096 + 2 x 2048 rows of 2816), rotating over the same 644 MB
+    q_rows, kv_rows = 4096, 2048
+    span = q_rows + 2 * kv_rows
+    qkv_reps = (reps * F_SHARED) // span
+    qo, ko, vo = (torch.zeros(r, dtype=torch.float16, device="cuda") for r in (q_rows, kv_rows, kv_rows))
+
+    def qkv(i):
+        r = (i % qkv_reps) * span
+        args = []
+        for first in (r, r + q_rows, r + q_rows + kv_rows):
+            args += [W.data_ptr(), first * row_w, S.data_ptr(), first * row_s, B.data_ptr(), first * row_s]
+        rc = lib.tf_fused_qkv_gemv(h, stream, *args, xs.data_ptr() + (i % 8) * D * 2, qo.data_ptr(), 0, ko.data_ptr(), 0, vo.data_ptr(), 0,
+                                   q_rows, kv_rows, D, tfk.TF_BF16)
+        assert rc == 0, k.last_error()
+    us = time_loop(torch, qkv, 200, warmup=20)
+    nbytes = int4_matrix_bytes(span, D) + D * 2 + span * 2
+    res["fused_qkv_gemv_8192x2816"] = {"us_per_call": round(us, 3), "GBps": round(nbytes / (us * 1e-6) / 1e9, 1),
+                                       "frac_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": nbytes}
+
     # shared expert chain (gate/up 2112x2816 fused + GeGLU, down 2816x2112), rotating over 64 replicas of each matrix
     sreps = 64
     gu = W[: sreps * 2 * F_SHARED], S[: sreps * 2 * F_SHARED], B[: sreps * 2 * F_SHARED]

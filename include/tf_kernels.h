@@ -150,6 +150,18 @@ int32_t tf_dequant_int8_gemv(tf_ctx *ctx, tf_stream stream,
                              void *y, uint64_t y_offset,
                              uint32_t m, uint32_t n, tf_dtype scale_dtype, tf_dtype out_dtype);
 
+/* FusedQKVGEMV.encode (Kernels/Fusions/FusedQKVGEMV.swift:38-97) -> dequant_int4_qkv_gemv_simd
+ * (Metal/Quant/dequant_int4.metal:194-244): the q, k and v projections of one token in one launch;
+ * q [q_rows, n], k and v [kv_rows, n] int4 group-64 with bf16/fp16 scales, x fp16[n], outputs fp16.
+ * Each output equals tf_dequant_int4_gemv of its matrix bit for bit.  n % 64 == 0, even weights offsets. */
+int32_t tf_fused_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *q_weights, uint64_t q_weights_offset, const void *q_scales,
+                          uint64_t q_scales_offset, const void *q_biases, uint64_t q_biases_offset, const void *k_weights,
+                          uint64_t k_weights_offset, const void *k_scales, uint64_t k_scales_offset, const void *k_biases,
+                          uint64_t k_biases_offset, const void *v_weights, uint64_t v_weights_offset, const void *v_scales,
+                          uint64_t v_scales_offset, const void *v_biases, uint64_t v_biases_offset, const void *x, void *q_out,
+                          uint64_t q_out_offset, void *k_out, uint64_t k_out_offset, void *v_out, uint64_t v_out_offset, uint32_t q_rows,
+                          uint32_t kv_rows, uint32_t n, tf_dtype scale_dtype);
+
 /* ---- primitives on the path -------------------------------------------------------------------------------- */
 /* gelu_mul_fp16 (Metal/Primitives/utility.metal:6-18; dispatched at SharedExpertInt4.swift:76-86):
  * out = half(gelu_tanh(float(gate)) * float(up)). */
@@ -384,6 +396,7 @@ int32_t tf_prefill_grouped_routed_moe_streamed(tf_ctx *ctx, tf_stream stream,
  * pool + expert * pool_stride, the work list comes from tf_prefill_group_pairs_device, nothing is read by the host.  Groups
  * of a few pairs stream each expert row once and apply it to every routed token (weight-read bound, the small-M regime);
  * large groups run as a grouped GEMM on the matrix cores (weights expanded to fp16 in LDS, fp32 accumulation).
+ * hidden holds pair_count / top_k token rows and every (token, rank) combination appears once among the pairs.
  * acts_scratch: pair_count * f halves.  max_chunks: capacity of `chunks`. */
 int32_t tf_prefill_grouped_routed_moe_resident(tf_ctx *ctx, tf_stream stream,
                                                const void *hidden, uint64_t hidden_offset, uint32_t hidden_stride_elements,

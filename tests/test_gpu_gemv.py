@@ -161,3 +161,39 @@ def test_contract_violations_return_status_and_enqueue_nothing():
     assert k.dequant_int4_gemv(None, dS, dB, dx, y, 64, 128, raise_on_error=False) == tfk.TF_ERR_INVALID_ARGUMENT
     k.synchronize()
     assert np.all(host(y, np.uint8) == 0xEE)
+
+
+@pytest.mark.parametrize("q_rows,kv_rows,n,w_off,seed", [(64, 32, 128, 0, 0x51564745), (128, 64, 2816, 2, 0x51564746), (128, 64, 2816, 0, 0x51564746),
+                                                        (4096, 2048, 2816, 0, 7), (8192, 1024, 2816, 0, 8), (33, 7, 2112, 0, 9)])
+def test_fused_qkv_gemv_equals_three_gemvs(q_rows, kv_rows, n, w_off, seed):
+    # FusedQKVGEMVTests.swift:8-127 (one launch == the three projections, also at a +2 weight offset) + the decode shapes
+    rng = tfo.SplitMix64(seed)
+    mats = []
+    for rows in (q_rows, kv_rows, kv_rows):
+        if rows * n <= 1 << 20:
+            mats.append(tfo.quantize_int4(rng.uniform_array(-0.5, 0.5, rows * n).reshape(rows, n)))
+        else:
+            mats.append(refcases.synthetic_int4(rows, n, seed + rows))
+    x_bits = tfo.to_f16_bits(rng.uniform_array(-1.0, 1.0, n))
+    k = ctx()
+    d = [(dev(W, w_off), dev(S), dev(B)) for W, S, B in mats]
+    dx = dev(x_bits)
+    fused = [zeros_bytes(r * 2 + 16, 0xEE) for r in (q_rows, kv_rows, kv_rows)]
+    args = []
+    for W, S, B in d:
+        args += [W.data_ptr(), w_off, S.data_ptr(), 0, B.data_ptr(), 0]
+    outs = []
+    for o in fused:
+        outs += [o.data_ptr(), 0]
+    k.check(k.lib.tf_fused_qkv_gemv(k.handle, None, *args, dx.data_ptr(), *outs, q_rows, kv_rows, n, tfk.TF_BF16))
+    for (W, S, B), (dW, dS, dB), o, rows in zip(mats, d, fused, (q_rows, kv_rows, kv_rows)):
+        single = zeros_bytes(rows * 2)
+        k.dequant_int4_gemv(dW, dS, dB, dx, single, rows, n, offsets=(w_off, 0, 0, 0, 0))
+        got = host(o, np.uint16, rows)
+        assert np.array_equal(got, host(single, np.uint16, rows))
+        assert np.all(host(o, np.uint8)[rows * 2:] == 0xEE)
+        ref = tfo.int4_gemv_ref(W, S, B, tfo.from_f16_bits(x_bits), threads=8)
+        assert within_north_star(tfo.from_f16_bits(got), ref, abs_=1e-3 * max(1.0, float(np.max(np.abs(ref)))))
+    bad = list(args)
+    bad[1] = 1                                     # odd q weights offset (FusedQKVGEMV.swift:60-63)
+    assert k.lib.tf_fused_qkv_gemv(k.handle, None, *bad, dx.data_ptr(), *outs, q_rows, kv_rows, n, tfk.TF_BF16) == tfk.TF_ERR_INVALID_ARGUMENT

@@ -101,6 +101,7 @@ EXPORTS = {
     "tf_dequantize_int8_affine": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32]),
     "tf_dequant_int4_gemv": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32, i32]),
     "tf_dequant_int8_gemv": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32, i32]),
+    "tf_fused_qkv_gemv": (i32, [vp, vp] + [vp, u64] * 9 + [vp] + [vp, u64] * 3 + [u32, u32, u32, i32]),
     "tf_gelu_mul_fp16": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32]),
     "tf_rmsnorm_bf16w": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32, C.c_float]),
     "tf_fused_post_attn_setup": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, u64, vp, u64, vp, u64, u32, C.c_float]),

@@ -102,6 +102,72 @@ __global__ __launch_bounds__(256, 4) void gemv4_long_kernel(const uint8_t *W, co
     }
 }
 
+// The same streamer over up to three matrices that share the activations (the q, k and v projections of one token):
+// one launch, one staging of x; a tile never straddles two matrices.  Output fp16.
+struct GemvSegments {
+    const uint8_t *W[3], *S[3], *B[3];
+    half_t *y[3];
+    uint32_t rows[3];
+    uint32_t tile_end[3];   // running total of tiles up to and including each matrix
+};
+
+template <int RT, int NP, int SD>
+__global__ __launch_bounds__(256, 4) void qkv_gemv_long_kernel(GemvSegments g, const half_t *x, int k) {
+    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
+    __shared__ float xsum[XStage::kMaxK / 32];
+    const int lane = threadIdx.x & 63;
+    const long wave = uniform_int((int)(((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6));
+    const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
+    const long ntiles = g.tile_end[2];
+    const size_t tile_bytes = (size_t)RT * (k >> 1);
+    const size_t sb_bytes = (size_t)RT * (k >> 6) * 2;
+
+    RowStream<RT, NP> rs;
+    typename RowStream<RT, NP>::Tile ta, tb;
+    rs.init_map(k, lane);
+    // global tile -> (matrix, tile inside it); everything here is wave-uniform
+    auto locate = [&](long at, int &seg, long &local) {
+        seg = at < (long)g.tile_end[0] ? 0 : (at < (long)g.tile_end[1] ? 1 : 2);
+        local = at - (seg == 0 ? 0 : (long)g.tile_end[seg - 1]);
+    };
+    auto request = [&](typename RowStream<RT, NP>::Tile &t, long at) {
+        int seg;
+        long local;
+        locate(at, seg, local);
+        rs.load(t, g.W[seg] + local * tile_bytes, g.S[seg] + local * sb_bytes, g.B[seg] + local * sb_bytes, (long)g.rows[seg] - local * RT);
+    };
+    long t0 = wave, t1 = wave + nwaves;
+    XStage stage;
+    stage.request(x, k);
+    if (t0 < ntiles) request(ta, t0);
+    if (t1 < ntiles) request(tb, t1);
+    stage.publish(k, xa, xsum);
+    if (t0 >= ntiles) return;
+    rs.init_x_lds(xa, xsum, k);
+    auto emit = [&](const typename RowStream<RT, NP>::Tile &t, long at) {
+        int seg;
+        long local;
+        locate(at, seg, local);
+        float out[RT];
+        rs.template reduce<SD>(t, out);
+        if (lane == 0) {
+#pragma unroll
+            for (int r = 0; r < RT; ++r)
+                if (local * RT + r < (long)g.rows[seg]) g.y[seg][local * RT + r] = (half_t)out[r];
+        }
+    };
+    for (;;) {
+        emit(ta, t0);
+        t0 += 2 * nwaves;
+        if (t0 < ntiles) request(ta, t0);
+        if (t1 >= ntiles) break;
+        emit(tb, t1);
+        t1 += 2 * nwaves;
+        if (t1 < ntiles) request(tb, t1);
+        if (t0 >= ntiles) break;
+    }
+}
+
 // K <= 1024: each wave covers 2 * NPASS consecutive rows, one row per half-wave per pass.
 template <int NPASS, int SD, typename OutT>
 __global__ __launch_bounds__(256) void gemv4_short_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B,
@@ -431,6 +497,65 @@ int32_t tf_rmsnorm_bf16w(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t 
     TF_REQUIRE(ctx, x_offset % 2 == 0 && weight_offset % 2 == 0 && out_offset % 2 == 0, TF_ERR_INVALID_ARGUMENT,
                "rmsnorm_bf16w: offsets must be 2-byte aligned");
     return launch_rmsnorm_bf16w(ctx, static_cast<hipStream_t>(stream), at(x, x_offset), at(weight, weight_offset), at(out, out_offset), d, eps);
+}
+
+int32_t tf_fused_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *q_weights, uint64_t q_weights_offset, const void *q_scales,
+                          uint64_t q_scales_offset, const void *q_biases, uint64_t q_biases_offset, const void *k_weights,
+                          uint64_t k_weights_offset, const void *k_scales, uint64_t k_scales_offset, const void *k_biases,
+                          uint64_t k_biases_offset, const void *v_weights, uint64_t v_weights_offset, const void *v_scales,
+                          uint64_t v_scales_offset, const void *v_biases, uint64_t v_biases_offset, const void *x, void *q_out,
+                          uint64_t q_out_offset, void *k_out, uint64_t k_out_offset, void *v_out, uint64_t v_out_offset, uint32_t q_rows,
+                          uint32_t kv_rows, uint32_t n, tf_dtype scale_dtype) {
+    const void *w[3] = {q_weights, k_weights, v_weights};
+    const void *s[3] = {q_scales, k_scales, v_scales};
+    const void *b[3] = {q_biases, k_biases, v_biases};
+    void *y[3] = {q_out, k_out, v_out};
+    const uint64_t wo[3] = {q_weights_offset, k_weights_offset, v_weights_offset};
+    const uint64_t so[3] = {q_scales_offset, k_scales_offset, v_scales_offset};
+    const uint64_t bo[3] = {q_biases_offset, k_biases_offset, v_biases_offset};
+    const uint64_t yo[3] = {q_out_offset, k_out_offset, v_out_offset};
+    const uint32_t rows[3] = {q_rows, kv_rows, kv_rows};
+    for (int i = 0; i < 3; ++i) {
+        const int32_t rc = validate_gemv(ctx, "fused_qkv_gemv", w[i], wo[i], s[i], so[i], b[i], bo[i], x, 0, y[i], yo[i], rows[i], n,
+                                         scale_dtype, TF_FP16, 2);
+        if (rc != TF_OK) return rc;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const LongPlan plan = plan_long_rows((int)n);
+    bool fast = aligned16(x) && n > 1024 && n <= (uint32_t)XStage::kMaxK && plan.rt > 0;
+    for (int i = 0; i < 3; ++i) fast = fast && aligned16(at(w[i], wo[i]));
+    if (fast) {
+        GemvSegments g;
+        uint32_t total = 0;
+        for (int i = 0; i < 3; ++i) {
+            g.W[i] = at(w[i], wo[i]);
+            g.S[i] = at(s[i], so[i]);
+            g.B[i] = at(b[i], bo[i]);
+            g.y[i] = reinterpret_cast<half_t *>(at(y[i], yo[i]));
+            g.rows[i] = rows[i];
+            total += (rows[i] + plan.rt - 1) / plan.rt;
+            g.tile_end[i] = total;
+        }
+        const long max_blocks = (long)ctx->num_cus * ctx->stream_blocks_per_cu;
+        const uint32_t grid = (uint32_t)std::max<long>(1, std::min<long>(((long)total + 3) / 4, max_blocks));
+        const half_t *xh = static_cast<const half_t *>(x);
+#define TF_QKV_CASE(RT_, NP_)                                                                                             \
+    if (plan.rt == RT_ && plan.np == NP_) {                                                                               \
+        if (scale_dtype == TF_BF16) hipLaunchKernelGGL((qkv_gemv_long_kernel<RT_, NP_, 0>), dim3(grid), dim3(256), 0, st, g, xh, (int)n); \
+        else hipLaunchKernelGGL((qkv_gemv_long_kernel<RT_, NP_, 1>), dim3(grid), dim3(256), 0, st, g, xh, (int)n);        \
+        return check_launch(ctx, "fused_qkv_gemv");                                                                       \
+    }
+        TF_QKV_CASE(1, 1) TF_QKV_CASE(1, 2) TF_QKV_CASE(1, 3) TF_QKV_CASE(1, 4)
+        TF_QKV_CASE(2, 1) TF_QKV_CASE(2, 2) TF_QKV_CASE(2, 3) TF_QKV_CASE(2, 4)
+        TF_QKV_CASE(4, 1) TF_QKV_CASE(4, 2) TF_QKV_CASE(4, 3) TF_QKV_CASE(4, 4)
+#undef TF_QKV_CASE
+    }
+    // any other shape or alignment: the three projections one after the other (same arithmetic per row)
+    for (int i = 0; i < 3; ++i) {
+        const int32_t rc = launch_gemv4(ctx, st, at(w[i], wo[i]), at(s[i], so[i]), at(b[i], bo[i]), x, at(y[i], yo[i]), rows[i], n, scale_dtype, TF_FP16);
+        if (rc != TF_OK) return rc;
+    }
+    return TF_OK;
 }
 
 }  // extern "C"

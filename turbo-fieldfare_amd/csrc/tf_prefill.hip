@@ -435,6 +435,99 @@ __global__ __launch_bounds__(256) void grouped_phase1_long_kernel(ExpertTable ta
     }
 }
 
+// Few tokens (verification / small batches): the experts' weights dominate and every touched expert must stream through
+// once at full rate.  Persistent blocks of 8 waves, one per CU: the activations of ALL tokens (at most kStreamTokens rows)
+// are staged once per block in LDS in dot-product order, the chunk list and the pairs' token numbers too, so the tile
+// loop touches global memory only for weights (two tile buffers, refilled as soon as reduced) and for the results.
+constexpr int kStreamTokens = 16;
+constexpr int kStreamMaxD = 4096;
+constexpr int kStreamMaxPairs = 256;   // pairs and chunks the LDS copies hold
+
+template <int RT, int NP, int SD>
+__global__ __launch_bounds__(512) void grouped_phase1_stream_kernel(ExpertTable tab, tf_expert_offsets off, const tf_prefill_group *chunks,
+                                                                    const uint32_t *chunk_count, const tf_prefill_pair *pairs,
+                                                                    uint32_t n_pairs, const half_t *hidden, long hidden_stride,
+                                                                    uint32_t tokens, half_t *acts, uint32_t acts_pair_base, int d, int f) {
+    __shared__ __align__(16) u32x4 xa[kStreamTokens * kStreamMaxD / 8];
+    __shared__ float xsum[kStreamTokens * kStreamMaxD / 32];
+    __shared__ uint32_t pair_token[kStreamMaxPairs];
+    __shared__ uint32_t ch_expert[kStreamMaxPairs], ch_start[kStreamMaxPairs], ch_count[kStreamMaxPairs];
+    const int lane = threadIdx.x & 63;
+    const int nch = d >> 5, pieces = d >> 3;
+    // everything the prologue needs is requested before anything is used
+    u32x4 raw[kStreamTokens];
+#pragma unroll
+    for (int t = 0; t < kStreamTokens; ++t) {
+        raw[t] = u32x4{0u, 0u, 0u, 0u};
+        if ((uint32_t)t < tokens && (int)threadIdx.x < pieces) raw[t] = load16(hidden + (size_t)t * hidden_stride + threadIdx.x * 8);
+    }
+    uint32_t n_chunks = *chunk_count;
+    n_chunks = n_chunks < (uint32_t)kStreamMaxPairs ? n_chunks : (uint32_t)kStreamMaxPairs;
+    if (threadIdx.x < n_chunks) {
+        const tf_prefill_group c = chunks[threadIdx.x];
+        ch_expert[threadIdx.x] = c.expert;
+        ch_start[threadIdx.x] = c.pair_start;
+        ch_count[threadIdx.x] = c.pair_count;
+    }
+    if (threadIdx.x < n_pairs) {
+        const uint32_t t = pairs[threadIdx.x].token;
+        pair_token[threadIdx.x] = t < tokens ? t : tokens - 1;
+    }
+    __syncthreads();
+    const uint32_t tpe = (uint32_t)(f + RT - 1) / RT;                 // tiles per expert
+    const uint32_t total = n_chunks * tpe;
+    const uint32_t wave = uniform_u32((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
+    const uint32_t nwaves = (gridDim.x * blockDim.x) >> 6;
+    RowStream<RT, NP> rs;
+    typename RowStream<RT, NP>::Tile ga, ua, gb, ub;
+    rs.init_map(d, lane);
+    auto request = [&](typename RowStream<RT, NP>::Tile &tg, typename RowStream<RT, NP>::Tile &tu, uint32_t at) {
+        const uint32_t c = uniform_u32(at / tpe);
+        const uint32_t row0 = (at - c * tpe) * RT;
+        const uint8_t *base = uniform_ptr(expert_base(tab, ch_expert[c]));
+        const size_t w_byte = (size_t)row0 * (d >> 1), sb_byte = (size_t)row0 * (d >> 6) * 2;
+        rs.load(tg, base + off.gate_W_off + w_byte, base + off.gate_s_off + sb_byte, base + off.gate_b_off + sb_byte, f - row0);
+        rs.load(tu, base + off.up_W_off + w_byte, base + off.up_s_off + sb_byte, base + off.up_b_off + sb_byte, f - row0);
+    };
+    uint32_t t0 = wave, t1 = wave + nwaves;
+    if (t0 < total) request(ga, ua, t0);
+    if (t1 < total) request(gb, ub, t1);
+    // arrange the activations while the first tiles are in flight
+#pragma unroll
+    for (int t = 0; t < kStreamTokens; ++t)
+        if ((uint32_t)t < tokens) XStage::publish_piece(raw[t], threadIdx.x, pieces, nch, xa + (size_t)t * pieces, xsum + (size_t)t * nch);
+    __syncthreads();
+    if (t0 >= total) return;
+    auto consume = [&](const typename RowStream<RT, NP>::Tile &tg, const typename RowStream<RT, NP>::Tile &tu, uint32_t at) {
+        const uint32_t c = uniform_u32(at / tpe);
+        const uint32_t row0 = (at - c * tpe) * RT;
+        const uint32_t first = uniform_u32(ch_start[c]), count = uniform_u32(ch_count[c]);
+        for (uint32_t j = 0; j < count; ++j) {
+            const uint32_t pi = first + j;
+            const uint32_t token = uniform_u32(pair_token[pi < (uint32_t)kStreamMaxPairs ? pi : 0]);
+            rs.init_x_lds(xa + (size_t)token * pieces, xsum + (size_t)token * nch, d);
+            float gate[RT], up[RT];
+            rs.template reduce<SD>(tg, gate);
+            rs.template reduce<SD>(tu, up);
+            if (lane == 0) {
+#pragma unroll
+                for (int r = 0; r < RT; ++r)
+                    if (row0 + r < (uint32_t)f) store_act(acts, (size_t)(pi - acts_pair_base) * f + row0 + r, gate[r], up[r]);
+            }
+        }
+    };
+    for (;;) {
+        consume(ga, ua, t0);
+        t0 += 2 * nwaves;
+        if (t0 < total) request(ga, ua, t0);
+        if (t1 >= total) break;
+        consume(gb, ub, t1);
+        t1 += 2 * nwaves;
+        if (t1 < total) request(gb, ub, t1);
+        if (t0 >= total) break;
+    }
+}
+
 template <int SD>
 __global__ __launch_bounds__(256) void grouped_phase1_generic_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl,
                                                                      const tf_prefill_pair *pairs, const half_t *hidden,
@@ -477,9 +570,20 @@ __global__ __launch_bounds__(256) void grouped_down_short_kernel(ExpertTable tab
 #pragma unroll
     for (int p = 0; p < NPASS; ++p)
         sr.load(t[p], base + off.down_W_off, base + off.down_s_off, base + off.down_b_off, row0 + 2 * p, d, f);
+    // the pair record and the activations of pair j + 1 are requested before pair j is reduced
+    const int col = sr.col < 0 ? 0 : sr.col;
+    auto fetch = [&](uint32_t j, tf_prefill_pair &pr, u32x4 *xr) {
+        pr = pairs[ch.pair_start + j];
+        const half_t *a = acts + (size_t)(ch.pair_start + j - acts_pair_base) * f + col * 32;
+#pragma unroll
+        for (int dd = 0; dd < 4; ++dd) xr[dd] = load16(a + dd * 8);
+    };
+    tf_prefill_pair pr, pr_next;
+    u32x4 xr[4], xr_next[4];
+    fetch(0, pr, xr);
     for (uint32_t j = 0; j < ch.pair_count; ++j) {
-        const tf_prefill_pair pr = pairs[ch.pair_start + j];
-        sr.init_x(acts + (size_t)(ch.pair_start + j - acts_pair_base) * f);
+        if (j + 1 < ch.pair_count) fetch(j + 1, pr_next, xr_next);
+        sr.xs = arrange_x(xr, sr.xq);
         half_t *out = route_partials + ((size_t)pr.token * top_k + pr.rank) * d;
 #pragma unroll
         for (int p = 0; p < NPASS; ++p) {
@@ -490,6 +594,9 @@ __global__ __launch_bounds__(256) void grouped_down_short_kernel(ExpertTable tab
                 if (row0 + 2 * p + 1 < d) out[row0 + 2 * p + 1] = (half_t)hi;
             }
         }
+        pr = pr_next;
+#pragma unroll
+        for (int dd = 0; dd < 4; ++dd) xr[dd] = xr_next[dd];
     }
 }
 
@@ -547,7 +654,8 @@ bool table_aligned(const ExpertTable &t) {
 
 // use_mfma: the chunks are large enough for the matrix cores to pay
 int32_t run_grouped(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off, const ChunkList &cl,
-                    uint32_t n_chunks_upper, const GroupedGeom &g, tf_dtype sd, bool use_mfma) {
+                    uint32_t n_chunks_upper, const GroupedGeom &g, tf_dtype sd, bool use_mfma, uint32_t stream_tokens = 0,
+                    uint32_t stream_pairs = 0) {
     if (n_chunks_upper == 0) return TF_OK;
     const bool blobs16 = table_aligned(tab);
     const bool hidden16 = aligned16(g.hidden) && g.hidden_stride % 8 == 0;
@@ -561,7 +669,25 @@ int32_t run_grouped(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const t
     } else {
         const LongPlan plan = plan_long_rows(g.d);
         bool launched = false;
-        if (p1_fast && g.d > 1024 && plan.rt > 0) {
+        // all tokens known and few: persistent streaming with the activations staged in LDS
+        if (p1_fast && tab.pool && cl.dev && stream_tokens > 0 && stream_tokens <= (uint32_t)kStreamTokens && stream_pairs <= (uint32_t)kStreamMaxPairs &&
+            g.d > 1024 && g.d <= kStreamMaxD && g.d <= 512 * 8 && plan.rt > 0) {
+            const dim3 grid((uint32_t)ctx->num_cus);
+#define TF_GP1S(RT_, NP_)                                                                                                  \
+    if (!launched && plan.rt == RT_ && plan.np == NP_) {                                                                   \
+        launched = true;                                                                                                   \
+        if (sd == TF_BF16)                                                                                                 \
+            hipLaunchKernelGGL((grouped_phase1_stream_kernel<RT_, NP_, 0>), grid, dim3(512), 0, st, tab, off, cl.dev, cl.dev_n, g.pairs, \
+                               stream_pairs, g.hidden, g.hidden_stride, stream_tokens, g.acts, g.acts_pair_base, g.d, g.f); \
+        else                                                                                                               \
+            hipLaunchKernelGGL((grouped_phase1_stream_kernel<RT_, NP_, 1>), grid, dim3(512), 0, st, tab, off, cl.dev, cl.dev_n, g.pairs, \
+                               stream_pairs, g.hidden, g.hidden_stride, stream_tokens, g.acts, g.acts_pair_base, g.d, g.f); \
+    }
+            TF_GP1S(1, 1) TF_GP1S(1, 2) TF_GP1S(1, 3) TF_GP1S(1, 4) TF_GP1S(2, 1) TF_GP1S(2, 2) TF_GP1S(2, 3) TF_GP1S(2, 4)
+            TF_GP1S(4, 1) TF_GP1S(4, 2) TF_GP1S(4, 3) TF_GP1S(4, 4)
+#undef TF_GP1S
+        }
+        if (!launched && p1_fast && g.d > 1024 && plan.rt > 0) {
             const dim3 grid(((g.f + plan.rt - 1) / plan.rt + 3) / 4, n_chunks_upper);
 #define TF_GP1(RT_, NP_)                                                                                                   \
     if (!launched && plan.rt == RT_ && plan.np == NP_) {                                                                   \
@@ -884,7 +1010,9 @@ int32_t tf_prefill_grouped_routed_moe_resident(tf_ctx *ctx, tf_stream stream, co
                   (int)f, (int)top_k};
     // the host only knows the average group size: matrix cores once experts see 8 or more tokens on average
     const bool use_mfma = (uint64_t)pair_count >= (uint64_t)num_experts * 8;
-    return run_grouped(ctx, static_cast<hipStream_t>(stream), tab, *routed_offsets, cl, max_chunks, g, scale_dtype, use_mfma);
+    // the pairs are all (token, rank) combinations of pair_count / top_k token rows
+    const uint32_t tokens = pair_count % top_k == 0 ? pair_count / top_k : 0u;
+    return run_grouped(ctx, static_cast<hipStream_t>(stream), tab, *routed_offsets, cl, max_chunks, g, scale_dtype, use_mfma, tokens, pair_count);
 }
 
 int32_t tf_prefill_moe_reduce_token_major(tf_ctx *ctx, tf_stream stream, const void *route_partials, uint64_t route_partials_offset,

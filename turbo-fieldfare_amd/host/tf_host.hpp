@@ -414,6 +414,26 @@ private:
     uint32_t vocab_;
 };
 
+
+// FusedQKVGEMV (Kernels/Fusions/FusedQKVGEMV.swift)
+class FusedQKVGEMV {
+public:
+    explicit FusedQKVGEMV(const Context &context) : c_(context) {}
+    void encode(const void *qWeights, uint64_t qWeightsOffset, const void *qScales, uint64_t qScalesOffset, const void *qBiases,
+                uint64_t qBiasesOffset, const void *kWeights, uint64_t kWeightsOffset, const void *kScales, uint64_t kScalesOffset,
+                const void *kBiases, uint64_t kBiasesOffset, const void *vWeights, uint64_t vWeightsOffset, const void *vScales,
+                uint64_t vScalesOffset, const void *vBiases, uint64_t vBiasesOffset, const void *x, void *qOut, uint64_t qOutOffset,
+                void *kOut, uint64_t kOutOffset, void *vOut, uint64_t vOutOffset, uint32_t qRows, uint32_t kvRows, uint32_t n) const {
+        c_.check(tf_fused_qkv_gemv(c_.raw(), c_.stream(), qWeights, qWeightsOffset, qScales, qScalesOffset, qBiases, qBiasesOffset, kWeights,
+                                   kWeightsOffset, kScales, kScalesOffset, kBiases, kBiasesOffset, vWeights, vWeightsOffset, vScales,
+                                   vScalesOffset, vBiases, vBiasesOffset, x, qOut, qOutOffset, kOut, kOutOffset, vOut, vOutOffset, qRows, kvRows,
+                                   n, TF_BF16));
+    }
+
+private:
+    const Context &c_;
+};
+
 // MPPPrefillInt4QMM (Kernels/TensorCore/MPPPrefillInt4QMM.swift)
 class MPPPrefillInt4QMM {
 public:
