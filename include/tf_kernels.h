@@ -466,6 +466,17 @@ int32_t tf_sample(tf_ctx *ctx, tf_stream stream, const void *probs, void *out_to
 int32_t tf_sample_topk64(tf_ctx *ctx, tf_stream stream, const void *probs, void *out_token, uint32_t vocab, float temperature, float top_p,
                          uint64_t seed);
 
+/* ---- resident experts ------------------------------------------------------------------------------------------ */
+/* Fills a caller-owned device pool [num_experts, expert_stride] from one packed-experts layer file
+ * (packed_experts/layer_XX.bin: num_experts blobs of expert_stride bytes), placing LOGICAL expert e, stored at position
+ * physical_rank[e] of the file (host array; NULL = identity), at pool + e * expert_stride.  Replaces the reference's SSD
+ * streamer + slot cache (Runtime/Inference/ModelExpertIO.swift:45-110, Infrastructure/Streaming/PreadExpertStreamer.swift) with one
+ * upload per layer; the layout comes from packed_experts/layout.json (GTurboPackedExpertsLayoutV1.swift).
+ * Blocks until the upload is complete.  The file must be a regular file of exactly num_experts * expert_stride bytes
+ * (TF_ERR_DIMENSION_MISMATCH otherwise). */
+int32_t tf_upload_packed_experts_layer(tf_ctx *ctx, tf_stream stream, const char *layer_file_path, uint64_t expert_stride,
+                                       uint32_t num_experts, const uint32_t *physical_rank, void *device_pool);
+
 #ifdef __cplusplus
 }
 #endif
