@@ -714,7 +714,7 @@ int32_t run_grouped(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const t
     }
     if (rc != TF_OK) return rc;
     // ---- down
-    if (use_mfma && dn_fast) {
+    if (use_mfma && dn_fast && aligned16(g.route_partials)) {
         return launch_grouped_down_mfma(ctx, st, tab, off, cl, n_chunks_upper, g.pairs, g.acts, g.acts_pair_base, g.route_partials, g.d, g.f, g.top_k, sd);
     }
     if (dn_fast && g.f <= 1024) {

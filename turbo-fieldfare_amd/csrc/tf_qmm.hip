@@ -37,10 +37,40 @@ __device__ __forceinline__ void zero_acc(float16_t acc[4][2]) {
             for (int r = 0; r < 16; ++r) acc[mt][j][r] = 0.0f;
 }
 
+// ---- output tiles
+// The accumulator layout gives a lane one column of 16 scattered rows: written straight to memory that is a 2-byte store
+// per value, 64-byte runs per wave.  Instead the block's tile goes through LDS (free once the K loop has drained) as fp16
+// and leaves as 16-byte pieces of whole rows: 512-byte (256-column tiles) or 256-byte runs per row.
+constexpr int kOutPadBytes = 16;   // keeps the rows of a wave's two half-waves on different LDS banks
+
+template <int COLS>
+__device__ __forceinline__ uint32_t out_tile_offset(int row, int col) {
+    return (uint32_t)row * (uint32_t)(COLS * 2 + kOutPadBytes) + (uint32_t)col * 2u;
+}
+template <int COLS>
+__device__ __forceinline__ void out_tile_put(uint8_t *lds, int row, int col, float v) {
+    *reinterpret_cast<half_t *>(lds + out_tile_offset<COLS>(row, col)) = (half_t)v;
+}
+// row_base(row): where column 0 of the block's tile of that row lives (16-byte aligned); rows_valid / cols_valid bound
+// the part of the tile that exists (cols_valid a multiple of 8).  Ends with every thread past the barrier it needs.
+template <int COLS, typename RowBase>
+__device__ __forceinline__ void out_tile_store(const uint8_t *lds, int rows_valid, int cols_valid, RowBase row_base) {
+    constexpr int kPieces = COLS / 8;
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < kQmmBM * kPieces; idx += 256) {
+        const int row = idx / kPieces, piece = idx - row * kPieces;
+        if (row < rows_valid && piece * 8 < cols_valid) {
+            const u32x4 v = *reinterpret_cast<const u32x4 *>(lds + out_tile_offset<COLS>(row, piece * 8));
+            *reinterpret_cast<u32x4 *>(row_base(row) + piece * 8) = v;
+        }
+    }
+}
+static_assert(kQmmBM * (kQmmBN * 2 + kOutPadBytes) + kQmmBM * 4 <= kQmmLdsBytes, "the output tile and its row table must fit the K loop's LDS");
+
 // ------------------------------------------------------------------------------------------------ dense
 template <int SD>
 __global__ __launch_bounds__(256, 2) void qmm_dense_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *X,
-                                                           long ldx, half_t *Y, long ldy, int M, int N, int K) {
+                                                           long ldx, half_t *Y, long ldy, int M, int N, int K, bool rows_vectorizable) {
     __shared__ __align__(128) uint8_t lds[kQmmLdsBytes];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int n0 = blockIdx.x * kQmmBN + wave * kQmmWaveN, m0 = blockIdx.y * kQmmBM;
@@ -55,6 +85,19 @@ __global__ __launch_bounds__(256, 2) void qmm_dense_kernel(const uint8_t *W, con
     float16_t acc[4][2];
     zero_acc(acc);
     qmm_k_loop<SD>(K >> 6, arow, rows, (uint32_t)(uintptr_t)lds, lane, row_tiles, acc);
+    if (rows_vectorizable) {
+        __syncthreads();   // every wave has left the K loop and nothing it requested is still on its way into LDS
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    out_tile_put<kQmmBN>(lds, mt * 32 + acc_row(r, lane), wave * kQmmWaveN + j * 32 + acc_col(lane), acc[mt][j][r]);
+        const int nb = blockIdx.x * kQmmBN;
+        out_tile_store<kQmmBN>(lds, min(kQmmBM, M - m0), min(kQmmBN, N - nb), [&](int row) { return Y + (size_t)(m0 + row) * ldy + nb; });
+        return;
+    }
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int n = n0 + j * 32 + acc_col(lane);
@@ -66,6 +109,19 @@ __global__ __launch_bounds__(256, 2) void qmm_dense_kernel(const uint8_t *W, con
                 if (m < M && n < N) Y[(size_t)m * ldy + n] = (half_t)acc[mt][j][r];
             }
     }
+}
+
+// Block number -> (chunk, column tile) for the grouped kernels.  Workgroups go to the 8 XCDs round-robin by linear id and
+// each XCD has its own L2; the column tiles of one chunk all read the same activation rows, so they are given ids that
+// are congruent modulo 8: a run of 8 * tiles consecutive ids serves 8 chunks, one per XCD, and a chunk's activations are
+// fetched into one L2 once instead of into all eight.
+constexpr uint32_t kXcds = 8;
+__device__ __forceinline__ void chunk_and_tile(uint32_t tiles, uint32_t &chunk, uint32_t &tile) {
+    const uint32_t id = blockIdx.x;
+    const uint32_t run = kXcds * tiles;
+    const uint32_t within = id % run;
+    chunk = (id / run) * kXcds + within % kXcds;
+    tile = within / kXcds;
 }
 
 // ------------------------------------------------------------------------------------------------ grouped phase 1
@@ -81,7 +137,9 @@ __global__ __launch_bounds__(256, 2) void grouped_phase1_mfma_kernel(ExpertTable
                                                                      int D, int F) {
     __shared__ __align__(128) uint8_t lds[kQmmLdsBytes];
     tf_prefill_group ch;
-    if (!get_chunk(cl, blockIdx.y, ch)) return;
+    uint32_t chunk_index, col_tile;
+    chunk_and_tile((uint32_t)(F + kP1BN - 1) / kP1BN, chunk_index, col_tile);
+    if (!get_chunk(cl, chunk_index, ch)) return;
     // everything taken from the work list is the same in all lanes: say so, the descriptors built from it live in
     // scalar registers
     ch.expert = uniform_u32(ch.expert);
@@ -90,7 +148,7 @@ __global__ __launch_bounds__(256, 2) void grouped_phase1_mfma_kernel(ExpertTable
     const uint8_t *base = uniform_ptr(expert_base(tab, ch.expert));
     if (!base) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n0 = blockIdx.x * kP1BN + wave * 32;
+    const int n0 = (int)col_tile * kP1BN + wave * 32;
     // the pairs of a chunk ascend by token: offsets are taken from the first pair's row
     const uint32_t token0 = uniform_u32(pairs[ch.pair_start].token);
     QmmARows arow;
@@ -109,15 +167,16 @@ __global__ __launch_bounds__(256, 2) void grouped_phase1_mfma_kernel(ExpertTable
     float16_t acc[4][2];
     zero_acc(acc);
     qmm_k_loop<SD>(D >> 6, arow, rows, (uint32_t)(uintptr_t)lds, lane, row_tiles, acc);
-    const int n = n0 + acc_col(lane);
+    // acts rows of a chunk are consecutive; F % 64 == 0 and a 16-byte aligned acts keep every row piece aligned
+    __syncthreads();
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const uint32_t m = mt * 32 + acc_row(r, lane);
-            if (m < ch.pair_count && n < F)
-                acts[(size_t)(ch.pair_start + m - acts_pair_base) * F + n] = (half_t)(gelu_tanh(acc[mt][0][r]) * acc[mt][1][r]);
-        }
+        for (int r = 0; r < 16; ++r)
+            out_tile_put<kP1BN>(lds, mt * 32 + acc_row(r, lane), wave * 32 + acc_col(lane), gelu_tanh(acc[mt][0][r]) * acc[mt][1][r]);
+    const int nb = (int)col_tile * kP1BN;
+    half_t *tile = acts + (size_t)(ch.pair_start - acts_pair_base) * F + nb;
+    out_tile_store<kP1BN>(lds, (int)ch.pair_count, min(kP1BN, F - nb), [&](int row) { return tile + (size_t)row * F; });
 }
 
 // ------------------------------------------------------------------------------------------------ grouped down
@@ -130,7 +189,9 @@ __global__ __launch_bounds__(256, 2) void grouped_down_mfma_kernel(ExpertTable t
                                                                    int top_k) {
     __shared__ __align__(128) uint8_t lds[kQmmLdsBytes];
     tf_prefill_group ch;
-    if (!get_chunk(cl, blockIdx.y, ch)) return;
+    uint32_t chunk_index, col_tile;
+    chunk_and_tile((uint32_t)(D + kQmmBN - 1) / kQmmBN, chunk_index, col_tile);
+    if (!get_chunk(cl, chunk_index, ch)) return;
     // everything taken from the work list is the same in all lanes: say so, the descriptors built from it live in
     // scalar registers
     ch.expert = uniform_u32(ch.expert);
@@ -139,7 +200,7 @@ __global__ __launch_bounds__(256, 2) void grouped_down_mfma_kernel(ExpertTable t
     const uint8_t *base = uniform_ptr(expert_base(tab, ch.expert));
     if (!base) return;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n0 = blockIdx.x * kQmmBN + wave * kQmmWaveN;
+    const int n0 = (int)col_tile * kQmmBN + wave * kQmmWaveN;
     QmmARows arow;
     arow.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(acts + (size_t)(ch.pair_start - acts_pair_base) * F), 0, (int)0xFFFFFFFFu, 0x00020000);
 #pragma unroll
@@ -156,21 +217,22 @@ __global__ __launch_bounds__(256, 2) void grouped_down_mfma_kernel(ExpertTable t
     float16_t acc[4][2];
     zero_acc(acc);
     qmm_k_loop<SD>(F >> 6, arow, rows, (uint32_t)(uintptr_t)lds, lane, row_tiles, acc);
+    __syncthreads();
+    // where each row of the tile goes: route_partials row token * top_k + rank (D % 64 == 0 keeps the pieces aligned)
+    uint32_t *row_slot = reinterpret_cast<uint32_t *>(lds + kQmmBM * (kQmmBN * 2 + kOutPadBytes));
+    if (threadIdx.x < ch.pair_count) {
+        const tf_prefill_pair p = pairs[ch.pair_start + threadIdx.x];
+        row_slot[threadIdx.x] = p.token * (uint32_t)top_k + p.rank;
+    }
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const uint32_t m = mt * 32 + acc_row(r, lane);
-            if (m < ch.pair_count) {
-                const tf_prefill_pair p = pairs[ch.pair_start + m];
-                half_t *out = route_partials + ((size_t)p.token * top_k + p.rank) * D;
+        for (int j = 0; j < 2; ++j)
 #pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int n = n0 + j * 32 + acc_col(lane);
-                    if (n < D) out[n] = (half_t)acc[mt][j][r];
-                }
-            }
-        }
+            for (int r = 0; r < 16; ++r)
+                out_tile_put<kQmmBN>(lds, mt * 32 + acc_row(r, lane), wave * kQmmWaveN + j * 32 + acc_col(lane), acc[mt][j][r]);
+    const int nb = (int)col_tile * kQmmBN;
+    out_tile_store<kQmmBN>(lds, (int)ch.pair_count, min(kQmmBN, D - nb), [&](int row) { return route_partials + (size_t)row_slot[row] * D + nb; });
 }
 
 }  // namespace
@@ -185,7 +247,7 @@ int32_t launch_grouped_phase1_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTabl
                                    const ChunkList &cl, uint32_t n_chunks_upper, const tf_prefill_pair *pairs,
                                    const half_t *hidden, long hidden_stride, half_t *acts, uint32_t acts_pair_base, int d, int f,
                                    tf_dtype sd) {
-    const dim3 grid((f + kP1BN - 1) / kP1BN, n_chunks_upper);
+    const dim3 grid((uint32_t)((f + kP1BN - 1) / kP1BN) * ((n_chunks_upper + kXcds - 1) / kXcds * kXcds));
     if (sd == TF_BF16)
         hipLaunchKernelGGL(grouped_phase1_mfma_kernel<0>, grid, dim3(256), 0, st, tab, off, cl, pairs, hidden, hidden_stride, acts, acts_pair_base, d, f);
     else
@@ -196,7 +258,7 @@ int32_t launch_grouped_phase1_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTabl
 int32_t launch_grouped_down_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off,
                                  const ChunkList &cl, uint32_t n_chunks_upper, const tf_prefill_pair *pairs, const half_t *acts,
                                  uint32_t acts_pair_base, half_t *route_partials, int d, int f, int top_k, tf_dtype sd) {
-    const dim3 grid((d + kQmmBN - 1) / kQmmBN, n_chunks_upper);
+    const dim3 grid((uint32_t)((d + kQmmBN - 1) / kQmmBN) * ((n_chunks_upper + kXcds - 1) / kXcds * kXcds));
     if (sd == TF_BF16)
         hipLaunchKernelGGL(grouped_down_mfma_kernel<0>, grid, dim3(256), 0, st, tab, off, cl, pairs, acts, acts_pair_base, route_partials, d, f, top_k);
     else
@@ -222,10 +284,11 @@ int32_t tf_int4_qmm(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t
     const dim3 grid((n + kQmmBN - 1) / kQmmBN, (m + kQmmBM - 1) / kQmmBM);
     hipStream_t st = static_cast<hipStream_t>(stream);
     half_t *yp = reinterpret_cast<half_t *>(at(y, y_offset));
+    const bool rows_vec = aligned16(yp) && n % 8 == 0;   // whole 16-byte pieces of output rows
     if (scale_dtype == TF_BF16)
-        hipLaunchKernelGGL(qmm_dense_kernel<0>, grid, dim3(256), 0, st, w, at(scales, scales_offset), at(biases, biases_offset), xp, (long)k, yp, (long)n, m, n, k);
+        hipLaunchKernelGGL(qmm_dense_kernel<0>, grid, dim3(256), 0, st, w, at(scales, scales_offset), at(biases, biases_offset), xp, (long)k, yp, (long)n, m, n, k, rows_vec);
     else
-        hipLaunchKernelGGL(qmm_dense_kernel<1>, grid, dim3(256), 0, st, w, at(scales, scales_offset), at(biases, biases_offset), xp, (long)k, yp, (long)n, m, n, k);
+        hipLaunchKernelGGL(qmm_dense_kernel<1>, grid, dim3(256), 0, st, w, at(scales, scales_offset), at(biases, biases_offset), xp, (long)k, yp, (long)n, m, n, k, rows_vec);
     return check_launch(ctx, "int4_qmm");
 }
 
