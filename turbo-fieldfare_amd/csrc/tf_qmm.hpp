@@ -1,6 +1,6 @@
 // int4 x fp16 matrix multiply on the CDNA4 matrix cores: Y[M,N] = X[M,K] . W[N,K]^T with W in the affine group-64
-// int4 layout.  A 256-thread block owns a 128 x 256 output tile (four waves, each 128 rows x 64 columns) and walks K one
-// quantization group (64) at a time:
+// int4 layout.  A block of four (or eight) waves owns a 128 x 256 (or 128 x 512) output tile, each wave 128 rows x 64
+// columns, and walks K one quantization group (64) at a time:
 //
 //   W   In v_mfma_f32_32x32x16_f16 lane (i, kb) supplies, for output column i, the 8 weights of k-slots 8 kb .. 8 kb + 7.
 //       The lane reads 16 packed bytes of "its" row (32 nibbles: the kb-th half of the group) and expands one 32-bit
@@ -31,11 +31,19 @@ typedef float float16_t __attribute__((ext_vector_type(16)));
 
 constexpr int kQmmBM = 128;      // rows per block tile (4 MFMA row tiles)
 constexpr int kQmmWaveN = 64;    // columns per wave (2 MFMA column tiles)
-constexpr int kQmmBN = 256;      // columns per block tile (4 waves)
-constexpr int kQmmAChunks = kQmmBM * 8 / 256;    // 16-byte X chunks copied per thread and K step
 constexpr int kQmmStageBytes = kQmmBM * 8 * 16;  // one X stage
 constexpr int kQmmWBytes = 64 * 64;               // packed W rows of one wave for two K steps: 64 rows x 64 bytes
-constexpr int kQmmLdsBytes = 3 * kQmmStageBytes + 4 * 2 * kQmmWBytes;   // X ring + two W buffers per wave
+// A block is NW waves (4 or 8) that share the X ring: with 8 waves the same activation rows serve twice as many output
+// columns, so a tile's activations are fetched half as often; such a block has a CU to itself.
+template <int NW>
+struct QmmGeom {
+    static constexpr int kThreads = NW * 64;
+    static constexpr int kBN = NW * kQmmWaveN;                                     // columns per block tile
+    static constexpr int kAChunks = kQmmBM * 8 / kThreads;                         // 16-byte X chunks copied per thread and K step
+    static constexpr int kLoopLdsBytes = 3 * kQmmStageBytes + NW * 2 * kQmmWBytes; // X ring + two W buffers per wave
+};
+constexpr int kQmmBN = QmmGeom<4>::kBN;
+constexpr int kQmmLdsBytes = QmmGeom<4>::kLoopLdsBytes;
 
 // 8 nibbles of one word -> 8 fp16 weights half(q * s + b) in element order.  A byte holds two neighbouring elements:
 // v_perm_b32 copies it into both halves of a register, one mask leaves the low nibble in the low half as 1024 + q
@@ -62,18 +70,25 @@ __device__ __forceinline__ half2_t sb_to_half2(uint16_t v) {
 // 16-byte slot of X chunk (row r, chunk c of 8) inside one stage
 __device__ __forceinline__ int a_slot(int r, int c) { return r * 8 + (c ^ ((r >> 1) & 7)); }
 
-// What a thread needs to know about the X chunks it copies: slot 256 q + threadIdx.x of every stage receives the chunk
+// What a thread needs to know about the X chunks it copies: slot (threads per block) q + threadIdx.x of every stage receives the chunk
 // at byte offset off[q] + 128 kt of the tensor the descriptor covers (rows beyond the tile repeat a valid row; nobody
 // reads what they produce).  32-bit offsets: the rows of one tile must lie within 4 GiB of the descriptor's base.
 typedef __amdgpu_buffer_rsrc_t qmm_rsrc_t;
+// 16 bytes per lane from a buffer straight into LDS: lane l's bytes land at dst + 16 l (dst wave-uniform)
+__device__ __forceinline__ void lds_copy16(qmm_rsrc_t rsrc, uint32_t dst, uint32_t lane_offset, int uniform_offset) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)(uintptr_t)dst, 16, lane_offset, uniform_offset, 0, 0);
+}
+template <int NW>
 struct QmmARows {
     qmm_rsrc_t rsrc;
-    uint32_t off[kQmmAChunks];
+    uint32_t off[QmmGeom<NW>::kAChunks];
 };
-__device__ __forceinline__ int qmm_a_row_of(int q) { return (256 * q + (int)threadIdx.x) >> 3; }
+template <int NW>
+__device__ __forceinline__ int qmm_a_row_of(int q) { return (QmmGeom<NW>::kThreads * q + (int)threadIdx.x) >> 3; }
 // row_byte_offset: where the row of slot group q starts, relative to the descriptor's base
-__device__ __forceinline__ void qmm_a_rows_set(QmmARows &a, int q, uint64_t row_byte_offset) {
-    const int p = 256 * q + (int)threadIdx.x, r = p >> 3;
+template <int NW>
+__device__ __forceinline__ void qmm_a_rows_set(QmmARows<NW> &a, int q, uint64_t row_byte_offset) {
+    const int p = QmmGeom<NW>::kThreads * q + (int)threadIdx.x, r = p >> 3;
     a.off[q] = (uint32_t)row_byte_offset + (uint32_t)(((p & 7) ^ ((r >> 1) & 7)) * 16);
 }
 
@@ -113,18 +128,15 @@ __device__ __forceinline__ void qmm_sb_load(QmmSB &sb, const QmmBRows &rows, int
 // packed W rows of K steps 2 pair, 2 pair + 1 -> the wave's LDS buffer at byte address `dst` (wave-uniform)
 __device__ __forceinline__ void qmm_w_copy(const QmmBRows &rows, int pair, uint32_t dst) {
 #pragma unroll
-    for (int t = 0; t < 4; ++t)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(rows.w[t >> 1], (__attribute__((address_space(3))) void *)(uintptr_t)(dst + t * 1024u), 16,
-                                                 rows.copy_off[t], pair * 64, 0, 0);
+    for (int t = 0; t < 4; ++t) lds_copy16(rows.w[t >> 1], dst + t * 1024u, rows.copy_off[t], pair * 64);
 }
 
-// X tile of step kt -> LDS stage at byte address `stage` (wave-uniform); four copies of 64 x 16 bytes per wave
-__device__ __forceinline__ void qmm_a_copy(const QmmARows &a, int kt, uint32_t stage) {
+// X tile of step kt -> LDS stage at byte address `stage` (wave-uniform); kAChunks copies of 64 x 16 bytes per wave
+template <int NW>
+__device__ __forceinline__ void qmm_a_copy(const QmmARows<NW> &a, int kt, uint32_t stage) {
     const uint32_t wave_base = stage + (threadIdx.x >> 6) * 1024u;
 #pragma unroll
-    for (int q = 0; q < kQmmAChunks; ++q)
-        __builtin_amdgcn_raw_ptr_buffer_load_lds(a.rsrc, (__attribute__((address_space(3))) void *)(uintptr_t)(wave_base + q * 4096u), 16,
-                                                 a.off[q], kt * 128, 0, 0);
+    for (int q = 0; q < QmmGeom<NW>::kAChunks; ++q) lds_copy16(a.rsrc, wave_base + (uint32_t)q * (uint32_t)(QmmGeom<NW>::kThreads * 16), a.off[q], kt * 128);
 }
 
 // ds_read_b128 at addr + OFFSET, invisible to the compiler's memory tracking (see the header comment)
@@ -195,16 +207,17 @@ __device__ __forceinline__ void qmm_group(const u32x4 w[2], const QmmSB &sb, con
 // The K loop.  The X tile of step kt lives in LDS stage kt % 3; the packed W rows of steps 2p, 2p + 1 in the wave's
 // buffer p & 1, the scales / biases of those two groups in register slot p & 1.
 // Even step kt = 2p:  barrier; request X(kt + 2), W(p + 1); multiply with the W words read from LDS at the end of the
-//                     previous step; request the scales of pair p + 1; wait for X(kt + 1) (12 newer requests stay in
-//                     flight).
-// Odd step:           barrier; request X(kt + 2); multiply; wait for X(kt + 1), W(p + 1) and the scales (4 newer
-//                     requests stay in flight); read the W words of both steps of pair p + 1 from LDS, switch to
-//                     its scales.
+//                     previous step; request the scales of pair p + 1; wait for X(kt + 1) (the kAChunks + 8 newer
+//                     requests stay in flight).
+// Odd step:           barrier; request X(kt + 2); multiply; wait for X(kt + 1), W(p + 1) and the scales (the kAChunks
+//                     newer requests stay in flight); read the W words of both steps of pair p + 1 from LDS, switch
+//                     to its scales.
 // Requests are unconditional: past the end they repeat the last step or pair, which nobody reads, so that the number
 // of requests in flight is the same at every wait.
-template <int SD, int RT>
+template <int SD, int RT, int NW>
 struct QmmLoop {
-    const QmmARows &a;
+    static_assert(QmmGeom<NW>::kAChunks == 4 || QmmGeom<NW>::kAChunks == 2, "the waits below are written for 4 or 2 X copies per step");
+    const QmmARows<NW> &a;
     const QmmBRows &rows;
     uint32_t lds;
     uint32_t frag[4];
@@ -228,19 +241,21 @@ struct QmmLoop {
     __device__ __forceinline__ void even_step(int kt, float16_t acc[4][2]) {
         const int pair = kt >> 1;
         __builtin_amdgcn_s_barrier();
-        qmm_a_copy(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
+        qmm_a_copy<NW>(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
         qmm_w_copy(rows, min(pair + 1, last_pair), wbuf + (pb ^ kQmmWBytes));
         qmm_group<SD, RT, U3, 0>(w[0], sb, frag, acc);
         const int next_pair = min(pair + 1, last_pair);
         qmm_sb_load(sb_next, rows, next_pair, odd_count && next_pair == last_pair);
-        asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+        if constexpr (QmmGeom<NW>::kAChunks == 4) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
     }
     template <int U3>
     __device__ __forceinline__ void odd_step(int kt, float16_t acc[4][2]) {
         __builtin_amdgcn_s_barrier();
-        qmm_a_copy(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
+        qmm_a_copy<NW>(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
         qmm_group<SD, RT, U3, 1>(w[1], sb, frag, acc);
-        asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        if constexpr (QmmGeom<NW>::kAChunks == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
         pb ^= kQmmWBytes;
         read_w(wread + pb);
         sb = sb_next;
@@ -254,11 +269,11 @@ struct QmmLoop {
         const uint32_t frag0 = lds + (uint32_t)i * 128u + ((((uint32_t)kb * 4u) ^ (uint32_t)((i >> 1) & 7)) << 4);
 #pragma unroll
         for (int d = 0; d < 4; ++d) frag[d] = frag0 ^ ((uint32_t)d << 4);   // lds is 128-byte aligned
-        wbuf = lds + 3 * kQmmStageBytes + (threadIdx.x >> 6) * (2 * kQmmWBytes);
+        wbuf = lds + 3 * kQmmStageBytes + (threadIdx.x >> 6) * (2 * kQmmWBytes);   // NW such pairs of buffers follow the X ring
         wread = wbuf + (uint32_t)i * 64u + ((((uint32_t)kb) ^ (uint32_t)((i >> 2) & 3)) << 4);
         pb = 0;
-        qmm_a_copy(a, 0, lds);
-        qmm_a_copy(a, min(1, last), lds + kQmmStageBytes);
+        qmm_a_copy<NW>(a, 0, lds);
+        qmm_a_copy<NW>(a, min(1, last), lds + kQmmStageBytes);
         qmm_w_copy(rows, 0, wbuf);
         qmm_sb_load(sb, rows, 0, odd_count && last_pair == 0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -282,23 +297,23 @@ struct QmmLoop {
     }
 };
 
-template <int SD, int RT>
-__device__ __forceinline__ void qmm_k_loop_rt(int kt_count, const QmmARows &a, const QmmBRows &rows, uint32_t lds, int lane,
+template <int SD, int RT, int NW>
+__device__ __forceinline__ void qmm_k_loop_rt(int kt_count, const QmmARows<NW> &a, const QmmBRows &rows, uint32_t lds, int lane,
                                               float16_t acc[4][2]) {
-    QmmLoop<SD, RT> loop{a, rows, lds};
+    QmmLoop<SD, RT, NW> loop{a, rows, lds};
     loop.run(kt_count, lane, acc);
 }
 
 // row_tiles (1..4, block-uniform): 32-row tiles that hold rows; the others are not multiplied.
-// lds: byte address of kQmmLdsBytes of LDS, 128-byte aligned.
-template <int SD>
-__device__ __forceinline__ void qmm_k_loop(int kt_count, const QmmARows &a, const QmmBRows &rows, uint32_t lds, int lane,
+// lds: byte address of QmmGeom<NW>::kLoopLdsBytes of LDS, 128-byte aligned.
+template <int SD, int NW>
+__device__ __forceinline__ void qmm_k_loop(int kt_count, const QmmARows<NW> &a, const QmmBRows &rows, uint32_t lds, int lane,
                                            int row_tiles, float16_t acc[4][2]) {
     switch (row_tiles) {
-        case 1: qmm_k_loop_rt<SD, 1>(kt_count, a, rows, lds, lane, acc); break;
-        case 2: qmm_k_loop_rt<SD, 2>(kt_count, a, rows, lds, lane, acc); break;
-        case 3: qmm_k_loop_rt<SD, 3>(kt_count, a, rows, lds, lane, acc); break;
-        default: qmm_k_loop_rt<SD, 4>(kt_count, a, rows, lds, lane, acc); break;
+        case 1: qmm_k_loop_rt<SD, 1, NW>(kt_count, a, rows, lds, lane, acc); break;
+        case 2: qmm_k_loop_rt<SD, 2, NW>(kt_count, a, rows, lds, lane, acc); break;
+        case 3: qmm_k_loop_rt<SD, 3, NW>(kt_count, a, rows, lds, lane, acc); break;
+        default: qmm_k_loop_rt<SD, 4, NW>(kt_count, a, rows, lds, lane, acc); break;
     }
 }
 
