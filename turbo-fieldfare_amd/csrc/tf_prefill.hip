@@ -62,12 +62,21 @@ __global__ __launch_bounds__(256) void prefill_logits_kernel(const uint8_t *W, c
     if (lane == 0) logits[(size_t)t * num_experts + e] = v;
 }
 
-__global__ __launch_bounds__(64) void prefill_select_kernel(const float *logits, const uint16_t *per_expert_scale,
+// planes > 0: the token's logits are first summed, in plane order, from `planes` partial planes that follow the
+// [tokens, experts] logits array (each lane sums the entries it will read back), then selected from.
+__global__ __launch_bounds__(64) void prefill_select_kernel(float *logits, const uint16_t *per_expert_scale,
                                                             uint32_t *out_indices, half_t *out_weights, uint32_t num_experts,
-                                                            uint32_t top_k) {
+                                                            uint32_t top_k, uint32_t planes, size_t plane_stride) {
     const uint32_t t = blockIdx.x;
-    router_select(logits + (size_t)t * num_experts, per_expert_scale, out_indices + (size_t)t * top_k, out_weights + (size_t)t * top_k,
-                  num_experts, top_k, threadIdx.x);
+    float *row = logits + (size_t)t * num_experts;
+    if (planes > 0) {
+        for (uint32_t e = threadIdx.x; e < num_experts; e += 64) {
+            float v = 0.0f;
+            for (uint32_t p = 1; p <= planes; ++p) v += row[p * plane_stride + e];
+            row[e] = v;
+        }
+    }
+    router_select(row, per_expert_scale, out_indices + (size_t)t * top_k, out_weights + (size_t)t * top_k, num_experts, top_k, threadIdx.x);
 }
 
 // Many tokens: the router projection as a matrix product on the matrix cores.  A block takes 32 tokens and up to 128
@@ -83,26 +92,31 @@ __global__ __launch_bounds__(64) void prefill_select_kernel(const float *logits,
 template <int SD>
 __global__ __launch_bounds__(256) void prefill_logits_mfma_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B,
                                                                   const half_t *hidden, long hidden_stride, const uint16_t *eff,
-                                                                  float *logits, uint32_t query_count, uint32_t num_experts, int d) {
+                                                                  float *logits, uint32_t query_count, uint32_t num_experts, int d,
+                                                                  int groups_per_split) {
     __shared__ __align__(16) u32x4 x_hi[2][256], x_lo[2][256];   // [stage][a_slot(token, chunk)]
     __shared__ float xsum[32][65];                                // [token][group], padded
     __shared__ __align__(16) u32x4 g_hi[256], g_lo[256];         // the sums as fp16 parts, a_slot(token, chunk of 8 groups)
     __shared__ __align__(16) half_t bias_h[128][64];              // [expert of the block][group] biases as fp16, 0 beyond
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int i = lane & 31, kb = lane >> 5;
-    const int groups = d >> 6;
+    // blockIdx.y: which run of quantization groups this block sums; its partial logits go to plane blockIdx.y
+    const int all_groups = d >> 6;
+    const int group0 = (int)blockIdx.y * groups_per_split;
+    const int groups = min(groups_per_split, all_groups - group0);
+    logits += (size_t)blockIdx.y * query_count * num_experts;
     const uint32_t t0 = blockIdx.x * 32;
     // producer role: token p_tok, 8 columns p_chunk * 8 .. of every group
     const int p_tok = threadIdx.x >> 3, p_chunk = threadIdx.x & 7;
-    const half_t *p_row = hidden + (size_t)min(t0 + (uint32_t)p_tok, query_count - 1) * hidden_stride + p_chunk * 8;
-    const uint16_t *p_eff = eff + p_chunk * 8;
+    const half_t *p_row = hidden + (size_t)min(t0 + (uint32_t)p_tok, query_count - 1) * hidden_stride + group0 * 64 + p_chunk * 8;
+    const uint16_t *p_eff = eff + group0 * 64 + p_chunk * 8;
     const int p_slot = a_slot(p_tok, p_chunk);
     // consumer role: expert row e_row (clamped), the kb-th 32 columns of every group
     const uint32_t e_lane = (uint32_t)wave * 32u + (uint32_t)i;
     const uint32_t e_row = min(e_lane, num_experts - 1);
-    const uint8_t *w_row = W + (size_t)e_row * d + kb * 32;
-    const uint8_t *s_row = S + (size_t)e_row * groups * 2;
-    const uint8_t *b_row = B + (size_t)e_row * groups * 2;
+    const uint8_t *w_row = W + (size_t)e_row * d + group0 * 64 + kb * 32;
+    const uint8_t *s_row = S + ((size_t)e_row * all_groups + group0) * 2;
+    const uint8_t *b_row = B + ((size_t)e_row * all_groups + group0) * 2;
     const bool wave_live = (uint32_t)wave * 32u < num_experts;
 
     auto produce = [&](const u32x4 hraw, const u32x4 eraw, int stage, int g) {
@@ -253,16 +267,16 @@ __global__ __launch_bounds__(256) void group_scan_kernel(uint32_t *seg_counts, u
                                                          tf_prefill_group *chunks, uint32_t *chunk_count) {
     __shared__ uint32_t scan_pairs[256], scan_chunks[256];
     const uint32_t e = threadIdx.x;
+    // all of this expert's segment counts are requested at once (one memory round trip), then summed in registers
+    uint32_t v[kGroupSegments];
+#pragma unroll
+    for (uint32_t s = 0; s < kGroupSegments; ++s) v[s] = s < n_segments ? seg_counts[s * 256 + e] : 0u;
     uint32_t total = 0;
-    for (uint32_t s0 = 0; s0 < n_segments; s0 += 8) {
-        uint32_t v[8];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = s0 + j < n_segments ? seg_counts[(s0 + j) * 256 + e] : 0u;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            if (s0 + j < n_segments) seg_counts[(s0 + j) * 256 + e] = total;   // exclusive prefix inside expert e
-            total += v[j];
-        }
+    for (uint32_t s = 0; s < kGroupSegments; ++s) {
+        const uint32_t c = v[s];
+        v[s] = total;   // exclusive prefix inside expert e
+        total += c;
     }
     const uint32_t nch = (total + kChunkPairs - 1) / kChunkPairs;
     scan_pairs[e] = total;
@@ -281,7 +295,9 @@ __global__ __launch_bounds__(256) void group_scan_kernel(uint32_t *seg_counts, u
         per_expert_offsets[e] = total ? start : 0xFFFFFFFFu;
         per_expert_counts[e] = total;
     }
-    for (uint32_t s = 0; s < n_segments; ++s) seg_counts[s * 256 + e] += start;   // the read-modify-writes are independent
+#pragma unroll
+    for (uint32_t s = 0; s < kGroupSegments; ++s)
+        if (s < n_segments) seg_counts[s * 256 + e] = v[s] + start;
     for (uint32_t c = 0; c < nch; ++c) {
         tf_prefill_group g;
         g.expert = e;
@@ -291,31 +307,48 @@ __global__ __launch_bounds__(256) void group_scan_kernel(uint32_t *seg_counts, u
     }
 }
 
+// Ranks 64 pairs at a time: every lane ORs its bit into its expert's 64-bit mask in LDS, then reads the mask back: the
+// set bits below its own are the earlier pairs of the same expert (order = (token, rank) order, whatever the timing).
+__device__ __forceinline__ uint32_t place_batch(uint32_t e, bool valid, uint32_t lane, unsigned long long *mask, uint32_t *next) {
+    const unsigned long long bit = 1ull << lane;
+    if (valid) atomicOr(&mask[e], bit);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    uint32_t pos = 0;
+    unsigned long long same = 0ull;
+    if (valid) {
+        same = mask[e];
+        pos = next[e] + (uint32_t)__builtin_popcountll(same & (bit - 1ull));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    if (valid && (same & (bit - 1ull)) == 0ull) {   // the first pair of its expert in this batch moves the expert on
+        next[e] += (uint32_t)__builtin_popcountll(same);
+        mask[e] = 0ull;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    return pos;
+}
+
 __global__ __launch_bounds__(64) void group_place_kernel(const uint32_t *indices, const uint16_t *weights, uint32_t n_pairs,
                                                          uint32_t seg_pairs, uint32_t top_k, uint32_t num_experts,
                                                          const uint32_t *seg_starts, tf_prefill_pair *sorted_pairs) {
     __shared__ uint32_t next[256];
+    __shared__ unsigned long long mask[256];
     const uint32_t lane = threadIdx.x;
-    for (uint32_t e = lane; e < 256; e += 64) next[e] = seg_starts[blockIdx.x * 256 + e];
+    for (uint32_t e = lane; e < 256; e += 64) {
+        next[e] = seg_starts[blockIdx.x * 256 + e];
+        mask[e] = 0ull;
+    }
     __syncthreads();
     const uint32_t first = blockIdx.x * seg_pairs, last = min(first + seg_pairs, n_pairs);
-    const uint64_t below = (1ull << lane) - 1ull;
     for (uint32_t i0 = first; i0 < last; i0 += 64) {
         const uint32_t i = i0 + lane;
         const bool valid = i < last;
-        const uint32_t e = valid ? clamp_expert(indices[i], num_experts) : 0xFFFFFFFFu;
+        const uint32_t e = valid ? clamp_expert(indices[i], num_experts) : 0u;
         const uint16_t wbits = valid ? weights[i] : (uint16_t)0;
-        uint64_t remaining = __ballot(valid);
-        uint32_t pos = 0;
-        while (remaining) {   // one round per distinct expert among the 64 pairs
-            const int leader = __builtin_ctzll(remaining);
-            const uint32_t v = (uint32_t)__builtin_amdgcn_readlane((int)e, leader);
-            const uint64_t same = __ballot(e == v);
-            const uint32_t at = next[v];
-            if (e == v) pos = at + (uint32_t)__builtin_popcountll(same & below);
-            if ((int)lane == leader) next[v] = at + (uint32_t)__builtin_popcountll(same);
-            remaining &= ~same;
-        }
+        const uint32_t pos = place_batch(e, valid, lane, mask, next);
         if (valid) {
             tf_prefill_pair p;
             p.token = i / top_k;
@@ -333,8 +366,10 @@ __global__ __launch_bounds__(256) void group_small_kernel(const uint32_t *indice
                                                           uint32_t *per_expert_offsets, uint32_t *per_expert_counts,
                                                           tf_prefill_group *chunks, uint32_t *chunk_count) {
     __shared__ uint32_t cnt[256], scan_pairs[256], scan_chunks[256], next[256];
+    __shared__ unsigned long long mask[256];
     const uint32_t e = threadIdx.x;
     cnt[e] = 0;
+    mask[e] = 0ull;
     __syncthreads();
     for (uint32_t i = e; i < n_pairs; i += 256) atomicAdd(&cnt[clamp_expert(indices[i], num_experts)], 1u);
     __syncthreads();
@@ -367,23 +402,12 @@ __global__ __launch_bounds__(256) void group_small_kernel(const uint32_t *indice
     __syncthreads();
     if (threadIdx.x >= 64) return;
     const uint32_t lane = threadIdx.x;
-    const uint64_t below = (1ull << lane) - 1ull;
     for (uint32_t i0 = 0; i0 < n_pairs; i0 += 64) {
         const uint32_t i = i0 + lane;
         const bool valid = i < n_pairs;
-        const uint32_t x = valid ? clamp_expert(indices[i], num_experts) : 0xFFFFFFFFu;
+        const uint32_t x = valid ? clamp_expert(indices[i], num_experts) : 0u;
         const uint16_t wbits = valid ? weights[i] : (uint16_t)0;
-        uint64_t remaining = __ballot(valid);
-        uint32_t pos = 0;
-        while (remaining) {
-            const int leader = __builtin_ctzll(remaining);
-            const uint32_t v = (uint32_t)__builtin_amdgcn_readlane((int)x, leader);
-            const uint64_t same = __ballot(x == v);
-            const uint32_t at = next[v];
-            if (x == v) pos = at + (uint32_t)__builtin_popcountll(same & below);
-            if ((int)lane == leader) next[v] = at + (uint32_t)__builtin_popcountll(same);
-            remaining &= ~same;
-        }
+        const uint32_t pos = place_batch(x, valid, lane, mask, next);
         if (valid) {
             tf_prefill_pair p;
             p.token = i / top_k;
@@ -766,7 +790,17 @@ int32_t tf_prefill_router_gemma4_block(tf_ctx *ctx, tf_stream stream, const void
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool mfma_ok = fast && num_experts <= 128 && d <= 4096 && aligned16(w) && d % 64 == 0;
     if (query_count <= kFewTokens || mfma_ok) {
-        const size_t need = std::max<size_t>((size_t)kFewTokens * 256, (size_t)query_count * num_experts);
+        // many tokens: enough blocks to fill the chip, by cutting the reduction dimension into up to four runs of groups
+        // whose partial logits the selection kernel adds up in a fixed order
+        const uint32_t token_blocks = (query_count + 31) / 32;
+        const uint32_t groups = d / 64;
+        uint32_t splits = 1;
+        if (query_count > kFewTokens) {
+            while (splits < 4 && token_blocks * splits < (uint32_t)ctx->num_cus && groups / (splits * 2) >= 8) splits *= 2;
+        }
+        const uint32_t planes = splits > 1 ? splits : 0;   // partial planes behind the logits
+        const size_t plane = (size_t)query_count * num_experts;
+        const size_t need = std::max<size_t>((size_t)kFewTokens * 256, plane * (1 + planes));
         if (ctx->prefill_logits_count < need) {
             if (ctx->prefill_logits) (void)hipFree(ctx->prefill_logits);
             ctx->prefill_logits = nullptr;
@@ -776,8 +810,10 @@ int32_t tf_prefill_router_gemma4_block(tf_ctx *ctx, tf_stream stream, const void
             ctx->prefill_logits_count = need;
         }
         if (query_count > kFewTokens) {
-            hipLaunchKernelGGL(prefill_logits_mfma_kernel<0>, dim3((query_count + 31) / 32), dim3(256), 0, st, w, s, b, h,
-                               (long)hidden_stride_elements, eff, ctx->prefill_logits, query_count, num_experts, (int)d);
+            const int groups_per_split = (int)((groups + splits - 1) / splits);
+            hipLaunchKernelGGL(prefill_logits_mfma_kernel<0>, dim3(token_blocks, splits), dim3(256), 0, st, w, s, b, h,
+                               (long)hidden_stride_elements, eff, ctx->prefill_logits + (planes ? plane : 0), query_count, num_experts, (int)d,
+                               groups_per_split);
         } else {
             const dim3 grid((num_experts + 3) / 4, query_count);
 #define TF_PL(NP_)                                                                                                           \
@@ -794,7 +830,7 @@ int32_t tf_prefill_router_gemma4_block(tf_ctx *ctx, tf_stream stream, const void
         }
         const int32_t rc = check_launch(ctx, "prefill_router logits");
         if (rc != TF_OK) return rc;
-        hipLaunchKernelGGL(prefill_select_kernel, dim3(query_count), dim3(64), 0, st, ctx->prefill_logits, pes, oi, ow, num_experts, top_k);
+        hipLaunchKernelGGL(prefill_select_kernel, dim3(query_count), dim3(64), 0, st, ctx->prefill_logits, pes, oi, ow, num_experts, top_k, planes, plane);
         return check_launch(ctx, "prefill_router select");
     }
 #define TF_PR(NP_)                                                                                                           \
