@@ -658,6 +658,38 @@ __global__ __launch_bounds__(256) void reduce_token_major_kernel(const half_t *p
     h2[(size_t)t * D + c] = (half_t)acc;
 }
 
+// Same sums, eight columns a thread: 16-byte aligned operands and D % 8 == 0. Each column still adds its ranks in rank order.
+constexpr uint32_t kReduceRanksInFlight = 8;
+__global__ __launch_bounds__(256) void reduce_token_major_vec_kernel(const half_t *partials, const half_t *weights, half_t *h2,
+                                                                     uint32_t T, uint32_t top_k, uint32_t D) {
+    const uint32_t c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
+    const uint32_t t = blockIdx.y;
+    if (c >= D || t >= T) return;
+    float acc[8] = {};
+    for (uint32_t r0 = 0; r0 < top_k; r0 += kReduceRanksInFlight) {
+        uint4 raw[kReduceRanksInFlight];
+        float w[kReduceRanksInFlight];
+#pragma unroll
+        for (uint32_t j = 0; j < kReduceRanksInFlight; ++j) {
+            const uint32_t r = min(r0 + j, top_k - 1);
+            raw[j] = *reinterpret_cast<const uint4 *>(partials + ((size_t)t * top_k + r) * D + c);
+            w[j] = (float)weights[t * top_k + r];
+        }
+#pragma unroll
+        for (uint32_t j = 0; j < kReduceRanksInFlight; ++j) {
+            if (r0 + j >= top_k) break;
+            const half_t *v = reinterpret_cast<const half_t *>(&raw[j]);
+#pragma unroll
+            for (uint32_t e = 0; e < 8; ++e) acc[e] = fmaf(w[j], (float)v[e], acc[e]);
+        }
+    }
+    uint4 packed;
+    half_t *o = reinterpret_cast<half_t *>(&packed);
+#pragma unroll
+    for (uint32_t e = 0; e < 8; ++e) o[e] = (half_t)acc[e];
+    *reinterpret_cast<uint4 *>(h2 + (size_t)t * D + c) = packed;
+}
+
 // ------------------------------------------------------------------------------------------------ launch helpers
 struct GroupedGeom {
     const tf_prefill_pair *pairs;
@@ -1060,11 +1092,18 @@ int32_t tf_prefill_moe_reduce_token_major(tf_ctx *ctx, tf_stream stream, const v
     TF_REQUIRE(ctx, d > 0, TF_ERR_INVALID_ARGUMENT, "moe_reduce_token_major: D must be positive");
     TF_REQUIRE(ctx, route_partials_offset % 2 == 0 && route_weights_offset % 2 == 0 && h2_offset % 2 == 0, TF_ERR_INVALID_ARGUMENT,
                "moe_reduce_token_major: offsets must be 2-byte aligned");
-    const dim3 grid((d + 255) / 256, query_count);
-    hipLaunchKernelGGL(reduce_token_major_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream),
-                       reinterpret_cast<const half_t *>(at(route_partials, route_partials_offset)),
-                       reinterpret_cast<const half_t *>(at(route_weights, route_weights_offset)),
-                       reinterpret_cast<half_t *>(at(h2, h2_offset)), query_count, top_k, d);
+    const half_t *partials_at = reinterpret_cast<const half_t *>(at(route_partials, route_partials_offset));
+    const half_t *weights_at = reinterpret_cast<const half_t *>(at(route_weights, route_weights_offset));
+    half_t *h2_at = reinterpret_cast<half_t *>(at(h2, h2_offset));
+    if (d % 8 == 0 && aligned16(partials_at) && aligned16(h2_at)) {
+        const dim3 grid((d / 8 + 255) / 256, query_count);
+        hipLaunchKernelGGL(reduce_token_major_vec_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), partials_at, weights_at,
+                           h2_at, query_count, top_k, d);
+    } else {
+        const dim3 grid((d + 255) / 256, query_count);
+        hipLaunchKernelGGL(reduce_token_major_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), partials_at, weights_at,
+                           h2_at, query_count, top_k, d);
+    }
     return check_launch(ctx, "moe_reduce_token_major");
 }
 
