@@ -179,6 +179,17 @@ __device__ __forceinline__ float gelu_tanh(float x) {
     return 0.5f * x * (1.0f + tanhf(inner));
 }
 
+// The same function through the identity 0.5 (1 + tanh u) = 1 / (1 + exp(-2u)): one hardware exponential and one
+// hardware reciprocal (about a dozen instructions against about forty), a few fp32 ulps from gelu_tanh() and without
+// its cancellation for very negative u.  For epilogues that apply it to whole accumulator tiles.
+__device__ __forceinline__ float gelu_tanh_fast(float x) {
+    const float x3 = x * x * x;
+    float inner = 0.7978845608028654f * (x + 0.044715f * x3);
+    inner = fminf(fmaxf(inner, -20.0f), 20.0f);
+    const float e = __builtin_amdgcn_exp2f(inner * -2.885390081777927f);   // exp(-2 u) = 2^(-2 u log2 e)
+    return x * __builtin_amdgcn_rcpf(1.0f + e);
+}
+
 __device__ __forceinline__ uint16_t f32_to_f16_bits(float v) { return __builtin_bit_cast(uint16_t, (half_t)v); }
 
 }  // namespace tfk

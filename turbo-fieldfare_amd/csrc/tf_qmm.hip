@@ -179,10 +179,12 @@ __global__ __launch_bounds__(64 * kGroupedWaves, 8 / kGroupedWaves) void grouped
     // acts rows of a chunk are consecutive; F % 64 == 0 and a 16-byte aligned acts keep every row piece aligned
     __syncthreads();
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt)
+    for (int mt = 0; mt < 4; ++mt) {
+        if (mt >= row_tiles) break;   // tiles without rows were not multiplied and are not stored
 #pragma unroll
         for (int r = 0; r < 16; ++r)
-            out_tile_put<kP1BN>(lds, mt * 32 + acc_row(r, lane), wave * 32 + acc_col(lane), gelu_tanh(acc[mt][0][r]) * acc[mt][1][r]);
+            out_tile_put<kP1BN>(lds, mt * 32 + acc_row(r, lane), wave * 32 + acc_col(lane), gelu_tanh_fast(acc[mt][0][r]) * acc[mt][1][r]);
+    }
     const int nb = (int)col_tile * kP1BN;
     half_t *tile = acts + (size_t)(ch.pair_start - acts_pair_base) * F + nb;
     out_tile_store<kP1BN>(lds, (int)ch.pair_count, min(kP1BN, F - nb), [&](int row) { return tile + (size_t)row * F; });

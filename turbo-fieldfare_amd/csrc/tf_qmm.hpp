@@ -46,16 +46,25 @@ constexpr int kQmmBN = QmmGeom<4>::kBN;
 constexpr int kQmmLdsBytes = QmmGeom<4>::kLoopLdsBytes;
 
 // 8 nibbles of one word -> 8 fp16 weights half(q * s + b) in element order.  A byte holds two neighbouring elements:
-// v_perm_b32 copies it into both halves of a register, one mask leaves the low nibble in the low half as 1024 + q
-// (0x6400 | q) and the high nibble in place in the high half as 64 + q (0x5400 | q << 4); both offsets are removed
-// exactly, and q * s + b is one fp16 fused multiply-add on fp16 copies of s and b.
-__device__ __forceinline__ half8_t dequant_word(uint32_t v, half2_t s2, half2_t b2) {
+// v_perm_b32 copies it into both halves of a register, one v_and_or_b32 leaves the low nibble in the low half as
+// 1024 + q (0x6400 | q) and the high nibble in place in the high half as 64 + q (0x5400 | q << 4); both offsets are
+// removed exactly, and q * s + b is one fp16 fused multiply-add on fp16 copies of s and b: four instructions a pair.
+// v_and_or_b32 takes no literal operands, so mask and exponent bits live in registers (see nibble_consts()).
+struct NibbleConsts {
+    uint32_t mask, exponents;
+};
+__device__ __forceinline__ NibbleConsts nibble_consts() {
+    NibbleConsts c{0x00F0000Fu, 0x54006400u};
+    asm("" : "+v"(c.mask), "+v"(c.exponents));   // opaque: kept in registers instead of being re-materialised as literals
+    return c;
+}
+__device__ __forceinline__ half8_t dequant_word(uint32_t v, half2_t s2, half2_t b2, const NibbleConsts &c) {
     const half2_t offs = {(half_t)1024.0f, (half_t)64.0f};
     half2_t w[4];
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
         const uint32_t both = __builtin_amdgcn_perm(0u, v, 0x0c000c00u | ((uint32_t)p << 16) | (uint32_t)p);
-        const half2_t q = as_half2((both & 0x00F0000Fu) | 0x54006400u) - offs;
+        const half2_t q = as_half2((both & c.mask) | c.exponents) - offs;
         w[p] = __builtin_elementwise_fma(q, s2, b2);
     }
     return half8_t{w[0][0], w[0][1], w[1][0], w[1][1], w[2][0], w[2][1], w[3][0], w[3][1]};
@@ -152,7 +161,7 @@ __device__ __forceinline__ u32x4 lds_read16(uint32_t addr) {
 // The fragments of MFMA group d + 1 are requested before group d is multiplied, and the weights of group d + 1 are
 // expanded between the MFMAs of group d.
 template <int SD, int RT, int STAGE, int HALF>
-__device__ __forceinline__ void qmm_group(const u32x4 w[2], const QmmSB &sb, const uint32_t frag[4], float16_t acc[4][2]) {
+__device__ __forceinline__ void qmm_group(const u32x4 w[2], const QmmSB &sb, const uint32_t frag[4], const NibbleConsts &nc, float16_t acc[4][2]) {
     half2_t s2[2], b2[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
@@ -160,8 +169,8 @@ __device__ __forceinline__ void qmm_group(const u32x4 w[2], const QmmSB &sb, con
         b2[j] = sb_to_half2<SD>((uint16_t)(HALF ? sb.b[j] >> 16 : sb.b[j] & 0xFFFFu));
     }
     constexpr int base = STAGE * kQmmStageBytes;
-    half8_t bf0 = dequant_word(w[0][0], s2[0], b2[0]);
-    half8_t bf1 = dequant_word(w[1][0], s2[1], b2[1]);
+    half8_t bf0 = dequant_word(w[0][0], s2[0], b2[0], nc);
+    half8_t bf1 = dequant_word(w[1][0], s2[1], b2[1], nc);
     u32x4 af[2][4];
     af[0][0] = lds_read16<base>(frag[0]);
     if constexpr (RT > 1) af[0][1] = lds_read16<base + 4096>(frag[0]);
@@ -196,8 +205,8 @@ __device__ __forceinline__ void qmm_group(const u32x4 w[2], const QmmSB &sb, con
             acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a8, bf0, acc[mt][0], 0, 0, 0);
             acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a8, bf1, acc[mt][1], 0, 0, 0);
             // the next group's weights are expanded between the MFMAs
-            if (d < 3 && mt == 0) nf0 = dequant_word(w[0][d + 1], s2[0], b2[0]);
-            if (d < 3 && mt == (RT > 1 ? 1 : 0)) nf1 = dequant_word(w[1][d + 1], s2[1], b2[1]);
+            if (d < 3 && mt == 0) nf0 = dequant_word(w[0][d + 1], s2[0], b2[0], nc);
+            if (d < 3 && mt == (RT > 1 ? 1 : 0)) nf1 = dequant_word(w[1][d + 1], s2[1], b2[1], nc);
         }
         bf0 = nf0;
         bf1 = nf1;
@@ -228,6 +237,7 @@ struct QmmLoop {
     u32x4 w[2][2];       // [step of the pair][column tile]
     QmmSB sb, sb_next;
     uint32_t pb;         // (current pair & 1) * kQmmWBytes: which W buffer holds the current pair
+    NibbleConsts nc;
 
     __device__ __forceinline__ void read_w(uint32_t at) {
         w[0][0] = lds_read16<0>(at);
@@ -243,7 +253,7 @@ struct QmmLoop {
         __builtin_amdgcn_s_barrier();
         qmm_a_copy<NW>(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
         qmm_w_copy(rows, min(pair + 1, last_pair), wbuf + (pb ^ kQmmWBytes));
-        qmm_group<SD, RT, U3, 0>(w[0], sb, frag, acc);
+        qmm_group<SD, RT, U3, 0>(w[0], sb, frag, nc, acc);
         const int next_pair = min(pair + 1, last_pair);
         qmm_sb_load(sb_next, rows, next_pair, odd_count && next_pair == last_pair);
         if constexpr (QmmGeom<NW>::kAChunks == 4) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
@@ -253,7 +263,7 @@ struct QmmLoop {
     __device__ __forceinline__ void odd_step(int kt, float16_t acc[4][2]) {
         __builtin_amdgcn_s_barrier();
         qmm_a_copy<NW>(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
-        qmm_group<SD, RT, U3, 1>(w[1], sb, frag, acc);
+        qmm_group<SD, RT, U3, 1>(w[1], sb, frag, nc, acc);
         if constexpr (QmmGeom<NW>::kAChunks == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
         pb ^= kQmmWBytes;
@@ -272,6 +282,7 @@ struct QmmLoop {
         wbuf = lds + 3 * kQmmStageBytes + (threadIdx.x >> 6) * (2 * kQmmWBytes);   // NW such pairs of buffers follow the X ring
         wread = wbuf + (uint32_t)i * 64u + ((((uint32_t)kb) ^ (uint32_t)((i >> 2) & 3)) << 4);
         pb = 0;
+        nc = nibble_consts();
         qmm_a_copy<NW>(a, 0, lds);
         qmm_a_copy<NW>(a, min(1, last), lds + kQmmStageBytes);
         qmm_w_copy(rows, 0, wbuf);
