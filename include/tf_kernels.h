@@ -223,6 +223,26 @@ int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream,
                               void *scratch_act, uint64_t scratch_act_offset, uint64_t scratch_act_length,
                               uint32_t weight_bits, tf_dtype scale_dtype);
 
+/* PrefillSharedExpert.encodeBlock (Kernels/Prefill/MoE/PrefillSharedExpert.swift:11-58): the shared expert for
+ * query_count rows of x (row stride x_stride_elements halves) into query_count rows of y.  The reference runs the
+ * single-row chain once per row through the same one-row scratch buffers; so does this entry for fewer than 8 rows and
+ * for operands the matrix-core path cannot take (weights or x rows not 16-byte aligned, intermediate % 64 != 0).
+ * Otherwise the rows go through the matrix cores: gate and up in one pass with both sums rounded to fp16 before GeGLU
+ * (the chain's stage boundary), activations in a buffer the context owns, then the down projection; weights are
+ * expanded to fp16 half(q*s+b) per group as in tf_int4_qmm, so results agree with the row chain within the shared
+ * expert's tolerance, not bit for bit, and the caller's scratch (still validated: one row each, lengths in BYTES) is
+ * left untouched.  query_count == 0 is a no-op.  d, intermediate > 0, strides >= d (TF_ERR_INVALID_ARGUMENT);
+ * gate/up = (intermediate, d), down = (d, intermediate) or TF_ERR_DIMENSION_MISMATCH. */
+int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream,
+                                            const void *x, uint64_t x_offset, void *y, uint64_t y_offset,
+                                            const tf_projection *gate, const tf_projection *up, const tf_projection *down,
+                                            void *scratch_gate, uint64_t scratch_gate_offset, uint64_t scratch_gate_length,
+                                            void *scratch_up, uint64_t scratch_up_offset, uint64_t scratch_up_length,
+                                            void *scratch_act, uint64_t scratch_act_offset, uint64_t scratch_act_length,
+                                            uint32_t query_count, uint32_t d, uint32_t intermediate,
+                                            uint32_t x_stride_elements, uint32_t y_stride_elements,
+                                            uint32_t weight_bits, tf_dtype scale_dtype);
+
 /* ---- router ----------------------------------------------------------------------------------------------------- */
 /* MoE.encodeRouterGemma4 (Kernels/MoE/MoE.swift:109-159) -> router_gemv_gemma4_r4 + router_topk_select_k8
  * (Metal/MoE/moe.metal:78-185).  hidden fp16 [d] (no offset, as in the reference), effective_scale bf16 [d],

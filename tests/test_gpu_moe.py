@@ -245,6 +245,88 @@ def test_shared_expert_errors():
     assert rc == tfk.TF_ERR_DIMENSION_MISMATCH                                    # :41-45
 
 
+# ---------------------------------------------------------------------------------------------------- shared expert, block of rows
+def _shared_block_case(rows, d, f, seed):
+    c = dict(d=d, f=f, gate=refcases.synthetic_int4(f, d, seed, "g"), up=refcases.synthetic_int4(f, d, seed, "u"),
+             down=refcases.synthetic_int4(d, f, seed, "d"))
+    c["x_bits"] = refcases.normal_f16(rows * d, seed).reshape(rows, d)
+    return c
+
+
+SENTINEL = np.float16(-7.25).view(np.uint16)   # PrefillSharedExpertTests.swift:13
+
+
+def run_shared_block(c, rows, x_stride, y_stride, weight_bits=4, scratch_halves=None):
+    d, f = c["d"], c["f"]
+    k = ctx()
+    t = {n: [dev(a) for a in c[n]] for n in ("gate", "up", "down")}
+    x_host = np.full((max(rows, 1), max(x_stride, d)), SENTINEL, np.uint16)   # a too-small stride is refused before any read
+    x_host[:rows, :d] = c["x_bits"][:rows]
+    keep = dict(x=dev(x_host), y=dev(np.full((max(rows, 1), max(y_stride, d)), SENTINEL, np.uint16)))
+    n_s = (scratch_halves if scratch_halves is not None else f) * 2
+    sg, su, sa = zeros_bytes(n_s), zeros_bytes(n_s), zeros_bytes(n_s)
+    rc = k.prefill_shared_expert_block(keep["x"], _proj(*t["gate"], f, d), _proj(*t["up"], f, d), _proj(*t["down"], d, f), keep["y"],
+                                       sg, su, sa, rows, d, f, x_stride=x_stride, y_stride=y_stride, weight_bits=weight_bits,
+                                       raise_on_error=False)
+    return rc, host(keep["y"], np.uint16).reshape(max(rows, 1), max(y_stride, d))
+
+
+def _repeated_rows(c, rows):
+    out = []
+    for r in range(rows):
+        one = dict(c)
+        one["x_bits"] = c["x_bits"][r]
+        rc, y, _ = run_shared(one)
+        assert rc == tfk.TF_OK
+        out.append(y)
+    return np.stack(out)
+
+
+def test_prefill_shared_expert_block_equals_repeated_rows_bit_for_bit():
+    # PrefillSharedExpertTests.swift:8-13,178-243: 4 rows, d 128, f 64, x stride 144, y stride 137, sentinel padding
+    rows, d, f = 4, 128, 64
+    c = _shared_block_case(rows, d, f, 0xC0FFEE)
+    rc, y = run_shared_block(c, rows, 144, 137)
+    assert rc == tfk.TF_OK
+    assert np.array_equal(y[:, :d], _repeated_rows(c, rows))
+    assert np.all(y[:, d:] == SENTINEL)
+
+
+@pytest.mark.parametrize("rows,d,f,x_stride,y_stride", [(8, 128, 64, 144, 136), (40, 128, 64, 128, 137), (133, 256, 192, 264, 256),
+                                                       (200, 2816, 2112, 2816, 2816)])
+def test_prefill_shared_expert_block_on_matrix_cores(rows, d, f, x_stride, y_stride):
+    c = _shared_block_case(rows, d, f, 0x5B + rows)
+    rc, y = run_shared_block(c, rows, x_stride, y_stride)
+    assert rc == tfk.TF_OK
+    assert np.all(y[:, d:] == SENTINEL)
+    check = range(rows) if rows <= 40 else [0, 1, 31, 32, 127, 128, rows - 2, rows - 1]
+    for r in check:
+        ref = tfo.shared_expert_ref(c["gate"], c["up"], c["down"], tfo.from_f16_bits(c["x_bits"][r]), threads=8)
+        assert tfo.rel_error(tfo.from_f16_bits(y[r, :d]), ref) < 6e-3, r       # SharedExpertInt4Tests.swift:52
+    # and against the single-row chain of the same library (fp32 weights there, fp16-rounded weights here)
+    chain = _repeated_rows(c, min(rows, 3))
+    for r in range(min(rows, 3)):
+        assert tfo.rel_error(tfo.from_f16_bits(y[r, :d]), tfo.from_f16_bits(chain[r])) < 6e-3
+
+
+def test_prefill_shared_expert_block_contract():
+    c = _shared_block_case(4, 128, 64, 7)
+    assert run_shared_block(c, 0, 128, 128)[0] == tfk.TF_OK                       # queryCount 0: nothing to do
+    assert np.all(run_shared_block(c, 0, 128, 128)[1] == SENTINEL)
+    assert run_shared_block(c, 4, 127, 128)[0] == tfk.TF_ERR_INVALID_ARGUMENT     # PrefillSharedExpert.swift:35
+    assert run_shared_block(c, 4, 128, 127)[0] == tfk.TF_ERR_INVALID_ARGUMENT     # :36
+    assert run_shared_block(c, 4, 128, 128, weight_bits=8)[0] == tfk.TF_ERR_UNSUPPORTED_BITS
+    assert run_shared_block(c, 4, 128, 128, scratch_halves=63)[0] == tfk.TF_ERR_SCRATCH_TOO_SMALL
+    big = _shared_block_case(16, 128, 64, 7)
+    assert run_shared_block(big, 16, 128, 128, scratch_halves=63)[0] == tfk.TF_ERR_SCRATCH_TOO_SMALL
+    k = ctx()
+    t = {n: [dev(a) for a in c[n]] for n in ("gate", "up")}
+    x, y, s = dev(c["x_bits"]), zeros_bytes(4 * 256), zeros_bytes(128)
+    rc = k.prefill_shared_expert_block(x, _proj(*t["gate"], 64, 128), _proj(*t["up"], 64, 128), _proj(*t["gate"], 64, 128), y, s, s, s,
+                                       4, 128, 64, raise_on_error=False)
+    assert rc == tfk.TF_ERR_DIMENSION_MISMATCH                                   # :37-42
+
+
 # ---------------------------------------------------------------------------------------------------- decode step
 def _decode_step_case(d, f, num_experts, seed):
     rng = np.random.default_rng(seed)

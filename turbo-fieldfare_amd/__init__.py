@@ -112,6 +112,9 @@ EXPORTS = {
                                           C.c_float, C.c_float]),
     "tf_shared_expert_int4": (i32, [vp, vp, vp, u64, u64, C.POINTER(Projection), C.POINTER(Projection), C.POINTER(Projection),
                                     vp, u64, u64, vp, u64, u64, vp, u64, u64, vp, u64, u64, u32, i32]),
+    "tf_prefill_shared_expert_int4_block": (i32, [vp, vp, vp, u64, vp, u64, C.POINTER(Projection), C.POINTER(Projection),
+                                                  C.POINTER(Projection), vp, u64, u64, vp, u64, u64, vp, u64, u64, u32, u32, u32,
+                                                  u32, u32, u32, i32]),
     "tf_router_gemma4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, vp, u64, vp, u64, vp, vp, u32, u32, u32]),
     "tf_moe_phase1_gate_up_act": (i32, [vp, vp, C.POINTER(RoutedBlobs), C.POINTER(ExpertOffsets), vp, vp, u32, u32, u32, i32]),
     "tf_moe_phase1_gate_up_act_subset": (i32, [vp, vp, C.POINTER(RoutedBlobs), C.POINTER(ExpertOffsets), vp, vp, vp, u32,
@@ -297,6 +300,18 @@ class Context:
         rc = self.lib.tf_shared_expert_int4(self.handle, _stream(), _p(x), 0, ln[0], C.byref(gate), C.byref(up), C.byref(down),
                                             _p(y), 0, ln[1], _p(sg), 0, ln[2], _p(su), 0, ln[3], _p(sa), 0, ln[4],
                                             weight_bits, scale_dtype)
+        return self.check(rc) if raise_on_error else rc
+
+    def prefill_shared_expert_block(self, x, gate: Projection, up: Projection, down: Projection, y, sg, su, sa, query_count, d,
+                                    intermediate, x_stride=None, y_stride=None, x_offset=0, y_offset=0, weight_bits=4,
+                                    scale_dtype=TF_BF16, raise_on_error=True):
+        def nbytes(t):
+            return t.numel() * t.element_size()
+        rc = self.lib.tf_prefill_shared_expert_int4_block(self.handle, _stream(), _p(x), x_offset, _p(y), y_offset, C.byref(gate),
+                                                          C.byref(up), C.byref(down), _p(sg), 0, nbytes(sg), _p(su), 0, nbytes(su),
+                                                          _p(sa), 0, nbytes(sa), query_count, d, intermediate,
+                                                          d if x_stride is None else x_stride, d if y_stride is None else y_stride,
+                                                          weight_bits, scale_dtype)
         return self.check(rc) if raise_on_error else rc
 
     def lm_head_greedy(self, hidden, norm_w, W, S, B, out_token, d, vocab, eps=1e-6, scale_dtype=TF_BF16,

@@ -69,6 +69,7 @@ void tf_ctx_destroy(tf_ctx *ctx) {
     if (ctx->group_scratch) (void)hipFree(ctx->group_scratch);
     if (ctx->prefill_logits) (void)hipFree(ctx->prefill_logits);
     if (ctx->sample_scratch) (void)hipFree(ctx->sample_scratch);
+    if (ctx->shared_block_acts) (void)hipFree(ctx->shared_block_acts);
     for (hipEvent_t e : ctx->step_events)
         if (e) (void)hipEventDestroy(e);
     delete ctx;

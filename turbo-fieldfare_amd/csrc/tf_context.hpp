@@ -23,6 +23,8 @@ struct tf_ctx {
     size_t prefill_logits_count = 0;
     void *sample_scratch = nullptr;     // lazily sized: argmax cells, softmax partials, top-k pair buffers of the samplers
     size_t sample_scratch_bytes = 0;
+    void *shared_block_acts = nullptr;  // lazily sized [rows, intermediate] fp16 activations of the block shared expert
+    size_t shared_block_acts_bytes = 0;
     // optional device-time bracketing of the decode step's three launches
     bool step_timing = false;
     bool step_timed = false;            // a step has been recorded since timing was enabled

@@ -73,12 +73,36 @@ constexpr int block_lds_bytes() {
 }
 
 // ------------------------------------------------------------------------------------------------ dense
+// Block number -> (row tile, column tile) of a dense product.  Workgroups go to the 8 XCDs round-robin by linear id and
+// each XCD has its own L2: row tile r belongs to XCD r % 8, which computes all of its column tiles, so the activation rows
+// of a tile are fetched into one L2 only and every XCD streams the (much smaller) weight matrix once.  With fewer row
+// tiles than XCDs the plain numbering is used.  The grid is dense_grid() blocks; surplus ones return false.
+constexpr uint32_t kDenseXcds = 8;
+__host__ __device__ inline uint32_t dense_grid(uint32_t row_tiles, uint32_t col_tiles) {
+    if (row_tiles < kDenseXcds) return row_tiles * col_tiles;
+    return kDenseXcds * ((row_tiles + kDenseXcds - 1) / kDenseXcds) * col_tiles;
+}
+__device__ __forceinline__ bool dense_tile(uint32_t row_tiles, uint32_t col_tiles, uint32_t &row_tile, uint32_t &col_tile) {
+    const uint32_t id = blockIdx.x;
+    if (row_tiles < kDenseXcds) {
+        row_tile = id / col_tiles;
+        col_tile = id - row_tile * col_tiles;
+        return true;
+    }
+    const uint32_t xcd = id % kDenseXcds, j = id / kDenseXcds;
+    row_tile = (j / col_tiles) * kDenseXcds + xcd;
+    col_tile = j % col_tiles;
+    return row_tile < row_tiles;
+}
+
 template <int SD>
 __global__ __launch_bounds__(256, 2) void qmm_dense_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *X,
                                                            long ldx, half_t *Y, long ldy, int M, int N, int K, bool rows_vectorizable) {
     __shared__ __align__(128) uint8_t lds[block_lds_bytes<4, kQmmBN>()];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int n0 = blockIdx.x * kQmmBN + wave * kQmmWaveN, m0 = blockIdx.y * kQmmBM;
+    uint32_t row_tile, col_tile;
+    if (!dense_tile((uint32_t)(M + kQmmBM - 1) / kQmmBM, (uint32_t)(N + kQmmBN - 1) / kQmmBN, row_tile, col_tile)) return;
+    const int n0 = (int)col_tile * kQmmBN + wave * kQmmWaveN, m0 = (int)row_tile * kQmmBM;
     QmmARows<4> arow;
     arow.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(X), 0, (int)0xFFFFFFFFu, 0x00020000);
 #pragma unroll
@@ -99,7 +123,7 @@ __global__ __launch_bounds__(256, 2) void qmm_dense_kernel(const uint8_t *W, con
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
                     out_tile_put<kQmmBN>(lds, mt * 32 + acc_row(r, lane), wave * kQmmWaveN + j * 32 + acc_col(lane), acc[mt][j][r]);
-        const int nb = blockIdx.x * kQmmBN;
+        const int nb = (int)col_tile * kQmmBN;
         out_tile_store<kQmmBN>(lds, min(kQmmBM, M - m0), min(kQmmBN, N - nb), [&](int row) { return Y + (size_t)(m0 + row) * ldy + nb; });
         return;
     }
@@ -114,6 +138,44 @@ __global__ __launch_bounds__(256, 2) void qmm_dense_kernel(const uint8_t *W, con
                 if (m < M && n < N) Y[(size_t)m * ldy + n] = (half_t)acc[mt][j][r];
             }
     }
+}
+
+// Shared-expert gate and up projections of a block of rows in one pass: a wave's first column tile is 32 rows of the gate
+// matrix, its second the same 32 rows of the up matrix.  Both sums are rounded to fp16 before GeGLU, the stage boundary of
+// the reference's chain (two GEMVs writing fp16, then gelu_mul_fp16: SharedExpertInt4.swift:60-84).
+constexpr int kGegluBN = 32 * 4;
+template <int SD>
+__global__ __launch_bounds__(256, 2) void qmm_dense_geglu_kernel(const uint8_t *gW, const uint8_t *gS, const uint8_t *gB, const uint8_t *uW,
+                                                                 const uint8_t *uS, const uint8_t *uB, const half_t *X, long ldx,
+                                                                 half_t *A, long lda, int M, int F, int K) {
+    __shared__ __align__(128) uint8_t lds[block_lds_bytes<4, kGegluBN>()];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t row_tile, col_tile;
+    if (!dense_tile((uint32_t)(M + kQmmBM - 1) / kQmmBM, (uint32_t)(F + kGegluBN - 1) / kGegluBN, row_tile, col_tile)) return;
+    const int n0 = (int)col_tile * kGegluBN + wave * 32, m0 = (int)row_tile * kQmmBM;
+    QmmARows<4> arow;
+    arow.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(X), 0, (int)0xFFFFFFFFu, 0x00020000);
+#pragma unroll
+    for (int q = 0; q < QmmGeom<4>::kAChunks; ++q) qmm_a_rows_set(arow, q, (uint64_t)min(m0 + qmm_a_row_of<4>(q), M - 1) * (uint64_t)ldx * 2u);
+    const uint8_t *w[2] = {gW, uW}, *s[2] = {gS, uS}, *b[2] = {gB, uB};
+    const int row0[2] = {n0, n0}, limit[2] = {F, F};
+    const QmmBRows rows = make_b_rows(w, s, b, row0, limit, K >> 1, K >> 6, lane);
+    const int row_tiles = min(4, (M - m0 + 31) >> 5);
+    float16_t acc[4][2];
+    zero_acc(acc);
+    qmm_k_loop<SD, 4>(K >> 6, arow, rows, (uint32_t)(uintptr_t)lds, lane, row_tiles, acc);
+    __syncthreads();
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+        if (mt >= row_tiles) break;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const float gate = (float)(half_t)acc[mt][0][r], up = (float)(half_t)acc[mt][1][r];
+            out_tile_put<kGegluBN>(lds, mt * 32 + acc_row(r, lane), wave * 32 + acc_col(lane), gelu_tanh_fast(gate) * up);
+        }
+    }
+    const int nb = (int)col_tile * kGegluBN;
+    out_tile_store<kGegluBN>(lds, min(kQmmBM, M - m0), min(kGegluBN, F - nb), [&](int row) { return A + (size_t)(m0 + row) * lda + nb; });
 }
 
 // Block number -> (chunk, column tile) for the grouped kernels.  Workgroups go to the 8 XCDs round-robin by linear id and
@@ -279,6 +341,58 @@ int32_t launch_grouped_down_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTable 
 
 }  // namespace tfk
 
+namespace {
+
+// Y[m, n] = X[m, k] . W[n, k]^T on the matrix cores.  Operands as qmm_operands_ok() demands; ldx / ldy in halves.
+// 128-row tiles even when they leave compute units idle (144 blocks at 2048 x 2112): 64-row blocks, twice as many, repeat
+// each weight tile's dequantisation and measured slower (0.18 ms against 0.155 ms for the three shared-expert GEMMs).
+int32_t launch_qmm_dense(tf_ctx *ctx, hipStream_t st, const uint8_t *w, const uint8_t *s, const uint8_t *b, const half_t *x, long ldx,
+                         half_t *y, long ldy, int m, int n, int k, tf_dtype sd) {
+    const dim3 grid(dense_grid((uint32_t)(m + kQmmBM - 1) / kQmmBM, (uint32_t)(n + kQmmBN - 1) / kQmmBN));
+    const bool rows_vec = aligned16(y) && n % 8 == 0 && ldy % 8 == 0;   // whole 16-byte pieces of output rows
+    if (sd == TF_BF16)
+        hipLaunchKernelGGL(qmm_dense_kernel<0>, grid, dim3(256), 0, st, w, s, b, x, ldx, y, ldy, m, n, k, rows_vec);
+    else
+        hipLaunchKernelGGL(qmm_dense_kernel<1>, grid, dim3(256), 0, st, w, s, b, x, ldx, y, ldy, m, n, k, rows_vec);
+    return check_launch(ctx, "int4_qmm");
+}
+
+// A[m, f] = GeGLU(half(X . gate^T), half(X . up^T)); a 16-byte aligned, lda % 8 == 0, f % 8 == 0
+int32_t launch_qmm_dense_geglu(tf_ctx *ctx, hipStream_t st, const tf_projection *gate, const tf_projection *up, const half_t *x, long ldx,
+                               half_t *a, long lda, int m, tf_dtype sd) {
+    const int f = (int)gate->rows, k = (int)gate->cols;
+    const dim3 grid(dense_grid((uint32_t)(m + kQmmBM - 1) / kQmmBM, (uint32_t)(f + kGegluBN - 1) / kGegluBN));
+    const uint8_t *gw = at(gate->weights, gate->weights_offset), *gs = at(gate->scales, gate->scales_offset), *gb = at(gate->biases, gate->biases_offset);
+    const uint8_t *uw = at(up->weights, up->weights_offset), *us = at(up->scales, up->scales_offset), *ub = at(up->biases, up->biases_offset);
+    if (sd == TF_BF16)
+        hipLaunchKernelGGL(qmm_dense_geglu_kernel<0>, grid, dim3(256), 0, st, gw, gs, gb, uw, us, ub, x, ldx, a, lda, m, f, k);
+    else
+        hipLaunchKernelGGL(qmm_dense_geglu_kernel<1>, grid, dim3(256), 0, st, gw, gs, gb, uw, us, ub, x, ldx, a, lda, m, f, k);
+    return check_launch(ctx, "prefill_shared_expert gate/up");
+}
+
+// [rows, intermediate] fp16 activations of the block form of the shared expert, owned by the context and grown on demand
+int32_t shared_block_acts(tf_ctx *ctx, size_t halves, half_t *&out) {
+    const size_t need = halves * sizeof(half_t);
+    if (ctx->shared_block_acts_bytes < need) {
+        if (ctx->shared_block_acts) {
+            // kernels of earlier calls may still be using the old buffer
+            if (hipDeviceSynchronize() != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "prefill_shared_expert: device synchronize failed");
+            (void)hipFree(ctx->shared_block_acts);
+            ctx->shared_block_acts = nullptr;
+            ctx->shared_block_acts_bytes = 0;
+        }
+        if (hipMalloc(&ctx->shared_block_acts, need) != hipSuccess) return fail(ctx, TF_ERR_OUT_OF_MEMORY, "prefill_shared_expert: out of device memory");
+        ctx->shared_block_acts_bytes = need;
+    }
+    out = static_cast<half_t *>(ctx->shared_block_acts);
+    return TF_OK;
+}
+
+constexpr uint32_t kSharedBlockMinRows = 8;   // fewer rows go through the single-row chain, bit-identical to decode
+
+}  // namespace
+
 extern "C" {
 
 int32_t tf_int4_qmm(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset, const void *scales,
@@ -292,17 +406,66 @@ int32_t tf_int4_qmm(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t
     const uint8_t *w = at(weights, weights_offset);
     const half_t *xp = reinterpret_cast<const half_t *>(at(x, x_offset));
     if (!qmm_operands_ok(w, xp, k, k) || !aligned(at(y, y_offset), 2)) return fail(ctx, TF_ERR_UNAVAILABLE, "int4_qmm: operands are not 16-byte aligned");
-    // 128-row tiles even when they leave compute units idle (144 blocks at 2048 x 2112): 64-row blocks, twice as many,
-    // repeat each weight tile's dequantisation and measured slower (0.18 ms against 0.155 ms for the three shared-expert GEMMs).
-    const dim3 grid((n + kQmmBN - 1) / kQmmBN, (m + kQmmBM - 1) / kQmmBM);
-    hipStream_t st = static_cast<hipStream_t>(stream);
     half_t *yp = reinterpret_cast<half_t *>(at(y, y_offset));
-    const bool rows_vec = aligned16(yp) && n % 8 == 0;   // whole 16-byte pieces of output rows
-    if (scale_dtype == TF_BF16)
-        hipLaunchKernelGGL(qmm_dense_kernel<0>, grid, dim3(256), 0, st, w, at(scales, scales_offset), at(biases, biases_offset), xp, (long)k, yp, (long)n, m, n, k, rows_vec);
-    else
-        hipLaunchKernelGGL(qmm_dense_kernel<1>, grid, dim3(256), 0, st, w, at(scales, scales_offset), at(biases, biases_offset), xp, (long)k, yp, (long)n, m, n, k, rows_vec);
-    return check_launch(ctx, "int4_qmm");
+    return launch_qmm_dense(ctx, static_cast<hipStream_t>(stream), w, at(scales, scales_offset), at(biases, biases_offset), xp, k, yp, n, m,
+                            n, k, scale_dtype);
+}
+
+int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, void *y, uint64_t y_offset,
+                                            const tf_projection *gate, const tf_projection *up, const tf_projection *down,
+                                            void *scratch_gate, uint64_t scratch_gate_offset, uint64_t scratch_gate_length,
+                                            void *scratch_up, uint64_t scratch_up_offset, uint64_t scratch_up_length, void *scratch_act,
+                                            uint64_t scratch_act_offset, uint64_t scratch_act_length, uint32_t query_count, uint32_t d,
+                                            uint32_t intermediate, uint32_t x_stride_elements, uint32_t y_stride_elements,
+                                            uint32_t weight_bits, tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "prefill_shared_expert: null context");
+    TF_REQUIRE(ctx, weight_bits == 4, TF_ERR_UNSUPPORTED_BITS, "SharedExpert unsupported weight bits: %u", weight_bits);
+    TF_REQUIRE(ctx, x && y && gate && up && down && scratch_gate && scratch_up && scratch_act, TF_ERR_INVALID_ARGUMENT,
+               "prefill_shared_expert: null argument");
+    TF_REQUIRE(ctx, d > 0, TF_ERR_INVALID_ARGUMENT, "prefill_shared_expert: d must be positive");
+    TF_REQUIRE(ctx, intermediate > 0, TF_ERR_INVALID_ARGUMENT, "prefill_shared_expert: intermediate must be positive");
+    TF_REQUIRE(ctx, x_stride_elements >= d, TF_ERR_INVALID_ARGUMENT, "prefill_shared_expert: x stride is too small");
+    TF_REQUIRE(ctx, y_stride_elements >= d, TF_ERR_INVALID_ARGUMENT, "prefill_shared_expert: y stride is too small");
+    TF_REQUIRE(ctx, gate->rows == intermediate && gate->cols == d && up->rows == intermediate && up->cols == d && down->rows == d &&
+                        down->cols == intermediate,
+               TF_ERR_DIMENSION_MISMATCH, "expected gate/up=(%u,%u) down=(%u,%u)", intermediate, d, d, intermediate);
+    if (query_count == 0) return TF_OK;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const half_t *xp = reinterpret_cast<const half_t *>(at(x, x_offset));
+    half_t *yp = reinterpret_cast<half_t *>(at(y, y_offset));
+    const uint8_t *gw = at(gate->weights, gate->weights_offset), *uw = at(up->weights, up->weights_offset);
+    const uint8_t *dw = at(down->weights, down->weights_offset);
+    const bool pointers = gate->weights && gate->scales && gate->biases && up->weights && up->scales && up->biases && down->weights &&
+                          down->scales && down->biases;
+    const bool even = x_offset % 2 == 0 && y_offset % 2 == 0 && gate->scales_offset % 2 == 0 && gate->biases_offset % 2 == 0 &&
+                      up->scales_offset % 2 == 0 && up->biases_offset % 2 == 0 && down->scales_offset % 2 == 0 && down->biases_offset % 2 == 0;
+    const bool block_path = pointers && even && query_count >= kSharedBlockMinRows && (scale_dtype == TF_BF16 || scale_dtype == TF_FP16) &&
+                            qmm_operands_ok(gw, xp, x_stride_elements, (int)d) && aligned16(uw) && aligned16(dw) &&
+                            intermediate % TF_GROUP_SIZE == 0 && query_count <= (uint32_t)INT32_MAX;
+    if (!block_path) {
+        // PrefillSharedExpert.encodeBlock itself: the single-row chain once per row, every row through the same scratch
+        for (uint32_t row = 0; row < query_count; ++row) {
+            const uint64_t xo = x_offset + (uint64_t)row * x_stride_elements * 2, yo = y_offset + (uint64_t)row * y_stride_elements * 2;
+            const int32_t rc = tf_shared_expert_int4(ctx, stream, x, xo, xo + (uint64_t)d * 2, gate, up, down, y, yo, yo + (uint64_t)d * 2,
+                                                     scratch_gate, scratch_gate_offset, scratch_gate_length, scratch_up, scratch_up_offset,
+                                                     scratch_up_length, scratch_act, scratch_act_offset, scratch_act_length, weight_bits,
+                                                     scale_dtype);
+            if (rc != TF_OK) return rc;
+        }
+        return TF_OK;
+    }
+    // the caller's scratch holds one row (the reference's contract); it must still be large enough for that row
+    const uint64_t required = (uint64_t)intermediate * 2;
+    TF_REQUIRE(ctx, scratch_gate_offset + required <= scratch_gate_length && scratch_up_offset + required <= scratch_up_length &&
+                        scratch_act_offset + required <= scratch_act_length,
+               TF_ERR_SCRATCH_TOO_SMALL, "SharedExpert scratch too small: need %llu bytes per intermediate buffer", (unsigned long long)required);
+    half_t *acts = nullptr;
+    int32_t rc = shared_block_acts(ctx, (size_t)query_count * intermediate, acts);
+    if (rc != TF_OK) return rc;
+    rc = launch_qmm_dense_geglu(ctx, st, gate, up, xp, (long)x_stride_elements, acts, (long)intermediate, (int)query_count, scale_dtype);
+    if (rc != TF_OK) return rc;
+    return launch_qmm_dense(ctx, st, dw, at(down->scales, down->scales_offset), at(down->biases, down->biases_offset), acts, (long)intermediate,
+                            yp, (long)y_stride_elements, (int)query_count, (int)d, (int)intermediate, scale_dtype);
 }
 
 }  // extern "C"

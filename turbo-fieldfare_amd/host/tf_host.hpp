@@ -146,6 +146,28 @@ private:
     int weightBits_;
 };
 
+// PrefillSharedExpert (Kernels/Prefill/MoE/PrefillSharedExpert.swift:4-58): the shared expert over a block of rows
+class PrefillSharedExpert {
+public:
+    PrefillSharedExpert(const Context &context, int weightBits = 4) : c_(context), weightBits_(weightBits) {
+        if (weightBits != 4) throw Error(TF_ERR_UNSUPPORTED_BITS, "SharedExpert unsupported weight bits: " + std::to_string(weightBits));
+    }
+    using Buffer = SharedExpertRuntime::Buffer;
+    void encodeBlock(const void *x, uint64_t xOffset, void *y, uint64_t yOffset, const SharedExpertProjection &gate,
+                     const SharedExpertProjection &up, const SharedExpertProjection &down, Buffer scratchGate, uint64_t scratchGateOffset,
+                     Buffer scratchUp, uint64_t scratchUpOffset, Buffer scratchAct, uint64_t scratchActOffset, uint32_t queryCount,
+                     uint32_t d, uint32_t intermediate, uint32_t xStrideElements, uint32_t yStrideElements) const {
+        c_.check(tf_prefill_shared_expert_int4_block(c_.raw(), c_.stream(), x, xOffset, y, yOffset, &gate, &up, &down, scratchGate.ptr,
+                                                     scratchGateOffset, scratchGate.length, scratchUp.ptr, scratchUpOffset,
+                                                     scratchUp.length, scratchAct.ptr, scratchActOffset, scratchAct.length, queryCount, d,
+                                                     intermediate, xStrideElements, yStrideElements, (uint32_t)weightBits_, TF_BF16));
+    }
+
+private:
+    const Context &c_;
+    int weightBits_;
+};
+
 // SharedExpertInt4 (Kernels/MoE/SharedExpertInt4.swift:6-100) is the 4-bit instance of the runtime.
 struct SharedExpertInt4 : SharedExpertRuntime {
     explicit SharedExpertInt4(const Context &context) : SharedExpertRuntime(context, 4) {}
