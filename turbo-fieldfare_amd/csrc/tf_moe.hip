@@ -204,6 +204,8 @@ __global__ __launch_bounds__(512) void phase2_short_kernel(RoutedArg routed, tf_
 #pragma unroll
     for (int dd = 0; dd < 4; ++dd) xr[dd] = load16(acts + (size_t)slot * f + (sr.col < 0 ? 0 : sr.col) * 32 + dd * 8);
     const half_t w16 = routing_w[slot];
+    const bool writer = threadIdx.x < 2 * NPASS && row0 + threadIdx.x < d;
+    const half_t res16 = writer ? residual[row0 + threadIdx.x] : (half_t)0.0f;   // requested now, needed after the barrier
     const uint8_t *base = uniform_ptr(blob_base(routed, slot));
 #pragma unroll
     for (int p = 0; p < NPASS; ++p)
@@ -220,8 +222,8 @@ __global__ __launch_bounds__(512) void phase2_short_kernel(RoutedArg routed, tf_
         }
     }
     __syncthreads();
-    if (threadIdx.x < 2 * NPASS && row0 + threadIdx.x < d) {
-        float acc = (float)residual[row0 + threadIdx.x];
+    if (writer) {
+        float acc = (float)res16;
 #pragma unroll
         for (int s = 0; s < 8; ++s) acc += partial[s][threadIdx.x];
         y[row0 + threadIdx.x] = (half_t)acc;
