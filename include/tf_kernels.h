@@ -497,6 +497,14 @@ int32_t tf_sample_topk64(tf_ctx *ctx, tf_stream stream, const void *probs, void 
 int32_t tf_upload_packed_experts_layer(tf_ctx *ctx, tf_stream stream, const char *layer_file_path, uint64_t expert_stride,
                                        uint32_t num_experts, const uint32_t *physical_rank, void *device_pool);
 
+/* ResidentBuffer.init (Infrastructure/ModelIO/ResidentBuffer.swift:15-78) for a discrete GPU: where the reference maps
+ * [file_offset, file_offset + bytes) of model_weights.bin into one shared MTLBuffer, this copies the range into
+ * `device_dst` (bytes long, caller-owned) through two pinned staging buffers.  The path must be a regular file that
+ * holds the whole range (TF_ERR_DIMENSION_MISMATCH otherwise).  Blocks until the copy is complete.  The index that
+ * says which tensor lives where inside the range is read on the host (tf::gturbo::loadResidentIndex). */
+int32_t tf_upload_file_region(tf_ctx *ctx, tf_stream stream, const char *file_path, uint64_t file_offset, uint64_t bytes,
+                              void *device_dst);
+
 #ifdef __cplusplus
 }
 #endif

@@ -48,3 +48,50 @@ def test_layer_file_upload_in_logical_order_feeds_the_decode_step(tmp_path):
     assert k.lib.tf_upload_packed_experts_layer(k.handle, None, str(path).encode(), stride, num_experts, twice.ctypes.data_as(C.POINTER(C.c_uint32)),
                                                 pool.data_ptr()) == bad
     assert k.lib.tf_upload_packed_experts_layer(k.handle, None, str(tmp_path).encode(), stride, num_experts, None, pool.data_ptr()) == bad   # a directory
+
+
+def test_resident_payload_upload_and_shared_expert_through_tensor_views(tmp_path):
+    """model_weights.bin = index region (16 KiB aligned) + payload: the payload goes to one device allocation
+    (ResidentBuffer.swift:15-78) and the shared expert runs on (payload, offset) operands as Model.resident hands them out
+    (Model.swift:186-227)."""
+    import refcases
+    from oracle import tfo
+    d, f = 128, 64
+    c = refcases.shared_expert_case(d, f)
+    index_size = 16384
+    # payload: filler so that the copy takes several staging chunks, then gate / up / down as W, S, B back to back
+    filler = np.random.default_rng(5).integers(0, 256, 35 * 1024 * 1024 + 2, dtype=np.uint8)
+    parts, offsets, pos = [filler], {}, filler.size
+    for name in ("gate", "up", "down"):
+        for role, arr in zip(("w", "s", "b"), c[name]):
+            raw = np.ascontiguousarray(arr).view(np.uint8).ravel()
+            offsets[name, role] = pos
+            parts.append(raw)
+            pos += raw.size
+    payload = np.concatenate(parts)
+    path = tmp_path / "model_weights.bin"
+    with open(path, "wb") as fh:
+        fh.write(bytes(index_size))
+        fh.write(payload.tobytes())
+    k = ctx()
+    device = zeros_bytes(payload.size, 0xEE)
+    k.check(k.lib.tf_upload_file_region(k.handle, None, str(path).encode(), index_size, payload.size, device.data_ptr()))
+    assert np.array_equal(host(device, np.uint8), payload)
+
+    def proj(name, rows, cols):
+        return tfk.projection(device, device, device, rows, cols, offsets=(offsets[name, "w"], offsets[name, "s"], offsets[name, "b"]))
+    x, y = dev(c["x_bits"]), zeros_bytes(d * 2)
+    sg, su, sa = zeros_bytes(f * 2), zeros_bytes(f * 2), zeros_bytes(f * 2)
+    k.shared_expert_int4(x, proj("gate", f, d), proj("up", f, d), proj("down", d, f), y, sg, su, sa)
+    ref = tfo.shared_expert_ref(c["gate"], c["up"], c["down"], tfo.from_f16_bits(c["x_bits"]))
+    assert tfo.rel_error(tfo.from_f16_bits(host(y, np.uint16, d)), ref) < 6e-3
+    # the contract
+    enc = str(path).encode()
+    assert k.lib.tf_upload_file_region(k.handle, None, enc, index_size, payload.size + 1, device.data_ptr()) == tfk.TF_ERR_DIMENSION_MISMATCH
+    assert k.lib.tf_upload_file_region(k.handle, None, enc, index_size, 0, device.data_ptr()) == tfk.TF_ERR_INVALID_ARGUMENT
+    assert k.lib.tf_upload_file_region(k.handle, None, str(tmp_path).encode(), 0, 16, device.data_ptr()) == tfk.TF_ERR_INVALID_ARGUMENT
+    assert k.lib.tf_upload_file_region(k.handle, None, str(tmp_path / "missing.bin").encode(), 0, 16, device.data_ptr()) == tfk.TF_ERR_INVALID_ARGUMENT
+    # a sub-range in the middle
+    part = zeros_bytes(1000, 0xEE)
+    k.check(k.lib.tf_upload_file_region(k.handle, None, enc, index_size + 12345, 1000, part.data_ptr()))
+    assert np.array_equal(host(part, np.uint8), payload[12345:13345])

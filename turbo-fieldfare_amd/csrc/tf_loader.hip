@@ -1,4 +1,5 @@
-// Upload of one packed-experts layer file into an HBM-resident pool, in logical expert order.
+// File -> HBM uploads: one packed-experts layer file into a resident pool in logical expert order, and a byte range of a
+// file (the resident payload of model_weights.bin) into one allocation.
 #include <errno.h>
 #include <fcntl.h>
 #include <string.h>
@@ -104,6 +105,52 @@ int32_t tf_upload_packed_experts_layer(tf_ctx *ctx, tf_stream stream, const char
     // the staging buffers are released on return
     const hipError_t err = hipStreamSynchronize(s);
     if (err != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "upload_packed_experts_layer: %s", hipGetErrorString(err));
+    return TF_OK;
+}
+
+int32_t tf_upload_file_region(tf_ctx *ctx, tf_stream stream, const char *file_path, uint64_t file_offset, uint64_t bytes,
+                              void *device_dst) {
+    TF_REQUIRE(ctx, ctx && file_path && device_dst, TF_ERR_INVALID_ARGUMENT, "upload_file_region: null argument");
+    TF_REQUIRE(ctx, bytes > 0 && file_offset <= (uint64_t)INT64_MAX && bytes <= UINT64_MAX - file_offset, TF_ERR_INVALID_ARGUMENT,
+               "upload_file_region: empty or overflowing range");
+    Fd file;
+    file.fd = open(file_path, O_RDONLY | O_CLOEXEC | O_NONBLOCK);
+    TF_REQUIRE(ctx, file.fd >= 0, TF_ERR_INVALID_ARGUMENT, "upload_file_region: cannot open %s: %s", file_path, strerror(errno));
+    struct stat st;
+    TF_REQUIRE(ctx, fstat(file.fd, &st) == 0 && S_ISREG(st.st_mode) && st.st_size >= 0, TF_ERR_INVALID_ARGUMENT,
+               "upload_file_region: %s is not a regular file", file_path);
+    // ResidentBuffer.init's bound (ResidentBuffer.swift:37-41)
+    TF_REQUIRE(ctx, file_offset + bytes <= (uint64_t)st.st_size, TF_ERR_DIMENSION_MISMATCH,
+               "upload_file_region: range [%llu, %llu) exceeds the %llu bytes of %s", (unsigned long long)file_offset,
+               (unsigned long long)(file_offset + bytes), (unsigned long long)st.st_size, file_path);
+    constexpr uint64_t kChunk = 16ull << 20;
+    const uint64_t chunk = bytes < kChunk ? bytes : kChunk;
+    Pinned staging[2];
+    Event done[2];
+    for (int i = 0; i < 2; ++i) {
+        if (hipHostMalloc(&staging[i].p, chunk, hipHostMallocDefault) != hipSuccess) return fail(ctx, TF_ERR_OUT_OF_MEMORY, "upload_file_region: no pinned staging memory");
+        if (hipEventCreateWithFlags(&done[i].e, hipEventDisableTiming) != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "upload_file_region: event creation failed");
+    }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    bool in_use[2] = {false, false};
+    int slot = 0;
+    for (uint64_t pos = 0; pos < bytes; pos += chunk, slot ^= 1) {
+        const uint64_t n = bytes - pos < chunk ? bytes - pos : chunk;
+        if (in_use[slot] && hipEventSynchronize(done[slot].e) != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "upload_file_region: copy failed");
+        if (!read_exact(file.fd, staging[slot].p, n, file_offset + pos)) {
+            (void)hipStreamSynchronize(s);
+            return fail(ctx, TF_ERR_DEVICE, "upload_file_region: short read from %s at byte %llu", file_path, (unsigned long long)(file_offset + pos));
+        }
+        hipError_t err = hipMemcpyAsync(static_cast<uint8_t *>(device_dst) + pos, staging[slot].p, n, hipMemcpyHostToDevice, s);
+        if (err == hipSuccess) err = hipEventRecord(done[slot].e, s);
+        if (err != hipSuccess) {
+            (void)hipStreamSynchronize(s);
+            return fail(ctx, TF_ERR_DEVICE, "upload_file_region: %s", hipGetErrorString(err));
+        }
+        in_use[slot] = true;
+    }
+    const hipError_t err = hipStreamSynchronize(s);   // the staging buffers are released on return
+    if (err != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "upload_file_region: %s", hipGetErrorString(err));
     return TF_OK;
 }
 
