@@ -320,6 +320,29 @@ def extras(torch, tfk, k, gen, lib, h, stream):
     res["fused_qkv_gemv_8192x2816"] = {"us_per_call": round(us, 3), "GBps": round(nbytes / (us * 1e-6) / 1e9, 1),
                                        "frac_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": nbytes}
 
+    # decode attention over an fp16 KV cache: a global layer (16 query heads on 2 kv heads, head_dim 512) at 32768 positions and a
+    # sliding-window layer (16 on 8, head_dim 256, window 1024); three caches each, rotated, so the rows come from HBM
+    attn = {}
+    for name, hd, nq, nkv, seq, window in (("full_16q_2kv_d512_T32768", 512, 16, 2, 32768, None), ("swa_16q_8kv_d256_w1024", 256, 16, 8, 4096, 1024)):
+        caches = [(torch.randn((seq, nkv, hd), device="cuda", generator=gen).to(torch.float16) * 0.3,
+                   torch.randn((seq, nkv, hd), device="cuda", generator=gen).to(torch.float16)) for _ in range(3)]
+        qv = torch.randn((nq, hd), device="cuda", generator=gen).to(torch.float16) * 0.3
+        ov = torch.zeros((nq, hd), dtype=torch.float16, device="cuda")
+
+        def attend(i):
+            kc, vc = caches[i % 3]
+            if window is None:
+                k.attention_full(qv, kc, vc, ov, hd, nq, nkv, seq, 1.0)
+            else:
+                k.attention_swa(qv, kc, vc, ov, hd, nq, nkv, seq, window, 1.0)
+        us = time_loop(torch, attend, 100, warmup=10)
+        rows = seq if window is None else min(seq, window)
+        nbytes = rows * nkv * hd * 2 * 2 + 2 * nq * hd * 2
+        attn[name] = {"us_per_call": round(us, 2), "GBps": round(nbytes / (us * 1e-6) / 1e9, 1),
+                      "frac_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4), "algorithmic_bytes": nbytes}
+        del caches
+    res["decode_attention"] = attn
+
     # shared expert chain (gate/up 2112x2816 fused + GeGLU, down 2816x2112), rotating over 64 replicas of each matrix
     sreps = 64
     gu = W[: sreps * 2 * F_SHARED], S[: sreps * 2 * F_SHARED], B[: sreps * 2 * F_SHARED]

@@ -243,6 +243,33 @@ int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream,
                                             uint32_t x_stride_elements, uint32_t y_stride_elements,
                                             uint32_t weight_bits, tf_dtype scale_dtype);
 
+/* ---- decode attention (next in line after the quantized matmuls: the step between the QKV and the O projection) --- */
+/* Attention.encodeSWA / encodeFull (Kernels/Attention/Attention.swift:150-214) -> attention_decode_partial,
+ * attention_decode_gqa_swa_partial, attention_decode_combine (Metal/Attention/attention.metal:135-377): one query token,
+ * q fp16 [num_q_heads, head_dim], k and v fp16 [rows, num_kv_heads, head_dim], out fp16 [num_q_heads, head_dim];
+ * query head h reads kv head h / (num_q_heads / num_kv_heads).  Split-KV online softmax in fp32: un-normalized partial
+ * states per chunk of positions, then a merge; the number of chunks is chosen for this GPU, not the reference's 8 / 16
+ * (which only changes fp32 rounding of the partial sums, as the reference notes at :128-133).  scale <= 0 selects
+ * 1 / sqrt(head_dim) (the reference's nil).  SWA attends to [max(0, seq_len - window), seq_len); ring_capacity != 0:
+ * position p lives in row p % ring_capacity and the window must fit the ring.  Preconditions as the reference's:
+ * num_q_heads % num_kv_heads == 0, head_dim <= 512, num_q_heads <= 16, (full) seq_len > 0 -> TF_ERR_INVALID_ARGUMENT.
+ * An empty SWA range writes zeros.  Partial states live in scratch owned by the context, as in the reference. */
+int32_t tf_attention_swa(tf_ctx *ctx, tf_stream stream, const void *q, uint64_t q_offset, const void *k, uint64_t k_offset,
+                         const void *v, uint64_t v_offset, void *out, uint64_t out_offset, uint32_t head_dim,
+                         uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len, uint32_t window, float scale,
+                         uint32_t ring_capacity);
+int32_t tf_attention_full(tf_ctx *ctx, tf_stream stream, const void *q, uint64_t q_offset, const void *k, uint64_t k_offset,
+                          const void *v, uint64_t v_offset, void *out, uint64_t out_offset, uint32_t head_dim,
+                          uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len, float scale);
+
+/* AttentionSplitGeometry / Attention.splitGeometry (Attention.swift:5-11,128-147): the reference's own dispatch shape for
+ * a range, kept for callers that report it; pure host function, no context. */
+typedef struct tf_attention_split_geometry_t {
+    int32_t effective_length, num_chunks, chunk_length, partial_threadgroups, use_swa_grouped_partial;
+} tf_attention_split_geometry_t;
+void tf_attention_split_geometry(uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len, uint32_t kv_start,
+                                 int32_t prefer_gqa_swa, tf_attention_split_geometry_t *out);
+
 /* ---- router ----------------------------------------------------------------------------------------------------- */
 /* MoE.encodeRouterGemma4 (Kernels/MoE/MoE.swift:109-159) -> router_gemv_gemma4_r4 + router_topk_select_k8
  * (Metal/MoE/moe.metal:78-185).  hidden fp16 [d] (no offset, as in the reference), effective_scale bf16 [d],

@@ -997,4 +997,103 @@ float tfo_k_prefill_int4_row(const uint8_t *W, const uint16_t *S, const uint16_t
     return acc;
 }
 
+// ---------------------------------------------------------------------------------------------------- attention (decode)
+// V/Support/Reference/Attention/Attention.swift:14-108 (AttentionRef.apply): per query head all scores of the window
+// [kv_start, seq_len), a stable softmax, then the probability-weighted sum of V.  q [num_q_heads, head_dim] fp32;
+// k, v [seq_len, num_kv_heads, head_dim] fp32; window < 0: none; scale <= 0: 1/sqrt(head_dim).  Accumulation in double
+// (the reference sums in fp32 through vDSP, whose order is not specified).
+void tfo_attention_ref(const float *q, const float *k, const float *v, int head_dim, int num_q_heads, int num_kv_heads, int seq_len,
+                       int window, float scale, float *out) {
+    const int group = num_q_heads / num_kv_heads;
+    const double sc = scale > 0.0f ? (double)scale : 1.0 / std::sqrt((double)head_dim);
+    const int kv_start = (window >= 0 && seq_len > window) ? seq_len - window : 0;
+    std::vector<double> scores((size_t)std::max(1, seq_len - kv_start));
+    for (int qh = 0; qh < num_q_heads; ++qh) {
+        const int kvh = qh / group;
+        const float *qr = q + (size_t)qh * head_dim;
+        double mx = -INFINITY;
+        for (int p = kv_start; p < seq_len; ++p) {
+            const float *kr = k + ((size_t)p * num_kv_heads + kvh) * head_dim;
+            double dot = 0.0;
+            for (int i = 0; i < head_dim; ++i) dot += (double)qr[i] * (double)kr[i];
+            scores[(size_t)(p - kv_start)] = dot * sc;
+            mx = std::max(mx, dot * sc);
+        }
+        double sum = 0.0;
+        for (int p = kv_start; p < seq_len; ++p) {
+            scores[(size_t)(p - kv_start)] = std::exp(scores[(size_t)(p - kv_start)] - mx);
+            sum += scores[(size_t)(p - kv_start)];
+        }
+        for (int i = 0; i < head_dim; ++i) {
+            double acc = 0.0;
+            for (int p = kv_start; p < seq_len; ++p) acc += scores[(size_t)(p - kv_start)] * (double)v[((size_t)p * num_kv_heads + kvh) * head_dim + i];
+            out[(size_t)qh * head_dim + i] = sum > 0.0 ? (float)(acc / sum) : 0.0f;
+        }
+    }
+}
+
+// Kernel-order restatement of the split-KV decode path (M/Attention/attention.metal:135-222 attention_decode_partial and
+// :339-377 attention_decode_combine; K/Attention/Attention.swift:128-147 for the split): fp16 inputs, the online-softmax
+// recurrence in fp32 position by position inside each of num_chunks chunks of chunk_len positions, the un-normalized
+// partial (m, d, o) per chunk, then the merge and the fp16 result.  ring_capacity != 0: position p lives in row
+// p % ring_capacity of k / v (attn_ring_slot, :76-81).  Physical k, v: [rows, num_kv_heads, head_dim] fp16.
+void tfo_k_attention_split(const uint16_t *q_f16, const uint16_t *k_f16, const uint16_t *v_f16, int head_dim, int num_q_heads,
+                           int num_kv_heads, int seq_len, int kv_start, int chunk_len, int num_chunks, float scale, int ring_capacity,
+                           uint16_t *out_f16) {
+    const int group = num_q_heads / num_kv_heads;
+    std::vector<float> m((size_t)num_chunks), d((size_t)num_chunks), o((size_t)num_chunks * head_dim);
+    for (int qh = 0; qh < num_q_heads; ++qh) {
+        const int kvh = qh / group;
+        for (int c = 0; c < num_chunks; ++c) {
+            const int p_start = kv_start + c * chunk_len, p_end = std::min(p_start + chunk_len, seq_len);
+            float m_run = -INFINITY, d_run = 0.0f;
+            float *oc = o.data() + (size_t)c * head_dim;
+            for (int i = 0; i < head_dim; ++i) oc[i] = 0.0f;
+            for (int p = p_start; p < p_end; ++p) {
+                const int row = ring_capacity ? p % ring_capacity : p;
+                const uint16_t *kr = k_f16 + ((size_t)row * num_kv_heads + kvh) * head_dim;
+                const uint16_t *vr = v_f16 + ((size_t)row * num_kv_heads + kvh) * head_dim;
+                float s = 0.0f;
+                for (int i = 0; i < head_dim; ++i) s = std::fma(tfo_f16_to_float(q_f16[(size_t)qh * head_dim + i]), tfo_f16_to_float(kr[i]), s);
+                s *= scale;
+                const float m_new = std::max(m_run, s);
+                const float alpha = std::exp(m_run - m_new), p_exp = std::exp(s - m_new);
+                d_run = d_run * alpha + p_exp;
+                for (int i = 0; i < head_dim; ++i) oc[i] = oc[i] * alpha + p_exp * tfo_f16_to_float(vr[i]);
+                m_run = m_new;
+            }
+            m[(size_t)c] = m_run;
+            d[(size_t)c] = d_run;
+        }
+        float m_glob = -INFINITY;
+        for (int c = 0; c < num_chunks; ++c) m_glob = std::max(m_glob, m[(size_t)c]);
+        float D = 0.0f;
+        for (int c = 0; c < num_chunks; ++c) D += d[(size_t)c] * std::exp(m[(size_t)c] - m_glob);
+        const float inv_d = D > 0.0f ? 1.0f / D : 0.0f;
+        for (int i = 0; i < head_dim; ++i) {
+            float acc = 0.0f;
+            for (int c = 0; c < num_chunks; ++c) acc += o[(size_t)c * head_dim + i] * std::exp(m[(size_t)c] - m_glob);
+            out_f16[(size_t)qh * head_dim + i] = tfo_f16_bits(acc * inv_d);
+        }
+    }
+}
+
+// K/Attention/Attention.swift:122-147 (Attention.chunkCount / splitGeometry): out = {effectiveLength, numChunks, chunkLength,
+// partialThreadgroups, useSWAGroupedPartial}
+void tfo_attention_split_geometry(uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len, uint32_t kv_start, int prefer_gqa_swa,
+                                  int32_t *out5) {
+    const int q_per_kv = (int)(num_q_heads / num_kv_heads);
+    const bool grouped = prefer_gqa_swa && q_per_kv <= 2;
+    const int effective = (int)seq_len - (int)kv_start;
+    const int eff = std::max(1, effective);
+    const int default_chunks = grouped ? 8 : 16;
+    const int base = std::max(1, std::min(default_chunks, std::min(64, eff)));
+    const int chunks = grouped ? std::max(base, std::min(64, base * q_per_kv)) : base;
+    out5[0] = effective;
+    out5[1] = chunks;
+    out5[2] = (eff + chunks - 1) / chunks;
+    out5[3] = (grouped ? (int)num_kv_heads : (int)num_q_heads) * chunks;
+    out5[4] = grouped ? 1 : 0;
+}
+
 }  // extern "C"

@@ -197,6 +197,15 @@ void tfo_k_prefill_router_logits(const uint8_t *W, const uint16_t *S, const uint
 float tfo_k_prefill_int4_row(const uint8_t *W, const uint16_t *S, const uint16_t *B, const uint16_t *x_f16,
                              int row, int n);                                  /* M/Prefill/prefill.metal:406-440 */
 
+/* decode attention: AttentionRef.apply, the kernel-order split-KV path, Attention.splitGeometry */
+void tfo_attention_ref(const float *q, const float *k, const float *v, int head_dim, int num_q_heads, int num_kv_heads, int seq_len,
+                       int window, float scale, float *out);
+void tfo_k_attention_split(const uint16_t *q_f16, const uint16_t *k_f16, const uint16_t *v_f16, int head_dim, int num_q_heads,
+                           int num_kv_heads, int seq_len, int kv_start, int chunk_len, int num_chunks, float scale, int ring_capacity,
+                           uint16_t *out_f16);
+void tfo_attention_split_geometry(uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len, uint32_t kv_start, int prefer_gqa_swa,
+                                  int32_t *out5);
+
 #ifdef __cplusplus
 }
 #endif

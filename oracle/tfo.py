@@ -604,3 +604,31 @@ def to_f16_bits(x) -> np.ndarray:
 
 def from_f16_bits(b) -> np.ndarray:
     return np.asarray(b, np.uint16).view(np.float16).astype(np.float32)
+
+
+# ---- decode attention ----------------------------------------------------------------------
+_sig("tfo_attention_ref", None, f32p, f32p, f32p, i32, i32, i32, i32, i32, C.c_float, f32p)
+_sig("tfo_k_attention_split", None, u16p, u16p, u16p, i32, i32, i32, i32, i32, i32, i32, C.c_float, i32, u16p)
+_sig("tfo_attention_split_geometry", None, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, i32, C.POINTER(C.c_int32))
+
+
+def attention_ref(q, k, v, head_dim: int, num_q_heads: int, num_kv_heads: int, seq_len: int, window=None, scale=None) -> np.ndarray:
+    """AttentionRef.apply: q [Hq, D], k / v [T, Hkv, D] as float32 -> [Hq * D] float32."""
+    out = np.empty(num_q_heads * head_dim, np.float32)
+    lib.tfo_attention_ref(_flat32(q), _flat32(k), _flat32(v), head_dim, num_q_heads, num_kv_heads, seq_len,
+                          -1 if window is None else int(window), 0.0 if scale is None else float(scale), out)
+    return out
+
+
+def k_attention_split(q_bits, k_bits, v_bits, head_dim, num_q_heads, num_kv_heads, seq_len, kv_start, chunk_len, num_chunks, scale,
+                      ring_capacity=0) -> np.ndarray:
+    out = np.empty(num_q_heads * head_dim, np.uint16)
+    lib.tfo_k_attention_split(_u16(q_bits), _u16(k_bits), _u16(v_bits), head_dim, num_q_heads, num_kv_heads, seq_len, kv_start,
+                              chunk_len, num_chunks, float(scale), ring_capacity, out)
+    return out
+
+
+def attention_split_geometry(num_q_heads, num_kv_heads, seq_len, kv_start, prefer_gqa_swa: bool) -> dict:
+    out = (C.c_int32 * 5)()
+    lib.tfo_attention_split_geometry(num_q_heads, num_kv_heads, seq_len, kv_start, int(prefer_gqa_swa), out)
+    return dict(effectiveLength=out[0], numChunks=out[1], chunkLength=out[2], partialThreadgroups=out[3], useSWAGroupedPartial=bool(out[4]))

@@ -45,6 +45,12 @@ class Projection(C.Structure):
                 ("biases", vp), ("biases_offset", u64), ("rows", u32), ("cols", u32)]
 
 
+class AttentionSplitGeometry(C.Structure):
+    """AttentionSplitGeometry (Kernels/Attention/Attention.swift:5-11)."""
+    _fields_ = [("effective_length", C.c_int32), ("num_chunks", C.c_int32), ("chunk_length", C.c_int32),
+                ("partial_threadgroups", C.c_int32), ("use_swa_grouped_partial", C.c_int32)]
+
+
 class RoutedBlobs(C.Structure):
     """tf_routed_blobs."""
     _fields_ = [("blobs", vp * 8), ("pool", vp), ("pool_stride", u64), ("indices", vp), ("num_experts", u32)]
@@ -115,6 +121,9 @@ EXPORTS = {
     "tf_prefill_shared_expert_int4_block": (i32, [vp, vp, vp, u64, vp, u64, C.POINTER(Projection), C.POINTER(Projection),
                                                   C.POINTER(Projection), vp, u64, u64, vp, u64, u64, vp, u64, u64, u32, u32, u32,
                                                   u32, u32, u32, i32]),
+    "tf_attention_swa": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, u32, C.c_float, u32]),
+    "tf_attention_full": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, C.c_float]),
+    "tf_attention_split_geometry": (None, [u32, u32, u32, u32, i32, C.POINTER(AttentionSplitGeometry)]),
     "tf_router_gemma4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, vp, u64, vp, u64, vp, vp, u32, u32, u32]),
     "tf_moe_phase1_gate_up_act": (i32, [vp, vp, C.POINTER(RoutedBlobs), C.POINTER(ExpertOffsets), vp, vp, u32, u32, u32, i32]),
     "tf_moe_phase1_gate_up_act_subset": (i32, [vp, vp, C.POINTER(RoutedBlobs), C.POINTER(ExpertOffsets), vp, vp, vp, u32,
@@ -313,6 +322,18 @@ class Context:
                                                           _p(sa), 0, nbytes(sa), query_count, d, intermediate,
                                                           d if x_stride is None else x_stride, d if y_stride is None else y_stride,
                                                           weight_bits, scale_dtype)
+        return self.check(rc) if raise_on_error else rc
+
+    def attention_swa(self, q, k, v, out, head_dim, num_q_heads, num_kv_heads, seq_len, window, scale=0.0, ring_capacity=0,
+                      offsets=(0, 0, 0, 0), raise_on_error=True):
+        rc = self.lib.tf_attention_swa(self.handle, _stream(), _p(q), offsets[0], _p(k), offsets[1], _p(v), offsets[2], _p(out), offsets[3],
+                                       head_dim, num_q_heads, num_kv_heads, seq_len, window, scale, ring_capacity)
+        return self.check(rc) if raise_on_error else rc
+
+    def attention_full(self, q, k, v, out, head_dim, num_q_heads, num_kv_heads, seq_len, scale=0.0, offsets=(0, 0, 0, 0),
+                       raise_on_error=True):
+        rc = self.lib.tf_attention_full(self.handle, _stream(), _p(q), offsets[0], _p(k), offsets[1], _p(v), offsets[2], _p(out), offsets[3],
+                                        head_dim, num_q_heads, num_kv_heads, seq_len, scale)
         return self.check(rc) if raise_on_error else rc
 
     def lm_head_greedy(self, hidden, norm_w, W, S, B, out_token, d, vocab, eps=1e-6, scale_dtype=TF_BF16,

@@ -1,0 +1,438 @@
+// Single-token decode attention over an fp16 KV cache: split-KV online softmax (partial states per chunk, then a merge),
+// sliding-window and full-causal, grouped-query, optional ring addressing of the window's rows.
+//
+// One block serves ALL query heads of one KV head for one chunk of positions, so every K and V row is read once however
+// many query heads share it.  A wave takes 16 positions at a time:
+//   scores  S[16 positions, heads] = K_tile . Q^T on the matrix cores (v_mfma_f32_16x16x32_f16: lane (i, kb) supplies
+//           8 consecutive elements of K row i, the query fragments stay in registers), which also does the cross-lane
+//           reduction that a vector-ALU dot product would need per position and head;
+//   softmax the online recurrence per head, once per tile (m, d and the rescale factor alpha);
+//   values  O[head, :] = alpha O[head, :] + sum_p P[p, head] V[p, :] on the vector ALU with V rows read fully coalesced
+//           (a lane owns 8 consecutive output elements), probabilities passed through a per-wave LDS tile.
+// The four waves of a block, and then the chunks, are merged with the usual rescale by exp(m - m_max).
+#include "tf_common.hpp"
+#include "tf_context.hpp"
+
+using namespace tfk;
+
+namespace {
+
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+constexpr int kAttnThreads = 256;
+constexpr int kAttnWaves = kAttnThreads / 64;
+constexpr int kTilePositions = 16;
+constexpr int kTileHeads = 16;        // columns of the score tile; heads beyond the group are zero
+constexpr uint32_t kMaxHeadDim = 512; // Attention.maxHeadDim
+constexpr uint32_t kMaxQHeads = 16;   // Attention.maxQHeads
+constexpr uint32_t kMaxDeviceChunks = 512;
+
+struct AttnShape {
+    uint32_t num_q_heads, num_kv_heads;
+    uint32_t seq_len, kv_start, chunk_len, num_chunks, ring_capacity;
+    float scale;
+};
+
+__device__ __forceinline__ uint32_t physical_row(const AttnShape &s, uint32_t p) { return s.ring_capacity ? p % s.ring_capacity : p; }
+
+__device__ __forceinline__ float exp_weight(float m, float m_max) { return m == -INFINITY ? 0.0f : __expf(m - m_max); }
+
+// ---- matrix-core path: HD in {64, 128, 256, 512}, G = query heads per KV head in {1, 2, 4, 8}, 16-byte aligned rows
+template <int HD, int G>
+__global__ __launch_bounds__(kAttnThreads, 1) void attention_partial_kernel(const half_t *Q, const half_t *K, const half_t *V, float *m_out,
+                                                                            float *d_out, float *o_out, AttnShape s) {
+    constexpr int KS = HD / 32;                 // MFMA steps over the head dimension
+    constexpr int LPR = HD / 8;                 // lanes that cover one V row
+    constexpr int R = 64 / LPR;                 // V rows per load instruction
+    constexpr int VLOADS = kTilePositions / R;  // V load instructions per tile
+    __shared__ __align__(16) half_t p_tile[kAttnWaves][kTilePositions][kTileHeads];   // probabilities, rounded to fp16 for the packed dot
+    __shared__ float alpha_tile[kAttnWaves][kTileHeads];
+    __shared__ float m_wave[kAttnWaves][kTileHeads], d_wave[kAttnWaves][kTileHeads];
+    __shared__ float o_wave[kAttnWaves][G][HD];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t kv_head = blockIdx.x / s.num_chunks, chunk = blockIdx.x % s.num_chunks;
+    const uint32_t p_start = s.kv_start + chunk * s.chunk_len;
+    const uint32_t p_end = min(p_start + s.chunk_len, s.seq_len);
+    const int col = lane & 15, quad = lane >> 4;   // score tile: head `col`, positions 4 quad .. 4 quad + 3
+    const size_t row_halves = (size_t)s.num_kv_heads * HD;
+
+    // query fragments: lane (n, kb) holds Q[head n][32 d + 8 kb ..] for every step d; heads beyond the group are zero
+    half8_t qf[KS];
+#pragma unroll
+    for (int d = 0; d < KS; ++d) {
+        u32x4 raw = {0u, 0u, 0u, 0u};
+        if (col < G) raw = load16(Q + (size_t)(kv_head * G + (uint32_t)col) * HD + 32 * d + 8 * quad);
+        qf[d] = __builtin_bit_cast(half8_t, raw);
+    }
+    float o[G][8];
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[g][e] = 0.0f;
+    float m_run = -INFINITY, d_run = 0.0f;   // of head `col`
+    const int vrow = lane / LPR, ve = lane % LPR;
+
+    // two tiles of K and V rows in flight: the next tile is requested before the current one is reduced
+    auto request = [&](u32x4 *kf, u32x4 *vf, uint32_t t0) {
+        // rows past the chunk repeat its last row; their scores are masked and their probabilities are zero
+        const uint32_t pk = min(t0 + (uint32_t)col, p_end - 1);
+        const half_t *k_row = K + (size_t)physical_row(s, pk) * row_halves + (size_t)kv_head * HD + 8 * quad;
+#pragma unroll
+        for (int d = 0; d < KS; ++d) kf[d] = load16(k_row + 32 * d);
+#pragma unroll
+        for (int j = 0; j < VLOADS; ++j) {
+            const uint32_t pv = min(t0 + (uint32_t)(j * R + vrow), p_end - 1);
+            vf[j] = load16(V + (size_t)physical_row(s, pv) * row_halves + (size_t)kv_head * HD + 8 * ve);
+        }
+    };
+    auto consume = [&](const u32x4 *kf, const u32x4 *vf, uint32_t t0) {
+        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int d = 0; d < KS; ++d) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, kf[d]), qf[d], acc, 0, 0, 0);
+        float sc[4], tile_max = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            sc[r] = t0 + (uint32_t)(4 * quad + r) < p_end ? acc[r] * s.scale : -INFINITY;
+            tile_max = fmaxf(tile_max, sc[r]);
+        }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+        const float m_new = fmaxf(m_run, tile_max);          // finite: the tile holds at least one position
+        const float alpha = exp_weight(m_run, m_new);
+        float sum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float pe = exp_weight(sc[r], m_new);
+            p_tile[wave][4 * quad + r][col] = (half_t)pe;
+            sum += pe;
+        }
+        sum += __shfl_xor(sum, 16);
+        sum += __shfl_xor(sum, 32);
+        d_run = d_run * alpha + sum;
+        m_run = m_new;
+        if (quad == 0) alpha_tile[wave][col] = alpha;
+        // the wave reads back what its own lanes wrote: LDS operations of one wave complete in order
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+        for (int g = 0; g < G; ++g) {
+            const float a = alpha_tile[wave][g];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[g][e] *= a;
+        }
+        // two positions per instruction: v_dot2_f32_f16 adds p_a v_a + p_b v_b to the fp32 sum.  Loads j and j + 1 of a
+        // lane hold rows a = j R + vrow and b = a + R; their elements are interleaved into (v_a[e], v_b[e]) pairs and the
+        // two probability rows into (p_a[g], p_b[g]) pairs.
+#pragma unroll
+        for (int j = 0; j < VLOADS; j += 2) {
+            const u32x4 ra = vf[j], rb = vf[j + 1];
+            uint32_t vv[8];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                vv[2 * w] = __builtin_amdgcn_perm(rb[w], ra[w], 0x05040100u);       // (a.lo, b.lo)
+                vv[2 * w + 1] = __builtin_amdgcn_perm(rb[w], ra[w], 0x07060302u);   // (a.hi, b.hi)
+            }
+            const u32x4 pa = *reinterpret_cast<const u32x4 *>(&p_tile[wave][j * R + vrow][0]);
+            const u32x4 pb = *reinterpret_cast<const u32x4 *>(&p_tile[wave][(j + 1) * R + vrow][0]);
+#pragma unroll
+            for (int g = 0; g < G; ++g) {
+                const uint32_t sel = (g & 1) ? 0x07060302u : 0x05040100u;
+                const half2_t pg = as_half2(__builtin_amdgcn_perm(pb[g >> 1], pa[g >> 1], sel));
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[g][e] = __builtin_amdgcn_fdot2(pg, as_half2(vv[e]), o[g][e], false);
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the tile is rewritten by the next one
+    };
+    constexpr uint32_t kStride = kAttnWaves * kTilePositions;
+    u32x4 ka[KS], va[VLOADS], kb[KS], vb[VLOADS];
+    uint32_t ta = p_start + (uint32_t)wave * kTilePositions, tb = ta + kStride;
+    if (ta < p_end) {
+        request(ka, va, ta);
+        for (;;) {
+            if (tb < p_end) request(kb, vb, tb);
+            consume(ka, va, ta);
+            ta += 2 * kStride;
+            if (tb >= p_end) break;
+            if (ta < p_end) request(ka, va, ta);
+            consume(kb, vb, tb);
+            tb += 2 * kStride;
+            if (ta >= p_end) break;
+        }
+    }
+
+    // lanes that served different rows of a load hold different parts of the same sums
+#pragma unroll
+    for (int g = 0; g < G; ++g)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            float v = o[g][e];
+            if constexpr (R >= 2) v += __shfl_xor(v, 32);
+            if constexpr (R >= 4) v += __shfl_xor(v, 16);
+            if constexpr (R >= 8) v += __shfl_xor(v, 8);
+            o[g][e] = v;
+        }
+    if (quad == 0) {
+        m_wave[wave][col] = m_run;
+        d_wave[wave][col] = d_run;
+    }
+    if (vrow == 0) {
+#pragma unroll
+        for (int g = 0; g < G; ++g)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o_wave[wave][g][8 * ve + e] = o[g][e];
+    }
+    __syncthreads();
+    // merge of the four waves -> the chunk's un-normalized partial state per query head
+    for (int idx = threadIdx.x; idx < G * HD; idx += kAttnThreads) {
+        const int g = idx / HD, i = idx - g * HD;
+        float m_max = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < kAttnWaves; ++w) m_max = fmaxf(m_max, m_wave[w][g]);
+        float acc = 0.0f, den = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kAttnWaves; ++w) {
+            const float wt = exp_weight(m_wave[w][g], m_max);
+            acc += o_wave[w][g][i] * wt;
+            den += d_wave[w][g] * wt;
+        }
+        const size_t base = (size_t)(kv_head * G + (uint32_t)g) * s.num_chunks + chunk;
+        o_out[base * HD + i] = acc;
+        if (i == 0) {
+            m_out[base] = m_max;
+            d_out[base] = den;
+        }
+    }
+}
+
+// ---- any head dimension, group size and alignment: one block per (query head, chunk), position by position, the
+// reference kernel's own shape (attention.metal:135-222)
+__global__ __launch_bounds__(kAttnThreads) void attention_partial_generic_kernel(const half_t *Q, const half_t *K, const half_t *V,
+                                                                                 float *m_out, float *d_out, float *o_out, uint32_t head_dim,
+                                                                                 AttnShape s) {
+    __shared__ float q_s[kMaxHeadDim];
+    __shared__ float part[kAttnWaves];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t q_head = blockIdx.x / s.num_chunks, chunk = blockIdx.x % s.num_chunks;
+    const uint32_t kv_head = q_head / (s.num_q_heads / s.num_kv_heads);
+    const uint32_t p_start = s.kv_start + chunk * s.chunk_len, p_end = min(p_start + s.chunk_len, s.seq_len);
+    for (uint32_t i = threadIdx.x; i < head_dim; i += kAttnThreads) q_s[i] = (float)Q[(size_t)q_head * head_dim + i];
+    __syncthreads();
+    float o_local[(kMaxHeadDim + kAttnThreads - 1) / kAttnThreads] = {};
+    float m_run = -INFINITY, d_run = 0.0f;
+    for (uint32_t p = p_start; p < p_end; ++p) {
+        const size_t row = ((size_t)physical_row(s, p) * s.num_kv_heads + kv_head) * head_dim;
+        float partial = 0.0f;
+        for (uint32_t i = threadIdx.x; i < head_dim; i += kAttnThreads) partial = fmaf(q_s[i], (float)K[row + i], partial);
+        partial = wave_sum(partial);
+        __syncthreads();   // the previous position's sums have been read
+        if (lane == 0) part[wave] = partial;
+        __syncthreads();
+        float sc = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kAttnWaves; ++w) sc += part[w];
+        sc *= s.scale;
+        const float m_new = fmaxf(m_run, sc);
+        const float alpha = exp_weight(m_run, m_new), pe = __expf(sc - m_new);
+        d_run = d_run * alpha + pe;
+        int slot = 0;
+        for (uint32_t i = threadIdx.x; i < head_dim; i += kAttnThreads, ++slot) o_local[slot] = o_local[slot] * alpha + pe * (float)V[row + i];
+        m_run = m_new;
+    }
+    const size_t base = (size_t)q_head * s.num_chunks + chunk;
+    if (threadIdx.x == 0) {
+        m_out[base] = m_run;
+        d_out[base] = d_run;
+    }
+    int slot = 0;
+    for (uint32_t i = threadIdx.x; i < head_dim; i += kAttnThreads, ++slot) o_out[base * head_dim + i] = o_local[slot];
+}
+
+// attention_decode_combine (attention.metal:339-377): out = sum_c o_c e^{m_c - m} / sum_c d_c e^{m_c - m}.
+// Block = one query head x 64 output elements; the chunk weights e^{m_c - m} are formed once per block in LDS, and the
+// four waves each add every fourth chunk (in ascending order) before the four sums are added in wave order.
+constexpr uint32_t kCombineElems = 64;
+__global__ __launch_bounds__(kAttnThreads) void attention_combine_kernel(const float *m_in, const float *d_in, const float *o_in, half_t *out,
+                                                                         uint32_t head_dim, uint32_t num_chunks) {
+    __shared__ float weight[kMaxDeviceChunks];
+    __shared__ float red[kAttnWaves], sums[kAttnWaves][kCombineElems];
+    const uint32_t q_head = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float *m_row = m_in + (size_t)q_head * num_chunks, *d_row = d_in + (size_t)q_head * num_chunks;
+    float m_max = -INFINITY;
+    for (uint32_t c = threadIdx.x; c < num_chunks; c += kAttnThreads) m_max = fmaxf(m_max, m_row[c]);
+    m_max = wave_max(m_max);
+    if (lane == 0) red[wave] = m_max;
+    __syncthreads();
+    m_max = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    float den = 0.0f;
+    for (uint32_t c = threadIdx.x; c < num_chunks; c += kAttnThreads) {
+        const float w = exp_weight(m_row[c], m_max);
+        weight[c] = w;
+        den += d_row[c] * w;
+    }
+    den = wave_sum(den);
+    if (lane == 0) red[wave] = den;
+    __syncthreads();
+    den = (red[0] + red[1]) + (red[2] + red[3]);
+    const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+    const uint32_t i = blockIdx.y * kCombineElems + lane;
+    float acc = 0.0f;
+    if (i < head_dim) {
+        const float *o_base = o_in + (size_t)q_head * num_chunks * head_dim + i;
+        // eight loads in flight per lane; the additions stay in ascending chunk order
+        for (uint32_t c0 = wave; c0 < num_chunks; c0 += 8 * kAttnWaves) {
+            float part[8];
+#pragma unroll
+            for (uint32_t j = 0; j < 8; ++j) {
+                const uint32_t c = c0 + j * kAttnWaves;
+                part[j] = c < num_chunks ? o_base[(size_t)c * head_dim] : 0.0f;
+            }
+#pragma unroll
+            for (uint32_t j = 0; j < 8; ++j) {
+                const uint32_t c = c0 + j * kAttnWaves;
+                if (c < num_chunks) acc = fmaf(part[j], weight[c], acc);
+            }
+        }
+    }
+    sums[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && i < head_dim) out[(size_t)q_head * head_dim + i] = (half_t)(((sums[0][lane] + sums[1][lane]) + (sums[2][lane] + sums[3][lane])) * inv);
+}
+
+// the context's partial-state scratch: m and d [heads x chunks], o [heads x chunks x head_dim]
+int32_t attention_scratch(tf_ctx *ctx, size_t floats, float *&out) {
+    const size_t need = floats * sizeof(float);
+    if (ctx->attn_scratch_bytes < need) {
+        if (ctx->attn_scratch) {
+            if (hipDeviceSynchronize() != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "attention: device synchronize failed");
+            (void)hipFree(ctx->attn_scratch);
+            ctx->attn_scratch = nullptr;
+            ctx->attn_scratch_bytes = 0;
+        }
+        if (hipMalloc(&ctx->attn_scratch, need) != hipSuccess) return fail(ctx, TF_ERR_OUT_OF_MEMORY, "attention: out of device memory");
+        ctx->attn_scratch_bytes = need;
+    }
+    out = static_cast<float *>(ctx->attn_scratch);
+    return TF_OK;
+}
+
+template <int HD>
+bool launch_partial_hd(uint32_t group, dim3 grid, hipStream_t st, const half_t *q, const half_t *k, const half_t *v, float *m, float *d, float *o,
+                       const AttnShape &s) {
+    switch (group) {
+        case 1: hipLaunchKernelGGL((attention_partial_kernel<HD, 1>), grid, dim3(kAttnThreads), 0, st, q, k, v, m, d, o, s); return true;
+        case 2: hipLaunchKernelGGL((attention_partial_kernel<HD, 2>), grid, dim3(kAttnThreads), 0, st, q, k, v, m, d, o, s); return true;
+        case 4: hipLaunchKernelGGL((attention_partial_kernel<HD, 4>), grid, dim3(kAttnThreads), 0, st, q, k, v, m, d, o, s); return true;
+        case 8: hipLaunchKernelGGL((attention_partial_kernel<HD, 8>), grid, dim3(kAttnThreads), 0, st, q, k, v, m, d, o, s); return true;
+        default: return false;
+    }
+}
+
+int32_t attention_split(tf_ctx *ctx, tf_stream stream, const void *q, uint64_t q_offset, const void *k, uint64_t k_offset, const void *v,
+                        uint64_t v_offset, void *out, uint64_t out_offset, uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
+                        uint32_t seq_len, uint32_t kv_start, float scale, uint32_t ring_capacity, const char *who) {
+    TF_REQUIRE(ctx, q && k && v && out, TF_ERR_INVALID_ARGUMENT, "%s: null argument", who);
+    TF_REQUIRE(ctx, num_kv_heads > 0 && num_q_heads > 0 && num_q_heads % num_kv_heads == 0, TF_ERR_INVALID_ARGUMENT,
+               "%s: numQHeads must be a multiple of numKVHeads for GQA", who);
+    TF_REQUIRE(ctx, head_dim > 0 && head_dim <= kMaxHeadDim, TF_ERR_INVALID_ARGUMENT, "%s: head_dim must be <= 512", who);
+    TF_REQUIRE(ctx, num_q_heads <= kMaxQHeads, TF_ERR_INVALID_ARGUMENT, "%s: numQHeads %u exceeds split-KV scratch (max %u)", who, num_q_heads,
+               kMaxQHeads);
+    TF_REQUIRE(ctx, q_offset % 2 == 0 && k_offset % 2 == 0 && v_offset % 2 == 0 && out_offset % 2 == 0, TF_ERR_INVALID_ARGUMENT,
+               "%s: offsets must be 2-byte aligned", who);
+    const half_t *qp = reinterpret_cast<const half_t *>(at(q, q_offset));
+    const half_t *kp = reinterpret_cast<const half_t *>(at(k, k_offset));
+    const half_t *vp = reinterpret_cast<const half_t *>(at(v, v_offset));
+    half_t *op = reinterpret_cast<half_t *>(at(out, out_offset));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const uint32_t group = num_q_heads / num_kv_heads;
+    const uint32_t effective = seq_len > kv_start ? seq_len - kv_start : 0;
+    const bool mfma = (head_dim == 64 || head_dim == 128 || head_dim == 256 || head_dim == 512) && (group == 1 || group == 2 || group == 4 || group == 8) &&
+                      aligned16(qp) && aligned16(kp) && aligned16(vp);
+    // chunks: enough blocks for every compute unit, whole 64-position rounds of a block's four waves
+    AttnShape s;
+    s.num_q_heads = num_q_heads;
+    s.num_kv_heads = num_kv_heads;
+    s.seq_len = seq_len;
+    s.kv_start = kv_start;
+    s.ring_capacity = ring_capacity;
+    s.scale = scale;
+    const uint32_t blocks_per_chunk = mfma ? num_kv_heads : num_q_heads;
+    const uint32_t round = mfma ? kAttnWaves * kTilePositions : 16;
+    uint32_t want = ((uint32_t)ctx->num_cus * (mfma ? 1u : 4u) + blocks_per_chunk - 1) / blocks_per_chunk;
+    want = want < kMaxDeviceChunks ? want : kMaxDeviceChunks;
+    const uint32_t eff = effective ? effective : 1;
+    uint32_t chunk_len = (eff + want - 1) / want;
+    chunk_len = (chunk_len + round - 1) / round * round;
+    s.chunk_len = chunk_len;
+    s.num_chunks = (eff + chunk_len - 1) / chunk_len;
+    float *scratch = nullptr;
+    const size_t states = (size_t)num_q_heads * s.num_chunks;
+    const int32_t rc = attention_scratch(ctx, states * (2 + (size_t)head_dim), scratch);
+    if (rc != TF_OK) return rc;
+    float *m = scratch, *d = scratch + states, *o = scratch + 2 * states;
+    const dim3 grid(blocks_per_chunk * s.num_chunks);
+    bool launched = false;
+    if (mfma) {
+        switch (head_dim) {
+            case 64: launched = launch_partial_hd<64>(group, grid, st, qp, kp, vp, m, d, o, s); break;
+            case 128: launched = launch_partial_hd<128>(group, grid, st, qp, kp, vp, m, d, o, s); break;
+            case 256: launched = launch_partial_hd<256>(group, grid, st, qp, kp, vp, m, d, o, s); break;
+            default: launched = launch_partial_hd<512>(group, grid, st, qp, kp, vp, m, d, o, s); break;
+        }
+    }
+    if (!launched) hipLaunchKernelGGL(attention_partial_generic_kernel, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, m, d, o, head_dim, s);
+    hipLaunchKernelGGL(attention_combine_kernel, dim3(num_q_heads, (head_dim + kCombineElems - 1) / kCombineElems), dim3(kAttnThreads), 0, st, m, d, o, op,
+                       head_dim, s.num_chunks);
+    return check_launch(ctx, who);
+}
+
+float default_scale(uint32_t head_dim) { return 1.0f / sqrtf((float)head_dim); }
+
+}  // namespace
+
+extern "C" {
+
+int32_t tf_attention_swa(tf_ctx *ctx, tf_stream stream, const void *q, uint64_t q_offset, const void *k, uint64_t k_offset, const void *v,
+                         uint64_t v_offset, void *out, uint64_t out_offset, uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
+                         uint32_t seq_len, uint32_t window, float scale, uint32_t ring_capacity) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "attention_swa: null context");
+    const uint32_t kv_start = seq_len > window ? seq_len - window : 0;
+    // every position of the window must still be in the ring
+    TF_REQUIRE(ctx, ring_capacity == 0 || seq_len - kv_start <= ring_capacity, TF_ERR_INVALID_ARGUMENT,
+               "attention_swa: the window (%u positions) does not fit the ring (%u rows)", seq_len - kv_start, ring_capacity);
+    return attention_split(ctx, stream, q, q_offset, k, k_offset, v, v_offset, out, out_offset, head_dim, num_q_heads, num_kv_heads, seq_len,
+                           kv_start, scale > 0.0f ? scale : default_scale(head_dim ? head_dim : 1), ring_capacity, "attention_swa");
+}
+
+int32_t tf_attention_full(tf_ctx *ctx, tf_stream stream, const void *q, uint64_t q_offset, const void *k, uint64_t k_offset, const void *v,
+                          uint64_t v_offset, void *out, uint64_t out_offset, uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
+                          uint32_t seq_len, float scale) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "attention_full: null context");
+    TF_REQUIRE(ctx, seq_len > 0, TF_ERR_INVALID_ARGUMENT, "attention_full: full attention requires at least one KV position");
+    return attention_split(ctx, stream, q, q_offset, k, k_offset, v, v_offset, out, out_offset, head_dim, num_q_heads, num_kv_heads, seq_len, 0,
+                           scale > 0.0f ? scale : default_scale(head_dim ? head_dim : 1), 0, "attention_full");
+}
+
+void tf_attention_split_geometry(uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len, uint32_t kv_start, int32_t prefer_gqa_swa,
+                                 tf_attention_split_geometry_t *out) {
+    if (!out || num_kv_heads == 0) return;
+    const int q_per_kv = (int)(num_q_heads / num_kv_heads);
+    const bool grouped = prefer_gqa_swa != 0 && q_per_kv <= 2;
+    const int effective = (int)seq_len - (int)kv_start;
+    const int eff = effective > 1 ? effective : 1;
+    const int default_chunks = grouped ? 8 : 16;
+    int base = default_chunks < 64 ? default_chunks : 64;
+    base = base < eff ? base : eff;
+    base = base > 1 ? base : 1;
+    int scaled = base * q_per_kv;
+    scaled = scaled < 64 ? scaled : 64;
+    const int chunks = grouped ? (base > scaled ? base : scaled) : base;
+    out->effective_length = effective;
+    out->num_chunks = chunks;
+    out->chunk_length = (eff + chunks - 1) / chunks;
+    out->partial_threadgroups = (grouped ? (int)num_kv_heads : (int)num_q_heads) * chunks;
+    out->use_swa_grouped_partial = grouped ? 1 : 0;
+}
+
+}  // extern "C"

@@ -120,6 +120,33 @@ private:
     const Context &c_;
 };
 
+// Attention (Kernels/Attention/Attention.swift:26-214): sliding-window and full-causal decode attention
+using AttentionSplitGeometry = tf_attention_split_geometry_t;
+class Attention {
+public:
+    explicit Attention(const Context &context) : c_(context) {}
+    static AttentionSplitGeometry splitGeometry(uint32_t numQHeads, uint32_t numKVHeads, uint32_t seqLen, uint32_t kvStart, bool preferGQASWA) {
+        AttentionSplitGeometry g{};
+        tf_attention_split_geometry(numQHeads, numKVHeads, seqLen, kvStart, preferGQASWA ? 1 : 0, &g);
+        return g;
+    }
+    // scale <= 0: 1 / sqrt(headDim), the reference's nil
+    void encodeSWA(const void *q, uint64_t qOffset, const void *k, uint64_t kOffset, const void *v, uint64_t vOffset, void *out, uint64_t outOffset,
+                   uint32_t headDim, uint32_t numQHeads, uint32_t numKVHeads, uint32_t seqLen, uint32_t window, float scale = 0.0f,
+                   uint32_t ringCapacity = 0) const {
+        c_.check(tf_attention_swa(c_.raw(), c_.stream(), q, qOffset, k, kOffset, v, vOffset, out, outOffset, headDim, numQHeads, numKVHeads, seqLen,
+                                  window, scale, ringCapacity));
+    }
+    void encodeFull(const void *q, uint64_t qOffset, const void *k, uint64_t kOffset, const void *v, uint64_t vOffset, void *out, uint64_t outOffset,
+                    uint32_t headDim, uint32_t numQHeads, uint32_t numKVHeads, uint32_t seqLen, float scale = 0.0f) const {
+        c_.check(tf_attention_full(c_.raw(), c_.stream(), q, qOffset, k, kOffset, v, vOffset, out, outOffset, headDim, numQHeads, numKVHeads, seqLen,
+                                   scale));
+    }
+
+private:
+    const Context &c_;
+};
+
 using SharedExpertProjection = tf_projection;   // Kernels/MoE/SharedExpertInt8.swift:9-31
 
 // SharedExpertRuntime / SharedExpertInt4 (Kernels/MoE/SharedExpertInt4.swift)
