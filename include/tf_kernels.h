@@ -262,6 +262,26 @@ int32_t tf_attention_full(tf_ctx *ctx, tf_stream stream, const void *q, uint64_t
                           const void *v, uint64_t v_offset, void *out, uint64_t out_offset, uint32_t head_dim,
                           uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len, float scale);
 
+/* RoPE.encodeDefaultNeox / encodeProportionalNeox (Kernels/Primitives/RoPE.swift:27-90) -> rope_default_neox,
+ * rope_proportional_neox (Metal/Primitives/rope.metal:33-96): data fp16 [num_tokens, num_heads, head_dim], in place; the
+ * pairs (x[i], x[i + head_dim/2]), i < rotated_pairs (default: head_dim / 2), rotate by position * theta^(-2i/head_dim);
+ * every token of the block gets the same position, as in the reference.  head_dim even, rotated_pairs * 2 <= head_dim. */
+int32_t tf_rope_default_neox(tf_ctx *ctx, tf_stream stream, void *data, uint64_t data_offset, uint32_t position,
+                             uint32_t head_dim, uint32_t num_heads, uint32_t num_tokens, float theta);
+int32_t tf_rope_proportional_neox(tf_ctx *ctx, tf_stream stream, void *data, uint64_t data_offset, uint32_t position,
+                                  uint32_t head_dim, uint32_t num_heads, uint32_t num_tokens, uint32_t rotated_pairs,
+                                  float theta);
+
+/* FusedQKVEpilogue.encode (Kernels/Fusions/FusedQKVEpilogue.swift:43-99) -> fused_qkv_epilogue
+ * (Metal/Fusions/fused.metal:84-173): in place, per head, q [num_q_heads, head_dim] and k [num_kv_heads, head_dim]:
+ * RMSNorm with the bf16 weight [head_dim] shared by the heads, rounded to fp16, then NeoX RoPE on the first
+ * rotated_pairs pairs; v [num_kv_heads, head_dim]: RMSNorm without weight.  head_dim <= 512 and even,
+ * rotated_pairs * 2 <= head_dim. */
+int32_t tf_fused_qkv_epilogue(tf_ctx *ctx, tf_stream stream, void *q, uint64_t q_offset, void *k, uint64_t k_offset,
+                              void *v, uint64_t v_offset, const void *q_weight, uint64_t q_weight_offset,
+                              const void *k_weight, uint64_t k_weight_offset, uint32_t head_dim, uint32_t num_q_heads,
+                              uint32_t num_kv_heads, uint32_t position, float theta, uint32_t rotated_pairs, float eps);
+
 /* AttentionSplitGeometry / Attention.splitGeometry (Attention.swift:5-11,128-147): the reference's own dispatch shape for
  * a range, kept for callers that report it; pure host function, no context. */
 typedef struct tf_attention_split_geometry_t {

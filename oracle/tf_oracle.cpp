@@ -1096,4 +1096,63 @@ void tfo_attention_split_geometry(uint32_t num_q_heads, uint32_t num_kv_heads, u
     out5[4] = grouped ? 1 : 0;
 }
 
+// ---------------------------------------------------------------------------------------------------- RoPE, QKV epilogue
+// V/Support/Reference/Attention/RoPE.swift:82-128 (RopeRef.applyNeox): pairs (x[i], x[i + head_dim / 2]) for
+// i < rotated_pairs rotate by angle position * theta^(-2 i / head_dim); everything else passes through.  fp32 in / out;
+// the angle and its cosine / sine in double (the reference uses vForce, whose rounding is not specified).
+void tfo_rope_neox_ref(const float *input, int num_tokens, int num_heads, int head_dim, int rotated_pairs, int position, float theta,
+                       float *out) {
+    const int half_dim = head_dim / 2;
+    for (size_t i = 0; i < (size_t)num_tokens * num_heads * head_dim; ++i) out[i] = input[i];
+    for (int k = 0; k < rotated_pairs; ++k) {
+        const double angle = (double)position * std::pow((double)theta, -(double)(2 * k) / (double)head_dim);
+        const double c = std::cos(angle), sn = std::sin(angle);
+        for (int th = 0; th < num_tokens * num_heads; ++th) {
+            const size_t base = (size_t)th * head_dim;
+            const double x0 = input[base + k], x1 = input[base + half_dim + k];
+            out[base + k] = (float)(x0 * c - x1 * sn);
+            out[base + half_dim + k] = (float)(x0 * sn + x1 * c);
+        }
+    }
+}
+
+// Kernel-order restatement of rope_default_neox / rope_proportional_neox (M/Primitives/rope.metal:33-96): fp16 data in
+// place, fp32 arithmetic, fp16 results.
+void tfo_k_rope_neox(uint16_t *data_f16, int num_tokens, int num_heads, int head_dim, int rotated_pairs, uint32_t position, float theta) {
+    const int half_dim = head_dim / 2;
+    for (int th = 0; th < num_tokens * num_heads; ++th) {
+        uint16_t *head = data_f16 + (size_t)th * head_dim;
+        for (int pair = 0; pair < rotated_pairs; ++pair) {
+            const float exponent = -(float)(2u * (uint32_t)pair) / (float)head_dim;
+            const float angle = (float)position * std::pow(theta, exponent);
+            const float c = std::cos(angle), sn = std::sin(angle);
+            const float x0 = tfo_f16_to_float(head[pair]), x1 = tfo_f16_to_float(head[half_dim + pair]);
+            head[pair] = tfo_f16_bits(x0 * c - x1 * sn);
+            head[half_dim + pair] = tfo_f16_bits(x0 * sn + x1 * c);
+        }
+    }
+}
+
+// Kernel-order restatement of fused_qkv_epilogue (M/Fusions/fused.metal:84-173): per head RMSNorm (q and k with their
+// bf16 weight, v without), the normalized values rounded to fp16, then NeoX RoPE on the first rotated_pairs pairs of q
+// and k; all in place.
+void tfo_k_fused_qkv_epilogue(uint16_t *q_f16, uint16_t *k_f16, uint16_t *v_f16, const uint16_t *q_weight_bf16, const uint16_t *k_weight_bf16,
+                              int head_dim, int num_q_heads, int num_kv_heads, uint32_t position, float theta, int rotated_pairs, float eps) {
+    std::vector<uint16_t> normed((size_t)head_dim);
+    for (int hg = 0; hg < num_q_heads + 2 * num_kv_heads; ++hg) {
+        const bool is_q = hg < num_q_heads, is_k = !is_q && hg < num_q_heads + num_kv_heads;
+        uint16_t *dst = is_q ? q_f16 + (size_t)hg * head_dim
+                             : (is_k ? k_f16 + (size_t)(hg - num_q_heads) * head_dim : v_f16 + (size_t)(hg - num_q_heads - num_kv_heads) * head_dim);
+        const uint16_t *w = is_q ? q_weight_bf16 : k_weight_bf16;
+        const float inv = 1.0f / std::sqrt(k_block_sum_squares(dst, head_dim) / (float)head_dim + eps);
+        for (int i = 0; i < head_dim; ++i) {
+            float xv = tfo_f16_to_float(dst[i]) * inv;
+            if (is_q || is_k) xv *= tfo_bf16_to_float(w[i]);
+            normed[(size_t)i] = tfo_f16_bits(xv);
+        }
+        for (int i = 0; i < head_dim; ++i) dst[i] = normed[(size_t)i];
+        if (is_q || is_k) tfo_k_rope_neox(dst, 1, 1, head_dim, rotated_pairs, position, theta);
+    }
+}
+
 }  // extern "C"

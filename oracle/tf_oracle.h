@@ -206,6 +206,13 @@ void tfo_k_attention_split(const uint16_t *q_f16, const uint16_t *k_f16, const u
 void tfo_attention_split_geometry(uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len, uint32_t kv_start, int prefer_gqa_swa,
                                   int32_t *out5);
 
+/* RoPE (NeoX pairs) and the fused per-head Q/K/V epilogue */
+void tfo_rope_neox_ref(const float *input, int num_tokens, int num_heads, int head_dim, int rotated_pairs, int position, float theta,
+                       float *out);
+void tfo_k_rope_neox(uint16_t *data_f16, int num_tokens, int num_heads, int head_dim, int rotated_pairs, uint32_t position, float theta);
+void tfo_k_fused_qkv_epilogue(uint16_t *q_f16, uint16_t *k_f16, uint16_t *v_f16, const uint16_t *q_weight_bf16, const uint16_t *k_weight_bf16,
+                              int head_dim, int num_q_heads, int num_kv_heads, uint32_t position, float theta, int rotated_pairs, float eps);
+
 #ifdef __cplusplus
 }
 #endif

@@ -632,3 +632,30 @@ def attention_split_geometry(num_q_heads, num_kv_heads, seq_len, kv_start, prefe
     out = (C.c_int32 * 5)()
     lib.tfo_attention_split_geometry(num_q_heads, num_kv_heads, seq_len, kv_start, int(prefer_gqa_swa), out)
     return dict(effectiveLength=out[0], numChunks=out[1], chunkLength=out[2], partialThreadgroups=out[3], useSWAGroupedPartial=bool(out[4]))
+
+
+# ---- RoPE and the Q/K/V epilogue -------------------------------------------------------------
+_sig("tfo_rope_neox_ref", None, f32p, i32, i32, i32, i32, i32, C.c_float, f32p)
+_sig("tfo_k_rope_neox", None, u16p, i32, i32, i32, i32, C.c_uint32, C.c_float)
+_sig("tfo_k_fused_qkv_epilogue", None, u16p, u16p, u16p, u16p, u16p, i32, i32, i32, C.c_uint32, C.c_float, i32, C.c_float)
+
+
+def rope_neox_ref(x, num_tokens, num_heads, head_dim, rotated_pairs, position, theta) -> np.ndarray:
+    x = _flat32(x)
+    out = np.empty_like(x)
+    lib.tfo_rope_neox_ref(x, num_tokens, num_heads, head_dim, rotated_pairs, position, float(theta), out)
+    return out
+
+
+def k_rope_neox(bits, num_tokens, num_heads, head_dim, rotated_pairs, position, theta) -> np.ndarray:
+    data = _u16(bits).copy()
+    lib.tfo_k_rope_neox(data, num_tokens, num_heads, head_dim, rotated_pairs, position, float(theta))
+    return data
+
+
+def k_fused_qkv_epilogue(q_bits, k_bits, v_bits, q_weight_bits, k_weight_bits, head_dim, num_q_heads, num_kv_heads, position, theta,
+                         rotated_pairs, eps):
+    q, k, v = _u16(q_bits).copy(), _u16(k_bits).copy(), _u16(v_bits).copy()
+    lib.tfo_k_fused_qkv_epilogue(q, k, v, _u16(q_weight_bits), _u16(k_weight_bits), head_dim, num_q_heads, num_kv_heads, position,
+                                 float(theta), rotated_pairs, float(eps))
+    return q, k, v

@@ -121,6 +121,9 @@ EXPORTS = {
     "tf_prefill_shared_expert_int4_block": (i32, [vp, vp, vp, u64, vp, u64, C.POINTER(Projection), C.POINTER(Projection),
                                                   C.POINTER(Projection), vp, u64, u64, vp, u64, u64, vp, u64, u64, u32, u32, u32,
                                                   u32, u32, u32, i32]),
+    "tf_rope_default_neox": (i32, [vp, vp, vp, u64, u32, u32, u32, u32, C.c_float]),
+    "tf_rope_proportional_neox": (i32, [vp, vp, vp, u64, u32, u32, u32, u32, u32, C.c_float]),
+    "tf_fused_qkv_epilogue": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, C.c_float, u32, C.c_float]),
     "tf_attention_swa": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, u32, C.c_float, u32]),
     "tf_attention_full": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, C.c_float]),
     "tf_attention_split_geometry": (None, [u32, u32, u32, u32, i32, C.POINTER(AttentionSplitGeometry)]),

@@ -120,6 +120,38 @@ private:
     const Context &c_;
 };
 
+// RoPE (Kernels/Primitives/RoPE.swift:4-90)
+class RoPE {
+public:
+    explicit RoPE(const Context &context) : c_(context) {}
+    void encodeDefaultNeox(void *data, uint64_t dataOffset, uint32_t position, uint32_t headDim, uint32_t numHeads, uint32_t numTokens,
+                           float theta = 10000.0f) const {
+        c_.check(tf_rope_default_neox(c_.raw(), c_.stream(), data, dataOffset, position, headDim, numHeads, numTokens, theta));
+    }
+    void encodeProportionalNeox(void *data, uint64_t dataOffset, uint32_t position, uint32_t headDim, uint32_t numHeads, uint32_t numTokens,
+                                uint32_t rotatedPairs, float theta = 1000000.0f) const {
+        c_.check(tf_rope_proportional_neox(c_.raw(), c_.stream(), data, dataOffset, position, headDim, numHeads, numTokens, rotatedPairs, theta));
+    }
+
+private:
+    const Context &c_;
+};
+
+// FusedQKVEpilogue (Kernels/Fusions/FusedQKVEpilogue.swift:10-100)
+class FusedQKVEpilogue {
+public:
+    explicit FusedQKVEpilogue(const Context &context) : c_(context) {}
+    void encode(void *q, uint64_t qOffset, void *k, uint64_t kOffset, void *v, uint64_t vOffset, const void *qWeight, uint64_t qWeightOffset,
+                const void *kWeight, uint64_t kWeightOffset, uint32_t headDim, uint32_t numQHeads, uint32_t numKVHeads, uint32_t position,
+                float theta, uint32_t rotatedPairs, float eps) const {
+        c_.check(tf_fused_qkv_epilogue(c_.raw(), c_.stream(), q, qOffset, k, kOffset, v, vOffset, qWeight, qWeightOffset, kWeight, kWeightOffset,
+                                       headDim, numQHeads, numKVHeads, position, theta, rotatedPairs, eps));
+    }
+
+private:
+    const Context &c_;
+};
+
 // Attention (Kernels/Attention/Attention.swift:26-214): sliding-window and full-causal decode attention
 using AttentionSplitGeometry = tf_attention_split_geometry_t;
 class Attention {
