@@ -233,6 +233,7 @@ def main():
     if not args.no_extras:
         out["extras"] = extras(torch, tfk, k, gen, lib, h, stream)
         out["extras"].update(multi_token_extras(torch, tfk, k, gen, lib, h, stream, layers[0], offs, stride))
+        out["extras"].update(layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride))
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, layers, hidden, idx, wts, y, offs, stride, payload, args)
@@ -367,6 +368,89 @@ def extras(torch, tfk, k, gen, lib, h, stream):
     res["shared_expert_int4"] = {"us_per_call": round(us, 3), "GBps": round(SHARED_BYTES / (us * 1e-6) / 1e9, 1),
                                  "algorithmic_bytes": SHARED_BYTES}
     return res
+
+
+def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride):
+    """One token through whole sliding-window decoder layers, every stage a call of the library and nothing on the host in
+    between: input norm -> q/k/v projections (k, v straight into their cache row) -> per-head norm + RoPE -> attention over a
+    1024-row window -> output projection -> post-attention setup -> shared expert + norm, router + 8 routed experts -> layer
+    tail.  The layers rotate over the resident expert pools and as many sets of dense weights; replayed from a HIP graph."""
+    import ctypes as C
+    HD, NQ, NKV, WINDOW = 256, 16, 8, 1024
+    n_layers = len(layers)
+    off = tfk.ExpertOffsets(*offs)
+    dense = []
+    for _ in range(n_layers):
+        w = {name: make_int4(torch, gen, rows, cols) for name, rows, cols in (("q", NQ * HD, D), ("k", NKV * HD, D), ("v", NKV * HD, D), ("o", D, NQ * HD),
+                                                                              ("gate", F_SHARED, D), ("up", F_SHARED, D), ("down", D, F_SHARED))}
+        for name, n in (("input_norm", D), ("post_attn", D), ("pre_ffn", D), ("pre_ffn2", D), ("post_ffn1", D), ("post_ffn2", D), ("post_ffn", D),
+                        ("q_norm", HD), ("k_norm", HD)):
+            w[name] = bf16_bits_cuda(torch.rand(n, device="cuda", generator=gen) * 0.2 + 0.9)
+        w["k_cache"] = torch.randn((WINDOW + 128, NKV, HD), device="cuda", generator=gen).to(torch.float16)
+        w["v_cache"] = torch.randn((WINDOW + 128, NKV, HD), device="cuda", generator=gen).to(torch.float16)
+        w["proj"] = [tfk.projection(*w[n], r, c) for n, r, c in (("gate", F_SHARED, D), ("up", F_SHARED, D), ("down", D, F_SHARED))]
+        dense.append(w)
+    z = lambda n: torch.zeros(n, dtype=torch.float16, device="cuda")
+    b = dict(hidden=(torch.randn(D, device="cuda", generator=gen) * 0.5).to(torch.float16), x_norm=z(D), q=z(NQ * HD), attn=z(NQ * HD), o=z(D),
+             dense_x=z(D), routed_x=z(D), router_x=z(D), shared=z(D), h1=z(D), h2=z(D), sg=z(F_SHARED), su=z(F_SHARED), sa=z(F_SHARED), zero=z(D),
+             acts=z(TOPK * F_MOE), idx=torch.zeros(TOPK, dtype=torch.int32, device="cuda"), wts=z(TOPK))
+    p = lambda name: b[name].data_ptr()
+    position = WINDOW + 60
+    kv_off = position * NKV * HD * 2
+
+    def layer_step(i, st):
+        w, (pool, r) = dense[i % n_layers], layers[i % n_layers]
+        ptr = lambda name: w[name].data_ptr()
+        rc = lib.tf_rmsnorm_bf16w(h, st, p("hidden"), 0, ptr("input_norm"), 0, p("x_norm"), 0, D, 1e-6)
+        qkv = []
+        for name in ("q", "k", "v"):
+            qkv += [w[name][0].data_ptr(), 0, w[name][1].data_ptr(), 0, w[name][2].data_ptr(), 0]
+        rc |= lib.tf_fused_qkv_gemv(h, st, *qkv, p("x_norm"), p("q"), 0, ptr("k_cache"), kv_off, ptr("v_cache"), kv_off, NQ * HD, NKV * HD, D, tfk.TF_BF16)
+        rc |= lib.tf_fused_qkv_epilogue(h, st, p("q"), 0, ptr("k_cache"), kv_off, ptr("v_cache"), kv_off, ptr("q_norm"), 0, ptr("k_norm"), 0,
+                                        HD, NQ, NKV, position, 1e4, HD // 2, 1e-6)
+        rc |= lib.tf_attention_swa(h, st, p("q"), 0, ptr("k_cache"), 0, ptr("v_cache"), 0, p("attn"), 0, HD, NQ, NKV, position + 1, WINDOW, 1.0, 0)
+        rc |= lib.tf_dequant_int4_gemv(h, st, w["o"][0].data_ptr(), 0, w["o"][1].data_ptr(), 0, w["o"][2].data_ptr(), 0, p("attn"), 0, p("o"), 0,
+                                       D, NQ * HD, tfk.TF_BF16, tfk.TF_FP16)
+        rc |= lib.tf_fused_post_attn_setup(h, st, p("hidden"), p("o"), p("dense_x"), p("routed_x"), p("router_x"), ptr("post_attn"), 0,
+                                           ptr("pre_ffn"), 0, ptr("pre_ffn2"), 0, D, 1e-6)
+        g, u, dn = w["proj"]
+        rc |= lib.tf_shared_expert_int4(h, st, p("dense_x"), 0, D * 2, C.byref(g), C.byref(u), C.byref(dn), p("shared"), 0, D * 2, p("sg"), 0,
+                                        F_SHARED * 2, p("su"), 0, F_SHARED * 2, p("sa"), 0, F_SHARED * 2, 4, tfk.TF_BF16)
+        rc |= lib.tf_rmsnorm_bf16w(h, st, p("shared"), 0, ptr("post_ffn1"), 0, p("h1"), 0, D, 1e-6)
+        rc |= lib.tf_moe_decode_step(h, st, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, p("router_x"), r["eff"].data_ptr(), 0,
+                                     r["gain"].data_ptr(), 0, pool.data_ptr(), stride, E, C.byref(off), p("routed_x"), p("acts"), p("zero"), p("h2"),
+                                     p("idx"), p("wts"), D, F_MOE, TOPK, tfk.TF_BF16)
+        rc |= lib.tf_fused_layer_tail(h, st, p("h2"), p("h1"), p("hidden"), ptr("post_ffn2"), 0, ptr("post_ffn"), 0, D, 1e-6, 1.0)
+        if rc != 0:
+            raise RuntimeError("layer chain failed: " + k.last_error())
+
+    per_graph = 30                                          # the model has 30 layers: one replay = one token's layers
+    st0 = torch.cuda.current_stream().cuda_stream
+    for i in range(2 * n_layers):
+        layer_step(i, st0)                                  # warm-up; also sizes every context-owned scratch before the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            st = torch.cuda.current_stream().cuda_stream
+            for i in range(per_graph):
+                layer_step(i, st)
+        g.replay()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        replays = 20
+        for _ in range(replays):
+            g.replay()
+        torch.cuda.synchronize()
+        us = (time.perf_counter() - t0) * 1e6 / (replays * per_graph)
+    assert bool(torch.isfinite(b["hidden"].float()).all()), "the residual stream left the finite range"
+    layer_bytes = (int4_matrix_bytes(NQ * HD + 2 * NKV * HD, D) + int4_matrix_bytes(D, NQ * HD) + SHARED_BYTES + STEP_BYTES
+                   + 2 * WINDOW * NKV * HD * 2)
+    return {"decode_layer_sliding_window": {
+        "workload": "one token through one whole decoder layer (16q/8kv x 256, window 1024, shared 2112, 8 of 128 experts), 30 layers per graph replay",
+        "us_per_layer": round(us, 2), "ms_per_30_layers": round(us * 30 / 1e3, 3), "algorithmic_bytes_per_layer": layer_bytes,
+        "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 17}}
 
 
 def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride):

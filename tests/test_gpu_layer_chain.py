@@ -1,0 +1,167 @@
+"""One decode step of a whole sliding-window decoder layer, enqueued through the C ABI with no host step in between, at the
+production widths (d 2816, 16 query heads on 8 kv heads of 256, shared expert 2112, routed experts 704 wide; 16 experts to
+keep the CPU side short).  Every stage reads what the previous stage left on the device, K and V land in their cache row
+through offsets.  Each stage's output is checked against the oracle applied to that stage's own device inputs, so a
+near-tie that tips differently upstream cannot hide or fake a defect downstream; when both sides pick the same experts the
+end result is also compared with the oracle's chain run from the start."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import refcases
+import test_gpu_moe as M
+from gpu_helpers import ctx, dev, host, tfk, zeros_bytes
+from oracle import tfo
+
+pytestmark = pytest.mark.gpu
+
+D, HD, NQ, NKV = 2816, 256, 16, 8
+F_SHARED, F_MOE, E = 2112, 704, 16
+WINDOW, THETA, EPS, PAIRS, ATTN_SCALE, LAYER_SCALAR = 1024, 1e4, 1e-6, HD // 2, 1.0, 0.75
+TOL = tfo.Tolerance.fp16ChainedReduction
+
+
+def gemv(wsb, x_bits):
+    """The GEMV kernels' arithmetic on the CPU, rounded to fp16 as they store it."""
+    return tfo.to_f16_bits(tfo.k_int4_gemv(*wsb, x_bits))
+
+
+def norm_weight(seed):
+    return tfo.bf16_bits_array(1.0 + 0.1 * np.random.default_rng(seed).standard_normal(D).astype(np.float32))
+
+
+def build_layer(seed):
+    L = dict(q=refcases.synthetic_int4(NQ * HD, D, seed, "q"), k=refcases.synthetic_int4(NKV * HD, D, seed, "k"),
+             v=refcases.synthetic_int4(NKV * HD, D, seed, "v"), o=refcases.synthetic_int4(D, NQ * HD, seed, "o"),
+             gate=refcases.synthetic_int4(F_SHARED, D, seed, "sg"), up=refcases.synthetic_int4(F_SHARED, D, seed, "su"),
+             down=refcases.synthetic_int4(D, F_SHARED, seed, "sd"))
+    for i, name in enumerate(("input_norm", "post_attn", "pre_ffn", "pre_ffn2", "post_ffn1", "post_ffn2", "post_ffn")):
+        L[name] = norm_weight(seed * 31 + i)
+    rng = np.random.default_rng(seed + 5)
+    L["q_norm"] = tfo.bf16_bits_array(1.0 + 0.1 * rng.standard_normal(HD).astype(np.float32))
+    L["k_norm"] = tfo.bf16_bits_array(1.0 + 0.1 * rng.standard_normal(HD).astype(np.float32))
+    L["moe"] = M._decode_step_case(D, F_MOE, E, seed + 11)
+    return L
+
+
+def test_decode_step_of_a_sliding_window_layer():
+    L = build_layer(0x1A7E)
+    position = 37                                            # rows 0..36 of the cache are history
+    rng = np.random.default_rng(3)
+    hidden0 = (rng.standard_normal(D) * 0.5).astype(np.float32).astype(np.float16).view(np.uint16)
+    cache_rows = 64
+    k_cache0 = (rng.uniform(-1, 1, cache_rows * NKV * HD)).astype(np.float32).astype(np.float16).view(np.uint16)
+    v_cache0 = (rng.uniform(-1, 1, cache_rows * NKV * HD)).astype(np.float32).astype(np.float16).view(np.uint16)
+    k = ctx()
+    lib, h = k.lib, k.handle
+    t = {name: [dev(a) for a in L[name]] for name in ("q", "k", "v", "o", "gate", "up", "down")}
+    w = {name: dev(L[name]) for name in ("input_norm", "post_attn", "pre_ffn", "pre_ffn2", "post_ffn1", "post_ffn2", "post_ffn", "q_norm", "k_norm")}
+    mt = M._decode_step_tensors(L["moe"])
+    b = dict(hidden=dev(hidden0), x_norm=zeros_bytes(D * 2), q=zeros_bytes(NQ * HD * 2), k_cache=dev(k_cache0), v_cache=dev(v_cache0),
+             attn=zeros_bytes(NQ * HD * 2), o=zeros_bytes(D * 2), dense_x=zeros_bytes(D * 2), routed_x=zeros_bytes(D * 2),
+             router_x=zeros_bytes(D * 2), shared=zeros_bytes(D * 2), h1=zeros_bytes(D * 2), h2=zeros_bytes(D * 2),
+             sg=zeros_bytes(F_SHARED * 2), su=zeros_bytes(F_SHARED * 2), sa=zeros_bytes(F_SHARED * 2), zero=zeros_bytes(D * 2),
+             idx=zeros_bytes(32), wts=zeros_bytes(16), acts=zeros_bytes(8 * F_MOE * 2))
+    row_bytes = NKV * HD * 2
+    kv_off = position * row_bytes                             # the new K and V rows are written straight into the cache
+    p = lambda name: b[name].data_ptr()
+    snap = {}
+
+    def grab(*names):
+        for n in names:
+            snap[n] = host(b[n], np.uint16).copy()
+
+    # 1. input norm, q / k / v projections in one launch, per-head norm + RoPE in place (k, v inside the cache)
+    k.check(lib.tf_rmsnorm_bf16w(h, None, p("hidden"), 0, w["input_norm"].data_ptr(), 0, p("x_norm"), 0, D, EPS))
+    qkv = []
+    for name in ("q", "k", "v"):
+        qkv += [t[name][0].data_ptr(), 0, t[name][1].data_ptr(), 0, t[name][2].data_ptr(), 0]
+    k.check(lib.tf_fused_qkv_gemv(h, None, *qkv, p("x_norm"), p("q"), 0, p("k_cache"), kv_off, p("v_cache"), kv_off, NQ * HD, NKV * HD, D, tfk.TF_BF16))
+    grab("x_norm", "q", "k_cache", "v_cache")
+    raw_q, raw_k, raw_v = snap["q"].copy(), snap["k_cache"].copy(), snap["v_cache"].copy()
+    k.check(lib.tf_fused_qkv_epilogue(h, None, p("q"), 0, p("k_cache"), kv_off, p("v_cache"), kv_off, w["q_norm"].data_ptr(), 0,
+                                      w["k_norm"].data_ptr(), 0, HD, NQ, NKV, position, THETA, PAIRS, EPS))
+    grab("q", "k_cache", "v_cache")
+    # 2. attention over rows [0, position], output projection
+    seq_len = position + 1
+    k.check(lib.tf_attention_swa(h, None, p("q"), 0, p("k_cache"), 0, p("v_cache"), 0, p("attn"), 0, HD, NQ, NKV, seq_len, WINDOW, ATTN_SCALE, 0))
+    k.check(lib.tf_dequant_int4_gemv(h, None, t["o"][0].data_ptr(), 0, t["o"][1].data_ptr(), 0, t["o"][2].data_ptr(), 0, p("attn"), 0, p("o"), 0,
+                                     D, NQ * HD, tfk.TF_BF16, tfk.TF_FP16))
+    grab("attn", "o")
+    hidden_before_setup = host(b["hidden"], np.uint16).copy()
+    # 3. residual + the three inputs of the FFN sandwich
+    k.check(lib.tf_fused_post_attn_setup(h, None, p("hidden"), p("o"), p("dense_x"), p("routed_x"), p("router_x"), w["post_attn"].data_ptr(), 0,
+                                         w["pre_ffn"].data_ptr(), 0, w["pre_ffn2"].data_ptr(), 0, D, EPS))
+    grab("hidden", "dense_x", "routed_x", "router_x")
+    hidden_after_setup = snap["hidden"].copy()
+    # 4. shared expert + its output norm; routed experts (router, gate/up, down) on the resident pool
+    gate, up, down = (tfk.projection(*t[n], r, c) for n, r, c in (("gate", F_SHARED, D), ("up", F_SHARED, D), ("down", D, F_SHARED)))
+    k.shared_expert_int4(b["dense_x"], gate, up, down, b["shared"], b["sg"], b["su"], b["sa"])
+    k.check(lib.tf_rmsnorm_bf16w(h, None, p("shared"), 0, w["post_ffn1"].data_ptr(), 0, p("h1"), 0, D, EPS))
+    off = tfk.ExpertOffsets(*L["moe"]["off"].as_tuple())
+    k.check(lib.tf_moe_decode_step(h, None, mt["rW"].data_ptr(), 0, mt["rS"].data_ptr(), 0, mt["rB"].data_ptr(), 0, p("router_x"),
+                                   mt["eff"].data_ptr(), 0, mt["gain"].data_ptr(), 0, mt["pool"].data_ptr(), L["moe"]["stride"], E, off,
+                                   p("routed_x"), p("acts"), p("zero"), p("h2"), p("idx"), p("wts"), D, F_MOE, 8, tfk.TF_BF16))
+    grab("shared", "h1", "h2", "acts")
+    idx, wts = host(b["idx"], np.uint32, 8), host(b["wts"], np.uint16, 8)
+    # 5. both branches folded back into the residual stream
+    k.check(lib.tf_fused_layer_tail(h, None, p("h2"), p("h1"), p("hidden"), w["post_ffn2"].data_ptr(), 0, w["post_ffn"].data_ptr(), 0, D, EPS, LAYER_SCALAR))
+    hidden_out = host(b["hidden"], np.uint16)
+
+    f = tfo.from_f16_bits
+    close = lambda got, want, tol=TOL: tfo.rel_error(f(got), f(want)) < tol
+    # ---- stage by stage, each against the oracle on the device's own inputs
+    assert close(snap["x_norm"], tfo.k_rmsnorm_bf16w(hidden0, L["input_norm"], EPS))
+    assert close(raw_q, gemv(L["q"], snap["x_norm"]))
+    new_row = slice(position * NKV * HD, (position + 1) * NKV * HD)
+    assert close(raw_k[new_row], gemv(L["k"], snap["x_norm"]))
+    assert close(raw_v[new_row], gemv(L["v"], snap["x_norm"]))
+    untouched = np.ones(cache_rows * NKV * HD, bool)
+    untouched[new_row] = False
+    assert np.array_equal(snap["k_cache"][untouched], k_cache0[untouched]) and np.array_equal(snap["v_cache"][untouched], v_cache0[untouched])
+    eq, ek, ev = tfo.k_fused_qkv_epilogue(raw_q, raw_k[new_row], raw_v[new_row], L["q_norm"], L["k_norm"], HD, NQ, NKV, position, THETA, PAIRS, EPS)
+    assert close(snap["q"], eq) and close(snap["k_cache"][new_row], ek) and close(snap["v_cache"][new_row], ev)
+    rows = seq_len * NKV * HD
+    attn_ref = tfo.attention_ref(f(snap["q"]), f(snap["k_cache"][:rows]), f(snap["v_cache"][:rows]), HD, NQ, NKV, seq_len, WINDOW, ATTN_SCALE)
+    assert tfo.rel_error(f(snap["attn"]), attn_ref) < TOL
+    assert close(snap["o"], gemv(L["o"], snap["attn"]))
+    want_hidden, want_dense, want_routed, want_router = tfo.k_post_attn_setup(hidden_before_setup, snap["o"], L["post_attn"], L["pre_ffn"], L["pre_ffn2"], EPS)
+    for got, want in ((hidden_after_setup, want_hidden), (snap["dense_x"], want_dense), (snap["routed_x"], want_routed), (snap["router_x"], want_router)):
+        assert close(got, want, tfo.Tolerance.fp16Reduction)
+    shared_ref = tfo.shared_expert_ref(L["gate"], L["up"], L["down"], f(snap["dense_x"]), threads=8)
+    assert tfo.rel_error(f(snap["shared"]), shared_ref) < 6e-3
+    assert close(snap["h1"], tfo.k_rmsnorm_bf16w(snap["shared"], L["post_ffn1"], EPS))
+    mo = L["moe"]
+    logits = tfo.k_router_logits(mo["rW"], mo["rS"], mo["rB"], snap["router_x"], mo["eff_bits"])
+    want_idx, want_wts = tfo.k_router_topk(logits, mo["gain_bits"])
+    assert np.array_equal(idx, want_idx)
+    assert np.max(np.abs(f(wts) - f(want_wts))) < 5e-3
+    blobs = [mo["blobs"][int(e)] for e in idx]
+    want_acts = tfo.k_moe_phase1(blobs, mo["off"], snap["routed_x"], D, F_MOE)
+    assert close(snap["acts"], want_acts)
+    assert close(snap["h2"], tfo.k_moe_phase2(blobs, mo["off"], snap["acts"], wts, np.zeros(D, np.uint16), D, F_MOE))
+    assert close(hidden_out, tfo.k_layer_tail(snap["h2"], snap["h1"], hidden_after_setup, L["post_ffn2"], L["post_ffn"], EPS, LAYER_SCALAR),
+                 tfo.Tolerance.fp16Reduction)
+
+    # ---- the oracle's own chain from the start; comparable end to end when it picks the same experts
+    x_norm = tfo.k_rmsnorm_bf16w(hidden0, L["input_norm"], EPS)
+    oq, ok, ov = (gemv(L[n], x_norm) for n in ("q", "k", "v"))
+    oq, ok, ov = tfo.k_fused_qkv_epilogue(oq, ok, ov, L["q_norm"], L["k_norm"], HD, NQ, NKV, position, THETA, PAIRS, EPS)
+    kc, vc = k_cache0.copy(), v_cache0.copy()
+    kc[new_row], vc[new_row] = ok, ov
+    geo = tfo.attention_split_geometry(NQ, NKV, seq_len, 0, True)
+    oattn = tfo.k_attention_split(oq, kc, vc, HD, NQ, NKV, seq_len, 0, geo["chunkLength"], geo["numChunks"], ATTN_SCALE)
+    oo = gemv(L["o"], oattn)
+    ohid, odense, orouted, orouter = tfo.k_post_attn_setup(hidden0, oo, L["post_attn"], L["pre_ffn"], L["pre_ffn2"], EPS)
+    og = gemv(L["gate"], odense)
+    ou = gemv(L["up"], odense)
+    oshared = gemv(L["down"], tfo.k_gelu_mul_fp16(og, ou))
+    oh1 = tfo.k_rmsnorm_bf16w(oshared, L["post_ffn1"], EPS)
+    oidx, owts = tfo.k_router_topk(tfo.k_router_logits(mo["rW"], mo["rS"], mo["rB"], orouter, mo["eff_bits"]), mo["gain_bits"])
+    if np.array_equal(oidx, idx):
+        oblobs = [mo["blobs"][int(e)] for e in oidx]
+        oacts = tfo.k_moe_phase1(oblobs, mo["off"], orouted, D, F_MOE)
+        oh2 = tfo.k_moe_phase2(oblobs, mo["off"], oacts, owts, np.zeros(D, np.uint16), D, F_MOE)
+        ofinal = tfo.k_layer_tail(oh2, oh1, ohid, L["post_ffn2"], L["post_ffn"], EPS, LAYER_SCALAR)
+        assert tfo.rel_error(f(hidden_out), f(ofinal)) < 2 * TOL
