@@ -282,6 +282,25 @@ int32_t tf_fused_qkv_epilogue(tf_ctx *ctx, tf_stream stream, void *q, uint64_t q
                               const void *k_weight, uint64_t k_weight_offset, uint32_t head_dim, uint32_t num_q_heads,
                               uint32_t num_kv_heads, uint32_t position, float theta, uint32_t rotated_pairs, float eps);
 
+/* PrefillAttentionParams (Kernels/Attention/PrefillAttention.swift:4-40; Metal/Prefill/prefill.metal:775-788): 44 bytes. */
+typedef struct tf_prefill_attention_params {
+    uint32_t start_position, query_count, head_dim, num_q_heads, num_kv_heads, kv_valid_count, sliding_window;
+    uint32_t kv_token_stride_elements, q_token_stride_elements, o_token_stride_elements;
+    float scale;
+} tf_prefill_attention_params;
+/* PrefillAttention.encodeCausal (PrefillAttention.swift:56-118) -> attention_prefill_causal_tiled (prefill.metal:835-902):
+ * query t of the block (row t of q, stride q_token_stride_elements) sits at position start_position + t and attends to
+ * the keys [first, last): first = position + 1 - sliding_window when a window is set and exceeded, else 0;
+ * last = min(kv_valid_count, position + 1).  k, v rows at kv_token_stride_elements (row p % kv_ring_capacity when a
+ * ring is given); out row t at o_token_stride_elements; query head h reads kv head h / (num_q_heads / num_kv_heads);
+ * a query that sees no key gets zeros; bytes between rows are untouched.  Preconditions as PrefillAttention.validate
+ * (:120-136) -> TF_ERR_INVALID_ARGUMENT.  The reference's choice between its tiled and tensor-op pipelines (`path`) has
+ * no counterpart: 16-byte aligned rows with head_dim in {64,128,256,512} run on the matrix cores, everything else on a
+ * kernel of the reference's own shape. */
+int32_t tf_prefill_attention_causal(tf_ctx *ctx, tf_stream stream, const void *q, uint64_t q_offset, const void *k,
+                                    uint64_t k_offset, const void *v, uint64_t v_offset, void *out, uint64_t out_offset,
+                                    const tf_prefill_attention_params *params, uint32_t kv_ring_capacity);
+
 /* AttentionSplitGeometry / Attention.splitGeometry (Attention.swift:5-11,128-147): the reference's own dispatch shape for
  * a range, kept for callers that report it; pure host function, no context. */
 typedef struct tf_attention_split_geometry_t {

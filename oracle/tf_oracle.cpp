@@ -1096,6 +1096,81 @@ void tfo_attention_split_geometry(uint32_t num_q_heads, uint32_t num_kv_heads, u
     out5[4] = grouped ? 1 : 0;
 }
 
+// ---------------------------------------------------------------------------------------------------- attention (prefill)
+// T/Core/Kernels/Attention/PrefillAttentionTests.swift:310-352 (reference): query t of the block sits at position
+// start + t and sees keys [first, last) with first = max(0, start + t + 1 - window) (window 0: none) and
+// last = min(kv_valid, start + t + 1).  q [chunk, q_stride], k / v [rows, kv_stride], out compact [chunk, q_heads, head_dim].
+// Accumulation in double.
+void tfo_prefill_attention_ref(const float *q, const float *k, const float *v, int start, int chunk, int head_dim, int q_heads, int kv_heads,
+                               int kv_valid, int window, int q_stride, int kv_stride, float scale, float *out) {
+    const int q_per_kv = q_heads / kv_heads;
+    std::vector<double> w;
+    for (int t = 0; t < chunk; ++t) {
+        const int abs_q = start + t;
+        const int first = window == 0 ? 0 : std::max(0, abs_q + 1 - window);
+        const int last = std::min(kv_valid, abs_q + 1);
+        for (int qh = 0; qh < q_heads; ++qh) {
+            const int kvh = qh / q_per_kv;
+            w.assign((size_t)std::max(0, last - first), 0.0);
+            double mx = -INFINITY;
+            for (int key = first; key < last; ++key) {
+                double sc = 0.0;
+                for (int d = 0; d < head_dim; ++d)
+                    sc += (double)q[(size_t)t * q_stride + (size_t)qh * head_dim + d] * (double)k[(size_t)key * kv_stride + (size_t)kvh * head_dim + d];
+                w[(size_t)(key - first)] = sc * (double)scale;
+                mx = std::max(mx, sc * (double)scale);
+            }
+            double denom = 0.0;
+            for (double &x : w) {
+                x = std::exp(x - mx);
+                denom += x;
+            }
+            for (int d = 0; d < head_dim; ++d) {
+                double acc = 0.0;
+                for (int key = first; key < last; ++key) acc += w[(size_t)(key - first)] * (double)v[(size_t)key * kv_stride + (size_t)kvh * head_dim + d];
+                out[((size_t)t * q_heads + qh) * head_dim + d] = denom > 0.0 ? (float)(acc / denom) : 0.0f;
+            }
+        }
+    }
+}
+
+// Kernel-order restatement of attention_prefill_causal_tiled (M/Prefill/prefill.metal:835-902): fp16 operands, one online
+// softmax per (query, head) in fp32, key by key, fp16 result into out [chunk, o_stride]; ring_capacity != 0: key p lives in
+// row p % ring_capacity.  Elements of out between rows are left as they are.
+void tfo_k_prefill_attention(const uint16_t *q_f16, const uint16_t *k_f16, const uint16_t *v_f16, uint16_t *out_f16, int start, int chunk,
+                             int head_dim, int q_heads, int kv_heads, int kv_valid, int window, int q_stride, int kv_stride, int o_stride,
+                             float scale, int ring_capacity) {
+    const int q_per_kv = q_heads / kv_heads;
+    std::vector<float> acc((size_t)head_dim);
+    for (int t = 0; t < chunk; ++t) {
+        const int abs_q = start + t;
+        const int first = (window != 0 && abs_q + 1 > window) ? abs_q + 1 - window : 0;
+        const int last = std::min(kv_valid, abs_q + 1);
+        for (int qh = 0; qh < q_heads; ++qh) {
+            const int kvh = qh / q_per_kv;
+            const uint16_t *qr = q_f16 + (size_t)t * q_stride + (size_t)qh * head_dim;
+            float row_max = -INFINITY, row_sum = 0.0f;
+            std::fill(acc.begin(), acc.end(), 0.0f);
+            for (int key = first; key < last; ++key) {
+                const int row = ring_capacity ? key % ring_capacity : key;
+                const uint16_t *kr = k_f16 + (size_t)row * kv_stride + (size_t)kvh * head_dim;
+                const uint16_t *vr = v_f16 + (size_t)row * kv_stride + (size_t)kvh * head_dim;
+                float sc = 0.0f;
+                for (int d = 0; d < head_dim; ++d) sc += tfo_f16_to_float(qr[d]) * tfo_f16_to_float(kr[d]);
+                sc *= scale;
+                const float new_max = std::max(row_max, sc);
+                const float old_scale = row_sum > 0.0f ? std::exp(row_max - new_max) : 0.0f;
+                const float new_scale = std::exp(sc - new_max);
+                for (int d = 0; d < head_dim; ++d) acc[(size_t)d] = std::fma(new_scale, tfo_f16_to_float(vr[d]), acc[(size_t)d] * old_scale);
+                row_sum = row_sum * old_scale + new_scale;
+                row_max = new_max;
+            }
+            uint16_t *orow = out_f16 + (size_t)t * o_stride + (size_t)qh * head_dim;
+            for (int d = 0; d < head_dim; ++d) orow[d] = tfo_f16_bits(row_sum > 0.0f ? acc[(size_t)d] / row_sum : 0.0f);
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------- RoPE, QKV epilogue
 // V/Support/Reference/Attention/RoPE.swift:82-128 (RopeRef.applyNeox): pairs (x[i], x[i + head_dim / 2]) for
 // i < rotated_pairs rotate by angle position * theta^(-2 i / head_dim); everything else passes through.  fp32 in / out;

@@ -206,6 +206,13 @@ void tfo_k_attention_split(const uint16_t *q_f16, const uint16_t *k_f16, const u
 void tfo_attention_split_geometry(uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len, uint32_t kv_start, int prefer_gqa_swa,
                                   int32_t *out5);
 
+/* causal attention of a block of query tokens (prefill): the test-embedded reference and the kernel-order path */
+void tfo_prefill_attention_ref(const float *q, const float *k, const float *v, int start, int chunk, int head_dim, int q_heads, int kv_heads,
+                               int kv_valid, int window, int q_stride, int kv_stride, float scale, float *out);
+void tfo_k_prefill_attention(const uint16_t *q_f16, const uint16_t *k_f16, const uint16_t *v_f16, uint16_t *out_f16, int start, int chunk,
+                             int head_dim, int q_heads, int kv_heads, int kv_valid, int window, int q_stride, int kv_stride, int o_stride,
+                             float scale, int ring_capacity);
+
 /* RoPE (NeoX pairs) and the fused per-head Q/K/V epilogue */
 void tfo_rope_neox_ref(const float *input, int num_tokens, int num_heads, int head_dim, int rotated_pairs, int position, float theta,
                        float *out);

@@ -659,3 +659,23 @@ def k_fused_qkv_epilogue(q_bits, k_bits, v_bits, q_weight_bits, k_weight_bits, h
     lib.tfo_k_fused_qkv_epilogue(q, k, v, _u16(q_weight_bits), _u16(k_weight_bits), head_dim, num_q_heads, num_kv_heads, position,
                                  float(theta), rotated_pairs, float(eps))
     return q, k, v
+
+
+# ---- causal attention of a block of query tokens (prefill) ------------------------------------
+_sig("tfo_prefill_attention_ref", None, f32p, f32p, f32p, i32, i32, i32, i32, i32, i32, i32, i32, i32, C.c_float, f32p)
+_sig("tfo_k_prefill_attention", None, u16p, u16p, u16p, u16p, i32, i32, i32, i32, i32, i32, i32, i32, i32, i32, C.c_float, i32)
+
+
+def prefill_attention_ref(q, k, v, start, chunk, head_dim, q_heads, kv_heads, kv_valid, window, q_stride, kv_stride, scale) -> np.ndarray:
+    out = np.empty(chunk * q_heads * head_dim, np.float32)
+    lib.tfo_prefill_attention_ref(_flat32(q), _flat32(k), _flat32(v), start, chunk, head_dim, q_heads, kv_heads, kv_valid, window, q_stride,
+                                  kv_stride, float(scale), out)
+    return out
+
+
+def k_prefill_attention(q_bits, k_bits, v_bits, out_bits, start, chunk, head_dim, q_heads, kv_heads, kv_valid, window, q_stride, kv_stride,
+                        o_stride, scale, ring_capacity=0) -> np.ndarray:
+    out = _u16(out_bits).copy()
+    lib.tfo_k_prefill_attention(_u16(q_bits), _u16(k_bits), _u16(v_bits), out, start, chunk, head_dim, q_heads, kv_heads, kv_valid, window,
+                                q_stride, kv_stride, o_stride, float(scale), ring_capacity)
+    return out

@@ -45,6 +45,14 @@ class Projection(C.Structure):
                 ("biases", vp), ("biases_offset", u64), ("rows", u32), ("cols", u32)]
 
 
+class PrefillAttentionParams(C.Structure):
+    """PrefillAttentionParams (Kernels/Attention/PrefillAttention.swift:4-40)."""
+    _fields_ = [("start_position", C.c_uint32), ("query_count", C.c_uint32), ("head_dim", C.c_uint32), ("num_q_heads", C.c_uint32),
+                ("num_kv_heads", C.c_uint32), ("kv_valid_count", C.c_uint32), ("sliding_window", C.c_uint32),
+                ("kv_token_stride_elements", C.c_uint32), ("q_token_stride_elements", C.c_uint32), ("o_token_stride_elements", C.c_uint32),
+                ("scale", C.c_float)]
+
+
 class AttentionSplitGeometry(C.Structure):
     """AttentionSplitGeometry (Kernels/Attention/Attention.swift:5-11)."""
     _fields_ = [("effective_length", C.c_int32), ("num_chunks", C.c_int32), ("chunk_length", C.c_int32),
@@ -126,6 +134,7 @@ EXPORTS = {
     "tf_fused_qkv_epilogue": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, C.c_float, u32, C.c_float]),
     "tf_attention_swa": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, u32, C.c_float, u32]),
     "tf_attention_full": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, C.c_float]),
+    "tf_prefill_attention_causal": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, C.POINTER(PrefillAttentionParams), u32]),
     "tf_attention_split_geometry": (None, [u32, u32, u32, u32, i32, C.POINTER(AttentionSplitGeometry)]),
     "tf_router_gemma4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, vp, u64, vp, u64, vp, vp, u32, u32, u32]),
     "tf_moe_phase1_gate_up_act": (i32, [vp, vp, C.POINTER(RoutedBlobs), C.POINTER(ExpertOffsets), vp, vp, u32, u32, u32, i32]),

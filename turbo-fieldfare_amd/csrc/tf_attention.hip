@@ -300,6 +300,197 @@ __global__ __launch_bounds__(kAttnThreads) void attention_combine_kernel(const f
     if (wave == 0 && i < head_dim) out[(size_t)q_head * head_dim + i] = (half_t)(((sums[0][lane] + sums[1][lane]) + (sums[2][lane] + sums[3][lane])) * inv);
 }
 
+// ---- causal attention of a block of query tokens (prefill) ---------------------------------------------------------
+struct PrefillShape {
+    uint32_t start, count, num_q_heads, num_kv_heads, kv_valid, window, kv_stride, q_stride, o_stride, ring_capacity;
+    float scale;
+};
+
+__device__ __forceinline__ uint32_t prefill_row(const PrefillShape &s, uint32_t p) { return s.ring_capacity ? p % s.ring_capacity : p; }
+// keys query t sees: [first, last)
+__device__ __forceinline__ void visible_keys(const PrefillShape &s, uint32_t t, uint32_t &first, uint32_t &last) {
+    const uint32_t abs_q = s.start + t;
+    first = (s.window != 0u && abs_q + 1u > s.window) ? abs_q + 1u - s.window : 0u;
+    last = min(s.kv_valid, abs_q + 1u);
+}
+
+// Matrix-core path: a wave owns 16 (query, head) columns that share one kv head - with G query heads per kv head that is
+// 16 / G consecutive queries - and walks the keys any of them sees, 16 at a time, exactly as the decode kernel does for its
+// G columns; a key outside a column's causal range or window is masked for that column only.  The K and V rows of a
+// range are thus read once per 16 / G queries instead of once per query and head.  No split over keys: a block of queries
+// makes enough waves.  HD in {64, 128, 256, 512}, G in {1, 2, 4, 8, 16}, rows 16-byte aligned.
+template <int HD>
+__global__ __launch_bounds__(kAttnThreads, 1) void attention_prefill_kernel(const half_t *Q, const half_t *K, const half_t *V, half_t *O,
+                                                                            PrefillShape s, uint32_t group_shift, uint32_t tiles_per_kv_head) {
+    constexpr int KS = HD / 32, LPR = HD / 8, R = 64 / LPR, VLOADS = kTilePositions / R;
+    __shared__ __align__(16) half_t p_tile[kAttnWaves][kTilePositions][kTileHeads];
+    __shared__ float alpha_tile[kAttnWaves][kTileHeads];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t item = blockIdx.x * kAttnWaves + (uint32_t)wave;
+    if (item >= tiles_per_kv_head * s.num_kv_heads) return;   // whole waves leave; the kernel has no block-wide barrier
+    const uint32_t kv_head = item / tiles_per_kv_head, col_tile = item % tiles_per_kv_head;
+    const uint32_t group = 1u << group_shift, pairs = s.count << group_shift;
+    const int col = lane & 15, quad = lane >> 4;
+    // this lane's column: pair index -> (query, head of the group)
+    const uint32_t pair = col_tile * kTileHeads + (uint32_t)col;
+    const bool col_live = pair < pairs;
+    const uint32_t t_col = col_live ? pair >> group_shift : 0u, g_col = pair & (group - 1u);
+    uint32_t first_col = 0u, last_col = 0u;
+    if (col_live) visible_keys(s, t_col, first_col, last_col);
+    // the keys any live column of the tile sees: columns ascend by query, so the first column starts first and the last
+    // live one ends last
+    const uint32_t t_lo = min((col_tile * kTileHeads) >> group_shift, s.count - 1u);
+    const uint32_t t_hi = min((col_tile * kTileHeads + kTileHeads - 1u) >> group_shift, s.count - 1u);
+    uint32_t p_lo, p_hi, unused;
+    visible_keys(s, t_lo, p_lo, unused);
+    visible_keys(s, t_hi, unused, p_hi);
+
+    half8_t qf[KS];
+#pragma unroll
+    for (int d = 0; d < KS; ++d) {
+        u32x4 raw = {0u, 0u, 0u, 0u};
+        if (col_live) raw = load16(Q + (size_t)t_col * s.q_stride + (size_t)(kv_head * group + g_col) * HD + 32 * d + 8 * quad);
+        qf[d] = __builtin_bit_cast(half8_t, raw);
+    }
+    float o[kTileHeads][8];
+#pragma unroll
+    for (int c = 0; c < kTileHeads; ++c)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[c][e] = 0.0f;
+    float m_run = -INFINITY, d_run = 0.0f;
+    const int vrow = lane / LPR, ve = lane % LPR;
+
+    for (uint32_t t0 = p_lo; t0 < p_hi; t0 += kTilePositions) {
+        const uint32_t pk = min(t0 + (uint32_t)col, p_hi - 1u);
+        const half_t *k_row = K + (size_t)prefill_row(s, pk) * s.kv_stride + (size_t)kv_head * HD + 8 * quad;
+        u32x4 kf[KS], vf[VLOADS];
+#pragma unroll
+        for (int d = 0; d < KS; ++d) kf[d] = load16(k_row + 32 * d);
+#pragma unroll
+        for (int j = 0; j < VLOADS; ++j) {
+            const uint32_t pv = min(t0 + (uint32_t)(j * R + vrow), p_hi - 1u);
+            vf[j] = load16(V + (size_t)prefill_row(s, pv) * s.kv_stride + (size_t)kv_head * HD + 8 * ve);
+        }
+        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int d = 0; d < KS; ++d) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, kf[d]), qf[d], acc, 0, 0, 0);
+        float sc[4], tile_max = -INFINITY;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const uint32_t p = t0 + (uint32_t)(4 * quad + r);
+            sc[r] = (p >= first_col && p < last_col) ? acc[r] * s.scale : -INFINITY;
+            tile_max = fmaxf(tile_max, sc[r]);
+        }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+        const float m_new = fmaxf(m_run, tile_max);      // stays -inf while the column has seen no key
+        const float alpha = exp_weight(m_run, m_new);
+        float sum = 0.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const float pe = exp_weight(sc[r], m_new);
+            p_tile[wave][4 * quad + r][col] = (half_t)pe;
+            sum += pe;
+        }
+        sum += __shfl_xor(sum, 16);
+        sum += __shfl_xor(sum, 32);
+        d_run = d_run * alpha + sum;
+        m_run = m_new;
+        if (quad == 0) alpha_tile[wave][col] = alpha;
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave reads back what its own lanes wrote
+#pragma unroll
+        for (int c = 0; c < kTileHeads; ++c) {
+            const float a = alpha_tile[wave][c];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) o[c][e] *= a;
+        }
+#pragma unroll
+        for (int j = 0; j < VLOADS; j += 2) {
+            const u32x4 ra = vf[j], rb = vf[j + 1];
+            uint32_t vv[8];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                vv[2 * w] = __builtin_amdgcn_perm(rb[w], ra[w], 0x05040100u);
+                vv[2 * w + 1] = __builtin_amdgcn_perm(rb[w], ra[w], 0x07060302u);
+            }
+            const u32x4 *pa = reinterpret_cast<const u32x4 *>(&p_tile[wave][j * R + vrow][0]);
+            const u32x4 *pb = reinterpret_cast<const u32x4 *>(&p_tile[wave][(j + 1) * R + vrow][0]);
+            const u32x4 pa0 = pa[0], pa1 = pa[1], pb0 = pb[0], pb1 = pb[1];
+#pragma unroll
+            for (int c = 0; c < kTileHeads; ++c) {
+                const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
+                const uint32_t wa = c < 8 ? pa0[(c >> 1) & 3] : pa1[(c >> 1) & 3], wb = c < 8 ? pb0[(c >> 1) & 3] : pb1[(c >> 1) & 3];
+                const half2_t pc = as_half2(__builtin_amdgcn_perm(wb, wa, sel));
+#pragma unroll
+                for (int e = 0; e < 8; ++e) o[c][e] = __builtin_amdgcn_fdot2(pc, as_half2(vv[e]), o[c][e], false);
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    }
+    // 1 / d of every column, then the rows: out[t, head, :] = o / d, zero where a column saw no key
+    if (quad == 0) alpha_tile[wave][col] = d_run > 0.0f ? 1.0f / d_run : 0.0f;
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+#pragma unroll
+    for (int c = 0; c < kTileHeads; ++c) {
+        const uint32_t pc = col_tile * kTileHeads + (uint32_t)c;
+        if (pc >= pairs) break;
+        const float inv = alpha_tile[wave][c];
+        u32x4 packed;
+#pragma unroll
+        for (int e = 0; e < 8; e += 2) {
+            float a = o[c][e], b = o[c][e + 1];
+            if constexpr (R >= 2) { a += __shfl_xor(a, 32); b += __shfl_xor(b, 32); }
+            if constexpr (R >= 4) { a += __shfl_xor(a, 16); b += __shfl_xor(b, 16); }
+            if constexpr (R >= 8) { a += __shfl_xor(a, 8); b += __shfl_xor(b, 8); }
+            const half2_t h = {(half_t)(a * inv), (half_t)(b * inv)};
+            packed[e >> 1] = as_u32(h);
+        }
+        if (vrow == 0) {
+            half_t *dst = O + (size_t)(pc >> group_shift) * s.o_stride + (size_t)(kv_head * group + (pc & (group - 1u))) * HD + 8 * ve;
+            *reinterpret_cast<u32x4 *>(dst) = packed;
+        }
+    }
+}
+
+// any shape and alignment: one block per (query, head), key by key (attention_prefill_causal_tiled, prefill.metal:835-902)
+__global__ __launch_bounds__(kAttnThreads) void attention_prefill_generic_kernel(const half_t *Q, const half_t *K, const half_t *V, half_t *O,
+                                                                                 uint32_t head_dim, PrefillShape s) {
+    __shared__ float part[kAttnWaves];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint32_t t = blockIdx.x, qh = blockIdx.y;
+    const uint32_t kvh = qh / (s.num_q_heads / s.num_kv_heads);
+    uint32_t first, last;
+    visible_keys(s, t, first, last);
+    const half_t *q_row = Q + (size_t)t * s.q_stride + (size_t)qh * head_dim;
+    float qv[(kMaxHeadDim + kAttnThreads - 1) / kAttnThreads], acc[(kMaxHeadDim + kAttnThreads - 1) / kAttnThreads] = {};
+    int slot = 0;
+    for (uint32_t i = threadIdx.x; i < head_dim; i += kAttnThreads, ++slot) qv[slot] = (float)q_row[i];
+    float row_max = -INFINITY, row_sum = 0.0f;
+    for (uint32_t key = first; key < last; ++key) {
+        const size_t row = (size_t)prefill_row(s, key) * s.kv_stride + (size_t)kvh * head_dim;
+        float partial = 0.0f;
+        slot = 0;
+        for (uint32_t i = threadIdx.x; i < head_dim; i += kAttnThreads, ++slot) partial = fmaf(qv[slot], (float)K[row + i], partial);
+        partial = wave_sum(partial);
+        __syncthreads();
+        if (lane == 0) part[wave] = partial;
+        __syncthreads();
+        float sc = 0.0f;
+#pragma unroll
+        for (int w = 0; w < kAttnWaves; ++w) sc += part[w];
+        sc *= s.scale;
+        const float new_max = fmaxf(row_max, sc);
+        const float old_scale = row_sum > 0.0f ? __expf(row_max - new_max) : 0.0f, new_scale = __expf(sc - new_max);
+        slot = 0;
+        for (uint32_t i = threadIdx.x; i < head_dim; i += kAttnThreads, ++slot) acc[slot] = fmaf(new_scale, (float)V[row + i], acc[slot] * old_scale);
+        row_sum = row_sum * old_scale + new_scale;
+        row_max = new_max;
+    }
+    half_t *out_row = O + (size_t)t * s.o_stride + (size_t)qh * head_dim;
+    slot = 0;
+    for (uint32_t i = threadIdx.x; i < head_dim; i += kAttnThreads, ++slot) out_row[i] = (half_t)(row_sum > 0.0f ? acc[slot] / row_sum : 0.0f);
+}
+
 // the context's partial-state scratch: m and d [heads x chunks], o [heads x chunks x head_dim]
 int32_t attention_scratch(tf_ctx *ctx, size_t floats, float *&out) {
     const size_t need = floats * sizeof(float);
@@ -412,6 +603,62 @@ int32_t tf_attention_full(tf_ctx *ctx, tf_stream stream, const void *q, uint64_t
     TF_REQUIRE(ctx, seq_len > 0, TF_ERR_INVALID_ARGUMENT, "attention_full: full attention requires at least one KV position");
     return attention_split(ctx, stream, q, q_offset, k, k_offset, v, v_offset, out, out_offset, head_dim, num_q_heads, num_kv_heads, seq_len, 0,
                            scale > 0.0f ? scale : default_scale(head_dim ? head_dim : 1), 0, "attention_full");
+}
+
+int32_t tf_prefill_attention_causal(tf_ctx *ctx, tf_stream stream, const void *q, uint64_t q_offset, const void *k, uint64_t k_offset,
+                                    const void *v, uint64_t v_offset, void *out, uint64_t out_offset, const tf_prefill_attention_params *p,
+                                    uint32_t kv_ring_capacity) {
+    TF_REQUIRE(ctx, ctx && q && k && v && out && p, TF_ERR_INVALID_ARGUMENT, "prefill_attention: null argument");
+    // PrefillAttention.validate (PrefillAttention.swift:120-136)
+    TF_REQUIRE(ctx, p->head_dim > 0, TF_ERR_INVALID_ARGUMENT, "headDim must be positive");
+    TF_REQUIRE(ctx, p->query_count > 0, TF_ERR_INVALID_ARGUMENT, "queryCount must be positive");
+    TF_REQUIRE(ctx, p->num_q_heads > 0, TF_ERR_INVALID_ARGUMENT, "numQHeads must be positive");
+    TF_REQUIRE(ctx, p->num_kv_heads > 0, TF_ERR_INVALID_ARGUMENT, "numKVHeads must be positive");
+    TF_REQUIRE(ctx, p->num_q_heads % p->num_kv_heads == 0, TF_ERR_INVALID_ARGUMENT, "numQHeads must be divisible by numKVHeads");
+    TF_REQUIRE(ctx, (uint64_t)p->q_token_stride_elements >= (uint64_t)p->num_q_heads * p->head_dim, TF_ERR_INVALID_ARGUMENT, "qTokenStrideElements too small");
+    TF_REQUIRE(ctx, (uint64_t)p->o_token_stride_elements >= (uint64_t)p->num_q_heads * p->head_dim, TF_ERR_INVALID_ARGUMENT, "oTokenStrideElements too small");
+    TF_REQUIRE(ctx, (uint64_t)p->kv_token_stride_elements >= (uint64_t)p->num_kv_heads * p->head_dim, TF_ERR_INVALID_ARGUMENT, "kvTokenStrideElements too small");
+    TF_REQUIRE(ctx, (uint64_t)p->start_position + p->query_count <= p->kv_valid_count, TF_ERR_INVALID_ARGUMENT,
+               "query block exceeds kvValidCount");
+    TF_REQUIRE(ctx, p->head_dim <= kMaxHeadDim, TF_ERR_INVALID_ARGUMENT, "prefill_attention: head_dim must be <= 512");
+    TF_REQUIRE(ctx, p->query_count <= 65535 && p->num_q_heads <= 65535, TF_ERR_INVALID_ARGUMENT, "prefill_attention: more than 65535 queries or heads");
+    TF_REQUIRE(ctx, q_offset % 2 == 0 && k_offset % 2 == 0 && v_offset % 2 == 0 && out_offset % 2 == 0, TF_ERR_INVALID_ARGUMENT,
+               "prefill_attention: offsets must be 2-byte aligned");
+    const half_t *qp = reinterpret_cast<const half_t *>(at(q, q_offset));
+    const half_t *kp = reinterpret_cast<const half_t *>(at(k, k_offset));
+    const half_t *vp = reinterpret_cast<const half_t *>(at(v, v_offset));
+    half_t *op = reinterpret_cast<half_t *>(at(out, out_offset));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    PrefillShape s;
+    s.start = p->start_position;
+    s.count = p->query_count;
+    s.num_q_heads = p->num_q_heads;
+    s.num_kv_heads = p->num_kv_heads;
+    s.kv_valid = p->kv_valid_count;
+    s.window = p->sliding_window;
+    s.kv_stride = p->kv_token_stride_elements;
+    s.q_stride = p->q_token_stride_elements;
+    s.o_stride = p->o_token_stride_elements;
+    s.ring_capacity = kv_ring_capacity;
+    s.scale = p->scale;
+    const uint32_t group = p->num_q_heads / p->num_kv_heads, hd = p->head_dim;
+    uint32_t shift = 0;
+    while ((1u << shift) < group) ++shift;
+    const bool mfma = (hd == 64 || hd == 128 || hd == 256 || hd == 512) && (1u << shift) == group && group <= (uint32_t)kTileHeads && aligned16(qp) &&
+                      aligned16(kp) && aligned16(vp) && aligned16(op) && s.q_stride % 8 == 0 && s.kv_stride % 8 == 0 && s.o_stride % 8 == 0;
+    if (mfma) {
+        const uint32_t tiles = (s.count * group + kTileHeads - 1) / kTileHeads;
+        const dim3 grid((tiles * s.num_kv_heads + kAttnWaves - 1) / kAttnWaves);
+        switch (hd) {
+            case 64: hipLaunchKernelGGL(attention_prefill_kernel<64>, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, op, s, shift, tiles); break;
+            case 128: hipLaunchKernelGGL(attention_prefill_kernel<128>, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, op, s, shift, tiles); break;
+            case 256: hipLaunchKernelGGL(attention_prefill_kernel<256>, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, op, s, shift, tiles); break;
+            default: hipLaunchKernelGGL(attention_prefill_kernel<512>, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, op, s, shift, tiles); break;
+        }
+    } else {
+        hipLaunchKernelGGL(attention_prefill_generic_kernel, dim3(s.count, s.num_q_heads), dim3(kAttnThreads), 0, st, qp, kp, vp, op, hd, s);
+    }
+    return check_launch(ctx, "prefill_attention");
 }
 
 void tf_attention_split_geometry(uint32_t num_q_heads, uint32_t num_kv_heads, uint32_t seq_len, uint32_t kv_start, int32_t prefer_gqa_swa,

@@ -179,6 +179,20 @@ private:
     const Context &c_;
 };
 
+// PrefillAttention (Kernels/Attention/PrefillAttention.swift:43-118)
+using PrefillAttentionParams = tf_prefill_attention_params;
+class PrefillAttention {
+public:
+    explicit PrefillAttention(const Context &context) : c_(context) {}
+    void encodeCausal(const void *q, uint64_t qOffset, const void *k, uint64_t kOffset, const void *v, uint64_t vOffset, void *out, uint64_t outOffset,
+                      const PrefillAttentionParams &params, uint32_t kvRingCapacity = 0) const {
+        c_.check(tf_prefill_attention_causal(c_.raw(), c_.stream(), q, qOffset, k, kOffset, v, vOffset, out, outOffset, &params, kvRingCapacity));
+    }
+
+private:
+    const Context &c_;
+};
+
 using SharedExpertProjection = tf_projection;   // Kernels/MoE/SharedExpertInt8.swift:9-31
 
 // SharedExpertRuntime / SharedExpertInt4 (Kernels/MoE/SharedExpertInt4.swift)
