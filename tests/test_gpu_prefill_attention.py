@@ -50,7 +50,11 @@ def test_reference_suite_cases(label, start, chunk, window, hd, hq, hkv, pad):
 @pytest.mark.parametrize("start,chunk,window,hd,hq,hkv", [(1000, 128, 1024, 256, 16, 8),     # a chunk of a sliding-window layer
                                                           (640, 128, 0, 512, 16, 2),        # a chunk of a global layer
                                                           (0, 77, 0, 128, 8, 8),            # no grouping, ragged count
-                                                          (5, 33, 9, 64, 16, 1)])           # sixteen query heads on one kv head
+                                                          (5, 33, 9, 64, 16, 1),            # sixteen query heads on one kv head
+                                                          (1500, 64, 0, 512, 16, 2),        # long context: the keys are split into chunks
+                                                          (2100, 128, 1024, 256, 16, 8),    # ... and a window that starts mid-cache
+                                                          (700, 40, 0, 128, 4, 4),
+                                                          (900, 24, 300, 64, 8, 2)])
 def test_production_chunks(start, chunk, window, hd, hq, hkv):
     fx = make_fixture(start, chunk, window, 0xB000 + chunk, hd, hq, hkv, (0, 0, 0))
     rc, rows = run(fx)

@@ -10,6 +10,11 @@
 //   values  O[head, :] = alpha O[head, :] + sum_p P[p, head] V[p, :] on the vector ALU with V rows read fully coalesced
 //           (a lane owns 8 consecutive output elements), probabilities passed through a per-wave LDS tile.
 // The four waves of a block, and then the chunks, are merged with the usual rescale by exp(m - m_max).
+//
+// Causal attention of a block of query tokens (prefill) follows further down: both products on the matrix cores, K and V
+// tiles shared by a block's waves through LDS.
+#include <algorithm>
+
 #include "tf_common.hpp"
 #include "tf_context.hpp"
 
@@ -314,141 +319,329 @@ __device__ __forceinline__ void visible_keys(const PrefillShape &s, uint32_t t, 
     last = min(s.kv_valid, abs_q + 1u);
 }
 
-// Matrix-core path: a wave owns 16 (query, head) columns that share one kv head - with G query heads per kv head that is
-// 16 / G consecutive queries - and walks the keys any of them sees, 16 at a time, exactly as the decode kernel does for its
-// G columns; a key outside a column's causal range or window is masked for that column only.  The K and V rows of a
-// range are thus read once per 16 / G queries instead of once per query and head.  No split over keys: a block of queries
-// makes enough waves.  HD in {64, 128, 256, 512}, G in {1, 2, 4, 8, 16}, rows 16-byte aligned.
+// Matrix-core path.  A block owns 64 (query, head) columns that share one kv head - with G query heads per kv head that
+// is 64 / G consecutive queries - and one chunk of the keys any of them sees; each of its four waves owns 16 of the columns.
+// The block walks its keys 32 at a time: the K and V rows of a tile go through LDS once for all four waves.
+//   scores  S^T[32 keys, 16 columns] = K_tile . Q^T (v_mfma_f32_16x16x32_f16, A = K rows out of LDS, B = the wave's query
+//           fragments, which stay in registers); a lane ends up with 8 keys of ONE column, so the online softmax state
+//           (m, d) and the rescale factor are per-lane scalars, and a key outside the column's causal range or window is
+//           masked for that column only;
+//   values  O^T[HD, 16 columns] += V_tile^T . P^T: the lane's 8 probabilities are already laid out as the B operand; the A
+//           operand (8 keys of one element of V) is put together from 8 row pieces of 16 bytes with byte permutes - the
+//           lane's pieces hold 8 neighbouring elements, which feed 8 matrix instructions - so V needs no transposed copy.
+// With several chunks the block leaves an unnormalised partial state (m, d, o) per column for the merge kernel; with one
+// it writes the rows itself.  HD in {64, 128, 256, 512}, G in {1, 2, 4, 8, 16}, rows 16-byte aligned.
+constexpr int kPrefillKeys = 32, kPrefillCols = 64;
+constexpr uint32_t kMaxPrefillChunks = 16, kMinChunkKeys = 256;
+constexpr uint32_t kXcds = 8;
+
+typedef __amdgpu_buffer_rsrc_t attn_rsrc_t;
+// 16 bytes per lane from a buffer straight into LDS: lane l's bytes land at dst + 16 l (dst wave-uniform)
+__device__ __forceinline__ void attn_lds_copy16(attn_rsrc_t rsrc, uint32_t dst, uint32_t lane_offset) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void *)(uintptr_t)dst, 16, lane_offset, 0, 0, 0);
+}
+// LDS reads the compiler does not see as memory accesses: it would make each of them wait for every copy still on its way
+// into LDS, the prefetched tiles included.  The result registers are only valid after attn_lds_wait on them.
+template <int OFFSET>
+__device__ __forceinline__ u32x4 attn_lds_read16(uint32_t addr) {
+    u32x4 v;
+    asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+__device__ __forceinline__ void attn_lds_wait(u32x4 (&r)[8]) {
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(r[0]), "+v"(r[1]), "+v"(r[2]), "+v"(r[3]), "+v"(r[4]), "+v"(r[5]), "+v"(r[6]), "+v"(r[7]));
+}
+
+// lane l and the lanes l ^ 16, l ^ 32, l ^ 48 (the four row groups of a score tile's column) combined, through the row
+// swaps of the vector ALU instead of four trips through the LDS crossbar: after a swap of a value with itself the two
+// results hold the lane's own row group and its partner's
+template <typename Op>
+__device__ __forceinline__ float column_reduce(float v, Op op) {
+    const uint32_t u = __builtin_bit_cast(uint32_t, v);
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const float a = op(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+    const uint32_t ua = __builtin_bit_cast(uint32_t, a);
+    const auto q = __builtin_amdgcn_permlane32_swap(ua, ua, false, false);
+    return op(__builtin_bit_cast(float, (uint32_t)q[0]), __builtin_bit_cast(float, (uint32_t)q[1]));
+}
+
 template <int HD>
-__global__ __launch_bounds__(kAttnThreads, 1) void attention_prefill_kernel(const half_t *Q, const half_t *K, const half_t *V, half_t *O,
-                                                                            PrefillShape s, uint32_t group_shift, uint32_t tiles_per_kv_head) {
-    constexpr int KS = HD / 32, LPR = HD / 8, R = 64 / LPR, VLOADS = kTilePositions / R;
-    __shared__ __align__(16) half_t p_tile[kAttnWaves][kTilePositions][kTileHeads];
-    __shared__ float alpha_tile[kAttnWaves][kTileHeads];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint32_t item = blockIdx.x * kAttnWaves + (uint32_t)wave;
-    if (item >= tiles_per_kv_head * s.num_kv_heads) return;   // whole waves leave; the kernel has no block-wide barrier
-    const uint32_t kv_head = item / tiles_per_kv_head, col_tile = item % tiles_per_kv_head;
-    const uint32_t group = 1u << group_shift, pairs = s.count << group_shift;
+__global__ __launch_bounds__(kAttnThreads, HD > 256 ? 1 : 2) void attention_prefill_kernel(const half_t *Q, const half_t *K, const half_t *V, half_t *O,
+                                                                                           float *m_part, float *d_part, float *o_part, PrefillShape s,
+                                                                                           uint32_t group_shift, uint32_t col_blocks, uint32_t num_chunks) {
+    constexpr int KS = HD / 32;                         // matrix steps over the head dimension for the scores
+    constexpr int NG = HD >= 128 ? HD / 128 : 1;        // groups of 128 output elements (16 lanes x 8)
+    constexpr int CPR = HD / 8;                         // 16-byte pieces per row
+    // A tile in LDS: one copy instruction moves 64 pieces = RPI rows; copy n of a tile carries rows n, n + NI, n + 2 NI, ...
+    // into the 1024 contiguous bytes of block n, and blocks are 1040 bytes apart: the 16 rows (or row groups) a score
+    // operand touches then start 4 banks apart.  Row r, piece c: block r % NI, byte (r / NI) * RB + 16 c.
+    constexpr int RPI = CPR >= 64 ? 1 : 64 / CPR, NI = kPrefillKeys / RPI, RB = CPR * 16, BLK = 1040, TILEB = NI * BLK;
+    constexpr int JOFF = NI >= 32 ? 16 * BLK : (16 / NI) * RB;   // from row r to row r + 16
+    constexpr int CPW = NI >= kAttnWaves ? NI / kAttnWaves : 1;  // copies per wave, tile and matrix
+    constexpr int DB = KS < 4 ? KS : 4, NB = KS / DB;            // score steps per batch of LDS reads, batches
+    __shared__ __align__(16) uint8_t k_lds[2][TILEB];
+    __shared__ __align__(16) uint8_t v_lds[2][TILEB];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int col = lane & 15, quad = lane >> 4;
-    // this lane's column: pair index -> (query, head of the group)
-    const uint32_t pair = col_tile * kTileHeads + (uint32_t)col;
-    const bool col_live = pair < pairs;
-    const uint32_t t_col = col_live ? pair >> group_shift : 0u, g_col = pair & (group - 1u);
-    uint32_t first_col = 0u, last_col = 0u;
-    if (col_live) visible_keys(s, t_col, first_col, last_col);
-    // the keys any live column of the tile sees: columns ascend by query, so the first column starts first and the last
-    // live one ends last
-    const uint32_t t_lo = min((col_tile * kTileHeads) >> group_shift, s.count - 1u);
-    const uint32_t t_hi = min((col_tile * kTileHeads + kTileHeads - 1u) >> group_shift, s.count - 1u);
+
+    // which (kv head, chunk, column block): blocks are dealt round-robin to the 8 XCDs, so when the number of
+    // (kv head, chunk) groups allows it every group's column blocks - which read the same K and V rows - share one XCD's L2
+    const uint32_t groups = s.num_kv_heads * num_chunks;
+    uint32_t grp, col_block;
+    if (groups % kXcds == 0u) {
+        const uint32_t xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+        grp = xcd + kXcds * (slot / col_blocks);
+        col_block = slot % col_blocks;
+    } else {
+        grp = blockIdx.x / col_blocks;
+        col_block = blockIdx.x % col_blocks;
+    }
+    const uint32_t kv_head = grp / num_chunks, chunk = grp % num_chunks;
+    const uint32_t group = 1u << group_shift, pairs = s.count << group_shift;
+
+    // the keys any live column of the block sees (columns ascend by query), cut into num_chunks runs of whole tiles
+    const uint32_t col0 = col_block * kPrefillCols;
+    const uint32_t t_lo = min(col0 >> group_shift, s.count - 1u), t_hi = min((col0 + kPrefillCols - 1u) >> group_shift, s.count - 1u);
     uint32_t p_lo, p_hi, unused;
     visible_keys(s, t_lo, p_lo, unused);
     visible_keys(s, t_hi, unused, p_hi);
+    const uint32_t span = p_hi > p_lo ? p_hi - p_lo : 0u;
+    const uint32_t chunk_len = ((span + num_chunks - 1u) / num_chunks + kPrefillKeys - 1u) / kPrefillKeys * kPrefillKeys;
+    const uint32_t c_lo = p_lo + chunk * chunk_len, c_hi = min(p_hi, c_lo + chunk_len);
+
+    // this lane's column: pair index -> (query, head of the group)
+    const uint32_t pair = col0 + (uint32_t)(wave * kTileHeads + col);
+    const bool col_live = pair < pairs;
+    const uint32_t t_col = col_live ? pair >> group_shift : 0u, q_head = kv_head * group + (pair & (group - 1u));
+    uint32_t first_col = 0u, last_col = 0u;
+    if (col_live) visible_keys(s, t_col, first_col, last_col);
 
     half8_t qf[KS];
 #pragma unroll
     for (int d = 0; d < KS; ++d) {
         u32x4 raw = {0u, 0u, 0u, 0u};
-        if (col_live) raw = load16(Q + (size_t)t_col * s.q_stride + (size_t)(kv_head * group + g_col) * HD + 32 * d + 8 * quad);
+        if (col_live) raw = load16(Q + (size_t)t_col * s.q_stride + (size_t)q_head * HD + 32 * d + 8 * quad);
         qf[d] = __builtin_bit_cast(half8_t, raw);
     }
-    float o[kTileHeads][8];
+    float4_t o[NG][8];   // o[g][t][r]: element 128 g + 8 (4 quad + r) + t of column `col`
 #pragma unroll
-    for (int c = 0; c < kTileHeads; ++c)
+    for (int g = 0; g < NG; ++g)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[c][e] = 0.0f;
+        for (int t = 0; t < 8; ++t) o[g][t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
     float m_run = -INFINITY, d_run = 0.0f;
-    const int vrow = lane / LPR, ve = lane % LPR;
 
-    for (uint32_t t0 = p_lo; t0 < p_hi; t0 += kTilePositions) {
-        const uint32_t pk = min(t0 + (uint32_t)col, p_hi - 1u);
-        const half_t *k_row = K + (size_t)prefill_row(s, pk) * s.kv_stride + (size_t)kv_head * HD + 8 * quad;
-        u32x4 kf[KS], vf[VLOADS];
+    // Copies: descriptors over this kv head's part of the caches (32-bit byte offsets; the host checks that the rows fit).
+    // Rows past the chunk repeat its last row: their scores are masked, their probabilities zero.
+    const attn_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(K + (size_t)kv_head * HD), 0, (int)0xFFFFFFFFu, 0x00020000);
+    const attn_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(V + (size_t)kv_head * HD), 0, (int)0xFFFFFFFFu, 0x00020000);
+    const uint32_t lane_rows = RPI > 1 ? (uint32_t)(lane / CPR) * NI : 0u, lane_piece = (uint32_t)(lane % CPR) * 16u;
+    const uint32_t row_bytes = s.kv_stride * 2u;
+    auto copy_tile = [&](attn_rsrc_t rsrc, uint32_t tile, uint32_t t0) {
+        if (wave >= NI) return;               // fewer copies than waves (head_dim 64)
 #pragma unroll
-        for (int d = 0; d < KS; ++d) kf[d] = load16(k_row + 32 * d);
-#pragma unroll
-        for (int j = 0; j < VLOADS; ++j) {
-            const uint32_t pv = min(t0 + (uint32_t)(j * R + vrow), p_hi - 1u);
-            vf[j] = load16(V + (size_t)prefill_row(s, pv) * s.kv_stride + (size_t)kv_head * HD + 8 * ve);
+        for (int q = 0; q < CPW; ++q) {
+            const uint32_t n = (uint32_t)wave + (uint32_t)(kAttnWaves * q);
+            const uint32_t p = min(t0 + n + lane_rows, c_hi - 1u);
+            attn_lds_copy16(rsrc, tile + n * BLK, prefill_row(s, p) * row_bytes + lane_piece);
         }
-        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    };
+    const uint32_t k_tile[2] = {(uint32_t)(uintptr_t)k_lds[0], (uint32_t)(uintptr_t)k_lds[1]};
+    const uint32_t v_tile[2] = {(uint32_t)(uintptr_t)v_lds[0], (uint32_t)(uintptr_t)v_lds[1]};
+    // this lane's operand pieces inside a tile: K row `col`, piece `quad` of every step; V rows 4 quad .., piece `col`
+    const uint32_t k_lane = (uint32_t)((col % NI) * BLK + (col / NI) * RB + quad * 16);
+    const uint32_t v_lane = (uint32_t)(((4 * quad) % NI) * BLK + ((4 * quad) / NI) * RB + (HD >= 128 ? col : (col & 7)) * 16);
+
+    // scores of keys 16 j + 4 quad + r of a K tile for column `col`; the reads of a batch of steps are in flight while the
+    // previous batch is multiplied
+    auto scores = [&](uint32_t tile, float4_t &acc0, float4_t &acc1) {
+        const uint32_t at = tile + k_lane;
+        acc0 = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        acc1 = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        u32x4 kf[2][8];
+        auto issue = [&](u32x4 (&f)[8], int b) {   // b is a compile-time constant after unrolling
 #pragma unroll
-        for (int d = 0; d < KS; ++d) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, kf[d]), qf[d], acc, 0, 0, 0);
-        float sc[4], tile_max = -INFINITY;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const uint32_t p = t0 + (uint32_t)(4 * quad + r);
-            sc[r] = (p >= first_col && p < last_col) ? acc[r] * s.scale : -INFINITY;
-            tile_max = fmaxf(tile_max, sc[r]);
-        }
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 16));
-        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
-        const float m_new = fmaxf(m_run, tile_max);      // stays -inf while the column has seen no key
-        const float alpha = exp_weight(m_run, m_new);
-        float sum = 0.0f;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const float pe = exp_weight(sc[r], m_new);
-            p_tile[wave][4 * quad + r][col] = (half_t)pe;
-            sum += pe;
-        }
-        sum += __shfl_xor(sum, 16);
-        sum += __shfl_xor(sum, 32);
-        d_run = d_run * alpha + sum;
-        m_run = m_new;
-        if (quad == 0) alpha_tile[wave][col] = alpha;
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // the wave reads back what its own lanes wrote
-#pragma unroll
-        for (int c = 0; c < kTileHeads; ++c) {
-            const float a = alpha_tile[wave][c];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) o[c][e] *= a;
-        }
-#pragma unroll
-        for (int j = 0; j < VLOADS; j += 2) {
-            const u32x4 ra = vf[j], rb = vf[j + 1];
-            uint32_t vv[8];
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                vv[2 * w] = __builtin_amdgcn_perm(rb[w], ra[w], 0x05040100u);
-                vv[2 * w + 1] = __builtin_amdgcn_perm(rb[w], ra[w], 0x07060302u);
+            for (int d = 0; d < DB; ++d) {
+                switch (b) {
+                    case 0: f[2 * d] = attn_lds_read16<0 * DB * 64>(at + d * 64); f[2 * d + 1] = attn_lds_read16<0 * DB * 64 + JOFF>(at + d * 64); break;
+                    case 1: f[2 * d] = attn_lds_read16<1 * DB * 64>(at + d * 64); f[2 * d + 1] = attn_lds_read16<1 * DB * 64 + JOFF>(at + d * 64); break;
+                    case 2: f[2 * d] = attn_lds_read16<2 * DB * 64>(at + d * 64); f[2 * d + 1] = attn_lds_read16<2 * DB * 64 + JOFF>(at + d * 64); break;
+                    default: f[2 * d] = attn_lds_read16<3 * DB * 64>(at + d * 64); f[2 * d + 1] = attn_lds_read16<3 * DB * 64 + JOFF>(at + d * 64); break;
+                }
             }
-            const u32x4 *pa = reinterpret_cast<const u32x4 *>(&p_tile[wave][j * R + vrow][0]);
-            const u32x4 *pb = reinterpret_cast<const u32x4 *>(&p_tile[wave][(j + 1) * R + vrow][0]);
-            const u32x4 pa0 = pa[0], pa1 = pa[1], pb0 = pb[0], pb1 = pb[1];
 #pragma unroll
-            for (int c = 0; c < kTileHeads; ++c) {
-                const uint32_t sel = (c & 1) ? 0x07060302u : 0x05040100u;
-                const uint32_t wa = c < 8 ? pa0[(c >> 1) & 3] : pa1[(c >> 1) & 3], wb = c < 8 ? pb0[(c >> 1) & 3] : pb1[(c >> 1) & 3];
-                const half2_t pc = as_half2(__builtin_amdgcn_perm(wb, wa, sel));
+            for (int d = 2 * DB; d < 8; ++d) f[d] = u32x4{0u, 0u, 0u, 0u};
+        };
+        issue(kf[0], 0);
 #pragma unroll
-                for (int e = 0; e < 8; ++e) o[c][e] = __builtin_amdgcn_fdot2(pc, as_half2(vv[e]), o[c][e], false);
+        for (int b = 0; b < NB; ++b) {
+            attn_lds_wait(kf[b & 1]);
+            if (b + 1 < NB) issue(kf[(b + 1) & 1], b + 1);
+#pragma unroll
+            for (int d = 0; d < DB; ++d) {
+                acc0 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, kf[b & 1][2 * d]), qf[b * DB + d], acc0, 0, 0, 0);
+                acc1 = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, kf[b & 1][2 * d + 1]), qf[b * DB + d], acc1, 0, 0, 0);
             }
         }
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    };
+    auto issue_values = [&](u32x4 (&in)[8], uint32_t tile, int g) {
+        const uint32_t at = tile + v_lane + (uint32_t)(g * 256);
+        in[0] = attn_lds_read16<0 * BLK>(at);
+        in[1] = attn_lds_read16<1 * BLK>(at);
+        in[2] = attn_lds_read16<2 * BLK>(at);
+        in[3] = attn_lds_read16<3 * BLK>(at);
+        in[4] = attn_lds_read16<JOFF + 0 * BLK>(at);
+        in[5] = attn_lds_read16<JOFF + 1 * BLK>(at);
+        in[6] = attn_lds_read16<JOFF + 2 * BLK>(at);
+        in[7] = attn_lds_read16<JOFF + 3 * BLK>(at);
+    };
+
+    if (c_lo < c_hi) {
+        const uint32_t n_tiles = (c_hi - c_lo + kPrefillKeys - 1u) / kPrefillKeys;
+        copy_tile(k_rsrc, k_tile[0], c_lo);
+        copy_tile(k_rsrc, k_tile[1], c_lo + kPrefillKeys);
+        copy_tile(v_rsrc, v_tile[0], c_lo);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        float4_t acc0, acc1;
+        scores(k_tile[0], acc0, acc1);
+        __syncthreads();
+        // Step i, first half: start the copies of the tiles two (K) and one (V) ahead, take the scores of tile i + 1, and
+        // turn the scores of tile i into probabilities.  Here K tiles i (its scores are in acc0/acc1) and i + 1 and V tile
+        // i are in LDS and nobody reads the other two buffers any more.
+        // The reference maximum of a column only moves when a score exceeds it by more than kMaxSlack (probabilities then
+        // reach at most e^kMaxSlack, far inside fp16): after the first tiles the accumulators are hardly ever rescaled.
+        constexpr float kMaxSlack = 8.0f;
+        auto first_half = [&](uint32_t i, float &alpha, half8_t &p8, float4_t &next0, float4_t &next1) {
+            const uint32_t t0 = c_lo + i * kPrefillKeys, cur = i & 1u;
+            copy_tile(k_rsrc, k_tile[cur], t0 + 2 * kPrefillKeys);
+            copy_tile(v_rsrc, v_tile[cur ^ 1u], t0 + kPrefillKeys);
+            scores(k_tile[cur ^ 1u], next0, next1);   // of tile i + 1 (past the chunk: repeated rows, never used)
+            float sc[8], tile_max = -INFINITY;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const uint32_t p = t0 + (uint32_t)(16 * (e >> 2) + 4 * quad + (e & 3));
+                const float raw = e < 4 ? acc0[e & 3] : acc1[e & 3];
+                sc[e] = (p >= first_col && p < last_col) ? raw * s.scale : -INFINITY;
+                tile_max = fmaxf(tile_max, sc[e]);
+            }
+            tile_max = column_reduce(tile_max, [](float a, float b) { return fmaxf(a, b); });
+            // stays -inf while the column has seen no key; the first finite maximum costs no rescale (o and d are zero)
+            const bool fresh = m_run == -INFINITY;
+            const float m_new = (fresh || tile_max > m_run + kMaxSlack) ? fmaxf(m_run, tile_max) : m_run;
+            alpha = fresh ? 1.0f : __expf(m_run - m_new);
+            float sum = 0.0f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float pe = exp_weight(sc[e], m_new);
+                p8[e] = (half_t)pe;
+                sum += pe;
+            }
+            sum = column_reduce(sum, [](float a, float b) { return a + b; });
+            d_run = d_run * alpha + sum;
+            m_run = m_new;
+        };
+        // Step i, second half: values.  Slot e of the lane's 8 keys is row 16 (e / 4) + 4 quad + e % 4 of the tile.
+        auto second_half = [&](uint32_t i, const half8_t &p8, const float4_t &next0, const float4_t &next1) {
+            const uint32_t cur = i & 1u;
+            u32x4 in[2][8];
+            issue_values(in[0], v_tile[cur], 0);
+#pragma unroll
+            for (int g = 0; g < NG; ++g) {
+                attn_lds_wait(in[g & 1]);
+                if (g + 1 < NG) issue_values(in[(g + 1) & 1], v_tile[cur], g + 1);
+#pragma unroll
+                for (int t = 0; t < 8; ++t) {
+                    const uint32_t sel = (t & 1) ? 0x07060302u : 0x05040100u;
+                    u32x4 a;
+#pragma unroll
+                    for (int kp = 0; kp < 4; ++kp) a[kp] = __builtin_amdgcn_perm(in[g & 1][2 * kp + 1][t >> 1], in[g & 1][2 * kp][t >> 1], sel);
+                    o[g][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(half8_t, a), p8, o[g][t], 0, 0, 0);
+                }
+            }
+            acc0 = next0;
+            acc1 = next1;
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wave's copies have landed
+            __syncthreads();
+        };
+        for (uint32_t i = 0; i < n_tiles; ++i) {
+            float alpha;
+            half8_t p8;
+            float4_t next0, next1;
+            first_half(i, alpha, p8, next0, next1);
+            if (__builtin_expect(__any(alpha != 1.0f), 0)) {
+                // The accumulators live in the accumulation registers, where the matrix instructions update them in
+                // place.  Written as plain multiplications, this rare path makes the register allocator move all of them
+                // to vector registers and back in EVERY step; so it does the move itself.  The matrix instructions that
+                // last wrote them finished long ago (the scores came after them and have been read), and the next ones to
+                // read them follow LDS reads and a wait.
+#pragma unroll
+                for (int g = 0; g < NG; ++g)
+#pragma unroll
+                    for (int t = 0; t < 8; ++t) o[g][t] *= alpha;
+            }
+            second_half(i, p8, next0, next1);
+        }
     }
-    // 1 / d of every column, then the rows: out[t, head, :] = o / d, zero where a column saw no key
-    if (quad == 0) alpha_tile[wave][col] = d_run > 0.0f ? 1.0f / d_run : 0.0f;
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+
+    if (!col_live || (HD < 128 && quad >= 2)) return;      // no barrier follows
+    if (num_chunks == 1u) {
+        // out[t, head, :] = o / d, zero where the column saw no key
+        const float inv = d_run > 0.0f ? 1.0f / d_run : 0.0f;
+        half_t *dst = O + (size_t)t_col * s.o_stride + (size_t)q_head * HD + 32 * quad;
 #pragma unroll
-    for (int c = 0; c < kTileHeads; ++c) {
-        const uint32_t pc = col_tile * kTileHeads + (uint32_t)c;
-        if (pc >= pairs) break;
-        const float inv = alpha_tile[wave][c];
-        u32x4 packed;
+        for (int g = 0; g < NG; ++g)
 #pragma unroll
-        for (int e = 0; e < 8; e += 2) {
-            float a = o[c][e], b = o[c][e + 1];
-            if constexpr (R >= 2) { a += __shfl_xor(a, 32); b += __shfl_xor(b, 32); }
-            if constexpr (R >= 4) { a += __shfl_xor(a, 16); b += __shfl_xor(b, 16); }
-            if constexpr (R >= 8) { a += __shfl_xor(a, 8); b += __shfl_xor(b, 8); }
-            const half2_t h = {(half_t)(a * inv), (half_t)(b * inv)};
-            packed[e >> 1] = as_u32(h);
+            for (int r = 0; r < 4; ++r) {
+                u32x4 packed;
+#pragma unroll
+                for (int t = 0; t < 8; t += 2) {
+                    const half2_t h = {(half_t)(o[g][t][r] * inv), (half_t)(o[g][t + 1][r] * inv)};
+                    packed[t >> 1] = as_u32(h);
+                }
+                *reinterpret_cast<u32x4 *>(dst + 128 * g + 8 * r) = packed;
+            }
+    } else {
+        const size_t state = ((size_t)t_col * s.num_q_heads + q_head) * num_chunks + chunk;
+        if (quad == 0) {
+            m_part[state] = m_run;
+            d_part[state] = d_run;
         }
-        if (vrow == 0) {
-            half_t *dst = O + (size_t)(pc >> group_shift) * s.o_stride + (size_t)(kv_head * group + (pc & (group - 1u))) * HD + 8 * ve;
-            *reinterpret_cast<u32x4 *>(dst) = packed;
-        }
+        float *dst = o_part + state * HD + 32 * quad;
+#pragma unroll
+        for (int g = 0; g < NG; ++g)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                *reinterpret_cast<float4_t *>(dst + 128 * g + 8 * r) = float4_t{o[g][0][r], o[g][1][r], o[g][2][r], o[g][3][r]};
+                *reinterpret_cast<float4_t *>(dst + 128 * g + 8 * r + 4) = float4_t{o[g][4][r], o[g][5][r], o[g][6][r], o[g][7][r]};
+            }
+    }
+}
+
+// merge of the chunks' partial states of one (query, head) column: out = sum_c w_c o_c / sum_c w_c d_c, w_c = exp(m_c - max m);
+// chunks are added in ascending order; a chunk that saw no key has weight zero and its o is not read
+__global__ __launch_bounds__(128) void attention_prefill_combine_kernel(const float *m_part, const float *d_part, const float *o_part, half_t *O,
+                                                                        uint32_t head_dim, uint32_t num_chunks, uint32_t num_q_heads,
+                                                                        uint32_t o_stride) {
+    const uint32_t column = blockIdx.x, t = column / num_q_heads, q_head = column % num_q_heads;
+    const float *m_row = m_part + (size_t)column * num_chunks, *d_row = d_part + (size_t)column * num_chunks;
+    float w[kMaxPrefillChunks], m_max = -INFINITY, den = 0.0f;
+    for (uint32_t c = 0; c < num_chunks; ++c) m_max = fmaxf(m_max, m_row[c]);
+#pragma unroll
+    for (uint32_t c = 0; c < kMaxPrefillChunks; ++c) {
+        w[c] = c < num_chunks ? exp_weight(m_row[c], m_max) : 0.0f;
+        if (c < num_chunks) den += d_row[c] * w[c];
+    }
+    const float inv = den > 0.0f ? 1.0f / den : 0.0f;
+    for (uint32_t e = threadIdx.x * 4u; e < head_dim; e += 128u * 4u) {
+        float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+        const float *src = o_part + (size_t)column * num_chunks * head_dim + e;
+#pragma unroll
+        for (uint32_t c = 0; c < kMaxPrefillChunks; ++c)
+            if (c < num_chunks && w[c] != 0.0f) acc += *reinterpret_cast<const float4_t *>(src + (size_t)c * head_dim) * w[c];
+        const half2_t lo = {(half_t)(acc[0] * inv), (half_t)(acc[1] * inv)}, hi = {(half_t)(acc[2] * inv), (half_t)(acc[3] * inv)};
+        uint32_t *dst = reinterpret_cast<uint32_t *>(O + (size_t)t * o_stride + (size_t)q_head * head_dim + e);
+        dst[0] = as_u32(lo);
+        dst[1] = as_u32(hi);
     }
 }
 
@@ -644,17 +837,39 @@ int32_t tf_prefill_attention_causal(tf_ctx *ctx, tf_stream stream, const void *q
     const uint32_t group = p->num_q_heads / p->num_kv_heads, hd = p->head_dim;
     uint32_t shift = 0;
     while ((1u << shift) < group) ++shift;
+    const uint64_t cache_bytes = (uint64_t)(kv_ring_capacity ? kv_ring_capacity : p->kv_valid_count) * p->kv_token_stride_elements * 2u;
     const bool mfma = (hd == 64 || hd == 128 || hd == 256 || hd == 512) && (1u << shift) == group && group <= (uint32_t)kTileHeads && aligned16(qp) &&
-                      aligned16(kp) && aligned16(vp) && aligned16(op) && s.q_stride % 8 == 0 && s.kv_stride % 8 == 0 && s.o_stride % 8 == 0;
+                      aligned16(kp) && aligned16(vp) && aligned16(op) && s.q_stride % 8 == 0 && s.kv_stride % 8 == 0 && s.o_stride % 8 == 0 &&
+                      cache_bytes < (1ull << 32);   // the copies address cache rows with 32-bit byte offsets
     if (mfma) {
-        const uint32_t tiles = (s.count * group + kTileHeads - 1) / kTileHeads;
-        const dim3 grid((tiles * s.num_kv_heads + kAttnWaves - 1) / kAttnWaves);
-        switch (hd) {
-            case 64: hipLaunchKernelGGL(attention_prefill_kernel<64>, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, op, s, shift, tiles); break;
-            case 128: hipLaunchKernelGGL(attention_prefill_kernel<128>, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, op, s, shift, tiles); break;
-            case 256: hipLaunchKernelGGL(attention_prefill_kernel<256>, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, op, s, shift, tiles); break;
-            default: hipLaunchKernelGGL(attention_prefill_kernel<512>, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, op, s, shift, tiles); break;
+        const uint32_t col_blocks = (s.count * group + kPrefillCols - 1) / kPrefillCols, base = col_blocks * s.num_kv_heads;
+        // enough chunks to give every CU a block (two where two fit), none shorter than kMinChunkKeys
+        const uint32_t abs_first = s.start, abs_last = s.start + s.count - 1u;
+        const uint32_t lo_first = (s.window != 0u && abs_first + 1u > s.window) ? abs_first + 1u - s.window : 0u;
+        const uint32_t hi_last = std::min(s.kv_valid, abs_last + 1u);
+        const uint32_t span = hi_last > lo_first ? hi_last - lo_first : 0u;
+        const uint32_t target = (uint32_t)ctx->num_cus * (hd > 256 ? 1u : 2u);
+        uint32_t chunks = std::max(1u, std::min({(target + base - 1) / base, span / kMinChunkKeys, kMaxPrefillChunks}));
+        float *m = nullptr, *d = nullptr, *o = nullptr;
+        if (chunks > 1) {
+            const size_t states = (size_t)s.count * s.num_q_heads * chunks;
+            float *scratch = nullptr;
+            const int32_t rc = attention_scratch(ctx, states * (2 + (size_t)hd), scratch);
+            if (rc != TF_OK) return rc;
+            m = scratch;
+            d = scratch + states;
+            o = scratch + 2 * states;
         }
+        const dim3 grid(base * chunks);
+        switch (hd) {
+            case 64: hipLaunchKernelGGL(attention_prefill_kernel<64>, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, op, m, d, o, s, shift, col_blocks, chunks); break;
+            case 128: hipLaunchKernelGGL(attention_prefill_kernel<128>, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, op, m, d, o, s, shift, col_blocks, chunks); break;
+            case 256: hipLaunchKernelGGL(attention_prefill_kernel<256>, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, op, m, d, o, s, shift, col_blocks, chunks); break;
+            default: hipLaunchKernelGGL(attention_prefill_kernel<512>, grid, dim3(kAttnThreads), 0, st, qp, kp, vp, op, m, d, o, s, shift, col_blocks, chunks); break;
+        }
+        if (chunks > 1)
+            hipLaunchKernelGGL(attention_prefill_combine_kernel, dim3(s.count * s.num_q_heads), dim3(128), 0, st, m, d, o, op, hd, chunks, s.num_q_heads,
+                               s.o_stride);
     } else {
         hipLaunchKernelGGL(attention_prefill_generic_kernel, dim3(s.count, s.num_q_heads), dim3(kAttnThreads), 0, st, qp, kp, vp, op, hd, s);
     }
