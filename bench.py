@@ -530,7 +530,7 @@ def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride):
         return us, unique
 
     small = {}
-    for M in (2, 4, 8, 16):
+    for M in (2, 4, 8, 16, 32, 64, 128):      # verification sizes, then the reference's prefill chunk sizes (RuntimeConfiguration.swift:24)
         us, unique = run(M, iters=50)
         nbytes = unique * expert_bytes + E * D + M * (2 * D * 2 + TOPK * F_MOE * 2 * 2 + TOPK * D * 2 * 2)
         small[str(M)] = {"us": round(us, 2), "unique_experts": unique, "GBps_on_unique_expert_bytes": round(nbytes / (us * 1e-6) / 1e9, 1),

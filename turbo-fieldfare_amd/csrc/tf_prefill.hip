@@ -1076,8 +1076,9 @@ int32_t tf_prefill_grouped_routed_moe_resident(tf_ctx *ctx, tf_stream stream, co
     GroupedGeom g{static_cast<const tf_prefill_pair *>(sorted_pairs), reinterpret_cast<const half_t *>(at(hidden, hidden_offset)),
                   (long)hidden_stride_elements, static_cast<half_t *>(acts_scratch), 0u, static_cast<half_t *>(route_partials), (int)d,
                   (int)f, (int)top_k};
-    // the host only knows the average group size: matrix cores once experts see 8 or more tokens on average
-    const bool use_mfma = (uint64_t)pair_count >= (uint64_t)num_experts * 8;
+    // the host only knows the average group size: the matrix cores pay once experts see 2 or more tokens on average (with
+    // fewer, up to kStreamTokens tokens, the row-streaming kernels read every touched expert once at a higher rate)
+    const bool use_mfma = (uint64_t)pair_count >= (uint64_t)num_experts * 2;
     // the pairs are all (token, rank) combinations of pair_count / top_k token rows
     const uint32_t tokens = pair_count % top_k == 0 ? pair_count / top_k : 0u;
     return run_grouped(ctx, static_cast<hipStream_t>(stream), tab, *routed_offsets, cl, max_chunks, g, scale_dtype, use_mfma, tokens, pair_count);
