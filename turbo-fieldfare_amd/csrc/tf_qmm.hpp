@@ -140,12 +140,15 @@ __device__ __forceinline__ void qmm_w_copy(const QmmBRows &rows, int pair, uint3
     for (int t = 0; t < 4; ++t) lds_copy16(rows.w[t >> 1], dst + t * 1024u, rows.copy_off[t], pair * 64);
 }
 
-// X tile of step kt -> LDS stage at byte address `stage` (wave-uniform); kAChunks copies of 64 x 16 bytes per wave
-template <int NW>
+// X tile of step kt -> LDS stage at byte address `stage` (wave-uniform); COPIES copies of 64 x 16 bytes per wave.  Copy q of
+// the block covers rows 8 NW q .. 8 NW (q + 1) - 1, so a block that multiplies RT row tiles needs the first
+// ceil(4 RT / NW) of the kAChunks copies only; the rows of the others are never read.
+template <int NW, int COPIES>
 __device__ __forceinline__ void qmm_a_copy(const QmmARows<NW> &a, int kt, uint32_t stage) {
+    static_assert(COPIES >= 1 && COPIES <= QmmGeom<NW>::kAChunks, "copies per step");
     const uint32_t wave_base = stage + (threadIdx.x >> 6) * 1024u;
 #pragma unroll
-    for (int q = 0; q < QmmGeom<NW>::kAChunks; ++q) lds_copy16(a.rsrc, wave_base + (uint32_t)q * (uint32_t)(QmmGeom<NW>::kThreads * 16), a.off[q], kt * 128);
+    for (int q = 0; q < COPIES; ++q) lds_copy16(a.rsrc, wave_base + (uint32_t)q * (uint32_t)(QmmGeom<NW>::kThreads * 16), a.off[q], kt * 128);
 }
 
 // ds_read_b128 at addr + OFFSET, invisible to the compiler's memory tracking (see the header comment)
@@ -216,16 +219,18 @@ __device__ __forceinline__ void qmm_group(const u32x4 w[2], const QmmSB &sb, con
 // The K loop.  The X tile of step kt lives in LDS stage kt % 3; the packed W rows of steps 2p, 2p + 1 in the wave's
 // buffer p & 1, the scales / biases of those two groups in register slot p & 1.
 // Even step kt = 2p:  barrier; request X(kt + 2), W(p + 1); multiply with the W words read from LDS at the end of the
-//                     previous step; request the scales of pair p + 1; wait for X(kt + 1) (the kAChunks + 8 newer
+//                     previous step; request the scales of pair p + 1; wait for X(kt + 1) (the AC + 8 newer
 //                     requests stay in flight).
-// Odd step:           barrier; request X(kt + 2); multiply; wait for X(kt + 1), W(p + 1) and the scales (the kAChunks
+// Odd step:           barrier; request X(kt + 2); multiply; wait for X(kt + 1), W(p + 1) and the scales (the AC
 //                     newer requests stay in flight); read the W words of both steps of pair p + 1 from LDS, switch
 //                     to its scales.
 // Requests are unconditional: past the end they repeat the last step or pair, which nobody reads, so that the number
 // of requests in flight is the same at every wait.
 template <int SD, int RT, int NW>
 struct QmmLoop {
-    static_assert(QmmGeom<NW>::kAChunks == 4 || QmmGeom<NW>::kAChunks == 2, "the waits below are written for 4 or 2 X copies per step");
+    // X copies per step and thread: those that carry rows of the RT row tiles.  A block with a single row tile keeps all
+    // of them (the others re-read valid rows out of L2): without them chunks of 32 to 128 tokens measured 5 % slower.
+    static constexpr int AC = RT == 1 ? QmmGeom<NW>::kAChunks : (4 * RT + NW - 1) / NW;
     const QmmARows<NW> &a;
     const QmmBRows &rows;
     uint32_t lds;
@@ -251,21 +256,20 @@ struct QmmLoop {
     __device__ __forceinline__ void even_step(int kt, float16_t acc[4][2]) {
         const int pair = kt >> 1;
         __builtin_amdgcn_s_barrier();
-        qmm_a_copy<NW>(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
+        qmm_a_copy<NW, AC>(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
         qmm_w_copy(rows, min(pair + 1, last_pair), wbuf + (pb ^ kQmmWBytes));
         qmm_group<SD, RT, U3, 0>(w[0], sb, frag, nc, acc);
         const int next_pair = min(pair + 1, last_pair);
         qmm_sb_load(sb_next, rows, next_pair, odd_count && next_pair == last_pair);
-        if constexpr (QmmGeom<NW>::kAChunks == 4) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(10)" ::: "memory");
+        // everything older than this step's AC + 4 + 4 requests (X, W, scales and biases) has landed
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AC + 8) : "memory");
     }
     template <int U3>
     __device__ __forceinline__ void odd_step(int kt, float16_t acc[4][2]) {
         __builtin_amdgcn_s_barrier();
-        qmm_a_copy<NW>(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
+        qmm_a_copy<NW, AC>(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
         qmm_group<SD, RT, U3, 1>(w[1], sb, frag, nc, acc);
-        if constexpr (QmmGeom<NW>::kAChunks == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AC) : "memory");   // only this step's X copies may still be on their way
         pb ^= kQmmWBytes;
         read_w(wread + pb);
         sb = sb_next;
@@ -283,8 +287,8 @@ struct QmmLoop {
         wread = wbuf + (uint32_t)i * 64u + ((((uint32_t)kb) ^ (uint32_t)((i >> 2) & 3)) << 4);
         pb = 0;
         nc = nibble_consts();
-        qmm_a_copy<NW>(a, 0, lds);
-        qmm_a_copy<NW>(a, min(1, last), lds + kQmmStageBytes);
+        qmm_a_copy<NW, AC>(a, 0, lds);
+        qmm_a_copy<NW, AC>(a, min(1, last), lds + kQmmStageBytes);
         qmm_w_copy(rows, 0, wbuf);
         qmm_sb_load(sb, rows, 0, odd_count && last_pair == 0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
