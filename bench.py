@@ -95,6 +95,7 @@ def main():
     ap.add_argument("--layers", type=int, default=4, help="layer replicas the steps rotate through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip lm_head / GEMV / shared-expert side measurements")
+    ap.add_argument("--no-layer-chain", action="store_true", help="skip the whole-decoder-layer graph (long under a counter-collecting profiler)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (a known-size reference for hardware byte counters)")
     args = ap.parse_args()
@@ -233,7 +234,8 @@ def main():
     if not args.no_extras:
         out["extras"] = extras(torch, tfk, k, gen, lib, h, stream)
         out["extras"].update(multi_token_extras(torch, tfk, k, gen, lib, h, stream, layers[0], offs, stride))
-        out["extras"].update(layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride))
+        if not args.no_layer_chain:
+            out["extras"].update(layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride))
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, layers, hidden, idx, wts, y, offs, stride, payload, args)
