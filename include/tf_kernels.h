@@ -172,6 +172,33 @@ int32_t tf_gelu_mul_fp16(tf_ctx *ctx, tf_stream stream,
 int32_t tf_rmsnorm_bf16w(tf_ctx *ctx, tf_stream stream,
                          const void *x, uint64_t x_offset, const void *weight, uint64_t weight_offset,
                          void *out, uint64_t out_offset, uint32_t d, float eps);
+/* RMSNorm.encodeNoScale (RMSNorm.swift:67-87) -> rmsnorm_no_scale (rmsnorm.metal:153-175): out = half(x * inv). */
+int32_t tf_rmsnorm_no_scale(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, void *out, uint64_t out_offset,
+                            uint32_t d, float eps);
+/* RMSNorm.encodeBF16WPerHead / encodeNoScalePerHead (RMSNorm.swift:89-136) -> rmsnorm_bf16w_perhead,
+ * rmsnorm_no_scale_perhead (rmsnorm.metal:100-151): num_heads contiguous heads of head_dim, each normalised on its own;
+ * weight bf16[head_dim] shared by the heads.  In place is allowed. */
+int32_t tf_rmsnorm_bf16w_perhead(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, const void *weight,
+                                 uint64_t weight_offset, void *out, uint64_t out_offset, uint32_t head_dim,
+                                 uint32_t num_heads, float eps);
+int32_t tf_rmsnorm_no_scale_perhead(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, void *out,
+                                    uint64_t out_offset, uint32_t head_dim, uint32_t num_heads, float eps);
+/* PrefillRMSNorm.encodeBF16W (Kernels/Prefill/Primitives/PrefillPrimitives.swift:41-71) -> prefill_rmsnorm_bf16w_block
+ * (Metal/Prefill/prefill.metal:86-111): `tokens` contiguous rows of d. */
+int32_t tf_prefill_rmsnorm_bf16w_block(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, const void *weight,
+                                       uint64_t weight_offset, void *out, uint64_t out_offset, uint32_t tokens, uint32_t d,
+                                       float eps);
+/* PrefillPerHeadNorm.encodeBF16W / encodeNoScale (Kernels/Prefill/Primitives/PrefillPerHeadNorm.swift:13-84) ->
+ * prefill_rmsnorm_bf16w_perhead_block, prefill_rmsnorm_no_scale_perhead_block (prefill.metal:113-176): head h of token t at
+ * t * token_stride_elements + h * head_dim in x and in out; elements between token rows are untouched.  Every row equals
+ * the single-row call on that row, bit for bit (the reference suite's own check, PrefillPerHeadNormTests.swift:90,144). */
+int32_t tf_prefill_rmsnorm_bf16w_perhead_block(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset,
+                                               const void *weight, uint64_t weight_offset, void *out, uint64_t out_offset,
+                                               uint32_t query_count, uint32_t head_dim, uint32_t num_heads,
+                                               uint32_t token_stride_elements, float eps);
+int32_t tf_prefill_rmsnorm_no_scale_perhead_block(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, void *out,
+                                                  uint64_t out_offset, uint32_t query_count, uint32_t head_dim,
+                                                  uint32_t num_heads, uint32_t token_stride_elements, float eps);
 
 /* ---- the stages either side of the MoE block ------------------------------------------------------------------- */
 /* FusedPostAttentionSetup.encode (Kernels/Fusions/FusedPostAttentionSetup.swift:19-56) -> fused_post_attn_setup
@@ -281,6 +308,25 @@ int32_t tf_fused_qkv_epilogue(tf_ctx *ctx, tf_stream stream, void *q, uint64_t q
                               void *v, uint64_t v_offset, const void *q_weight, uint64_t q_weight_offset,
                               const void *k_weight, uint64_t k_weight_offset, uint32_t head_dim, uint32_t num_q_heads,
                               uint32_t num_kv_heads, uint32_t position, float theta, uint32_t rotated_pairs, float eps);
+/* PrefillRoPE.encodeDefaultNeox / encodeProportionalNeox (Kernels/Prefill/Primitives/PrefillRoPE.swift:13-88) ->
+ * prefill_rope_default_neox_block, prefill_rope_proportional_neox_block (Metal/Prefill/prefill.metal:709-775): token t of
+ * the block (row t, token_stride_elements apart) is rotated for position start_position + t, in place. */
+int32_t tf_prefill_rope_default_neox_block(tf_ctx *ctx, tf_stream stream, void *data, uint64_t data_offset,
+                                           uint32_t start_position, uint32_t query_count, uint32_t head_dim,
+                                           uint32_t num_heads, uint32_t token_stride_elements, float theta);
+int32_t tf_prefill_rope_proportional_neox_block(tf_ctx *ctx, tf_stream stream, void *data, uint64_t data_offset,
+                                                uint32_t start_position, uint32_t query_count, uint32_t head_dim,
+                                                uint32_t num_heads, uint32_t rotated_pairs, uint32_t token_stride_elements,
+                                                float theta);
+/* PrefillQKVEpilogue.encode (Kernels/Prefill/Epilogues/PrefillQKVEpilogue.swift:13-121): per token of the block the
+ * per-head norms of q, k (bf16 weight) and v (no scale), then the rotation of q and k for position start_position + t; one
+ * launch here, the reference's five.  Each token equals tf_fused_qkv_epilogue on its rows, bit for bit. */
+int32_t tf_prefill_qkv_epilogue_block(tf_ctx *ctx, tf_stream stream, void *q, uint64_t q_offset, void *k, uint64_t k_offset,
+                                      void *v, uint64_t v_offset, const void *q_weight, uint64_t q_weight_offset,
+                                      const void *k_weight, uint64_t k_weight_offset, uint32_t start_position,
+                                      uint32_t query_count, uint32_t head_dim, uint32_t num_q_heads, uint32_t num_kv_heads,
+                                      uint32_t q_token_stride_elements, uint32_t kv_token_stride_elements, float theta,
+                                      uint32_t rotated_pairs, float eps);
 
 /* PrefillAttentionParams (Kernels/Attention/PrefillAttention.swift:4-40; Metal/Prefill/prefill.metal:775-788): 44 bytes. */
 typedef struct tf_prefill_attention_params {

@@ -731,6 +731,26 @@ void tfo_k_rmsnorm_bf16w(const uint16_t *x_f16, const uint16_t *w_bf16, float ep
         out_f16[i] = tfo_f16_bits(tfo_f16_to_float(x_f16[i]) * inv * tfo_bf16_to_float(w_bf16[i]));
 }
 
+// Kernel-order restatement of the row-grid norms: rmsnorm_no_scale / rmsnorm_*_perhead (M/Primitives/rmsnorm.metal:100-175)
+// and their prefill twins (M/Prefill/prefill.metal:86-176): head h of token t at t * token_stride + h * d, each row
+// normalised on its own exactly as tfo_k_rmsnorm_bf16w does; w_bf16 == nullptr: no scale.  Elements between rows keep
+// what out_f16 held.
+void tfo_k_rmsnorm_rows(const uint16_t *x_f16, const uint16_t *w_bf16, float eps, uint16_t *out_f16, int tokens, int heads, int d,
+                        int token_stride) {
+    std::vector<uint16_t> ones;
+    for (int t = 0; t < tokens; ++t)
+        for (int h = 0; h < heads; ++h) {
+            const size_t at = (size_t)t * token_stride + (size_t)h * d;
+            if (w_bf16) {
+                tfo_k_rmsnorm_bf16w(x_f16 + at, w_bf16, eps, out_f16 + at, d);
+            } else {
+                // x * inv * 1.0f is x * inv: the weighted routine with unit weights is the unweighted one
+                if (ones.empty()) ones.assign((size_t)d, (uint16_t)0x3F80);
+                tfo_k_rmsnorm_bf16w(x_f16 + at, ones.data(), eps, out_f16 + at, d);
+            }
+        }
+}
+
 // ---- neighbours of the output head ---------------------------------------------------------------------------------
 // VS/Reference/Quant/EmbedLookup.swift:41-68 (applyInt4): one row of the tied int4 table, dequantized and scaled.
 void tfo_embed_lookup_int4(const uint8_t *table, const uint16_t *S, const uint16_t *B, uint32_t token, int d, float out_scale, float *out) {

@@ -192,6 +192,8 @@ void tfo_k_layer_tail(const uint16_t *h2_f16, const uint16_t *h1_f16, uint16_t *
 void tfo_layer_tail_ref(const uint16_t *h2_f16, const uint16_t *h1_f16, const uint16_t *hidden_f16, const uint16_t *w_postffn2_bf16,
                         const uint16_t *w_postffn_bf16, float eps, float layer_scalar, float *out, int d); /* T/Core/Kernels/Fusions/FusedLayerTailTests.swift:76-92 */
 void tfo_k_rmsnorm_bf16w(const uint16_t *x_f16, const uint16_t *w_bf16, float eps, uint16_t *out_f16, int d); /* M/Primitives/rmsnorm.metal:32-93 */
+void tfo_k_rmsnorm_rows(const uint16_t *x_f16, const uint16_t *w_bf16, float eps, uint16_t *out_f16, int tokens, int heads, int d,
+                        int token_stride); /* M/Primitives/rmsnorm.metal:100-175, M/Prefill/prefill.metal:86-176 */
 void tfo_k_prefill_router_logits(const uint8_t *W, const uint16_t *S, const uint16_t *B, const uint16_t *hidden_f16,
                                  const uint16_t *eff_scale_bf16, float *logits, int num_experts, int d); /* M/Prefill/prefill.metal:503-525 */
 float tfo_k_prefill_int4_row(const uint8_t *W, const uint16_t *S, const uint16_t *B, const uint16_t *x_f16,

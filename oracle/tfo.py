@@ -276,6 +276,7 @@ _sig("tfo_gelu_tanh", None, f32p, f32p, i64)
 _sig("tfo_rmsnorm_ref", None, f32p, f32p, C.c_float, f32p, i32)
 _sig("tfo_k_gelu_mul_fp16", None, u16p, u16p, u16p, i32)
 _sig("tfo_k_rmsnorm_bf16w", None, u16p, u16p, C.c_float, u16p, i32)
+_sig("tfo_k_rmsnorm_rows", None, u16p, C.c_void_p, C.c_float, u16p, i32, i32, i32, i32)
 
 
 def gelu_tanh(x) -> np.ndarray:
@@ -297,6 +298,15 @@ def k_gelu_mul_fp16(gate_bits, up_bits) -> np.ndarray:
     u = np.ascontiguousarray(up_bits, np.uint16)
     out = np.empty_like(g)
     lib.tfo_k_gelu_mul_fp16(g, u, out, g.size)
+    return out
+
+
+def k_rmsnorm_rows(x_bits, w_bits, eps: float, tokens: int, heads: int, d: int, token_stride: int, out_bits=None) -> np.ndarray:
+    """Row-grid norms in kernel order (w_bits None: no scale); `out_bits` supplies what lies between the rows (default: x)."""
+    x = np.ascontiguousarray(x_bits, np.uint16)
+    out = np.array(x if out_bits is None else out_bits, np.uint16, copy=True)
+    w = None if w_bits is None else np.ascontiguousarray(w_bits, np.uint16)
+    lib.tfo_k_rmsnorm_rows(x, None if w is None else w.ctypes.data_as(C.c_void_p), eps, out, tokens, heads, d, token_stride)
     return out
 
 

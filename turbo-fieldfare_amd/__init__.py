@@ -132,6 +132,16 @@ EXPORTS = {
     "tf_rope_default_neox": (i32, [vp, vp, vp, u64, u32, u32, u32, u32, C.c_float]),
     "tf_rope_proportional_neox": (i32, [vp, vp, vp, u64, u32, u32, u32, u32, u32, C.c_float]),
     "tf_fused_qkv_epilogue": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, C.c_float, u32, C.c_float]),
+    "tf_rmsnorm_no_scale": (i32, [vp, vp, vp, u64, vp, u64, u32, C.c_float]),
+    "tf_rmsnorm_bf16w_perhead": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32, u32, C.c_float]),
+    "tf_rmsnorm_no_scale_perhead": (i32, [vp, vp, vp, u64, vp, u64, u32, u32, C.c_float]),
+    "tf_prefill_rmsnorm_bf16w_block": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32, u32, C.c_float]),
+    "tf_prefill_rmsnorm_bf16w_perhead_block": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, C.c_float]),
+    "tf_prefill_rmsnorm_no_scale_perhead_block": (i32, [vp, vp, vp, u64, vp, u64, u32, u32, u32, u32, C.c_float]),
+    "tf_prefill_rope_default_neox_block": (i32, [vp, vp, vp, u64, u32, u32, u32, u32, u32, C.c_float]),
+    "tf_prefill_rope_proportional_neox_block": (i32, [vp, vp, vp, u64, u32, u32, u32, u32, u32, u32, C.c_float]),
+    "tf_prefill_qkv_epilogue_block": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, u32, u32, u32, C.c_float, u32,
+                                            C.c_float]),
     "tf_attention_swa": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, u32, C.c_float, u32]),
     "tf_attention_full": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, C.c_float]),
     "tf_prefill_attention_causal": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, C.POINTER(PrefillAttentionParams), u32]),

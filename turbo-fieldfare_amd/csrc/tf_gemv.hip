@@ -265,18 +265,20 @@ __global__ __launch_bounds__(256) void gelu_mul_vec_kernel(const half_t *gate, c
     *reinterpret_cast<uint4 *>(out + i) = packed;
 }
 
-__global__ __launch_bounds__(256) void rmsnorm_bf16w_kernel(const half_t *x, const uint16_t *weight, half_t *out, uint32_t d, float eps) {
-    __shared__ float partial[4];
+// One row of RMSNorm by a 256-thread block: out = half(x * inv [* weight]), weight bf16.  In place is fine.
+template <bool WEIGHTED>
+__device__ __forceinline__ void rmsnorm_row_scalar(const half_t *x, const uint16_t *weight, half_t *out, uint32_t d, float eps, float *partial) {
     const float inv = block_rms_inv(x, d, eps, partial);
-    for (uint32_t i = threadIdx.x; i < d; i += blockDim.x)
-        out[i] = (half_t)((float)x[i] * inv * bf16_to_f32(weight[i]));
+    for (uint32_t i = threadIdx.x; i < d; i += blockDim.x) {
+        if constexpr (WEIGHTED) out[i] = (half_t)((float)x[i] * inv * bf16_to_f32(weight[i]));
+        else out[i] = (half_t)((float)x[i] * inv);
+    }
 }
 
 // 16-byte aligned operands, d % 8 == 0, d <= 2048 * PASSES: every thread requests all of its (at most PASSES) 8-element
 // chunks of x and of the weight up front, so the row costs one memory round trip instead of one per element.
-template <int PASSES>
-__global__ __launch_bounds__(256) void rmsnorm_bf16w_vec_kernel(const half_t *x, const uint16_t *weight, half_t *out, uint32_t d, float eps) {
-    __shared__ float partial[4];
+template <int PASSES, bool WEIGHTED>
+__device__ __forceinline__ void rmsnorm_row_vec(const half_t *x, const uint16_t *weight, half_t *out, uint32_t d, float eps, float *partial) {
     u32x4 xr[PASSES], wr[PASSES];
     float acc = 0.0f;
 #pragma unroll
@@ -285,7 +287,7 @@ __global__ __launch_bounds__(256) void rmsnorm_bf16w_vec_kernel(const half_t *x,
         xr[p] = wr[p] = u32x4{0u, 0u, 0u, 0u};
         if (i < d) {
             xr[p] = load16(x + i);
-            wr[p] = load16(weight + i);
+            if constexpr (WEIGHTED) wr[p] = load16(weight + i);
         }
     }
 #pragma unroll
@@ -308,15 +310,39 @@ __global__ __launch_bounds__(256) void rmsnorm_bf16w_vec_kernel(const half_t *x,
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const half2_t h = as_half2(xr[p][j]);
-                const uint32_t wv = wr[p][j];
                 half2_t n;
-                n[0] = (half_t)((float)h[0] * inv * __uint_as_float(wv << 16));
-                n[1] = (half_t)((float)h[1] * inv * __uint_as_float(wv & 0xFFFF0000u));
+                if constexpr (WEIGHTED) {
+                    const uint32_t wv = wr[p][j];
+                    n[0] = (half_t)((float)h[0] * inv * __uint_as_float(wv << 16));
+                    n[1] = (half_t)((float)h[1] * inv * __uint_as_float(wv & 0xFFFF0000u));
+                } else {
+                    n[0] = (half_t)((float)h[0] * inv);
+                    n[1] = (half_t)((float)h[1] * inv);
+                }
                 o[j] = as_u32(n);
             }
             *reinterpret_cast<u32x4 *>(out + i) = o;
         }
     }
+}
+
+// Rows of a block: grid (heads, tokens), row (t, h) = x + t * token_stride + h * d, one shared weight row [d].  PASSES > 0
+// says that d and the weight allow the vector path; a row takes it when its own addresses do, exactly as a single-row call
+// on that row would, so a block of rows equals the rows done one by one, bit for bit.
+template <int PASSES, bool WEIGHTED>
+__global__ __launch_bounds__(256) void rmsnorm_rows_kernel(const half_t *x, const uint16_t *weight, half_t *out, uint32_t d, float eps,
+                                                           uint32_t token_stride) {
+    __shared__ float partial[4];
+    const size_t row = (size_t)blockIdx.y * token_stride + (size_t)blockIdx.x * d;
+    const half_t *xr = x + row;
+    half_t *outr = out + row;
+    if constexpr (PASSES > 0) {
+        if ((reinterpret_cast<uintptr_t>(xr) | reinterpret_cast<uintptr_t>(outr)) % 16 == 0) {
+            rmsnorm_row_vec<PASSES, WEIGHTED>(xr, weight, outr, d, eps, partial);
+            return;
+        }
+    }
+    rmsnorm_row_scalar<WEIGHTED>(xr, weight, outr, d, eps, partial);
 }
 
 template <int BITS>
@@ -397,17 +423,49 @@ int32_t launch_gemv4(tf_ctx *ctx, hipStream_t st, const uint8_t *w, const uint8_
     return launch_gemv4_typed<1, float>(ctx, st, w, s, b, xh, static_cast<float *>(y), m, n, nw, eps);
 }
 
-int32_t launch_rmsnorm_bf16w(tf_ctx *ctx, hipStream_t st, const void *x, const void *w, void *out, uint32_t d, float eps) {
+// weight == nullptr: no scale.  heads x tokens rows of d elements, token rows token_stride elements apart.
+int32_t launch_rmsnorm_rows(tf_ctx *ctx, hipStream_t st, const void *x, const void *w, void *out, uint32_t d, uint32_t heads, uint32_t tokens,
+                            uint32_t token_stride, float eps, const char *who) {
     const half_t *xh = static_cast<const half_t *>(x);
     const uint16_t *wh = static_cast<const uint16_t *>(w);
     half_t *oh = static_cast<half_t *>(out);
-    const bool vec = aligned16(x) && aligned16(w) && aligned16(out) && d % 8 == 0 && d <= 16384;
-    if (vec && d <= 2048) hipLaunchKernelGGL(rmsnorm_bf16w_vec_kernel<1>, dim3(1), dim3(256), 0, st, xh, wh, oh, d, eps);
-    else if (vec && d <= 4096) hipLaunchKernelGGL(rmsnorm_bf16w_vec_kernel<2>, dim3(1), dim3(256), 0, st, xh, wh, oh, d, eps);
-    else if (vec && d <= 8192) hipLaunchKernelGGL(rmsnorm_bf16w_vec_kernel<4>, dim3(1), dim3(256), 0, st, xh, wh, oh, d, eps);
-    else if (vec) hipLaunchKernelGGL(rmsnorm_bf16w_vec_kernel<8>, dim3(1), dim3(256), 0, st, xh, wh, oh, d, eps);
-    else hipLaunchKernelGGL(rmsnorm_bf16w_kernel, dim3(1), dim3(256), 0, st, xh, wh, oh, d, eps);
-    return check_launch(ctx, "rmsnorm_bf16w");
+    const bool vec = (w == nullptr || aligned16(w)) && d % 8 == 0 && d <= 16384;
+    const int passes = !vec ? 0 : d <= 2048 ? 1 : d <= 4096 ? 2 : d <= 8192 ? 4 : 8;
+    const dim3 grid(heads, tokens);
+#define TF_NORM_ROWS(P_)                                                                                                       \
+    case P_:                                                                                                                   \
+        if (w) hipLaunchKernelGGL((rmsnorm_rows_kernel<P_, true>), grid, dim3(256), 0, st, xh, wh, oh, d, eps, token_stride);   \
+        else hipLaunchKernelGGL((rmsnorm_rows_kernel<P_, false>), grid, dim3(256), 0, st, xh, wh, oh, d, eps, token_stride);    \
+        break;
+    switch (passes) {
+        TF_NORM_ROWS(1) TF_NORM_ROWS(2) TF_NORM_ROWS(4) TF_NORM_ROWS(8)
+        default:
+            if (w) hipLaunchKernelGGL((rmsnorm_rows_kernel<0, true>), grid, dim3(256), 0, st, xh, wh, oh, d, eps, token_stride);
+            else hipLaunchKernelGGL((rmsnorm_rows_kernel<0, false>), grid, dim3(256), 0, st, xh, wh, oh, d, eps, token_stride);
+            break;
+    }
+#undef TF_NORM_ROWS
+    return check_launch(ctx, who);
+}
+
+int32_t launch_rmsnorm_bf16w(tf_ctx *ctx, hipStream_t st, const void *x, const void *w, void *out, uint32_t d, float eps) {
+    return launch_rmsnorm_rows(ctx, st, x, w, out, d, 1, 1, 0, eps, "rmsnorm_bf16w");
+}
+
+// argument checks shared by the RMSNorm entry points
+int32_t rmsnorm_rows_entry(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, const void *weight, uint64_t weight_offset, bool weighted,
+                           void *out, uint64_t out_offset, uint32_t d, uint32_t heads, uint32_t tokens, uint32_t token_stride, float eps,
+                           const char *who) {
+    TF_REQUIRE(ctx, ctx && x && out && (!weighted || weight), TF_ERR_INVALID_ARGUMENT, "%s: null argument", who);
+    TF_REQUIRE(ctx, tokens > 0, TF_ERR_INVALID_ARGUMENT, "%s: queryCount must be positive", who);
+    TF_REQUIRE(ctx, d > 0, TF_ERR_INVALID_ARGUMENT, "%s: headDim must be positive", who);
+    TF_REQUIRE(ctx, heads > 0, TF_ERR_INVALID_ARGUMENT, "%s: numHeads must be positive", who);
+    TF_REQUIRE(ctx, tokens == 1 || (uint64_t)token_stride >= (uint64_t)d * heads, TF_ERR_INVALID_ARGUMENT, "%s: token stride is too small", who);
+    TF_REQUIRE(ctx, heads <= 65535 && tokens <= 65535, TF_ERR_INVALID_ARGUMENT, "%s: more than 65535 heads or tokens", who);
+    TF_REQUIRE(ctx, x_offset % 2 == 0 && out_offset % 2 == 0 && (!weighted || weight_offset % 2 == 0), TF_ERR_INVALID_ARGUMENT,
+               "%s: offsets must be 2-byte aligned", who);
+    return launch_rmsnorm_rows(ctx, static_cast<hipStream_t>(stream), at(x, x_offset), weighted ? at(weight, weight_offset) : nullptr,
+                               at(out, out_offset), d, heads, tokens, token_stride, eps, who);
 }
 
 int32_t launch_gelu_mul(tf_ctx *ctx, hipStream_t st, const void *gate, const void *up, void *out, uint32_t count) {
@@ -516,6 +574,42 @@ int32_t tf_rmsnorm_bf16w(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t 
     TF_REQUIRE(ctx, x_offset % 2 == 0 && weight_offset % 2 == 0 && out_offset % 2 == 0, TF_ERR_INVALID_ARGUMENT,
                "rmsnorm_bf16w: offsets must be 2-byte aligned");
     return launch_rmsnorm_bf16w(ctx, static_cast<hipStream_t>(stream), at(x, x_offset), at(weight, weight_offset), at(out, out_offset), d, eps);
+}
+
+int32_t tf_rmsnorm_no_scale(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, void *out, uint64_t out_offset, uint32_t d, float eps) {
+    return rmsnorm_rows_entry(ctx, stream, x, x_offset, nullptr, 0, false, out, out_offset, d, 1, 1, 0, eps, "rmsnorm_no_scale");
+}
+
+int32_t tf_rmsnorm_bf16w_perhead(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, const void *weight, uint64_t weight_offset,
+                                 void *out, uint64_t out_offset, uint32_t head_dim, uint32_t num_heads, float eps) {
+    return rmsnorm_rows_entry(ctx, stream, x, x_offset, weight, weight_offset, true, out, out_offset, head_dim, num_heads, 1, 0, eps,
+                              "rmsnorm_bf16w_perhead");
+}
+
+int32_t tf_rmsnorm_no_scale_perhead(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, void *out, uint64_t out_offset,
+                                    uint32_t head_dim, uint32_t num_heads, float eps) {
+    return rmsnorm_rows_entry(ctx, stream, x, x_offset, nullptr, 0, false, out, out_offset, head_dim, num_heads, 1, 0, eps,
+                              "rmsnorm_no_scale_perhead");
+}
+
+int32_t tf_prefill_rmsnorm_bf16w_block(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, const void *weight, uint64_t weight_offset,
+                                       void *out, uint64_t out_offset, uint32_t tokens, uint32_t d, float eps) {
+    return rmsnorm_rows_entry(ctx, stream, x, x_offset, weight, weight_offset, true, out, out_offset, d, 1, tokens, d, eps,
+                              "prefill_rmsnorm_bf16w_block");
+}
+
+int32_t tf_prefill_rmsnorm_bf16w_perhead_block(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, const void *weight,
+                                               uint64_t weight_offset, void *out, uint64_t out_offset, uint32_t query_count, uint32_t head_dim,
+                                               uint32_t num_heads, uint32_t token_stride_elements, float eps) {
+    return rmsnorm_rows_entry(ctx, stream, x, x_offset, weight, weight_offset, true, out, out_offset, head_dim, num_heads, query_count,
+                              token_stride_elements, eps, "prefill_rmsnorm_bf16w_perhead_block");
+}
+
+int32_t tf_prefill_rmsnorm_no_scale_perhead_block(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, void *out, uint64_t out_offset,
+                                                  uint32_t query_count, uint32_t head_dim, uint32_t num_heads, uint32_t token_stride_elements,
+                                                  float eps) {
+    return rmsnorm_rows_entry(ctx, stream, x, x_offset, nullptr, 0, false, out, out_offset, head_dim, num_heads, query_count,
+                              token_stride_elements, eps, "prefill_rmsnorm_no_scale_perhead_block");
 }
 
 int32_t tf_fused_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *q_weights, uint64_t q_weights_offset, const void *q_scales,

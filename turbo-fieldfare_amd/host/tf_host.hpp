@@ -137,6 +137,97 @@ private:
     const Context &c_;
 };
 
+// RMSNorm (Kernels/Primitives/RMSNorm.swift:52-136)
+class RMSNorm {
+public:
+    explicit RMSNorm(const Context &context) : c_(context) {}
+    void encodeBF16W(const void *x, uint64_t xOffset, const void *weight, uint64_t weightOffset, void *out, uint64_t outOffset, uint32_t d,
+                     float eps) const {
+        c_.check(tf_rmsnorm_bf16w(c_.raw(), c_.stream(), x, xOffset, weight, weightOffset, out, outOffset, d, eps));
+    }
+    void encodeNoScale(const void *x, uint64_t xOffset, void *out, uint64_t outOffset, uint32_t d, float eps) const {
+        c_.check(tf_rmsnorm_no_scale(c_.raw(), c_.stream(), x, xOffset, out, outOffset, d, eps));
+    }
+    void encodeBF16WPerHead(const void *x, uint64_t xOffset, const void *weight, uint64_t weightOffset, void *out, uint64_t outOffset,
+                            uint32_t headDim, uint32_t numHeads, float eps) const {
+        c_.check(tf_rmsnorm_bf16w_perhead(c_.raw(), c_.stream(), x, xOffset, weight, weightOffset, out, outOffset, headDim, numHeads, eps));
+    }
+    void encodeNoScalePerHead(const void *x, uint64_t xOffset, void *out, uint64_t outOffset, uint32_t headDim, uint32_t numHeads, float eps) const {
+        c_.check(tf_rmsnorm_no_scale_perhead(c_.raw(), c_.stream(), x, xOffset, out, outOffset, headDim, numHeads, eps));
+    }
+
+private:
+    const Context &c_;
+};
+
+// PrefillRMSNorm (Kernels/Prefill/Primitives/PrefillPrimitives.swift:41-71)
+class PrefillRMSNorm {
+public:
+    explicit PrefillRMSNorm(const Context &context) : c_(context) {}
+    void encodeBF16W(const void *x, uint64_t xOffset, const void *weight, uint64_t weightOffset, void *out, uint64_t outOffset, uint32_t t,
+                     uint32_t d, float eps) const {
+        c_.check(tf_prefill_rmsnorm_bf16w_block(c_.raw(), c_.stream(), x, xOffset, weight, weightOffset, out, outOffset, t, d, eps));
+    }
+
+private:
+    const Context &c_;
+};
+
+// PrefillPerHeadNorm (Kernels/Prefill/Primitives/PrefillPerHeadNorm.swift:4-85)
+class PrefillPerHeadNorm {
+public:
+    explicit PrefillPerHeadNorm(const Context &context) : c_(context) {}
+    void encodeBF16W(const void *x, uint64_t xOffset, const void *weight, uint64_t weightOffset, void *out, uint64_t outOffset,
+                     uint32_t queryCount, uint32_t headDim, uint32_t numHeads, uint32_t tokenStrideElements, float eps) const {
+        c_.check(tf_prefill_rmsnorm_bf16w_perhead_block(c_.raw(), c_.stream(), x, xOffset, weight, weightOffset, out, outOffset, queryCount, headDim,
+                                                        numHeads, tokenStrideElements, eps));
+    }
+    void encodeNoScale(const void *x, uint64_t xOffset, void *out, uint64_t outOffset, uint32_t queryCount, uint32_t headDim, uint32_t numHeads,
+                       uint32_t tokenStrideElements, float eps) const {
+        c_.check(tf_prefill_rmsnorm_no_scale_perhead_block(c_.raw(), c_.stream(), x, xOffset, out, outOffset, queryCount, headDim, numHeads,
+                                                           tokenStrideElements, eps));
+    }
+
+private:
+    const Context &c_;
+};
+
+// PrefillRoPE (Kernels/Prefill/Primitives/PrefillRoPE.swift:4-89)
+class PrefillRoPE {
+public:
+    explicit PrefillRoPE(const Context &context) : c_(context) {}
+    void encodeDefaultNeox(void *data, uint64_t dataOffset, uint32_t startPosition, uint32_t queryCount, uint32_t headDim, uint32_t numHeads,
+                           uint32_t tokenStrideElements, float theta = 10000.0f) const {
+        c_.check(tf_prefill_rope_default_neox_block(c_.raw(), c_.stream(), data, dataOffset, startPosition, queryCount, headDim, numHeads,
+                                                    tokenStrideElements, theta));
+    }
+    void encodeProportionalNeox(void *data, uint64_t dataOffset, uint32_t startPosition, uint32_t queryCount, uint32_t headDim, uint32_t numHeads,
+                                uint32_t rotatedPairs, uint32_t tokenStrideElements, float theta = 1000000.0f) const {
+        c_.check(tf_prefill_rope_proportional_neox_block(c_.raw(), c_.stream(), data, dataOffset, startPosition, queryCount, headDim, numHeads,
+                                                         rotatedPairs, tokenStrideElements, theta));
+    }
+
+private:
+    const Context &c_;
+};
+
+// PrefillQKVEpilogue (Kernels/Prefill/Epilogues/PrefillQKVEpilogue.swift:4-122)
+class PrefillQKVEpilogue {
+public:
+    explicit PrefillQKVEpilogue(const Context &context) : c_(context) {}
+    void encode(void *q, uint64_t qOffset, void *k, uint64_t kOffset, void *v, uint64_t vOffset, const void *qWeight, uint64_t qWeightOffset,
+                const void *kWeight, uint64_t kWeightOffset, uint32_t startPosition, uint32_t queryCount, uint32_t headDim, uint32_t numQHeads,
+                uint32_t numKVHeads, uint32_t qTokenStrideElements, uint32_t kvTokenStrideElements, float theta, uint32_t rotatedPairs,
+                float eps) const {
+        c_.check(tf_prefill_qkv_epilogue_block(c_.raw(), c_.stream(), q, qOffset, k, kOffset, v, vOffset, qWeight, qWeightOffset, kWeight,
+                                               kWeightOffset, startPosition, queryCount, headDim, numQHeads, numKVHeads, qTokenStrideElements,
+                                               kvTokenStrideElements, theta, rotatedPairs, eps));
+    }
+
+private:
+    const Context &c_;
+};
+
 // FusedQKVEpilogue (Kernels/Fusions/FusedQKVEpilogue.swift:10-100)
 class FusedQKVEpilogue {
 public:
