@@ -239,8 +239,8 @@ int32_t tf_prefill_layer_tail_block(tf_ctx *ctx, tf_stream stream, const void *h
 /* ---- shared expert ------------------------------------------------------------------------------------------- */
 /* SharedExpertInt4.encode (Kernels/MoE/SharedExpertInt4.swift:31-99): gate GEMV, up GEMV (fp16 out),
  * gelu_mul_fp16, down GEMV.  Scratch sizes are in BYTES (the MTLBuffer.length checks at :46-58); each must hold
- * gate.rows halves.  `weight_bits` mirrors SharedExpertRuntime (:102-113): only 4 is built, 8 returns
- * TF_ERR_UNSUPPORTED_BITS (the pinned checkpoint uses the 4-bit shared expert). */
+ * gate.rows halves.  `weight_bits` mirrors SharedExpertRuntime (:96-137): 4 runs this chain, 8 hands over to
+ * tf_shared_expert_int8 (which uses scratch_act only), anything else returns TF_ERR_UNSUPPORTED_BITS. */
 int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream,
                               const void *x, uint64_t x_offset, uint64_t x_length,
                               const tf_projection *gate, const tf_projection *up, const tf_projection *down,
@@ -249,6 +249,21 @@ int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream,
                               void *scratch_up, uint64_t scratch_up_offset, uint64_t scratch_up_length,
                               void *scratch_act, uint64_t scratch_act_offset, uint64_t scratch_act_length,
                               uint32_t weight_bits, tf_dtype scale_dtype);
+/* SharedExpertInt8.encode / encodePhase1 / encodeDown (Kernels/MoE/SharedExpertInt8.swift:67-170) ->
+ * shared_int8_gate_up_act_simd (Metal/Quant/dequant_int8.metal:100-157) then dequant_int8_gemv_simd: 8-bit affine group-64
+ * projections (one byte per weight), act = half(gelu_tanh(half(gate)) * half(up)) into scratch_act (gate.rows halves), then
+ * the down GEMV.  Lengths in bytes; SharedExpertInt8Error.dimensionMismatch -> TF_ERR_DIMENSION_MISMATCH, .scratchTooSmall ->
+ * TF_ERR_SCRATCH_TOO_SMALL. */
+int32_t tf_shared_expert_int8(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, uint64_t x_length,
+                              const tf_projection *gate, const tf_projection *up, const tf_projection *down, void *y,
+                              uint64_t y_offset, uint64_t y_length, void *scratch_act, uint64_t scratch_act_offset,
+                              uint64_t scratch_act_length, tf_dtype scale_dtype);
+int32_t tf_shared_expert_int8_phase1(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, uint64_t x_length,
+                                     const tf_projection *gate, const tf_projection *up, void *scratch_act,
+                                     uint64_t scratch_act_offset, uint64_t scratch_act_length, tf_dtype scale_dtype);
+int32_t tf_shared_expert_int8_down(tf_ctx *ctx, tf_stream stream, const tf_projection *down, void *y, uint64_t y_offset,
+                                   uint64_t y_length, const void *scratch_act, uint64_t scratch_act_offset,
+                                   uint64_t scratch_act_length, tf_dtype scale_dtype);
 
 /* PrefillSharedExpert.encodeBlock (Kernels/Prefill/MoE/PrefillSharedExpert.swift:11-58): the shared expert for
  * query_count rows of x (row stride x_stride_elements halves) into query_count rows of y.  The reference runs the

@@ -234,7 +234,7 @@ def test_shared_expert_production_shape_fused_gate_up():
 def test_shared_expert_errors():
     c = refcases.shared_expert_case()
     assert run_shared(c, weight_bits=3)[0] == tfk.TF_ERR_UNSUPPORTED_BITS        # SharedExpertInt4.swift:110
-    assert run_shared(c, weight_bits=8)[0] == tfk.TF_ERR_UNSUPPORTED_BITS
+    assert run_shared(c, weight_bits=16)[0] == tfk.TF_ERR_UNSUPPORTED_BITS
     assert run_shared(c, scratch_halves=c["f"] - 1)[0] == tfk.TF_ERR_SCRATCH_TOO_SMALL   # :46-50
     bad = dict(c)
     bad["down"] = c["gate"]
@@ -243,6 +243,112 @@ def test_shared_expert_errors():
     x, y, s = dev(c["x_bits"]), zeros_bytes(256), zeros_bytes(128)
     rc = k.shared_expert_int4(x, _proj(*t["gate"], 64, 128), _proj(*t["up"], 64, 128), _proj(*t["gate"], 64, 128), y, s, s, s, raise_on_error=False)
     assert rc == tfk.TF_ERR_DIMENSION_MISMATCH                                    # :41-45
+
+
+# ---------------------------------------------------------------------------------------------------- shared expert, 8-bit
+def _int8_case(d, f, seed):
+    rng = np.random.default_rng(seed)
+    mats = {name: tfo.quantize_int8(rng.uniform(-0.4, 0.4, shape).astype(np.float32))       # SharedExpertInt8Tests.swift:50-60
+            for name, shape in (("gate", (f, d)), ("up", (f, d)), ("down", (d, f)))}
+    return dict(d=d, f=f, x_bits=tfo.to_f16_bits(rng.uniform(-0.4, 0.4, d).astype(np.float32)), **mats)
+
+
+def _gelu64(g):
+    g = g.astype(np.float64)
+    return 0.5 * g * (1.0 + np.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))
+
+
+def _int8_reference(c):
+    # SharedExpertInt8Tests.swift:61-70: the reference GEMVs, the activation rounded through fp16 once, the down GEMV
+    x = tfo.from_f16_bits(c["x_bits"])
+    g, u = tfo.int8_gemv_ref(*c["gate"], x, threads=8), tfo.int8_gemv_ref(*c["up"], x, threads=8)
+    act = tfo.from_f16_bits(tfo.to_f16_bits((_gelu64(g) * u).astype(np.float32)))
+    return g, u, tfo.int8_gemv_ref(*c["down"], act, threads=8)
+
+
+def _run_int8(c, through_runtime, pad=0):
+    k = ctx()
+    d, f = c["d"], c["f"]
+    t = {name: tuple(dev(np.concatenate([np.zeros(pad, np.uint8), np.ascontiguousarray(a).view(np.uint8).ravel()])) for a in c[name])
+         for name in ("gate", "up", "down")}
+    def proj(name, rows, cols):
+        w, s_, b = t[name]
+        return tfk.Projection(w.data_ptr(), pad, s_.data_ptr(), pad, b.data_ptr(), pad, rows, cols)
+    x, y, sa = dev(c["x_bits"]), zeros_bytes(d * 2), zeros_bytes(f * 2)
+    g, u, dn = proj("gate", f, d), proj("up", f, d), proj("down", d, f)
+    import ctypes as C
+    if through_runtime:      # SharedExpertRuntime with weightBits 8: the scratch of gate and up is not used
+        sg = zeros_bytes(2)
+        rc = k.lib.tf_shared_expert_int4(k.handle, None, x.data_ptr(), 0, d * 2, C.byref(g), C.byref(u), C.byref(dn), y.data_ptr(), 0, d * 2,
+                                         sg.data_ptr(), 0, 2, sg.data_ptr(), 0, 2, sa.data_ptr(), 0, f * 2, 8, tfk.TF_BF16)
+    else:
+        rc = k.lib.tf_shared_expert_int8(k.handle, None, x.data_ptr(), 0, d * 2, C.byref(g), C.byref(u), C.byref(dn), y.data_ptr(), 0, d * 2,
+                                         sa.data_ptr(), 0, f * 2, tfk.TF_BF16)
+    return rc, host(y, np.uint16, d), host(sa, np.uint16, f), (t, x, y, sa, g, u, dn)
+
+
+@pytest.mark.parametrize("d,f,pad", [(256, 128, 0), (2816, 2112, 0), (5120, 64, 0), (256, 128, 2)])     # small, production, long rows, unaligned weights
+@pytest.mark.parametrize("through_runtime", [False, True])
+def test_shared_expert_int8_matches_reference(d, f, pad, through_runtime):
+    c = _int8_case(d, f, 0x601 + d + f)
+    rc, y, act, _ = _run_int8(c, through_runtime, pad)
+    assert rc == tfk.TF_OK
+    g_ref, u_ref, y_ref = _int8_reference(c)
+    assert tfo.rel_error(tfo.from_f16_bits(y), y_ref) < tfo.Tolerance.quantInt8 * 4                 # SharedExpertInt8Tests.swift:110
+    # stage boundary: act = gelu_mul_fp16 of the fp16-rounded gate and up sums (dequant_int8.metal:152-156)
+    want_act = tfo.from_f16_bits(tfo.k_gelu_mul_fp16(tfo.to_f16_bits(g_ref), tfo.to_f16_bits(u_ref)))
+    assert np.max(np.abs(tfo.from_f16_bits(act) - want_act)) <= 2e-3 * max(1.0, float(np.max(np.abs(want_act))))
+    assert tfo.rel_error(tfo.from_f16_bits(y), tfo.int8_gemv_ref(*c["down"], tfo.from_f16_bits(act), threads=8)) < tfo.Tolerance.fp16Reduction
+
+
+def test_shared_expert_int8_phases_and_contract():
+    import ctypes as C
+    c = _int8_case(256, 128, 0x602)
+    rc, y, act, (t, x, yb, sa, g, u, dn) = _run_int8(c, False)
+    assert rc == tfk.TF_OK
+    k = ctx()
+    lib, h = k.lib, k.handle
+    d, f = 256, 128
+    # encodePhase1 + encodeDown give what encode gives
+    y2, sa2 = zeros_bytes(d * 2), zeros_bytes(f * 2)
+    k.check(lib.tf_shared_expert_int8_phase1(h, None, x.data_ptr(), 0, d * 2, C.byref(g), C.byref(u), sa2.data_ptr(), 0, f * 2, tfk.TF_BF16))
+    k.check(lib.tf_shared_expert_int8_down(h, None, C.byref(dn), y2.data_ptr(), 0, d * 2, sa2.data_ptr(), 0, f * 2, tfk.TF_BF16))
+    assert np.array_equal(host(y2, np.uint16, d), y) and np.array_equal(host(sa2, np.uint16, f), act)
+    # SharedExpertInt8.swift:75-97
+    assert lib.tf_shared_expert_int8(h, None, x.data_ptr(), 0, d * 2, C.byref(g), C.byref(dn), C.byref(dn), yb.data_ptr(), 0, d * 2,
+                                     sa.data_ptr(), 0, f * 2, tfk.TF_BF16) == tfk.TF_ERR_DIMENSION_MISMATCH        # gate/up shapes differ
+    assert lib.tf_shared_expert_int8(h, None, x.data_ptr(), 0, d * 2, C.byref(g), C.byref(u), C.byref(g), yb.data_ptr(), 0, d * 2,
+                                     sa.data_ptr(), 0, f * 2, tfk.TF_BF16) == tfk.TF_ERR_DIMENSION_MISMATCH        # down is not the transpose shape
+    assert lib.tf_shared_expert_int8(h, None, x.data_ptr(), 0, d * 2, C.byref(g), C.byref(u), C.byref(dn), yb.data_ptr(), 0, d * 2,
+                                     sa.data_ptr(), 0, f * 2 - 2, tfk.TF_BF16) == tfk.TF_ERR_SCRATCH_TOO_SMALL
+    assert lib.tf_shared_expert_int8(h, None, x.data_ptr(), 2, d * 2, C.byref(g), C.byref(u), C.byref(dn), yb.data_ptr(), 0, d * 2,
+                                     sa.data_ptr(), 0, f * 2, tfk.TF_BF16) == tfk.TF_ERR_SCRATCH_TOO_SMALL         # x range exceeds its buffer
+    assert lib.tf_shared_expert_int8(h, None, x.data_ptr(), 0, d * 2, C.byref(g), C.byref(u), C.byref(dn), yb.data_ptr(), 2, d * 2,
+                                     sa.data_ptr(), 0, f * 2, tfk.TF_BF16) == tfk.TF_ERR_SCRATCH_TOO_SMALL         # y range exceeds its buffer
+
+
+def test_prefill_shared_expert_block_with_8_bit_weights_is_the_row_chain():
+    # PrefillSharedExpert(weightBits: 8) (PrefillSharedExpert.swift:7-8): every row through the 8-bit single-row chain
+    import ctypes as C
+    c = _int8_case(256, 128, 0x603)
+    _, _, _, (t, _, _, sa, g, u, dn) = _run_int8(c, False)
+    k = ctx()
+    d, f, rows, stride = 256, 128, 3, 256 + 8
+    rng = np.random.default_rng(0x603)
+    xs = tfo.to_f16_bits(rng.uniform(-0.4, 0.4, rows * stride).astype(np.float32))
+    x, y = dev(xs), dev(np.full(rows * stride, 0x7BFF, np.uint16))
+    sg = zeros_bytes(f * 2)
+    k.check(k.lib.tf_prefill_shared_expert_int4_block(k.handle, None, x.data_ptr(), 0, y.data_ptr(), 0, C.byref(g), C.byref(u), C.byref(dn),
+                                                      sg.data_ptr(), 0, f * 2, sg.data_ptr(), 0, f * 2, sa.data_ptr(), 0, f * 2, rows, d, f,
+                                                      stride, stride, 8, tfk.TF_BF16))
+    got = host(y, np.uint16).reshape(rows, stride)
+    assert np.all(got[:, d:] == 0x7BFF)
+    for r in range(rows):
+        y1 = zeros_bytes(d * 2)
+        k.check(k.lib.tf_shared_expert_int8(k.handle, None, x.data_ptr(), r * stride * 2, (r * stride + d) * 2, C.byref(g), C.byref(u), C.byref(dn),
+                                            y1.data_ptr(), 0, d * 2, sa.data_ptr(), 0, f * 2, tfk.TF_BF16))
+        assert np.array_equal(host(y1, np.uint16, d), got[r, :d])
+
 
 
 # ---------------------------------------------------------------------------------------------------- shared expert, block of rows
@@ -315,7 +421,7 @@ def test_prefill_shared_expert_block_contract():
     assert np.all(run_shared_block(c, 0, 128, 128)[1] == SENTINEL)
     assert run_shared_block(c, 4, 127, 128)[0] == tfk.TF_ERR_INVALID_ARGUMENT     # PrefillSharedExpert.swift:35
     assert run_shared_block(c, 4, 128, 127)[0] == tfk.TF_ERR_INVALID_ARGUMENT     # :36
-    assert run_shared_block(c, 4, 128, 128, weight_bits=8)[0] == tfk.TF_ERR_UNSUPPORTED_BITS
+    assert run_shared_block(c, 4, 128, 128, weight_bits=16)[0] == tfk.TF_ERR_UNSUPPORTED_BITS
     assert run_shared_block(c, 4, 128, 128, scratch_halves=63)[0] == tfk.TF_ERR_SCRATCH_TOO_SMALL
     big = _shared_block_case(16, 128, 64, 7)
     assert run_shared_block(big, 16, 128, 128, scratch_halves=63)[0] == tfk.TF_ERR_SCRATCH_TOO_SMALL

@@ -126,6 +126,10 @@ EXPORTS = {
                                           C.c_float, C.c_float]),
     "tf_shared_expert_int4": (i32, [vp, vp, vp, u64, u64, C.POINTER(Projection), C.POINTER(Projection), C.POINTER(Projection),
                                     vp, u64, u64, vp, u64, u64, vp, u64, u64, vp, u64, u64, u32, i32]),
+    "tf_shared_expert_int8": (i32, [vp, vp, vp, u64, u64, C.POINTER(Projection), C.POINTER(Projection), C.POINTER(Projection), vp, u64, u64,
+                                    vp, u64, u64, i32]),
+    "tf_shared_expert_int8_phase1": (i32, [vp, vp, vp, u64, u64, C.POINTER(Projection), C.POINTER(Projection), vp, u64, u64, i32]),
+    "tf_shared_expert_int8_down": (i32, [vp, vp, C.POINTER(Projection), vp, u64, u64, vp, u64, u64, i32]),
     "tf_prefill_shared_expert_int4_block": (i32, [vp, vp, vp, u64, vp, u64, C.POINTER(Projection), C.POINTER(Projection),
                                                   C.POINTER(Projection), vp, u64, u64, vp, u64, u64, vp, u64, u64, u32, u32, u32,
                                                   u32, u32, u32, i32]),

@@ -386,6 +386,87 @@ int32_t phase1_entry(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *route
     return check_launch(ctx, "moe_phase1_generic");
 }
 
+// ------------------------------------------------------------------------------------------------ shared expert, 8-bit
+// shared_int8_gate_up_act_simd (Metal/Quant/dequant_int8.metal:100-157): one wave per row takes the gate row and the up
+// row against the same activations; act[row] = half(gelu_tanh(float(half(gate))) * float(half(up))).
+__device__ __forceinline__ void int8_chunk(const u32x4 w, const u32x4 xa, const u32x4 xb, float s, float b, float &acc) {
+    float dot = 0.0f, sum = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+        const uint32_t xw = i < 8 ? xa[i >> 1] : xb[(i - 8) >> 1];
+        const float xv = (float)__builtin_bit_cast(half_t, (uint16_t)((i & 1) ? (xw >> 16) : (xw & 0xFFFFu)));
+        const float q = (float)((w[i >> 2] >> (8 * (i & 3))) & 0xFFu);
+        dot = fmaf(q, xv, dot);
+        sum += xv;
+    }
+    acc = fmaf(s, dot, acc);
+    acc = fmaf(b, sum, acc);
+}
+
+// MODE > 0: 16-byte aligned rows and activations, k <= 1024 * MODE: the lane's chunks of both rows are all requested before
+// the first is used.  MODE == 0: aligned, any k.  MODE < 0: any alignment (16-bit loads).
+template <int SD, int MODE>
+__global__ __launch_bounds__(256) void shared8_gate_up_kernel(const uint8_t *gW, const uint8_t *gS, const uint8_t *gB, const uint8_t *uW,
+                                                              const uint8_t *uS, const uint8_t *uB, const half_t *x, half_t *act, uint32_t m, int k) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t row = (blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    if (row >= m) return;
+    const int groups = k >> 6, chunks = k >> 4;
+    const uint8_t *gw = gW + (size_t)row * k, *uw = uW + (size_t)row * k;
+    const uint8_t *gs = gS + (size_t)row * groups * 2, *gb = gB + (size_t)row * groups * 2;
+    const uint8_t *us = uS + (size_t)row * groups * 2, *ub = uB + (size_t)row * groups * 2;
+    float gate = 0.0f, up = 0.0f;
+    if constexpr (MODE > 0) {
+        u32x4 wg[MODE], wu[MODE], xa[MODE], xb[MODE];
+        uint16_t sg[MODE], bg[MODE], su[MODE], bu[MODE];
+#pragma unroll
+        for (int p = 0; p < MODE; ++p) {
+            const int c = lane + 64 * p;
+            wg[p] = wu[p] = xa[p] = xb[p] = u32x4{0u, 0u, 0u, 0u};
+            sg[p] = bg[p] = su[p] = bu[p] = 0;
+            if (c < chunks) {
+                wg[p] = load16(gw + (size_t)c * 16);
+                wu[p] = load16(uw + (size_t)c * 16);
+                xa[p] = load16(x + c * 16);
+                xb[p] = load16(x + c * 16 + 8);
+                sg[p] = *reinterpret_cast<const uint16_t *>(gs + (c >> 2) * 2);
+                bg[p] = *reinterpret_cast<const uint16_t *>(gb + (c >> 2) * 2);
+                su[p] = *reinterpret_cast<const uint16_t *>(us + (c >> 2) * 2);
+                bu[p] = *reinterpret_cast<const uint16_t *>(ub + (c >> 2) * 2);
+            }
+        }
+#pragma unroll
+        for (int p = 0; p < MODE; ++p) {
+            int8_chunk(wg[p], xa[p], xb[p], sb_to_f32<SD>(sg[p]), sb_to_f32<SD>(bg[p]), gate);
+            int8_chunk(wu[p], xa[p], xb[p], sb_to_f32<SD>(su[p]), sb_to_f32<SD>(bu[p]), up);
+        }
+        gate = wave_sum(gate);
+        up = wave_sum(up);
+    } else if constexpr (MODE == 0) {
+        for (int c = lane; c < chunks; c += kWave) {
+            const u32x4 xa = load16(x + c * 16), xb = load16(x + c * 16 + 8);
+            int8_chunk(load16(gw + (size_t)c * 16), xa, xb, sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(gs + (c >> 2) * 2)),
+                       sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(gb + (c >> 2) * 2)), gate);
+            int8_chunk(load16(uw + (size_t)c * 16), xa, xb, sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(us + (c >> 2) * 2)),
+                       sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(ub + (c >> 2) * 2)), up);
+        }
+        gate = wave_sum(gate);
+        up = wave_sum(up);
+    } else {
+        gate = generic_row_dot8<SD>(gw, gs, gb, x, k, lane);
+        up = generic_row_dot8<SD>(uw, us, ub, x, k, lane);
+    }
+    if (lane == 0) {
+        const half_t g16 = (half_t)gate, u16 = (half_t)up;
+        act[row] = (half_t)(gelu_tanh((float)g16) * (float)u16);
+    }
+}
+
+bool projection_ok(const tf_projection *p) {
+    return p->weights && p->scales && p->biases && p->cols % TF_GROUP_SIZE == 0 && p->cols > 0 && p->rows > 0 &&
+           aligned(at(p->scales, p->scales_offset), 2) && aligned(at(p->biases, p->biases_offset), 2);
+}
+
 // Router stage 1: validates the whole router call and writes the logits into the context's scratch.
 int32_t router_logits_entry(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset, const void *scales,
                             uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *hidden,
@@ -539,6 +620,10 @@ int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream, const void *x, uint
                               void *scratch_act, uint64_t scratch_act_offset, uint64_t scratch_act_length, uint32_t weight_bits,
                               tf_dtype scale_dtype) {
     TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "shared_expert: null context");
+    // SharedExpertRuntime (SharedExpertInt4.swift:96-137): 8-bit weights take the 8-bit wrapper, which needs scratchAct only
+    if (weight_bits == 8)
+        return tf_shared_expert_int8(ctx, stream, x, x_offset, x_length, gate, up, down, y, y_offset, y_length, scratch_act, scratch_act_offset,
+                                     scratch_act_length, scale_dtype);
     TF_REQUIRE(ctx, weight_bits == 4, TF_ERR_UNSUPPORTED_BITS, "SharedExpert unsupported weight bits: %u", weight_bits);
     TF_REQUIRE(ctx, x && gate && up && down && y && scratch_gate && scratch_up && scratch_act, TF_ERR_INVALID_ARGUMENT, "shared_expert: null argument");
     TF_REQUIRE(ctx, gate->rows == up->rows && gate->cols == up->cols && down->rows == gate->cols && down->cols == gate->rows,
@@ -606,5 +691,85 @@ int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream, const void *x, uint
     return launch_gemv4(ctx, st, at(down->weights, down->weights_offset), at(down->scales, down->scales_offset),
                         at(down->biases, down->biases_offset), sa, at(y, y_offset), down->rows, down->cols, scale_dtype, TF_FP16);
 }
+
+int32_t tf_shared_expert_int8_phase1(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, uint64_t x_length, const tf_projection *gate,
+                                     const tf_projection *up, void *scratch_act, uint64_t scratch_act_offset, uint64_t scratch_act_length,
+                                     tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "shared_expert_int8: null context");
+    TF_REQUIRE(ctx, x && gate && up && scratch_act, TF_ERR_INVALID_ARGUMENT, "shared_expert_int8: null argument");
+    TF_REQUIRE(ctx, gate->rows == up->rows && gate->cols == up->cols, TF_ERR_DIMENSION_MISMATCH,
+               "SharedExpertInt8 dimension mismatch: gate/up shapes differ: gate=(%u,%u) up=(%u,%u)", gate->rows, gate->cols, up->rows, up->cols);
+    TF_REQUIRE(ctx, scratch_act_offset + (uint64_t)gate->rows * 2 <= scratch_act_length, TF_ERR_SCRATCH_TOO_SMALL,
+               "SharedExpertInt8 scratch too small: scratchAct offset %llu + needed %llu exceeds length %llu", (unsigned long long)scratch_act_offset,
+               (unsigned long long)gate->rows * 2, (unsigned long long)scratch_act_length);
+    TF_REQUIRE(ctx, x_offset + (uint64_t)gate->cols * 2 <= x_length, TF_ERR_SCRATCH_TOO_SMALL,
+               "SharedExpertInt8 scratch too small: x offset %llu + needed %llu exceeds length %llu", (unsigned long long)x_offset,
+               (unsigned long long)gate->cols * 2, (unsigned long long)x_length);
+    TF_REQUIRE(ctx, projection_ok(gate) && projection_ok(up), TF_ERR_INVALID_ARGUMENT,
+               "shared_expert_int8: a projection needs its three buffers, 2-byte aligned scales and biases, and N a multiple of 64");
+    TF_REQUIRE(ctx, scale_dtype == TF_BF16 || scale_dtype == TF_FP16, TF_ERR_INVALID_ARGUMENT, "shared_expert_int8: scale dtype must be bf16 or fp16");
+    TF_REQUIRE(ctx, x_offset % 2 == 0 && scratch_act_offset % 2 == 0, TF_ERR_INVALID_ARGUMENT, "shared_expert_int8: offsets must be 2-byte aligned");
+    const uint8_t *gw = at(gate->weights, gate->weights_offset), *uw = at(up->weights, up->weights_offset);
+    const uint8_t *gs = at(gate->scales, gate->scales_offset), *gb = at(gate->biases, gate->biases_offset);
+    const uint8_t *us = at(up->scales, up->scales_offset), *ub = at(up->biases, up->biases_offset);
+    const half_t *xp = reinterpret_cast<const half_t *>(at(x, x_offset));
+    half_t *act = reinterpret_cast<half_t *>(at(scratch_act, scratch_act_offset));
+    const uint32_t m = gate->rows, k = gate->cols;
+    const bool fast = aligned16(gw) && aligned16(uw) && aligned16(xp);   // k % 64 == 0 keeps every row aligned
+    const int mode = !fast ? -1 : k <= 1024 ? 1 : k <= 2048 ? 2 : k <= 3072 ? 3 : k <= 4096 ? 4 : 0;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 grid((m + 3) / 4);
+#define TF_SH8(MODE_)                                                                                                                  \
+    case MODE_:                                                                                                                        \
+        if (scale_dtype == TF_BF16)                                                                                                    \
+            hipLaunchKernelGGL((shared8_gate_up_kernel<0, MODE_>), grid, dim3(256), 0, st, gw, gs, gb, uw, us, ub, xp, act, m, (int)k); \
+        else                                                                                                                           \
+            hipLaunchKernelGGL((shared8_gate_up_kernel<1, MODE_>), grid, dim3(256), 0, st, gw, gs, gb, uw, us, ub, xp, act, m, (int)k); \
+        break;
+    switch (mode) {
+        TF_SH8(1) TF_SH8(2) TF_SH8(3) TF_SH8(4) TF_SH8(0)
+        default:
+            if (scale_dtype == TF_BF16)
+                hipLaunchKernelGGL((shared8_gate_up_kernel<0, -1>), grid, dim3(256), 0, st, gw, gs, gb, uw, us, ub, xp, act, m, (int)k);
+            else
+                hipLaunchKernelGGL((shared8_gate_up_kernel<1, -1>), grid, dim3(256), 0, st, gw, gs, gb, uw, us, ub, xp, act, m, (int)k);
+            break;
+    }
+#undef TF_SH8
+    return check_launch(ctx, "shared_int8_gate_up_act");
+}
+
+int32_t tf_shared_expert_int8_down(tf_ctx *ctx, tf_stream stream, const tf_projection *down, void *y, uint64_t y_offset, uint64_t y_length,
+                                   const void *scratch_act, uint64_t scratch_act_offset, uint64_t scratch_act_length, tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "shared_expert_int8: null context");
+    TF_REQUIRE(ctx, down && y && scratch_act, TF_ERR_INVALID_ARGUMENT, "shared_expert_int8: null argument");
+    TF_REQUIRE(ctx, scratch_act_offset + (uint64_t)down->cols * 2 <= scratch_act_length, TF_ERR_SCRATCH_TOO_SMALL,
+               "SharedExpertInt8 scratch too small: scratchAct offset %llu + needed %llu exceeds length %llu", (unsigned long long)scratch_act_offset,
+               (unsigned long long)down->cols * 2, (unsigned long long)scratch_act_length);
+    TF_REQUIRE(ctx, y_offset + (uint64_t)down->rows * 2 <= y_length, TF_ERR_SCRATCH_TOO_SMALL,
+               "SharedExpertInt8 scratch too small: y offset %llu + needed %llu exceeds length %llu", (unsigned long long)y_offset,
+               (unsigned long long)down->rows * 2, (unsigned long long)y_length);
+    return tf_dequant_int8_gemv(ctx, stream, down->weights, down->weights_offset, down->scales, down->scales_offset, down->biases,
+                                down->biases_offset, scratch_act, scratch_act_offset, y, y_offset, down->rows, down->cols, scale_dtype, TF_FP16);
+}
+
+int32_t tf_shared_expert_int8(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, uint64_t x_length, const tf_projection *gate,
+                              const tf_projection *up, const tf_projection *down, void *y, uint64_t y_offset, uint64_t y_length,
+                              void *scratch_act, uint64_t scratch_act_offset, uint64_t scratch_act_length, tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "shared_expert_int8: null context");
+    TF_REQUIRE(ctx, x && gate && up && down && y && scratch_act, TF_ERR_INVALID_ARGUMENT, "shared_expert_int8: null argument");
+    TF_REQUIRE(ctx, gate->rows == up->rows && gate->cols == up->cols, TF_ERR_DIMENSION_MISMATCH,
+               "SharedExpertInt8 dimension mismatch: gate/up shapes differ: gate=(%u,%u) up=(%u,%u)", gate->rows, gate->cols, up->rows, up->cols);
+    TF_REQUIRE(ctx, down->rows == gate->cols && down->cols == gate->rows, TF_ERR_DIMENSION_MISMATCH,
+               "SharedExpertInt8 dimension mismatch: down expected (%u,%u), got (%u,%u)", gate->cols, gate->rows, down->rows, down->cols);
+    TF_REQUIRE(ctx, y_offset + (uint64_t)down->rows * 2 <= y_length, TF_ERR_SCRATCH_TOO_SMALL,
+               "SharedExpertInt8 scratch too small: y offset %llu + needed %llu exceeds length %llu", (unsigned long long)y_offset,
+               (unsigned long long)down->rows * 2, (unsigned long long)y_length);
+    const int32_t rc = tf_shared_expert_int8_phase1(ctx, stream, x, x_offset, x_length, gate, up, scratch_act, scratch_act_offset,
+                                                    scratch_act_length, scale_dtype);
+    if (rc != TF_OK) return rc;
+    return tf_shared_expert_int8_down(ctx, stream, down, y, y_offset, y_length, scratch_act, scratch_act_offset, scratch_act_length, scale_dtype);
+}
+
 
 }  // extern "C"

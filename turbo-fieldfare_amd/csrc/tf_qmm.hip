@@ -422,7 +422,7 @@ int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream, const
                                             uint32_t intermediate, uint32_t x_stride_elements, uint32_t y_stride_elements,
                                             uint32_t weight_bits, tf_dtype scale_dtype) {
     TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "prefill_shared_expert: null context");
-    TF_REQUIRE(ctx, weight_bits == 4, TF_ERR_UNSUPPORTED_BITS, "SharedExpert unsupported weight bits: %u", weight_bits);
+    TF_REQUIRE(ctx, weight_bits == 4 || weight_bits == 8, TF_ERR_UNSUPPORTED_BITS, "SharedExpert unsupported weight bits: %u", weight_bits);
     TF_REQUIRE(ctx, x && y && gate && up && down && scratch_gate && scratch_up && scratch_act, TF_ERR_INVALID_ARGUMENT,
                "prefill_shared_expert: null argument");
     TF_REQUIRE(ctx, d > 0, TF_ERR_INVALID_ARGUMENT, "prefill_shared_expert: d must be positive");
@@ -442,7 +442,7 @@ int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream, const
                           down->scales && down->biases;
     const bool even = x_offset % 2 == 0 && y_offset % 2 == 0 && gate->scales_offset % 2 == 0 && gate->biases_offset % 2 == 0 &&
                       up->scales_offset % 2 == 0 && up->biases_offset % 2 == 0 && down->scales_offset % 2 == 0 && down->biases_offset % 2 == 0;
-    const bool block_path = pointers && even && query_count >= kSharedBlockMinRows && (scale_dtype == TF_BF16 || scale_dtype == TF_FP16) &&
+    const bool block_path = weight_bits == 4 && pointers && even && query_count >= kSharedBlockMinRows && (scale_dtype == TF_BF16 || scale_dtype == TF_FP16) &&
                             qmm_operands_ok(gw, xp, x_stride_elements, (int)d) && aligned16(uw) && aligned16(dw) &&
                             intermediate % TF_GROUP_SIZE == 0 && query_count <= (uint32_t)INT32_MAX;
     if (!block_path) {

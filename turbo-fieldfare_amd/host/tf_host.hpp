@@ -286,11 +286,12 @@ private:
 
 using SharedExpertProjection = tf_projection;   // Kernels/MoE/SharedExpertInt8.swift:9-31
 
-// SharedExpertRuntime / SharedExpertInt4 (Kernels/MoE/SharedExpertInt4.swift)
+// SharedExpertRuntime / SharedExpertInt4 (Kernels/MoE/SharedExpertInt4.swift): 4- or 8-bit projections
 class SharedExpertRuntime {
 public:
     SharedExpertRuntime(const Context &context, int weightBits) : c_(context), weightBits_(weightBits) {
-        if (weightBits != 4) throw Error(TF_ERR_UNSUPPORTED_BITS, "SharedExpert unsupported weight bits: " + std::to_string(weightBits));
+        if (weightBits != 4 && weightBits != 8)
+            throw Error(TF_ERR_UNSUPPORTED_BITS, "SharedExpert unsupported weight bits: " + std::to_string(weightBits));
     }
     struct Buffer {   // an MTLBuffer's (contents, length)
         void *ptr;
@@ -313,8 +314,9 @@ private:
 // PrefillSharedExpert (Kernels/Prefill/MoE/PrefillSharedExpert.swift:4-58): the shared expert over a block of rows
 class PrefillSharedExpert {
 public:
-    PrefillSharedExpert(const Context &context, int weightBits = 4) : c_(context), weightBits_(weightBits) {
-        if (weightBits != 4) throw Error(TF_ERR_UNSUPPORTED_BITS, "SharedExpert unsupported weight bits: " + std::to_string(weightBits));
+    PrefillSharedExpert(const Context &context, int weightBits = 8) : c_(context), weightBits_(weightBits) {
+        if (weightBits != 4 && weightBits != 8)
+            throw Error(TF_ERR_UNSUPPORTED_BITS, "SharedExpert unsupported weight bits: " + std::to_string(weightBits));
     }
     using Buffer = SharedExpertRuntime::Buffer;
     void encodeBlock(const void *x, uint64_t xOffset, void *y, uint64_t yOffset, const SharedExpertProjection &gate,
@@ -330,6 +332,30 @@ public:
 private:
     const Context &c_;
     int weightBits_;
+};
+
+// SharedExpertInt8 (Kernels/MoE/SharedExpertInt8.swift:54-170): gate, up and the activation in one launch, then the down GEMV
+class SharedExpertInt8 {
+public:
+    explicit SharedExpertInt8(const Context &context) : c_(context) {}
+    using Buffer = SharedExpertRuntime::Buffer;
+    void encode(Buffer x, uint64_t xOffset, const SharedExpertProjection &gate, const SharedExpertProjection &up,
+                const SharedExpertProjection &down, Buffer y, uint64_t yOffset, Buffer scratchAct, uint64_t scratchActOffset) const {
+        c_.check(tf_shared_expert_int8(c_.raw(), c_.stream(), x.ptr, xOffset, x.length, &gate, &up, &down, y.ptr, yOffset, y.length,
+                                       scratchAct.ptr, scratchActOffset, scratchAct.length, TF_BF16));
+    }
+    void encodePhase1(Buffer x, uint64_t xOffset, const SharedExpertProjection &gate, const SharedExpertProjection &up, Buffer scratchAct,
+                      uint64_t scratchActOffset) const {
+        c_.check(tf_shared_expert_int8_phase1(c_.raw(), c_.stream(), x.ptr, xOffset, x.length, &gate, &up, scratchAct.ptr, scratchActOffset,
+                                              scratchAct.length, TF_BF16));
+    }
+    void encodeDown(const SharedExpertProjection &down, Buffer y, uint64_t yOffset, Buffer scratchAct, uint64_t scratchActOffset) const {
+        c_.check(tf_shared_expert_int8_down(c_.raw(), c_.stream(), &down, y.ptr, yOffset, y.length, scratchAct.ptr, scratchActOffset,
+                                            scratchAct.length, TF_BF16));
+    }
+
+private:
+    const Context &c_;
 };
 
 // SharedExpertInt4 (Kernels/MoE/SharedExpertInt4.swift:6-100) is the 4-bit instance of the runtime.
