@@ -390,6 +390,27 @@ def extras(torch, tfk, k, gen, lib, h, stream):
     us = time_loop(torch, shared, 300, warmup=20)
     res["shared_expert_int4"] = {"us_per_call": round(us, 3), "GBps": round(SHARED_BYTES / (us * 1e-6) / 1e9, 1),
                                  "algorithmic_bytes": SHARED_BYTES}
+
+    # the same chain with 8-bit projections (one byte per weight), rotating over 32 replicas of each matrix
+    r8 = 32
+    def int8_matrix(rows, cols):
+        return (torch.randint(0, 256, (rows, cols), dtype=torch.uint8, device="cuda", generator=gen),
+                bf16_bits_cuda(torch.rand((rows, cols // 64), device="cuda", generator=gen) * 0.0012 + 0.0004),
+                bf16_bits_cuda(torch.rand((rows, cols // 64), device="cuda", generator=gen) * 0.2 - 0.2))
+    g8, u8, d8 = int8_matrix(r8 * F_SHARED, D), int8_matrix(r8 * F_SHARED, D), int8_matrix(r8 * D, F_SHARED)
+
+    def shared8(i):
+        r = i % r8
+        def proj(m, first, rows, cols):
+            return tfk.Projection(m[0].data_ptr(), first * cols, m[1].data_ptr(), first * (cols // 64) * 2, m[2].data_ptr(), first * (cols // 64) * 2,
+                                  rows, cols)
+        g, u, dn = proj(g8, r * F_SHARED, F_SHARED, D), proj(u8, r * F_SHARED, F_SHARED, D), proj(d8, r * D, D, F_SHARED)
+        rc = lib.tf_shared_expert_int8(h, stream, xs.data_ptr(), (i % 8) * D * 2, 8 * D * 2, C.byref(g), C.byref(u), C.byref(dn), ys.data_ptr(), 0,
+                                       D * 2, sa.data_ptr(), 0, F_SHARED * 2, tfk.TF_BF16)
+        assert rc == 0, k.last_error()
+    us = time_loop(torch, shared8, 200, warmup=20)
+    bytes8 = 3 * (F_SHARED * D + 2 * F_SHARED * (D // 64) * 2) + 2 * D * 2 + 2 * F_SHARED * 2
+    res["shared_expert_int8"] = {"us_per_call": round(us, 3), "GBps": round(bytes8 / (us * 1e-6) / 1e9, 1), "algorithmic_bytes": bytes8}
     return res
 
 

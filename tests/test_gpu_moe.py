@@ -327,13 +327,15 @@ def test_shared_expert_int8_phases_and_contract():
                                      sa.data_ptr(), 0, f * 2, tfk.TF_BF16) == tfk.TF_ERR_SCRATCH_TOO_SMALL         # y range exceeds its buffer
 
 
-def test_prefill_shared_expert_block_with_8_bit_weights_is_the_row_chain():
-    # PrefillSharedExpert(weightBits: 8) (PrefillSharedExpert.swift:7-8): every row through the 8-bit single-row chain
+@pytest.mark.parametrize("d,f,rows,pad", [(256, 128, 3, 8), (2816, 2112, 37, 0), (256, 128, 5, 3), (1024, 64, 1, 0)])
+def test_prefill_shared_expert_block_with_8_bit_weights_is_the_row_chain(d, f, rows, pad):
+    # PrefillSharedExpert(weightBits: 8) (PrefillSharedExpert.swift:7-8): every row as the 8-bit single-row chain leaves it, bit
+    # for bit - rows in groups against each weight row where the operands are aligned, one by one otherwise (odd stride, one row)
     import ctypes as C
-    c = _int8_case(256, 128, 0x603)
+    c = _int8_case(d, f, 0x603 + d)
     _, _, _, (t, _, _, sa, g, u, dn) = _run_int8(c, False)
     k = ctx()
-    d, f, rows, stride = 256, 128, 3, 256 + 8
+    stride = d + pad
     rng = np.random.default_rng(0x603)
     xs = tfo.to_f16_bits(rng.uniform(-0.4, 0.4, rows * stride).astype(np.float32))
     x, y = dev(xs), dev(np.full(rows * stride, 0x7BFF, np.uint16))

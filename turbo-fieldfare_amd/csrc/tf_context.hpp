@@ -61,6 +61,12 @@ inline uint8_t *at(void *base, uint64_t off) { return static_cast<uint8_t *>(bas
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline bool aligned(const void *p, unsigned a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1u)) == 0; }
 
+// The 8-bit shared expert over a block of rows (tf_moe.hip), for the block entry of the shared expert (tf_qmm.hip): two
+// launches, every row bit-identical to the single-row chain.  acts: [rows, intermediate] fp16 scratch.  TF_ERR_UNAVAILABLE when
+// the operands do not allow it (alignment, K > 4096): the caller runs the rows one by one.
+int32_t shared8_block(tf_ctx *ctx, hipStream_t st, const tf_projection *gate, const tf_projection *up, const tf_projection *down, const void *x,
+                      uint32_t x_stride_elements, void *y, uint32_t y_stride_elements, uint32_t rows, void *acts, tf_dtype scale_dtype);
+
 }  // namespace tfk
 
 #define TF_REQUIRE(ctx, cond, status, ...) \

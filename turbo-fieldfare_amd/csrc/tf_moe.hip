@@ -462,6 +462,108 @@ __global__ __launch_bounds__(256) void shared8_gate_up_kernel(const uint8_t *gW,
     }
 }
 
+// A block of rows: a wave takes one weight row (gate and up, or one down row) against kSharedRows activation rows at a time,
+// with the chunk assignment and the order of operations of the single-row kernels, so every row comes out as the single-row
+// chain leaves it, bit for bit, while a weight row is fetched once per kSharedRows rows instead of once per row.
+constexpr int kSharedRows = 4;
+
+// gate / up + activation: acts[t, row]; x rows x_stride elements apart
+template <int SD, int NPASS>
+__global__ __launch_bounds__(256) void shared8_gate_up_rows_kernel(const uint8_t *gW, const uint8_t *gS, const uint8_t *gB, const uint8_t *uW,
+                                                                   const uint8_t *uS, const uint8_t *uB, const half_t *x, uint32_t x_stride,
+                                                                   half_t *acts, uint32_t m, int k, uint32_t tokens) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t row = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, t0 = blockIdx.y * kSharedRows;
+    if (row >= m) return;
+    const int groups = k >> 6, chunks = k >> 4;
+    u32x4 wg[NPASS], wu[NPASS], xa[kSharedRows][NPASS], xb[kSharedRows][NPASS];
+    float sg[NPASS], bg[NPASS], su[NPASS], bu[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+        const int c = lane + 64 * p;
+        wg[p] = wu[p] = u32x4{0u, 0u, 0u, 0u};
+        uint16_t s0 = 0, b0 = 0, s1 = 0, b1 = 0;
+        if (c < chunks) {
+            wg[p] = load16(gW + (size_t)row * k + (size_t)c * 16);
+            wu[p] = load16(uW + (size_t)row * k + (size_t)c * 16);
+            s0 = *reinterpret_cast<const uint16_t *>(gS + ((size_t)row * groups + (c >> 2)) * 2);
+            b0 = *reinterpret_cast<const uint16_t *>(gB + ((size_t)row * groups + (c >> 2)) * 2);
+            s1 = *reinterpret_cast<const uint16_t *>(uS + ((size_t)row * groups + (c >> 2)) * 2);
+            b1 = *reinterpret_cast<const uint16_t *>(uB + ((size_t)row * groups + (c >> 2)) * 2);
+        }
+        sg[p] = sb_to_f32<SD>(s0);
+        bg[p] = sb_to_f32<SD>(b0);
+        su[p] = sb_to_f32<SD>(s1);
+        bu[p] = sb_to_f32<SD>(b1);
+#pragma unroll
+        for (int t = 0; t < kSharedRows; ++t) {
+            xa[t][p] = xb[t][p] = u32x4{0u, 0u, 0u, 0u};
+            if (c < chunks && t0 + t < tokens) {
+                const half_t *xr = x + (size_t)(t0 + t) * x_stride + c * 16;
+                xa[t][p] = load16(xr);
+                xb[t][p] = load16(xr + 8);
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < kSharedRows; ++t) {
+        float gate = 0.0f, up = 0.0f;
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p) {
+            int8_chunk(wg[p], xa[t][p], xb[t][p], sg[p], bg[p], gate);
+            int8_chunk(wu[p], xa[t][p], xb[t][p], su[p], bu[p], up);
+        }
+        gate = wave_sum(gate);
+        up = wave_sum(up);
+        if (lane == 0 && t0 + t < tokens) {
+            const half_t g16 = (half_t)gate, u16 = (half_t)up;
+            acts[(size_t)(t0 + t) * m + row] = (half_t)(gelu_tanh((float)g16) * (float)u16);
+        }
+    }
+}
+
+// down: y[t, row] = half(W[row, :] . acts[t, :]); acts rows k elements apart, y rows y_stride apart
+template <int SD, int NPASS>
+__global__ __launch_bounds__(256) void gemv8_rows_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *acts, half_t *y,
+                                                         uint32_t y_stride, uint32_t m, int k, uint32_t tokens) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t row = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, t0 = blockIdx.y * kSharedRows;
+    if (row >= m) return;
+    const int groups = k >> 6, chunks = k >> 4;
+    u32x4 w[NPASS], xa[kSharedRows][NPASS], xb[kSharedRows][NPASS];
+    float sv[NPASS], bv[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+        const int c = lane + 64 * p;
+        w[p] = u32x4{0u, 0u, 0u, 0u};
+        uint16_t s0 = 0, b0 = 0;
+        if (c < chunks) {
+            w[p] = load16(W + (size_t)row * k + (size_t)c * 16);
+            s0 = *reinterpret_cast<const uint16_t *>(S + ((size_t)row * groups + (c >> 2)) * 2);
+            b0 = *reinterpret_cast<const uint16_t *>(B + ((size_t)row * groups + (c >> 2)) * 2);
+        }
+        sv[p] = sb_to_f32<SD>(s0);
+        bv[p] = sb_to_f32<SD>(b0);
+#pragma unroll
+        for (int t = 0; t < kSharedRows; ++t) {
+            xa[t][p] = xb[t][p] = u32x4{0u, 0u, 0u, 0u};
+            if (c < chunks && t0 + t < tokens) {
+                const half_t *xr = acts + (size_t)(t0 + t) * k + c * 16;
+                xa[t][p] = load16(xr);
+                xb[t][p] = load16(xr + 8);
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < kSharedRows; ++t) {
+        float acc = 0.0f;
+#pragma unroll
+        for (int p = 0; p < NPASS; ++p) int8_chunk(w[p], xa[t][p], xb[t][p], sv[p], bv[p], acc);
+        acc = wave_sum(acc);
+        if (lane == 0 && t0 + t < tokens) y[(size_t)(t0 + t) * y_stride + row] = (half_t)acc;
+    }
+}
+
 bool projection_ok(const tf_projection *p) {
     return p->weights && p->scales && p->biases && p->cols % TF_GROUP_SIZE == 0 && p->cols > 0 && p->rows > 0 &&
            aligned(at(p->scales, p->scales_offset), 2) && aligned(at(p->biases, p->biases_offset), 2);
@@ -514,6 +616,52 @@ int32_t router_select_entry(tf_ctx *ctx, tf_stream stream, const void *per_exper
 }
 
 }  // namespace
+
+namespace tfk {
+
+int32_t shared8_block(tf_ctx *ctx, hipStream_t st, const tf_projection *gate, const tf_projection *up, const tf_projection *down, const void *x,
+                      uint32_t x_stride_elements, void *y, uint32_t y_stride_elements, uint32_t rows, void *acts, tf_dtype scale_dtype) {
+    const uint32_t f = gate->rows, d = gate->cols;
+    const uint8_t *gw = at(gate->weights, gate->weights_offset), *uw = at(up->weights, up->weights_offset);
+    const uint8_t *dw = at(down->weights, down->weights_offset);
+    // every chunk of every row 16-byte aligned: the single-row kernels then take the same (vector) path row by row
+    const bool ok = projection_ok(gate) && projection_ok(up) && projection_ok(down) && aligned16(gw) && aligned16(uw) && aligned16(dw) &&
+                    aligned16(x) && aligned16(acts) && x_stride_elements % 8 == 0 && d <= 4096 && f <= 4096 && rows <= 65535 * (uint32_t)kSharedRows &&
+                    (scale_dtype == TF_BF16 || scale_dtype == TF_FP16);
+    if (!ok) return TF_ERR_UNAVAILABLE;
+    const uint8_t *gs = at(gate->scales, gate->scales_offset), *gb = at(gate->biases, gate->biases_offset);
+    const uint8_t *us = at(up->scales, up->scales_offset), *ub = at(up->biases, up->biases_offset);
+    const uint8_t *ds = at(down->scales, down->scales_offset), *db = at(down->biases, down->biases_offset);
+    const half_t *xp = static_cast<const half_t *>(x);
+    half_t *ap = static_cast<half_t *>(acts), *yp = static_cast<half_t *>(y);
+    const uint32_t groups_of_rows = (rows + kSharedRows - 1) / kSharedRows;
+    const int sd = scale_dtype == TF_BF16 ? 0 : 1;
+#define TF_SH8_ROWS(SD_, NP_)                                                                                                          \
+    hipLaunchKernelGGL((shared8_gate_up_rows_kernel<SD_, NP_>), dim3((f + 3) / 4, groups_of_rows), dim3(256), 0, st, gw, gs, gb, uw, us, ub, xp, \
+                       x_stride_elements, ap, f, (int)d, rows)
+#define TF_GEMV8_ROWS(SD_, NP_)                                                                                                        \
+    hipLaunchKernelGGL((gemv8_rows_kernel<SD_, NP_>), dim3((d + 3) / 4, groups_of_rows), dim3(256), 0, st, dw, ds, db, ap, yp,         \
+                       y_stride_elements, d, (int)f, rows)
+#define TF_PICK(MACRO_, K_)                                                                                                            \
+    do {                                                                                                                               \
+        const int np = ((K_) + 1023) / 1024;                                                                                           \
+        if (sd == 0) {                                                                                                                 \
+            if (np == 1) MACRO_(0, 1); else if (np == 2) MACRO_(0, 2); else if (np == 3) MACRO_(0, 3); else MACRO_(0, 4);              \
+        } else {                                                                                                                       \
+            if (np == 1) MACRO_(1, 1); else if (np == 2) MACRO_(1, 2); else if (np == 3) MACRO_(1, 3); else MACRO_(1, 4);              \
+        }                                                                                                                              \
+    } while (0)
+    TF_PICK(TF_SH8_ROWS, d);
+    int32_t rc = check_launch(ctx, "shared_int8_gate_up_act rows");
+    if (rc != TF_OK) return rc;
+    TF_PICK(TF_GEMV8_ROWS, f);
+#undef TF_PICK
+#undef TF_GEMV8_ROWS
+#undef TF_SH8_ROWS
+    return check_launch(ctx, "int8 gemv rows");
+}
+
+}  // namespace tfk
 
 extern "C" {
 

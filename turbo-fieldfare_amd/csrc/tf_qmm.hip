@@ -445,6 +445,17 @@ int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream, const
     const bool block_path = weight_bits == 4 && pointers && even && query_count >= kSharedBlockMinRows && (scale_dtype == TF_BF16 || scale_dtype == TF_FP16) &&
                             qmm_operands_ok(gw, xp, x_stride_elements, (int)d) && aligned16(uw) && aligned16(dw) &&
                             intermediate % TF_GROUP_SIZE == 0 && query_count <= (uint32_t)INT32_MAX;
+    if (weight_bits == 8 && pointers && even && query_count >= 2) {
+        // 8-bit projections: rows in groups against each weight row, bit-identical to the rows one by one
+        TF_REQUIRE(ctx, scratch_act_offset + (uint64_t)intermediate * 2 <= scratch_act_length, TF_ERR_SCRATCH_TOO_SMALL,
+                   "SharedExpertInt8 scratch too small: scratchAct offset %llu + needed %llu exceeds length %llu",
+                   (unsigned long long)scratch_act_offset, (unsigned long long)intermediate * 2, (unsigned long long)scratch_act_length);
+        half_t *acts8 = nullptr;
+        int32_t rc8 = shared_block_acts(ctx, (size_t)query_count * intermediate, acts8);
+        if (rc8 != TF_OK) return rc8;
+        rc8 = shared8_block(ctx, st, gate, up, down, xp, x_stride_elements, yp, y_stride_elements, query_count, acts8, scale_dtype);
+        if (rc8 != TF_ERR_UNAVAILABLE) return rc8;
+    }
     if (!block_path) {
         // PrefillSharedExpert.encodeBlock itself: the single-row chain once per row, every row through the same scratch
         for (uint32_t row = 0; row < query_count; ++row) {
