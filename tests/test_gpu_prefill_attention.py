@@ -103,6 +103,35 @@ def test_block_equals_decode_attention_row_by_row():
     assert np.max(np.abs(single - tfo.from_f16_bits(rows[t, :16 * 256]))) <= 2e-3
 
 
+@pytest.mark.parametrize("start,count,window,hd,hq,hkv", [(32640, 128, 0, 512, 16, 2),       # a global layer at the end of a 32768-token context
+                                                          (8000, 128, 1024, 256, 16, 8)])   # a sliding-window layer deep into the context
+def test_full_context_sizes_through_the_identical_keys_property(start, count, window, hd, hq, hkv):
+    # every key row identical: all visible positions weigh the same whatever the queries are, so query t must return the mean
+    # of the V rows it sees - a closed form that needs no O(N^2) reference at these sizes
+    import torch
+    rng = np.random.default_rng(0xC0DE + hd)
+    kv_valid = start + count
+    key = rng.standard_normal(hkv * hd).astype(np.float16) * np.float16(0.25)
+    k_rows = np.broadcast_to(key, (kv_valid, hkv * hd)).copy()
+    v_rows = rng.standard_normal((kv_valid, hkv * hd)).astype(np.float16)
+    q_rows = (rng.standard_normal((count, hq * hd)) * 0.25).astype(np.float16)
+    kk = ctx()
+    d_q, d_k, d_v = dev(q_rows.view(np.uint16).ravel()), dev(k_rows.view(np.uint16).ravel()), dev(v_rows.view(np.uint16).ravel())
+    out = dev(np.zeros(count * hq * hd, np.uint16))
+    p = tfk.PrefillAttentionParams(start, count, hd, hq, hkv, kv_valid, window, hkv * hd, hq * hd, hq * hd, 1.0 / np.sqrt(hd))
+    import ctypes as C
+    kk.check(kk.lib.tf_prefill_attention_causal(kk.handle, None, d_q.data_ptr(), 0, d_k.data_ptr(), 0, d_v.data_ptr(), 0, out.data_ptr(), 0, C.byref(p), 0))
+    got = tfo.from_f16_bits(host(out, np.uint16)).reshape(count, hq, hd)
+    prefix = np.concatenate([np.zeros((1, hkv * hd)), np.cumsum(v_rows.astype(np.float64), axis=0)])
+    group = hq // hkv
+    for t in range(count):
+        last = start + t + 1
+        first = max(0, last - window) if window else 0
+        mean = ((prefix[last] - prefix[first]) / (last - first)).reshape(hkv, hd)
+        want = np.repeat(mean, group, axis=0)
+        assert np.max(np.abs(got[t] - want)) <= 2e-3, t
+
+
 def test_contract():
     fx = make_fixture(4, 3, 0, 1, head_dim=64, pad=(0, 0, 0))
     bad = tfk.TF_ERR_INVALID_ARGUMENT
