@@ -389,16 +389,32 @@ int32_t phase1_entry(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *route
 // ------------------------------------------------------------------------------------------------ shared expert, 8-bit
 // shared_int8_gate_up_act_simd (Metal/Quant/dequant_int8.metal:100-157): one wave per row takes the gate row and the up
 // row against the same activations; act[row] = half(gelu_tanh(float(half(gate))) * float(half(up))).
-__device__ __forceinline__ void int8_chunk(const u32x4 w, const u32x4 xa, const u32x4 xb, float s, float b, float &acc) {
-    float dot = 0.0f, sum = 0.0f;
+// A chunk = 16 weights (one byte each) against 16 activations.  The weights become fp16 pairs once (byte b -> the half
+// 0x6400 | b = 1024 + b, minus 1024: exact), then every pair of products is one packed dot instruction with an fp32 sum;
+// 255 * x is exact in fp32.  Expanded weights serve every activation row they meet, and the sum of a row's activations
+// serves gate and up.
+struct Int8Weights {
+    half2_t q[8];
+};
+__device__ __forceinline__ Int8Weights int8_expand(const u32x4 w) {
+    const half2_t bias = {(half_t)1024.0f, (half_t)1024.0f};
+    Int8Weights e;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-        const uint32_t xw = i < 8 ? xa[i >> 1] : xb[(i - 8) >> 1];
-        const float xv = (float)__builtin_bit_cast(half_t, (uint16_t)((i & 1) ? (xw >> 16) : (xw & 0xFFFFu)));
-        const float q = (float)((w[i >> 2] >> (8 * (i & 3))) & 0xFFu);
-        dot = fmaf(q, xv, dot);
-        sum += xv;
-    }
+    for (int j = 0; j < 8; ++j)
+        e.q[j] = as_half2(__builtin_amdgcn_perm(0x64646464u, w[j >> 1], (j & 1) ? 0x04030402u : 0x04010400u)) - bias;
+    return e;
+}
+__device__ __forceinline__ float int8_sum(const u32x4 xa, const u32x4 xb) {
+    const half2_t ones = {(half_t)1.0f, (half_t)1.0f};
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sum = __builtin_amdgcn_fdot2(as_half2(j < 4 ? xa[j] : xb[j - 4]), ones, sum, false);
+    return sum;
+}
+__device__ __forceinline__ void int8_chunk(const Int8Weights &e, const u32x4 xa, const u32x4 xb, float sum, float s, float b, float &acc) {
+    float dot = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dot = __builtin_amdgcn_fdot2(e.q[j], as_half2(j < 4 ? xa[j] : xb[j - 4]), dot, false);
     acc = fmaf(s, dot, acc);
     acc = fmaf(b, sum, acc);
 }
@@ -437,17 +453,19 @@ __global__ __launch_bounds__(256) void shared8_gate_up_kernel(const uint8_t *gW,
         }
 #pragma unroll
         for (int p = 0; p < MODE; ++p) {
-            int8_chunk(wg[p], xa[p], xb[p], sb_to_f32<SD>(sg[p]), sb_to_f32<SD>(bg[p]), gate);
-            int8_chunk(wu[p], xa[p], xb[p], sb_to_f32<SD>(su[p]), sb_to_f32<SD>(bu[p]), up);
+            const float sum = int8_sum(xa[p], xb[p]);
+            int8_chunk(int8_expand(wg[p]), xa[p], xb[p], sum, sb_to_f32<SD>(sg[p]), sb_to_f32<SD>(bg[p]), gate);
+            int8_chunk(int8_expand(wu[p]), xa[p], xb[p], sum, sb_to_f32<SD>(su[p]), sb_to_f32<SD>(bu[p]), up);
         }
         gate = wave_sum(gate);
         up = wave_sum(up);
     } else if constexpr (MODE == 0) {
         for (int c = lane; c < chunks; c += kWave) {
             const u32x4 xa = load16(x + c * 16), xb = load16(x + c * 16 + 8);
-            int8_chunk(load16(gw + (size_t)c * 16), xa, xb, sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(gs + (c >> 2) * 2)),
+            const float sum = int8_sum(xa, xb);
+            int8_chunk(int8_expand(load16(gw + (size_t)c * 16)), xa, xb, sum, sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(gs + (c >> 2) * 2)),
                        sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(gb + (c >> 2) * 2)), gate);
-            int8_chunk(load16(uw + (size_t)c * 16), xa, xb, sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(us + (c >> 2) * 2)),
+            int8_chunk(int8_expand(load16(uw + (size_t)c * 16)), xa, xb, sum, sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(us + (c >> 2) * 2)),
                        sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(ub + (c >> 2) * 2)), up);
         }
         gate = wave_sum(gate);
@@ -505,13 +523,20 @@ __global__ __launch_bounds__(256) void shared8_gate_up_rows_kernel(const uint8_t
             }
         }
     }
+    Int8Weights eg[NPASS], eu[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) {
+        eg[p] = int8_expand(wg[p]);
+        eu[p] = int8_expand(wu[p]);
+    }
 #pragma unroll
     for (int t = 0; t < kSharedRows; ++t) {
         float gate = 0.0f, up = 0.0f;
 #pragma unroll
         for (int p = 0; p < NPASS; ++p) {
-            int8_chunk(wg[p], xa[t][p], xb[t][p], sg[p], bg[p], gate);
-            int8_chunk(wu[p], xa[t][p], xb[t][p], su[p], bu[p], up);
+            const float sum = int8_sum(xa[t][p], xb[t][p]);
+            int8_chunk(eg[p], xa[t][p], xb[t][p], sum, sg[p], bg[p], gate);
+            int8_chunk(eu[p], xa[t][p], xb[t][p], sum, su[p], bu[p], up);
         }
         gate = wave_sum(gate);
         up = wave_sum(up);
@@ -554,11 +579,14 @@ __global__ __launch_bounds__(256) void gemv8_rows_kernel(const uint8_t *W, const
             }
         }
     }
+    Int8Weights e[NPASS];
+#pragma unroll
+    for (int p = 0; p < NPASS; ++p) e[p] = int8_expand(w[p]);
 #pragma unroll
     for (int t = 0; t < kSharedRows; ++t) {
         float acc = 0.0f;
 #pragma unroll
-        for (int p = 0; p < NPASS; ++p) int8_chunk(w[p], xa[t][p], xb[t][p], sv[p], bv[p], acc);
+        for (int p = 0; p < NPASS; ++p) int8_chunk(e[p], xa[t][p], xb[t][p], int8_sum(xa[t][p], xb[t][p]), sv[p], bv[p], acc);
         acc = wave_sum(acc);
         if (lane == 0 && t0 + t < tokens) y[(size_t)(t0 + t) * y_stride + row] = (half_t)acc;
     }
@@ -897,6 +925,25 @@ int32_t tf_shared_expert_int8_down(tf_ctx *ctx, tf_stream stream, const tf_proje
     TF_REQUIRE(ctx, y_offset + (uint64_t)down->rows * 2 <= y_length, TF_ERR_SCRATCH_TOO_SMALL,
                "SharedExpertInt8 scratch too small: y offset %llu + needed %llu exceeds length %llu", (unsigned long long)y_offset,
                (unsigned long long)down->rows * 2, (unsigned long long)y_length);
+    // aligned operands: the row kernel of the block form with one row, so a block equals its rows one by one bit for bit
+    const uint8_t *dw = at(down->weights, down->weights_offset);
+    const half_t *ap = reinterpret_cast<const half_t *>(at(scratch_act, scratch_act_offset));
+    if (projection_ok(down) && aligned16(dw) && aligned16(ap) && down->cols <= 4096 && y_offset % 2 == 0 &&
+        (scale_dtype == TF_BF16 || scale_dtype == TF_FP16)) {
+        const uint8_t *ds = at(down->scales, down->scales_offset), *db = at(down->biases, down->biases_offset);
+        half_t *yp = reinterpret_cast<half_t *>(at(y, y_offset));
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        const uint32_t m = down->rows, k = down->cols;
+        const int np = (int)((k + 1023) / 1024);
+#define TF_DOWN8(SD_, NP_) hipLaunchKernelGGL((gemv8_rows_kernel<SD_, NP_>), dim3((m + 3) / 4, 1), dim3(256), 0, st, dw, ds, db, ap, yp, m, m, (int)k, 1u)
+        if (scale_dtype == TF_BF16) {
+            if (np == 1) TF_DOWN8(0, 1); else if (np == 2) TF_DOWN8(0, 2); else if (np == 3) TF_DOWN8(0, 3); else TF_DOWN8(0, 4);
+        } else {
+            if (np == 1) TF_DOWN8(1, 1); else if (np == 2) TF_DOWN8(1, 2); else if (np == 3) TF_DOWN8(1, 3); else TF_DOWN8(1, 4);
+        }
+#undef TF_DOWN8
+        return check_launch(ctx, "shared_int8_down");
+    }
     return tf_dequant_int8_gemv(ctx, stream, down->weights, down->weights_offset, down->scales, down->scales_offset, down->biases,
                                 down->biases_offset, scratch_act, scratch_act_offset, y, y_offset, down->rows, down->cols, scale_dtype, TF_FP16);
 }
