@@ -70,7 +70,6 @@ void tf_ctx_destroy(tf_ctx *ctx) {
     if (ctx->prefill_logits) (void)hipFree(ctx->prefill_logits);
     if (ctx->sample_scratch) (void)hipFree(ctx->sample_scratch);
     if (ctx->shared_block_acts) (void)hipFree(ctx->shared_block_acts);
-    if (ctx->shared8_weights) (void)hipFree(ctx->shared8_weights);
     if (ctx->attn_scratch) (void)hipFree(ctx->attn_scratch);
     for (hipEvent_t e : ctx->step_events)
         if (e) (void)hipEventDestroy(e);

@@ -25,8 +25,6 @@ struct tf_ctx {
     size_t sample_scratch_bytes = 0;
     void *shared_block_acts = nullptr;  // lazily sized [rows, intermediate] fp16 activations of the block shared expert
     size_t shared_block_acts_bytes = 0;
-    void *shared8_weights = nullptr;    // lazily sized fp16 copies of the three 8-bit projections of the block shared expert
-    size_t shared8_weights_bytes = 0;
     void *attn_scratch = nullptr;       // lazily sized split-KV partial states of decode attention (m, d, o per head and chunk)
     size_t attn_scratch_bytes = 0;
     // optional device-time bracketing of the decode step's three launches

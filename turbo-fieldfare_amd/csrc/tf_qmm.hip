@@ -395,75 +395,93 @@ int32_t shared_block_acts(tf_ctx *ctx, size_t halves, half_t *&out) {
 constexpr uint32_t kSharedBlockMinRows = 8;   // fewer rows go through the single-row chain, bit-identical to decode
 
 // ---- 8-bit projections over a block of rows ----------------------------------------------------------------------
-// The 8-bit shared expert has no matrix-core loop of its own yet: the three projections are expanded to fp16 once per call,
-// w = half(q * s + b) - the rounding point of the 4-bit matrix-core path - into a buffer the context owns, and a plain
-// fp16 product runs on the matrix cores: a wave owns a 32 x 32 tile of the output and reads its operands straight from
-// memory in the instruction's own layout (lane (i, kb): 8 consecutive k of row i).
-template <int SD>
-__global__ __launch_bounds__(256) void dequant8_f16_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, half_t *out, uint32_t rows, uint32_t k) {
-    const size_t chunk = (size_t)blockIdx.x * blockDim.x + threadIdx.x;       // 16 weights
-    const uint32_t per_row = k >> 4;
-    if (chunk >= (size_t)rows * per_row) return;
-    const uint32_t row = (uint32_t)(chunk / per_row), c = (uint32_t)(chunk % per_row);
-    const u32x4 w = load16(W + (size_t)row * k + (size_t)c * 16);
-    const size_t g = (size_t)row * (k >> 6) + (c >> 2);
-    const half_t s = (half_t)sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(S + g * 2));
-    const half_t b = (half_t)sb_to_f32<SD>(*reinterpret_cast<const uint16_t *>(B + g * 2));
-    const half2_t s2 = {s, s}, b2 = {b, b}, bias = {(half_t)1024.0f, (half_t)1024.0f};
-    u32x4 lo, hi;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-        const half2_t q = as_half2(__builtin_amdgcn_perm(0x64646464u, w[j >> 1], (j & 1) ? 0x04030402u : 0x04010400u)) - bias;
-        const uint32_t v = as_u32(__builtin_elementwise_fma(q, s2, b2));
-        if (j < 4) lo[j] = v; else hi[j - 4] = v;
-    }
-    u32x4 *dst = reinterpret_cast<u32x4 *>(out + (size_t)row * k + (size_t)c * 16);
-    dst[0] = lo;
-    dst[1] = hi;
-}
-
-// Y[M, N] = X[M, K] . W[N, K]^T in fp16 with fp32 sums; GEGLU: two weight matrices, Y = half(gelu_tanh(half(gate)) * half(up)).
-// grid (N / 32, ceil(M / 32)), one wave per block (a block of a few dozen rows makes few tiles: they should land on as many CUs
-// as possible); K % 16 == 0, N % 32 == 0, rows 16-byte aligned.  The operands of the next eight K steps are requested
-// before the current eight are multiplied.
-template <bool GEGLU>
-__global__ __launch_bounds__(64) void hgemm_nt_kernel(const half_t *X, long ldx, const half_t *W0, const half_t *W1, half_t *Y, long ldy, int M, int N,
-                                                      int K) {
-    constexpr int KB = 8;
+// Y[M, N] = X[M, K] . W[N, K]^T on the matrix cores with the 8-bit weights expanded on the way into the instruction,
+// w = half(q * s + b) - the rounding point of the 4-bit matrix-core path; GEGLU: two weight matrices,
+// Y = half(gelu_tanh(half(gate)) * half(up)).  No LDS: a wave owns a 32 x 32 tile of the output and reads its operands
+// straight from memory in the instruction's own layout; grid (N / 32, ceil(M / 32)), one wave per block (a block of a few
+// dozen rows makes few tiles: they should land on as many CUs as possible).
+// K is walked in runs of 32: lane (i, kb) takes bytes 32 p + 16 kb .. + 15 of weight row i and the same 16 activations of its
+// activation row; the first 8 of each run feed one matrix instruction, the last 8 the next (the order of the contraction
+// index is free as long as both operands agree).  Two quantization groups (128 k) are in
+// flight while the previous two are multiplied.  K % 64 == 0, N % 32 == 0, rows 16-byte aligned.
+template <bool GEGLU, int SD>
+__global__ __launch_bounds__(64) void qmm8_nt_kernel(const half_t *X, long ldx, const uint8_t *W0, const uint8_t *S0, const uint8_t *B0, const uint8_t *W1,
+                                                     const uint8_t *S1, const uint8_t *B1, half_t *Y, long ldy, int M, int N, int K) {
+    constexpr int GB = 2;                    // groups per block of requests
     const int lane = threadIdx.x;
     const int i = lane & 31, kb = lane >> 5;
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
-    const half_t *xr = X + (size_t)min(m0 + i, M - 1) * ldx + 8 * kb;
-    const size_t wrow = (size_t)(n0 + i) * K + 8 * kb;
-    const int steps = K >> 4, blocks = (steps + KB - 1) / KB;
+    const half_t *xr = X + (size_t)min(m0 + i, M - 1) * ldx + 16 * kb;
+    const size_t wrow = (size_t)(n0 + i) * K + 16 * kb, sbrow = (size_t)(n0 + i) * (K >> 6) * 2;
+    const int groups = K >> 6, blocks = (groups + GB - 1) / GB;
     float16_t acc0, acc1;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc0[r] = acc1[r] = 0.0f;
-    u32x4 a[2][KB], b0[2][KB], b1[2][KB];
-    auto request = [&](u32x4 (&ar)[KB], u32x4 (&br0)[KB], u32x4 (&br1)[KB], int blk) {
+    struct Operands {
+        u32x4 a[GB][2][2];                   // [group][run of 32][first / last 8 activations]
+        u32x4 w0[GB][2], w1[GB][2];          // [group][run]: 16 weights
+        uint16_t s0[GB], b0[GB], s1[GB], b1[GB];
+    };
+    Operands op[2];
+    auto request = [&](Operands &o, int blk) {
 #pragma unroll
-        for (int j = 0; j < KB; ++j) {
-            const int k = min(blk * KB + j, steps - 1) * 16;      // past the end: the last step again, never multiplied
-            ar[j] = load16(xr + k);
-            br0[j] = load16(W0 + wrow + k);
-            if constexpr (GEGLU) br1[j] = load16(W1 + wrow + k);
+        for (int g = 0; g < GB; ++g) {
+            const int grp = min(blk * GB + g, groups - 1);     // past the end: the last group again, never multiplied
+#pragma unroll
+            for (int run = 0; run < 2; ++run) {
+                const int k = grp * 64 + run * 32;
+                o.a[g][run][0] = load16(xr + k);
+                o.a[g][run][1] = load16(xr + k + 8);
+                o.w0[g][run] = load16(W0 + wrow + k);
+                if constexpr (GEGLU) o.w1[g][run] = load16(W1 + wrow + k);
+            }
+            o.s0[g] = *reinterpret_cast<const uint16_t *>(S0 + sbrow + grp * 2);
+            o.b0[g] = *reinterpret_cast<const uint16_t *>(B0 + sbrow + grp * 2);
+            if constexpr (GEGLU) {
+                o.s1[g] = *reinterpret_cast<const uint16_t *>(S1 + sbrow + grp * 2);
+                o.b1[g] = *reinterpret_cast<const uint16_t *>(B1 + sbrow + grp * 2);
+            }
         }
     };
-    auto multiply = [&](const u32x4 (&ar)[KB], const u32x4 (&br0)[KB], const u32x4 (&br1)[KB], int blk) {
+    auto expand = [&](const u32x4 w, uint16_t sv, uint16_t bv, half8_t &first, half8_t &last) {
+        const half_t sh = (half_t)sb_to_f32<SD>(sv), bh = (half_t)sb_to_f32<SD>(bv);
+        const half2_t s2 = {sh, sh}, b2 = {bh, bh}, bias = {(half_t)1024.0f, (half_t)1024.0f};
+        u32x4 lo, hi;
 #pragma unroll
-        for (int j = 0; j < KB; ++j) {
-            if (blk * KB + j >= steps) break;
-            const half8_t av = __builtin_bit_cast(half8_t, ar[j]);
-            acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, __builtin_bit_cast(half8_t, br0[j]), acc0, 0, 0, 0);
-            if constexpr (GEGLU) acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(av, __builtin_bit_cast(half8_t, br1[j]), acc1, 0, 0, 0);
+        for (int j = 0; j < 8; ++j) {
+            const half2_t q = as_half2(__builtin_amdgcn_perm(0x64646464u, w[j >> 1], (j & 1) ? 0x04030402u : 0x04010400u)) - bias;
+            const uint32_t v = as_u32(__builtin_elementwise_fma(q, s2, b2));
+            if (j < 4) lo[j] = v; else hi[j - 4] = v;
+        }
+        first = __builtin_bit_cast(half8_t, lo);
+        last = __builtin_bit_cast(half8_t, hi);
+    };
+    auto multiply = [&](const Operands &o, int blk) {
+#pragma unroll
+        for (int g = 0; g < GB; ++g) {
+            if (blk * GB + g >= groups) break;
+#pragma unroll
+            for (int run = 0; run < 2; ++run) {
+                half8_t f0, l0;
+                expand(o.w0[g][run], o.s0[g], o.b0[g], f0, l0);
+                const half8_t af = __builtin_bit_cast(half8_t, o.a[g][run][0]), al = __builtin_bit_cast(half8_t, o.a[g][run][1]);
+                acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, f0, acc0, 0, 0, 0);
+                acc0 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, l0, acc0, 0, 0, 0);
+                if constexpr (GEGLU) {
+                    half8_t f1, l1;
+                    expand(o.w1[g][run], o.s1[g], o.b1[g], f1, l1);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(af, f1, acc1, 0, 0, 0);
+                    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, l1, acc1, 0, 0, 0);
+                }
+            }
         }
     };
-    request(a[0], b0[0], b1[0], 0);
+    request(op[0], 0);
     for (int blk = 0; blk < blocks; blk += 2) {
-        request(a[1], b0[1], b1[1], blk + 1);
-        multiply(a[0], b0[0], b1[0], blk);
-        request(a[0], b0[0], b1[0], blk + 2);
-        if (blk + 1 < blocks) multiply(a[1], b0[1], b1[1], blk + 1);
+        request(op[1], blk + 1);
+        multiply(op[0], blk);
+        request(op[0], blk + 2);
+        if (blk + 1 < blocks) multiply(op[1], blk + 1);
     }
     const int n = n0 + acc_col(lane);
 #pragma unroll
@@ -484,32 +502,24 @@ int32_t shared8_block_mfma(tf_ctx *ctx, hipStream_t st, const tf_projection *gat
     if (!(aligned16(w[0]) && aligned16(w[1]) && aligned16(w[2]) && aligned16(x) && x_stride % 8 == 0 && d % 64 == 0 && f % 64 == 0 &&
           (sd == TF_BF16 || sd == TF_FP16) && rows <= 65535u * 32u))
         return TF_ERR_UNAVAILABLE;
-    const size_t elems = (size_t)f * d, need = 3 * elems * sizeof(half_t);
-    if (ctx->shared8_weights_bytes < need) {
-        if (ctx->shared8_weights) {
-            if (hipDeviceSynchronize() != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "prefill_shared_expert: device synchronize failed");
-            (void)hipFree(ctx->shared8_weights);
-            ctx->shared8_weights = nullptr;
-            ctx->shared8_weights_bytes = 0;
-        }
-        if (hipMalloc(&ctx->shared8_weights, need) != hipSuccess) return fail(ctx, TF_ERR_OUT_OF_MEMORY, "prefill_shared_expert: out of device memory");
-        ctx->shared8_weights_bytes = need;
-    }
-    half_t *wh = static_cast<half_t *>(ctx->shared8_weights);
+    const uint8_t *sc[3], *bi[3];
     const tf_projection *proj[3] = {gate, up, down};
     for (int p = 0; p < 3; ++p) {
-        const uint32_t r = proj[p]->rows, k = proj[p]->cols;
-        const size_t chunks = (size_t)r * (k >> 4);
-        const uint8_t *s = at(proj[p]->scales, proj[p]->scales_offset), *b = at(proj[p]->biases, proj[p]->biases_offset);
-        if (sd == TF_BF16) hipLaunchKernelGGL(dequant8_f16_kernel<0>, dim3((uint32_t)((chunks + 255) / 256)), dim3(256), 0, st, w[p], s, b, wh + p * elems, r, k);
-        else hipLaunchKernelGGL(dequant8_f16_kernel<1>, dim3((uint32_t)((chunks + 255) / 256)), dim3(256), 0, st, w[p], s, b, wh + p * elems, r, k);
+        sc[p] = at(proj[p]->scales, proj[p]->scales_offset);
+        bi[p] = at(proj[p]->biases, proj[p]->biases_offset);
     }
-    int32_t rc = check_launch(ctx, "shared expert 8-bit expand");
-    if (rc != TF_OK) return rc;
-    hipLaunchKernelGGL(hgemm_nt_kernel<true>, dim3(f / 32, (rows + 31) / 32), dim3(64), 0, st, x, (long)x_stride, wh, wh + elems, acts, (long)f, (int)rows,
-                       (int)f, (int)d);
-    hipLaunchKernelGGL(hgemm_nt_kernel<false>, dim3(d / 32, (rows + 31) / 32), dim3(64), 0, st, acts, (long)f, wh + 2 * elems, nullptr, y, (long)y_stride,
-                       (int)rows, (int)d, (int)f);
+    const dim3 g1(f / 32, (rows + 31) / 32), g2(d / 32, (rows + 31) / 32);
+    if (sd == TF_BF16) {
+        hipLaunchKernelGGL((qmm8_nt_kernel<true, 0>), g1, dim3(64), 0, st, x, (long)x_stride, w[0], sc[0], bi[0], w[1], sc[1], bi[1], acts, (long)f, (int)rows,
+                           (int)f, (int)d);
+        hipLaunchKernelGGL((qmm8_nt_kernel<false, 0>), g2, dim3(64), 0, st, acts, (long)f, w[2], sc[2], bi[2], nullptr, nullptr, nullptr, y, (long)y_stride,
+                           (int)rows, (int)d, (int)f);
+    } else {
+        hipLaunchKernelGGL((qmm8_nt_kernel<true, 1>), g1, dim3(64), 0, st, x, (long)x_stride, w[0], sc[0], bi[0], w[1], sc[1], bi[1], acts, (long)f, (int)rows,
+                           (int)f, (int)d);
+        hipLaunchKernelGGL((qmm8_nt_kernel<false, 1>), g2, dim3(64), 0, st, acts, (long)f, w[2], sc[2], bi[2], nullptr, nullptr, nullptr, y, (long)y_stride,
+                           (int)rows, (int)d, (int)f);
+    }
     return check_launch(ctx, "shared expert 8-bit block");
 }
 
