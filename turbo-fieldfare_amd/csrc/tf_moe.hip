@@ -548,9 +548,10 @@ __global__ __launch_bounds__(256) void shared8_gate_up_rows_kernel(const uint8_t
 }
 
 // down: y[t, row] = half(W[row, :] . acts[t, :]); acts rows k elements apart, y rows y_stride apart
-template <int SD, int NPASS>
+template <int SD, int NPASS, int ROWS = kSharedRows>
 __global__ __launch_bounds__(256) void gemv8_rows_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *acts, half_t *y,
                                                          uint32_t y_stride, uint32_t m, int k, uint32_t tokens) {
+    constexpr int kSharedRows = ROWS;      // activation rows per weight row fetch (1: the single-row chain)
     const int lane = threadIdx.x & 63;
     const uint32_t row = (blockIdx.x * blockDim.x + threadIdx.x) >> 6, t0 = blockIdx.y * kSharedRows;
     if (row >= m) return;
@@ -935,7 +936,7 @@ int32_t tf_shared_expert_int8_down(tf_ctx *ctx, tf_stream stream, const tf_proje
         hipStream_t st = static_cast<hipStream_t>(stream);
         const uint32_t m = down->rows, k = down->cols;
         const int np = (int)((k + 1023) / 1024);
-#define TF_DOWN8(SD_, NP_) hipLaunchKernelGGL((gemv8_rows_kernel<SD_, NP_>), dim3((m + 3) / 4, 1), dim3(256), 0, st, dw, ds, db, ap, yp, m, m, (int)k, 1u)
+#define TF_DOWN8(SD_, NP_) hipLaunchKernelGGL((gemv8_rows_kernel<SD_, NP_, 1>), dim3((m + 3) / 4, 1), dim3(256), 0, st, dw, ds, db, ap, yp, m, m, (int)k, 1u)
         if (scale_dtype == TF_BF16) {
             if (np == 1) TF_DOWN8(0, 1); else if (np == 2) TF_DOWN8(0, 2); else if (np == 3) TF_DOWN8(0, 3); else TF_DOWN8(0, 4);
         } else {
