@@ -98,6 +98,9 @@ def main():
     ap.add_argument("--no-layer-chain", action="store_true", help="skip the whole-decoder-layer graph (long under a counter-collecting profiler)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (a known-size reference for hardware byte counters)")
+    ap.add_argument("--only-small-m", type=int, nargs="+", metavar="M",
+                    help="run nothing but the few-token routed-MoE measurement at these token counts and print its JSON "
+                         "(a short program whose launches a profiler can attribute to one size)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -113,6 +116,11 @@ def main():
     offs, payload, stride = expert_layout()
     off = tfk.ExpertOffsets(*offs)
     layers = [make_layer(torch, gen, offs, stride) for _ in range(args.layers)]
+    if args.only_small_m:
+        only = multi_token_extras(torch, tfk, k, gen, k.lib, k.handle, torch.cuda.current_stream().cuda_stream, layers[0], offs, stride,
+                                  small_sizes=tuple(args.only_small_m), small_only=True)
+        print(json.dumps(only))
+        return
     n_hidden = 64
     hidden = torch.randn((n_hidden, D), device="cuda", generator=gen).to(torch.float16)
     idx = torch.zeros((n_hidden, TOPK), dtype=torch.int32, device="cuda")
@@ -513,7 +521,7 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride):
         "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 17}}
 
 
-def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride):
+def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, small_sizes=(2, 4, 8, 16, 32, 64, 128), small_only=False):
     """configs[3] (small-M verification, M in {2,4,8,16}) and configs[4] (2048-token prefill, Zipf(1.1) routing) over one
     resident layer: router block -> device grouping -> grouped experts -> token-major reduce, no host round trip."""
     import ctypes as C
@@ -553,13 +561,15 @@ def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride):
         return us, unique
 
     small = {}
-    for M in (2, 4, 8, 16, 32, 64, 128):      # verification sizes, then the reference's prefill chunk sizes (RuntimeConfiguration.swift:24)
+    for M in small_sizes:      # by default: verification sizes, then the reference's prefill chunk sizes (RuntimeConfiguration.swift:24)
         us, unique = run(M, iters=50)
         nbytes = unique * expert_bytes + E * D + M * (2 * D * 2 + TOPK * F_MOE * 2 * 2 + TOPK * D * 2 * 2)
         small[str(M)] = {"us": round(us, 2), "unique_experts": unique, "GBps_on_unique_expert_bytes": round(nbytes / (us * 1e-6) / 1e9, 1),
                          "tokens_per_s": round(M / (us * 1e-6), 1)}
     res["small_m"] = {"workload": "configs[3]: M tokens x top-8 over 128 resident experts (router block + grouping + grouped experts + reduce)",
                       "per_M": small}
+    if small_only:
+        return res
 
     # configs[4]: 2048 tokens, Zipf(1.1) expert popularity, 8 distinct experts per token
     T = 2048
