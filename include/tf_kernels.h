@@ -19,7 +19,9 @@
  *     aligned (DequantInt4GEMV.swift:57-62); 16-byte aligned operands take the
  *     vector path, anything else a slower path with identical results;
  *   - calls only enqueue work on `stream` (one in-order stream = the reference's
- *     command queue); nothing blocks except tf_stream_synchronize;
+ *     command queue); nothing blocks or allocates except tf_ctx_create,
+ *     tf_ctx_reserve, tf_stream_synchronize and the tf_upload_* loaders, so every
+ *     other entry point may be recorded into a HIP graph;
  *   - the caller owns every buffer; the library never frees caller memory;
  *   - where the reference traps on a broken precondition or throws, the call
  *     returns a negative tf_status and enqueues nothing.
@@ -98,6 +100,23 @@ typedef struct tf_routed_blobs {
  * and row summaries: LMHeadChainInt4.swift:38-51). */
 int32_t tf_ctx_create(int32_t device, tf_ctx **out_ctx);
 void tf_ctx_destroy(tf_ctx *ctx);
+/* The reference's wrappers size their own scratch once, in `init` (MoE.swift:92-99 routerLogits for 256 experts;
+ * LMHeadChainInt4.swift:38-51 xNormed/rowSummaries for maxD/maxVocab; PrefillRouter, PrefillSharedExpert and the samplers
+ * likewise).  Here that is tf_ctx_create, which sizes every wrapper buffer for the limits below, and tf_ctx_reserve,
+ * which raises them (limits only grow; it waits for the device and reallocates, so call it at set-up, never while a
+ * stream is being captured).  An entry point whose arguments exceed the limits returns TF_ERR_SCRATCH_TOO_SMALL and
+ * enqueues nothing; no entry point allocates, frees or synchronises.  tf_ctx_create's limits are
+ * {262144, 2048, 256, 2112, 16, 512, 128}. */
+typedef struct tf_scratch_limits {
+    uint32_t max_vocab;                  /* lm_head rows: fp32 logits of the unaligned greedy path, the samplers' cells and top-k pair buffers */
+    uint32_t max_block_tokens;           /* rows of one prefill block: router logits [tokens, experts], shared-expert activations */
+    uint32_t max_experts;                /* router width of the multi-token router */
+    uint32_t max_shared_intermediate;    /* shared expert's intermediate size (activations [tokens, intermediate] of the block form) */
+    uint32_t max_q_heads, max_head_dim;  /* decode and block attention: split-KV partial states */
+    uint32_t max_attention_block_tokens; /* queries of one tf_prefill_attention_causal call */
+} tf_scratch_limits;
+int32_t tf_ctx_reserve(tf_ctx *ctx, const tf_scratch_limits *limits);
+int32_t tf_ctx_scratch_limits(const tf_ctx *ctx, tf_scratch_limits *out_limits);
 /* commandBuffer.waitUntilCompleted + checkCommandBufferError (MetalContext.swift:22-26): returns TF_ERR_DEVICE if
  * anything enqueued on the stream failed. */
 int32_t tf_stream_synchronize(tf_ctx *ctx, tf_stream stream);

@@ -59,6 +59,12 @@ class AttentionSplitGeometry(C.Structure):
                 ("partial_threadgroups", C.c_int32), ("use_swa_grouped_partial", C.c_int32)]
 
 
+class ScratchLimits(C.Structure):
+    """tf_scratch_limits: what the context's wrapper scratch is sized for (tf_ctx_reserve raises it)."""
+    _fields_ = [(n, C.c_uint32) for n in ("max_vocab", "max_block_tokens", "max_experts", "max_shared_intermediate", "max_q_heads",
+                                          "max_head_dim", "max_attention_block_tokens")]
+
+
 class RoutedBlobs(C.Structure):
     """tf_routed_blobs."""
     _fields_ = [("blobs", vp * 8), ("pool", vp), ("pool_stride", u64), ("indices", vp), ("num_experts", u32)]
@@ -103,6 +109,8 @@ class TFError(RuntimeError):
 EXPORTS = {
     "tf_ctx_create": (i32, [i32, C.POINTER(vp)]),
     "tf_ctx_destroy": (None, [vp]),
+    "tf_ctx_reserve": (i32, [vp, C.POINTER(ScratchLimits)]),
+    "tf_ctx_scratch_limits": (i32, [vp, C.POINTER(ScratchLimits)]),
     "tf_stream_synchronize": (i32, [vp, vp]),
     "tf_status_string": (C.c_char_p, [i32]),
     "tf_last_error": (C.c_char_p, [vp]),
@@ -255,6 +263,17 @@ class Context:
 
     def synchronize(self, stream=None):
         return self.check(self.lib.tf_stream_synchronize(self.handle, _stream() if stream is None else stream))
+
+    def reserve(self, **limits) -> "ScratchLimits":
+        """Raises the wrapper-scratch limits (tf_ctx_reserve; set-up time only: it may wait for the device) and returns them."""
+        want = ScratchLimits(**limits)
+        self.check(self.lib.tf_ctx_reserve(self.handle, C.byref(want)))
+        return self.scratch_limits()
+
+    def scratch_limits(self) -> "ScratchLimits":
+        out = ScratchLimits()
+        self.check(self.lib.tf_ctx_scratch_limits(self.handle, C.byref(out)))
+        return out
 
     def set_step_timing(self, enabled: bool):
         return self.check(self.lib.tf_ctx_set_step_timing(self.handle, 1 if enabled else 0))

@@ -687,16 +687,7 @@ __global__ __launch_bounds__(kAttnThreads) void attention_prefill_generic_kernel
 // the context's partial-state scratch: m and d [heads x chunks], o [heads x chunks x head_dim]
 int32_t attention_scratch(tf_ctx *ctx, size_t floats, float *&out) {
     const size_t need = floats * sizeof(float);
-    if (ctx->attn_scratch_bytes < need) {
-        if (ctx->attn_scratch) {
-            if (hipDeviceSynchronize() != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "attention: device synchronize failed");
-            (void)hipFree(ctx->attn_scratch);
-            ctx->attn_scratch = nullptr;
-            ctx->attn_scratch_bytes = 0;
-        }
-        if (hipMalloc(&ctx->attn_scratch, need) != hipSuccess) return fail(ctx, TF_ERR_OUT_OF_MEMORY, "attention: out of device memory");
-        ctx->attn_scratch_bytes = need;
-    }
+    if (ctx->attn_scratch_bytes < need) return scratch_too_small(ctx, "attention", need, ctx->attn_scratch_bytes);
     out = static_cast<float *>(ctx->attn_scratch);
     return TF_OK;
 }
@@ -774,6 +765,25 @@ int32_t attention_split(tf_ctx *ctx, tf_stream stream, const void *q, uint64_t q
 float default_scale(uint32_t head_dim) { return 1.0f / sqrtf((float)head_dim); }
 
 }  // namespace
+
+namespace tfk {
+
+// Upper bound of the partial states (m, d and head_dim values of o each) any call within the limits asks for.
+// Decode: q_heads x chunks with at most kMaxDeviceChunks chunks.  Block attention: n = queries x q_heads columns make at
+// least ceil(n / 64) blocks per chunk, and chunks stop at two blocks per compute unit or kMaxPrefillChunks.
+size_t attention_scratch_floats_for(int num_cus, uint32_t q_heads, uint32_t head_dim, uint32_t block_tokens) {
+    size_t states = (size_t)q_heads * kMaxDeviceChunks;
+    const size_t target = (size_t)(num_cus > 0 ? num_cus : 256) * 2;
+    const size_t max_n = (size_t)block_tokens * q_heads;
+    for (size_t n = 1; n <= max_n; ++n) {
+        const size_t base = (n + kPrefillCols - 1) / kPrefillCols;
+        const size_t chunks = std::min<size_t>(kMaxPrefillChunks, (target + base - 1) / base);
+        states = std::max(states, n * chunks);
+    }
+    return states * (2 + (size_t)head_dim);
+}
+
+}  // namespace tfk
 
 extern "C" {
 

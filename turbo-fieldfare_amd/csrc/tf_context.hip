@@ -48,6 +48,9 @@ int32_t tf_ctx_create(int32_t device, tf_ctx **out_ctx) {
     ok = ok && hipMalloc(&ctx->head_summaries, summary_bytes) == hipSuccess;
     ok = ok && hipMemset(ctx->head_summaries, 0, summary_bytes) == hipSuccess;
     ok = ok && hipMalloc(&ctx->group_scratch, (size_t)kGroupSegments * 256 * sizeof(uint32_t)) == hipSuccess;
+    // the reference's model (Infrastructure/ModelIO/ModelTypes.swift:78-100) at the largest block sizes this library is run at
+    const tf_scratch_limits defaults = {262144u, 2048u, 256u, 2112u, 16u, 512u, 128u};
+    ok = ok && tf_ctx_reserve(ctx, &defaults) == TF_OK;
     if (const char *env = getenv("TF_STREAM_BLOCKS_PER_CU")) {
         const int v = atoi(env);
         if (v >= 1 && v <= 8) ctx->stream_blocks_per_cu = v;
@@ -74,6 +77,57 @@ void tf_ctx_destroy(tf_ctx *ctx) {
     for (hipEvent_t e : ctx->step_events)
         if (e) (void)hipEventDestroy(e);
     delete ctx;
+}
+
+namespace {
+
+// Grows one wrapper buffer; kernels of earlier calls may still use the old one, so the device is drained first.
+bool regrow(void **buf, size_t *have, size_t need, size_t unit) {
+    if (*have * unit >= need) return true;
+    if (*buf) {
+        if (hipDeviceSynchronize() != hipSuccess) return false;
+        (void)hipFree(*buf);
+        *buf = nullptr;
+        *have = 0;
+    }
+    if (need == 0) return true;
+    if (hipMalloc(buf, need) != hipSuccess) return false;
+    *have = need / unit;
+    return true;
+}
+
+}  // namespace
+
+int32_t tf_ctx_reserve(tf_ctx *ctx, const tf_scratch_limits *limits) {
+    TF_REQUIRE(ctx, ctx && limits, TF_ERR_INVALID_ARGUMENT, "ctx_reserve: null argument");
+    if (hipSetDevice(ctx->device) != hipSuccess) return fail(ctx, TF_ERR_NO_DEVICE, "ctx_reserve: cannot select device %d", ctx->device);
+    tf_scratch_limits want = ctx->limits;   // limits only ever grow
+    want.max_vocab = limits->max_vocab > want.max_vocab ? limits->max_vocab : want.max_vocab;
+    want.max_block_tokens = limits->max_block_tokens > want.max_block_tokens ? limits->max_block_tokens : want.max_block_tokens;
+    want.max_experts = limits->max_experts > want.max_experts ? limits->max_experts : want.max_experts;
+    want.max_shared_intermediate = limits->max_shared_intermediate > want.max_shared_intermediate ? limits->max_shared_intermediate : want.max_shared_intermediate;
+    want.max_q_heads = limits->max_q_heads > want.max_q_heads ? limits->max_q_heads : want.max_q_heads;
+    want.max_head_dim = limits->max_head_dim > want.max_head_dim ? limits->max_head_dim : want.max_head_dim;
+    want.max_attention_block_tokens = limits->max_attention_block_tokens > want.max_attention_block_tokens ? limits->max_attention_block_tokens : want.max_attention_block_tokens;
+    bool ok = regrow(reinterpret_cast<void **>(&ctx->head_logits), &ctx->head_logits_count, (size_t)want.max_vocab * sizeof(float), sizeof(float));
+    ok = ok && regrow(reinterpret_cast<void **>(&ctx->prefill_logits), &ctx->prefill_logits_count,
+                      prefill_logits_floats_for(want.max_block_tokens, want.max_experts) * sizeof(float), sizeof(float));
+    const size_t sample_before = ctx->sample_scratch_bytes;
+    ok = ok && regrow(&ctx->sample_scratch, &ctx->sample_scratch_bytes, sample_scratch_bytes_for(want.max_vocab), 1);
+    if (ok && ctx->sample_scratch_bytes != sample_before && ctx->sample_scratch)
+        ok = hipMemset(ctx->sample_scratch, 0, sample_scratch_clear_bytes()) == hipSuccess;   // cells and ticket start at zero
+    ok = ok && regrow(&ctx->shared_block_acts, &ctx->shared_block_acts_bytes, (size_t)want.max_block_tokens * want.max_shared_intermediate * 2, 1);
+    ok = ok && regrow(&ctx->attn_scratch, &ctx->attn_scratch_bytes,
+                      attention_scratch_floats_for(ctx->num_cus, want.max_q_heads, want.max_head_dim, want.max_attention_block_tokens) * sizeof(float), 1);
+    if (!ok) return fail(ctx, TF_ERR_OUT_OF_MEMORY, "ctx_reserve: out of device memory");
+    ctx->limits = want;
+    return TF_OK;
+}
+
+int32_t tf_ctx_scratch_limits(const tf_ctx *ctx, tf_scratch_limits *out_limits) {
+    if (!ctx || !out_limits) return TF_ERR_INVALID_ARGUMENT;
+    *out_limits = ctx->limits;
+    return TF_OK;
 }
 
 int32_t tf_stream_synchronize(tf_ctx *ctx, tf_stream stream) {

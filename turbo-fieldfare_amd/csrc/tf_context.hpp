@@ -16,17 +16,19 @@ struct tf_ctx {
     float *router_logits = nullptr;     // 256 floats (MoE.swift:92-99)
     void *head_x_normed = nullptr;      // kMaxHeadD halves (LMHeadChainInt4.swift:38-51)
     float *head_summaries = nullptr;    // kMaxHeadWaves x {value, index bits}
-    float *head_logits = nullptr;       // lazily sized fp32 logits for the unaligned lm_head path
+    float *head_logits = nullptr;       // fp32 logits of the unaligned lm_head path, limits.max_vocab of them
     size_t head_logits_count = 0;
     uint32_t *group_scratch = nullptr;  // kGroupSegments x 256 per-segment expert counts of the device pair grouping
-    float *prefill_logits = nullptr;    // lazily sized [tokens, experts] router logits of the multi-token router
+    float *prefill_logits = nullptr;    // [tokens, experts] router logits (+ partial planes) of the multi-token router
     size_t prefill_logits_count = 0;
-    void *sample_scratch = nullptr;     // lazily sized: argmax cells, softmax partials, top-k pair buffers of the samplers
+    void *sample_scratch = nullptr;     // argmax cells, softmax partials, top-k pair buffers of the samplers
     size_t sample_scratch_bytes = 0;
-    void *shared_block_acts = nullptr;  // lazily sized [rows, intermediate] fp16 activations of the block shared expert
+    void *shared_block_acts = nullptr;  // [rows, intermediate] fp16 activations of the block shared expert
     size_t shared_block_acts_bytes = 0;
-    void *attn_scratch = nullptr;       // lazily sized split-KV partial states of decode attention (m, d, o per head and chunk)
+    void *attn_scratch = nullptr;       // split-KV partial states of decode and block attention (m, d, o per head and chunk)
     size_t attn_scratch_bytes = 0;
+    // what the five buffers above are sized for; only tf_ctx_create and tf_ctx_reserve allocate them
+    tf_scratch_limits limits = {0, 0, 0, 0, 0, 0, 0};
     // optional device-time bracketing of the decode step's three launches
     bool step_timing = false;
     bool step_timed = false;            // a step has been recorded since timing was enabled
@@ -60,6 +62,18 @@ inline const uint8_t *at(const void *base, uint64_t off) { return static_cast<co
 inline uint8_t *at(void *base, uint64_t off) { return static_cast<uint8_t *>(base) + off; }
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline bool aligned(const void *p, unsigned a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1u)) == 0; }
+
+// Wrapper scratch is sized once (tf_ctx_create, tf_ctx_reserve); an entry point that finds it too small enqueues nothing.
+inline int32_t scratch_too_small(tf_ctx *ctx, const char *who, size_t need, size_t have) {
+    return fail(ctx, TF_ERR_SCRATCH_TOO_SMALL, "%s: needs %zu bytes of wrapper scratch, the context holds %zu: raise the limits with tf_ctx_reserve",
+                who, need, have);
+}
+
+// Sizes of the wrapper scratch as functions of the limits, each defined beside the entry points that use the buffer.
+size_t sample_scratch_bytes_for(uint32_t vocab);                                    // tf_sampling.hip
+size_t sample_scratch_clear_bytes();                                                // leading bytes that must start at zero
+size_t prefill_logits_floats_for(uint32_t tokens, uint32_t experts);                // tf_prefill.hip
+size_t attention_scratch_floats_for(int num_cus, uint32_t q_heads, uint32_t head_dim, uint32_t block_tokens);   // tf_attention.hip
 
 // The 8-bit shared expert over a block of rows (tf_moe.hip), for the block entry of the shared expert (tf_qmm.hip): two
 // launches, every row bit-identical to the single-row chain.  acts: [rows, intermediate] fp16 scratch.  TF_ERR_UNAVAILABLE when

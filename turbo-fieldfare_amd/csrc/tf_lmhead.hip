@@ -189,14 +189,8 @@ int32_t tf_lm_head_greedy_int4(tf_ctx *ctx, tf_stream stream, const void *hidden
         return check_launch(ctx, "lm_head_greedy rows");
     } else {
         // short or unaligned rows: fp32 logits into wrapper-owned scratch, then a two-stage argmax
-        if (ctx->head_logits_count < vocab) {
-            if (ctx->head_logits) (void)hipFree(ctx->head_logits);
-            ctx->head_logits = nullptr;
-            ctx->head_logits_count = 0;
-            if (hipMalloc(&ctx->head_logits, (size_t)vocab * sizeof(float)) != hipSuccess)
-                return fail(ctx, TF_ERR_OUT_OF_MEMORY, "lm_head_greedy_int4: cannot allocate %u logits", vocab);
-            ctx->head_logits_count = vocab;
-        }
+        if (ctx->head_logits_count < vocab)
+            return scratch_too_small(ctx, "lm_head_greedy_int4 (unaligned rows)", (size_t)vocab * sizeof(float), ctx->head_logits_count * sizeof(float));
         rc = launch_gemv4(ctx, st, w, s, b, xn, ctx->head_logits, vocab, d, scale_dtype, TF_FP32);
         if (rc != TF_OK) return rc;
         const uint32_t grid = (uint32_t)std::min<long>(((long)vocab + 255) / 256, 1024);

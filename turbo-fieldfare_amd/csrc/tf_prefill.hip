@@ -792,6 +792,15 @@ int32_t run_grouped(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const t
 
 }  // namespace
 
+namespace tfk {
+
+// logits [tokens, experts] plus up to four partial planes of the split reduction, never less than the few-token router needs
+size_t prefill_logits_floats_for(uint32_t tokens, uint32_t experts) {
+    return std::max<size_t>((size_t)kFewTokens * 256, (size_t)tokens * experts * 5);
+}
+
+}  // namespace tfk
+
 extern "C" {
 
 int32_t tf_prefill_router_gemma4_block(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset,
@@ -833,14 +842,8 @@ int32_t tf_prefill_router_gemma4_block(tf_ctx *ctx, tf_stream stream, const void
         const uint32_t planes = splits > 1 ? splits : 0;   // partial planes behind the logits
         const size_t plane = (size_t)query_count * num_experts;
         const size_t need = std::max<size_t>((size_t)kFewTokens * 256, plane * (1 + planes));
-        if (ctx->prefill_logits_count < need) {
-            if (ctx->prefill_logits) (void)hipFree(ctx->prefill_logits);
-            ctx->prefill_logits = nullptr;
-            ctx->prefill_logits_count = 0;
-            if (hipMalloc(&ctx->prefill_logits, need * sizeof(float)) != hipSuccess)
-                return fail(ctx, TF_ERR_OUT_OF_MEMORY, "prefill_router: cannot allocate the logits scratch");
-            ctx->prefill_logits_count = need;
-        }
+        if (ctx->prefill_logits_count < need)
+            return scratch_too_small(ctx, "prefill_router", need * sizeof(float), ctx->prefill_logits_count * sizeof(float));
         if (query_count > kFewTokens) {
             const int groups_per_split = (int)((groups + splits - 1) / splits);
             hipLaunchKernelGGL(prefill_logits_mfma_kernel<0>, dim3(token_blocks, splits), dim3(256), 0, st, w, s, b, h,

@@ -374,20 +374,10 @@ int32_t launch_qmm_dense_geglu(tf_ctx *ctx, hipStream_t st, const tf_projection 
     return check_launch(ctx, "prefill_shared_expert gate/up");
 }
 
-// [rows, intermediate] fp16 activations of the block form of the shared expert, owned by the context and grown on demand
+// [rows, intermediate] fp16 activations of the block form of the shared expert, owned by the context
 int32_t shared_block_acts(tf_ctx *ctx, size_t halves, half_t *&out) {
     const size_t need = halves * sizeof(half_t);
-    if (ctx->shared_block_acts_bytes < need) {
-        if (ctx->shared_block_acts) {
-            // kernels of earlier calls may still be using the old buffer
-            if (hipDeviceSynchronize() != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "prefill_shared_expert: device synchronize failed");
-            (void)hipFree(ctx->shared_block_acts);
-            ctx->shared_block_acts = nullptr;
-            ctx->shared_block_acts_bytes = 0;
-        }
-        if (hipMalloc(&ctx->shared_block_acts, need) != hipSuccess) return fail(ctx, TF_ERR_OUT_OF_MEMORY, "prefill_shared_expert: out of device memory");
-        ctx->shared_block_acts_bytes = need;
-    }
+    if (ctx->shared_block_acts_bytes < need) return scratch_too_small(ctx, "prefill_shared_expert", need, ctx->shared_block_acts_bytes);
     out = static_cast<half_t *>(ctx->shared_block_acts);
     return TF_OK;
 }

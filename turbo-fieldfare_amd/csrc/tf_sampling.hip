@@ -256,7 +256,7 @@ __global__ __launch_bounds__(256) void topk_final_kernel(const half_t *probs, co
     out_token[0] = picked == 0xFFFFFFFFu ? 0u : picked;
 }
 
-// Wrapper-owned scratch of the samplers, grown on demand: [argmax cells + ticket | softmax partials | two pair buffers].
+// Wrapper-owned scratch of the samplers: [argmax cells + ticket | softmax partials | two pair buffers].
 struct SampleScratch {
     unsigned long long *cells;
     float *partials;
@@ -267,21 +267,14 @@ struct SampleScratch {
 constexpr size_t kCellBytes = (kHeadCells + 1) * sizeof(unsigned long long);
 constexpr size_t kPartialBytes = kSoftmaxMaxBlocks * 2 * sizeof(float);
 
-int32_t sample_scratch(tf_ctx *ctx, uint32_t pair_capacity, SampleScratch &out) {
+size_t sample_need(uint32_t pair_capacity) {
     const size_t pairs = ((size_t)pair_capacity + 255) / 256 * 256;
-    const size_t need = kCellBytes + kPartialBytes + pairs * 16;
-    if (ctx->sample_scratch_bytes < need) {
-        if (ctx->sample_scratch) {
-            // kernels of earlier calls may still be using the old buffer
-            if (hipDeviceSynchronize() != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "sampler scratch: device synchronize failed");
-            (void)hipFree(ctx->sample_scratch);
-            ctx->sample_scratch = nullptr;
-            ctx->sample_scratch_bytes = 0;
-        }
-        if (hipMalloc(&ctx->sample_scratch, need) != hipSuccess) return fail(ctx, TF_ERR_OUT_OF_MEMORY, "sampler scratch: out of device memory");
-        if (hipMemset(ctx->sample_scratch, 0, kCellBytes) != hipSuccess) return fail(ctx, TF_ERR_DEVICE, "sampler scratch: clear failed");
-        ctx->sample_scratch_bytes = need;
-    }
+    return kCellBytes + kPartialBytes + pairs * 16;
+}
+
+int32_t sample_scratch(tf_ctx *ctx, uint32_t pair_capacity, SampleScratch &out) {
+    const size_t need = sample_need(pair_capacity);
+    if (ctx->sample_scratch_bytes < need) return scratch_too_small(ctx, "sampler", need, ctx->sample_scratch_bytes);
     uint8_t *base = static_cast<uint8_t *>(ctx->sample_scratch);
     const size_t have_pairs = (ctx->sample_scratch_bytes - kCellBytes - kPartialBytes) / 16;
     out.cells = reinterpret_cast<unsigned long long *>(base);
@@ -335,6 +328,14 @@ int32_t launch_truncating_sampler(tf_ctx *ctx, hipStream_t st, const half_t *pro
 }
 
 }  // namespace
+
+namespace tfk {
+
+// the truncating samplers keep up to 256 candidates of every 1024-element tile of the first pass
+size_t sample_scratch_bytes_for(uint32_t vocab) { return sample_need((vocab + kTile - 1) / kTile * 256u); }
+size_t sample_scratch_clear_bytes() { return kCellBytes; }
+
+}  // namespace tfk
 
 extern "C" {
 

@@ -31,6 +31,9 @@ public:
     void check(int32_t rc) const {
         if (rc != TF_OK) throw Error(rc, tf_last_error(ctx_));
     }
+    // The Swift wrappers size their scratch in `init` (MoE.swift:92-99, LMHeadChainInt4.swift:38-51); here one call raises the
+    // context's limits for all of them.  Set-up time only.
+    void reserve(const tf_scratch_limits &limits) const { check(tf_ctx_reserve(ctx_, &limits)); }
     // commandBuffer.commit + waitUntilCompleted + checkCommandBufferError (MetalContext.swift:22-26)
     void waitUntilCompleted() const { check(tf_stream_synchronize(ctx_, stream_)); }
 
