@@ -40,6 +40,17 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t *W, co
     if (lane == 0) logits[e] = v;
 }
 
+// One block per expert row (aligned operands, d <= 4096).
+template <int SD>
+__global__ __launch_bounds__(256) void router_logits_block_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *hidden,
+                                                                  const uint16_t *eff, float *logits, int d) {
+    __shared__ float partial[4];
+    const uint32_t e = blockIdx.x;
+    const int groups = d >> 6;
+    const float v = router_row_block<SD>(W + (size_t)e * d, S + (size_t)e * groups * 2, B + (size_t)e * groups * 2, hidden, eff, d, partial);
+    if (threadIdx.x == 0) logits[e] = v;
+}
+
 __global__ __launch_bounds__(64) void router_select_kernel(const float *logits, const uint16_t *per_expert_scale,
                                                            uint32_t *out_indices, half_t *out_weights, uint32_t num_experts,
                                                            uint32_t top_k) {
@@ -48,7 +59,7 @@ __global__ __launch_bounds__(64) void router_select_kernel(const float *logits, 
 
 // ------------------------------------------------------------------------------------------------ phase 1
 __device__ __forceinline__ void store_act(half_t *acts, uint32_t index, float gate, float up) {
-    acts[index] = (half_t)(gelu_tanh(gate) * up);
+    acts[index] = (half_t)(gelu_tanh_fast(gate) * up);
 }
 
 struct Phase1Geom {
@@ -70,9 +81,10 @@ __device__ __forceinline__ bool phase1_slot(const Phase1Geom &g, uint32_t unit, 
     return slot < g.top_k;
 }
 
-// Selection fused into phase 1 (the decode step): wave 0 of every block repeats the top-k over the router's logits
-// while the block's activation loads are in flight, instead of the grid waiting for a selection kernel and then for its
-// indices; block 0 publishes indices and weights for phase 2 and for the caller.
+// Selection fused into phase 1 (the decode step): every block repeats the top-k over the router's logits (by counting,
+// all four waves at once; the one-wave serial selection only when scores tie) while its activation loads are in flight,
+// instead of the grid waiting for a selection kernel and then for its indices; block 0 publishes indices and weights for
+// phase 2 and for the caller.
 struct FusedSelect {
     const float *logits;
     const uint16_t *per_expert_scale;
@@ -90,9 +102,12 @@ __global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_e
     __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
     __shared__ float xsum[XStage::kMaxK / 32];
     __shared__ uint32_t chosen[TF_MAX_STREAMED_EXPERTS];
+    __shared__ RankSelectLds sel;
     const int lane = threadIdx.x & 63;
     const uint32_t unit = uniform_u32((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
     const uint32_t tiles = (g.f + RT - 1) / RT;
+    float my_logit = 0.0f;
+    if constexpr (FUSED) my_logit = rank_select_load(fs.logits, fs.num_experts);   // requested first: the selection waits for nothing else
     XStage stage;
     stage.request(x, (int)g.d);
     uint32_t slot = 0, tile = 0;
@@ -107,8 +122,10 @@ __global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_e
         rs.load(tg, base + off.gate_W_off + w_byte, base + off.gate_s_off + sb_byte, base + off.gate_b_off + sb_byte, g.f - row0);
         rs.load(tu, base + off.up_W_off + w_byte, base + off.up_s_off + sb_byte, base + off.up_b_off + sb_byte, g.f - row0);
     };
+    bool ranked = false;
     if constexpr (FUSED) {
-        if (uniform_u32(threadIdx.x >> 6) == 0) {
+        ranked = rank_select_block(my_logit, fs.num_experts, sel, chosen);
+        if (!ranked && uniform_u32(threadIdx.x >> 6) == 0) {
             uint32_t idx;
             half_t weight;
             router_select_lanes(fs.logits, fs.per_expert_scale, fs.num_experts, g.top_k, lane, idx, weight);
@@ -125,7 +142,18 @@ __global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_e
     }
     stage.publish((int)g.d, xa, xsum);
     if (!live) return;
-    if constexpr (FUSED) request_weights(routed.pool + (uint64_t)uniform_u32(chosen[slot]) * routed.stride);
+    if constexpr (FUSED) {
+        request_weights(routed.pool + (uint64_t)uniform_u32(chosen[slot]) * routed.stride);
+        if (ranked && blockIdx.x == 0 && threadIdx.x < 64) {   // the step's outputs, off the path of the weight requests
+            uint32_t idx;
+            half_t weight;
+            rank_select_weights(sel, chosen, fs.per_expert_scale, lane, idx, weight);
+            if ((uint32_t)lane < g.top_k) {
+                fs.out_indices[lane] = idx;
+                fs.out_weights[lane] = weight;
+            }
+        }
+    }
     rs.init_x_lds(xa, xsum, (int)g.d);
     float gate[RT], up[RT];
     rs.template reduce<SD>(tg, gate);
@@ -603,7 +631,7 @@ int32_t router_logits_entry(tf_ctx *ctx, tf_stream stream, const void *weights, 
                             uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *hidden,
                             const void *effective_scale, uint64_t effective_scale_offset, const void *per_expert_scale,
                             uint64_t per_expert_scale_offset, void *out_indices, void *out_weights, uint32_t num_experts,
-                            uint32_t d, uint32_t top_k) {
+                            uint32_t d, uint32_t top_k, float *logits) {
     TF_REQUIRE(ctx, ctx && weights && scales && biases && hidden && effective_scale && per_expert_scale && out_indices && out_weights,
                TF_ERR_INVALID_ARGUMENT, "router_gemma4: null argument");
     TF_REQUIRE(ctx, d > 0 && d % TF_GROUP_SIZE == 0, TF_ERR_INVALID_ARGUMENT, "router_gemma4: d must be a multiple of 64, got %u", d);
@@ -620,10 +648,15 @@ int32_t router_logits_entry(tf_ctx *ctx, tf_stream stream, const void *weights, 
     const bool fast = aligned16(w) && aligned16(hidden) && aligned16(eff) && d <= 4096;
     const int npass = fast ? (int)((d / 16 + 63) / 64) : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (fast) {
+        hipLaunchKernelGGL((router_logits_block_kernel<0>), dim3(num_experts), dim3(256), 0, st, w, s, b, static_cast<const half_t *>(hidden),
+                           reinterpret_cast<const uint16_t *>(eff), logits, (int)d);
+        return check_launch(ctx, "router_gemma4 logits");
+    }
     const dim3 grid((num_experts + 3) / 4);
 #define TF_ROUTER(NP_)                                                                                                        \
     hipLaunchKernelGGL((router_logits_kernel<0, NP_>), grid, dim3(256), 0, st, w, s, b, static_cast<const half_t *>(hidden),  \
-                       reinterpret_cast<const uint16_t *>(eff), ctx->router_logits, num_experts, (int)d)
+                       reinterpret_cast<const uint16_t *>(eff), logits, num_experts, (int)d)
     switch (npass) {
         case 1: TF_ROUTER(1); break;
         case 2: TF_ROUTER(2); break;
@@ -637,11 +670,55 @@ int32_t router_logits_entry(tf_ctx *ctx, tf_stream stream, const void *weights, 
 
 // Router stage 2: one wave selects from the logits.
 int32_t router_select_entry(tf_ctx *ctx, tf_stream stream, const void *per_expert_scale, uint64_t per_expert_scale_offset,
-                            void *out_indices, void *out_weights, uint32_t num_experts, uint32_t top_k) {
-    hipLaunchKernelGGL(router_select_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), ctx->router_logits,
+                            void *out_indices, void *out_weights, uint32_t num_experts, uint32_t top_k, const float *logits) {
+    hipLaunchKernelGGL(router_select_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), logits,
                        reinterpret_cast<const uint16_t *>(at(per_expert_scale, per_expert_scale_offset)),
                        static_cast<uint32_t *>(out_indices), static_cast<half_t *>(out_weights), num_experts, top_k);
     return check_launch(ctx, "router_gemma4 select");
+}
+
+// router logits -> (selection + phase 1) -> phase 2 on one stream; `logits` is the num_experts-float scratch between the launches
+int32_t decode_step_impl(tf_ctx *ctx, tf_stream stream, const void *router_weights, uint64_t router_weights_offset,
+                           const void *router_scales, uint64_t router_scales_offset, const void *router_biases,
+                           uint64_t router_biases_offset, const void *router_x, const void *effective_scale,
+                           uint64_t effective_scale_offset, const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                           const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                           const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
+                           void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype, float *logits,
+                         bool may_time) {
+    TF_REQUIRE(ctx, ctx && expert_pool && out_indices, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: null argument");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const bool timed = may_time && ctx->step_timing;
+    auto mark = [&](int i) {
+        if (timed) (void)hipEventRecord(ctx->step_events[i], st);
+    };
+    mark(0);
+    int32_t rc = router_logits_entry(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset,
+                                     router_biases, router_biases_offset, router_x, effective_scale, effective_scale_offset,
+                                     per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, d, top_k, logits);
+    if (rc != TF_OK) return rc;
+    tf_routed_blobs routed = {};
+    routed.pool = expert_pool;
+    routed.pool_stride = expert_pool_stride;
+    routed.indices = static_cast<const uint32_t *>(out_indices);
+    routed.num_experts = num_experts;
+    // Three launches when the vector path applies: logits, phase 1 with the selection repeated by every wave, phase 2.
+    const FusedSelect fused = {logits, reinterpret_cast<const uint16_t *>(at(per_expert_scale, per_expert_scale_offset)),
+                               static_cast<uint32_t *>(out_indices), static_cast<half_t *>(out_weights), num_experts};
+    rc = phase1_entry(ctx, stream, &routed, routed_offsets, x, acts, nullptr, 0, false, d, f, top_k, scale_dtype, &fused, timed ? 1 : -1);
+    if (rc == TF_ERR_UNAVAILABLE) {
+        rc = router_select_entry(ctx, stream, per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, top_k, logits);
+        if (rc != TF_OK) return rc;
+        mark(1);
+        rc = phase1_entry(ctx, stream, &routed, routed_offsets, x, acts, nullptr, 0, false, d, f, top_k, scale_dtype);
+    }
+    if (rc != TF_OK) return rc;
+    mark(2);
+    rc = tf_moe_phase2_down_reduce(ctx, stream, &routed, routed_offsets, acts, out_weights, residual, y, d, f, top_k, scale_dtype);
+    mark(3);
+    mark(4);
+    if (timed && rc == TF_OK) ctx->step_timed = true;
+    return rc;
 }
 
 }  // namespace
@@ -701,9 +778,10 @@ int32_t tf_router_gemma4(tf_ctx *ctx, tf_stream stream, const void *weights, uin
                          uint32_t d, uint32_t top_k) {
     int32_t rc = router_logits_entry(ctx, stream, weights, weights_offset, scales, scales_offset, biases, biases_offset, hidden,
                                      effective_scale, effective_scale_offset, per_expert_scale, per_expert_scale_offset,
-                                     out_indices, out_weights, num_experts, d, top_k);
+                                     out_indices, out_weights, num_experts, d, top_k, ctx ? ctx->router_logits : nullptr);
     if (rc != TF_OK) return rc;
-    return router_select_entry(ctx, stream, per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, top_k);
+    return router_select_entry(ctx, stream, per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, top_k,
+                               ctx->router_logits);
 }
 
 int32_t tf_moe_phase1_gate_up_act(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *routed, const tf_expert_offsets *routed_offsets,
@@ -755,39 +833,11 @@ int32_t tf_moe_decode_step(tf_ctx *ctx, tf_stream stream, const void *router_wei
                            const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
                            const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
                            void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype) {
-    TF_REQUIRE(ctx, ctx && expert_pool && out_indices, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: null argument");
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    const bool timed = ctx->step_timing;
-    auto mark = [&](int i) {
-        if (timed) (void)hipEventRecord(ctx->step_events[i], st);
-    };
-    mark(0);
-    int32_t rc = router_logits_entry(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset,
-                                     router_biases, router_biases_offset, router_x, effective_scale, effective_scale_offset,
-                                     per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, d, top_k);
-    if (rc != TF_OK) return rc;
-    tf_routed_blobs routed = {};
-    routed.pool = expert_pool;
-    routed.pool_stride = expert_pool_stride;
-    routed.indices = static_cast<const uint32_t *>(out_indices);
-    routed.num_experts = num_experts;
-    // Three launches when the vector path applies: logits, phase 1 with the selection repeated by every wave, phase 2.
-    const FusedSelect fused = {ctx->router_logits, reinterpret_cast<const uint16_t *>(at(per_expert_scale, per_expert_scale_offset)),
-                               static_cast<uint32_t *>(out_indices), static_cast<half_t *>(out_weights), num_experts};
-    rc = phase1_entry(ctx, stream, &routed, routed_offsets, x, acts, nullptr, 0, false, d, f, top_k, scale_dtype, &fused, 1);
-    if (rc == TF_ERR_UNAVAILABLE) {
-        rc = router_select_entry(ctx, stream, per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, top_k);
-        if (rc != TF_OK) return rc;
-        mark(1);
-        rc = phase1_entry(ctx, stream, &routed, routed_offsets, x, acts, nullptr, 0, false, d, f, top_k, scale_dtype);
-    }
-    if (rc != TF_OK) return rc;
-    mark(2);
-    rc = tf_moe_phase2_down_reduce(ctx, stream, &routed, routed_offsets, acts, out_weights, residual, y, d, f, top_k, scale_dtype);
-    mark(3);
-    mark(4);
-    if (timed && rc == TF_OK) ctx->step_timed = true;
-    return rc;
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: null context");
+    return decode_step_impl(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset, router_biases,
+                            router_biases_offset, router_x, effective_scale, effective_scale_offset, per_expert_scale,
+                            per_expert_scale_offset, expert_pool, expert_pool_stride, num_experts, routed_offsets, x, acts, residual, y,
+                            out_indices, out_weights, d, f, top_k, scale_dtype, ctx->router_logits, true);
 }
 
 int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, uint64_t x_length,

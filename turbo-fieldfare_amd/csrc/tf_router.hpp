@@ -73,6 +73,28 @@ __device__ __forceinline__ float router_row(const uint8_t *w_row, const uint8_t 
     return wave_sum(acc);
 }
 
+// The same row by a whole 256-thread block (d <= 4096, every operand 16-byte aligned): thread t takes chunk t of 16 weights,
+// so the arithmetic after the one memory round trip is a third of a wave-per-row pass at d = 2816; the four wave sums meet in
+// LDS and are added in wave order.  Returns the logit in every thread.  `partial`: 4 floats of LDS.
+template <int SD>
+__device__ __forceinline__ float router_row_block(const uint8_t *w_row, const uint8_t *s_row, const uint8_t *b_row, const half_t *hidden,
+                                                  const uint16_t *eff, int d, float *partial) {
+    const int c = threadIdx.x, chunks = d >> 4;
+    float acc = 0.0f;
+    if (c < chunks) {
+        const u32x4 w = load16(w_row + (size_t)c * 16);
+        const u32x4 ha = load16(hidden + c * 16), hb = load16(hidden + c * 16 + 8);
+        const u32x4 ea = load16(eff + c * 16), eb = load16(eff + c * 16 + 8);
+        const uint16_t sv = *reinterpret_cast<const uint16_t *>(s_row + (c >> 2) * 2);
+        const uint16_t bv = *reinterpret_cast<const uint16_t *>(b_row + (c >> 2) * 2);
+        router_chunk(w, ha, hb, ea, eb, sb_to_f32<SD>(sv), sb_to_f32<SD>(bv), acc);
+    }
+    acc = wave_sum(acc);
+    if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    return ((partial[0] + partial[1]) + partial[2]) + partial[3];
+}
+
 // Top-k over <= 256 fp32 logits by one wave, then softmax over the selected and the per-expert gain.
 // Same ordering as the reference's serial insertion (moe.metal:152-171): score descending, ties to the lower index;
 // NaN and -inf are never selected; an unfilled position reads index 0 with score -inf.
@@ -140,6 +162,76 @@ __device__ __forceinline__ void router_select_lanes(const float *logits, const u
                                                     uint32_t top_k, int lane, uint32_t &sel_index, half_t &sel_weight) {
     if (num_experts <= 128) router_select_lanes<2>(logits, per_expert_scale, num_experts, top_k, lane, sel_index, sel_weight);
     else router_select_lanes<4>(logits, per_expert_scale, num_experts, top_k, lane, sel_index, sel_weight);
+}
+
+// Top-8 of <= 256 logits by a whole 256-thread block, by counting: a candidate's position in the order (score descending,
+// ties to the lower index) is the number of candidates that beat it, and with 128 experts two threads share a candidate's
+// 128 comparisons, so the selection costs the block a few hundred instructions with no serial chain where the one-wave
+// selection above walks eight dependent rounds.  The count ignores ties; when any of the first eight positions is claimed
+// twice or not at all (equal scores, fewer than eight finite logits) the block says so and the caller falls back to the
+// one-wave selection, which is exact in every case.  On success chosen[0..8) holds the expert indices in selection order and
+// cand[e] the logit of expert e (NaN read as -inf).  Every thread of the block must call; ends with a barrier.
+struct RankSelectLds {
+    __attribute__((aligned(16))) float cand[256];
+    uint32_t part[2][128];
+    __attribute__((aligned(16))) uint32_t claims[8];
+};
+__device__ __forceinline__ float rank_select_load(const float *logits, uint32_t num_experts) {
+    const uint32_t c = num_experts <= 128 ? (threadIdx.x & 127) : threadIdx.x;
+    float v = c < num_experts ? logits[c] : -INFINITY;
+    return v;
+}
+__device__ __forceinline__ bool rank_select_block(float my_logit, uint32_t num_experts, RankSelectLds &l, uint32_t *chosen) {
+    const bool two_per_candidate = num_experts <= 128;
+    const uint32_t c = two_per_candidate ? (threadIdx.x & 127) : threadIdx.x;
+    const float v = (my_logit != my_logit) ? -INFINITY : my_logit;
+    l.cand[threadIdx.x] = (two_per_candidate && threadIdx.x >= 128) ? -INFINITY : v;
+    if (threadIdx.x < 8) l.claims[threadIdx.x] = 0u;
+    lds_barrier();
+    uint32_t beaten_by = 0;
+    if (two_per_candidate) {
+        const uint32_t h = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 7));
+        const f32x4 *src = reinterpret_cast<const f32x4 *>(l.cand + 64 * h);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const f32x4 q = src[j];
+            beaten_by += (q[0] > v) + (q[1] > v) + (q[2] > v) + (q[3] > v);
+        }
+        l.part[h][c] = beaten_by;
+        lds_barrier();
+        beaten_by = l.part[0][c] + l.part[1][c];
+    } else {
+        const f32x4 *src = reinterpret_cast<const f32x4 *>(l.cand);
+#pragma unroll 8
+        for (int j = 0; j < 64; ++j) {
+            const f32x4 q = src[j];
+            beaten_by += (q[0] > v) + (q[1] > v) + (q[2] > v) + (q[3] > v);
+        }
+    }
+    const bool owner = !two_per_candidate || threadIdx.x < 128;
+    if (owner && beaten_by < 8u && v > -INFINITY) {
+        chosen[beaten_by] = c;
+        atomicAdd(&l.claims[beaten_by], 1u);
+    }
+    lds_barrier();
+    const u32x4 c0 = *reinterpret_cast<const u32x4 *>(l.claims), c1 = *reinterpret_cast<const u32x4 *>(l.claims + 4);
+    const bool ok = c0[0] == 1u && c0[1] == 1u && c0[2] == 1u && c0[3] == 1u && c1[0] == 1u && c1[1] == 1u && c1[2] == 1u && c1[3] == 1u;
+    return __builtin_amdgcn_readfirstlane((int)ok) != 0;
+}
+
+// The routing weights of a selection made by rank_select_block, computed by one wave exactly as router_select_core's tail
+// does: softmax over the selected scores in selection order, times the per-expert gain.  Lane i < 8 gets selection i.
+__device__ __forceinline__ void rank_select_weights(const RankSelectLds &l, const uint32_t *chosen, const uint16_t *per_expert_scale, int lane,
+                                                    uint32_t &sel_index, half_t &sel_weight) {
+    const uint32_t e = lane < 8 ? chosen[lane] : 0u;
+    const float score = lane < 8 ? l.cand[e] : -INFINITY;
+    const float gain = bf16_to_f32(per_expert_scale[e]);
+    const float max_s = read_lane(score, 0);
+    const float ex = lane < 8 ? expf(score - max_s) : 0.0f;
+    float sum_exp = 0.0f;
+    for (int i = 0; i < 8; ++i) sum_exp += read_lane(ex, i);
+    sel_index = e;
+    sel_weight = (half_t)((ex / sum_exp) * gain);
 }
 
 __device__ __forceinline__ void router_select(const float *logits, const uint16_t *per_expert_scale, uint32_t *out_indices,
