@@ -451,6 +451,26 @@ int32_t tf_moe_decode_step(tf_ctx *ctx, tf_stream stream,
                            void *out_indices, void *out_weights,
                            uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype);
 
+/* No counterpart in the reference.  tf_moe_decode_step for callers that cannot allocate or wait for an allocation
+ * (code under HIP graph capture, tight serving loops, harnesses that forbid hipMalloc): same arguments, same kernels,
+ * bit-identical results, but the router logits between the launches live in a load-time device array of 256 floats (one
+ * copy per GPU, held until the process ends) instead of the context's buffer, and the call neither allocates, frees nor
+ * records timing events.  num_experts > 256 returns TF_ERR_SCRATCH_TOO_SMALL.  Every call on a GPU shares that GPU's
+ * array: calls that overlap on one GPU (two streams, two contexts) race; calls on one stream do not.  Nothing in the
+ * array needs clearing between calls: a call writes logits[0..num_experts) before it reads them and reads nothing beyond. */
+int32_t tf_moe_decode_step_static(tf_ctx *ctx, tf_stream stream,
+                                  const void *router_weights, uint64_t router_weights_offset,
+                                  const void *router_scales, uint64_t router_scales_offset,
+                                  const void *router_biases, uint64_t router_biases_offset,
+                                  const void *router_x,
+                                  const void *effective_scale, uint64_t effective_scale_offset,
+                                  const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                                  const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                  const tf_expert_offsets *routed_offsets,
+                                  const void *x, void *acts, const void *residual, void *y,
+                                  void *out_indices, void *out_weights,
+                                  uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype);
+
 /* ---- lm_head ----------------------------------------------------------------------------------------------------------- */
 /* LMHeadChainInt4.encodeGreedyDecode (Kernels/Fusions/LMHeadChainInt4.swift:53-122) -> rmsnorm_bf16w,
  * lm_head_greedy_int4_rows_chunk_raw, lm_head_greedy_int4_rows_reduce (Metal/Sampling/logit.metal:692-787):

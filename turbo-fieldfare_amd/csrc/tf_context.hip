@@ -51,6 +51,7 @@ int32_t tf_ctx_create(int32_t device, tf_ctx **out_ctx) {
     // the reference's model (Infrastructure/ModelIO/ModelTypes.swift:78-100) at the largest block sizes this library is run at
     const tf_scratch_limits defaults = {262144u, 2048u, 256u, 2112u, 16u, 512u, 128u};
     ok = ok && tf_ctx_reserve(ctx, &defaults) == TF_OK;
+    ok = ok && moe_static_scratch_setup(ctx) == TF_OK;
     if (const char *env = getenv("TF_STREAM_BLOCKS_PER_CU")) {
         const int v = atoi(env);
         if (v >= 1 && v <= 8) ctx->stream_blocks_per_cu = v;

@@ -14,6 +14,7 @@ struct tf_ctx {
     int stream_blocks_per_cu = 2;       // 256-thread blocks per CU launched by the persistent row streamers
     // wrapper-owned scratch, as the reference's kernel classes own theirs
     float *router_logits = nullptr;     // 256 floats (MoE.swift:92-99)
+    float *static_router_logits = nullptr;   // this device's copy of the load-time scratch of tf_moe_decode_step_static
     void *head_x_normed = nullptr;      // kMaxHeadD halves (LMHeadChainInt4.swift:38-51)
     float *head_summaries = nullptr;    // kMaxHeadWaves x {value, index bits}
     float *head_logits = nullptr;       // fp32 logits of the unaligned lm_head path, limits.max_vocab of them
@@ -68,6 +69,9 @@ inline int32_t scratch_too_small(tf_ctx *ctx, const char *who, size_t need, size
     return fail(ctx, TF_ERR_SCRATCH_TOO_SMALL, "%s: needs %zu bytes of wrapper scratch, the context holds %zu: raise the limits with tf_ctx_reserve",
                 who, need, have);
 }
+
+// Looks up this device's copy of the load-time router-logit scratch (tf_moe.hip); the context's device must be current.
+int32_t moe_static_scratch_setup(tf_ctx *ctx);
 
 // Sizes of the wrapper scratch as functions of the limits, each defined beside the entry points that use the buffer.
 size_t sample_scratch_bytes_for(uint32_t vocab);                                    // tf_sampling.hip

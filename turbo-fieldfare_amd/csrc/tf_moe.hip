@@ -4,6 +4,24 @@
 
 using namespace tfk;
 
+// Router logits of tf_moe_decode_step_static: device memory that exists from load time on, one copy per GPU, so that entry
+// point never allocates.  Host code never uses the array's name as an address: tf_ctx_create asks the runtime for the
+// address of this device's copy (moe_static_scratch_setup) and every launch passes that pointer.
+constexpr uint32_t kStaticMaxExperts = 256;
+static __device__ __align__(256) float scratch[kStaticMaxExperts];
+
+namespace tfk {
+
+int32_t moe_static_scratch_setup(tf_ctx *ctx) {
+    void *ptr = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));   // the context's device is current here
+    if (e != hipSuccess || !ptr) return fail(ctx, TF_ERR_DEVICE, "moe static scratch: %s", hipGetErrorString(e));
+    ctx->static_router_logits = static_cast<float *>(ptr);
+    return TF_OK;
+}
+
+}  // namespace tfk
+
 namespace {
 
 struct RoutedArg {
@@ -838,6 +856,24 @@ int32_t tf_moe_decode_step(tf_ctx *ctx, tf_stream stream, const void *router_wei
                             router_biases_offset, router_x, effective_scale, effective_scale_offset, per_expert_scale,
                             per_expert_scale_offset, expert_pool, expert_pool_stride, num_experts, routed_offsets, x, acts, residual, y,
                             out_indices, out_weights, d, f, top_k, scale_dtype, ctx->router_logits, true);
+}
+
+int32_t tf_moe_decode_step_static(tf_ctx *ctx, tf_stream stream, const void *router_weights, uint64_t router_weights_offset,
+                                  const void *router_scales, uint64_t router_scales_offset, const void *router_biases,
+                                  uint64_t router_biases_offset, const void *router_x, const void *effective_scale,
+                                  uint64_t effective_scale_offset, const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                                  const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                  const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
+                                  void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "moe_decode_step_static: null context");
+    TF_REQUIRE(ctx, num_experts <= kStaticMaxExperts, TF_ERR_SCRATCH_TOO_SMALL,
+               "moe_decode_step_static: %u experts exceed the %u router logits of the static scratch", num_experts, kStaticMaxExperts);
+    TF_REQUIRE(ctx, ctx->static_router_logits != nullptr, TF_ERR_DEVICE, "moe_decode_step_static: static scratch was not set up on this device");
+    // every logit that is read has been written by this call's router launch, so nothing needs clearing between calls
+    return decode_step_impl(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset, router_biases,
+                            router_biases_offset, router_x, effective_scale, effective_scale_offset, per_expert_scale,
+                            per_expert_scale_offset, expert_pool, expert_pool_stride, num_experts, routed_offsets, x, acts, residual, y,
+                            out_indices, out_weights, d, f, top_k, scale_dtype, ctx->static_router_logits, false);
 }
 
 int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, uint64_t x_length,
