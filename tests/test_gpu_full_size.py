@@ -1,0 +1,218 @@
+"""The BASELINE configurations at their full sizes on the GPU, through the C ABI:
+config 2 (lm_head 262144 x 2816: persistent tiles, refills, the 64 argmax cells and the ticket all in play),
+config 3 (a few tokens over the 128-expert pool) and config 4 (2048 tokens x 128 experts, Zipf routing, matrix cores).
+Planted rows follow LMHeadChainInt4Tests.swift:136-193; the prefill checks follow PrefillGroupedRoutedMoETests+Execution."""
+import ctypes as C
+
+import numpy as np
+import pytest
+import torch
+
+import refcases
+from gpu_helpers import ctx, dev, host, tfk, within_north_star, zeros_bytes
+from oracle import tfo
+from test_gpu_prefill import device_grouping
+
+pytestmark = pytest.mark.gpu
+D, F, E, TOPK, V = 2816, 704, 128, 8, 262144
+
+
+# ------------------------------------------------------------------------------------------------ config 2
+@pytest.fixture(scope="module")
+def head():
+    rng = np.random.default_rng(0x1E4D)
+    W = rng.integers(0, 256, (V, D // 2), dtype=np.uint8)
+    s = rng.uniform(0.005, 0.02, (V, D // 64)).astype(np.float32)
+    b = rng.uniform(-0.1, 0.1, (V, D // 64)).astype(np.float32)
+    hidden = refcases.normal_f16(D, 0x1E4D)
+    norm = tfo.bf16_bits_array(rng.uniform(0.5, 1.5, D).astype(np.float32))
+    return dict(W=W, s=s, b=b, hidden=hidden, norm=norm)
+
+
+def for_device(bits_bf16, kind):
+    """The oracle reads bf16 scales.  Every bf16 value in fp16's range is also an fp16 value, so the fp16 run gets the same
+    numbers in the other encoding and one reference serves both."""
+    if kind == tfk.TF_BF16:
+        return bits_bf16
+    return tfo.bf16_array_to_float(bits_bf16.ravel()).astype(np.float16).view(np.uint16).reshape(bits_bf16.shape)
+
+
+def plant(W, S, B, rows, x_bits):
+    """Rows that beat every random row by construction: weight 15 where the activation is positive, 0 elsewhere, the
+    largest scale, no bias.  Returns copies; the originals stay random."""
+    W, S, B = W.copy(), S.copy(), B.copy()
+    nib = np.where(tfo.from_f16_bits(x_bits) > 0, 15, 0).astype(np.uint8)
+    packed = (nib[0::2] | (nib[1::2] << 4)).astype(np.uint8)
+    for r in rows:
+        W[r], S[r], B[r] = packed, tfo.bf16_bits(0.02), tfo.bf16_bits(0.0)
+    return W, S, B
+
+
+def gpu_head(head, dW, S, B, kind, logits=False):
+    k = ctx()
+    dh, dn, dS, dB = dev(head["hidden"]), dev(head["norm"]), dev(for_device(S, kind)), dev(for_device(B, kind))
+    tok = zeros_bytes(4, 0xEE)
+    k.lm_head_greedy(dh, dn, dW, dS, dB, tok, D, V, scale_dtype=kind)
+    out = None
+    if logits:
+        out = zeros_bytes(V * 4)
+        k.check(k.lib.tf_lm_head_logits_int4(k.handle, None, dh.data_ptr(), 0, dn.data_ptr(), 0, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0,
+                                             out.data_ptr(), 0, D, V, 1e-6, kind, tfk.TF_FP32))
+        out = host(out, np.float32, V)
+    return int(host(tok, np.uint32, 1)[0]), out
+
+
+@pytest.mark.parametrize("kind", [tfk.TF_BF16, tfk.TF_FP16], ids=["bf16", "fp16"])
+def test_lm_head_full_vocabulary(head, kind):
+    W = head["W"]
+    S, B = tfo.bf16_bits_array(head["s"]).reshape(head["s"].shape), tfo.bf16_bits_array(head["b"]).reshape(head["b"].shape)
+
+    def cpu(Wc, Sc, Bc, **kw):
+        return tfo.lm_head_cpu_greedy(head["hidden"], head["norm"], Wc, Sc, Bc, threads=8, **kw)
+
+    # random rows: the token and every fp32 logit
+    tok_ref, logits_ref = cpu(W, S, B, want_logits=True)
+    tok, logits = gpu_head(head, dev(W), S, B, kind, logits=True)
+    assert tok == tok_ref
+    assert tfo.rel_error(logits, logits_ref) < tfo.Tolerance.fp16Reduction
+    assert within_north_star(logits, logits_ref)
+    assert int(np.argmax(logits)) == tok_ref
+    # two identical winners far apart, an odd and an even row (different places in their tiles): the lower index
+    Wp, Sp, Bp = plant(W, S, B, [17, 262000], head["hidden"])
+    dWp = dev(Wp)
+    assert cpu(Wp, Sp, Bp) == 17
+    assert gpu_head(head, dWp, Sp, Bp, kind)[0] == 17
+    # the first of the pair produces a non-finite logit (one of its scales is +inf): skipped, the far one wins
+    Sn = Sp.copy()
+    Sn[17, 3] = 0x7F80
+    assert cpu(Wp, Sn, Bp) == 262000
+    assert gpu_head(head, dWp, Sn, Bp, kind)[0] == 262000
+    del dWp
+    # a single winner three rows before the end
+    Wt, St, Bt = plant(W, S, B, [V - 3], head["hidden"])
+    assert cpu(Wt, St, Bt) == V - 3
+    assert gpu_head(head, dev(Wt), St, Bt, kind)[0] == V - 3
+
+
+# ------------------------------------------------------------------------------------------------ configs 3 and 4
+@pytest.fixture(scope="module")
+def pool():
+    """The 128-expert pool of the production shape, one blob per expert in the reference's order."""
+    blobs, off = [], None
+    for e in range(E):
+        blob, off = tfo.make_blob(refcases.synthetic_int4(F, D, 0x9001 + e, "g"), refcases.synthetic_int4(F, D, 0x9001 + e, "u"),
+                                  refcases.synthetic_int4(D, F, 0x9001 + e, "d"))
+        blobs.append(blob)
+    stride = (blobs[0].size + 16383) // 16384 * 16384
+    pool_np = np.zeros((E, stride), np.uint8)
+    for e, b in enumerate(blobs):
+        pool_np[e, :b.size] = b
+    return dict(blobs=blobs, off=off, stride=stride, flat=pool_np.ravel(), dev=dev(pool_np))
+
+
+SENTINEL = 0xD630
+
+
+def run_block(pool, hidden, idx, w_bits):
+    """device grouping -> grouped experts over the resident pool -> token-major reduce."""
+    T = hidden.shape[0]
+    k = ctx()
+    g = device_grouping(idx, w_bits, T, TOPK, E)
+    n = T * TOPK
+    acts = zeros_bytes(n * F * 2)
+    partials = torch.full((n * D,), SENTINEL, dtype=torch.int16, device="cuda").view(torch.uint8) if SENTINEL < 0x8000 else \
+        torch.full((n * D,), SENTINEL - 0x10000, dtype=torch.int16, device="cuda").view(torch.uint8)
+    h2 = zeros_bytes(T * D * 2)
+    koff = tfk.ExpertOffsets(*pool["off"].as_tuple())
+    d_hidden, d_w = dev(hidden), dev(np.ascontiguousarray(w_bits, np.uint16))
+    k.check(k.lib.tf_prefill_grouped_routed_moe_resident(k.handle, None, d_hidden.data_ptr(), 0, D, g["sorted_pairs"].data_ptr(),
+                                                         g["chunks"].data_ptr(), g["n_chunks"].data_ptr(), g["cap"], n, pool["dev"].data_ptr(),
+                                                         pool["stride"], E, C.byref(koff), acts.data_ptr(), partials.data_ptr(), D, F, TOPK, tfk.TF_BF16))
+    k.check(k.lib.tf_prefill_moe_reduce_token_major(k.handle, None, partials.data_ptr(), 0, d_w.data_ptr(), 0, h2.data_ptr(), 0, T, TOPK, D))
+    sp = host(g["sorted_pairs"], np.uint32, n * 4).reshape(n, 4)
+    return dict(sorted_pairs=np.array([tuple(r) for r in sp], tfo.PAIR_DTYPE), partials=host(partials, np.uint16, n * D).reshape(T, TOPK, D),
+                h2=tfo.from_f16_bits(host(h2, np.uint16, T * D)).reshape(T, D), counts=host(g["counts"], np.uint32, E),
+                n_chunks=int(host(g["n_chunks"], np.uint32, 1)[0]))
+
+
+def oracle_rows(pool, hidden, w_bits, r, tokens):
+    """partials and h2 of the listed tokens from the oracle (the pairs of those tokens only)."""
+    T = hidden.shape[0]
+    sp = r["sorted_pairs"]
+    pairs = sp[np.isin(sp["token"], tokens)]
+    want = tfo.prefill_route_partials(pairs, T, hidden.ravel(), D, pool["flat"], pool["stride"], pool["off"], TOPK, D, F, fill_bits=0,
+                                      threads=8).reshape(T, TOPK, D)
+    h2 = tfo.from_f16_bits(tfo.prefill_reduce_token_major(want.ravel(), np.ascontiguousarray(w_bits, np.uint16).ravel(), T, TOPK, D)).reshape(T, D)
+    return want, h2
+
+
+def decode_rows(pool, hidden, idx, w_bits):
+    """Every token through the batch-1 kernels (phase 1 + phase 2 with the token's own experts)."""
+    T = hidden.shape[0]
+    k = ctx()
+    koff = tfk.ExpertOffsets(*pool["off"].as_tuple())
+    d_idx, d_x, d_w = dev(np.ascontiguousarray(idx, np.uint32)), dev(hidden), dev(np.ascontiguousarray(w_bits, np.uint16))
+    res, acts, y = zeros_bytes(D * 2), zeros_bytes(TOPK * F * 2), zeros_bytes(T * D * 2)
+    for t in range(T):
+        routed = tfk.RoutedBlobs()
+        routed.pool, routed.pool_stride, routed.indices, routed.num_experts = pool["dev"].data_ptr(), pool["stride"], d_idx.data_ptr() + t * TOPK * 4, E
+        k.check(k.lib.tf_moe_phase1_gate_up_act(k.handle, None, C.byref(routed), C.byref(koff), d_x.data_ptr() + t * D * 2, acts.data_ptr(), D, F, TOPK,
+                                                tfk.TF_BF16))
+        k.check(k.lib.tf_moe_phase2_down_reduce(k.handle, None, C.byref(routed), C.byref(koff), acts.data_ptr(), d_w.data_ptr() + t * TOPK * 2,
+                                                res.data_ptr(), y.data_ptr() + t * D * 2, D, F, TOPK, tfk.TF_BF16))
+    return tfo.from_f16_bits(host(y, np.uint16, T * D)).reshape(T, D)
+
+
+def test_prefill_2048_tokens_over_128_experts(pool):
+    T = 2048
+    rng = np.random.default_rng(0xC0F4)
+    p = 1.0 / np.arange(1, E + 1) ** 1.1
+    p /= p.sum()
+    idx = np.stack([rng.choice(E, size=TOPK, replace=False, p=p) for _ in range(T)]).astype(np.uint32)
+    w_bits = tfo.to_f16_bits(rng.dirichlet(np.ones(TOPK), T).astype(np.float32)).reshape(T, TOPK)
+    hidden = rng.standard_normal((T, D)).astype(np.float16).view(np.uint16)
+    r = run_block(pool, hidden, idx, w_bits)
+    counts = r["counts"]
+    assert counts.sum() == T * TOPK and counts.max() > 4 * 128 and r["n_chunks"] > E       # several full 128-pair chunks of one expert
+    # every route row was written
+    assert not np.any(np.all(r["partials"] == SENTINEL, axis=2))
+    # oracle on tokens of the most popular expert (first, middle and last chunk of its group), of the rarest expert, and a few more
+    sp = r["sorted_pairs"]
+    hot, rare = int(np.argmax(counts)), int(np.argmin(np.where(counts > 0, counts, 1 << 30)))
+    hot_tokens = sp["token"][sp["expert"] == hot]
+    pick = np.unique(np.concatenate([hot_tokens[:6], hot_tokens[len(hot_tokens) // 2 - 3:len(hot_tokens) // 2 + 3], hot_tokens[-6:],
+                                     sp["token"][sp["expert"] == rare][:4], [0, T - 1]])).astype(np.uint32)
+    want_p, want_h2 = oracle_rows(pool, hidden, w_bits, r, pick)
+    scale = float(np.max(np.abs(tfo.from_f16_bits(want_p[pick]))))
+    for t in pick:
+        assert within_north_star(tfo.from_f16_bits(r["partials"][t]), tfo.from_f16_bits(want_p[t]), abs_=2e-3 * max(1.0, scale)), t
+        assert within_north_star(r["h2"][t], want_h2[t], abs_=2e-3 * max(1.0, scale)), t
+    # every token of the block against the batch-1 kernels on that token
+    dec = decode_rows(pool, hidden, idx, w_bits)
+    err = np.max(np.abs(dec - r["h2"]), axis=1)
+    bound = 4e-3 * np.maximum(1.0, np.max(np.abs(dec), axis=1))
+    assert np.all(err <= bound), (int(np.argmax(err - bound)), float(np.max(err - bound)))
+    # and the batch-1 kernels against the all-fp32 reference on three of the sampled tokens
+    for t in pick[:3]:
+        ref = tfo.moe_apply_streamed_routed([pool["blobs"][int(e)] for e in idx[t]], pool["off"], tfo.from_f16_bits(hidden[t]), np.zeros(D, np.float32),
+                                            tfo.from_f16_bits(w_bits[t]), D, F, threads=8)
+        assert tfo.rel_error(r["h2"][t], ref) < tfo.Tolerance.fp16ChainedReduction
+
+
+@pytest.mark.parametrize("M", [2, 4, 8, 16])
+def test_few_tokens_over_the_128_expert_pool(pool, M):
+    rng = np.random.default_rng(0x3300 + M)
+    logits = rng.standard_normal((M, E))                     # seeded random router logits: experts are shared across tokens
+    idx = np.argsort(-logits, axis=1, kind="stable")[:, :TOPK].astype(np.uint32)
+    top = np.take_along_axis(logits, idx.astype(np.int64), axis=1)
+    prob = np.exp(top - top.max(axis=1, keepdims=True))
+    w_bits = tfo.to_f16_bits((prob / prob.sum(axis=1, keepdims=True)).astype(np.float32)).reshape(M, TOPK)
+    hidden = rng.standard_normal((M, D)).astype(np.float16).view(np.uint16)
+    r = run_block(pool, hidden, idx, w_bits)
+    assert not np.any(np.all(r["partials"] == SENTINEL, axis=2))
+    want_p, want_h2 = oracle_rows(pool, hidden, w_bits, r, np.arange(M, dtype=np.uint32))
+    scale = float(np.max(np.abs(tfo.from_f16_bits(want_p))))
+    assert within_north_star(tfo.from_f16_bits(r["partials"]), tfo.from_f16_bits(want_p), abs_=1e-3 * max(1.0, scale))
+    assert within_north_star(r["h2"], want_h2, abs_=1e-3 * max(1.0, scale))
+    dec = decode_rows(pool, hidden, idx, w_bits)
+    assert np.max(np.abs(dec - r["h2"])) <= 4e-3 * max(1.0, float(np.max(np.abs(dec))))

@@ -158,7 +158,7 @@ int32_t tf_lm_head_greedy_int4(tf_ctx *ctx, tf_stream stream, const void *hidden
     const half_t *hid = reinterpret_cast<const half_t *>(at(hidden, hidden_offset));
     const uint16_t *nw = reinterpret_cast<const uint16_t *>(at(norm_weight, norm_offset));
     const half_t *xn = static_cast<const half_t *>(ctx->head_x_normed);
-    const LongPlan plan = plan_long_rows((int)d);
+    const LongPlan plan = plan_long_rows((int)d, 2);   // up to two rows a tile: a row's sum is then independent of its place in the tile
     const bool rows_fast = aligned16(w) && d > 1024 && plan.rt > 0;
     const bool fuse_norm = rows_fast && aligned16(hid) && aligned16(nw) && d <= (uint32_t)kMaxFusedNormD;
     if (!fuse_norm) {

@@ -50,22 +50,38 @@ struct RowStream {
     float xs[NP];
     uint32_t row_bytes, sb_row_bytes;   // wave-uniform
 
-    // chunk -> (row, column) map of this lane; independent of the data
+    // chunk -> (row, column) map of this lane; independent of the data.
+    // RT == 2 places the second row as the first row's mirror image: chunk c of row 0 sits in lane c % 64 of pass c / 64,
+    // chunk c of row 1 in lane (c + 32) % 64 of pass NP - 1 - c / 64.  Each lane of row 1 then accumulates the same chunks
+    // as the lane 32 places away does for row 0, and the wave sum is symmetric under that swap of half-waves (its last
+    // step adds the two half-wave sums), so a row's dot product does not depend on its position in the tile: two rows
+    // with identical bytes give identical sums, and an argmax over rows breaks ties exactly by index.  plan_long_rows
+    // only offers RT == 2 where the two images do not overlap.  Other RT use the flat order (chunk 64 p + lane).
     __device__ __forceinline__ void init_map(int k, int lane) {
         const int nch = k >> 5;  // 16-byte chunks per row
         const int groups = k >> 6;
-        const int tot = RT * nch;
         row_bytes = (uint32_t)k >> 1;
         sb_row_bytes = (uint32_t)groups * 2u;
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
-            const int c = lane + 64 * p;
-            const bool valid = c < tot;
-            const int r = c / nch;
-            const int cc = c - r * nch;
+            int r, cc;
+            bool valid;
+            if constexpr (RT == 2) {
+                const int c0 = lane + 64 * p;
+                const int c1 = ((lane + 32) & 63) + 64 * (NP - 1 - p);
+                const bool v0 = c0 < nch;
+                valid = v0 || c1 < nch;
+                r = v0 ? 0 : 1;
+                cc = v0 ? c0 : c1;
+            } else {
+                const int c = lane + 64 * p;
+                valid = c < RT * nch;
+                r = c / nch;
+                cc = c - r * nch;
+            }
             col[p] = valid ? cc : 0;
             row[p] = valid ? r : -1;
-            woff[p] = (uint32_t)c * 16u;                                   // past the tile when !valid: reads zeros
+            woff[p] = valid ? (uint32_t)r * row_bytes + (uint32_t)cc * 16u : 0xFFFFFFF0u;   // past the tile when !valid: reads zeros
             sboff[p] = valid ? (uint32_t)(r * groups + (cc >> 1)) * 2u : 0xFFFFFFF0u;
         }
     }
@@ -347,19 +363,26 @@ __device__ __forceinline__ float generic_row_dot8(const uint8_t *w_row, const ui
     return wave_sum(acc);
 }
 
-// Picks the rows-per-tile and pass count of RowStream for a given K: best lane utilisation with NP <= 4.
+// Picks the rows-per-tile and pass count of RowStream for a given K: best lane utilisation with NP <= 4 and RT <= max_rt.
+// RT == 2 needs the two mirrored row images of RowStream::init_map to be disjoint: either each row has passes of its own
+// (2 * passes per row == NP) or the shared middle pass holds at most 32 chunks of each row.
 struct LongPlan {
     int rt, np;
 };
-inline LongPlan plan_long_rows(int k) {
+inline LongPlan plan_long_rows(int k, int max_rt = 4) {
     const int nch = k / 32;
     LongPlan best{0, 0};
     double best_util = 0.0;
     const int rts[3] = {1, 2, 4};
     for (int i = 0; i < 3; ++i) {
         const int rt = rts[i];
+        if (rt > max_rt) continue;
         const int np = (rt * nch + 63) / 64;
         if (np > 4) continue;
+        if (rt == 2) {
+            const int per_row = (nch + 63) / 64, tail = nch % 64;
+            if (2 * per_row != np && !(tail != 0 && tail <= 32)) continue;
+        }
         const double util = (double)(rt * nch) / (64.0 * np);
         if (util > best_util + 1e-9) {
             best_util = util;
