@@ -36,6 +36,10 @@ __device__ __forceinline__ uint32_t uniform_u32(uint32_t v) { return (uint32_t)_
 // branches.  The descriptor ends where the tile (or the matrix) ends: lanes without a chunk in the last pass and rows
 // past the end of the matrix read zeros and contribute nothing.
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
+// Cache policy of the packed-weight loads: non-temporal.  A launch reads every weight byte once, so keeping the lines in L2
+// only evicts what is reused (activations, scales); a plain streaming read measures 7.0-7.2 TB/s with this hint against
+// 6.5 TB/s without it, and the vocabulary-sized head 64 us against 69 us.
+constexpr int kStreamOnce = 2;
 __device__ __forceinline__ rsrc_t make_rsrc(const void *base, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
 }
@@ -138,7 +142,7 @@ struct RowStream {
         const rsrc_t rb = make_rsrc(b_tile, nr * sb_row_bytes);
 #pragma unroll
         for (int p = 0; p < NP; ++p) {
-            t.w[p] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, woff[p], 0, 0));
+            t.w[p] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, woff[p], 0, kStreamOnce));
             t.s[p] = __builtin_amdgcn_raw_buffer_load_b16(rs, sboff[p], 0, 0);
             t.b[p] = __builtin_amdgcn_raw_buffer_load_b16(rb, sboff[p], 0, 0);
         }
@@ -299,7 +303,7 @@ struct ShortRows {
         const long r = row0 + half;
         if (col >= 0 && r < rows) {
             const int groups = k >> 6;
-            t.w = load16(w + (size_t)r * (k >> 1) + (size_t)col * 16);
+            t.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(w + (size_t)r * (k >> 1) + (size_t)col * 16));
             t.s = *reinterpret_cast<const uint16_t *>(s + ((size_t)r * groups + (col >> 1)) * 2);
             t.b = *reinterpret_cast<const uint16_t *>(b + ((size_t)r * groups + (col >> 1)) * 2);
         }
