@@ -101,6 +101,8 @@ def main():
     ap.add_argument("--only-small-m", type=int, nargs="+", metavar="M",
                     help="run nothing but the few-token routed-MoE measurement at these token counts and print its JSON "
                          "(a short program whose launches a profiler can attribute to one size)")
+    ap.add_argument("--only-prefill-2048", action="store_true",
+                    help="run nothing but the 2048-token prefill measurement (configs[4]) and print its JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -116,9 +118,13 @@ def main():
     offs, payload, stride = expert_layout()
     off = tfk.ExpertOffsets(*offs)
     layers = [make_layer(torch, gen, offs, stride) for _ in range(args.layers)]
-    if args.only_small_m:
-        only = multi_token_extras(torch, tfk, k, gen, k.lib, k.handle, torch.cuda.current_stream().cuda_stream, layers[0], offs, stride,
-                                  small_sizes=tuple(args.only_small_m), small_only=True)
+    global TIMING_STREAM
+    side = torch.cuda.Stream()            # default priority; everything timed is recorded on it
+    TIMING_STREAM = side
+    if args.only_small_m or args.only_prefill_2048:
+        only = multi_token_extras(torch, tfk, k, gen, k.lib, k.handle, side.cuda_stream, layers[0], offs, stride,
+                                  small_sizes=tuple(args.only_small_m or ()), small_only=not args.only_prefill_2048,
+                                  prefill_only=bool(args.only_prefill_2048))
         print(json.dumps(only))
         return
     n_hidden = 64
@@ -128,12 +134,11 @@ def main():
     acts = torch.zeros(TOPK * F_MOE, dtype=torch.float16, device="cuda")
     residual = torch.zeros(D, dtype=torch.float16, device="cuda")
     y = torch.zeros((n_hidden, D), dtype=torch.float16, device="cuda")
-    stream = torch.cuda.current_stream().cuda_stream
     lib, h = k.lib, k.handle
 
     import ctypes as C
 
-    def step(i):
+    def step(i, stream):
         li, hi = i % args.layers, i % n_hidden
         pool, r = layers[li]
         hp = hidden.data_ptr() + hi * D * 2
@@ -146,46 +151,66 @@ def main():
         if rc != 0:
             raise RuntimeError("kernel call failed: " + k.last_error())
 
-    def run_steps(first, count):
+    def run_steps(first, count, stream):
         for j in range(count):
-            step(first + j)
+            step(first + j, stream)
 
     # ---- the decode loop is launch-bound on the host (3 short kernels per step), so the steps are captured once
     # into HIP graphs and replayed: `graph_steps` steps per graph, plus one remainder graph, exactly `steps` in all.
+    # One ROUND = exactly `steps` steps; rounds repeat until MIN_TIMED_MS of device time have passed (with the driver's
+    # --steps 20 a single round lasts 0.3 ms, far too short a sample) and the median round is reported.
     graph_steps = min(64, args.steps)
     n_full, rem = divmod(args.steps, graph_steps)
-    side = torch.cuda.Stream()            # default priority
     graphs = {}
-    run_steps(0, args.warmup)             # untimed warm-up (eager)
-    torch.cuda.synchronize()
     with torch.cuda.stream(side):
+        run_steps(0, args.warmup, side.cuda_stream)   # untimed warm-up (eager)
+        side.synchronize()
         for count in {graph_steps, rem} - {0}:
             g = torch.cuda.CUDAGraph()
-            stream = torch.cuda.current_stream().cuda_stream
             with torch.cuda.graph(g, stream=side):
-                stream = torch.cuda.current_stream().cuda_stream
-                run_steps(0, count)
+                run_steps(0, count, side.cuda_stream)
             graphs[count] = g
-        stream = torch.cuda.current_stream().cuda_stream
         graphs[graph_steps].replay()      # one untimed replay
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
+        side.synchronize()
+
+    def one_round():
         for _ in range(n_full):
             graphs[graph_steps].replay()
         if rem:
             graphs[rem].replay()
-        torch.cuda.synchronize()
-        elapsed = time.perf_counter() - t0
-    stream = torch.cuda.current_stream().cuda_stream
-    ms_per_step = elapsed * 1e3 / args.steps
+    rounds_ms, wall_ms = replay_rounds(torch, side, one_round)
+    ms_per_step = float(np.median(rounds_ms)) / args.steps
+    ms_per_step_wall = wall_ms / (len(rounds_ms) * args.steps)
     value = STEP_BYTES / (ms_per_step * 1e-3) / 1e9
+    stream = side.cuda_stream
 
     # the same loop launched call by call (no graph): what a host that encodes every step itself would see
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    run_steps(args.warmup, args.steps)
-    torch.cuda.synchronize()
-    ms_per_step_eager = (time.perf_counter() - t0) * 1e3 / args.steps
+    with torch.cuda.stream(side):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_steps(args.warmup, max(args.steps, 256), stream)
+        torch.cuda.synchronize()
+        ms_per_step_eager = (time.perf_counter() - t0) * 1e3 / max(args.steps, 256)
+
+    # ---- latency floor of the step: three dependent launches of the step's grid shapes that move no data, plus the step's
+    # bytes at the rate a plain streaming read reaches in this run.  The step cannot go below that with three launches.
+    words = torch.zeros(8, dtype=torch.int32, device="cuda")
+    wp0 = words.data_ptr()
+
+    def empty_chain(i):
+        rc = lib.tf_bench_empty_launch(h, stream, E, 256, wp0, wp0 + 4)                          # router: one block per expert row
+        rc |= lib.tf_bench_empty_launch(h, stream, TOPK * (F_MOE // 2) // 4, 256, wp0 + 4, wp0 + 8)   # phase 1: 704 blocks
+        rc |= lib.tf_bench_empty_launch(h, stream, D // 8, 512, wp0 + 8, wp0)                     # phase 2: 352 blocks
+        assert rc == 0, k.last_error()
+    empty_chain_us = time_loop(torch, empty_chain, 64)
+    read_bufs = [torch.randint(0, 256, (400 << 20,), dtype=torch.uint8, device="cuda", generator=gen) for _ in range(2)]
+
+    def stream_read(i):
+        assert lib.tf_bench_stream_read(h, stream, read_bufs[i % 2].data_ptr(), 400 << 20, wp0 + 16) == 0, k.last_error()
+    read_us = time_loop(torch, stream_read, 10)
+    read_gbps = (400 << 20) / (read_us * 1e-6) / 1e9
+    del read_bufs
+    latency_floor_us = empty_chain_us + STEP_BYTES / (read_gbps * 1e9) * 1e6
 
     # ---- per-kernel durations: the library brackets the step's three launches with HIP events on the launch stream
     # (eager launches; a spin kernel is queued first so that the host is ahead of the GPU and the events bracket
@@ -196,7 +221,7 @@ def main():
     for i0 in range(0, n_ev, 8):
         torch.cuda._sleep(int(2.4e9 * 0.002))
         for i in range(i0, min(i0 + 8, n_ev)):
-            step(args.warmup + i)
+            step(args.warmup + i, torch.cuda.current_stream().cuda_stream)
             times.append(None)
         times[-1] = k.last_step_timing()      # only the last step of a burst keeps its events
     k.set_step_timing(False)
@@ -222,8 +247,16 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "phase1_long_kernel<2,3,bf16,fused top-8> (expert selection + gate/up/GeGLU of 8 experts)",
                      "achieved": round(p1_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(p1_gbps / HBM_PEAK_GBPS, 4), "traffic": PHASE1_TRAFFIC_BYTES,
-                     "algorithmic_bytes_per_launch": PHASE1_BYTES, "avg_launch_us": round(t_p1, 3)},
-        "launch": f"HIP graph replay, {graph_steps} steps per graph",
+                     "algorithmic_bytes_per_launch": PHASE1_BYTES, "avg_launch_us": round(t_p1, 3),
+                     "latency_floor_us": round(latency_floor_us, 3),
+                     "latency_floor": {"what": "three dependent launches of the step's grid shapes that move no data + the step's "
+                                               "algorithmic bytes at the plain streaming-read rate, both measured in this run",
+                                       "empty_three_launch_chain_us": round(empty_chain_us, 3),
+                                       "stream_read_GBps": round(read_gbps, 1), "stream_read_frac_of_peak": round(read_gbps / HBM_PEAK_GBPS, 4),
+                                       "step_us": round(ms_per_step * 1e3, 3),
+                                       "step_over_floor": round(ms_per_step * 1e3 / latency_floor_us, 3)}},
+        "launch": f"HIP graph replay, {graph_steps} steps per graph; {len(rounds_ms)} rounds of {args.steps} steps, median round reported",
+        "ms_per_step_wallclock_all_rounds": round(ms_per_step_wall, 6),
         "step_per_s": round(1e3 / ms_per_step, 1),
         "ms_per_step_eager_launch": round(ms_per_step_eager, 6),
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
@@ -247,20 +280,59 @@ def main():
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(torch, layers, hidden, idx, wts, y, offs, stride, payload, args)
+        if not args.no_extras:
+            cpu_extras(torch, gen, out["extras"], layers[0], offs, stride, payload)
     print(json.dumps(out))
 
 
-def time_loop(torch, fn, iters, warmup=3):
-    for i in range(warmup):
-        fn(i)
+MIN_TIMED_MS = 50.0     # every figure comes from at least this much device time
+
+
+def replay_rounds(torch, side, replay_once, min_ms=MIN_TIMED_MS, min_rounds=5, max_rounds=4000):
+    """Replays `replay_once()` (graph launches on `side`) round after round until `min_ms` of device time have gone by;
+    every round is bracketed by events on that stream.  Returns (per-round ms list, wall-clock ms over all rounds between
+    two synchronisations)."""
+    events = []
     torch.cuda.synchronize()
-    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
-    for i in range(iters):
-        fn(warmup + i)
-    e1.record()
+    t0 = time.perf_counter()
+    with torch.cuda.stream(side):
+        while True:
+            batch = []
+            for _ in range(min_rounds):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(side)
+                replay_once()
+                e1.record(side)
+                batch.append((e0, e1))
+            events += batch
+            side.synchronize()
+            if (time.perf_counter() - t0) * 1e3 >= min_ms or len(events) >= max_rounds:
+                break
     torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / iters   # us per call
+    wall_ms = (time.perf_counter() - t0) * 1e3
+    return [a.elapsed_time(b) for a, b in events], wall_ms
+
+
+def time_loop(torch, fn, iters, warmup=3, side=None):
+    """Median device time of one call of fn, in microseconds: `iters` consecutive calls (fn(0) ... fn(iters-1), so that
+    rotating operands rotate) are recorded into a HIP graph once and the graph is replayed until MIN_TIMED_MS have passed.
+    The host only launches graphs, so its jitter stays out of the figure."""
+    side = side or TIMING_STREAM
+    with torch.cuda.stream(side):
+        for i in range(warmup):
+            fn(i)
+        side.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=side):
+            for i in range(iters):
+                fn(i)
+        g.replay()
+        side.synchronize()
+    rounds, _ = replay_rounds(torch, side, g.replay)
+    return float(np.median(rounds)) * 1e3 / iters
+
+
+TIMING_STREAM = None     # the side stream every measurement records on (set in main)
 
 
 def extras(torch, tfk, k, gen, lib, h, stream):
@@ -310,7 +382,9 @@ def extras(torch, tfk, k, gen, lib, h, stream):
     us = time_loop(torch, gemv, 400, warmup=20)
     nbytes = int4_matrix_bytes(F_SHARED, D) + D * 2 + F_SHARED * 2
     res["gemv_2112x2816"] = {"workload": "configs[0]: int4 g64 GEMV 2112x2816, batch 1", "us_per_call": round(us, 3),
-                             "GBps": round(nbytes / (us * 1e-6) / 1e9, 1), "algorithmic_bytes": nbytes}
+                             "GBps": round(nbytes / (us * 1e-6) / 1e9, 1), "algorithmic_bytes": nbytes,
+                             "note": "3.3 MB per call: at 8 TB/s the bytes take 0.4 us, the rest is one launch and one memory round trip; "
+                                     "a latency figure, not an HBM-bandwidth measurement (configs[2] is the bandwidth-sized GEMV)"}
 
     # q / k / v projections of one token in one launch (4096 + 2 x 2048 rows of 2816), rotating over the same 644 MB
     q_rows, kv_rows = 4096, 2048
@@ -506,7 +580,7 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride):
         g.replay()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        replays = 20
+        replays = 40
         for _ in range(replays):
             g.replay()
         torch.cuda.synchronize()
@@ -521,7 +595,8 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride):
         "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 17}}
 
 
-def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, small_sizes=(2, 4, 8, 16, 32, 64, 128), small_only=False):
+def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, small_sizes=(2, 4, 8, 16, 32, 64, 128), small_only=False,
+                       prefill_only=False):
     """configs[3] (small-M verification, M in {2,4,8,16}) and configs[4] (2048-token prefill, Zipf(1.1) routing) over one
     resident layer: router block -> device grouping -> grouped experts -> token-major reduce, no host round trip."""
     import ctypes as C
@@ -561,13 +636,14 @@ def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, 
         return us, unique
 
     small = {}
-    for M in small_sizes:      # by default: verification sizes, then the reference's prefill chunk sizes (RuntimeConfiguration.swift:24)
+    for M in (() if prefill_only else small_sizes):      # by default: verification sizes, then the reference's prefill chunk sizes (RuntimeConfiguration.swift:24)
         us, unique = run(M, iters=50)
         nbytes = unique * expert_bytes + E * D + M * (2 * D * 2 + TOPK * F_MOE * 2 * 2 + TOPK * D * 2 * 2)
         small[str(M)] = {"us": round(us, 2), "unique_experts": unique, "GBps_on_unique_expert_bytes": round(nbytes / (us * 1e-6) / 1e9, 1),
                          "tokens_per_s": round(M / (us * 1e-6), 1)}
-    res["small_m"] = {"workload": "configs[3]: M tokens x top-8 over 128 resident experts (router block + grouping + grouped experts + reduce)",
-                      "per_M": small}
+    if small:
+        res["small_m"] = {"workload": "configs[3]: M tokens x top-8 over 128 resident experts (router block + grouping + grouped experts + reduce)",
+                          "per_M": small}
     if small_only:
         return res
 
@@ -676,6 +752,94 @@ def cpu_baseline(torch, layers, hidden, idx, wts, y, offs, stride, payload, args
                        "ms_per_step": round(total_n / n_sample * 1e3, 3)},
             "parity_on_sample": {"steps_with_identical_expert_indices": idx_match, "of": n_sample,
                                  "worst_rel_error_vs_cpu": round(worst_rel, 6)}}
+
+
+def cpu_extras(torch, gen, extras_out, layer, offs, stride, payload):
+    """CPU rows beside the GPU numbers of configs 0, 2, 3, 4: the serial restatement of the reference's path (1 core, what the
+    Swift reference is) and the same with OpenMP over rows; bounded samples, extrapolation stated.  Also checks the full-size
+    lm_head token of the device against the CPU."""
+    import importlib
+    from oracle import tfo
+    tfk = importlib.import_module("turbo-fieldfare_amd")
+    cores = max(1, min(os.cpu_count() or 1, 16))
+
+    def med_time(fn, reps):
+        ts = []
+        for _ in range(reps):
+            t0 = time.perf_counter()
+            fn()
+            ts.append(time.perf_counter() - t0)
+        return float(np.median(ts))
+
+    to_np16 = lambda t: t.cpu().numpy().view(np.uint16)
+    # configs[0]: 2112 x 2816 GEMV
+    W, S, B = make_int4(torch, gen, F_SHARED, D)
+    Wn, Sn, Bn = W.cpu().numpy(), to_np16(S), to_np16(B)
+    x = np.random.default_rng(5).standard_normal(D).astype(np.float16).astype(np.float32)
+    nbytes0 = int4_matrix_bytes(F_SHARED, D) + D * 2 + F_SHARED * 2
+    t1 = med_time(lambda: tfo.int4_gemv_ref(Wn, Sn, Bn, x, threads=1), 5)
+    tn = med_time(lambda: tfo.int4_gemv_ref(Wn, Sn, Bn, x, threads=cores), 5)
+    extras_out["gemv_2112x2816"]["cpu"] = {"kind": "port", "sample": "the whole GEMV, median of 5", "ms_1_core": round(t1 * 1e3, 3),
+                                           "GBps_1_core": round(nbytes0 / t1 / 1e9, 3), "cores": cores, "ms_openmp": round(tn * 1e3, 3),
+                                           "GBps_openmp": round(nbytes0 / tn / 1e9, 3)}
+    # configs[2]: the full head on the device against the CPU (token), CPU timed on a row subset (1 core) and in full (OpenMP)
+    W, S, B = make_int4(torch, gen, VOCAB, D)
+    hid = torch.randn(D, device="cuda", generator=gen).to(torch.float16)
+    norm_w = bf16_bits_cuda(torch.rand(D, device="cuda", generator=gen) + 0.5)
+    tok = torch.zeros(1, dtype=torch.int32, device="cuda")
+    k = tfk.Context(0)
+    k.lm_head_greedy(hid, norm_w, W, S, B, tok, D, VOCAB)
+    torch.cuda.synchronize()
+    Wn, Sn, Bn, hn, nn = W.cpu().numpy(), to_np16(S), to_np16(B), to_np16(hid.view(torch.int16)), to_np16(norm_w)
+    del W, S, B
+    t0 = time.perf_counter()
+    cpu_tok = tfo.lm_head_cpu_greedy(hn, nn, Wn, Sn, Bn, threads=cores)
+    t_full_n = time.perf_counter() - t0
+    sub = 16384
+    t_sub_1 = med_time(lambda: tfo.lm_head_cpu_greedy(hn, nn, Wn[:sub], Sn[:sub], Bn[:sub], threads=1), 3)
+    extras_out["lm_head_greedy"]["cpu"] = {"kind": "port", "sample": f"1 core: the first {sub} of {VOCAB} rows, x{VOCAB // sub} extrapolated; OpenMP: all rows",
+                                           "ms_1_core_extrapolated": round(t_sub_1 * (VOCAB // sub) * 1e3, 1),
+                                           "GBps_1_core": round(LM_HEAD_BYTES / (t_sub_1 * (VOCAB // sub)) / 1e9, 3), "cores": cores,
+                                           "ms_openmp": round(t_full_n * 1e3, 1), "GBps_openmp": round(LM_HEAD_BYTES / t_full_n / 1e9, 3)}
+    extras_out["lm_head_greedy"]["token_equals_cpu_at_full_size"] = bool(int(tok.item()) == cpu_tok)
+    del Wn, Sn, Bn
+    k.close()
+    # configs[3] / configs[4]: the reference's CPU path has no batching: a token costs one routed decode step (router + 8 experts)
+    # and, for configs[4], one shared expert; timed on two tokens, multiplied out
+    pool, r = layer
+    off = tfo.ExpertOffsets(*offs)
+    rW, rS, rB = r["W"].cpu().numpy(), to_np16(r["S"]), to_np16(r["B"])
+    eff, gain = tfo.bf16_array_to_float(to_np16(r["eff"])), tfo.bf16_array_to_float(to_np16(r["gain"]))
+    rng = np.random.default_rng(11)
+    per_tok_1, per_tok_n = [], []
+    for _ in range(2):
+        xt = rng.standard_normal(D).astype(np.float16).astype(np.float32)
+        t0 = time.perf_counter()
+        ridx, rw, _ = tfo.router_reference(rW, rS, rB, xt, eff, gain)
+        t_r = time.perf_counter() - t0
+        blobs = [pool[int(e), :payload].cpu().numpy() for e in ridx]
+        zero = np.zeros(D, np.float32)
+        per_tok_1.append(t_r + med_time(lambda: tfo.moe_apply_streamed_routed(blobs, off, xt, zero, rw, D, F_MOE, threads=1), 1))
+        per_tok_n.append(t_r + med_time(lambda: tfo.moe_apply_streamed_routed(blobs, off, xt, zero, rw, D, F_MOE, threads=cores), 1))
+    routed_1, routed_n = float(np.mean(per_tok_1)), float(np.mean(per_tok_n))
+    if "small_m" in extras_out:
+        extras_out["small_m"]["cpu"] = {"kind": "port", "sample": "2 tokens (router + 8 experts each, no sharing of experts between tokens on the CPU path), "
+                                        "multiplied by M", "cores": cores,
+                                        "ms_per_M_1_core": {m: round(int(m) * routed_1 * 1e3, 1) for m in extras_out["small_m"]["per_M"]},
+                                        "ms_per_M_openmp": {m: round(int(m) * routed_n * 1e3, 1) for m in extras_out["small_m"]["per_M"]}}
+    g, u, dn = (tuple(a.cpu().numpy() if a.dtype == torch.uint8 else to_np16(a) for a in make_int4(torch, gen, rows, cols))
+                for rows, cols in ((F_SHARED, D), (F_SHARED, D), (D, F_SHARED)))
+    xt = rng.standard_normal(D).astype(np.float16).astype(np.float32)
+    sh_1 = med_time(lambda: tfo.shared_expert_ref(g, u, dn, xt, threads=1), 2)
+    sh_n = med_time(lambda: tfo.shared_expert_ref(g, u, dn, xt, threads=cores), 2)
+    if "prefill_2048_total" in extras_out:
+        flop = extras_out["prefill_2048_total"]["GFLOP"] * 1e9
+        extras_out["prefill_2048_total"]["cpu"] = {"kind": "port", "sample": "2 tokens routed + 1 token shared expert, x2048 extrapolated", "cores": cores,
+                                                   "s_1_core_extrapolated": round(2048 * (routed_1 + sh_1), 1),
+                                                   "GFLOPs_1_core": round(flop / (2048 * (routed_1 + sh_1)) / 1e9, 2),
+                                                   "s_openmp_extrapolated": round(2048 * (routed_n + sh_n), 2),
+                                                   "GFLOPs_openmp": round(flop / (2048 * (routed_n + sh_n)) / 1e9, 2),
+                                                   "tokens_per_s_1_core": round(1.0 / (routed_1 + sh_1), 2)}
 
 
 if __name__ == "__main__":

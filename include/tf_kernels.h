@@ -671,6 +671,17 @@ int32_t tf_upload_packed_experts_layer(tf_ctx *ctx, tf_stream stream, const char
 int32_t tf_upload_file_region(tf_ctx *ctx, tf_stream stream, const char *file_path, uint64_t file_offset, uint64_t bytes,
                               void *device_dst);
 
+/* ---- measurement helpers (no counterpart in the reference) ----------------------------------------------------- */
+/* A launch of `blocks` x `threads_per_block` that reads in_word[0] in every block and writes out_word[0] from one thread:
+ * chained on a stream, what dependent launches of those shapes cost when they move no data (the latency floor of a
+ * multi-launch step). */
+int32_t tf_bench_empty_launch(tf_ctx *ctx, tf_stream stream, uint32_t blocks, uint32_t threads_per_block,
+                              const void *in_word, void *out_word);
+/* A plain streaming read of `bytes` (multiple of 4096, 16-byte aligned) with the access pattern and cache policy of the
+ * row streamers and no arithmetic: the read rate this part sustains, to hold the GEMV kernels against beside the
+ * published peak. */
+int32_t tf_bench_stream_read(tf_ctx *ctx, tf_stream stream, const void *data, uint64_t bytes, void *out_word);
+
 #ifdef __cplusplus
 }
 #endif

@@ -185,6 +185,8 @@ EXPORTS = {
     "tf_logit_softcap_softmax": (i32, [vp, vp, vp, vp, u32, C.c_float, i32]),
     "tf_sample": (i32, [vp, vp, vp, vp, u32, C.c_float, u32, C.c_float, u64, u32]),
     "tf_sample_topk64": (i32, [vp, vp, vp, vp, u32, C.c_float, C.c_float, u64]),
+    "tf_bench_empty_launch": (i32, [vp, vp, u32, u32, vp, vp]),
+    "tf_bench_stream_read": (i32, [vp, vp, vp, u64, vp]),
     "tf_upload_packed_experts_layer": (i32, [vp, vp, C.c_char_p, u64, u32, C.POINTER(u32), vp]),
     "tf_upload_file_region": (i32, [vp, vp, C.c_char_p, u64, u64, vp]),
     "tf_lm_head_greedy_int4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u32, u32, C.c_float, i32]),

@@ -1,0 +1,55 @@
+// Measurement helpers behind the C ABI: what a kernel boundary and a plain streaming read cost on the part the library runs
+// on, so that a benchmark can print the latency floor of a chain of dependent launches and the read rate a streaming kernel
+// can be held against, measured in the same run as the kernels themselves.
+#include "tf_gemv_kernels.hpp"
+
+using namespace tfk;
+
+namespace {
+
+// A launch of a given shape that does next to nothing: every block reads one word (so the launch depends on what the
+// previous launch on the stream wrote) and block 0 writes one.
+__global__ void bench_empty_kernel(const uint32_t *in, uint32_t *out) {
+    const uint32_t v = in[0];
+    if (blockIdx.x == 0 && threadIdx.x == 0) out[0] = v + 1u;
+}
+
+// Streaming read: every wave takes contiguous 4 KiB pieces (four 1 KiB loads in flight), pieces strided by the number of
+// waves, non-temporal like the row streamers' weight loads.
+__global__ __launch_bounds__(256) void bench_stream_read_kernel(const uint8_t *in, uint32_t *out, size_t bytes) {
+    const size_t nwaves = ((size_t)gridDim.x * blockDim.x) >> 6;
+    const size_t wave = ((size_t)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int lane = threadIdx.x & 63;
+    const size_t npieces = bytes / 4096;
+    uint32_t acc = 0;
+    for (size_t pc = wave; pc < npieces; pc += nwaves) {
+        u32x4 v[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) v[u] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(in + pc * 4096 + u * 1024 + lane * 16));
+#pragma unroll
+        for (int u = 0; u < 4; ++u) acc ^= v[u][0] ^ v[u][1] ^ v[u][2] ^ v[u][3];
+    }
+    if (acc == 0x9E3779B9u) out[0] = acc;   // keeps the loads alive; practically never true
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t tf_bench_empty_launch(tf_ctx *ctx, tf_stream stream, uint32_t blocks, uint32_t threads_per_block, const void *in_word, void *out_word) {
+    TF_REQUIRE(ctx, ctx && in_word && out_word && blocks > 0 && threads_per_block > 0 && threads_per_block <= 1024, TF_ERR_INVALID_ARGUMENT,
+               "bench_empty_launch: bad argument");
+    hipLaunchKernelGGL(bench_empty_kernel, dim3(blocks), dim3(threads_per_block), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint32_t *>(in_word), static_cast<uint32_t *>(out_word));
+    return check_launch(ctx, "bench_empty_launch");
+}
+
+int32_t tf_bench_stream_read(tf_ctx *ctx, tf_stream stream, const void *data, uint64_t bytes, void *out_word) {
+    TF_REQUIRE(ctx, ctx && data && out_word && aligned16(data) && bytes % 4096 == 0 && bytes > 0, TF_ERR_INVALID_ARGUMENT,
+               "bench_stream_read: data must be 16-byte aligned and a multiple of 4096 bytes");
+    hipLaunchKernelGGL(bench_stream_read_kernel, dim3((uint32_t)ctx->num_cus * 2u), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint8_t *>(data), static_cast<uint32_t *>(out_word), (size_t)bytes);
+    return check_launch(ctx, "bench_stream_read");
+}
+
+}  // extern "C"
