@@ -535,7 +535,10 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride):
     position = WINDOW + 60
     kv_off = position * NKV * HD * 2
 
-    def layer_step(i, st):
+    def layer_step(i, st, branch=None):
+        """One layer on stream handle `st`.  With `branch` (a torch stream) the shared expert and its norm run beside the router and
+        the routed experts, as the reference commits its shared-expert command buffer without waiting
+        (RealForwardRunner.swift:1570-1594); the branch forks after the post-attention setup and joins before the layer tail."""
         w, (pool, r) = dense[i % n_layers], layers[i % n_layers]
         ptr = lambda name: w[name].data_ptr()
         rc = lib.tf_rmsnorm_bf16w(h, st, p("hidden"), 0, ptr("input_norm"), 0, p("x_norm"), 0, D, 1e-6)
@@ -551,12 +554,22 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride):
         rc |= lib.tf_fused_post_attn_setup(h, st, p("hidden"), p("o"), p("dense_x"), p("routed_x"), p("router_x"), ptr("post_attn"), 0,
                                            ptr("pre_ffn"), 0, ptr("pre_ffn2"), 0, D, 1e-6)
         g, u, dn = w["proj"]
-        rc |= lib.tf_shared_expert_int4(h, st, p("dense_x"), 0, D * 2, C.byref(g), C.byref(u), C.byref(dn), p("shared"), 0, D * 2, p("sg"), 0,
+        st_shared = st
+        if branch is not None:
+            fork = torch.cuda.Event()
+            fork.record(torch.cuda.current_stream())
+            branch.wait_event(fork)
+            st_shared = branch.cuda_stream
+        rc |= lib.tf_shared_expert_int4(h, st_shared, p("dense_x"), 0, D * 2, C.byref(g), C.byref(u), C.byref(dn), p("shared"), 0, D * 2, p("sg"), 0,
                                         F_SHARED * 2, p("su"), 0, F_SHARED * 2, p("sa"), 0, F_SHARED * 2, 4, tfk.TF_BF16)
-        rc |= lib.tf_rmsnorm_bf16w(h, st, p("shared"), 0, ptr("post_ffn1"), 0, p("h1"), 0, D, 1e-6)
+        rc |= lib.tf_rmsnorm_bf16w(h, st_shared, p("shared"), 0, ptr("post_ffn1"), 0, p("h1"), 0, D, 1e-6)
         rc |= lib.tf_moe_decode_step(h, st, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, p("router_x"), r["eff"].data_ptr(), 0,
                                      r["gain"].data_ptr(), 0, pool.data_ptr(), stride, E, C.byref(off), p("routed_x"), p("acts"), p("zero"), p("h2"),
                                      p("idx"), p("wts"), D, F_MOE, TOPK, tfk.TF_BF16)
+        if branch is not None:
+            join = torch.cuda.Event()
+            join.record(branch)
+            torch.cuda.current_stream().wait_event(join)
         rc |= lib.tf_fused_layer_tail(h, st, p("h2"), p("h1"), p("hidden"), ptr("post_ffn2"), 0, ptr("post_ffn"), 0, D, 1e-6, 1.0)
         if rc != 0:
             raise RuntimeError("layer chain failed: " + k.last_error())
@@ -568,23 +581,23 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride):
         layer_step(i, st0)                                  # warm-up; also sizes every context-owned scratch before the capture
     b["hidden"].copy_(start_hidden)
     torch.cuda.synchronize()
-    side = torch.cuda.Stream()
+    side, branch = torch.cuda.Stream(), torch.cuda.Stream()      # both at the default priority
+    results = {}
     with torch.cuda.stream(side):
         hidden0 = b["hidden"].clone()
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g, stream=side):
-            st = torch.cuda.current_stream().cuda_stream
-            b["hidden"].copy_(hidden0)                      # every replay is the same token: synthetic weights would otherwise drift it away
-            for i in range(per_graph):
-                layer_step(i, st)
-        g.replay()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        replays = 40
-        for _ in range(replays):
+        for label, br in (("serial", None), ("forked", branch)):
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=side):
+                st = torch.cuda.current_stream().cuda_stream
+                b["hidden"].copy_(hidden0)                  # every replay is the same token: synthetic weights would otherwise drift it away
+                for i in range(per_graph):
+                    layer_step(i, st, br)
             g.replay()
-        torch.cuda.synchronize()
-        us = (time.perf_counter() - t0) * 1e6 / (replays * per_graph)
+            side.synchronize()
+            rounds, _ = replay_rounds(torch, side, g.replay)
+            results[label] = (float(np.median(rounds)) * 1e3 / per_graph, b["hidden"].clone())
+    us, us_forked = results["serial"][0], results["forked"][0]
+    assert torch.equal(results["forked"][1], results["serial"][1]), "forked and serial layer chains disagree"
     bad = [n for n, t in b.items() if t.dtype == torch.float16 and not bool(torch.isfinite(t.float()).all())]
     assert not bad, f"non-finite values after the replays in {bad}"
     layer_bytes = (int4_matrix_bytes(NQ * HD + 2 * NKV * HD, D) + int4_matrix_bytes(D, NQ * HD) + SHARED_BYTES + STEP_BYTES
@@ -592,7 +605,12 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride):
     return {"decode_layer_sliding_window": {
         "workload": "one token through one whole decoder layer (16q/8kv x 256, window 1024, shared 2112, 8 of 128 experts), 30 layers per graph replay",
         "us_per_layer": round(us, 2), "ms_per_30_layers": round(us * 30 / 1e3, 3), "algorithmic_bytes_per_layer": layer_bytes,
-        "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 17}}
+        "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 17,
+        "graph": "one in-order chain of launches",
+        "us_per_layer_shared_expert_on_forked_branch": round(us_forked, 2),
+        "forked_branch_note": "the shared expert + its norm on a second captured stream (event fork after the post-attention setup, join before the "
+                              "layer tail, as the reference commits sharedCB without waiting); bit-identical; the cross-queue fork and join cost more than "
+                              "the 13 us of launches they overlap"}}
 
 
 def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, small_sizes=(2, 4, 8, 16, 32, 64, 128), small_only=False,

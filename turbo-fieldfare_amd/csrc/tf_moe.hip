@@ -10,6 +10,26 @@ using namespace tfk;
 constexpr uint32_t kStaticMaxExperts = 256;
 static __device__ __align__(256) float scratch[kStaticMaxExperts];
 
+// Per-wave timeline of the decode step's kernels for tuning, compiled only with -DTF_STAMPS (never in the shipped library):
+// lane 0 of a wave writes the 100 MHz wall clock into slot `slot` of its row in a load-time buffer that
+// tf_debug_stamps() hands to the host.
+#ifdef TF_STAMPS
+constexpr uint32_t kStampWaves = 4096;
+static __device__ unsigned long long stamp_buf[3 * kStampWaves * 8];
+#define TF_STAMP(kernel_, wave_, slot_)                                                                                   \
+    do {                                                                                                                  \
+        if ((threadIdx.x & 63) == 0 && (wave_) < kStampWaves) stamp_buf[(((kernel_) * kStampWaves + (wave_)) << 3) + (slot_)] = wall_clock64(); \
+    } while (0)
+#define TF_STAMP_WAIT() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
+extern "C" unsigned long long *tf_debug_stamps(void) {
+    void *ptr = nullptr;
+    return hipGetSymbolAddress(&ptr, HIP_SYMBOL(stamp_buf)) == hipSuccess ? static_cast<unsigned long long *>(ptr) : nullptr;
+}
+#else
+#define TF_STAMP(kernel_, wave_, slot_) do {} while (0)
+#define TF_STAMP_WAIT() do {} while (0)
+#endif
+
 namespace tfk {
 
 int32_t moe_static_scratch_setup(tf_ctx *ctx) {
@@ -64,9 +84,11 @@ __global__ __launch_bounds__(256) void router_logits_block_kernel(const uint8_t 
                                                                   const uint16_t *eff, float *logits, int d) {
     __shared__ float partial[4];
     const uint32_t e = blockIdx.x;
+    TF_STAMP(0, blockIdx.x * 4 + (threadIdx.x >> 6), 0);
     const int groups = d >> 6;
     const float v = router_row_block<SD>(W + (size_t)e * d, S + (size_t)e * groups * 2, B + (size_t)e * groups * 2, hidden, eff, d, partial);
     if (threadIdx.x == 0) logits[e] = v;
+    TF_STAMP(0, blockIdx.x * 4 + (threadIdx.x >> 6), 1);
 }
 
 __global__ __launch_bounds__(64) void router_select_kernel(const float *logits, const uint16_t *per_expert_scale,
@@ -124,6 +146,7 @@ __global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_e
     const int lane = threadIdx.x & 63;
     const uint32_t unit = uniform_u32((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
     const uint32_t tiles = (g.f + RT - 1) / RT;
+    TF_STAMP(1, unit, 0);
     float my_logit = 0.0f;
     if constexpr (FUSED) my_logit = rank_select_load(fs.logits, fs.num_experts);   // requested first: the selection waits for nothing else
     XStage stage;
@@ -158,7 +181,9 @@ __global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_e
     } else {
         if (live) request_weights(uniform_ptr(blob_base(routed, slot)));
     }
+    TF_STAMP(1, unit, 1);
     stage.publish((int)g.d, xa, xsum);
+    TF_STAMP(1, unit, 2);
     if (!live) return;
     if constexpr (FUSED) {
         request_weights(routed.pool + (uint64_t)uniform_u32(chosen[slot]) * routed.stride);
@@ -173,6 +198,8 @@ __global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_e
         }
     }
     rs.init_x_lds(xa, xsum, (int)g.d);
+    TF_STAMP_WAIT();
+    TF_STAMP(1, unit, 3);
     float gate[RT], up[RT];
     rs.template reduce<SD>(tg, gate);
     rs.template reduce<SD>(tu, up);
@@ -181,6 +208,7 @@ __global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_e
         for (int r = 0; r < RT; ++r)
             if (row0 + r < g.f) store_act(acts, slot * g.f + row0 + r, gate[r], up[r]);
     }
+    TF_STAMP(1, unit, 4);
 }
 
 // D <= 1024: half-wave per row, NPASS passes: 2 * NPASS rows of gate and up per wave.
@@ -241,6 +269,7 @@ __global__ __launch_bounds__(512) void phase2_short_kernel(RoutedArg routed, tf_
     const int lane = threadIdx.x & 63;
     const uint32_t slot = uniform_u32(threadIdx.x >> 6);
     const long row0 = (long)blockIdx.x * 2 * NPASS;
+    TF_STAMP(2, blockIdx.x * 8 + slot, 0);
     ShortRows sr;
     ShortRows::Pair t[NPASS];
     sr.init_map(f, lane);
@@ -253,11 +282,14 @@ __global__ __launch_bounds__(512) void phase2_short_kernel(RoutedArg routed, tf_
     const bool writer = threadIdx.x < 2 * NPASS && row0 + threadIdx.x < d;
     const half_t res16 = writer ? residual[row0 + threadIdx.x] : (half_t)0.0f;   // requested now, needed after the barrier
     const uint8_t *base = uniform_ptr(blob_base(routed, slot));
+    TF_STAMP(2, blockIdx.x * 8 + slot, 1);
 #pragma unroll
     for (int p = 0; p < NPASS; ++p)
         sr.load(t[p], base + off.down_W_off, base + off.down_s_off, base + off.down_b_off, row0 + 2 * p, d, f);
     sr.xs = arrange_x(xr, sr.xq);
     const float w = (float)w16;
+    TF_STAMP_WAIT();
+    TF_STAMP(2, blockIdx.x * 8 + slot, 2);
 #pragma unroll
     for (int p = 0; p < NPASS; ++p) {
         float lo, hi;
@@ -267,6 +299,7 @@ __global__ __launch_bounds__(512) void phase2_short_kernel(RoutedArg routed, tf_
             partial[slot][2 * p + 1] = w * hi;
         }
     }
+    TF_STAMP(2, blockIdx.x * 8 + slot, 3);
     __syncthreads();
     if (writer) {
         float acc = (float)res16;
@@ -274,6 +307,7 @@ __global__ __launch_bounds__(512) void phase2_short_kernel(RoutedArg routed, tf_
         for (int s = 0; s < 8; ++s) acc += partial[s][threadIdx.x];
         y[row0 + threadIdx.x] = (half_t)acc;
     }
+    TF_STAMP(2, blockIdx.x * 8 + slot, 4);
 }
 
 template <int SD>
