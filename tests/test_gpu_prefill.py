@@ -182,7 +182,33 @@ def test_streamed_batched_matches_reference_across_partial_microbatch():
     del blob_t
 
 
-def resident_pipeline(T, E, d, f, top_k, seed, zipf=False, from_router=True):
+def scales_as_fp16(blob, off, d, f):
+    """The same expert with its bf16 scales and biases rewritten as fp16 of the same value (a bf16 value inside fp16's normal
+    range converts exactly; the rare bias below it becomes zero)."""
+    out = blob.copy()
+    for name, count in (("gate_s_off", f * d // 64), ("gate_b_off", f * d // 64), ("up_s_off", f * d // 64), ("up_b_off", f * d // 64),
+                        ("down_s_off", d * f // 64), ("down_b_off", d * f // 64)):
+        at = getattr(off, name)
+        bf = out[at:at + 2 * count].view(np.uint16)
+        val = (bf.astype(np.uint32) << 16).view(np.float32)
+        h = val.astype(np.float16)
+        h[h.astype(np.float32) != val] = 0
+        out[at:at + 2 * count] = h.view(np.uint8)
+    return out
+
+
+def bf16_pool_matching(blob_fp16, off, d, f):
+    """Inverse of scales_as_fp16 for a blob whose fp16 scales all came from bf16 values."""
+    out = blob_fp16.copy()
+    for name, count in (("gate_s_off", f * d // 64), ("gate_b_off", f * d // 64), ("up_s_off", f * d // 64), ("up_b_off", f * d // 64),
+                        ("down_s_off", d * f // 64), ("down_b_off", d * f // 64)):
+        at = getattr(off, name)
+        val = out[at:at + 2 * count].view(np.float16).astype(np.float32)
+        out[at:at + 2 * count] = (val.view(np.uint32) >> 16).astype(np.uint16).view(np.uint8)
+    return out
+
+
+def resident_pipeline(T, E, d, f, top_k, seed, zipf=False, from_router=True, fp16_scales=False):
     """router block -> device grouping -> grouped experts (resident pool) -> token-major reduce; returns everything needed to check."""
     rng = np.random.default_rng(seed)
     blobs, off = [], None
@@ -190,6 +216,8 @@ def resident_pipeline(T, E, d, f, top_k, seed, zipf=False, from_router=True):
         blob, off = tfo.make_blob(refcases.synthetic_int4(f, d, seed + e, "g"), refcases.synthetic_int4(f, d, seed + e, "u"),
                                   refcases.synthetic_int4(d, f, seed + e, "d"))
         blobs.append(blob)
+    if fp16_scales:
+        blobs = [scales_as_fp16(b, off, d, f) for b in blobs]
     stride = (blobs[0].size + 255) // 256 * 256
     pool_np = np.zeros((E, stride), np.uint8)
     for e, b in enumerate(blobs):
@@ -214,7 +242,8 @@ def resident_pipeline(T, E, d, f, top_k, seed, zipf=False, from_router=True):
     d_pool, d_hidden, d_w = dev(pool_np), dev(hidden), dev(np.ascontiguousarray(w_bits, np.uint16))
     k.check(k.lib.tf_prefill_grouped_routed_moe_resident(k.handle, None, d_hidden.data_ptr(), 0, d, g["sorted_pairs"].data_ptr(),
                                                          g["chunks"].data_ptr(), g["n_chunks"].data_ptr(), g["cap"], n, d_pool.data_ptr(),
-                                                         stride, E, C.byref(koff), acts.data_ptr(), partials.data_ptr(), d, f, top_k, tfk.TF_BF16))
+                                                         stride, E, C.byref(koff), acts.data_ptr(), partials.data_ptr(), d, f, top_k,
+                                                         tfk.TF_FP16 if fp16_scales else tfk.TF_BF16))
     k.check(k.lib.tf_prefill_moe_reduce_token_major(k.handle, None, partials.data_ptr(), 0, d_w.data_ptr(), 0, h2.data_ptr(), 0, T, top_k, d))
     sp = host(g["sorted_pairs"], np.uint32, n * 4).reshape(n, 4)
     return dict(blobs=blobs, off=off, pool=pool_np.ravel(), stride=stride, hidden=hidden, idx=np.asarray(idx), w_bits=np.asarray(w_bits).reshape(T, top_k),
@@ -236,10 +265,11 @@ def check_against_oracle(r, T, d, f, top_k, abs_tol, rel_tol=1e-2):
         assert tfo.rel_error(r["h2"][t], ref) < tfo.Tolerance.fp16ChainedReduction
 
 
-@pytest.mark.parametrize("M", [2, 4, 8, 16, 24])
+@pytest.mark.parametrize("M", [2, 4, 8, 12, 16, 24])
 def test_small_m_resident_pipeline_matches_oracle(M):
-    # BASELINE config 3: M tokens, top-8 over the production expert shape; below two pairs per expert on average (M = 2, 4
-    # here) the groups take the row-streaming kernels, from there on the matrix cores
+    # BASELINE config 3: M tokens, top-8 over the production expert shape; below three pairs per expert on average (M = 2, 4,
+    # 8 here) every chunk takes the quad kernels, at M = 12 short chunks take them and long ones the matrix-core tiles, from
+    # four pairs per expert on the matrix-core tiles serve the call alone
     E, d, f, top_k = 32, 2816, 704, 8
     r = resident_pipeline(M, E, d, f, top_k, 0x300 + M)
     scale = float(np.max(np.abs(tfo.from_f16_bits(r["partials"]))))
@@ -261,6 +291,46 @@ def test_small_m_equals_decode_step_per_token():
         k.moe_phase2(routed, koff, acts, d_w, d_res, y, d, f)
         dec = tfo.from_f16_bits(host(y, np.uint16, d))
         assert np.max(np.abs(dec - r["h2"][t])) <= 4e-3 * max(1.0, float(np.max(np.abs(dec))))
+
+
+@pytest.mark.parametrize("T,E,d,f", [(10, 32, 2816, 704), (4, 16, 512, 128), (6, 16, 512, 128), (2, 8, 3072, 1024), (3, 8, 3072, 1024),
+                                     (5, 16, 64, 64)])
+def test_quad_kernels_long_chunks_and_row_widths(T, E, d, f):
+    # Zipf-skewed routing with few pairs per expert on average: some chunks are longer than the quad kernels' LDS image and go
+    # through in batches (first case) or to the matrix-core tiles of the same call (3 pairs per expert); rows of one pass, of a
+    # partly filled last pass and of the widest supported rows
+    top_k = 8
+    r = resident_pipeline(T, E, d, f, top_k, 0x4400 + T, zipf=True, from_router=False)
+    assert np.bincount(r["idx"].ravel(), minlength=E).max() > 8 or T <= 8
+    scale = float(np.max(np.abs(tfo.from_f16_bits(r["partials"]))))
+    check_against_oracle(r, T, d, f, top_k, abs_tol=1e-3 * max(1.0, scale))
+
+
+@pytest.mark.parametrize("T", [6, 12, 24])
+def test_grouped_experts_fp16_scales_equal_bf16_scales(T):
+    # the reference's expert blobs carry bf16 scales, and so does the oracle; the fp16 variant of the grouped kernels is pinned
+    # on pools whose scales hold the same values in either type: every partial must come out bit-identical (quad kernels alone,
+    # quad + matrix-core tiles, matrix-core tiles alone)
+    E, d, f, top_k = 32, 2816, 704, 8
+    a = resident_pipeline(T, E, d, f, top_k, 0x5500 + T, from_router=False, fp16_scales=True)
+    blobs16 = a["blobs"]
+    k = ctx()
+    pool = np.zeros((E, a["stride"]), np.uint8)
+    for e, b in enumerate(blobs16):
+        pool[e, :b.size] = bf16_pool_matching(b, a["off"], d, f)
+    n = T * top_k
+    g = device_grouping(a["idx"], a["w_bits"], T, top_k, E)
+    acts, partials = zeros_bytes(n * f * 2), zeros_bytes(n * d * 2)
+    koff = tfk.ExpertOffsets(*a["off"].as_tuple())
+    d_pool, d_hidden = dev(pool), dev(a["hidden"])
+    k.check(k.lib.tf_prefill_grouped_routed_moe_resident(k.handle, None, d_hidden.data_ptr(), 0, d, g["sorted_pairs"].data_ptr(),
+                                                         g["chunks"].data_ptr(), g["n_chunks"].data_ptr(), g["cap"], n, d_pool.data_ptr(),
+                                                         a["stride"], E, C.byref(koff), acts.data_ptr(), partials.data_ptr(), d, f, top_k, tfk.TF_BF16))
+    assert np.array_equal(host(partials, np.uint16, n * d), a["partials"])
+    # and the bf16 run itself is the one the oracle checks
+    b = dict(a, pool=pool.ravel(), blobs=[pool[e, :blobs16[0].size] for e in range(E)], partials=host(partials, np.uint16, n * d))
+    scale = float(np.max(np.abs(tfo.from_f16_bits(b["partials"]))))
+    check_against_oracle(b, T, d, f, top_k, abs_tol=2e-3 * max(1.0, scale))
 
 
 @pytest.mark.parametrize("T,E,d,f,zipf", [(64, 16, 2816, 704, True), (96, 8, 512, 128, False), (200, 16, 256, 192, True)])

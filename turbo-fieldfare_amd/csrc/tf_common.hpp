@@ -138,6 +138,38 @@ __device__ __forceinline__ float chunk_dot(const u32x4 w, const half2_t *xq) {
     return ((sel & 2) ? c23 : c01) * 16777216.0f;   // subnormal units -> integers
 }
 
+// The same in two steps, for a chunk of weights that meets many activation vectors: chunk_operands() isolates the nibble pairs
+// once (20 instructions), chunk_dot_pre() multiplies them with one vector's activations (8 matrix instructions and the pick
+// of the diagonal element).  chunk_dot(w, xq) == chunk_dot_pre(chunk_operands(w), xq) bit for bit.
+struct ChunkOperands {
+    u32x2 a[8];
+};
+__device__ __forceinline__ ChunkOperands chunk_operands(const u32x4 w) {
+    ChunkOperands o;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        const uint32_t v = w[d];
+        const uint32_t v8 = v >> 8;
+        o.a[2 * d] = u32x2{v & 0x000F000Fu, v & 0x00F000F0u};
+        o.a[2 * d + 1] = u32x2{v8 & 0x000F000Fu, v8 & 0x00F000F0u};
+    }
+    return o;
+}
+__device__ __forceinline__ float chunk_dot_pre(const ChunkOperands &o, const half2_t *xq) {
+    const int sel = lane_index() & 3;
+    f32x4 c = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+        const half4_t b0 = __builtin_shufflevector(xq[4 * d + 0], xq[4 * d + 1], 0, 1, 2, 3);
+        const half4_t b1 = __builtin_shufflevector(xq[4 * d + 2], xq[4 * d + 3], 0, 1, 2, 3);
+        c = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, o.a[2 * d]), b0, c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, o.a[2 * d + 1]), b1, c, 0, 0, 0);
+    }
+    const float c01 = (sel & 1) ? c[1] : c[0];
+    const float c23 = (sel & 1) ? c[3] : c[2];
+    return ((sel & 2) ? c23 : c01) * 16777216.0f;
+}
+
 // Arrange 32 consecutive activations (four 16-byte loads, xr[d] = elements 8d..8d+7 as 4 packed pairs)
 // into the order chunk_dot() consumes, and return their fp32 sum.
 __device__ __forceinline__ float arrange_x(const u32x4 *xr, half2_t *xq) {
