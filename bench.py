@@ -101,6 +101,9 @@ def main():
     ap.add_argument("--only-small-m", type=int, nargs="+", metavar="M",
                     help="run nothing but the few-token routed-MoE measurement at these token counts and print its JSON "
                          "(a short program whose launches a profiler can attribute to one size)")
+    ap.add_argument("--prefill-balanced", action="store_true",
+                    help="with --only-prefill-2048: every expert gets exactly 128 of the 16384 pairs instead of the Zipf(1.1) draw "
+                         "(all row tiles full: the grouped kernels' rate without the skew)")
     ap.add_argument("--only-prefill-2048", action="store_true",
                     help="run nothing but the 2048-token prefill measurement (configs[4]) and print its JSON")
     args = ap.parse_args()
@@ -124,7 +127,7 @@ def main():
     if args.only_small_m or args.only_prefill_2048:
         only = multi_token_extras(torch, tfk, k, gen, k.lib, k.handle, side.cuda_stream, layers[0], offs, stride,
                                   small_sizes=tuple(args.only_small_m or ()), small_only=not args.only_prefill_2048,
-                                  prefill_only=bool(args.only_prefill_2048))
+                                  prefill_only=bool(args.only_prefill_2048), balanced=bool(args.prefill_balanced))
         print(json.dumps(only))
         return
     n_hidden = 64
@@ -614,7 +617,7 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride):
 
 
 def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, small_sizes=(2, 4, 8, 16, 32, 64, 128), small_only=False,
-                       prefill_only=False):
+                       prefill_only=False, balanced=False):
     """configs[3] (small-M verification, M in {2,4,8,16}) and configs[4] (2048-token prefill, Zipf(1.1) routing) over one
     resident layer: router block -> device grouping -> grouped experts -> token-major reduce, no host round trip."""
     import ctypes as C
@@ -671,11 +674,14 @@ def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, 
     p = 1.0 / np.arange(1, E + 1) ** 1.1
     p /= p.sum()
     idx_np = np.stack([rng.choice(E, size=TOPK, replace=False, p=p) for _ in range(T)]).astype(np.int32)
+    if balanced:
+        idx_np = np.stack([(np.arange(TOPK) * (E // TOPK) + t) % E for t in range(T)]).astype(np.int32)
     idx_dev = torch.from_numpy(idx_np).cuda()
     wts_dev = torch.softmax(torch.randn((T, TOPK), device="cuda", generator=gen), dim=1).to(torch.float16)
     us, unique = run(T, idx_dev, wts_dev, iters=5, with_router=False)
     routed_flop = T * TOPK * 2 * 3 * F_MOE * D
-    res["prefill_routed_2048"] = {"workload": "configs[4] routed part: 2048 tokens, Zipf(1.1) top-8 over 128 int4 experts, grouped GEMM on MFMA",
+    res["prefill_routed_2048"] = {"workload": "configs[4] routed part: 2048 tokens, " + ("128 pairs for every one of" if balanced else "Zipf(1.1) top-8 over") +
+                                  " 128 int4 experts, grouped GEMM on MFMA",
                                   "ms": round(us / 1e3, 3), "tokens_per_s": round(T / (us * 1e-6), 1), "unique_experts": unique,
                                   "TFLOPs": round(routed_flop / (us * 1e-6) / 1e12, 2),
                                   "frac_mfma_fp16_peak": round(routed_flop / (us * 1e-6) / 2.5e15, 4)}

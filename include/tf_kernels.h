@@ -292,8 +292,12 @@ int32_t tf_shared_expert_int8_down(tf_ctx *ctx, tf_stream stream, const tf_proje
  * (the chain's stage boundary), activations in a buffer the context owns, then the down projection; weights are
  * expanded to fp16 half(q*s+b) per group as in tf_int4_qmm, so results agree with the row chain within the shared
  * expert's tolerance, not bit for bit, and the caller's scratch (still validated: one row each, lengths in BYTES) is
- * left untouched.  query_count == 0 is a no-op.  d, intermediate > 0, strides >= d (TF_ERR_INVALID_ARGUMENT);
- * gate/up = (intermediate, d), down = (d, intermediate) or TF_ERR_DIMENSION_MISMATCH. */
+ * left untouched.  weight_bits == 8 (PrefillSharedExpert's default): up to 15 rows in groups against each weight row,
+ * bit-identical to repeated tf_shared_expert_int8; from 16 aligned rows on on the matrix cores with every weight
+ * rounded to fp16 first, within the 8-bit shared expert's tolerance of the row chain (weights below fp16's normal
+ * range, scales under about 1e-7, would lose their grid there).  query_count == 0 is a no-op.  d, intermediate > 0,
+ * strides >= d (TF_ERR_INVALID_ARGUMENT); gate/up = (intermediate, d), down = (d, intermediate) or
+ * TF_ERR_DIMENSION_MISMATCH. */
 int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream,
                                             const void *x, uint64_t x_offset, void *y, uint64_t y_offset,
                                             const tf_projection *gate, const tf_projection *up, const tf_projection *down,

@@ -246,9 +246,9 @@ def test_shared_expert_errors():
 
 
 # ---------------------------------------------------------------------------------------------------- shared expert, 8-bit
-def _int8_case(d, f, seed):
+def _int8_case(d, f, seed, weight_range=0.4):
     rng = np.random.default_rng(seed)
-    mats = {name: tfo.quantize_int8(rng.uniform(-0.4, 0.4, shape).astype(np.float32))       # SharedExpertInt8Tests.swift:50-60
+    mats = {name: tfo.quantize_int8(rng.uniform(-weight_range, weight_range, shape).astype(np.float32))       # SharedExpertInt8Tests.swift:50-60
             for name, shape in (("gate", (f, d)), ("up", (f, d)), ("down", (d, f)))}
     return dict(d=d, f=f, x_bits=tfo.to_f16_bits(rng.uniform(-0.4, 0.4, d).astype(np.float32)), **mats)
 
@@ -358,6 +358,33 @@ def test_prefill_shared_expert_block_with_8_bit_weights_is_the_row_chain(d, f, r
         else:
             assert np.array_equal(row_chain, got[r, :d])
 
+
+
+def test_8_bit_block_on_matrix_cores_with_small_scales():
+    # From 16 rows on the 8-bit block rounds every weight to fp16 (half(q s + b), the reference's staged-affine rounding point,
+    # tensorops.metal:57-94) while the row chain keeps q s + b in fp32.  Weights of magnitude 1e-3 and less (scales near 8e-6)
+    # sit near the bottom of fp16's normal range, where its spacing is still finer than the quantization grid: the block must
+    # stay within the 8-bit shared expert's tolerance of the row chain.  (Scales below about 1e-7 would fall into fp16's
+    # subnormals and lose the grid; the row chain is the path for such tensors.)
+    import ctypes as C
+    d, f, rows = 1024, 256, 32
+    c = _int8_case(d, f, 0x6A1, weight_range=1e-3)
+    _, _, _, (t, _, _, sa, g, u, dn) = _run_int8(c, False)
+    k = ctx()
+    rng = np.random.default_rng(0x6A1)
+    xs = tfo.to_f16_bits(rng.uniform(-200.0, 200.0, rows * d).astype(np.float32))      # large activations keep the sums in fp16's normal range
+    x, y = dev(xs), zeros_bytes(rows * d * 2)
+    sg = zeros_bytes(f * 2)
+    k.check(k.lib.tf_prefill_shared_expert_int4_block(k.handle, None, x.data_ptr(), 0, y.data_ptr(), 0, C.byref(g), C.byref(u), C.byref(dn),
+                                                      sg.data_ptr(), 0, f * 2, sg.data_ptr(), 0, f * 2, sa.data_ptr(), 0, f * 2, rows, d, f,
+                                                      d, d, 8, tfk.TF_BF16))
+    got = tfo.from_f16_bits(host(y, np.uint16).reshape(rows, d))
+    assert float(np.max(np.abs(got))) > 1e-3          # the case is not degenerate
+    for r in range(rows):
+        y1 = zeros_bytes(d * 2)
+        k.check(k.lib.tf_shared_expert_int8(k.handle, None, x.data_ptr(), r * d * 2, (r + 1) * d * 2, C.byref(g), C.byref(u), C.byref(dn),
+                                            y1.data_ptr(), 0, d * 2, sa.data_ptr(), 0, f * 2, tfk.TF_BF16))
+        assert tfo.rel_error(got[r], tfo.from_f16_bits(host(y1, np.uint16, d))) < tfo.Tolerance.quantInt8 * 4
 
 
 # ---------------------------------------------------------------------------------------------------- shared expert, block of rows

@@ -568,7 +568,11 @@ int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream, const
                             qmm_operands_ok(gw, xp, x_stride_elements, (int)d) && aligned16(uw) && aligned16(dw) &&
                             intermediate % TF_GROUP_SIZE == 0 && query_count <= (uint32_t)INT32_MAX;
     if (weight_bits == 8 && pointers && even && query_count >= 2) {
-        // 8-bit projections: rows in groups against each weight row, bit-identical to the rows one by one
+        // 8-bit projections.  Up to kShared8MfmaMinRows - 1 rows: rows in groups against each weight row, bit-identical to the
+        // rows one by one.  From there on the matrix cores: every weight is rounded to fp16 as half(q s + b) first (the
+        // reference's staged-affine rounding point), so a row agrees with the single-row chain within the 8-bit shared
+        // expert's tolerance, not bit for bit; weights below fp16's normal range (scales under about 1e-7) would lose their
+        // grid there.
         TF_REQUIRE(ctx, scratch_act_offset + (uint64_t)intermediate * 2 <= scratch_act_length, TF_ERR_SCRATCH_TOO_SMALL,
                    "SharedExpertInt8 scratch too small: scratchAct offset %llu + needed %llu exceeds length %llu",
                    (unsigned long long)scratch_act_offset, (unsigned long long)intermediate * 2, (unsigned long long)scratch_act_length);
