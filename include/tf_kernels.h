@@ -294,8 +294,8 @@ int32_t tf_shared_expert_int8_down(tf_ctx *ctx, tf_stream stream, const tf_proje
  * expert's tolerance, not bit for bit, and the caller's scratch (still validated: one row each, lengths in BYTES) is
  * left untouched.  weight_bits == 8 (PrefillSharedExpert's default): up to 15 rows in groups against each weight row,
  * bit-identical to repeated tf_shared_expert_int8; from 16 aligned rows on on the matrix cores with every weight
- * rounded to fp16 first, within the 8-bit shared expert's tolerance of the row chain (weights below fp16's normal
- * range, scales under about 1e-7, would lose their grid there).  query_count == 0 is a no-op.  d, intermediate > 0,
+ * rounded to fp16 first, within the 8-bit shared expert's tolerance of the row chain (scales keep their precision
+ * down to 2^-24; a weight below fp16's normal range, 6e-5, is kept to 6e-8).  query_count == 0 is a no-op.  d, intermediate > 0,
  * strides >= d (TF_ERR_INVALID_ARGUMENT); gate/up = (intermediate, d), down = (d, intermediate) or
  * TF_ERR_DIMENSION_MISMATCH. */
 int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream,

@@ -362,10 +362,10 @@ def test_prefill_shared_expert_block_with_8_bit_weights_is_the_row_chain(d, f, r
 
 def test_8_bit_block_on_matrix_cores_with_small_scales():
     # From 16 rows on the 8-bit block rounds every weight to fp16 (half(q s + b), the reference's staged-affine rounding point,
-    # tensorops.metal:57-94) while the row chain keeps q s + b in fp32.  Weights of magnitude 1e-3 and less (scales near 8e-6)
-    # sit near the bottom of fp16's normal range, where its spacing is still finer than the quantization grid: the block must
-    # stay within the 8-bit shared expert's tolerance of the row chain.  (Scales below about 1e-7 would fall into fp16's
-    # subnormals and lose the grid; the row chain is the path for such tensors.)
+    # tensorops.metal:57-94) while the row chain keeps q s + b in fp32.  Weights of magnitude 1e-3 and less have scales near
+    # 8e-6, far below fp16's normal range: converted to fp16 directly they would lose mantissa bits (0.7 % error measured), so
+    # the kernel carries a scale as mantissa and power of two.  The block must stay within the 8-bit shared expert's tolerance
+    # of the row chain.
     import ctypes as C
     d, f, rows = 1024, 256, 32
     c = _int8_case(d, f, 0x6A1, weight_range=1e-3)

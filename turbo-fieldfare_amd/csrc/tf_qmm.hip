@@ -433,14 +433,27 @@ __global__ __launch_bounds__(64) void qmm8_nt_kernel(const half_t *X, long ldx, 
             }
         }
     };
+    // 16 bytes -> 16 fp16 weights half(q s + b).  An 8-bit scale is a 255th of the group's range and usually lies below
+    // fp16's normal range, where a direct conversion would drop mantissa bits: a bf16 scale goes in as its mantissa (in
+    // [1, 2)) and its power of two (exact in fp16 down to 2^-24) separately, w = (q m) 2^e + b.
     auto expand = [&](const u32x4 w, uint16_t sv, uint16_t bv, half8_t &first, half8_t &last) {
-        const half_t sh = (half_t)sb_to_f32<SD>(sv), bh = (half_t)sb_to_f32<SD>(bv);
-        const half2_t s2 = {sh, sh}, b2 = {bh, bh}, bias = {(half_t)1024.0f, (half_t)1024.0f};
+        const float sf = sb_to_f32<SD>(sv);
+        const half_t bh = (half_t)sb_to_f32<SD>(bv);
+        half_t mh, ph;
+        if constexpr (SD == 0) {
+            const uint32_t bits = __float_as_uint(sf);
+            mh = (half_t)__uint_as_float((bits & 0x807FFFFFu) | 0x3F800000u);
+            ph = (half_t)__uint_as_float(bits & 0x7F800000u);      // 0 for a zero scale
+        } else {
+            mh = (half_t)sf;                                       // an fp16 scale is what it is
+            ph = (half_t)1.0f;
+        }
+        const half2_t m2 = {mh, mh}, p2 = {ph, ph}, b2 = {bh, bh}, bias = {(half_t)1024.0f, (half_t)1024.0f};
         u32x4 lo, hi;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const half2_t q = as_half2(__builtin_amdgcn_perm(0x64646464u, w[j >> 1], (j & 1) ? 0x04030402u : 0x04010400u)) - bias;
-            const uint32_t v = as_u32(__builtin_elementwise_fma(q, s2, b2));
+            const uint32_t v = as_u32(__builtin_elementwise_fma(q * m2, p2, b2));
             if (j < 4) lo[j] = v; else hi[j - 4] = v;
         }
         first = __builtin_bit_cast(half8_t, lo);
@@ -571,8 +584,8 @@ int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream, const
         // 8-bit projections.  Up to kShared8MfmaMinRows - 1 rows: rows in groups against each weight row, bit-identical to the
         // rows one by one.  From there on the matrix cores: every weight is rounded to fp16 as half(q s + b) first (the
         // reference's staged-affine rounding point), so a row agrees with the single-row chain within the 8-bit shared
-        // expert's tolerance, not bit for bit; weights below fp16's normal range (scales under about 1e-7) would lose their
-        // grid there.
+        // expert's tolerance, not bit for bit (scales keep their precision down to 2^-24; weights themselves below fp16's
+        // normal range, 6e-5, keep an absolute spacing of 6e-8).
         TF_REQUIRE(ctx, scratch_act_offset + (uint64_t)intermediate * 2 <= scratch_act_length, TF_ERR_SCRATCH_TOO_SMALL,
                    "SharedExpertInt8 scratch too small: scratchAct offset %llu + needed %llu exceeds length %llu",
                    (unsigned long long)scratch_act_offset, (unsigned long long)intermediate * 2, (unsigned long long)scratch_act_length);
