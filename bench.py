@@ -34,7 +34,8 @@ def int4_matrix_bytes(rows, cols):
 # per-unit algorithmic bytes (what one launch must move at least once)
 ROUTER_BYTES = E * D + 2 * E * (D // 64) * 2 + D * 2 + D * 2 + E * 2 + TOPK * 4 + TOPK * 2   # W + s/b + hidden + eff + gains + outputs
 # HBM bytes one phase-1 launch moves, from hardware counters (profiles/bench_hbm_traffic_counters.txt): FETCH_SIZE 8895.6 KiB
-# x 2.0 (the factor a plain 1 GiB copy calibrates) + WRITE_SIZE 22.1 KiB x 1.0.
+# x 2.0 (the factor a plain 1 GiB copy calibrates) + WRITE_SIZE 22.1 KiB x 1.0.  Collected before the kernel's weight loads
+# became non-temporal; what it must fetch is the same.
 PHASE1_TRAFFIC_BYTES = int(8895.6 * 1024 * 1.9999 + 22.1 * 1024)
 PHASE1_BYTES = TOPK * 2 * int4_matrix_bytes(F_MOE, D) + D * 2 + TOPK * F_MOE * 2             # gate+up of 8 experts + x + acts out
 PHASE2_BYTES = TOPK * int4_matrix_bytes(D, F_MOE) + TOPK * F_MOE * 2 + TOPK * 2 + D * 2 + D * 2   # down of 8 + acts in + w + residual + y
@@ -96,6 +97,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip lm_head / GEMV / shared-expert side measurements")
     ap.add_argument("--no-layer-chain", action="store_true", help="skip the whole-decoder-layer graph (long under a counter-collecting profiler)")
+    ap.add_argument("--layer-chain-fork", action="store_true",
+                    help="also replay the layer chain with the shared expert on a second captured stream (a graph that forks and joins; "
+                         "not part of the default run, and not meant to run under a profiler)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (a known-size reference for hardware byte counters)")
     ap.add_argument("--only-small-m", type=int, nargs="+", metavar="M",
@@ -162,6 +166,7 @@ def main():
     # into HIP graphs and replayed: `graph_steps` steps per graph, plus one remainder graph, exactly `steps` in all.
     # One ROUND = exactly `steps` steps; rounds repeat until MIN_TIMED_MS of device time have passed (with the driver's
     # --steps 20 a single round lasts 0.3 ms, far too short a sample) and the median round is reported.
+    note("decode step: warm-up, graph capture, timed rounds")
     graph_steps = min(64, args.steps)
     n_full, rem = divmod(args.steps, graph_steps)
     graphs = {}
@@ -188,6 +193,7 @@ def main():
     stream = side.cuda_stream
 
     # the same loop launched call by call (no graph): what a host that encodes every step itself would see
+    note("decode step: eager launches")
     with torch.cuda.stream(side):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
@@ -197,6 +203,7 @@ def main():
 
     # ---- latency floor of the step: three dependent launches of the step's grid shapes that move no data, plus the step's
     # bytes at the rate a plain streaming read reaches in this run.  The step cannot go below that with three launches.
+    note("latency floor: empty launch chain, streaming read")
     words = torch.zeros(8, dtype=torch.int32, device="cuda")
     wp0 = words.data_ptr()
 
@@ -218,6 +225,7 @@ def main():
     # ---- per-kernel durations: the library brackets the step's three launches with HIP events on the launch stream
     # (eager launches; a spin kernel is queued first so that the host is ahead of the GPU and the events bracket
     # back-to-back execution, not host gaps).
+    note("decode step: per-kernel event brackets")
     n_ev = min(args.steps, 128)
     k.set_step_timing(True)
     times = []
@@ -250,6 +258,7 @@ def main():
         "roofline": {"bound": "hbm", "kernel": "phase1_long_kernel<2,3,bf16,fused top-8> (expert selection + gate/up/GeGLU of 8 experts)",
                      "achieved": round(p1_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(p1_gbps / HBM_PEAK_GBPS, 4), "traffic": PHASE1_TRAFFIC_BYTES,
+                     "traffic_from": "rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE of this kernel before its loads became non-temporal (same bytes to fetch)",
                      "algorithmic_bytes_per_launch": PHASE1_BYTES, "avg_launch_us": round(t_p1, 3),
                      "latency_floor_us": round(latency_floor_us, 3),
                      "latency_floor": {"what": "three dependent launches of the step's grid shapes that move no data + the step's "
@@ -276,12 +285,16 @@ def main():
         torch.cuda.synchronize()
         del src, dst
     if not args.no_extras:
+        note("extras: lm_head, GEMV, attention, shared expert")
         out["extras"] = extras(torch, tfk, k, gen, lib, h, stream)
+        note("extras: small-M verification sizes, 2048-token prefill")
         out["extras"].update(multi_token_extras(torch, tfk, k, gen, lib, h, stream, layers[0], offs, stride))
         if not args.no_layer_chain:
-            out["extras"].update(layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride))
+            note("extras: whole decoder layer chain")
+            out["extras"].update(layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=args.layer_chain_fork))
 
     if not args.no_cpu:
+        note("CPU baseline legs")
         out["cpu_baseline"] = cpu_baseline(torch, layers, hidden, idx, wts, y, offs, stride, payload, args)
         if not args.no_extras:
             cpu_extras(torch, gen, out["extras"], layers[0], offs, stride, payload)
@@ -289,6 +302,11 @@ def main():
 
 
 MIN_TIMED_MS = 50.0     # every figure comes from at least this much device time
+
+
+def note(section):
+    """Names the section that is about to use the GPU, on stderr and flushed: the last line seen names the case if a run dies."""
+    print(f"[bench] {section}", file=sys.stderr, flush=True)
 
 
 def replay_rounds(torch, side, replay_once, min_ms=MIN_TIMED_MS, min_rounds=5, max_rounds=4000):
@@ -499,7 +517,7 @@ def extras(torch, tfk, k, gen, lib, h, stream):
     return res
 
 
-def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride):
+def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=False):
     """One token through whole sliding-window decoder layers, every stage a call of the library and nothing on the host in
     between: input norm -> q/k/v projections (k, v straight into their cache row) -> per-head norm + RoPE -> attention over a
     1024-row window -> output projection -> post-attention setup -> shared expert + norm, router + 8 routed experts -> layer
@@ -588,7 +606,7 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride):
     results = {}
     with torch.cuda.stream(side):
         hidden0 = b["hidden"].clone()
-        for label, br in (("serial", None), ("forked", branch)):
+        for label, br in (("serial", None), ("forked", branch)) if fork else (("serial", None),):
             g = torch.cuda.CUDAGraph()
             with torch.cuda.graph(g, stream=side):
                 st = torch.cuda.current_stream().cuda_stream
@@ -599,21 +617,21 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride):
             side.synchronize()
             rounds, _ = replay_rounds(torch, side, g.replay)
             results[label] = (float(np.median(rounds)) * 1e3 / per_graph, b["hidden"].clone())
-    us, us_forked = results["serial"][0], results["forked"][0]
-    assert torch.equal(results["forked"][1], results["serial"][1]), "forked and serial layer chains disagree"
+    us = results["serial"][0]
+    if fork:
+        assert torch.equal(results["forked"][1], results["serial"][1]), "forked and serial layer chains disagree"
     bad = [n for n, t in b.items() if t.dtype == torch.float16 and not bool(torch.isfinite(t.float()).all())]
     assert not bad, f"non-finite values after the replays in {bad}"
     layer_bytes = (int4_matrix_bytes(NQ * HD + 2 * NKV * HD, D) + int4_matrix_bytes(D, NQ * HD) + SHARED_BYTES + STEP_BYTES
                    + 2 * WINDOW * NKV * HD * 2)
-    return {"decode_layer_sliding_window": {
-        "workload": "one token through one whole decoder layer (16q/8kv x 256, window 1024, shared 2112, 8 of 128 experts), 30 layers per graph replay",
-        "us_per_layer": round(us, 2), "ms_per_30_layers": round(us * 30 / 1e3, 3), "algorithmic_bytes_per_layer": layer_bytes,
-        "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 17,
-        "graph": "one in-order chain of launches",
-        "us_per_layer_shared_expert_on_forked_branch": round(us_forked, 2),
-        "forked_branch_note": "the shared expert + its norm on a second captured stream (event fork after the post-attention setup, join before the "
-                              "layer tail, as the reference commits sharedCB without waiting); bit-identical; the cross-queue fork and join cost more than "
-                              "the 13 us of launches they overlap"}}
+    res = {"workload": "one token through one whole decoder layer (16q/8kv x 256, window 1024, shared 2112, 8 of 128 experts), 30 layers per graph replay",
+           "us_per_layer": round(us, 2), "ms_per_30_layers": round(us * 30 / 1e3, 3), "algorithmic_bytes_per_layer": layer_bytes,
+           "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 17, "graph": "one in-order chain of launches"}
+    if fork:
+        res["us_per_layer_shared_expert_on_forked_branch"] = round(results["forked"][0], 2)
+        res["forked_branch_note"] = ("the shared expert + its norm on a second captured stream (event fork after the post-attention setup, join "
+                                     "before the layer tail, as the reference commits sharedCB without waiting); bit-identical")
+    return {"decode_layer_sliding_window": res}
 
 
 def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, small_sizes=(2, 4, 8, 16, 32, 64, 128), small_only=False,
