@@ -519,9 +519,9 @@ def extras(torch, tfk, k, gen, lib, h, stream):
 
 def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=False):
     """One token through whole sliding-window decoder layers, every stage a call of the library and nothing on the host in
-    between: input norm -> q/k/v projections (k, v straight into their cache row) -> per-head norm + RoPE -> attention over a
-    1024-row window -> output projection -> post-attention setup -> shared expert + norm, router + 8 routed experts -> layer
-    tail.  The layers rotate over the resident expert pools and as many sets of dense weights; replayed from a HIP graph."""
+    between: input norm + q/k/v projections in one launch (k, v straight into their cache row) -> per-head norm + RoPE ->
+    attention over a 1024-row window -> output projection -> post-attention setup -> shared expert, router + 8 routed experts ->
+    norm of the shared expert's output + layer tail in one launch.  The layers rotate over the resident expert pools and as many sets of dense weights; replayed from a HIP graph."""
     import ctypes as C
     HD, NQ, NKV, WINDOW = 256, 16, 8, 1024
     n_layers = len(layers)
@@ -562,11 +562,12 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=Fal
         (RealForwardRunner.swift:1570-1594); the branch forks after the post-attention setup and joins before the layer tail."""
         w, (pool, r) = dense[i % n_layers], layers[i % n_layers]
         ptr = lambda name: w[name].data_ptr()
-        rc = lib.tf_rmsnorm_bf16w(h, st, p("hidden"), 0, ptr("input_norm"), 0, p("x_norm"), 0, D, 1e-6)
         qkv = []
         for name in ("q", "k", "v"):
             qkv += [w[name][0].data_ptr(), 0, w[name][1].data_ptr(), 0, w[name][2].data_ptr(), 0]
-        rc |= lib.tf_fused_qkv_gemv(h, st, *qkv, p("x_norm"), p("q"), 0, ptr("k_cache"), kv_off, ptr("v_cache"), kv_off, NQ * HD, NKV * HD, D, tfk.TF_BF16)
+        # the input norm runs inside the projection launch
+        rc = lib.tf_fused_norm_qkv_gemv(h, st, ptr("input_norm"), 0, 1e-6, *qkv, p("hidden"), p("q"), 0, ptr("k_cache"), kv_off, ptr("v_cache"), kv_off,
+                                        NQ * HD, NKV * HD, D, tfk.TF_BF16)
         rc |= lib.tf_fused_qkv_epilogue(h, st, p("q"), 0, ptr("k_cache"), kv_off, ptr("v_cache"), kv_off, ptr("q_norm"), 0, ptr("k_norm"), 0,
                                         HD, NQ, NKV, position, 1e4, HD // 2, 1e-6)
         rc |= lib.tf_attention_swa(h, st, p("q"), 0, ptr("k_cache"), 0, ptr("v_cache"), 0, p("attn"), 0, HD, NQ, NKV, position + 1, WINDOW, 1.0, 0)
@@ -583,7 +584,6 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=Fal
             st_shared = branch.cuda_stream
         rc |= lib.tf_shared_expert_int4(h, st_shared, p("dense_x"), 0, D * 2, C.byref(g), C.byref(u), C.byref(dn), p("shared"), 0, D * 2, p("sg"), 0,
                                         F_SHARED * 2, p("su"), 0, F_SHARED * 2, p("sa"), 0, F_SHARED * 2, 4, tfk.TF_BF16)
-        rc |= lib.tf_rmsnorm_bf16w(h, st_shared, p("shared"), 0, ptr("post_ffn1"), 0, p("h1"), 0, D, 1e-6)
         rc |= lib.tf_moe_decode_step(h, st, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, p("router_x"), r["eff"].data_ptr(), 0,
                                      r["gain"].data_ptr(), 0, pool.data_ptr(), stride, E, C.byref(off), p("routed_x"), p("acts"), p("zero"), p("h2"),
                                      p("idx"), p("wts"), D, F_MOE, TOPK, tfk.TF_BF16)
@@ -591,7 +591,9 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=Fal
             join = torch.cuda.Event()
             join.record(branch)
             torch.cuda.current_stream().wait_event(join)
-        rc |= lib.tf_fused_layer_tail(h, st, p("h2"), p("h1"), p("hidden"), ptr("post_ffn2"), 0, ptr("post_ffn"), 0, D, 1e-6, 1.0)
+        # the norm of the shared expert's output runs inside the tail launch
+        rc |= lib.tf_fused_layer_tail_shared_norm(h, st, p("h2"), p("shared"), p("hidden"), ptr("post_ffn1"), 0, ptr("post_ffn2"), 0, ptr("post_ffn"), 0,
+                                                  D, 1e-6, 1.0)
         if rc != 0:
             raise RuntimeError("layer chain failed: " + k.last_error())
 
@@ -626,7 +628,7 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=Fal
                    + 2 * WINDOW * NKV * HD * 2)
     res = {"workload": "one token through one whole decoder layer (16q/8kv x 256, window 1024, shared 2112, 8 of 128 experts), 30 layers per graph replay",
            "us_per_layer": round(us, 2), "ms_per_30_layers": round(us * 30 / 1e3, 3), "algorithmic_bytes_per_layer": layer_bytes,
-           "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 17, "graph": "one in-order chain of launches"}
+           "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 15, "graph": "one in-order chain of launches"}
     if fork:
         res["us_per_layer_shared_expert_on_forked_branch"] = round(results["forked"][0], 2)
         res["forked_branch_note"] = ("the shared expert + its norm on a second captured stream (event fork after the post-attention setup, join "

@@ -181,6 +181,21 @@ int32_t tf_fused_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *q_weights, 
                           uint64_t q_out_offset, void *k_out, uint64_t k_out_offset, void *v_out, uint64_t v_out_offset, uint32_t q_rows,
                           uint32_t kv_rows, uint32_t n, tf_dtype scale_dtype);
 
+/* RMSNorm.encodeBF16W (Kernels/Primitives/RMSNorm.swift:17-66) + FusedQKVGEMV.encode in ONE launch: the input norm of a
+ * decoder layer feeds nothing but the three projections (RealForwardRunner.swift: the per-layer decode loop), so every
+ * block normalises `hidden` (fp16[n], raw) with norm_weight (bf16[n]) on its way into LDS instead of a launch of its own
+ * writing a normalised copy.  q_out / k_out / v_out equal tf_rmsnorm_bf16w followed by tf_fused_qkv_gemv bit for bit.
+ * Shapes the one-launch kernel does not take (n <= 1024, unaligned operands) run the two steps through the context's
+ * one-row buffer (n <= 16384, else TF_ERR_SCRATCH_TOO_SMALL). */
+int32_t tf_fused_norm_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *norm_weight, uint64_t norm_weight_offset, float eps,
+                               const void *q_weights, uint64_t q_weights_offset, const void *q_scales, uint64_t q_scales_offset,
+                               const void *q_biases, uint64_t q_biases_offset, const void *k_weights, uint64_t k_weights_offset,
+                               const void *k_scales, uint64_t k_scales_offset, const void *k_biases, uint64_t k_biases_offset,
+                               const void *v_weights, uint64_t v_weights_offset, const void *v_scales, uint64_t v_scales_offset,
+                               const void *v_biases, uint64_t v_biases_offset, const void *hidden, void *q_out, uint64_t q_out_offset,
+                               void *k_out, uint64_t k_out_offset, void *v_out, uint64_t v_out_offset, uint32_t q_rows, uint32_t kv_rows,
+                               uint32_t n, tf_dtype scale_dtype);
+
 /* ---- primitives on the path -------------------------------------------------------------------------------- */
 /* gelu_mul_fp16 (Metal/Primitives/utility.metal:6-18; dispatched at SharedExpertInt4.swift:76-86):
  * out = half(gelu_tanh(float(gate)) * float(up)). */
@@ -247,6 +262,14 @@ int32_t tf_prefill_post_attn_setup_block(tf_ctx *ctx, tf_stream stream, void *hi
 int32_t tf_fused_layer_tail(tf_ctx *ctx, tf_stream stream, const void *h2, const void *h1, void *hidden, const void *post_ffn2_weight,
                             uint64_t post_ffn2_weight_offset, const void *post_ffn_weight, uint64_t post_ffn_weight_offset, uint32_t d,
                             float eps, float layer_scalar);
+/* RMSNorm.encodeBF16W of the shared expert's output (RealForwardRunner.swift: h1 = rmsnorm(shared, post_ffn1)) + FusedLayerTail.encode
+ * in ONE launch: shared_out is the shared expert's raw output, h1 = half(shared_out * rsqrt(mean(shared_out^2) + eps) *
+ * post_ffn1_weight) is formed in registers and the tail proceeds as tf_fused_layer_tail.  Equal to the two calls up to the
+ * order in which the squares of shared_out are summed (a last-bit difference of 1/rms can move an fp16 rounding on a tie). */
+int32_t tf_fused_layer_tail_shared_norm(tf_ctx *ctx, tf_stream stream, const void *h2, const void *shared_out, void *hidden,
+                                        const void *post_ffn1_weight, uint64_t post_ffn1_weight_offset, const void *post_ffn2_weight,
+                                        uint64_t post_ffn2_weight_offset, const void *post_ffn_weight, uint64_t post_ffn_weight_offset,
+                                        uint32_t d, float eps, float layer_scalar);
 /* PrefillLayerTail.encode (Kernels/Prefill/Epilogues/PrefillLayerTail.swift:11-60) -> prefill_layer_tail_block
  * (Metal/Prefill/prefill.metal:255-334): the same for query_count strided rows. */
 int32_t tf_prefill_layer_tail_block(tf_ctx *ctx, tf_stream stream, const void *h2, uint64_t h2_offset, const void *h1,

@@ -165,3 +165,60 @@ def test_decode_step_of_a_sliding_window_layer():
         oh2 = tfo.k_moe_phase2(oblobs, mo["off"], oacts, owts, np.zeros(D, np.uint16), D, F_MOE)
         ofinal = tfo.k_layer_tail(oh2, oh1, ohid, L["post_ffn2"], L["post_ffn"], EPS, LAYER_SCALAR)
         assert tfo.rel_error(f(hidden_out), f(ofinal)) < 2 * TOL
+
+
+@pytest.mark.parametrize("n,q_rows,kv_rows", [(D, NQ * HD, NKV * HD), (512, 96, 64), (4096, 130, 66)])
+def test_norm_inside_the_qkv_launch_equals_norm_then_qkv(n, q_rows, kv_rows):
+    # tf_fused_norm_qkv_gemv = tf_rmsnorm_bf16w + tf_fused_qkv_gemv: one launch at the production width (every block normalises
+    # the row on its way into LDS), the two steps through the context's one-row buffer where the one-launch kernel does not apply
+    # (rows of at most 1024 values); bit for bit in both cases
+    rng = np.random.default_rng(n)
+    mats = [refcases.synthetic_int4(r, n, 0x77 + i, "qkv"[i]) for i, r in enumerate((q_rows, kv_rows, kv_rows))]
+    hidden = (rng.standard_normal(n) * 0.7).astype(np.float32).astype(np.float16).view(np.uint16)
+    nw = tfo.bf16_bits_array(1.0 + 0.1 * rng.standard_normal(n).astype(np.float32))
+    k = ctx()
+    lib, h = k.lib, k.handle
+    t = [[dev(a) for a in m] for m in mats]
+    d_hidden, d_nw, x_norm = dev(hidden), dev(nw), zeros_bytes(n * 2)
+    qkv = []
+    for m in t:
+        qkv += [m[0].data_ptr(), 0, m[1].data_ptr(), 0, m[2].data_ptr(), 0]
+    outs = [[dev(np.full(r, 0x7BFF, np.uint16)) for r in (q_rows, kv_rows, kv_rows)] for _ in range(2)]
+    k.check(lib.tf_rmsnorm_bf16w(h, None, d_hidden.data_ptr(), 0, d_nw.data_ptr(), 0, x_norm.data_ptr(), 0, n, EPS))
+    k.check(lib.tf_fused_qkv_gemv(h, None, *qkv, x_norm.data_ptr(), outs[0][0].data_ptr(), 0, outs[0][1].data_ptr(), 0, outs[0][2].data_ptr(), 0,
+                                  q_rows, kv_rows, n, tfk.TF_BF16))
+    k.check(lib.tf_fused_norm_qkv_gemv(h, None, d_nw.data_ptr(), 0, EPS, *qkv, d_hidden.data_ptr(), outs[1][0].data_ptr(), 0,
+                                       outs[1][1].data_ptr(), 0, outs[1][2].data_ptr(), 0, q_rows, kv_rows, n, tfk.TF_BF16))
+    for a, b_, m in zip(outs[0], outs[1], mats):
+        assert np.array_equal(host(a, np.uint16), host(b_, np.uint16))
+        want = gemv(m, tfo.k_rmsnorm_bf16w(hidden, nw, EPS))
+        assert tfo.rel_error(tfo.from_f16_bits(host(b_, np.uint16)), tfo.from_f16_bits(want)) < TOL
+    assert lib.tf_fused_norm_qkv_gemv(h, None, None, 0, EPS, *qkv, d_hidden.data_ptr(), outs[1][0].data_ptr(), 0, outs[1][1].data_ptr(), 0,
+                                      outs[1][2].data_ptr(), 0, q_rows, kv_rows, n, tfk.TF_BF16) == tfk.TF_ERR_INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("d", [D, 1000, 4096])
+def test_shared_norm_inside_the_layer_tail_equals_norm_then_tail(d):
+    # tf_fused_layer_tail_shared_norm = tf_rmsnorm_bf16w(shared, post_ffn1) + tf_fused_layer_tail: the squares of the shared
+    # expert's output are summed in another order, so 1/rms may differ in its last bit and move an fp16 rounding that sits on
+    # a tie: at most 0.5 % of the elements, each by one fp16 step of h1; and within the reference test's tolerance of the oracle
+    rng = np.random.default_rng(d)
+    bits = lambda a: a.astype(np.float32).astype(np.float16).view(np.uint16)
+    h2, shared, hidden = bits(rng.standard_normal(d) * 0.3), bits(rng.standard_normal(d) * 2.0), bits(rng.standard_normal(d))
+    w1, w2, w3 = (tfo.bf16_bits_array(1.0 + 0.1 * rng.standard_normal(d).astype(np.float32)) for _ in range(3))
+    k = ctx()
+    lib, h = k.lib, k.handle
+    d_h2, d_sh, d_w1, d_w2, d_w3 = dev(h2), dev(shared), dev(w1), dev(w2), dev(w3)
+    hid_a, hid_b, h1 = dev(hidden), dev(hidden), zeros_bytes(d * 2)
+    k.check(lib.tf_rmsnorm_bf16w(h, None, d_sh.data_ptr(), 0, d_w1.data_ptr(), 0, h1.data_ptr(), 0, d, EPS))
+    k.check(lib.tf_fused_layer_tail(h, None, d_h2.data_ptr(), h1.data_ptr(), hid_a.data_ptr(), d_w2.data_ptr(), 0, d_w3.data_ptr(), 0, d, EPS, LAYER_SCALAR))
+    k.check(lib.tf_fused_layer_tail_shared_norm(h, None, d_h2.data_ptr(), d_sh.data_ptr(), hid_b.data_ptr(), d_w1.data_ptr(), 0, d_w2.data_ptr(), 0,
+                                                d_w3.data_ptr(), 0, d, EPS, LAYER_SCALAR))
+    a, b_ = tfo.from_f16_bits(host(hid_a, np.uint16)), tfo.from_f16_bits(host(hid_b, np.uint16))
+    differ = a != b_
+    assert differ.mean() <= 0.005
+    assert np.max(np.abs(a - b_)) <= 2.0 ** -8 * max(1.0, float(np.max(np.abs(a))))
+    want = tfo.k_layer_tail(h2, tfo.k_rmsnorm_bf16w(shared, w1, EPS), hidden, w2, w3, EPS, LAYER_SCALAR)
+    assert tfo.rel_error(b_, tfo.from_f16_bits(want)) < tfo.Tolerance.fp16Reduction
+    assert lib.tf_fused_layer_tail_shared_norm(h, None, d_h2.data_ptr(), d_sh.data_ptr(), hid_b.data_ptr(), None, 0, d_w2.data_ptr(), 0,
+                                               d_w3.data_ptr(), 0, d, EPS, LAYER_SCALAR) == tfk.TF_ERR_INVALID_ARGUMENT

@@ -124,12 +124,14 @@ EXPORTS = {
     "tf_dequant_int4_gemv": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32, i32]),
     "tf_dequant_int8_gemv": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32, i32]),
     "tf_fused_qkv_gemv": (i32, [vp, vp] + [vp, u64] * 9 + [vp] + [vp, u64] * 3 + [u32, u32, u32, i32]),
+    "tf_fused_norm_qkv_gemv": (i32, [vp, vp, vp, u64, C.c_float] + [vp, u64] * 9 + [vp] + [vp, u64] * 3 + [u32, u32, u32, i32]),
     "tf_gelu_mul_fp16": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32]),
     "tf_rmsnorm_bf16w": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32, C.c_float]),
     "tf_fused_post_attn_setup": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, u64, vp, u64, vp, u64, u32, C.c_float]),
     "tf_prefill_post_attn_setup_block": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64,
                                                u32, u32, u32, u32, u32, u32, u32, C.c_float]),
     "tf_fused_layer_tail": (i32, [vp, vp, vp, vp, vp, vp, u64, vp, u64, u32, C.c_float, C.c_float]),
+    "tf_fused_layer_tail_shared_norm": (i32, [vp, vp, vp, vp, vp, vp, u64, vp, u64, vp, u64, u32, C.c_float, C.c_float]),
     "tf_prefill_layer_tail_block": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, u32, u32, u32,
                                           C.c_float, C.c_float]),
     "tf_shared_expert_int4": (i32, [vp, vp, vp, u64, u64, C.POINTER(Projection), C.POINTER(Projection), C.POINTER(Projection),

@@ -111,10 +111,13 @@ struct GemvSegments {
     uint32_t tile_end[3];   // running total of tiles up to and including each matrix
 };
 
-template <int RT, int NP, int SD>
-__global__ __launch_bounds__(256, 4) void qkv_gemv_long_kernel(GemvSegments g, const half_t *x, int k) {
+// FUSE_NORM: x is the raw hidden vector and every block normalises it on the way into LDS (rmsnorm_bf16w with norm_w), so the
+// input norm of a decoder layer needs no launch of its own.
+template <int RT, int NP, int SD, bool FUSE_NORM>
+__global__ __launch_bounds__(256, 4) void qkv_gemv_long_kernel(GemvSegments g, const half_t *x, const uint16_t *norm_w, float eps, int k) {
     __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
     __shared__ float xsum[XStage::kMaxK / 32];
+    __shared__ float norm_partial[4];
     const int lane = threadIdx.x & 63;
     const long wave = uniform_int((int)(((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6));
     const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
@@ -137,11 +140,19 @@ __global__ __launch_bounds__(256, 4) void qkv_gemv_long_kernel(GemvSegments g, c
         rs.load(t, g.W[seg] + local * tile_bytes, g.S[seg] + local * sb_bytes, g.B[seg] + local * sb_bytes, (long)g.rows[seg] - local * RT);
     };
     long t0 = wave, t1 = wave + nwaves;
-    XStage stage;
-    stage.request(x, k);
-    if (t0 < ntiles) request(ta, t0);
-    if (t1 < ntiles) request(tb, t1);
-    stage.publish(k, xa, xsum);
+    if constexpr (FUSE_NORM) {
+        XNormStage stage;
+        stage.request(x, norm_w, k);
+        if (t0 < ntiles) request(ta, t0);
+        if (t1 < ntiles) request(tb, t1);
+        stage.publish(eps, k, xa, xsum, norm_partial);
+    } else {
+        XStage stage;
+        stage.request(x, k);
+        if (t0 < ntiles) request(ta, t0);
+        if (t1 < ntiles) request(tb, t1);
+        stage.publish(k, xa, xsum);
+    }
     if (t0 >= ntiles) return;
     rs.init_x_lds(xa, xsum, k);
     auto emit = [&](const typename RowStream<RT, NP>::Tile &t, long at) {
@@ -612,13 +623,14 @@ int32_t tf_prefill_rmsnorm_no_scale_perhead_block(tf_ctx *ctx, tf_stream stream,
                               token_stride_elements, eps, "prefill_rmsnorm_no_scale_perhead_block");
 }
 
-int32_t tf_fused_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *q_weights, uint64_t q_weights_offset, const void *q_scales,
+static int32_t qkv_gemv_entry(tf_ctx *ctx, tf_stream stream, const char *who, const void *norm_weight, uint64_t norm_weight_offset, float eps, const void *q_weights, uint64_t q_weights_offset, const void *q_scales,
                           uint64_t q_scales_offset, const void *q_biases, uint64_t q_biases_offset, const void *k_weights,
                           uint64_t k_weights_offset, const void *k_scales, uint64_t k_scales_offset, const void *k_biases,
                           uint64_t k_biases_offset, const void *v_weights, uint64_t v_weights_offset, const void *v_scales,
                           uint64_t v_scales_offset, const void *v_biases, uint64_t v_biases_offset, const void *x, void *q_out,
                           uint64_t q_out_offset, void *k_out, uint64_t k_out_offset, void *v_out, uint64_t v_out_offset, uint32_t q_rows,
                           uint32_t kv_rows, uint32_t n, tf_dtype scale_dtype) {
+    const uint16_t *nw = norm_weight ? reinterpret_cast<const uint16_t *>(at(norm_weight, norm_weight_offset)) : nullptr;
     const void *w[3] = {q_weights, k_weights, v_weights};
     const void *s[3] = {q_scales, k_scales, v_scales};
     const void *b[3] = {q_biases, k_biases, v_biases};
@@ -629,13 +641,13 @@ int32_t tf_fused_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *q_weights, 
     const uint64_t yo[3] = {q_out_offset, k_out_offset, v_out_offset};
     const uint32_t rows[3] = {q_rows, kv_rows, kv_rows};
     for (int i = 0; i < 3; ++i) {
-        const int32_t rc = validate_gemv(ctx, "fused_qkv_gemv", w[i], wo[i], s[i], so[i], b[i], bo[i], x, 0, y[i], yo[i], rows[i], n,
+        const int32_t rc = validate_gemv(ctx, who, w[i], wo[i], s[i], so[i], b[i], bo[i], x, 0, y[i], yo[i], rows[i], n,
                                          scale_dtype, TF_FP16, 2);
         if (rc != TF_OK) return rc;
     }
     hipStream_t st = static_cast<hipStream_t>(stream);
     const LongPlan plan = plan_long_rows((int)n);
-    bool fast = aligned16(x) && n > 1024 && n <= (uint32_t)XStage::kMaxK && plan.rt > 0;
+    bool fast = aligned16(x) && n > 1024 && n <= (uint32_t)XStage::kMaxK && plan.rt > 0 && (!nw || aligned16(nw));
     for (int i = 0; i < 3; ++i) fast = fast && aligned16(at(w[i], wo[i]));
     if (fast) {
         GemvSegments g;
@@ -654,21 +666,63 @@ int32_t tf_fused_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *q_weights, 
         const half_t *xh = static_cast<const half_t *>(x);
 #define TF_QKV_CASE(RT_, NP_)                                                                                             \
     if (plan.rt == RT_ && plan.np == NP_) {                                                                               \
-        if (scale_dtype == TF_BF16) hipLaunchKernelGGL((qkv_gemv_long_kernel<RT_, NP_, 0>), dim3(grid), dim3(256), 0, st, g, xh, (int)n); \
-        else hipLaunchKernelGGL((qkv_gemv_long_kernel<RT_, NP_, 1>), dim3(grid), dim3(256), 0, st, g, xh, (int)n);        \
-        return check_launch(ctx, "fused_qkv_gemv");                                                                       \
+        if (nw) {                                                                                                         \
+            if (scale_dtype == TF_BF16) hipLaunchKernelGGL((qkv_gemv_long_kernel<RT_, NP_, 0, true>), dim3(grid), dim3(256), 0, st, g, xh, nw, eps, (int)n); \
+            else hipLaunchKernelGGL((qkv_gemv_long_kernel<RT_, NP_, 1, true>), dim3(grid), dim3(256), 0, st, g, xh, nw, eps, (int)n); \
+        } else {                                                                                                          \
+            if (scale_dtype == TF_BF16) hipLaunchKernelGGL((qkv_gemv_long_kernel<RT_, NP_, 0, false>), dim3(grid), dim3(256), 0, st, g, xh, nw, eps, (int)n); \
+            else hipLaunchKernelGGL((qkv_gemv_long_kernel<RT_, NP_, 1, false>), dim3(grid), dim3(256), 0, st, g, xh, nw, eps, (int)n); \
+        }                                                                                                                 \
+        return check_launch(ctx, who);                                                                                    \
     }
         TF_QKV_CASE(1, 1) TF_QKV_CASE(1, 2) TF_QKV_CASE(1, 3) TF_QKV_CASE(1, 4)
         TF_QKV_CASE(2, 1) TF_QKV_CASE(2, 2) TF_QKV_CASE(2, 3) TF_QKV_CASE(2, 4)
         TF_QKV_CASE(4, 1) TF_QKV_CASE(4, 2) TF_QKV_CASE(4, 3) TF_QKV_CASE(4, 4)
 #undef TF_QKV_CASE
     }
-    // any other shape or alignment: the three projections one after the other (same arithmetic per row)
+    // any other shape or alignment: the three projections one after the other (same arithmetic per row), after the norm as
+    // a launch of its own into the context's one-row buffer
+    if (nw) {
+        TF_REQUIRE(ctx, n <= kMaxHeadD, TF_ERR_SCRATCH_TOO_SMALL, "%s: rows of %u values exceed the context's one-row buffer (%u)", who, n, kMaxHeadD);
+        const int32_t rc = launch_rmsnorm_bf16w(ctx, st, x, nw, ctx->head_x_normed, n, eps);
+        if (rc != TF_OK) return rc;
+        x = ctx->head_x_normed;
+    }
     for (int i = 0; i < 3; ++i) {
         const int32_t rc = launch_gemv4(ctx, st, at(w[i], wo[i]), at(s[i], so[i]), at(b[i], bo[i]), x, at(y[i], yo[i]), rows[i], n, scale_dtype, TF_FP16);
         if (rc != TF_OK) return rc;
     }
     return TF_OK;
+}
+
+
+int32_t tf_fused_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *q_weights, uint64_t q_weights_offset, const void *q_scales,
+                          uint64_t q_scales_offset, const void *q_biases, uint64_t q_biases_offset, const void *k_weights,
+                          uint64_t k_weights_offset, const void *k_scales, uint64_t k_scales_offset, const void *k_biases,
+                          uint64_t k_biases_offset, const void *v_weights, uint64_t v_weights_offset, const void *v_scales,
+                          uint64_t v_scales_offset, const void *v_biases, uint64_t v_biases_offset, const void *x, void *q_out,
+                          uint64_t q_out_offset, void *k_out, uint64_t k_out_offset, void *v_out, uint64_t v_out_offset, uint32_t q_rows,
+                          uint32_t kv_rows, uint32_t n, tf_dtype scale_dtype) {
+    return qkv_gemv_entry(ctx, stream, "fused_qkv_gemv", nullptr, 0, 0.0f, q_weights, q_weights_offset, q_scales, q_scales_offset, q_biases,
+                          q_biases_offset, k_weights, k_weights_offset, k_scales, k_scales_offset, k_biases, k_biases_offset, v_weights,
+                          v_weights_offset, v_scales, v_scales_offset, v_biases, v_biases_offset, x, q_out, q_out_offset, k_out, k_out_offset,
+                          v_out, v_out_offset, q_rows, kv_rows, n, scale_dtype);
+}
+
+int32_t tf_fused_norm_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *norm_weight, uint64_t norm_weight_offset, float eps,
+                               const void *q_weights, uint64_t q_weights_offset, const void *q_scales, uint64_t q_scales_offset,
+                               const void *q_biases, uint64_t q_biases_offset, const void *k_weights, uint64_t k_weights_offset,
+                               const void *k_scales, uint64_t k_scales_offset, const void *k_biases, uint64_t k_biases_offset,
+                               const void *v_weights, uint64_t v_weights_offset, const void *v_scales, uint64_t v_scales_offset,
+                               const void *v_biases, uint64_t v_biases_offset, const void *hidden, void *q_out, uint64_t q_out_offset,
+                               void *k_out, uint64_t k_out_offset, void *v_out, uint64_t v_out_offset, uint32_t q_rows, uint32_t kv_rows,
+                               uint32_t n, tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx && norm_weight, TF_ERR_INVALID_ARGUMENT, "fused_norm_qkv_gemv: null argument");
+    TF_REQUIRE(ctx, norm_weight_offset % 2 == 0 && aligned(norm_weight, 2), TF_ERR_INVALID_ARGUMENT, "fused_norm_qkv_gemv: misaligned norm weight");
+    return qkv_gemv_entry(ctx, stream, "fused_norm_qkv_gemv", norm_weight, norm_weight_offset, eps, q_weights, q_weights_offset, q_scales,
+                          q_scales_offset, q_biases, q_biases_offset, k_weights, k_weights_offset, k_scales, k_scales_offset, k_biases,
+                          k_biases_offset, v_weights, v_weights_offset, v_scales, v_scales_offset, v_biases, v_biases_offset, hidden, q_out,
+                          q_out_offset, k_out, k_out_offset, v_out, v_out_offset, q_rows, kv_rows, n, scale_dtype);
 }
 
 }  // extern "C"

@@ -131,6 +131,7 @@ struct LayerTailArgs {
     const half_t *h2, *h1;
     half_t *hidden;
     const uint16_t *w_postffn2, *w_postffn;
+    const uint16_t *w_postffn1;   // not null: h1 is the shared expert's raw output and is normalised here first
     uint32_t rows, d;
     uint32_t h2_stride, h1_stride, hidden_stride;
     float eps, layer_scalar;
@@ -138,9 +139,11 @@ struct LayerTailArgs {
 
 // h12 = half(h1 + half(h2 * inv_rms(h2) * w_postffn2));
 // hidden <- half(half(hidden + half(h12 * inv_rms(h12) * w_postffn)) * half(layer_scalar)).
-template <bool VEC>
+// NORM_H1: h1 <- half(h1 * inv_rms(h1) * w_postffn1) first (rmsnorm_bf16w of the shared expert's output, otherwise a launch
+// of its own between the shared expert and this kernel).
+template <bool VEC, bool NORM_H1>
 __global__ __launch_bounds__(256) void layer_tail_kernel(LayerTailArgs a) {
-    __shared__ float partial[2][4];
+    __shared__ float partial[3][4];
     const uint32_t row = blockIdx.x;
     const RowSlice<VEC> rs{a.d};
     float x[kPerThread], w[kPerThread], h1[kPerThread], wp[kPerThread], hid[kPerThread];
@@ -149,6 +152,13 @@ __global__ __launch_bounds__(256) void layer_tail_kernel(LayerTailArgs a) {
     rs.load_f16(a.h1 + (size_t)row * a.h1_stride, h1);
     rs.load_bf16(a.w_postffn, wp);
     rs.load_f16(a.hidden + (size_t)row * a.hidden_stride, hid);
+    if constexpr (NORM_H1) {
+        float w1[kPerThread];
+        rs.load_bf16(a.w_postffn1, w1);
+        const float inv_h1 = block_inv_rms(h1, a.d, a.eps, partial[2]);
+#pragma unroll
+        for (int j = 0; j < kPerThread; ++j) h1[j] = round_half(h1[j] * inv_h1 * w1[j]);
+    }
     const float inv_h2 = block_inv_rms(x, a.d, a.eps, partial[0]);
 #pragma unroll
     for (int j = 0; j < kPerThread; ++j) x[j] = round_half(h1[j] + round_half(x[j] * inv_h2 * w[j]));
@@ -209,7 +219,8 @@ int32_t post_attn_setup_entry(tf_ctx *ctx, tf_stream stream, const char *who, vo
 }
 
 int32_t layer_tail_entry(tf_ctx *ctx, tf_stream stream, const char *who, const void *h2, uint64_t h2_offset, const void *h1,
-                         uint64_t h1_offset, void *hidden, uint64_t hidden_offset, const void *w_postffn2, uint64_t w_postffn2_offset,
+                         uint64_t h1_offset, void *hidden, uint64_t hidden_offset, const void *w_postffn1, uint64_t w_postffn1_offset,
+                         const void *w_postffn2, uint64_t w_postffn2_offset,
                          const void *w_postffn, uint64_t w_postffn_offset, uint32_t rows, uint32_t d, uint32_t h2_stride,
                          uint32_t h1_stride, uint32_t hidden_stride, float eps, float layer_scalar) {
     TF_REQUIRE(ctx, ctx && h2 && h1 && hidden && w_postffn2 && w_postffn, TF_ERR_INVALID_ARGUMENT, "%s: null argument", who);
@@ -224,7 +235,9 @@ int32_t layer_tail_entry(tf_ctx *ctx, tf_stream stream, const char *who, const v
     a.hidden = reinterpret_cast<half_t *>(at(hidden, hidden_offset));
     a.w_postffn2 = reinterpret_cast<const uint16_t *>(at(w_postffn2, w_postffn2_offset));
     a.w_postffn = reinterpret_cast<const uint16_t *>(at(w_postffn, w_postffn_offset));
-    TF_REQUIRE(ctx, aligned(a.h2, 2) && aligned(a.h1, 2) && aligned(a.hidden, 2) && aligned(a.w_postffn2, 2) && aligned(a.w_postffn, 2),
+    a.w_postffn1 = w_postffn1 ? reinterpret_cast<const uint16_t *>(at(w_postffn1, w_postffn1_offset)) : nullptr;
+    TF_REQUIRE(ctx, aligned(a.h2, 2) && aligned(a.h1, 2) && aligned(a.hidden, 2) && aligned(a.w_postffn2, 2) && aligned(a.w_postffn, 2) &&
+                   aligned(a.w_postffn1, 2),
                TF_ERR_INVALID_ARGUMENT, "%s: misaligned operand", who);
     a.rows = rows;
     a.d = d;
@@ -234,10 +247,16 @@ int32_t layer_tail_entry(tf_ctx *ctx, tf_stream stream, const char *who, const v
     a.eps = eps;
     a.layer_scalar = layer_scalar;
     const bool vec = d % 8 == 0 && rows_vectorizable(a.h2, h2_stride, rows) && rows_vectorizable(a.h1, h1_stride, rows) &&
-                     rows_vectorizable(a.hidden, hidden_stride, rows) && aligned16(a.w_postffn2) && aligned16(a.w_postffn);
+                     rows_vectorizable(a.hidden, hidden_stride, rows) && aligned16(a.w_postffn2) && aligned16(a.w_postffn) &&
+                     aligned16(a.w_postffn1);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (vec) hipLaunchKernelGGL(layer_tail_kernel<true>, dim3(rows), dim3(256), 0, st, a);
-    else hipLaunchKernelGGL(layer_tail_kernel<false>, dim3(rows), dim3(256), 0, st, a);
+    if (a.w_postffn1) {
+        if (vec) hipLaunchKernelGGL((layer_tail_kernel<true, true>), dim3(rows), dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((layer_tail_kernel<false, true>), dim3(rows), dim3(256), 0, st, a);
+    } else {
+        if (vec) hipLaunchKernelGGL((layer_tail_kernel<true, false>), dim3(rows), dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((layer_tail_kernel<false, false>), dim3(rows), dim3(256), 0, st, a);
+    }
     return check_launch(ctx, who);
 }
 
@@ -273,8 +292,18 @@ int32_t tf_prefill_post_attn_setup_block(tf_ctx *ctx, tf_stream stream, void *hi
 int32_t tf_fused_layer_tail(tf_ctx *ctx, tf_stream stream, const void *h2, const void *h1, void *hidden, const void *post_ffn2_weight,
                             uint64_t post_ffn2_weight_offset, const void *post_ffn_weight, uint64_t post_ffn_weight_offset, uint32_t d,
                             float eps, float layer_scalar) {
-    return layer_tail_entry(ctx, stream, "fused_layer_tail", h2, 0, h1, 0, hidden, 0, post_ffn2_weight, post_ffn2_weight_offset,
+    return layer_tail_entry(ctx, stream, "fused_layer_tail", h2, 0, h1, 0, hidden, 0, nullptr, 0, post_ffn2_weight, post_ffn2_weight_offset,
                             post_ffn_weight, post_ffn_weight_offset, 1, d, d, d, d, eps, layer_scalar);
+}
+
+int32_t tf_fused_layer_tail_shared_norm(tf_ctx *ctx, tf_stream stream, const void *h2, const void *shared_out, void *hidden,
+                                        const void *post_ffn1_weight, uint64_t post_ffn1_weight_offset, const void *post_ffn2_weight,
+                                        uint64_t post_ffn2_weight_offset, const void *post_ffn_weight, uint64_t post_ffn_weight_offset,
+                                        uint32_t d, float eps, float layer_scalar) {
+    TF_REQUIRE(ctx, ctx && post_ffn1_weight, TF_ERR_INVALID_ARGUMENT, "fused_layer_tail_shared_norm: null argument");
+    return layer_tail_entry(ctx, stream, "fused_layer_tail_shared_norm", h2, 0, shared_out, 0, hidden, 0, post_ffn1_weight,
+                            post_ffn1_weight_offset, post_ffn2_weight, post_ffn2_weight_offset, post_ffn_weight, post_ffn_weight_offset, 1, d,
+                            d, d, d, eps, layer_scalar);
 }
 
 int32_t tf_prefill_layer_tail_block(tf_ctx *ctx, tf_stream stream, const void *h2, uint64_t h2_offset, const void *h1,
@@ -282,7 +311,7 @@ int32_t tf_prefill_layer_tail_block(tf_ctx *ctx, tf_stream stream, const void *h
                                     uint64_t post_ffn2_weight_offset, const void *post_ffn_weight, uint64_t post_ffn_weight_offset,
                                     uint32_t query_count, uint32_t d, uint32_t h2_stride_elements, uint32_t h1_stride_elements,
                                     uint32_t hidden_stride_elements, float eps, float layer_scalar) {
-    return layer_tail_entry(ctx, stream, "prefill_layer_tail_block", h2, h2_offset, h1, h1_offset, hidden, hidden_offset,
+    return layer_tail_entry(ctx, stream, "prefill_layer_tail_block", h2, h2_offset, h1, h1_offset, hidden, hidden_offset, nullptr, 0,
                             post_ffn2_weight, post_ffn2_weight_offset, post_ffn_weight, post_ffn_weight_offset, query_count, d,
                             h2_stride_elements, h1_stride_elements, hidden_stride_elements, eps, layer_scalar);
 }
