@@ -520,8 +520,8 @@ def extras(torch, tfk, k, gen, lib, h, stream):
 def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=False):
     """One token through whole sliding-window decoder layers, every stage a call of the library and nothing on the host in
     between: input norm + q/k/v projections in one launch (k, v straight into their cache row) -> per-head norm + RoPE ->
-    attention over a 1024-row window -> output projection -> post-attention setup -> shared expert, router + 8 routed experts ->
-    norm of the shared expert's output + layer tail in one launch.  The layers rotate over the resident expert pools and as many sets of dense weights; replayed from a HIP graph."""
+    attention over a 1024-row window -> output projection -> post-attention setup -> router + 8 routed experts with the shared
+    expert riding along in the same three launches -> norm of the shared expert's output + layer tail in one launch.  The layers rotate over the resident expert pools and as many sets of dense weights; replayed from a HIP graph."""
     import ctypes as C
     HD, NQ, NKV, WINDOW = 256, 16, 8, 1024
     n_layers = len(layers)
@@ -582,11 +582,18 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=Fal
             fork.record(torch.cuda.current_stream())
             branch.wait_event(fork)
             st_shared = branch.cuda_stream
-        rc |= lib.tf_shared_expert_int4(h, st_shared, p("dense_x"), 0, D * 2, C.byref(g), C.byref(u), C.byref(dn), p("shared"), 0, D * 2, p("sg"), 0,
-                                        F_SHARED * 2, p("su"), 0, F_SHARED * 2, p("sa"), 0, F_SHARED * 2, 4, tfk.TF_BF16)
-        rc |= lib.tf_moe_decode_step(h, st, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, p("router_x"), r["eff"].data_ptr(), 0,
-                                     r["gain"].data_ptr(), 0, pool.data_ptr(), stride, E, C.byref(off), p("routed_x"), p("acts"), p("zero"), p("h2"),
-                                     p("idx"), p("wts"), D, F_MOE, TOPK, tfk.TF_BF16)
+        if branch is None:
+            # the shared expert rides along with the launches of the routed step (gate / up beside the router, down beside phase 1)
+            rc |= lib.tf_moe_decode_step_shared(h, st, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, p("router_x"), r["eff"].data_ptr(), 0,
+                                                r["gain"].data_ptr(), 0, pool.data_ptr(), stride, E, C.byref(off), p("routed_x"), p("acts"), p("zero"), p("h2"),
+                                                p("idx"), p("wts"), D, F_MOE, TOPK, tfk.TF_BF16, p("dense_x"), C.byref(g), C.byref(u), C.byref(dn), p("shared"),
+                                                p("sg"), p("su"), p("sa"))
+        else:
+            rc |= lib.tf_shared_expert_int4(h, st_shared, p("dense_x"), 0, D * 2, C.byref(g), C.byref(u), C.byref(dn), p("shared"), 0, D * 2, p("sg"), 0,
+                                            F_SHARED * 2, p("su"), 0, F_SHARED * 2, p("sa"), 0, F_SHARED * 2, 4, tfk.TF_BF16)
+            rc |= lib.tf_moe_decode_step(h, st, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, p("router_x"), r["eff"].data_ptr(), 0,
+                                         r["gain"].data_ptr(), 0, pool.data_ptr(), stride, E, C.byref(off), p("routed_x"), p("acts"), p("zero"), p("h2"),
+                                         p("idx"), p("wts"), D, F_MOE, TOPK, tfk.TF_BF16)
         if branch is not None:
             join = torch.cuda.Event()
             join.record(branch)
@@ -628,7 +635,7 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=Fal
                    + 2 * WINDOW * NKV * HD * 2)
     res = {"workload": "one token through one whole decoder layer (16q/8kv x 256, window 1024, shared 2112, 8 of 128 experts), 30 layers per graph replay",
            "us_per_layer": round(us, 2), "ms_per_30_layers": round(us * 30 / 1e3, 3), "algorithmic_bytes_per_layer": layer_bytes,
-           "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 15, "graph": "one in-order chain of launches"}
+           "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 13, "graph": "one in-order chain of launches"}
     if fork:
         res["us_per_layer_shared_expert_on_forked_branch"] = round(results["forked"][0], 2)
         res["forked_branch_note"] = ("the shared expert + its norm on a second captured stream (event fork after the post-attention setup, join "

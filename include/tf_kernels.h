@@ -498,6 +498,30 @@ int32_t tf_moe_decode_step_static(tf_ctx *ctx, tf_stream stream,
                                   void *out_indices, void *out_weights,
                                   uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype);
 
+/* tf_moe_decode_step with the layer's shared expert (tf_shared_expert_int4, 4-bit weights) riding along: the reference commits
+ * the shared expert on a command buffer of its own, beside the router and the routed experts
+ * (RealForwardRunner.swift:1570-1594); here its gate / up rows run as extra blocks of the router launch and its down rows as
+ * extra blocks of the routed phase 1, so the decoder layer has two launches fewer.  shared_x fp16[shared_gate->cols] ->
+ * shared_y fp16[shared_down->rows]; the three scratch vectors (fp16[shared_gate->rows] each) receive gate, up and the
+ * activation as tf_shared_expert_int4 leaves them.  Every output of either part equals the two separate calls bit for bit.
+ * Shapes whose rows do not take the shared tile shape (the production widths 2816 / 2112 do), or operands that are not 16-byte
+ * aligned, run the shared expert as its own launches first.  One scale_dtype for routed and shared weights. */
+int32_t tf_moe_decode_step_shared(tf_ctx *ctx, tf_stream stream,
+                                  const void *router_weights, uint64_t router_weights_offset,
+                                  const void *router_scales, uint64_t router_scales_offset,
+                                  const void *router_biases, uint64_t router_biases_offset,
+                                  const void *router_x,
+                                  const void *effective_scale, uint64_t effective_scale_offset,
+                                  const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                                  const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                  const tf_expert_offsets *routed_offsets,
+                                  const void *x, void *acts, const void *residual, void *y,
+                                  void *out_indices, void *out_weights,
+                                  uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype,
+                                  const void *shared_x, const tf_projection *shared_gate, const tf_projection *shared_up,
+                                  const tf_projection *shared_down, void *shared_y, void *shared_scratch_gate,
+                                  void *shared_scratch_up, void *shared_scratch_act);
+
 /* ---- lm_head ----------------------------------------------------------------------------------------------------------- */
 /* LMHeadChainInt4.encodeGreedyDecode (Kernels/Fusions/LMHeadChainInt4.swift:53-122) -> rmsnorm_bf16w,
  * lm_head_greedy_int4_rows_chunk_raw, lm_head_greedy_int4_rows_reduce (Metal/Sampling/logit.metal:692-787):

@@ -222,3 +222,49 @@ def test_shared_norm_inside_the_layer_tail_equals_norm_then_tail(d):
     assert tfo.rel_error(b_, tfo.from_f16_bits(want)) < tfo.Tolerance.fp16Reduction
     assert lib.tf_fused_layer_tail_shared_norm(h, None, d_h2.data_ptr(), d_sh.data_ptr(), hid_b.data_ptr(), None, 0, d_w2.data_ptr(), 0,
                                                d_w3.data_ptr(), 0, d, EPS, LAYER_SCALAR) == tfk.TF_ERR_INVALID_ARGUMENT
+
+
+@pytest.mark.parametrize("d,f,fs,misalign", [(D, F_MOE, F_SHARED, 0), (D, F_MOE, F_SHARED, 2), (256, 128, 192, 0), (2816, 704, 1088, 0)])
+def test_decode_step_with_the_shared_expert_riding_along_equals_the_two_calls(d, f, fs, misalign):
+    # tf_moe_decode_step_shared = tf_shared_expert_int4 + tf_moe_decode_step, every output of both bit for bit: at the production
+    # widths the shared expert's rows are extra blocks of the step's first two launches; with a misaligned shared input, rows too
+    # short for the row streamers or a width that takes another tile shape (1088 -> one-row tiles) it runs as its own launches
+    # first
+    c = M._decode_step_case(d, f, E, 0x5AE + d + fs)
+    shared = dict(gate=refcases.synthetic_int4(fs, d, 0x51, "sg"), up=refcases.synthetic_int4(fs, d, 0x52, "su"),
+                  down=refcases.synthetic_int4(d, fs, 0x53, "sd"))
+    dense_x = refcases.normal_f16(d, 0x54)
+    k = ctx()
+    lib, h = k.lib, k.handle
+    t = M._decode_step_tensors(c)
+    st = {n: [dev(a) for a in shared[n]] for n in shared}
+    gate, up, down = (tfk.projection(*st[n], r, cc) for n, r, cc in (("gate", fs, d), ("up", fs, d), ("down", d, fs)))
+    d_x = dev(np.concatenate([np.zeros(misalign // 2, np.uint16), dense_x]))
+    x_ptr = d_x.data_ptr() + misalign
+    off = tfk.ExpertOffsets(*c["off"].as_tuple())
+    results = []
+    for fused in (False, True):
+        outs = M._fresh_outs(d, f)
+        idx, wts, acts, y = outs
+        sy, sg, su, sa = (dev(np.full(n, 0x7BFF, np.uint16)) for n in (d, fs, fs, fs))
+        if fused:
+            k.check(lib.tf_moe_decode_step_shared(h, None, t["rW"].data_ptr(), 0, t["rS"].data_ptr(), 0, t["rB"].data_ptr(), 0, t["x"].data_ptr(),
+                                                  t["eff"].data_ptr(), 0, t["gain"].data_ptr(), 0, t["pool"].data_ptr(), c["stride"], E, off,
+                                                  t["x"].data_ptr(), acts.data_ptr(), t["res"].data_ptr(), y.data_ptr(), idx.data_ptr(),
+                                                  wts.data_ptr(), d, f, 8, tfk.TF_BF16, x_ptr, C.byref(gate), C.byref(up), C.byref(down),
+                                                  sy.data_ptr(), sg.data_ptr(), su.data_ptr(), sa.data_ptr()))
+        else:
+            k.check(lib.tf_shared_expert_int4(h, None, x_ptr, 0, d * 2, C.byref(gate), C.byref(up), C.byref(down), sy.data_ptr(), 0, d * 2,
+                                              sg.data_ptr(), 0, fs * 2, su.data_ptr(), 0, fs * 2, sa.data_ptr(), 0, fs * 2, 4, tfk.TF_BF16))
+            assert M._decode_step_call(k, t, c, d, f, E, outs) == tfk.TF_OK
+        results.append(M._read_outs(outs, d, f) + tuple(host(b_, np.uint16) for b_ in (sy, sg, su, sa)))
+    for a, b_ in zip(*results):
+        assert np.array_equal(a, b_)
+    # and the shared part is the shared expert the oracle computes
+    ref = tfo.shared_expert_ref(shared["gate"], shared["up"], shared["down"], tfo.from_f16_bits(dense_x), threads=8)
+    assert tfo.rel_error(tfo.from_f16_bits(results[1][4]), ref) < 6e-3
+    assert lib.tf_moe_decode_step_shared(h, None, t["rW"].data_ptr(), 0, t["rS"].data_ptr(), 0, t["rB"].data_ptr(), 0, t["x"].data_ptr(),
+                                         t["eff"].data_ptr(), 0, t["gain"].data_ptr(), 0, t["pool"].data_ptr(), c["stride"], E, off,
+                                         t["x"].data_ptr(), acts.data_ptr(), t["res"].data_ptr(), y.data_ptr(), idx.data_ptr(),
+                                         wts.data_ptr(), d, f, 8, tfk.TF_BF16, x_ptr, C.byref(gate), C.byref(up), C.byref(up),
+                                         sy.data_ptr(), sg.data_ptr(), su.data_ptr(), sa.data_ptr()) == tfk.TF_ERR_DIMENSION_MISMATCH

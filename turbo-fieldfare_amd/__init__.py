@@ -170,6 +170,9 @@ EXPORTS = {
                                  vp, vp, vp, vp, vp, vp, u32, u32, u32, i32]),
     "tf_moe_decode_step_static": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, vp, u64, vp, u64, vp, u64, u32, C.POINTER(ExpertOffsets),
                                         vp, vp, vp, vp, vp, vp, u32, u32, u32, i32]),
+    "tf_moe_decode_step_shared": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, vp, u64, vp, u64, vp, u64, u32, C.POINTER(ExpertOffsets),
+                                        vp, vp, vp, vp, vp, vp, u32, u32, u32, i32, vp, C.POINTER(Projection), C.POINTER(Projection),
+                                        C.POINTER(Projection), vp, vp, vp, vp]),
     "tf_prefill_router_gemma4_block": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64,
                                              u32, u32, u32, u32, u32]),
     "tf_prefill_make_token_expert_pairs": (i32, [vp, vp, i32, i32, vp]),

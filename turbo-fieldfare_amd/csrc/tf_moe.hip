@@ -78,17 +78,22 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t *W, co
     if (lane == 0) logits[e] = v;
 }
 
-// One block per expert row (aligned operands, d <= 4096).
+// One block per expert row (aligned operands, d <= 4096).  The kernels below are thin shells around `..._body` functions so
+// that two independent stages can share a launch (a block takes one role or the other by its index).
+template <int SD>
+__device__ __forceinline__ void router_logits_block_body(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *hidden,
+                                                         const uint16_t *eff, float *logits, int d, uint32_t e, float *partial) {
+    TF_STAMP(0, e * 4 + (threadIdx.x >> 6), 0);
+    const int groups = d >> 6;
+    const float v = router_row_block<SD>(W + (size_t)e * d, S + (size_t)e * groups * 2, B + (size_t)e * groups * 2, hidden, eff, d, partial);
+    if (threadIdx.x == 0) logits[e] = v;
+    TF_STAMP(0, e * 4 + (threadIdx.x >> 6), 1);
+}
 template <int SD>
 __global__ __launch_bounds__(256) void router_logits_block_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *hidden,
                                                                   const uint16_t *eff, float *logits, int d) {
     __shared__ float partial[4];
-    const uint32_t e = blockIdx.x;
-    TF_STAMP(0, blockIdx.x * 4 + (threadIdx.x >> 6), 0);
-    const int groups = d >> 6;
-    const float v = router_row_block<SD>(W + (size_t)e * d, S + (size_t)e * groups * 2, B + (size_t)e * groups * 2, hidden, eff, d, partial);
-    if (threadIdx.x == 0) logits[e] = v;
-    TF_STAMP(0, blockIdx.x * 4 + (threadIdx.x >> 6), 1);
+    router_logits_block_body<SD>(W, S, B, hidden, eff, logits, d, blockIdx.x, partial);
 }
 
 __global__ __launch_bounds__(64) void router_select_kernel(const float *logits, const uint16_t *per_expert_scale,
@@ -137,14 +142,11 @@ struct FusedSelect {
 // stages once in LDS.  Order of requests: activations, expert lookup, weights; the activations are arranged while the
 // weights are in flight (with the fused selection the weights are requested right after the block's barrier).
 template <int RT, int NP, int SD, bool FUSED>
-__global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_expert_offsets off, const half_t *x,
-                                                          half_t *acts, Phase1Geom g, FusedSelect fs) {
-    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
-    __shared__ float xsum[XStage::kMaxK / 32];
-    __shared__ uint32_t chosen[TF_MAX_STREAMED_EXPERTS];
-    __shared__ RankSelectLds sel;
+__device__ __forceinline__ void phase1_long_body(const RoutedArg &routed, const tf_expert_offsets &off, const half_t *x, half_t *acts,
+                                                 const Phase1Geom &g, const FusedSelect &fs, uint32_t block, u32x4 *xa, float *xsum,
+                                                 uint32_t *chosen, RankSelectLds &sel) {
     const int lane = threadIdx.x & 63;
-    const uint32_t unit = uniform_u32((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
+    const uint32_t unit = uniform_u32((block * blockDim.x + threadIdx.x) >> 6);
     const uint32_t tiles = (g.f + RT - 1) / RT;
     TF_STAMP(1, unit, 0);
     float my_logit = 0.0f;
@@ -172,7 +174,7 @@ __global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_e
             router_select_lanes(fs.logits, fs.per_expert_scale, fs.num_experts, g.top_k, lane, idx, weight);
             if ((uint32_t)lane < g.top_k) {
                 chosen[lane] = idx < fs.num_experts ? idx : fs.num_experts - 1;
-                if (blockIdx.x == 0) {
+                if (block == 0) {
                     fs.out_indices[lane] = idx;
                     fs.out_weights[lane] = weight;
                 }
@@ -187,7 +189,7 @@ __global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_e
     if (!live) return;
     if constexpr (FUSED) {
         request_weights(routed.pool + (uint64_t)uniform_u32(chosen[slot]) * routed.stride);
-        if (ranked && blockIdx.x == 0 && threadIdx.x < 64) {   // the step's outputs, off the path of the weight requests
+        if (ranked && block == 0 && threadIdx.x < 64) {   // the step's outputs, off the path of the weight requests
             uint32_t idx;
             half_t weight;
             rank_select_weights(sel, chosen, fs.per_expert_scale, lane, idx, weight);
@@ -209,6 +211,16 @@ __global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_e
             if (row0 + r < g.f) store_act(acts, slot * g.f + row0 + r, gate[r], up[r]);
     }
     TF_STAMP(1, unit, 4);
+}
+
+template <int RT, int NP, int SD, bool FUSED>
+__global__ __launch_bounds__(256) void phase1_long_kernel(RoutedArg routed, tf_expert_offsets off, const half_t *x,
+                                                          half_t *acts, Phase1Geom g, FusedSelect fs) {
+    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
+    __shared__ float xsum[XStage::kMaxK / 32];
+    __shared__ uint32_t chosen[TF_MAX_STREAMED_EXPERTS];
+    __shared__ RankSelectLds sel;
+    phase1_long_body<RT, NP, SD, FUSED>(routed, off, x, acts, g, fs, blockIdx.x, xa, xsum, chosen, sel);
 }
 
 // D <= 1024: half-wave per row, NPASS passes: 2 * NPASS rows of gate and up per wave.
@@ -335,15 +347,22 @@ __global__ __launch_bounds__(512) void phase2_generic_kernel(RoutedArg routed, t
 // ------------------------------------------------------------------------------------------------ shared expert
 // gate and up tiles share the activations; both sums are rounded to fp16 (the reference's two GEMVs write fp16)
 // before GeGLU (gelu_mul_fp16), and all three vectors land in the caller's scratch buffers.
+struct SharedGateUpArgs {
+    const uint8_t *gW, *gS, *gB, *uW, *uS, *uB;
+    const half_t *x;
+    half_t *gate_out, *up_out, *act_out;
+    uint32_t f;
+    int d;
+};
 template <int RT, int NP, int SD>
-__global__ __launch_bounds__(256) void shared_gate_up_long_kernel(const uint8_t *gW, const uint8_t *gS, const uint8_t *gB,
-                                                                  const uint8_t *uW, const uint8_t *uS, const uint8_t *uB,
-                                                                  const half_t *x, half_t *gate_out, half_t *up_out,
-                                                                  half_t *act_out, uint32_t f, int d) {
-    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
-    __shared__ float xsum[XStage::kMaxK / 32];
+__device__ __forceinline__ void shared_gate_up_long_body(const SharedGateUpArgs &a, uint32_t block, u32x4 *xa, float *xsum) {
+    const uint8_t *gW = a.gW, *gS = a.gS, *gB = a.gB, *uW = a.uW, *uS = a.uS, *uB = a.uB;
+    const half_t *x = a.x;
+    half_t *gate_out = a.gate_out, *up_out = a.up_out, *act_out = a.act_out;
+    const uint32_t f = a.f;
+    const int d = a.d;
     const int lane = threadIdx.x & 63;
-    const uint32_t tile = uniform_u32((blockIdx.x * blockDim.x + threadIdx.x) >> 6);
+    const uint32_t tile = uniform_u32((block * blockDim.x + threadIdx.x) >> 6);
     const uint32_t row0 = tile * RT;
     const bool live = row0 < f;
     XStage stage;
@@ -373,6 +392,83 @@ __global__ __launch_bounds__(256) void shared_gate_up_long_kernel(const uint8_t 
             act_out[row0 + r] = (half_t)(gelu_tanh((float)g16) * (float)u16);
         }
     }
+}
+
+template <int RT, int NP, int SD>
+__global__ __launch_bounds__(256) void shared_gate_up_long_kernel(SharedGateUpArgs a) {
+    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
+    __shared__ float xsum[XStage::kMaxK / 32];
+    shared_gate_up_long_body<RT, NP, SD>(a, blockIdx.x, xa, xsum);
+}
+
+// ------------------------------------------------------------------------------------------------ two stages, one launch
+// The shared expert does not depend on the router or the routed experts (the reference commits it on a command buffer of its
+// own).  In a chain of launches on one stream it can ride along: its gate / up rows as extra blocks of the router launch, its
+// down rows as extra blocks of the routed phase 1, so that the decoder layer has two launches fewer and their work overlaps.
+// A block takes one role by its index; the arithmetic of either role is that of the stand-alone kernel.
+struct RouterArgs {
+    const uint8_t *W, *S, *B;
+    const half_t *hidden;
+    const uint16_t *eff;
+    float *logits;
+    uint32_t num_experts;
+    int d;
+};
+template <int RT, int NP, int SD>
+__global__ __launch_bounds__(256) void router_and_shared_gate_up_kernel(RouterArgs r, SharedGateUpArgs sh) {
+    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
+    __shared__ float xsum[XStage::kMaxK / 32];
+    __shared__ float partial[4];
+    if (blockIdx.x < r.num_experts) {
+        router_logits_block_body<0>(r.W, r.S, r.B, r.hidden, r.eff, r.logits, r.d, blockIdx.x, partial);
+        return;
+    }
+    shared_gate_up_long_body<RT, NP, SD>(sh, blockIdx.x - r.num_experts, xa, xsum);
+}
+
+// One RT-row tile of y = W x per wave (fp16 out): the row streamer of the GEMV entry points, one tile a wave.
+struct GemvTileArgs {
+    const uint8_t *W, *S, *B;
+    const half_t *x;
+    half_t *y;
+    uint32_t m;
+    int k;
+};
+template <int RT, int NP, int SD>
+__device__ __forceinline__ void gemv_tile_body(const GemvTileArgs &a, uint32_t block, u32x4 *xa, float *xsum) {
+    const int lane = threadIdx.x & 63;
+    const uint32_t tile = uniform_u32((block * blockDim.x + threadIdx.x) >> 6);
+    const uint32_t row0 = tile * RT;
+    const bool live = row0 < a.m;
+    XStage stage;
+    stage.request(a.x, a.k);
+    RowStream<RT, NP> rs;
+    typename RowStream<RT, NP>::Tile t;
+    rs.init_map(a.k, lane);
+    if (live) rs.load(t, a.W + (size_t)row0 * (a.k >> 1), a.S + (size_t)row0 * (a.k >> 6) * 2, a.B + (size_t)row0 * (a.k >> 6) * 2, a.m - row0);
+    stage.publish(a.k, xa, xsum);
+    if (!live) return;
+    rs.init_x_lds(xa, xsum, a.k);
+    float out[RT];
+    rs.template reduce<SD>(t, out);
+    if (lane == 0) {
+#pragma unroll
+        for (int r = 0; r < RT; ++r)
+            if (row0 + r < a.m) a.y[row0 + r] = (half_t)out[r];
+    }
+}
+template <int RT, int NP, int SD>
+__global__ __launch_bounds__(256) void phase1_and_shared_down_kernel(RoutedArg routed, tf_expert_offsets off, const half_t *x, half_t *acts,
+                                                                     Phase1Geom g, FusedSelect fs, uint32_t moe_blocks, GemvTileArgs down) {
+    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
+    __shared__ float xsum[XStage::kMaxK / 32];
+    __shared__ uint32_t chosen[TF_MAX_STREAMED_EXPERTS];
+    __shared__ RankSelectLds sel;
+    if (blockIdx.x < moe_blocks) {
+        phase1_long_body<RT, NP, SD, true>(routed, off, x, acts, g, fs, blockIdx.x, xa, xsum, chosen, sel);
+        return;
+    }
+    gemv_tile_body<RT, NP, SD>(down, blockIdx.x - moe_blocks, xa, xsum);
 }
 
 bool routed_to_arg(const tf_routed_blobs *routed, uint32_t top_k, RoutedArg &arg, bool &all16) {
@@ -407,7 +503,9 @@ bool offsets_even(const tf_expert_offsets &o) {
 // kernel from fused->logits; returns TF_ERR_UNAVAILABLE when the operands do not allow the fused kernel.
 int32_t phase1_entry(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *routed, const tf_expert_offsets *off, const void *x,
                      void *acts, const uint32_t *active_slots, uint32_t active_count, bool subset, uint32_t d, uint32_t f,
-                     uint32_t top_k, tf_dtype sd, const FusedSelect *fused = nullptr, int mark_event = -1) {
+                     uint32_t top_k, tf_dtype sd, const FusedSelect *fused = nullptr, int mark_event = -1,
+                     const GemvTileArgs *ride = nullptr, bool *ride_taken = nullptr) {
+    if (ride_taken) *ride_taken = false;
     TF_REQUIRE(ctx, ctx && routed && off && x && acts, TF_ERR_INVALID_ARGUMENT, "moe_phase1: null argument");
     TF_REQUIRE(ctx, top_k == TF_MAX_STREAMED_EXPERTS, TF_ERR_INVALID_ARGUMENT, "moe_phase1: topK must be 8, got %u", top_k);
     TF_REQUIRE(ctx, d > 0 && d % TF_GROUP_SIZE == 0 && f > 0, TF_ERR_INVALID_ARGUMENT, "moe_phase1: d must be a multiple of 64 and f positive");
@@ -442,6 +540,15 @@ int32_t phase1_entry(tf_ctx *ctx, tf_stream stream, const tf_routed_blobs *route
         const uint32_t units = n_slots * ((f + plan.rt - 1) / plan.rt);
         const dim3 grid((units + 3) / 4);
         if (fused && mark_event >= 0 && ctx->step_timing) (void)hipEventRecord(ctx->step_events[mark_event], st);
+        // the shared expert's down rows ride along as extra blocks when both row widths take the same tile shape
+        if (fused && ride && plan.rt == 2 && plan.np == 3) {
+            const uint32_t down_blocks = ((ride->m + 1) / 2 + 3) / 4;
+            const dim3 both(grid.x + down_blocks);
+            if (SD == 0) hipLaunchKernelGGL((phase1_and_shared_down_kernel<2, 3, 0>), both, dim3(256), 0, st, arg, *off, xh, ah, g, *fused, grid.x, *ride);
+            else hipLaunchKernelGGL((phase1_and_shared_down_kernel<2, 3, 1>), both, dim3(256), 0, st, arg, *off, xh, ah, g, *fused, grid.x, *ride);
+            if (ride_taken) *ride_taken = true;
+            return check_launch(ctx, "moe_phase1_long + shared down");
+        }
 #define TF_P1_LAUNCH(RT_, NP_, SD_)                                                                                  \
     do {                                                                                                             \
         if (fused) hipLaunchKernelGGL((phase1_long_kernel<RT_, NP_, SD_, true>), grid, dim3(256), 0, st, arg, *off, xh, ah, g, *fused); \
@@ -683,7 +790,9 @@ int32_t router_logits_entry(tf_ctx *ctx, tf_stream stream, const void *weights, 
                             uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *hidden,
                             const void *effective_scale, uint64_t effective_scale_offset, const void *per_expert_scale,
                             uint64_t per_expert_scale_offset, void *out_indices, void *out_weights, uint32_t num_experts,
-                            uint32_t d, uint32_t top_k, float *logits) {
+                            uint32_t d, uint32_t top_k, float *logits, const SharedGateUpArgs *ride = nullptr, int ride_sd = 0,
+                            bool *ride_taken = nullptr) {
+    if (ride_taken) *ride_taken = false;
     TF_REQUIRE(ctx, ctx && weights && scales && biases && hidden && effective_scale && per_expert_scale && out_indices && out_weights,
                TF_ERR_INVALID_ARGUMENT, "router_gemma4: null argument");
     TF_REQUIRE(ctx, d > 0 && d % TF_GROUP_SIZE == 0, TF_ERR_INVALID_ARGUMENT, "router_gemma4: d must be a multiple of 64, got %u", d);
@@ -700,6 +809,15 @@ int32_t router_logits_entry(tf_ctx *ctx, tf_stream stream, const void *weights, 
     const bool fast = aligned16(w) && aligned16(hidden) && aligned16(eff) && d <= 4096;
     const int npass = fast ? (int)((d / 16 + 63) / 64) : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    if (fast && ride) {
+        // the shared expert's gate / up rows as extra blocks of this launch (two-row tiles of three passes: the caller checked)
+        const RouterArgs ra = {w, s, b, static_cast<const half_t *>(hidden), reinterpret_cast<const uint16_t *>(eff), logits, num_experts, (int)d};
+        const uint32_t shared_blocks = ((ride->f + 1) / 2 + 3) / 4;
+        if (ride_sd == 0) hipLaunchKernelGGL((router_and_shared_gate_up_kernel<2, 3, 0>), dim3(num_experts + shared_blocks), dim3(256), 0, st, ra, *ride);
+        else hipLaunchKernelGGL((router_and_shared_gate_up_kernel<2, 3, 1>), dim3(num_experts + shared_blocks), dim3(256), 0, st, ra, *ride);
+        if (ride_taken) *ride_taken = true;
+        return check_launch(ctx, "router_gemma4 logits + shared gate/up");
+    }
     if (fast) {
         hipLaunchKernelGGL((router_logits_block_kernel<0>), dim3(num_experts), dim3(256), 0, st, w, s, b, static_cast<const half_t *>(hidden),
                            reinterpret_cast<const uint16_t *>(eff), logits, (int)d);
@@ -730,6 +848,12 @@ int32_t router_select_entry(tf_ctx *ctx, tf_stream stream, const void *per_exper
 }
 
 // router logits -> (selection + phase 1) -> phase 2 on one stream; `logits` is the num_experts-float scratch between the launches
+// The shared expert riding along with the decode step's launches (see router_and_shared_gate_up_kernel).
+struct SharedRide {
+    SharedGateUpArgs gate_up;
+    GemvTileArgs down;
+};
+
 int32_t decode_step_impl(tf_ctx *ctx, tf_stream stream, const void *router_weights, uint64_t router_weights_offset,
                            const void *router_scales, uint64_t router_scales_offset, const void *router_biases,
                            uint64_t router_biases_offset, const void *router_x, const void *effective_scale,
@@ -737,7 +861,7 @@ int32_t decode_step_impl(tf_ctx *ctx, tf_stream stream, const void *router_weigh
                            const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
                            const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
                            void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype, float *logits,
-                         bool may_time) {
+                         bool may_time, const SharedRide *ride = nullptr) {
     TF_REQUIRE(ctx, ctx && expert_pool && out_indices, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: null argument");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool timed = may_time && ctx->step_timing;
@@ -745,10 +869,19 @@ int32_t decode_step_impl(tf_ctx *ctx, tf_stream stream, const void *router_weigh
         if (timed) (void)hipEventRecord(ctx->step_events[i], st);
     };
     mark(0);
+    const int ride_sd = scale_dtype == TF_BF16 ? 0 : 1;
+    bool rode = false;
     int32_t rc = router_logits_entry(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset,
                                      router_biases, router_biases_offset, router_x, effective_scale, effective_scale_offset,
-                                     per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, d, top_k, logits);
+                                     per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, d, top_k, logits,
+                                     ride ? &ride->gate_up : nullptr, ride_sd, &rode);
     if (rc != TF_OK) return rc;
+    if (ride && !rode) {   // the router took another kernel: the shared expert's gate / up rows get their own launch
+        if (ride_sd == 0) hipLaunchKernelGGL((shared_gate_up_long_kernel<2, 3, 0>), dim3(((ride->gate_up.f + 1) / 2 + 3) / 4), dim3(256), 0, st, ride->gate_up);
+        else hipLaunchKernelGGL((shared_gate_up_long_kernel<2, 3, 1>), dim3(((ride->gate_up.f + 1) / 2 + 3) / 4), dim3(256), 0, st, ride->gate_up);
+        rc = check_launch(ctx, "shared_gate_up");
+        if (rc != TF_OK) return rc;
+    }
     tf_routed_blobs routed = {};
     routed.pool = expert_pool;
     routed.pool_stride = expert_pool_stride;
@@ -757,7 +890,14 @@ int32_t decode_step_impl(tf_ctx *ctx, tf_stream stream, const void *router_weigh
     // Three launches when the vector path applies: logits, phase 1 with the selection repeated by every wave, phase 2.
     const FusedSelect fused = {logits, reinterpret_cast<const uint16_t *>(at(per_expert_scale, per_expert_scale_offset)),
                                static_cast<uint32_t *>(out_indices), static_cast<half_t *>(out_weights), num_experts};
-    rc = phase1_entry(ctx, stream, &routed, routed_offsets, x, acts, nullptr, 0, false, d, f, top_k, scale_dtype, &fused, timed ? 1 : -1);
+    rode = false;
+    rc = phase1_entry(ctx, stream, &routed, routed_offsets, x, acts, nullptr, 0, false, d, f, top_k, scale_dtype, &fused, timed ? 1 : -1,
+                      ride ? &ride->down : nullptr, &rode);
+    if (ride && !rode && (rc == TF_OK || rc == TF_ERR_UNAVAILABLE)) {   // phase 1 took another kernel: the down rows get their own launch
+        const int32_t rc_down = launch_gemv4(ctx, st, ride->down.W, ride->down.S, ride->down.B, ride->down.x, ride->down.y, ride->down.m,
+                                             (uint32_t)ride->down.k, scale_dtype, TF_FP16);
+        if (rc_down != TF_OK) return rc_down;
+    }
     if (rc == TF_ERR_UNAVAILABLE) {
         rc = router_select_entry(ctx, stream, per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, top_k, logits);
         if (rc != TF_OK) return rc;
@@ -910,6 +1050,64 @@ int32_t tf_moe_decode_step_static(tf_ctx *ctx, tf_stream stream, const void *rou
                             out_indices, out_weights, d, f, top_k, scale_dtype, ctx->static_router_logits, false);
 }
 
+int32_t tf_moe_decode_step_shared(tf_ctx *ctx, tf_stream stream, const void *router_weights, uint64_t router_weights_offset,
+                                  const void *router_scales, uint64_t router_scales_offset, const void *router_biases,
+                                  uint64_t router_biases_offset, const void *router_x, const void *effective_scale,
+                                  uint64_t effective_scale_offset, const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                                  const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                  const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
+                                  void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype,
+                                  const void *shared_x, const tf_projection *shared_gate, const tf_projection *shared_up,
+                                  const tf_projection *shared_down, void *shared_y, void *shared_scratch_gate, void *shared_scratch_up,
+                                  void *shared_scratch_act) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "moe_decode_step_shared: null context");
+    TF_REQUIRE(ctx, shared_x && shared_gate && shared_up && shared_down && shared_y && shared_scratch_gate && shared_scratch_up && shared_scratch_act,
+               TF_ERR_INVALID_ARGUMENT, "moe_decode_step_shared: null shared-expert argument");
+    TF_REQUIRE(ctx, shared_gate->rows == shared_up->rows && shared_gate->cols == shared_up->cols && shared_down->rows == shared_gate->cols &&
+                   shared_down->cols == shared_gate->rows,
+               TF_ERR_DIMENSION_MISMATCH, "SharedExpert dimension mismatch: gate=(%u,%u) up=(%u,%u) down=(%u,%u)", shared_gate->rows,
+               shared_gate->cols, shared_up->rows, shared_up->cols, shared_down->rows, shared_down->cols);
+    const uint32_t sf = shared_gate->rows, sdim = shared_gate->cols;
+    const tf_projection *proj[3] = {shared_gate, shared_up, shared_down};
+    bool proj_ok = true, proj16 = true;
+    for (int i = 0; i < 3; ++i) {
+        proj_ok = proj_ok && projection_ok(proj[i]) && proj[i]->rows > 0 && aligned(at(proj[i]->weights, proj[i]->weights_offset), 2);
+        proj16 = proj16 && proj_ok && aligned16(at(proj[i]->weights, proj[i]->weights_offset));
+    }
+    TF_REQUIRE(ctx, proj_ok, TF_ERR_INVALID_ARGUMENT,
+               "moe_decode_step_shared: a projection needs its three buffers, 2-byte aligned, and N a positive multiple of 64");
+    TF_REQUIRE(ctx, scale_dtype == TF_BF16 || scale_dtype == TF_FP16, TF_ERR_INVALID_ARGUMENT, "moe_decode_step_shared: scale dtype must be bf16 or fp16");
+    // the shared expert rides along when its row widths take the row streamers' two-row tiles of three passes (the production
+    // widths 2816 and 2112 do) and its operands the vector path; otherwise it runs first, as its own launches, same results
+    const LongPlan plan_up = plan_long_rows((int)sdim), plan_down = plan_long_rows((int)sf);
+    const bool ride_ok = proj16 && aligned16(shared_x) && aligned16(shared_scratch_act) && aligned(shared_scratch_gate, 2) && aligned(shared_scratch_up, 2) &&
+                         aligned(shared_y, 2) && sdim > 1024 && sdim <= (uint32_t)XStage::kMaxK && sf > 1024 && sf <= (uint32_t)XStage::kMaxK &&
+                         plan_up.rt == 2 && plan_up.np == 3 && plan_down.rt == 2 && plan_down.np == 3;
+    if (!ride_ok) {
+        const int32_t rc = tf_shared_expert_int4(ctx, stream, shared_x, 0, (uint64_t)sdim * 2, shared_gate, shared_up, shared_down, shared_y, 0,
+                                                 (uint64_t)sdim * 2, shared_scratch_gate, 0, (uint64_t)sf * 2, shared_scratch_up, 0, (uint64_t)sf * 2,
+                                                 shared_scratch_act, 0, (uint64_t)sf * 2, 4, scale_dtype);
+        if (rc != TF_OK) return rc;
+        return decode_step_impl(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset, router_biases,
+                                router_biases_offset, router_x, effective_scale, effective_scale_offset, per_expert_scale,
+                                per_expert_scale_offset, expert_pool, expert_pool_stride, num_experts, routed_offsets, x, acts, residual, y,
+                                out_indices, out_weights, d, f, top_k, scale_dtype, ctx->router_logits, true);
+    }
+    SharedRide ride;
+    ride.gate_up = {at(shared_gate->weights, shared_gate->weights_offset), at(shared_gate->scales, shared_gate->scales_offset),
+                    at(shared_gate->biases, shared_gate->biases_offset), at(shared_up->weights, shared_up->weights_offset),
+                    at(shared_up->scales, shared_up->scales_offset), at(shared_up->biases, shared_up->biases_offset),
+                    static_cast<const half_t *>(shared_x), static_cast<half_t *>(shared_scratch_gate), static_cast<half_t *>(shared_scratch_up),
+                    static_cast<half_t *>(shared_scratch_act), sf, (int)sdim};
+    ride.down = {at(shared_down->weights, shared_down->weights_offset), at(shared_down->scales, shared_down->scales_offset),
+                 at(shared_down->biases, shared_down->biases_offset), static_cast<const half_t *>(shared_scratch_act), static_cast<half_t *>(shared_y),
+                 shared_down->rows, (int)shared_down->cols};
+    return decode_step_impl(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset, router_biases,
+                            router_biases_offset, router_x, effective_scale, effective_scale_offset, per_expert_scale,
+                            per_expert_scale_offset, expert_pool, expert_pool_stride, num_experts, routed_offsets, x, acts, residual, y,
+                            out_indices, out_weights, d, f, top_k, scale_dtype, ctx->router_logits, true, &ride);
+}
+
 int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, uint64_t x_length,
                               const tf_projection *gate, const tf_projection *up, const tf_projection *down, void *y,
                               uint64_t y_offset, uint64_t y_length, void *scratch_gate, uint64_t scratch_gate_offset,
@@ -959,17 +1157,13 @@ int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream, const void *x, uint
         const uint8_t *gs = at(gate->scales, gate->scales_offset), *gb = at(gate->biases, gate->biases_offset);
         const uint8_t *us = at(up->scales, up->scales_offset), *ub = at(up->biases, up->biases_offset);
         bool launched = false;
+        const SharedGateUpArgs sga = {gw, gs, gb, uw, us, ub, reinterpret_cast<const half_t *>(xp), reinterpret_cast<half_t *>(sg),
+                                      reinterpret_cast<half_t *>(su), reinterpret_cast<half_t *>(sa), f, (int)d};
 #define TF_SH_CASE(RT_, NP_)                                                                                                    \
     if (!launched && plan.rt == RT_ && plan.np == NP_) {                                                                        \
         launched = true;                                                                                                        \
-        if (scale_dtype == TF_BF16)                                                                                             \
-            hipLaunchKernelGGL((shared_gate_up_long_kernel<RT_, NP_, 0>), grid, dim3(256), 0, st, gw, gs, gb, uw, us, ub,       \
-                               reinterpret_cast<const half_t *>(xp), reinterpret_cast<half_t *>(sg), reinterpret_cast<half_t *>(su), \
-                               reinterpret_cast<half_t *>(sa), f, (int)d);                                                      \
-        else                                                                                                                    \
-            hipLaunchKernelGGL((shared_gate_up_long_kernel<RT_, NP_, 1>), grid, dim3(256), 0, st, gw, gs, gb, uw, us, ub,       \
-                               reinterpret_cast<const half_t *>(xp), reinterpret_cast<half_t *>(sg), reinterpret_cast<half_t *>(su), \
-                               reinterpret_cast<half_t *>(sa), f, (int)d);                                                      \
+        if (scale_dtype == TF_BF16) hipLaunchKernelGGL((shared_gate_up_long_kernel<RT_, NP_, 0>), grid, dim3(256), 0, st, sga); \
+        else hipLaunchKernelGGL((shared_gate_up_long_kernel<RT_, NP_, 1>), grid, dim3(256), 0, st, sga);                        \
     }
         TF_SH_CASE(1, 1) TF_SH_CASE(1, 2) TF_SH_CASE(1, 3) TF_SH_CASE(1, 4)
         TF_SH_CASE(2, 1) TF_SH_CASE(2, 2) TF_SH_CASE(2, 3) TF_SH_CASE(2, 4)
