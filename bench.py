@@ -635,7 +635,7 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=Fal
                    + 2 * WINDOW * NKV * HD * 2)
     res = {"workload": "one token through one whole decoder layer (16q/8kv x 256, window 1024, shared 2112, 8 of 128 experts), 30 layers per graph replay",
            "us_per_layer": round(us, 2), "ms_per_30_layers": round(us * 30 / 1e3, 3), "algorithmic_bytes_per_layer": layer_bytes,
-           "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 13, "graph": "one in-order chain of launches"}
+           "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 10, "graph": "one in-order chain of launches"}
     if fork:
         res["us_per_layer_shared_expert_on_forked_branch"] = round(results["forked"][0], 2)
         res["forked_branch_note"] = ("the shared expert + its norm on a second captured stream (event fork after the post-attention setup, join "
