@@ -267,9 +267,8 @@ def check_against_oracle(r, T, d, f, top_k, abs_tol, rel_tol=1e-2):
 
 @pytest.mark.parametrize("M", [2, 4, 8, 12, 16, 24])
 def test_small_m_resident_pipeline_matches_oracle(M):
-    # BASELINE config 3: M tokens, top-8 over the production expert shape; below three pairs per expert on average (M = 2, 4,
-    # 8 here) every chunk takes the quad kernels, at M = 12 short chunks take them and long ones the matrix-core tiles, from
-    # four pairs per expert on the matrix-core tiles serve the call alone
+    # BASELINE config 3: M tokens, top-8 over the production expert shape; below four pairs per expert on average (M = 2, 4,
+    # 8, 12 here) the quad kernels serve the call, from there on the matrix-core tiles
     E, d, f, top_k = 32, 2816, 704, 8
     r = resident_pipeline(M, E, d, f, top_k, 0x300 + M)
     scale = float(np.max(np.abs(tfo.from_f16_bits(r["partials"]))))
@@ -297,8 +296,7 @@ def test_small_m_equals_decode_step_per_token():
                                      (5, 16, 64, 64)])
 def test_quad_kernels_long_chunks_and_row_widths(T, E, d, f):
     # Zipf-skewed routing with few pairs per expert on average: some chunks are longer than the quad kernels' LDS image and go
-    # through in batches (first case) or to the matrix-core tiles of the same call (3 pairs per expert); rows of one pass, of a
-    # partly filled last pass and of the widest supported rows
+    # through in batches; rows of one pass, of a partly filled last pass and of the widest supported rows
     top_k = 8
     r = resident_pipeline(T, E, d, f, top_k, 0x4400 + T, zipf=True, from_router=False)
     assert np.bincount(r["idx"].ravel(), minlength=E).max() > 8 or T <= 8
@@ -309,8 +307,8 @@ def test_quad_kernels_long_chunks_and_row_widths(T, E, d, f):
 @pytest.mark.parametrize("T", [6, 12, 24])
 def test_grouped_experts_fp16_scales_equal_bf16_scales(T):
     # the reference's expert blobs carry bf16 scales, and so does the oracle; the fp16 variant of the grouped kernels is pinned
-    # on pools whose scales hold the same values in either type: every partial must come out bit-identical (quad kernels alone,
-    # quad + matrix-core tiles, matrix-core tiles alone)
+    # on pools whose scales hold the same values in either type: every partial must come out bit-identical (quad kernels at 6
+    # and 12 tokens, matrix-core tiles at 24)
     E, d, f, top_k = 32, 2816, 704, 8
     a = resident_pipeline(T, E, d, f, top_k, 0x5500 + T, from_router=False, fp16_scales=True)
     blobs16 = a["blobs"]

@@ -728,7 +728,7 @@ __device__ __forceinline__ void quad_pass(const ChunkOperands &o, uint16_t s_bit
 
 template <int NPASS, int SD>
 __global__ __launch_bounds__(256, 2) void grouped_phase1_quad_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl, uint32_t n_chunks_upper,
-                                                                     bool take_all, const tf_prefill_pair *pairs, const half_t *hidden, long hidden_stride,
+                                                                     const tf_prefill_pair *pairs, const half_t *hidden, long hidden_stride,
                                                                      half_t *acts, uint32_t acts_pair_base, int d, int f) {
     constexpr int QC = 16, G = (int)kQuadMaxPairs / 4;
     typedef QuadMap<QC, NPASS> Map;
@@ -755,7 +755,6 @@ __global__ __launch_bounds__(256, 2) void grouped_phase1_quad_kernel(ExpertTable
     ch.expert = uniform_u32(ch.expert);
     ch.pair_start = uniform_u32(ch.pair_start);
     ch.pair_count = uniform_u32(ch.pair_count);
-    if (ch.pair_count > kQuadMaxPairs && !take_all) continue;
     const uint8_t *base = uniform_ptr(expert_base(tab, ch.expert));
     if (!base) continue;
     const rsrc_t blob = quad_blob_rsrc(base);
@@ -767,7 +766,7 @@ __global__ __launch_bounds__(256, 2) void grouped_phase1_quad_kernel(ExpertTable
         if (up) quad_request(t[p], qm, p, from, off.up_W_off + w_byte, off.up_s_off + sb_byte, off.up_b_off + sb_byte);
         else quad_request(t[p], qm, p, from, off.gate_W_off + w_byte, off.gate_s_off + sb_byte, off.gate_b_off + sb_byte);
     };
-    // a chunk longer than the LDS image (take_all only) goes through in batches, its weights once a batch
+    // a chunk longer than the LDS image goes through in batches, its weights once a batch
     for (uint32_t p0 = 0; p0 < ch.pair_count; p0 += kQuadMaxPairs) {
         const uint32_t nb = min(kQuadMaxPairs, ch.pair_count - p0), first = ch.pair_start + p0;
         const int groups_of_pairs = (int)((nb + 3) >> 2);
@@ -828,7 +827,7 @@ __global__ __launch_bounds__(256, 2) void grouped_phase1_quad_kernel(ExpertTable
 
 // down rows for such chunks: rows of 22 pieces (f = 704): eight quads along the row, two groups of four rows a wave.
 template <int NPASS, int SD>
-__global__ __launch_bounds__(256, 4) void grouped_down_quad_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl, uint32_t n_chunks_upper, bool take_all,
+__global__ __launch_bounds__(256, 4) void grouped_down_quad_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl, uint32_t n_chunks_upper,
                                                                    const tf_prefill_pair *pairs, const half_t *acts, uint32_t acts_pair_base,
                                                                    half_t *route_partials, int d, int f, int top_k) {
     constexpr int QC = 8, G = (int)kQuadMaxPairs / 4;
@@ -855,7 +854,6 @@ __global__ __launch_bounds__(256, 4) void grouped_down_quad_kernel(ExpertTable t
     ch.expert = uniform_u32(ch.expert);
     ch.pair_start = uniform_u32(ch.pair_start);
     ch.pair_count = uniform_u32(ch.pair_count);
-    if (ch.pair_count > kQuadMaxPairs && !take_all) continue;
     const uint8_t *base = uniform_ptr(expert_base(tab, ch.expert));
     if (!base) continue;
     const rsrc_t blob = quad_blob_rsrc(base);
@@ -1081,54 +1079,42 @@ int32_t run_grouped(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const t
     const bool p1_fast = blobs16 && hidden16 && off.gate_W_off % 16 == 0 && off.up_W_off % 16 == 0;
     const bool dn_fast = blobs16 && acts16 && off.down_W_off % 16 == 0;
     int32_t rc;
-    // Chunks of at most kQuadMaxPairs pairs go to the quad kernels, larger ones to the matrix-core tile kernels; each family
-    // skips the other's chunks (the host does not know the chunk sizes of a device-made list).  With fewer than three pairs
-    // per expert on average the quad kernels serve the call alone (long chunks, if any, in batches: launching the tile
-    // kernels to find nothing to do costs more); from four pairs per expert on, so few chunks are short that the tile
-    // kernels alone are faster.
+    // Fewer than four pairs per expert on average: the quad kernels serve the call (chunks longer than their LDS image, if any,
+    // in batches).  From there on so few chunks are short that the matrix-core tile kernels are faster (64 tokens: 193 us
+    // either way; 80 - 128 tokens: 198 - 200 us on the tiles against 224 - 281 us; running both families in one call, each on
+    // its chunks, was never better than the better of the two).
     const int p1_passes = ((g.d >> 5) + 15) / 16, dn_passes = ((g.f >> 5) + 7) / 8;
     const bool quad_ok = p1_fast && dn_fast && acts16 && g.d <= kQuadMaxD && p1_passes <= 6 && g.f <= kQuadMaxF && dn_passes <= 4 && g.d % 8 == 0 &&
                          g.f % 4 == 0 && aligned(g.route_partials, 8) && aligned(g.acts, 8) && tab.pool != nullptr;
-    const bool quad_alone = !use_mfma || (stream_pairs != 0 && (uint64_t)stream_pairs < (uint64_t)tab.num_experts * 3);
-    const bool quad_pays = quad_alone || (stream_pairs != 0 && (uint64_t)stream_pairs < (uint64_t)tab.num_experts * 4);
+    const bool quad_pays = !use_mfma || (stream_pairs != 0 && (uint64_t)stream_pairs < (uint64_t)tab.num_experts * 4);
     if (quad_ok && quad_pays) {
-        use_mfma = !quad_alone;
-        const bool take_all = quad_alone;
         // as many blocks as the compute units hold at once: two of the gate / up kernel, four of the down kernel
         const dim3 grid(2u * (uint32_t)ctx->num_cus), grid_down(4u * (uint32_t)ctx->num_cus);
 #define TF_GP1Q(NP_)                                                                                                       \
     if (p1_passes == NP_) {                                                                                                \
         if (sd == TF_BF16)                                                                                                 \
-            hipLaunchKernelGGL((grouped_phase1_quad_kernel<NP_, 0>), grid, dim3(256), 0, st, tab, off, cl, n_chunks_upper, take_all, g.pairs, g.hidden,        \
+            hipLaunchKernelGGL((grouped_phase1_quad_kernel<NP_, 0>), grid, dim3(256), 0, st, tab, off, cl, n_chunks_upper, g.pairs, g.hidden,        \
                                g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f);                                       \
         else                                                                                                               \
-            hipLaunchKernelGGL((grouped_phase1_quad_kernel<NP_, 1>), grid, dim3(256), 0, st, tab, off, cl, n_chunks_upper, take_all, g.pairs, g.hidden,        \
+            hipLaunchKernelGGL((grouped_phase1_quad_kernel<NP_, 1>), grid, dim3(256), 0, st, tab, off, cl, n_chunks_upper, g.pairs, g.hidden,        \
                                g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f);                                       \
     }
         TF_GP1Q(1) TF_GP1Q(2) TF_GP1Q(3) TF_GP1Q(4) TF_GP1Q(5) TF_GP1Q(6)
 #undef TF_GP1Q
         rc = check_launch(ctx, "grouped phase 1 quad");
         if (rc != TF_OK) return rc;
-        ChunkList big = cl;
-        big.min_pairs = kQuadMaxPairs + 1;
-        if (use_mfma) {
-            rc = launch_grouped_phase1_mfma(ctx, st, tab, off, big, n_chunks_upper, g.pairs, g.hidden, g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f, sd);
-            if (rc != TF_OK) return rc;
-        }
 #define TF_GDQ(NP_)                                                                                                        \
     if (dn_passes == NP_) {                                                                                                \
         if (sd == TF_BF16)                                                                                                 \
-            hipLaunchKernelGGL((grouped_down_quad_kernel<NP_, 0>), grid_down, dim3(256), 0, st, tab, off, cl, n_chunks_upper, take_all, g.pairs, g.acts,            \
+            hipLaunchKernelGGL((grouped_down_quad_kernel<NP_, 0>), grid_down, dim3(256), 0, st, tab, off, cl, n_chunks_upper, g.pairs, g.acts,            \
                                g.acts_pair_base, g.route_partials, g.d, g.f, g.top_k);                                     \
         else                                                                                                               \
-            hipLaunchKernelGGL((grouped_down_quad_kernel<NP_, 1>), grid_down, dim3(256), 0, st, tab, off, cl, n_chunks_upper, take_all, g.pairs, g.acts,            \
+            hipLaunchKernelGGL((grouped_down_quad_kernel<NP_, 1>), grid_down, dim3(256), 0, st, tab, off, cl, n_chunks_upper, g.pairs, g.acts,            \
                                g.acts_pair_base, g.route_partials, g.d, g.f, g.top_k);                                     \
     }
         TF_GDQ(1) TF_GDQ(2) TF_GDQ(3) TF_GDQ(4)
 #undef TF_GDQ
-        rc = check_launch(ctx, "grouped down quad");
-        if (rc != TF_OK || !use_mfma) return rc;
-        return launch_grouped_down_mfma(ctx, st, tab, off, big, n_chunks_upper, g.pairs, g.acts, g.acts_pair_base, g.route_partials, g.d, g.f, g.top_k, sd);
+        return check_launch(ctx, "grouped down quad");
     }
     // ---- phase 1
     if (use_mfma && p1_fast && acts16) {

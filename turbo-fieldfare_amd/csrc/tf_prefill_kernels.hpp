@@ -37,7 +37,6 @@ struct ChunkList {
     tf_prefill_group inline_chunks[kInlineChunks];
     const tf_prefill_group *dev;
     const uint32_t *dev_n;
-    uint32_t min_pairs;   // chunks with fewer pairs are left to another kernel of the same call (0: take every chunk)
 };
 
 __device__ __forceinline__ bool get_chunk(const ChunkList &cl, uint32_t i, tf_prefill_group &out) {
@@ -48,7 +47,7 @@ __device__ __forceinline__ bool get_chunk(const ChunkList &cl, uint32_t i, tf_pr
         if (i >= cl.n) return false;
         out = cl.inline_chunks[i];
     }
-    return out.pair_count >= cl.min_pairs;
+    return true;
 }
 
 }  // namespace tfk
