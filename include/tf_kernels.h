@@ -643,6 +643,32 @@ int32_t tf_prefill_grouped_routed_moe_resident(tf_ctx *ctx, tf_stream stream,
                                                const tf_expert_offsets *routed_offsets,
                                                void *acts_scratch, void *route_partials,
                                                uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype);
+/* tf_prefill_grouped_routed_moe_resident and tf_prefill_shared_expert_int4_block of the same token rows as one call
+ * (the reference encodes them back to back in one command buffer: the routed stages of PrefillGroupedRoutedMoE.swift:386-461,
+ * then PrefillSharedExpert.encodeBlock, PrefillSharedExpert.swift:12-67).  Neither reads what the other writes, so the
+ * shared expert's matrix-core tiles are placed ahead of the routed tiles in the same two launches (gate / up / GeGLU, then
+ * down) instead of under-filling the chip in launches of their own; results are bit-identical to the two calls.
+ * Applies when the routed pairs go to the matrix-core tile kernels and the shared expert is 4-bit with at least 8 rows and
+ * 16-byte aligned operands; otherwise the two calls are made one after the other.  Arguments: those of the routed call, then
+ * those of the shared call (its d is the routed d, its scale dtype the routed one; query_count token rows). */
+int32_t tf_prefill_grouped_routed_moe_resident_shared(tf_ctx *ctx, tf_stream stream,
+                                               const void *hidden, uint64_t hidden_offset, uint32_t hidden_stride_elements,
+                                               const void *sorted_pairs, const void *chunks, const void *chunk_count,
+                                               uint32_t max_chunks, uint32_t pair_count,
+                                               const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                               const tf_expert_offsets *routed_offsets,
+                                               void *acts_scratch, void *route_partials,
+                                               uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype,
+                                               const void *shared_x, uint64_t shared_x_offset,
+                                               void *shared_y, uint64_t shared_y_offset,
+                                               const tf_projection *shared_gate, const tf_projection *shared_up,
+                                               const tf_projection *shared_down,
+                                               void *scratch_gate, uint64_t scratch_gate_offset, uint64_t scratch_gate_length,
+                                               void *scratch_up, uint64_t scratch_up_offset, uint64_t scratch_up_length,
+                                               void *scratch_act, uint64_t scratch_act_offset, uint64_t scratch_act_length,
+                                               uint32_t query_count, uint32_t shared_intermediate,
+                                               uint32_t shared_x_stride_elements, uint32_t shared_y_stride_elements,
+                                               uint32_t shared_weight_bits);
 /* PrefillMoE.encodeReduceTokenMajor (Kernels/Prefill/MoE/PrefillMoE.swift:11-38) -> prefill_moe_reduce_token_major
  * (prefill.metal:575-596): h2[t, c] = half(sum_r float(w[t, r]) * float(partial[t, r, c])), r ascending, fused multiply-adds. */
 int32_t tf_prefill_moe_reduce_token_major(tf_ctx *ctx, tf_stream stream,

@@ -340,6 +340,64 @@ def test_grouped_gemm_on_matrix_cores_matches_oracle(T, E, d, f, zipf):
     check_against_oracle(r, T, d, f, top_k, abs_tol=2e-3 * max(1.0, scale))
 
 
+@pytest.mark.parametrize("T,E,d,f,shared_f,y_stride,bits", [
+    (64, 16, 2816, 704, 2112, 2816, 4),    # production row widths; routed tiles and shared tiles in the same two launches
+    (200, 16, 256, 192, 128, 264, 4),      # two row tiles of the shared expert, padded output rows
+    (1100, 8, 128, 64, 64, 128, 4),        # nine shared row tiles: the shared tiles numbered by XCD
+    (96, 8, 512, 128, 192, 515, 4),        # output rows that cannot leave as 16-byte pieces: the two calls one after the other
+    (6, 32, 2816, 704, 2112, 2816, 4),     # quad kernels serve the routed pairs: likewise
+    (64, 16, 512, 128, 192, 512, 8),       # 8-bit shared expert: likewise
+])
+def test_routed_and_shared_expert_in_one_call_equal_the_two_calls(T, E, d, f, shared_f, y_stride, bits):
+    top_k = 8
+    r = resident_pipeline(T, E, d, f, top_k, 0x6600 + T, zipf=True, from_router=False)
+    k = ctx()
+    n = T * top_k
+    g = device_grouping(r["idx"], r["w_bits"], T, top_k, E)
+    koff = tfk.ExpertOffsets(*r["off"].as_tuple())
+    d_pool, d_hidden = dev(r["pool"]), dev(r["hidden"])
+    if bits == 4:
+        mats = [refcases.synthetic_int4(shared_f, d, 0x77, "g"), refcases.synthetic_int4(shared_f, d, 0x77, "u"), refcases.synthetic_int4(d, shared_f, 0x77, "d")]
+    else:
+        mats = [refcases.synthetic_int8(shared_f, d, 0x78), refcases.synthetic_int8(shared_f, d, 0x79), refcases.synthetic_int8(d, shared_f, 0x7A)]
+    t = [[dev(a) for a in m] for m in mats]
+    gate, up, down = tfk.projection(*t[0], shared_f, d), tfk.projection(*t[1], shared_f, d), tfk.projection(*t[2], d, shared_f)
+    scratch = [zeros_bytes(shared_f * 2) for _ in range(3)]
+    sentinel = np.float16(-7.25).view(np.uint16)
+
+    def run(one_call):
+        acts, partials = zeros_bytes(n * f * 2), zeros_bytes(n * d * 2)
+        y = dev(np.full((T, y_stride), sentinel, np.uint16))
+        routed = (k.handle, None, d_hidden.data_ptr(), 0, d, g["sorted_pairs"].data_ptr(), g["chunks"].data_ptr(), g["n_chunks"].data_ptr(),
+                  g["cap"], n, d_pool.data_ptr(), r["stride"], E, C.byref(koff), acts.data_ptr(), partials.data_ptr(), d, f, top_k, tfk.TF_BF16)
+        shared_a = (d_hidden.data_ptr(), 0, y.data_ptr(), 0, C.byref(gate), C.byref(up), C.byref(down))
+        shared_s = tuple(v for s_ in scratch for v in (s_.data_ptr(), 0, shared_f * 2))
+        if one_call:
+            k.check(k.lib.tf_prefill_grouped_routed_moe_resident_shared(*routed, *shared_a, *shared_s, T, shared_f, d, y_stride, bits))
+        else:
+            k.check(k.lib.tf_prefill_grouped_routed_moe_resident(*routed))
+            k.check(k.lib.tf_prefill_shared_expert_int4_block(k.handle, None, *shared_a, *shared_s, T, d, shared_f, d, y_stride, bits, tfk.TF_BF16))
+        return host(partials, np.uint16, n * d), host(y, np.uint16, T * y_stride).reshape(T, y_stride)
+
+    want_partials, want_y = run(False)
+    got_partials, got_y = run(True)
+    assert np.array_equal(got_partials, want_partials)
+    assert np.array_equal(got_y, want_y)
+    assert np.all(got_y[:, d:] == sentinel) and not np.any(np.all(got_y[:, :d] == sentinel, axis=1))
+    # the separate calls are the ones the oracle checks
+    assert np.array_equal(want_partials, r["partials"])
+    # a refused shared expert launches nothing, the routed stages included
+    acts, partials = zeros_bytes(n * f * 2), zeros_bytes(n * d * 2)
+    y = zeros_bytes(T * y_stride * 2)
+    rc = k.lib.tf_prefill_grouped_routed_moe_resident_shared(
+        k.handle, None, d_hidden.data_ptr(), 0, d, g["sorted_pairs"].data_ptr(), g["chunks"].data_ptr(), g["n_chunks"].data_ptr(), g["cap"], n,
+        d_pool.data_ptr(), r["stride"], E, C.byref(koff), acts.data_ptr(), partials.data_ptr(), d, f, top_k, tfk.TF_BF16, d_hidden.data_ptr(), 0,
+        y.data_ptr(), 0, C.byref(gate), C.byref(up), C.byref(gate), *(v for s_ in scratch for v in (s_.data_ptr(), 0, shared_f * 2)), T, shared_f,
+        d, y_stride, bits)
+    assert rc == tfk.TF_ERR_DIMENSION_MISMATCH
+    assert not host(partials, np.uint16, n * d).any()
+
+
 def test_token_major_reduce_matches_cpu_reference():
     # PrefillMoETests.swift:11-44
     rows, top_k, d = 3, 8, 64

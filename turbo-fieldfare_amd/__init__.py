@@ -182,6 +182,11 @@ EXPORTS = {
                                                      C.POINTER(StreamedParams), vp, u32, i32, C.POINTER(i32), i32]),
     "tf_prefill_grouped_routed_moe_resident": (i32, [vp, vp, vp, u64, u32, vp, vp, vp, u32, u32, vp, u64, u32,
                                                      C.POINTER(ExpertOffsets), vp, vp, u32, u32, u32, i32]),
+    "tf_prefill_grouped_routed_moe_resident_shared": (i32, [vp, vp, vp, u64, u32, vp, vp, vp, u32, u32, vp, u64, u32,
+                                                            C.POINTER(ExpertOffsets), vp, vp, u32, u32, u32, i32,
+                                                            vp, u64, vp, u64, C.POINTER(Projection), C.POINTER(Projection),
+                                                            C.POINTER(Projection), vp, u64, u64, vp, u64, u64, vp, u64, u64,
+                                                            u32, u32, u32, u32, u32]),
     "tf_prefill_moe_reduce_token_major": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32, u32, u32]),
     "tf_int4_qmm": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, i32, i32, i32, i32]),
     "tf_prefill_int4_qmm": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, i32, i32, i32, i32]),

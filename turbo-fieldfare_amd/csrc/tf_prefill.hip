@@ -14,10 +14,17 @@ bool qmm_operands_ok(const void *w, const void *x, long ldx_halves, int k);
 int32_t launch_grouped_phase1_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off,
                                    const ChunkList &cl, uint32_t n_chunks_upper, const tf_prefill_pair *pairs,
                                    const half_t *hidden, long hidden_stride, half_t *acts, uint32_t acts_pair_base, int d, int f,
-                                   tf_dtype sd);
+                                   tf_dtype sd, const DenseRide *ride);
 int32_t launch_grouped_down_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off,
                                  const ChunkList &cl, uint32_t n_chunks_upper, const tf_prefill_pair *pairs, const half_t *acts,
-                                 uint32_t acts_pair_base, half_t *route_partials, int d, int f, int top_k, tf_dtype sd);
+                                 uint32_t acts_pair_base, half_t *route_partials, int d, int f, int top_k, tf_dtype sd, const DenseRide *ride);
+bool dense_ride_ok(const DenseRide &ride);
+int32_t shared_expert_block_plan(tf_ctx *ctx, const void *x, uint64_t x_offset, void *y, uint64_t y_offset, const tf_projection *gate,
+                                 const tf_projection *up, const tf_projection *down, void *scratch_gate, uint64_t scratch_gate_offset,
+                                 uint64_t scratch_gate_length, void *scratch_up, uint64_t scratch_up_offset, uint64_t scratch_up_length,
+                                 void *scratch_act, uint64_t scratch_act_offset, uint64_t scratch_act_length, uint32_t query_count,
+                                 uint32_t d, uint32_t intermediate, uint32_t x_stride_elements, uint32_t y_stride_elements,
+                                 uint32_t weight_bits, tf_dtype scale_dtype, DenseRide *plan);
 }  // namespace tfk
 
 namespace {
@@ -1068,10 +1075,12 @@ bool table_aligned(const ExpertTable &t) {
     return true;
 }
 
-// use_mfma: the chunks are large enough for the matrix cores to pay
+// use_mfma: the chunks are large enough for the matrix cores to pay.  ride: a shared expert's dense tiles to place ahead of the
+// grouped tiles when both stages run on the matrix-core tile kernels; *ride_taken says whether that happened.
 int32_t run_grouped(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off, const ChunkList &cl,
                     uint32_t n_chunks_upper, const GroupedGeom &g, tf_dtype sd, bool use_mfma, uint32_t stream_tokens = 0,
-                    uint32_t stream_pairs = 0) {
+                    uint32_t stream_pairs = 0, const DenseRide *ride = nullptr, bool *ride_taken = nullptr) {
+    if (ride_taken) *ride_taken = false;
     if (n_chunks_upper == 0) return TF_OK;
     const bool blobs16 = table_aligned(tab);
     const bool hidden16 = aligned16(g.hidden) && g.hidden_stride % 8 == 0;
@@ -1116,9 +1125,12 @@ int32_t run_grouped(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const t
 #undef TF_GDQ
         return check_launch(ctx, "grouped down quad");
     }
+    const bool p1_tiles = use_mfma && p1_fast && acts16, dn_tiles = use_mfma && dn_fast && aligned16(g.route_partials);
+    if (!(p1_tiles && dn_tiles) || (ride && !dense_ride_ok(*ride))) ride = nullptr;
+    if (ride && ride_taken) *ride_taken = true;
     // ---- phase 1
-    if (use_mfma && p1_fast && acts16) {
-        rc = launch_grouped_phase1_mfma(ctx, st, tab, off, cl, n_chunks_upper, g.pairs, g.hidden, g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f, sd);
+    if (p1_tiles) {
+        rc = launch_grouped_phase1_mfma(ctx, st, tab, off, cl, n_chunks_upper, g.pairs, g.hidden, g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f, sd, ride);
     } else {
         const LongPlan plan = plan_long_rows(g.d);
         bool launched = false;
@@ -1167,8 +1179,8 @@ int32_t run_grouped(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const t
     }
     if (rc != TF_OK) return rc;
     // ---- down
-    if (use_mfma && dn_fast && aligned16(g.route_partials)) {
-        return launch_grouped_down_mfma(ctx, st, tab, off, cl, n_chunks_upper, g.pairs, g.acts, g.acts_pair_base, g.route_partials, g.d, g.f, g.top_k, sd);
+    if (dn_tiles) {
+        return launch_grouped_down_mfma(ctx, st, tab, off, cl, n_chunks_upper, g.pairs, g.acts, g.acts_pair_base, g.route_partials, g.d, g.f, g.top_k, sd, ride);
     }
     if (dn_fast && g.f <= 1024) {
         constexpr int NPASS = 4;
@@ -1453,12 +1465,17 @@ int32_t tf_prefill_grouped_routed_moe_streamed(tf_ctx *ctx, tf_stream stream, co
     return TF_OK;
 }
 
-int32_t tf_prefill_grouped_routed_moe_resident(tf_ctx *ctx, tf_stream stream, const void *hidden, uint64_t hidden_offset,
-                                               uint32_t hidden_stride_elements, const void *sorted_pairs, const void *chunks,
-                                               const void *chunk_count, uint32_t max_chunks, uint32_t pair_count,
-                                               const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
-                                               const tf_expert_offsets *routed_offsets, void *acts_scratch, void *route_partials,
-                                               uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype) {
+}  // extern "C"
+
+namespace {
+
+int32_t grouped_resident_impl(tf_ctx *ctx, tf_stream stream, const void *hidden, uint64_t hidden_offset,
+                              uint32_t hidden_stride_elements, const void *sorted_pairs, const void *chunks,
+                              const void *chunk_count, uint32_t max_chunks, uint32_t pair_count,
+                              const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                              const tf_expert_offsets *routed_offsets, void *acts_scratch, void *route_partials,
+                              uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype, const DenseRide *ride, bool *ride_taken) {
+    if (ride_taken) *ride_taken = false;
     TF_REQUIRE(ctx, ctx && hidden && sorted_pairs && chunks && chunk_count && expert_pool && routed_offsets && acts_scratch && route_partials,
                TF_ERR_INVALID_ARGUMENT, "grouped_routed_moe_resident: null argument");
     TF_REQUIRE(ctx, d > 0 && d % TF_GROUP_SIZE == 0 && f > 0 && f % TF_GROUP_SIZE == 0 && top_k > 0 && num_experts > 0 &&
@@ -1481,7 +1498,56 @@ int32_t tf_prefill_grouped_routed_moe_resident(tf_ctx *ctx, tf_stream stream, co
     const bool use_mfma = (uint64_t)pair_count >= (uint64_t)num_experts * 2;
     // the pairs are all (token, rank) combinations of pair_count / top_k token rows
     const uint32_t tokens = pair_count % top_k == 0 ? pair_count / top_k : 0u;
-    return run_grouped(ctx, static_cast<hipStream_t>(stream), tab, *routed_offsets, cl, max_chunks, g, scale_dtype, use_mfma, tokens, pair_count);
+    return run_grouped(ctx, static_cast<hipStream_t>(stream), tab, *routed_offsets, cl, max_chunks, g, scale_dtype, use_mfma, tokens, pair_count,
+                       ride, ride_taken);
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t tf_prefill_grouped_routed_moe_resident(tf_ctx *ctx, tf_stream stream, const void *hidden, uint64_t hidden_offset,
+                                               uint32_t hidden_stride_elements, const void *sorted_pairs, const void *chunks,
+                                               const void *chunk_count, uint32_t max_chunks, uint32_t pair_count,
+                                               const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                               const tf_expert_offsets *routed_offsets, void *acts_scratch, void *route_partials,
+                                               uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype) {
+    return grouped_resident_impl(ctx, stream, hidden, hidden_offset, hidden_stride_elements, sorted_pairs, chunks, chunk_count, max_chunks,
+                                 pair_count, expert_pool, expert_pool_stride, num_experts, routed_offsets, acts_scratch, route_partials, d, f,
+                                 top_k, scale_dtype, nullptr, nullptr);
+}
+
+int32_t tf_prefill_grouped_routed_moe_resident_shared(tf_ctx *ctx, tf_stream stream, const void *hidden, uint64_t hidden_offset,
+                                                      uint32_t hidden_stride_elements, const void *sorted_pairs, const void *chunks,
+                                                      const void *chunk_count, uint32_t max_chunks, uint32_t pair_count,
+                                                      const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                                      const tf_expert_offsets *routed_offsets, void *acts_scratch, void *route_partials,
+                                                      uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype, const void *shared_x,
+                                                      uint64_t shared_x_offset, void *shared_y, uint64_t shared_y_offset,
+                                                      const tf_projection *shared_gate, const tf_projection *shared_up,
+                                                      const tf_projection *shared_down, void *scratch_gate, uint64_t scratch_gate_offset,
+                                                      uint64_t scratch_gate_length, void *scratch_up, uint64_t scratch_up_offset,
+                                                      uint64_t scratch_up_length, void *scratch_act, uint64_t scratch_act_offset,
+                                                      uint64_t scratch_act_length, uint32_t query_count, uint32_t shared_intermediate,
+                                                      uint32_t shared_x_stride_elements, uint32_t shared_y_stride_elements,
+                                                      uint32_t shared_weight_bits) {
+    // both calls' argument checks first, so that a refused call has launched nothing
+    DenseRide ride;
+    int32_t rc = shared_expert_block_plan(ctx, shared_x, shared_x_offset, shared_y, shared_y_offset, shared_gate, shared_up, shared_down,
+                                          scratch_gate, scratch_gate_offset, scratch_gate_length, scratch_up, scratch_up_offset, scratch_up_length,
+                                          scratch_act, scratch_act_offset, scratch_act_length, query_count, d, shared_intermediate,
+                                          shared_x_stride_elements, shared_y_stride_elements, shared_weight_bits, scale_dtype, &ride);
+    if (rc != TF_OK) return rc;
+    bool taken = false;
+    rc = grouped_resident_impl(ctx, stream, hidden, hidden_offset, hidden_stride_elements, sorted_pairs, chunks, chunk_count, max_chunks,
+                               pair_count, expert_pool, expert_pool_stride, num_experts, routed_offsets, acts_scratch, route_partials, d, f,
+                               top_k, scale_dtype, ride.rows > 0 ? &ride : nullptr, &taken);
+    if (rc != TF_OK || taken) return rc;
+    return tf_prefill_shared_expert_int4_block(ctx, stream, shared_x, shared_x_offset, shared_y, shared_y_offset, shared_gate, shared_up,
+                                               shared_down, scratch_gate, scratch_gate_offset, scratch_gate_length, scratch_up, scratch_up_offset,
+                                               scratch_up_length, scratch_act, scratch_act_offset, scratch_act_length, query_count, d,
+                                               shared_intermediate, shared_x_stride_elements, shared_y_stride_elements, shared_weight_bits,
+                                               scale_dtype);
 }
 
 int32_t tf_prefill_moe_reduce_token_major(tf_ctx *ctx, tf_stream stream, const void *route_partials, uint64_t route_partials_offset,

@@ -50,4 +50,16 @@ __device__ __forceinline__ bool get_chunk(const ChunkList &cl, uint32_t i, tf_pr
     return true;
 }
 
+// A shared expert's block of rows riding along in the launches of the grouped matrix-core kernels: its gate / up / GeGLU
+// tiles ahead of the grouped gate / up tiles, its down tiles ahead of the grouped down tiles.
+struct DenseRide {
+    const tf_projection *gate, *up, *down;
+    const half_t *x;      // [rows, gate->cols], row stride ldx halves
+    long ldx;
+    half_t *acts;         // [rows, gate->rows] activations between the two launches
+    half_t *y;            // [rows, down->rows], row stride ldy halves
+    long ldy;
+    int rows;
+};
+
 }  // namespace tfk

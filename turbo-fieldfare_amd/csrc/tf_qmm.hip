@@ -82,12 +82,11 @@ __host__ __device__ inline uint32_t dense_grid(uint32_t row_tiles, uint32_t col_
     if (row_tiles < kDenseXcds) return row_tiles * col_tiles;
     return kDenseXcds * ((row_tiles + kDenseXcds - 1) / kDenseXcds) * col_tiles;
 }
-__device__ __forceinline__ bool dense_tile(uint32_t row_tiles, uint32_t col_tiles, uint32_t &row_tile, uint32_t &col_tile) {
-    const uint32_t id = blockIdx.x;
+__device__ __forceinline__ bool dense_tile(uint32_t id, uint32_t row_tiles, uint32_t col_tiles, uint32_t &row_tile, uint32_t &col_tile) {
     if (row_tiles < kDenseXcds) {
         row_tile = id / col_tiles;
         col_tile = id - row_tile * col_tiles;
-        return true;
+        return row_tile < row_tiles;
     }
     const uint32_t xcd = id % kDenseXcds, j = id / kDenseXcds;
     row_tile = (j / col_tiles) * kDenseXcds + xcd;
@@ -95,13 +94,29 @@ __device__ __forceinline__ bool dense_tile(uint32_t row_tiles, uint32_t col_tile
     return row_tile < row_tiles;
 }
 
-template <int SD>
-__global__ __launch_bounds__(256, 2) void qmm_dense_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *X,
-                                                           long ldx, half_t *Y, long ldy, int M, int N, int K, bool rows_vectorizable) {
-    __shared__ __align__(128) uint8_t lds[block_lds_bytes<4, kQmmBN>()];
+// The four tile kernels are shells around `..._body` functions, so that a dense product can ride along in the launch of a
+// grouped one (a block takes one role or the other by its index).  `id`: the block's number within its own kind; `lds`: the
+// block's block_lds_bytes<4, columns>() of LDS, 128-byte aligned.
+struct DenseArgs {
+    const uint8_t *W, *S, *B;
+    const half_t *X;
+    long ldx;
+    half_t *Y;
+    long ldy;
+    int M, N, K;
+    bool rows_vectorizable;   // Y 16-byte aligned, N % 8 == 0, ldy % 8 == 0: whole 16-byte pieces of output rows
+};
+// VEC: a.rows_vectorizable holds and the tile leaves through LDS as row pieces
+template <int SD, bool VEC>
+__device__ __forceinline__ void qmm_dense_body(const DenseArgs &a, uint32_t id, uint8_t *lds) {
+    const uint8_t *W = a.W, *S = a.S, *B = a.B;
+    const half_t *X = a.X;
+    half_t *Y = a.Y;
+    const long ldx = a.ldx, ldy = a.ldy;
+    const int M = a.M, N = a.N, K = a.K;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint32_t row_tile, col_tile;
-    if (!dense_tile((uint32_t)(M + kQmmBM - 1) / kQmmBM, (uint32_t)(N + kQmmBN - 1) / kQmmBN, row_tile, col_tile)) return;
+    if (!dense_tile(id, (uint32_t)(M + kQmmBM - 1) / kQmmBM, (uint32_t)(N + kQmmBN - 1) / kQmmBN, row_tile, col_tile)) return;
     const int n0 = (int)col_tile * kQmmBN + wave * kQmmWaveN, m0 = (int)row_tile * kQmmBM;
     QmmARows<4> arow;
     arow.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(X), 0, (int)0xFFFFFFFFu, 0x00020000);
@@ -114,7 +129,7 @@ __global__ __launch_bounds__(256, 2) void qmm_dense_kernel(const uint8_t *W, con
     float16_t acc[4][2];
     zero_acc(acc);
     qmm_k_loop<SD, 4>(K >> 6, arow, rows, (uint32_t)(uintptr_t)lds, lane, row_tiles, acc);
-    if (rows_vectorizable) {
+    if constexpr (VEC) {
         __syncthreads();   // every wave has left the K loop and nothing it requested is still on its way into LDS
 #pragma unroll
         for (int j = 0; j < 2; ++j)
@@ -140,18 +155,34 @@ __global__ __launch_bounds__(256, 2) void qmm_dense_kernel(const uint8_t *W, con
     }
 }
 
+template <int SD, bool VEC>
+__global__ __launch_bounds__(256, 2) void qmm_dense_kernel(DenseArgs a) {
+    __shared__ __align__(128) uint8_t lds[block_lds_bytes<4, kQmmBN>()];
+    qmm_dense_body<SD, VEC>(a, blockIdx.x, lds);
+}
+
 // Shared-expert gate and up projections of a block of rows in one pass: a wave's first column tile is 32 rows of the gate
 // matrix, its second the same 32 rows of the up matrix.  Both sums are rounded to fp16 before GeGLU, the stage boundary of
 // the reference's chain (two GEMVs writing fp16, then gelu_mul_fp16: SharedExpertInt4.swift:60-84).
 constexpr int kGegluBN = 32 * 4;
+struct DenseGegluArgs {
+    const uint8_t *gW, *gS, *gB, *uW, *uS, *uB;
+    const half_t *X;
+    long ldx;
+    half_t *A;
+    long lda;
+    int M, F, K;
+};
 template <int SD>
-__global__ __launch_bounds__(256, 2) void qmm_dense_geglu_kernel(const uint8_t *gW, const uint8_t *gS, const uint8_t *gB, const uint8_t *uW,
-                                                                 const uint8_t *uS, const uint8_t *uB, const half_t *X, long ldx,
-                                                                 half_t *A, long lda, int M, int F, int K) {
-    __shared__ __align__(128) uint8_t lds[block_lds_bytes<4, kGegluBN>()];
+__device__ __forceinline__ void qmm_dense_geglu_body(const DenseGegluArgs &a, uint32_t id, uint8_t *lds) {
+    const uint8_t *gW = a.gW, *gS = a.gS, *gB = a.gB, *uW = a.uW, *uS = a.uS, *uB = a.uB;
+    const half_t *X = a.X;
+    half_t *A = a.A;
+    const long ldx = a.ldx, lda = a.lda;
+    const int M = a.M, F = a.F, K = a.K;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint32_t row_tile, col_tile;
-    if (!dense_tile((uint32_t)(M + kQmmBM - 1) / kQmmBM, (uint32_t)(F + kGegluBN - 1) / kGegluBN, row_tile, col_tile)) return;
+    if (!dense_tile(id, (uint32_t)(M + kQmmBM - 1) / kQmmBM, (uint32_t)(F + kGegluBN - 1) / kGegluBN, row_tile, col_tile)) return;
     const int n0 = (int)col_tile * kGegluBN + wave * 32, m0 = (int)row_tile * kQmmBM;
     QmmARows<4> arow;
     arow.rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t *>(X), 0, (int)0xFFFFFFFFu, 0x00020000);
@@ -178,13 +209,18 @@ __global__ __launch_bounds__(256, 2) void qmm_dense_geglu_kernel(const uint8_t *
     out_tile_store<kGegluBN>(lds, min(kQmmBM, M - m0), min(kGegluBN, F - nb), [&](int row) { return A + (size_t)(m0 + row) * lda + nb; });
 }
 
+template <int SD>
+__global__ __launch_bounds__(256, 2) void qmm_dense_geglu_kernel(DenseGegluArgs a) {
+    __shared__ __align__(128) uint8_t lds[block_lds_bytes<4, kGegluBN>()];
+    qmm_dense_geglu_body<SD>(a, blockIdx.x, lds);
+}
+
 // Block number -> (chunk, column tile) for the grouped kernels.  Workgroups go to the 8 XCDs round-robin by linear id and
 // each XCD has its own L2; the column tiles of one chunk all read the same activation rows, so they are given ids that
 // are congruent modulo 8: a run of 8 * tiles consecutive ids serves 8 chunks, one per XCD, and a chunk's activations are
 // fetched into one L2 once instead of into all eight.
 constexpr uint32_t kXcds = 8;
-__device__ __forceinline__ void chunk_and_tile(uint32_t tiles, uint32_t &chunk, uint32_t &tile) {
-    const uint32_t id = blockIdx.x;
+__device__ __forceinline__ void chunk_and_tile(uint32_t id, uint32_t tiles, uint32_t &chunk, uint32_t &tile) {
     const uint32_t run = kXcds * tiles;
     const uint32_t within = id % run;
     chunk = (id / run) * kXcds + within % kXcds;
@@ -201,15 +237,31 @@ constexpr int kGroupedWaves = 4;
 constexpr int kP1BN = 32 * kGroupedWaves;
 constexpr int kDownBN = QmmGeom<kGroupedWaves>::kBN;
 
+struct GroupedP1Args {
+    ExpertTable tab;
+    tf_expert_offsets off;
+    ChunkList cl;
+    const tf_prefill_pair *pairs;
+    const half_t *hidden;
+    long hidden_stride;
+    half_t *acts;
+    uint32_t acts_pair_base;
+    int D, F;
+};
 template <int SD>
-__global__ __launch_bounds__(64 * kGroupedWaves, 8 / kGroupedWaves) void grouped_phase1_mfma_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl,
-                                                                     const tf_prefill_pair *pairs, const half_t *hidden,
-                                                                     long hidden_stride, half_t *acts, uint32_t acts_pair_base,
-                                                                     int D, int F) {
-    __shared__ __align__(128) uint8_t lds[block_lds_bytes<kGroupedWaves, kP1BN>()];
+__device__ __forceinline__ void grouped_phase1_body(const GroupedP1Args &a, uint32_t id, uint8_t *lds) {
+    const ExpertTable &tab = a.tab;
+    const tf_expert_offsets &off = a.off;
+    const ChunkList &cl = a.cl;
+    const tf_prefill_pair *pairs = a.pairs;
+    const half_t *hidden = a.hidden;
+    const long hidden_stride = a.hidden_stride;
+    half_t *acts = a.acts;
+    const uint32_t acts_pair_base = a.acts_pair_base;
+    const int D = a.D, F = a.F;
     tf_prefill_group ch;
     uint32_t chunk_index, col_tile;
-    chunk_and_tile((uint32_t)(F + kP1BN - 1) / kP1BN, chunk_index, col_tile);
+    chunk_and_tile(id, (uint32_t)(F + kP1BN - 1) / kP1BN, chunk_index, col_tile);
     if (!get_chunk(cl, chunk_index, ch)) return;
     // everything taken from the work list is the same in all lanes: say so, the descriptors built from it live in
     // scalar registers
@@ -252,18 +304,49 @@ __global__ __launch_bounds__(64 * kGroupedWaves, 8 / kGroupedWaves) void grouped
     out_tile_store<kP1BN>(lds, (int)ch.pair_count, min(kP1BN, F - nb), [&](int row) { return tile + (size_t)row * F; });
 }
 
+template <int SD>
+__global__ __launch_bounds__(64 * kGroupedWaves, 8 / kGroupedWaves) void grouped_phase1_mfma_kernel(GroupedP1Args a) {
+    __shared__ __align__(128) uint8_t lds[block_lds_bytes<kGroupedWaves, kP1BN>()];
+    grouped_phase1_body<SD>(a, blockIdx.x, lds);
+}
+// the same launch with the dense gate / up / GeGLU tiles of a shared expert ahead of the grouped tiles: the blocks that start
+// first are the full-height ones, the grouped tiles of every height fill in behind them (0.461 -> 0.428 ms for the 2048-token
+// block against the dense tiles last)
+template <int SD>
+__global__ __launch_bounds__(64 * kGroupedWaves, 8 / kGroupedWaves) void grouped_phase1_and_dense_geglu_kernel(GroupedP1Args a, uint32_t dense_blocks,
+                                                                                                             DenseGegluArgs dense) {
+    static_assert(kP1BN == kGegluBN && kGroupedWaves == 4, "the two roles share one LDS layout");
+    __shared__ __align__(128) uint8_t lds[block_lds_bytes<kGroupedWaves, kP1BN>()];
+    if (blockIdx.x < dense_blocks) qmm_dense_geglu_body<SD>(dense, blockIdx.x, lds);
+    else grouped_phase1_body<SD>(a, blockIdx.x - dense_blocks, lds);
+}
+
 // ------------------------------------------------------------------------------------------------ grouped down
 // Block = one chunk x 64 NW output columns: X rows are the chunk's activation rows, Y rows scatter to
 // route_partials[(token * top_k + rank) * D + c].
+struct GroupedDownArgs {
+    ExpertTable tab;
+    tf_expert_offsets off;
+    ChunkList cl;
+    const tf_prefill_pair *pairs;
+    const half_t *acts;
+    uint32_t acts_pair_base;
+    half_t *route_partials;
+    int D, F, top_k;
+};
 template <int SD>
-__global__ __launch_bounds__(64 * kGroupedWaves, 8 / kGroupedWaves) void grouped_down_mfma_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl,
-                                                                   const tf_prefill_pair *pairs, const half_t *acts,
-                                                                   uint32_t acts_pair_base, half_t *route_partials, int D, int F,
-                                                                   int top_k) {
-    __shared__ __align__(128) uint8_t lds[block_lds_bytes<kGroupedWaves, kDownBN>()];
+__device__ __forceinline__ void grouped_down_body(const GroupedDownArgs &a, uint32_t id, uint8_t *lds) {
+    const ExpertTable &tab = a.tab;
+    const tf_expert_offsets &off = a.off;
+    const ChunkList &cl = a.cl;
+    const tf_prefill_pair *pairs = a.pairs;
+    const half_t *acts = a.acts;
+    const uint32_t acts_pair_base = a.acts_pair_base;
+    half_t *route_partials = a.route_partials;
+    const int D = a.D, F = a.F, top_k = a.top_k;
     tf_prefill_group ch;
     uint32_t chunk_index, col_tile;
-    chunk_and_tile((uint32_t)(D + kDownBN - 1) / kDownBN, chunk_index, col_tile);
+    chunk_and_tile(id, (uint32_t)(D + kDownBN - 1) / kDownBN, chunk_index, col_tile);
     if (!get_chunk(cl, chunk_index, ch)) return;
     // everything taken from the work list is the same in all lanes: say so, the descriptors built from it live in
     // scalar registers
@@ -307,6 +390,30 @@ __global__ __launch_bounds__(64 * kGroupedWaves, 8 / kGroupedWaves) void grouped
     const int nb = (int)col_tile * kDownBN;
     out_tile_store<kDownBN>(lds, (int)ch.pair_count, min(kDownBN, D - nb), [&](int row) { return route_partials + (size_t)row_slot[row] * D + nb; });
 }
+template <int SD>
+__global__ __launch_bounds__(64 * kGroupedWaves, 8 / kGroupedWaves) void grouped_down_mfma_kernel(GroupedDownArgs a) {
+    __shared__ __align__(128) uint8_t lds[block_lds_bytes<kGroupedWaves, kDownBN>()];
+    grouped_down_body<SD>(a, blockIdx.x, lds);
+}
+// the same launch with the tiles of a dense product (a shared expert's down projection; rows_vectorizable) ahead of the grouped tiles
+template <int SD>
+__global__ __launch_bounds__(64 * kGroupedWaves, 8 / kGroupedWaves) void grouped_down_and_dense_kernel(GroupedDownArgs a, uint32_t dense_blocks,
+                                                                                                     DenseArgs dense) {
+    static_assert(kDownBN == kQmmBN && kGroupedWaves == 4, "the two roles share one LDS layout");
+    __shared__ __align__(128) uint8_t lds[block_lds_bytes<kGroupedWaves, kDownBN>()];
+    if (blockIdx.x < dense_blocks) qmm_dense_body<SD, true>(dense, blockIdx.x, lds);
+    else grouped_down_body<SD>(a, blockIdx.x - dense_blocks, lds);
+}
+
+DenseArgs dense_args(const uint8_t *w, const uint8_t *s, const uint8_t *b, const half_t *x, long ldx, half_t *y, long ldy, int m, int n, int k) {
+    const bool rows_vec = aligned16(y) && n % 8 == 0 && ldy % 8 == 0;   // whole 16-byte pieces of output rows
+    return DenseArgs{w, s, b, x, ldx, y, ldy, m, n, k, rows_vec};
+}
+DenseGegluArgs dense_geglu_args(const tf_projection *gate, const tf_projection *up, const half_t *x, long ldx, half_t *a, long lda, int m) {
+    return DenseGegluArgs{at(gate->weights, gate->weights_offset), at(gate->scales, gate->scales_offset), at(gate->biases, gate->biases_offset),
+                          at(up->weights, up->weights_offset),     at(up->scales, up->scales_offset),     at(up->biases, up->biases_offset),
+                          x, ldx, a, lda, m, (int)gate->rows, (int)gate->cols};
+}
 
 }  // namespace
 
@@ -316,26 +423,47 @@ bool qmm_operands_ok(const void *w, const void *x, long ldx_halves, int k) {
     return aligned16(w) && aligned16(x) && (ldx_halves % 8 == 0) && k > 0 && (k % 64 == 0);
 }
 
+// a shared expert's tiles may ride in the grouped launches: its output rows leave as whole 16-byte pieces
+bool dense_ride_ok(const DenseRide &ride) {
+    return aligned16(ride.y) && ride.down->rows % 8 == 0 && ride.ldy % 8 == 0;
+}
+
 int32_t launch_grouped_phase1_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off,
                                    const ChunkList &cl, uint32_t n_chunks_upper, const tf_prefill_pair *pairs,
                                    const half_t *hidden, long hidden_stride, half_t *acts, uint32_t acts_pair_base, int d, int f,
-                                   tf_dtype sd) {
-    const dim3 grid((uint32_t)((f + kP1BN - 1) / kP1BN) * ((n_chunks_upper + kXcds - 1) / kXcds * kXcds));
-    if (sd == TF_BF16)
-        hipLaunchKernelGGL(grouped_phase1_mfma_kernel<0>, grid, dim3(64 * kGroupedWaves), 0, st, tab, off, cl, pairs, hidden, hidden_stride, acts, acts_pair_base, d, f);
-    else
-        hipLaunchKernelGGL(grouped_phase1_mfma_kernel<1>, grid, dim3(64 * kGroupedWaves), 0, st, tab, off, cl, pairs, hidden, hidden_stride, acts, acts_pair_base, d, f);
+                                   tf_dtype sd, const DenseRide *ride) {
+    const uint32_t grouped = (uint32_t)((f + kP1BN - 1) / kP1BN) * ((n_chunks_upper + kXcds - 1) / kXcds * kXcds);
+    const GroupedP1Args a = {tab, off, cl, pairs, hidden, hidden_stride, acts, acts_pair_base, d, f};
+    if (ride) {
+        // the shared expert's gate / up / GeGLU tiles ahead of the grouped tiles (the full-height, longest tiles first), padded
+        // to a multiple of 8 blocks so that both kinds keep their XCDs
+        const DenseGegluArgs dense = dense_geglu_args(ride->gate, ride->up, ride->x, ride->ldx, ride->acts, (long)ride->gate->rows, ride->rows);
+        const uint32_t extra = (dense_grid((uint32_t)(ride->rows + kQmmBM - 1) / kQmmBM, (uint32_t)((int)ride->gate->rows + kGegluBN - 1) / kGegluBN) + kXcds - 1) / kXcds * kXcds;
+        if (sd == TF_BF16) hipLaunchKernelGGL(grouped_phase1_and_dense_geglu_kernel<0>, dim3(grouped + extra), dim3(64 * kGroupedWaves), 0, st, a, extra, dense);
+        else hipLaunchKernelGGL(grouped_phase1_and_dense_geglu_kernel<1>, dim3(grouped + extra), dim3(64 * kGroupedWaves), 0, st, a, extra, dense);
+        return check_launch(ctx, "grouped_phase1_mfma + shared gate/up");
+    }
+    if (sd == TF_BF16) hipLaunchKernelGGL(grouped_phase1_mfma_kernel<0>, dim3(grouped), dim3(64 * kGroupedWaves), 0, st, a);
+    else hipLaunchKernelGGL(grouped_phase1_mfma_kernel<1>, dim3(grouped), dim3(64 * kGroupedWaves), 0, st, a);
     return check_launch(ctx, "grouped_phase1_mfma");
 }
 
 int32_t launch_grouped_down_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off,
                                  const ChunkList &cl, uint32_t n_chunks_upper, const tf_prefill_pair *pairs, const half_t *acts,
-                                 uint32_t acts_pair_base, half_t *route_partials, int d, int f, int top_k, tf_dtype sd) {
-    const dim3 grid((uint32_t)((d + kDownBN - 1) / kDownBN) * ((n_chunks_upper + kXcds - 1) / kXcds * kXcds));
-    if (sd == TF_BF16)
-        hipLaunchKernelGGL(grouped_down_mfma_kernel<0>, grid, dim3(64 * kGroupedWaves), 0, st, tab, off, cl, pairs, acts, acts_pair_base, route_partials, d, f, top_k);
-    else
-        hipLaunchKernelGGL(grouped_down_mfma_kernel<1>, grid, dim3(64 * kGroupedWaves), 0, st, tab, off, cl, pairs, acts, acts_pair_base, route_partials, d, f, top_k);
+                                 uint32_t acts_pair_base, half_t *route_partials, int d, int f, int top_k, tf_dtype sd, const DenseRide *ride) {
+    const uint32_t grouped = (uint32_t)((d + kDownBN - 1) / kDownBN) * ((n_chunks_upper + kXcds - 1) / kXcds * kXcds);
+    const GroupedDownArgs a = {tab, off, cl, pairs, acts, acts_pair_base, route_partials, d, f, top_k};
+    if (ride) {
+        const tf_projection *dn = ride->down;   // ride->y: 16-byte aligned rows of whole 16-byte pieces (dense_ride_ok)
+        const DenseArgs dense = dense_args(at(dn->weights, dn->weights_offset), at(dn->scales, dn->scales_offset), at(dn->biases, dn->biases_offset),
+                                           ride->acts, (long)dn->cols, ride->y, ride->ldy, ride->rows, (int)dn->rows, (int)dn->cols);
+        const uint32_t extra = (dense_grid((uint32_t)(ride->rows + kQmmBM - 1) / kQmmBM, (uint32_t)((int)dn->rows + kQmmBN - 1) / kQmmBN) + kXcds - 1) / kXcds * kXcds;
+        if (sd == TF_BF16) hipLaunchKernelGGL(grouped_down_and_dense_kernel<0>, dim3(grouped + extra), dim3(64 * kGroupedWaves), 0, st, a, extra, dense);
+        else hipLaunchKernelGGL(grouped_down_and_dense_kernel<1>, dim3(grouped + extra), dim3(64 * kGroupedWaves), 0, st, a, extra, dense);
+        return check_launch(ctx, "grouped_down_mfma + shared down");
+    }
+    if (sd == TF_BF16) hipLaunchKernelGGL(grouped_down_mfma_kernel<0>, dim3(grouped), dim3(64 * kGroupedWaves), 0, st, a);
+    else hipLaunchKernelGGL(grouped_down_mfma_kernel<1>, dim3(grouped), dim3(64 * kGroupedWaves), 0, st, a);
     return check_launch(ctx, "grouped_down_mfma");
 }
 
@@ -349,28 +477,28 @@ namespace {
 int32_t launch_qmm_dense(tf_ctx *ctx, hipStream_t st, const uint8_t *w, const uint8_t *s, const uint8_t *b, const half_t *x, long ldx,
                          half_t *y, long ldy, int m, int n, int k, tf_dtype sd) {
     const dim3 grid(dense_grid((uint32_t)(m + kQmmBM - 1) / kQmmBM, (uint32_t)(n + kQmmBN - 1) / kQmmBN));
-    const bool rows_vec = aligned16(y) && n % 8 == 0 && ldy % 8 == 0;   // whole 16-byte pieces of output rows
-    if (sd == TF_BF16)
-        hipLaunchKernelGGL(qmm_dense_kernel<0>, grid, dim3(256), 0, st, w, s, b, x, ldx, y, ldy, m, n, k, rows_vec);
-    else
-        hipLaunchKernelGGL(qmm_dense_kernel<1>, grid, dim3(256), 0, st, w, s, b, x, ldx, y, ldy, m, n, k, rows_vec);
+    const DenseArgs a = dense_args(w, s, b, x, ldx, y, ldy, m, n, k);
+    if (a.rows_vectorizable) {
+        if (sd == TF_BF16) hipLaunchKernelGGL((qmm_dense_kernel<0, true>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((qmm_dense_kernel<1, true>), grid, dim3(256), 0, st, a);
+    } else {
+        if (sd == TF_BF16) hipLaunchKernelGGL((qmm_dense_kernel<0, false>), grid, dim3(256), 0, st, a);
+        else hipLaunchKernelGGL((qmm_dense_kernel<1, false>), grid, dim3(256), 0, st, a);
+    }
     return check_launch(ctx, "int4_qmm");
 }
 
 // A[m, f] = GeGLU(half(X . gate^T), half(X . up^T)); a 16-byte aligned, lda % 8 == 0, f % 8 == 0
 int32_t launch_qmm_dense_geglu(tf_ctx *ctx, hipStream_t st, const tf_projection *gate, const tf_projection *up, const half_t *x, long ldx,
-                               half_t *a, long lda, int m, tf_dtype sd) {
-    const int f = (int)gate->rows, k = (int)gate->cols;
+                               half_t *a_out, long lda, int m, tf_dtype sd) {
+    const int f = (int)gate->rows;
     // 2048 x 2112 makes 272 blocks for 256 CUs: the 16 CUs that get two set the time (79 us; a block alone takes 46 us).
     // 544 half-height blocks, which fill every CU twice, measured slower still (+8 us): a block's weight expansion costs
     // the same for 64 rows as for 128.
     const dim3 grid(dense_grid((uint32_t)(m + kQmmBM - 1) / kQmmBM, (uint32_t)(f + kGegluBN - 1) / kGegluBN));
-    const uint8_t *gw = at(gate->weights, gate->weights_offset), *gs = at(gate->scales, gate->scales_offset), *gb = at(gate->biases, gate->biases_offset);
-    const uint8_t *uw = at(up->weights, up->weights_offset), *us = at(up->scales, up->scales_offset), *ub = at(up->biases, up->biases_offset);
-    if (sd == TF_BF16)
-        hipLaunchKernelGGL(qmm_dense_geglu_kernel<0>, grid, dim3(256), 0, st, gw, gs, gb, uw, us, ub, x, ldx, a, lda, m, f, k);
-    else
-        hipLaunchKernelGGL(qmm_dense_geglu_kernel<1>, grid, dim3(256), 0, st, gw, gs, gb, uw, us, ub, x, ldx, a, lda, m, f, k);
+    const DenseGegluArgs a = dense_geglu_args(gate, up, x, ldx, a_out, lda, m);
+    if (sd == TF_BF16) hipLaunchKernelGGL(qmm_dense_geglu_kernel<0>, grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL(qmm_dense_geglu_kernel<1>, grid, dim3(256), 0, st, a);
     return check_launch(ctx, "prefill_shared_expert gate/up");
 }
 
@@ -549,13 +677,21 @@ int32_t tf_int4_qmm(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t
                             n, k, scale_dtype);
 }
 
-int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, void *y, uint64_t y_offset,
-                                            const tf_projection *gate, const tf_projection *up, const tf_projection *down,
-                                            void *scratch_gate, uint64_t scratch_gate_offset, uint64_t scratch_gate_length,
-                                            void *scratch_up, uint64_t scratch_up_offset, uint64_t scratch_up_length, void *scratch_act,
-                                            uint64_t scratch_act_offset, uint64_t scratch_act_length, uint32_t query_count, uint32_t d,
-                                            uint32_t intermediate, uint32_t x_stride_elements, uint32_t y_stride_elements,
-                                            uint32_t weight_bits, tf_dtype scale_dtype) {
+}  // extern "C"
+
+namespace {
+
+// tf_prefill_shared_expert_int4_block.  With `plan`: nothing is launched; the arguments are checked as ever and, where the
+// call would run the 4-bit matrix-core kernels, *plan describes them (plan->rows > 0) for a caller that places their tiles
+// in launches of its own; plan->rows == 0: the call takes another route and is to be made as usual.
+int32_t shared_expert_block_impl(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, void *y, uint64_t y_offset,
+                                 const tf_projection *gate, const tf_projection *up, const tf_projection *down,
+                                 void *scratch_gate, uint64_t scratch_gate_offset, uint64_t scratch_gate_length,
+                                 void *scratch_up, uint64_t scratch_up_offset, uint64_t scratch_up_length, void *scratch_act,
+                                 uint64_t scratch_act_offset, uint64_t scratch_act_length, uint32_t query_count, uint32_t d,
+                                 uint32_t intermediate, uint32_t x_stride_elements, uint32_t y_stride_elements,
+                                 uint32_t weight_bits, tf_dtype scale_dtype, DenseRide *plan) {
+    if (plan) plan->rows = 0;
     TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "prefill_shared_expert: null context");
     TF_REQUIRE(ctx, weight_bits == 4 || weight_bits == 8, TF_ERR_UNSUPPORTED_BITS, "SharedExpert unsupported weight bits: %u", weight_bits);
     TF_REQUIRE(ctx, x && y && gate && up && down && scratch_gate && scratch_up && scratch_act, TF_ERR_INVALID_ARGUMENT,
@@ -580,6 +716,7 @@ int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream, const
     const bool block_path = weight_bits == 4 && pointers && even && query_count >= kSharedBlockMinRows && (scale_dtype == TF_BF16 || scale_dtype == TF_FP16) &&
                             qmm_operands_ok(gw, xp, x_stride_elements, (int)d) && aligned16(uw) && aligned16(dw) &&
                             intermediate % TF_GROUP_SIZE == 0 && query_count <= (uint32_t)INT32_MAX;
+    if (plan && !block_path) return TF_OK;
     if (weight_bits == 8 && pointers && even && query_count >= 2) {
         // 8-bit projections.  Up to kShared8MfmaMinRows - 1 rows: rows in groups against each weight row, bit-identical to the
         // rows one by one.  From there on the matrix cores: every weight is rounded to fp16 as half(q s + b) first (the
@@ -619,10 +756,45 @@ int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream, const
     half_t *acts = nullptr;
     int32_t rc = shared_block_acts(ctx, (size_t)query_count * intermediate, acts);
     if (rc != TF_OK) return rc;
+    if (plan) {
+        *plan = DenseRide{gate, up, down, xp, (long)x_stride_elements, acts, yp, (long)y_stride_elements, (int)query_count};
+        return TF_OK;
+    }
     rc = launch_qmm_dense_geglu(ctx, st, gate, up, xp, (long)x_stride_elements, acts, (long)intermediate, (int)query_count, scale_dtype);
     if (rc != TF_OK) return rc;
     return launch_qmm_dense(ctx, st, dw, at(down->scales, down->scales_offset), at(down->biases, down->biases_offset), acts, (long)intermediate,
                             yp, (long)y_stride_elements, (int)query_count, (int)d, (int)intermediate, scale_dtype);
+}
+
+}  // namespace
+
+namespace tfk {
+
+int32_t shared_expert_block_plan(tf_ctx *ctx, const void *x, uint64_t x_offset, void *y, uint64_t y_offset, const tf_projection *gate,
+                                 const tf_projection *up, const tf_projection *down, void *scratch_gate, uint64_t scratch_gate_offset,
+                                 uint64_t scratch_gate_length, void *scratch_up, uint64_t scratch_up_offset, uint64_t scratch_up_length,
+                                 void *scratch_act, uint64_t scratch_act_offset, uint64_t scratch_act_length, uint32_t query_count,
+                                 uint32_t d, uint32_t intermediate, uint32_t x_stride_elements, uint32_t y_stride_elements,
+                                 uint32_t weight_bits, tf_dtype scale_dtype, DenseRide *plan) {
+    return shared_expert_block_impl(ctx, nullptr, x, x_offset, y, y_offset, gate, up, down, scratch_gate, scratch_gate_offset, scratch_gate_length,
+                                    scratch_up, scratch_up_offset, scratch_up_length, scratch_act, scratch_act_offset, scratch_act_length,
+                                    query_count, d, intermediate, x_stride_elements, y_stride_elements, weight_bits, scale_dtype, plan);
+}
+
+}  // namespace tfk
+
+extern "C" {
+
+int32_t tf_prefill_shared_expert_int4_block(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, void *y, uint64_t y_offset,
+                                            const tf_projection *gate, const tf_projection *up, const tf_projection *down,
+                                            void *scratch_gate, uint64_t scratch_gate_offset, uint64_t scratch_gate_length,
+                                            void *scratch_up, uint64_t scratch_up_offset, uint64_t scratch_up_length, void *scratch_act,
+                                            uint64_t scratch_act_offset, uint64_t scratch_act_length, uint32_t query_count, uint32_t d,
+                                            uint32_t intermediate, uint32_t x_stride_elements, uint32_t y_stride_elements,
+                                            uint32_t weight_bits, tf_dtype scale_dtype) {
+    return shared_expert_block_impl(ctx, stream, x, x_offset, y, y_offset, gate, up, down, scratch_gate, scratch_gate_offset, scratch_gate_length,
+                                    scratch_up, scratch_up_offset, scratch_up_length, scratch_act, scratch_act_offset, scratch_act_length,
+                                    query_count, d, intermediate, x_stride_elements, y_stride_elements, weight_bits, scale_dtype, nullptr);
 }
 
 }  // extern "C"
