@@ -519,9 +519,10 @@ def extras(torch, tfk, k, gen, lib, h, stream):
 
 def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=False):
     """One token through whole sliding-window decoder layers, every stage a call of the library and nothing on the host in
-    between: input norm + q/k/v projections in one launch (k, v straight into their cache row) -> per-head norm + RoPE ->
-    attention over a 1024-row window -> output projection -> post-attention setup -> router + 8 routed experts with the shared
-    expert riding along in the same three launches -> norm of the shared expert's output + layer tail in one launch.  The layers rotate over the resident expert pools and as many sets of dense weights; replayed from a HIP graph."""
+    between, eight launches a layer: [previous layer's tail + input norm + q/k/v projections, k and v straight into their cache
+    row] -> per-head norm + RoPE -> attention over a 1024-row window (two launches) -> output projection -> [post-attention
+    setup + router logits + shared gate / up] -> [top-8 + routed phase 1 + shared down] -> routed phase 2.  The layers rotate
+    over the resident expert pools and as many sets of dense weights; replayed from a HIP graph."""
     import ctypes as C
     HD, NQ, NKV, WINDOW = 256, 16, 8, 1024
     n_layers = len(layers)
@@ -549,66 +550,76 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=Fal
         w["proj"] = [tfk.projection(*w[n], r, c) for n, r, c in (("gate", F_SHARED, D), ("up", F_SHARED, D), ("down", D, F_SHARED))]
         dense.append(w)
     z = lambda n: torch.zeros(n, dtype=torch.float16, device="cuda")
-    b = dict(hidden=(torch.randn(D, device="cuda", generator=gen) * 0.5).to(torch.float16), x_norm=z(D), q=z(NQ * HD), attn=z(NQ * HD), o=z(D),
+    b = dict(hidden=(torch.randn(D, device="cuda", generator=gen) * 0.5).to(torch.float16), hidden_alt=z(D), x_norm=z(D), q=z(NQ * HD), attn=z(NQ * HD), o=z(D),
              dense_x=z(D), routed_x=z(D), router_x=z(D), shared=z(D), h1=z(D), h2=z(D), sg=z(F_SHARED), su=z(F_SHARED), sa=z(F_SHARED), zero=z(D),
              acts=z(TOPK * F_MOE), idx=torch.zeros(TOPK, dtype=torch.int32, device="cuda"), wts=z(TOPK))
     p = lambda name: b[name].data_ptr()
     position = WINDOW + 60
     kv_off = position * NKV * HD * 2
 
-    def layer_step(i, st, branch=None):
-        """One layer on stream handle `st`.  With `branch` (a torch stream) the shared expert and its norm run beside the router and
-        the routed experts, as the reference commits its shared-expert command buffer without waiting
-        (RealForwardRunner.swift:1570-1594); the branch forks after the post-attention setup and joins before the layer tail."""
+    def layer_step(i, st, branch=None, first=True, last=True):
+        """One layer on stream handle `st`; first / last: whether the sequence of layers begins / ends with this one.
+        The residual stream lives in two buffers: `hidden` (a layer's input) and `hidden_alt` (after the post-attention setup):
+        a stage folded into the prologue of every block of another launch cannot write over the row those blocks are reading.
+        The layer tail is folded into the NEXT layer's projection launch, so only the last layer of a sequence runs its own
+        (in place on `hidden_alt`, where the sequence's output is then found).
+        With `branch` (a torch stream) the stages are separate launches, in place on `hidden`, and the shared expert and its
+        norm run beside the router and the routed experts, as the reference commits its shared-expert command buffer without
+        waiting (RealForwardRunner.swift:1570-1594); the branch forks after the post-attention setup and joins before the tail."""
         w, (pool, r) = dense[i % n_layers], layers[i % n_layers]
+        prev = dense[(i - 1) % n_layers]
         ptr = lambda name: w[name].data_ptr()
         qkv = []
         for name in ("q", "k", "v"):
             qkv += [w[name][0].data_ptr(), 0, w[name][1].data_ptr(), 0, w[name][2].data_ptr(), 0]
-        # the input norm runs inside the projection launch
-        rc = lib.tf_fused_norm_qkv_gemv(h, st, ptr("input_norm"), 0, 1e-6, *qkv, p("hidden"), p("q"), 0, ptr("k_cache"), kv_off, ptr("v_cache"), kv_off,
-                                        NQ * HD, NKV * HD, D, tfk.TF_BF16)
+        qkv_out = (p("q"), 0, ptr("k_cache"), kv_off, ptr("v_cache"), kv_off, NQ * HD, NKV * HD, D, tfk.TF_BF16)
+        if first or branch is not None:
+            # the input norm runs inside the projection launch
+            rc = lib.tf_fused_norm_qkv_gemv(h, st, ptr("input_norm"), 0, 1e-6, *qkv, p("hidden"), *qkv_out)
+        else:
+            # ... and so does the previous layer's tail (with the norm of the shared expert's output)
+            rc = lib.tf_fused_layer_tail_norm_qkv_gemv(h, st, p("h2"), p("shared"), p("hidden_alt"), p("hidden"), prev["post_ffn1"].data_ptr(), 0,
+                                                       prev["post_ffn2"].data_ptr(), 0, prev["post_ffn"].data_ptr(), 0, 1e-6, 1.0,
+                                                       ptr("input_norm"), 0, 1e-6, *qkv, *qkv_out)
         rc |= lib.tf_fused_qkv_epilogue(h, st, p("q"), 0, ptr("k_cache"), kv_off, ptr("v_cache"), kv_off, ptr("q_norm"), 0, ptr("k_norm"), 0,
                                         HD, NQ, NKV, position, 1e4, HD // 2, 1e-6)
         rc |= lib.tf_attention_swa(h, st, p("q"), 0, ptr("k_cache"), 0, ptr("v_cache"), 0, p("attn"), 0, HD, NQ, NKV, position + 1, WINDOW, 1.0, 0)
         rc |= lib.tf_dequant_int4_gemv(h, st, w["o"][0].data_ptr(), 0, w["o"][1].data_ptr(), 0, w["o"][2].data_ptr(), 0, p("attn"), 0, p("o"), 0,
                                        D, NQ * HD, tfk.TF_BF16, tfk.TF_FP16)
-        rc |= lib.tf_fused_post_attn_setup(h, st, p("hidden"), p("o"), p("dense_x"), p("routed_x"), p("router_x"), ptr("post_attn"), 0,
-                                           ptr("pre_ffn"), 0, ptr("pre_ffn2"), 0, D, 1e-6)
         g, u, dn = w["proj"]
-        st_shared = st
-        if branch is not None:
+        step = (r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, p("router_x"), r["eff"].data_ptr(), 0, r["gain"].data_ptr(), 0,
+                pool.data_ptr(), stride, E, C.byref(off), p("routed_x"), p("acts"), p("zero"), p("h2"), p("idx"), p("wts"), D, F_MOE, TOPK, tfk.TF_BF16)
+        if branch is None:
+            # post-attention setup, router + routed experts and the shared expert in three launches: the setup in the prologue of the
+            # first, the shared expert's gate / up beside the router and its down beside phase 1
+            rc |= lib.tf_moe_decode_step_shared_post_attn(h, st, p("hidden"), p("o"), p("hidden_alt"), ptr("post_attn"), 0, ptr("pre_ffn"), 0,
+                                                          ptr("pre_ffn2"), 0, 1e-6, *step, p("dense_x"), C.byref(g), C.byref(u), C.byref(dn),
+                                                          p("shared"), p("sg"), p("su"), p("sa"))
+            if last:
+                rc |= lib.tf_fused_layer_tail_shared_norm(h, st, p("h2"), p("shared"), p("hidden_alt"), ptr("post_ffn1"), 0, ptr("post_ffn2"), 0,
+                                                          ptr("post_ffn"), 0, D, 1e-6, 1.0)
+        else:
+            rc |= lib.tf_fused_post_attn_setup(h, st, p("hidden"), p("o"), p("dense_x"), p("routed_x"), p("router_x"), ptr("post_attn"), 0,
+                                               ptr("pre_ffn"), 0, ptr("pre_ffn2"), 0, D, 1e-6)
             fork = torch.cuda.Event()
             fork.record(torch.cuda.current_stream())
             branch.wait_event(fork)
-            st_shared = branch.cuda_stream
-        if branch is None:
-            # the shared expert rides along with the launches of the routed step (gate / up beside the router, down beside phase 1)
-            rc |= lib.tf_moe_decode_step_shared(h, st, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, p("router_x"), r["eff"].data_ptr(), 0,
-                                                r["gain"].data_ptr(), 0, pool.data_ptr(), stride, E, C.byref(off), p("routed_x"), p("acts"), p("zero"), p("h2"),
-                                                p("idx"), p("wts"), D, F_MOE, TOPK, tfk.TF_BF16, p("dense_x"), C.byref(g), C.byref(u), C.byref(dn), p("shared"),
-                                                p("sg"), p("su"), p("sa"))
-        else:
-            rc |= lib.tf_shared_expert_int4(h, st_shared, p("dense_x"), 0, D * 2, C.byref(g), C.byref(u), C.byref(dn), p("shared"), 0, D * 2, p("sg"), 0,
-                                            F_SHARED * 2, p("su"), 0, F_SHARED * 2, p("sa"), 0, F_SHARED * 2, 4, tfk.TF_BF16)
-            rc |= lib.tf_moe_decode_step(h, st, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, p("router_x"), r["eff"].data_ptr(), 0,
-                                         r["gain"].data_ptr(), 0, pool.data_ptr(), stride, E, C.byref(off), p("routed_x"), p("acts"), p("zero"), p("h2"),
-                                         p("idx"), p("wts"), D, F_MOE, TOPK, tfk.TF_BF16)
-        if branch is not None:
+            rc |= lib.tf_shared_expert_int4(h, branch.cuda_stream, p("dense_x"), 0, D * 2, C.byref(g), C.byref(u), C.byref(dn), p("shared"), 0, D * 2,
+                                            p("sg"), 0, F_SHARED * 2, p("su"), 0, F_SHARED * 2, p("sa"), 0, F_SHARED * 2, 4, tfk.TF_BF16)
+            rc |= lib.tf_moe_decode_step(h, st, *step)
             join = torch.cuda.Event()
             join.record(branch)
             torch.cuda.current_stream().wait_event(join)
-        # the norm of the shared expert's output runs inside the tail launch
-        rc |= lib.tf_fused_layer_tail_shared_norm(h, st, p("h2"), p("shared"), p("hidden"), ptr("post_ffn1"), 0, ptr("post_ffn2"), 0, ptr("post_ffn"), 0,
-                                                  D, 1e-6, 1.0)
+            rc |= lib.tf_fused_layer_tail_shared_norm(h, st, p("h2"), p("shared"), p("hidden"), ptr("post_ffn1"), 0, ptr("post_ffn2"), 0, ptr("post_ffn"), 0,
+                                                      D, 1e-6, 1.0)
         if rc != 0:
             raise RuntimeError("layer chain failed: " + k.last_error())
 
     per_graph = 30                                          # the model has 30 layers: one replay = one token's layers
     st0 = torch.cuda.current_stream().cuda_stream
     start_hidden = b["hidden"].clone()
-    for i in range(2 * n_layers):
-        layer_step(i, st0)                                  # warm-up; also sizes every context-owned scratch before the capture
+    for i in range(2 * n_layers):                           # warm-up; also sizes every context-owned scratch before the capture
+        layer_step(i, st0, first=i == 0, last=i == 2 * n_layers - 1)
     b["hidden"].copy_(start_hidden)
     torch.cuda.synchronize()
     side, branch = torch.cuda.Stream(), torch.cuda.Stream()      # both at the default priority
@@ -621,11 +632,11 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=Fal
                 st = torch.cuda.current_stream().cuda_stream
                 b["hidden"].copy_(hidden0)                  # every replay is the same token: synthetic weights would otherwise drift it away
                 for i in range(per_graph):
-                    layer_step(i, st, br)
+                    layer_step(i, st, br, first=i == 0, last=i == per_graph - 1)
             g.replay()
             side.synchronize()
             rounds, _ = replay_rounds(torch, side, g.replay)
-            results[label] = (float(np.median(rounds)) * 1e3 / per_graph, b["hidden"].clone())
+            results[label] = (float(np.median(rounds)) * 1e3 / per_graph, b["hidden" if br is not None else "hidden_alt"].clone())
     us = results["serial"][0]
     if fork:
         assert torch.equal(results["forked"][1], results["serial"][1]), "forked and serial layer chains disagree"
@@ -635,7 +646,7 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=Fal
                    + 2 * WINDOW * NKV * HD * 2)
     res = {"workload": "one token through one whole decoder layer (16q/8kv x 256, window 1024, shared 2112, 8 of 128 experts), 30 layers per graph replay",
            "us_per_layer": round(us, 2), "ms_per_30_layers": round(us * 30 / 1e3, 3), "algorithmic_bytes_per_layer": layer_bytes,
-           "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 10, "graph": "one in-order chain of launches"}
+           "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 8, "graph": "one in-order chain of launches"}
     if fork:
         res["us_per_layer_shared_expert_on_forked_branch"] = round(results["forked"][0], 2)
         res["forked_branch_note"] = ("the shared expert + its norm on a second captured stream (event fork after the post-attention setup, join "

@@ -195,6 +195,29 @@ int32_t tf_fused_norm_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *norm_w
                                const void *v_biases, uint64_t v_biases_offset, const void *hidden, void *q_out, uint64_t q_out_offset,
                                void *k_out, uint64_t k_out_offset, void *v_out, uint64_t v_out_offset, uint32_t q_rows, uint32_t kv_rows,
                                uint32_t n, tf_dtype scale_dtype);
+/* tf_fused_layer_tail_shared_norm of one decoder layer followed by tf_fused_norm_qkv_gemv of the next as one call: the runner
+ * encodes the layers back to back (RealForwardRunner.swift:1462-1685), and the tail's output is read by nothing but the next
+ * layer's input norm and the residual add after its attention.  Every block of the projection launch repeats the tail's row
+ * reductions in its prologue (FusedLayerTail.swift:19-52 -> fused_layer_tail, fused.metal:271-375, with the shared expert's
+ * post-norm first) and normalises the result on its way into LDS; block 0 writes it to hidden_out.  One launch fewer per decoder
+ * layer; every output equals the two calls bit for bit.  hidden_out must be a different buffer from h2, shared_out and hidden
+ * for the tail to be folded in; otherwise, or with operands that are not 16-byte aligned or rows the row streamer does not
+ * take, the tail runs as its own launch first.  n <= 4096. */
+int32_t tf_fused_layer_tail_norm_qkv_gemv(tf_ctx *ctx, tf_stream stream,
+                               const void *h2, const void *shared_out, const void *hidden, void *hidden_out,
+                               const void *post_ffn1_weight, uint64_t post_ffn1_weight_offset,
+                               const void *post_ffn2_weight, uint64_t post_ffn2_weight_offset,
+                               const void *post_ffn_weight, uint64_t post_ffn_weight_offset, float tail_eps, float layer_scalar,
+                               const void *norm_weight, uint64_t norm_weight_offset, float eps,
+                               const void *q_weights, uint64_t q_weights_offset, const void *q_scales, uint64_t q_scales_offset,
+                               const void *q_biases, uint64_t q_biases_offset,
+                               const void *k_weights, uint64_t k_weights_offset, const void *k_scales, uint64_t k_scales_offset,
+                               const void *k_biases, uint64_t k_biases_offset,
+                               const void *v_weights, uint64_t v_weights_offset, const void *v_scales, uint64_t v_scales_offset,
+                               const void *v_biases, uint64_t v_biases_offset,
+                               void *q_out, uint64_t q_out_offset, void *k_out, uint64_t k_out_offset,
+                               void *v_out, uint64_t v_out_offset,
+                               uint32_t q_rows, uint32_t kv_rows, uint32_t n, tf_dtype scale_dtype);
 
 /* ---- primitives on the path -------------------------------------------------------------------------------- */
 /* gelu_mul_fp16 (Metal/Primitives/utility.metal:6-18; dispatched at SharedExpertInt4.swift:76-86):
@@ -521,6 +544,34 @@ int32_t tf_moe_decode_step_shared(tf_ctx *ctx, tf_stream stream,
                                   const void *shared_x, const tf_projection *shared_gate, const tf_projection *shared_up,
                                   const tf_projection *shared_down, void *shared_y, void *shared_scratch_gate,
                                   void *shared_scratch_up, void *shared_scratch_act);
+/* tf_fused_post_attn_setup followed by tf_moe_decode_step_shared as one call: FusedPostAttentionSetup.encode
+ * (FusedPostAttentionSetup.swift:19-56) makes the three vectors the MoE block reads - router_x for the router, routed_x for the
+ * routed experts, dense_x for the shared expert - and nothing else runs between it and them (RealForwardRunner.swift:1462-1594).
+ * Here every block of the first launch (router logits + shared gate / up) repeats the setup's two row reductions in its own
+ * prologue instead of waiting for a launch of them, one launch fewer per decoder layer; block 0 writes hidden_out (the new
+ * residual stream), dense_x, routed_x and router_x as the stand-alone call does.  Every output equals the two calls bit for
+ * bit.  hidden_out must be a different buffer from hidden (other blocks are still reading it) for the setup to be folded in;
+ * with hidden_out == hidden, operands that are not 16-byte aligned or a step that does not take the shared launches, the
+ * setup runs as its own launch first.  d <= 4096; the shared expert reads d values. */
+int32_t tf_moe_decode_step_shared_post_attn(tf_ctx *ctx, tf_stream stream,
+                                  const void *hidden, const void *attn, void *hidden_out,
+                                  const void *post_attention_weight, uint64_t post_attention_weight_offset,
+                                  const void *pre_ffn_weight, uint64_t pre_ffn_weight_offset,
+                                  const void *pre_ffn2_weight, uint64_t pre_ffn2_weight_offset, float eps,
+                                  const void *router_weights, uint64_t router_weights_offset,
+                                  const void *router_scales, uint64_t router_scales_offset,
+                                  const void *router_biases, uint64_t router_biases_offset,
+                                  void *router_x,
+                                  const void *effective_scale, uint64_t effective_scale_offset,
+                                  const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                                  const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                  const tf_expert_offsets *routed_offsets,
+                                  void *routed_x, void *acts, const void *residual, void *y,
+                                  void *out_indices, void *out_weights,
+                                  uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype,
+                                  void *dense_x, const tf_projection *shared_gate, const tf_projection *shared_up,
+                                  const tf_projection *shared_down, void *shared_y,
+                                  void *shared_scratch_gate, void *shared_scratch_up, void *shared_scratch_act);
 
 /* ---- lm_head ----------------------------------------------------------------------------------------------------------- */
 /* LMHeadChainInt4.encodeGreedyDecode (Kernels/Fusions/LMHeadChainInt4.swift:53-122) -> rmsnorm_bf16w,

@@ -268,3 +268,105 @@ def test_decode_step_with_the_shared_expert_riding_along_equals_the_two_calls(d,
                                          t["x"].data_ptr(), acts.data_ptr(), t["res"].data_ptr(), y.data_ptr(), idx.data_ptr(),
                                          wts.data_ptr(), d, f, 8, tfk.TF_BF16, x_ptr, C.byref(gate), C.byref(up), C.byref(up),
                                          sy.data_ptr(), sg.data_ptr(), su.data_ptr(), sa.data_ptr()) == tfk.TF_ERR_DIMENSION_MISMATCH
+
+
+@pytest.mark.parametrize("d,f,fs,in_place,misalign", [(D, F_MOE, F_SHARED, False, 0), (D, F_MOE, F_SHARED, True, 0), (D, F_MOE, F_SHARED, False, 2),
+                                                      (256, 128, 192, False, 0), (4096, 704, 2112, False, 0)])
+def test_post_attention_setup_inside_the_decode_step_equals_the_two_calls(d, f, fs, in_place, misalign):
+    # tf_moe_decode_step_shared_post_attn = tf_fused_post_attn_setup + tf_moe_decode_step_shared, every output bit for bit.  At the
+    # production widths with separate buffers the setup runs in the prologue of every block of the first launch; written over its
+    # own input, with a misaligned attention row or with rows too short for the shared launches it runs as a launch of its own.
+    c = M._decode_step_case(d, f, E, 0x9A7 + d + fs)
+    shared = dict(gate=refcases.synthetic_int4(fs, d, 0x61, "sg"), up=refcases.synthetic_int4(fs, d, 0x62, "su"),
+                  down=refcases.synthetic_int4(d, fs, 0x63, "sd"))
+    rng = np.random.default_rng(0x64 + d)
+    weights = [tfo.bf16_bits_array(1.0 + 0.1 * rng.standard_normal(d).astype(np.float32)) for _ in range(3)]
+    hidden_bits, attn_bits = refcases.normal_f16(d, 0x65), refcases.normal_f16(d, 0x66)
+    k = ctx()
+    lib, h = k.lib, k.handle
+    t = M._decode_step_tensors(c)
+    st = {n: [dev(a) for a in shared[n]] for n in shared}
+    gate, up, down = (tfk.projection(*st[n], r, cc) for n, r, cc in (("gate", fs, d), ("up", fs, d), ("down", d, fs)))
+    d_w = [dev(w) for w in weights]
+    d_attn = dev(np.concatenate([np.zeros(misalign // 2, np.uint16), attn_bits]))
+    attn_ptr = d_attn.data_ptr() + misalign
+    off = tfk.ExpertOffsets(*c["off"].as_tuple())
+    results = []
+    for one_call in (False, True):
+        outs = M._fresh_outs(d, f)
+        idx, wts, acts, y = outs
+        sy, sg, su, sa = (dev(np.full(n, 0x7BFF, np.uint16)) for n in (d, fs, fs, fs))
+        hidden = dev(hidden_bits)
+        hidden_out = hidden if in_place else dev(np.full(d, 0x7BFF, np.uint16))
+        dense_x, routed_x, router_x = (dev(np.full(d, 0x7BFF, np.uint16)) for _ in range(3))
+        step = (t["rW"].data_ptr(), 0, t["rS"].data_ptr(), 0, t["rB"].data_ptr(), 0, router_x.data_ptr(), t["eff"].data_ptr(), 0,
+                t["gain"].data_ptr(), 0, t["pool"].data_ptr(), c["stride"], E, off, routed_x.data_ptr(), acts.data_ptr(), t["res"].data_ptr(),
+                y.data_ptr(), idx.data_ptr(), wts.data_ptr(), d, f, 8, tfk.TF_BF16, dense_x.data_ptr(), C.byref(gate), C.byref(up), C.byref(down),
+                sy.data_ptr(), sg.data_ptr(), su.data_ptr(), sa.data_ptr())
+        if one_call:
+            k.check(lib.tf_moe_decode_step_shared_post_attn(h, None, hidden.data_ptr(), attn_ptr, hidden_out.data_ptr(), d_w[0].data_ptr(), 0,
+                                                            d_w[1].data_ptr(), 0, d_w[2].data_ptr(), 0, EPS, *step))
+        else:
+            if not in_place:
+                hidden_out.copy_(hidden)
+            k.check(lib.tf_fused_post_attn_setup(h, None, hidden_out.data_ptr(), attn_ptr, dense_x.data_ptr(), routed_x.data_ptr(), router_x.data_ptr(),
+                                                 d_w[0].data_ptr(), 0, d_w[1].data_ptr(), 0, d_w[2].data_ptr(), 0, d, EPS))
+            k.check(lib.tf_moe_decode_step_shared(h, None, *step))
+        results.append(M._read_outs(outs, d, f) + tuple(host(b_, np.uint16) for b_ in (sy, sg, su, sa, hidden_out, dense_x, routed_x, router_x)))
+        if not in_place:
+            assert np.array_equal(host(hidden, np.uint16), hidden_bits)      # the input row is left alone
+    for a, b_ in zip(*results):
+        assert np.array_equal(a, b_)
+    # the setup itself against the oracle's post-attention setup
+    want = tfo.k_post_attn_setup(hidden_bits, attn_bits, weights[0], weights[1], weights[2], EPS)
+    for got, ref in zip(results[1][8:12], want):
+        assert np.max(np.abs(tfo.from_f16_bits(got) - tfo.from_f16_bits(ref))) <= 2e-3 * max(1.0, float(np.max(np.abs(tfo.from_f16_bits(ref)))))
+
+
+@pytest.mark.parametrize("n,q_rows,kv_rows,in_place,misalign", [(D, NQ * HD, NKV * HD, False, 0), (D, NQ * HD, NKV * HD, True, 0),
+                                                               (D, NQ * HD, NKV * HD, False, 2), (512, 96, 64, False, 0), (4096, 130, 66, False, 0)])
+def test_layer_tail_inside_the_next_qkv_launch_equals_the_two_calls(n, q_rows, kv_rows, in_place, misalign):
+    # tf_fused_layer_tail_norm_qkv_gemv = tf_fused_layer_tail_shared_norm + tf_fused_norm_qkv_gemv, every output bit for bit: with
+    # separate buffers at the production width every block of the projection launch repeats the tail in its prologue; written
+    # over its own input, with a misaligned h2 row or with rows the row streamer does not take, the tail is a launch of its own
+    rng = np.random.default_rng(n + 7)
+    bits = lambda a: a.astype(np.float32).astype(np.float16).view(np.uint16)
+    mats = [refcases.synthetic_int4(r, n, 0x87 + i, "qkv"[i]) for i, r in enumerate((q_rows, kv_rows, kv_rows))]
+    h2, shared, hidden = bits(rng.standard_normal(n) * 0.3), bits(rng.standard_normal(n) * 2.0), bits(rng.standard_normal(n))
+    w1, w2, w3, nw = (tfo.bf16_bits_array(1.0 + 0.1 * rng.standard_normal(n).astype(np.float32)) for _ in range(4))
+    k = ctx()
+    lib, h = k.lib, k.handle
+    t = [[dev(a) for a in m] for m in mats]
+    d_sh, d_w1, d_w2, d_w3, d_nw = dev(shared), dev(w1), dev(w2), dev(w3), dev(nw)
+    d_h2 = dev(np.concatenate([np.zeros(misalign // 2, np.uint16), h2]))
+    h2_ptr = d_h2.data_ptr() + misalign
+    qkv = []
+    for m in t:
+        qkv += [m[0].data_ptr(), 0, m[1].data_ptr(), 0, m[2].data_ptr(), 0]
+    results = []
+    for one_call in (False, True):
+        outs = [dev(np.full(r, 0x7BFF, np.uint16)) for r in (q_rows, kv_rows, kv_rows)]
+        hid = dev(hidden)
+        hid_out = hid if in_place else dev(np.full(n, 0x7BFF, np.uint16))
+        out_args = (outs[0].data_ptr(), 0, outs[1].data_ptr(), 0, outs[2].data_ptr(), 0, q_rows, kv_rows, n, tfk.TF_BF16)
+        if one_call:
+            k.check(lib.tf_fused_layer_tail_norm_qkv_gemv(h, None, h2_ptr, d_sh.data_ptr(), hid.data_ptr(), hid_out.data_ptr(), d_w1.data_ptr(), 0,
+                                                          d_w2.data_ptr(), 0, d_w3.data_ptr(), 0, EPS, LAYER_SCALAR, d_nw.data_ptr(), 0, EPS, *qkv, *out_args))
+        else:
+            if not in_place:
+                hid_out.copy_(hid)
+            k.check(lib.tf_fused_layer_tail_shared_norm(h, None, h2_ptr, d_sh.data_ptr(), hid_out.data_ptr(), d_w1.data_ptr(), 0, d_w2.data_ptr(), 0,
+                                                        d_w3.data_ptr(), 0, n, EPS, LAYER_SCALAR))
+            k.check(lib.tf_fused_norm_qkv_gemv(h, None, d_nw.data_ptr(), 0, EPS, *qkv, hid_out.data_ptr(), *out_args))
+        results.append([host(o, np.uint16) for o in outs] + [host(hid_out, np.uint16)])
+        if not in_place:
+            assert np.array_equal(host(hid, np.uint16), hidden)       # the input row is left alone
+    for a, b_ in zip(*results):
+        assert np.array_equal(a, b_)
+    want_hidden = tfo.k_layer_tail(h2, tfo.k_rmsnorm_bf16w(shared, w1, EPS), hidden, w2, w3, EPS, LAYER_SCALAR)
+    assert tfo.rel_error(tfo.from_f16_bits(results[1][3]), tfo.from_f16_bits(want_hidden)) < tfo.Tolerance.fp16Reduction
+    for got, m in zip(results[1][:3], mats):
+        want = gemv(m, tfo.k_rmsnorm_bf16w(results[1][3], nw, EPS))
+        assert tfo.rel_error(tfo.from_f16_bits(got), tfo.from_f16_bits(want)) < TOL
+    assert lib.tf_fused_layer_tail_norm_qkv_gemv(h, None, h2_ptr, d_sh.data_ptr(), hid.data_ptr(), None, d_w1.data_ptr(), 0, d_w2.data_ptr(), 0,
+                                                 d_w3.data_ptr(), 0, EPS, LAYER_SCALAR, d_nw.data_ptr(), 0, EPS, *qkv, *out_args) == tfk.TF_ERR_INVALID_ARGUMENT

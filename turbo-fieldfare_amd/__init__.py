@@ -125,6 +125,8 @@ EXPORTS = {
     "tf_dequant_int8_gemv": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, i32, i32]),
     "tf_fused_qkv_gemv": (i32, [vp, vp] + [vp, u64] * 9 + [vp] + [vp, u64] * 3 + [u32, u32, u32, i32]),
     "tf_fused_norm_qkv_gemv": (i32, [vp, vp, vp, u64, C.c_float] + [vp, u64] * 9 + [vp] + [vp, u64] * 3 + [u32, u32, u32, i32]),
+    "tf_fused_layer_tail_norm_qkv_gemv": (i32, [vp, vp, vp, vp, vp, vp] + [vp, u64] * 3 + [C.c_float, C.c_float, vp, u64, C.c_float] + [vp, u64] * 9 +
+                                          [vp, u64] * 3 + [u32, u32, u32, i32]),
     "tf_gelu_mul_fp16": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32]),
     "tf_rmsnorm_bf16w": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u32, C.c_float]),
     "tf_fused_post_attn_setup": (i32, [vp, vp, vp, vp, vp, vp, vp, vp, u64, vp, u64, vp, u64, u32, C.c_float]),
@@ -173,6 +175,10 @@ EXPORTS = {
     "tf_moe_decode_step_shared": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, vp, u64, vp, u64, vp, u64, u32, C.POINTER(ExpertOffsets),
                                         vp, vp, vp, vp, vp, vp, u32, u32, u32, i32, vp, C.POINTER(Projection), C.POINTER(Projection),
                                         C.POINTER(Projection), vp, vp, vp, vp]),
+    "tf_moe_decode_step_shared_post_attn": (i32, [vp, vp, vp, vp, vp, vp, u64, vp, u64, vp, u64, C.c_float,
+                                                  vp, u64, vp, u64, vp, u64, vp, vp, u64, vp, u64, vp, u64, u32, C.POINTER(ExpertOffsets),
+                                                  vp, vp, vp, vp, vp, vp, u32, u32, u32, i32, vp, C.POINTER(Projection),
+                                                  C.POINTER(Projection), C.POINTER(Projection), vp, vp, vp, vp]),
     "tf_prefill_router_gemma4_block": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64,
                                              u32, u32, u32, u32, u32]),
     "tf_prefill_make_token_expert_pairs": (i32, [vp, vp, i32, i32, vp]),

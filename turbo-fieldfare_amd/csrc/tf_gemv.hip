@@ -1,6 +1,7 @@
 // Affine int4/int8 dequantization and GEMV for gfx950, plus the two small primitives on the same path
 // (gelu_mul_fp16, rmsnorm_bf16w).
 #include "tf_gemv_kernels.hpp"
+#include "tf_rowslice.hpp"
 
 using namespace tfk;
 
@@ -111,13 +112,21 @@ struct GemvSegments {
     uint32_t tile_end[3];   // running total of tiles up to and including each matrix
 };
 
-// FUSE_NORM: x is the raw hidden vector and every block normalises it on the way into LDS (rmsnorm_bf16w with norm_w), so the
+// MODE 1: x is the raw hidden vector and every block normalises it on the way into LDS (rmsnorm_bf16w with norm_w), so the
 // input norm of a decoder layer needs no launch of its own.
-template <int RT, int NP, int SD, bool FUSE_NORM>
-__global__ __launch_bounds__(256, 4) void qkv_gemv_long_kernel(GemvSegments g, const half_t *x, const uint16_t *norm_w, float eps, int k) {
-    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
-    __shared__ float xsum[XStage::kMaxK / 32];
-    __shared__ float norm_partial[4];
+// MODE 2: the hidden vector is itself made here, by the layer tail of the previous decoder layer (layer_tail_row with the norm of
+// the shared expert's output; k <= 4096, every row and norm weight 16-byte aligned): every block repeats the tail's row
+// reductions in its prologue, block 0 writes the result to tail.hidden_out (not a buffer the other blocks still read), and the
+// input norm follows as in mode 1.
+struct TailFuse {
+    const half_t *h2, *h1, *hidden;
+    half_t *hidden_out;
+    const uint16_t *w_postffn2, *w_postffn, *w_postffn1;
+    float eps, layer_scalar;
+};
+template <int RT, int NP, int SD, int MODE>
+__device__ __forceinline__ void qkv_gemv_long_body(const GemvSegments &g, const half_t *x, const uint16_t *norm_w, float eps, int k, const TailFuse &tail,
+                                                   u32x4 *xa, float *xsum, float *norm_partial) {
     const int lane = threadIdx.x & 63;
     const long wave = uniform_int((int)(((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6));
     const long nwaves = ((long)gridDim.x * blockDim.x) >> 6;
@@ -140,7 +149,27 @@ __global__ __launch_bounds__(256, 4) void qkv_gemv_long_kernel(GemvSegments g, c
         rs.load(t, g.W[seg] + local * tile_bytes, g.S[seg] + local * sb_bytes, g.B[seg] + local * sb_bytes, (long)g.rows[seg] - local * RT);
     };
     long t0 = wave, t1 = wave + nwaves;
-    if constexpr (FUSE_NORM) {
+    if constexpr (MODE == 2) {
+        const RowSlice<true> slice{(uint32_t)k};
+        float h2[kPerThread], w2[kPerThread], h1[kPerThread], wp[kPerThread], hid[kPerThread], w1[kPerThread];
+        // the rows first: loads return in the order of their requests, and the tail's arithmetic should not wait for the weights
+        slice.load_f16(tail.h2, h2);
+        slice.load_bf16(tail.w_postffn2, w2);
+        slice.load_f16(tail.h1, h1);
+        slice.load_bf16(tail.w_postffn, wp);
+        slice.load_f16(tail.hidden, hid);
+        slice.load_bf16(tail.w_postffn1, w1);
+        XNormStage stage;
+        stage.request_weight(norm_w, k);
+        if (t0 < ntiles) request(ta, t0);
+        if (t1 < ntiles) request(tb, t1);
+        layer_tail_row<true>((uint32_t)k, h2, w2, h1, wp, hid, w1, tail.eps, tail.layer_scalar, norm_partial + 4);
+        if (blockIdx.x == 0) slice.store_f16(tail.hidden_out, hid);
+        stage.xr[0] = pack_half8(hid);
+        stage.xr[1] = pack_half8(hid + 8);
+        stage.xr[2] = stage.xr[3] = u32x4{0u, 0u, 0u, 0u};
+        stage.publish(eps, k, xa, xsum, norm_partial);
+    } else if constexpr (MODE == 1) {
         XNormStage stage;
         stage.request(x, norm_w, k);
         if (t0 < ntiles) request(ta, t0);
@@ -177,6 +206,22 @@ __global__ __launch_bounds__(256, 4) void qkv_gemv_long_kernel(GemvSegments g, c
         if (t1 < ntiles) request(tb, t1);
         if (t0 >= ntiles) break;
     }
+}
+
+template <int RT, int NP, int SD, bool FUSE_NORM>
+__global__ __launch_bounds__(256, 4) void qkv_gemv_long_kernel(GemvSegments g, const half_t *x, const uint16_t *norm_w, float eps, int k) {
+    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
+    __shared__ float xsum[XStage::kMaxK / 32];
+    __shared__ float norm_partial[4];
+    qkv_gemv_long_body<RT, NP, SD, FUSE_NORM ? 1 : 0>(g, x, norm_w, eps, k, TailFuse{}, xa, xsum, norm_partial);
+}
+// the rows of the tail live in registers beside the two weight tiles: two blocks per CU
+template <int RT, int NP, int SD>
+__global__ __launch_bounds__(256, 2) void qkv_gemv_after_tail_kernel(GemvSegments g, TailFuse tail, const uint16_t *norm_w, float eps, int k) {
+    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
+    __shared__ float xsum[XStage::kMaxK / 32];
+    __shared__ float norm_partial[16];
+    qkv_gemv_long_body<RT, NP, SD, 2>(g, nullptr, norm_w, eps, k, tail, xa, xsum, norm_partial);
 }
 
 // K <= 1024: each wave covers 2 * NPASS consecutive rows, one row per half-wave per pass.
@@ -623,13 +668,22 @@ int32_t tf_prefill_rmsnorm_no_scale_perhead_block(tf_ctx *ctx, tf_stream stream,
                               token_stride_elements, eps, "prefill_rmsnorm_no_scale_perhead_block");
 }
 
+// The layer tail that makes the hidden vector of a tf_fused_layer_tail_norm_qkv_gemv call
+struct TailCall {
+    const void *h2, *shared_out, *hidden;
+    void *hidden_out;
+    const void *w_postffn1, *w_postffn2, *w_postffn;
+    uint64_t w_postffn1_offset, w_postffn2_offset, w_postffn_offset;
+    float eps, layer_scalar;
+};
+
 static int32_t qkv_gemv_entry(tf_ctx *ctx, tf_stream stream, const char *who, const void *norm_weight, uint64_t norm_weight_offset, float eps, const void *q_weights, uint64_t q_weights_offset, const void *q_scales,
                           uint64_t q_scales_offset, const void *q_biases, uint64_t q_biases_offset, const void *k_weights,
                           uint64_t k_weights_offset, const void *k_scales, uint64_t k_scales_offset, const void *k_biases,
                           uint64_t k_biases_offset, const void *v_weights, uint64_t v_weights_offset, const void *v_scales,
                           uint64_t v_scales_offset, const void *v_biases, uint64_t v_biases_offset, const void *x, void *q_out,
                           uint64_t q_out_offset, void *k_out, uint64_t k_out_offset, void *v_out, uint64_t v_out_offset, uint32_t q_rows,
-                          uint32_t kv_rows, uint32_t n, tf_dtype scale_dtype) {
+                          uint32_t kv_rows, uint32_t n, tf_dtype scale_dtype, const TailCall *tail = nullptr) {
     const uint16_t *nw = norm_weight ? reinterpret_cast<const uint16_t *>(at(norm_weight, norm_weight_offset)) : nullptr;
     const void *w[3] = {q_weights, k_weights, v_weights};
     const void *s[3] = {q_scales, k_scales, v_scales};
@@ -649,6 +703,27 @@ static int32_t qkv_gemv_entry(tf_ctx *ctx, tf_stream stream, const char *who, co
     const LongPlan plan = plan_long_rows((int)n);
     bool fast = aligned16(x) && n > 1024 && n <= (uint32_t)XStage::kMaxK && plan.rt > 0 && (!nw || aligned16(nw));
     for (int i = 0; i < 3; ++i) fast = fast && aligned16(at(w[i], wo[i]));
+    TailFuse tf = {};
+    bool tail_fused = false;
+    if (tail) {
+        // x is tail->hidden_out, which the tail makes.  Inside the projection launch when that is the row streamer, every row and
+        // norm weight moves in 16-byte pieces and the output is not a row the other blocks still read; a launch of its own otherwise.
+        tf = {static_cast<const half_t *>(tail->h2), static_cast<const half_t *>(tail->shared_out), static_cast<const half_t *>(tail->hidden),
+              static_cast<half_t *>(tail->hidden_out), reinterpret_cast<const uint16_t *>(at(tail->w_postffn2, tail->w_postffn2_offset)),
+              reinterpret_cast<const uint16_t *>(at(tail->w_postffn, tail->w_postffn_offset)),
+              reinterpret_cast<const uint16_t *>(at(tail->w_postffn1, tail->w_postffn1_offset)), tail->eps, tail->layer_scalar};
+        const void *ins[3] = {tf.h2, tf.h1, tf.hidden};
+        bool distinct = true;
+        for (int i = 0; i < 3; ++i) distinct = distinct && ins[i] != (const void *)tf.hidden_out;
+        tail_fused = fast && nw && distinct && n <= kGlueMaxD && n % 8 == 0 && aligned16(tf.h2) && aligned16(tf.h1) && aligned16(tf.hidden) &&
+                     aligned16(tf.hidden_out) && aligned16(tf.w_postffn2) && aligned16(tf.w_postffn) && aligned16(tf.w_postffn1);
+        if (!tail_fused) {
+            const int32_t rc = layer_tail_shared_norm_to(ctx, stream, tail->h2, tail->shared_out, tail->hidden, tail->hidden_out, tail->w_postffn1,
+                                                         tail->w_postffn1_offset, tail->w_postffn2, tail->w_postffn2_offset, tail->w_postffn,
+                                                         tail->w_postffn_offset, n, tail->eps, tail->layer_scalar);
+            if (rc != TF_OK) return rc;
+        }
+    }
     if (fast) {
         GemvSegments g;
         uint32_t total = 0;
@@ -666,7 +741,10 @@ static int32_t qkv_gemv_entry(tf_ctx *ctx, tf_stream stream, const char *who, co
         const half_t *xh = static_cast<const half_t *>(x);
 #define TF_QKV_CASE(RT_, NP_)                                                                                             \
     if (plan.rt == RT_ && plan.np == NP_) {                                                                               \
-        if (nw) {                                                                                                         \
+        if (tail_fused) {                                                                                                 \
+            if (scale_dtype == TF_BF16) hipLaunchKernelGGL((qkv_gemv_after_tail_kernel<RT_, NP_, 0>), dim3(grid), dim3(256), 0, st, g, tf, nw, eps, (int)n); \
+            else hipLaunchKernelGGL((qkv_gemv_after_tail_kernel<RT_, NP_, 1>), dim3(grid), dim3(256), 0, st, g, tf, nw, eps, (int)n); \
+        } else if (nw) {                                                                                                  \
             if (scale_dtype == TF_BF16) hipLaunchKernelGGL((qkv_gemv_long_kernel<RT_, NP_, 0, true>), dim3(grid), dim3(256), 0, st, g, xh, nw, eps, (int)n); \
             else hipLaunchKernelGGL((qkv_gemv_long_kernel<RT_, NP_, 1, true>), dim3(grid), dim3(256), 0, st, g, xh, nw, eps, (int)n); \
         } else {                                                                                                          \
@@ -723,6 +801,29 @@ int32_t tf_fused_norm_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *norm_w
                           q_scales_offset, q_biases, q_biases_offset, k_weights, k_weights_offset, k_scales, k_scales_offset, k_biases,
                           k_biases_offset, v_weights, v_weights_offset, v_scales, v_scales_offset, v_biases, v_biases_offset, hidden, q_out,
                           q_out_offset, k_out, k_out_offset, v_out, v_out_offset, q_rows, kv_rows, n, scale_dtype);
+}
+
+int32_t tf_fused_layer_tail_norm_qkv_gemv(tf_ctx *ctx, tf_stream stream, const void *h2, const void *shared_out, const void *hidden,
+                                          void *hidden_out, const void *post_ffn1_weight, uint64_t post_ffn1_weight_offset,
+                                          const void *post_ffn2_weight, uint64_t post_ffn2_weight_offset, const void *post_ffn_weight,
+                                          uint64_t post_ffn_weight_offset, float tail_eps, float layer_scalar, const void *norm_weight,
+                                          uint64_t norm_weight_offset, float eps, const void *q_weights, uint64_t q_weights_offset,
+                                          const void *q_scales, uint64_t q_scales_offset, const void *q_biases, uint64_t q_biases_offset,
+                                          const void *k_weights, uint64_t k_weights_offset, const void *k_scales, uint64_t k_scales_offset,
+                                          const void *k_biases, uint64_t k_biases_offset, const void *v_weights, uint64_t v_weights_offset,
+                                          const void *v_scales, uint64_t v_scales_offset, const void *v_biases, uint64_t v_biases_offset,
+                                          void *q_out, uint64_t q_out_offset, void *k_out, uint64_t k_out_offset, void *v_out,
+                                          uint64_t v_out_offset, uint32_t q_rows, uint32_t kv_rows, uint32_t n, tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx && norm_weight && h2 && shared_out && hidden && hidden_out && post_ffn1_weight && post_ffn2_weight && post_ffn_weight,
+               TF_ERR_INVALID_ARGUMENT, "fused_layer_tail_norm_qkv_gemv: null argument");
+    TF_REQUIRE(ctx, norm_weight_offset % 2 == 0 && aligned(norm_weight, 2), TF_ERR_INVALID_ARGUMENT, "fused_layer_tail_norm_qkv_gemv: misaligned norm weight");
+    TF_REQUIRE(ctx, n > 0 && n <= kGlueMaxD, TF_ERR_INVALID_ARGUMENT, "fused_layer_tail_norm_qkv_gemv: D must be in 1...4096, got %u", n);
+    const TailCall tail = {h2, shared_out, hidden, hidden_out, post_ffn1_weight, post_ffn2_weight, post_ffn_weight, post_ffn1_weight_offset,
+                           post_ffn2_weight_offset, post_ffn_weight_offset, tail_eps, layer_scalar};
+    return qkv_gemv_entry(ctx, stream, "fused_layer_tail_norm_qkv_gemv", norm_weight, norm_weight_offset, eps, q_weights, q_weights_offset, q_scales,
+                          q_scales_offset, q_biases, q_biases_offset, k_weights, k_weights_offset, k_scales, k_scales_offset, k_biases,
+                          k_biases_offset, v_weights, v_weights_offset, v_scales, v_scales_offset, v_biases, v_biases_offset, hidden_out, q_out,
+                          q_out_offset, k_out, k_out_offset, v_out, v_out_offset, q_rows, kv_rows, n, scale_dtype, &tail);
 }
 
 }  // extern "C"

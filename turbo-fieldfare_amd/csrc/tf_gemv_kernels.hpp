@@ -36,4 +36,13 @@ int32_t validate_gemv(tf_ctx *ctx, const char *who, const void *weights, uint64_
                       const void *biases, uint64_t bo, const void *x, uint64_t xo, const void *y, uint64_t yo,
                       uint32_t m, uint32_t n, tf_dtype sd, tf_dtype od, unsigned weights_align);
 
+// tf_fused_post_attn_setup with the new residual stream written to hidden_out instead of over hidden (tf_glue.hip)
+int32_t post_attn_setup_to(tf_ctx *ctx, tf_stream stream, const void *hidden, void *hidden_out, const void *attn, void *dense_x, void *routed_x,
+                           void *router_x, const void *w_post, uint64_t w_post_offset, const void *w_pre, uint64_t w_pre_offset,
+                           const void *w_pre2, uint64_t w_pre2_offset, uint32_t d, float eps);
+// tf_fused_layer_tail_shared_norm with the layer's output written to hidden_out instead of over hidden (tf_glue.hip)
+int32_t layer_tail_shared_norm_to(tf_ctx *ctx, tf_stream stream, const void *h2, const void *shared_out, const void *hidden, void *hidden_out,
+                                  const void *w_postffn1, uint64_t w_postffn1_offset, const void *w_postffn2, uint64_t w_postffn2_offset,
+                                  const void *w_postffn, uint64_t w_postffn_offset, uint32_t d, float eps, float layer_scalar);
+
 }  // namespace tfk

@@ -1,6 +1,7 @@
 // Router (int8 GEMV + top-8 + softmax), routed expert phases 1 and 2, and the int4 shared expert, for gfx950.
 #include "tf_gemv_kernels.hpp"
 #include "tf_router.hpp"
+#include "tf_rowslice.hpp"
 
 using namespace tfk;
 
@@ -426,6 +427,126 @@ __global__ __launch_bounds__(256) void router_and_shared_gate_up_kernel(RouterAr
     shared_gate_up_long_body<RT, NP, SD>(sh, blockIdx.x - r.num_experts, xa, xsum);
 }
 
+// The same launch with the post-attention setup (FusedPostAttentionSetup: residual add, the norms that make dense_x, routed_x
+// and router_x) repeated by every block in its prologue instead of a launch of its own ahead of this one: a block requests
+// its weights, then the attention output, the residual stream and the norm weights (27 KB out of L2), computes the two
+// row reductions and keeps the one vector it multiplies with in LDS - router blocks router_x, shared-expert blocks dense_x.
+// Block 0 also writes the four vectors to memory: the new residual stream and routed_x for the launches that follow, dense_x
+// and router_x for the caller.  Thread t of the setup owns the same 8-element pieces as thread t of the staging code, and the
+// arithmetic is PostAttnRow's, so every value equals what the stand-alone setup kernel writes.  hidden_out must not be the
+// residual stream that the other blocks are still reading.
+struct PostAttnFuseArgs {
+    const half_t *hidden, *attn;
+    half_t *hidden_out, *dense_x, *routed_x, *router_x;
+    const uint16_t *w_post_attn, *w_pre_ffn, *w_pre_ffn2;
+    float eps;
+};
+template <int RT, int NP, int SD>
+__global__ __launch_bounds__(256) void post_attn_router_and_shared_gate_up_kernel(PostAttnFuseArgs pa, RouterArgs r, SharedGateUpArgs sh) {
+    __shared__ __align__(16) u32x4 xa[XStage::kMaxK / 8];
+    __shared__ float xsum[XStage::kMaxK / 32];
+    __shared__ float partial[4];
+    __shared__ float norm_partial[8];
+    const int d = r.d;
+    const RowSlice<true> rs{(uint32_t)d};
+    float at[kPerThread], w[kPerThread];
+    PostAttnRow<true> pr;
+    if (blockIdx.x < r.num_experts) {
+        // ---- router role: thread c multiplies chunk c (16 values) of the expert's row
+        const uint32_t e = blockIdx.x;
+        const int c = threadIdx.x, chunks = d >> 4, groups = d >> 6;
+        // the rows of the setup first: loads return in the order of their requests
+        rs.load_f16(pa.attn, at);
+        rs.load_bf16(pa.w_post_attn, w);
+        rs.load_f16(pa.hidden, pr.h);
+        float w2[kPerThread], w3[kPerThread];
+        if (e == 0) {
+            rs.load_bf16(pa.w_pre_ffn, w2);
+            rs.load_bf16(pa.w_pre_ffn2, w3);
+        }
+        u32x4 wv = {0u, 0u, 0u, 0u}, ea = wv, eb = wv;
+        uint16_t sv = 0, bv = 0;
+        if (c < chunks) {
+            wv = load16(r.W + (size_t)e * d + (size_t)c * 16);
+            ea = load16(r.eff + c * 16);
+            eb = load16(r.eff + c * 16 + 8);
+            sv = *reinterpret_cast<const uint16_t *>(r.S + (size_t)e * groups * 2 + (c >> 2) * 2);
+            bv = *reinterpret_cast<const uint16_t *>(r.B + (size_t)e * groups * 2 + (c >> 2) * 2);
+        }
+        pr.finish(rs, at, w, pa.eps, norm_partial);
+        if (e == 0) rs.store_f16(pa.hidden_out, pr.h);
+#pragma unroll
+        for (int j = 0; j < kPerThread; ++j) {
+            const float hn = pr.h[j] * pr.inv;
+            if (e == 0) {
+                w2[j] = round_half(hn * w2[j]);
+                w3[j] = round_half(hn * w3[j]);
+            }
+            pr.h[j] = round_half(hn);
+        }
+        if (e == 0) {
+            rs.store_f16(pa.dense_x, w2);
+            rs.store_f16(pa.routed_x, w3);
+            rs.store_f16(pa.router_x, pr.h);
+        }
+        half_t *row = reinterpret_cast<half_t *>(xa);   // router_x as a plain fp16 row
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+            if (rs.live(8 * p)) *reinterpret_cast<u32x4 *>(row + rs.index(8 * p)) = pack_half8(pr.h + 8 * p);
+        __syncthreads();
+        float acc = 0.0f;
+        if (c < chunks) {
+            const u32x4 ha = *reinterpret_cast<const u32x4 *>(row + c * 16), hb = *reinterpret_cast<const u32x4 *>(row + c * 16 + 8);
+            router_chunk(wv, ha, hb, ea, eb, sb_to_f32<0>(sv), sb_to_f32<0>(bv), acc);
+        }
+        acc = wave_sum(acc);
+        if ((threadIdx.x & 63) == 0) partial[threadIdx.x >> 6] = acc;
+        __syncthreads();
+        if (threadIdx.x == 0) r.logits[e] = ((partial[0] + partial[1]) + partial[2]) + partial[3];
+        return;
+    }
+    // ---- shared expert's gate / up role: shared_gate_up_long_body with dense_x made here
+    const int lane = threadIdx.x & 63;
+    const uint32_t tile = uniform_u32(((blockIdx.x - r.num_experts) * blockDim.x + threadIdx.x) >> 6);
+    const uint32_t row0 = tile * RT;
+    const bool live = row0 < sh.f;
+    float w2[kPerThread];
+    rs.load_f16(pa.attn, at);
+    rs.load_bf16(pa.w_post_attn, w);
+    rs.load_f16(pa.hidden, pr.h);
+    rs.load_bf16(pa.w_pre_ffn, w2);
+    RowStream<RT, NP> stream;
+    typename RowStream<RT, NP>::Tile tg, tu;
+    stream.init_map(d, lane);
+    if (live) {
+        const size_t w_byte = (size_t)row0 * (d >> 1);
+        const size_t sb_byte = (size_t)row0 * (d >> 6) * 2;
+        stream.load(tg, sh.gW + w_byte, sh.gS + sb_byte, sh.gB + sb_byte, sh.f - row0);
+        stream.load(tu, sh.uW + w_byte, sh.uS + sb_byte, sh.uB + sb_byte, sh.f - row0);
+    }
+    pr.finish(rs, at, w, pa.eps, norm_partial);
+#pragma unroll
+    for (int j = 0; j < kPerThread; ++j) w2[j] = round_half(pr.h[j] * pr.inv * w2[j]);
+#pragma unroll
+    for (int p = 0; p < 2; ++p) XStage::publish_piece(pack_half8(w2 + 8 * p), threadIdx.x + 256 * p, d >> 3, d >> 5, xa, xsum);
+    __syncthreads();
+    if (!live) return;
+    stream.init_x_lds(xa, xsum, d);
+    float gate[RT], up[RT];
+    stream.template reduce<SD>(tg, gate);
+    stream.template reduce<SD>(tu, up);
+    if (lane == 0) {
+#pragma unroll
+        for (int r_ = 0; r_ < RT; ++r_) {
+            if (row0 + r_ >= sh.f) continue;
+            const half_t g16 = (half_t)gate[r_], u16 = (half_t)up[r_];
+            sh.gate_out[row0 + r_] = g16;
+            sh.up_out[row0 + r_] = u16;
+            sh.act_out[row0 + r_] = (half_t)(gelu_tanh((float)g16) * (float)u16);
+        }
+    }
+}
+
 // One RT-row tile of y = W x per wave (fp16 out): the row streamer of the GEMV entry points, one tile a wave.
 struct GemvTileArgs {
     const uint8_t *W, *S, *B;
@@ -791,7 +912,7 @@ int32_t router_logits_entry(tf_ctx *ctx, tf_stream stream, const void *weights, 
                             const void *effective_scale, uint64_t effective_scale_offset, const void *per_expert_scale,
                             uint64_t per_expert_scale_offset, void *out_indices, void *out_weights, uint32_t num_experts,
                             uint32_t d, uint32_t top_k, float *logits, const SharedGateUpArgs *ride = nullptr, int ride_sd = 0,
-                            bool *ride_taken = nullptr) {
+                            bool *ride_taken = nullptr, const PostAttnFuseArgs *post = nullptr) {
     if (ride_taken) *ride_taken = false;
     TF_REQUIRE(ctx, ctx && weights && scales && biases && hidden && effective_scale && per_expert_scale && out_indices && out_weights,
                TF_ERR_INVALID_ARGUMENT, "router_gemma4: null argument");
@@ -809,10 +930,18 @@ int32_t router_logits_entry(tf_ctx *ctx, tf_stream stream, const void *weights, 
     const bool fast = aligned16(w) && aligned16(hidden) && aligned16(eff) && d <= 4096;
     const int npass = fast ? (int)((d / 16 + 63) / 64) : 0;
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // the post-attention setup in this launch's prologue needs this launch to be the one kernel below (the caller checked)
+    TF_REQUIRE(ctx, !post || (fast && ride), TF_ERR_INVALID_ARGUMENT, "router_gemma4: the fused post-attention setup does not apply to these operands");
     if (fast && ride) {
         // the shared expert's gate / up rows as extra blocks of this launch (two-row tiles of three passes: the caller checked)
         const RouterArgs ra = {w, s, b, static_cast<const half_t *>(hidden), reinterpret_cast<const uint16_t *>(eff), logits, num_experts, (int)d};
         const uint32_t shared_blocks = ((ride->f + 1) / 2 + 3) / 4;
+        if (post) {
+            if (ride_sd == 0) hipLaunchKernelGGL((post_attn_router_and_shared_gate_up_kernel<2, 3, 0>), dim3(num_experts + shared_blocks), dim3(256), 0, st, *post, ra, *ride);
+            else hipLaunchKernelGGL((post_attn_router_and_shared_gate_up_kernel<2, 3, 1>), dim3(num_experts + shared_blocks), dim3(256), 0, st, *post, ra, *ride);
+            if (ride_taken) *ride_taken = true;
+            return check_launch(ctx, "post-attention setup + router_gemma4 logits + shared gate/up");
+        }
         if (ride_sd == 0) hipLaunchKernelGGL((router_and_shared_gate_up_kernel<2, 3, 0>), dim3(num_experts + shared_blocks), dim3(256), 0, st, ra, *ride);
         else hipLaunchKernelGGL((router_and_shared_gate_up_kernel<2, 3, 1>), dim3(num_experts + shared_blocks), dim3(256), 0, st, ra, *ride);
         if (ride_taken) *ride_taken = true;
@@ -861,7 +990,7 @@ int32_t decode_step_impl(tf_ctx *ctx, tf_stream stream, const void *router_weigh
                            const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
                            const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
                            void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype, float *logits,
-                         bool may_time, const SharedRide *ride = nullptr) {
+                         bool may_time, const SharedRide *ride = nullptr, const PostAttnFuseArgs *post = nullptr) {
     TF_REQUIRE(ctx, ctx && expert_pool && out_indices, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: null argument");
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool timed = may_time && ctx->step_timing;
@@ -874,7 +1003,7 @@ int32_t decode_step_impl(tf_ctx *ctx, tf_stream stream, const void *router_weigh
     int32_t rc = router_logits_entry(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset,
                                      router_biases, router_biases_offset, router_x, effective_scale, effective_scale_offset,
                                      per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, d, top_k, logits,
-                                     ride ? &ride->gate_up : nullptr, ride_sd, &rode);
+                                     ride ? &ride->gate_up : nullptr, ride_sd, &rode, post);
     if (rc != TF_OK) return rc;
     if (ride && !rode) {   // the router took another kernel: the shared expert's gate / up rows get their own launch
         if (ride_sd == 0) hipLaunchKernelGGL((shared_gate_up_long_kernel<2, 3, 0>), dim3(((ride->gate_up.f + 1) / 2 + 3) / 4), dim3(256), 0, st, ride->gate_up);
@@ -1050,16 +1179,30 @@ int32_t tf_moe_decode_step_static(tf_ctx *ctx, tf_stream stream, const void *rou
                             out_indices, out_weights, d, f, top_k, scale_dtype, ctx->static_router_logits, false);
 }
 
-int32_t tf_moe_decode_step_shared(tf_ctx *ctx, tf_stream stream, const void *router_weights, uint64_t router_weights_offset,
-                                  const void *router_scales, uint64_t router_scales_offset, const void *router_biases,
-                                  uint64_t router_biases_offset, const void *router_x, const void *effective_scale,
-                                  uint64_t effective_scale_offset, const void *per_expert_scale, uint64_t per_expert_scale_offset,
-                                  const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
-                                  const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
-                                  void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype,
-                                  const void *shared_x, const tf_projection *shared_gate, const tf_projection *shared_up,
-                                  const tf_projection *shared_down, void *shared_y, void *shared_scratch_gate, void *shared_scratch_up,
-                                  void *shared_scratch_act) {
+}  // extern "C"
+
+namespace {
+
+// tf_moe_decode_step_shared; with `post` (the post-attention setup that makes router_x, x and shared_x) the setup runs in the
+// prologue of the first launch when that launch is the shared one (post->hidden_out must then differ from post->hidden),
+// as a launch of its own ahead of everything otherwise.
+struct PostAttnCall {
+    const void *hidden, *attn;
+    void *hidden_out;
+    const void *w_post_attn, *w_pre_ffn, *w_pre_ffn2;
+    uint64_t w_post_attn_offset, w_pre_ffn_offset, w_pre_ffn2_offset;
+    float eps;
+};
+int32_t decode_step_shared_impl(tf_ctx *ctx, tf_stream stream, const void *router_weights, uint64_t router_weights_offset,
+                                const void *router_scales, uint64_t router_scales_offset, const void *router_biases,
+                                uint64_t router_biases_offset, const void *router_x, const void *effective_scale,
+                                uint64_t effective_scale_offset, const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                                const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
+                                void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype,
+                                const void *shared_x, const tf_projection *shared_gate, const tf_projection *shared_up,
+                                const tf_projection *shared_down, void *shared_y, void *shared_scratch_gate, void *shared_scratch_up,
+                                void *shared_scratch_act, const PostAttnCall *post) {
     TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "moe_decode_step_shared: null context");
     TF_REQUIRE(ctx, shared_x && shared_gate && shared_up && shared_down && shared_y && shared_scratch_gate && shared_scratch_up && shared_scratch_act,
                TF_ERR_INVALID_ARGUMENT, "moe_decode_step_shared: null shared-expert argument");
@@ -1083,6 +1226,36 @@ int32_t tf_moe_decode_step_shared(tf_ctx *ctx, tf_stream stream, const void *rou
     const bool ride_ok = proj16 && aligned16(shared_x) && aligned16(shared_scratch_act) && aligned(shared_scratch_gate, 2) && aligned(shared_scratch_up, 2) &&
                          aligned(shared_y, 2) && sdim > 1024 && sdim <= (uint32_t)XStage::kMaxK && sf > 1024 && sf <= (uint32_t)XStage::kMaxK &&
                          plan_up.rt == 2 && plan_up.np == 3 && plan_down.rt == 2 && plan_down.np == 3;
+    // the setup inside the first launch: that launch must be the block-per-expert router with the shared rows riding along,
+    // every row and norm weight must move in 16-byte pieces, and nobody may write what other blocks still read
+    PostAttnFuseArgs fuse = {};
+    bool fuse_ok = false;
+    if (post) {
+        TF_REQUIRE(ctx, post->hidden && post->attn && post->hidden_out && post->w_post_attn && post->w_pre_ffn && post->w_pre_ffn2 && router_x && x,
+                   TF_ERR_INVALID_ARGUMENT, "moe_decode_step_shared_post_attn: null argument");
+        TF_REQUIRE(ctx, sdim == d, TF_ERR_DIMENSION_MISMATCH, "moe_decode_step_shared_post_attn: the shared expert reads %u values, the layer has %u", sdim, d);
+        fuse = {static_cast<const half_t *>(post->hidden), static_cast<const half_t *>(post->attn), static_cast<half_t *>(post->hidden_out),
+                static_cast<half_t *>(const_cast<void *>(shared_x)), static_cast<half_t *>(const_cast<void *>(x)),
+                static_cast<half_t *>(const_cast<void *>(router_x)),
+                reinterpret_cast<const uint16_t *>(at(post->w_post_attn, post->w_post_attn_offset)),
+                reinterpret_cast<const uint16_t *>(at(post->w_pre_ffn, post->w_pre_ffn_offset)),
+                reinterpret_cast<const uint16_t *>(at(post->w_pre_ffn2, post->w_pre_ffn2_offset)), post->eps};
+        const void *outs[4] = {fuse.hidden_out, fuse.dense_x, fuse.routed_x, fuse.router_x};
+        bool distinct = true;
+        for (int i = 0; i < 4; ++i) distinct = distinct && outs[i] != (const void *)fuse.hidden && outs[i] != (const void *)fuse.attn;
+        const bool router_fast = router_weights && effective_scale && aligned16(at(router_weights, router_weights_offset)) &&
+                                 aligned16(at(effective_scale, effective_scale_offset)) && d <= 4096 && d % TF_GROUP_SIZE == 0 && num_experts > 0 &&
+                                 num_experts <= 256;
+        fuse_ok = ride_ok && router_fast && distinct && aligned16(fuse.hidden) && aligned16(fuse.attn) && aligned16(fuse.hidden_out) &&
+                  aligned16(fuse.dense_x) && aligned16(fuse.routed_x) && aligned16(fuse.router_x) && aligned16(fuse.w_post_attn) &&
+                  aligned16(fuse.w_pre_ffn) && aligned16(fuse.w_pre_ffn2);
+        if (!fuse_ok) {
+            const int32_t rc = post_attn_setup_to(ctx, stream, post->hidden, post->hidden_out, post->attn, const_cast<void *>(shared_x), const_cast<void *>(x),
+                                                  const_cast<void *>(router_x), post->w_post_attn, post->w_post_attn_offset, post->w_pre_ffn,
+                                                  post->w_pre_ffn_offset, post->w_pre_ffn2, post->w_pre_ffn2_offset, d, post->eps);
+            if (rc != TF_OK) return rc;
+        }
+    }
     if (!ride_ok) {
         const int32_t rc = tf_shared_expert_int4(ctx, stream, shared_x, 0, (uint64_t)sdim * 2, shared_gate, shared_up, shared_down, shared_y, 0,
                                                  (uint64_t)sdim * 2, shared_scratch_gate, 0, (uint64_t)sf * 2, shared_scratch_up, 0, (uint64_t)sf * 2,
@@ -1105,7 +1278,50 @@ int32_t tf_moe_decode_step_shared(tf_ctx *ctx, tf_stream stream, const void *rou
     return decode_step_impl(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset, router_biases,
                             router_biases_offset, router_x, effective_scale, effective_scale_offset, per_expert_scale,
                             per_expert_scale_offset, expert_pool, expert_pool_stride, num_experts, routed_offsets, x, acts, residual, y,
-                            out_indices, out_weights, d, f, top_k, scale_dtype, ctx->router_logits, true, &ride);
+                            out_indices, out_weights, d, f, top_k, scale_dtype, ctx->router_logits, true, &ride, fuse_ok ? &fuse : nullptr);
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t tf_moe_decode_step_shared(tf_ctx *ctx, tf_stream stream, const void *router_weights, uint64_t router_weights_offset,
+                                  const void *router_scales, uint64_t router_scales_offset, const void *router_biases,
+                                  uint64_t router_biases_offset, const void *router_x, const void *effective_scale,
+                                  uint64_t effective_scale_offset, const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                                  const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                  const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
+                                  void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype,
+                                  const void *shared_x, const tf_projection *shared_gate, const tf_projection *shared_up,
+                                  const tf_projection *shared_down, void *shared_y, void *shared_scratch_gate, void *shared_scratch_up,
+                                  void *shared_scratch_act) {
+    return decode_step_shared_impl(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset, router_biases,
+                                   router_biases_offset, router_x, effective_scale, effective_scale_offset, per_expert_scale,
+                                   per_expert_scale_offset, expert_pool, expert_pool_stride, num_experts, routed_offsets, x, acts, residual, y,
+                                   out_indices, out_weights, d, f, top_k, scale_dtype, shared_x, shared_gate, shared_up, shared_down, shared_y,
+                                   shared_scratch_gate, shared_scratch_up, shared_scratch_act, nullptr);
+}
+
+int32_t tf_moe_decode_step_shared_post_attn(tf_ctx *ctx, tf_stream stream, const void *hidden, const void *attn, void *hidden_out,
+                                            const void *post_attention_weight, uint64_t post_attention_weight_offset,
+                                            const void *pre_ffn_weight, uint64_t pre_ffn_weight_offset, const void *pre_ffn2_weight,
+                                            uint64_t pre_ffn2_weight_offset, float eps, const void *router_weights,
+                                            uint64_t router_weights_offset, const void *router_scales, uint64_t router_scales_offset,
+                                            const void *router_biases, uint64_t router_biases_offset, void *router_x,
+                                            const void *effective_scale, uint64_t effective_scale_offset, const void *per_expert_scale,
+                                            uint64_t per_expert_scale_offset, const void *expert_pool, uint64_t expert_pool_stride,
+                                            uint32_t num_experts, const tf_expert_offsets *routed_offsets, void *routed_x, void *acts,
+                                            const void *residual, void *y, void *out_indices, void *out_weights, uint32_t d, uint32_t f,
+                                            uint32_t top_k, tf_dtype scale_dtype, void *dense_x, const tf_projection *shared_gate,
+                                            const tf_projection *shared_up, const tf_projection *shared_down, void *shared_y,
+                                            void *shared_scratch_gate, void *shared_scratch_up, void *shared_scratch_act) {
+    const PostAttnCall post = {hidden, attn, hidden_out, post_attention_weight, pre_ffn_weight, pre_ffn2_weight, post_attention_weight_offset,
+                               pre_ffn_weight_offset, pre_ffn2_weight_offset, eps};
+    return decode_step_shared_impl(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset, router_biases,
+                                   router_biases_offset, router_x, effective_scale, effective_scale_offset, per_expert_scale,
+                                   per_expert_scale_offset, expert_pool, expert_pool_stride, num_experts, routed_offsets, routed_x, acts, residual, y,
+                                   out_indices, out_weights, d, f, top_k, scale_dtype, dense_x, shared_gate, shared_up, shared_down, shared_y,
+                                   shared_scratch_gate, shared_scratch_up, shared_scratch_act, &post);
 }
 
 int32_t tf_shared_expert_int4(tf_ctx *ctx, tf_stream stream, const void *x, uint64_t x_offset, uint64_t x_length,

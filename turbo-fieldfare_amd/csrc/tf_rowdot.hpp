@@ -231,6 +231,17 @@ struct XNormStage {
         }
     }
 
+    // the norm weight only: the caller fills xr itself
+    __device__ __forceinline__ void request_weight(const uint16_t *w_bf16, int k) {
+        const int pieces = k >> 3;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int piece = threadIdx.x + 256 * i;
+            wr[i] = u32x4{0u, 0u, 0u, 0u};
+            if (piece < pieces) wr[i] = load16(w_bf16 + piece * 8);
+        }
+    }
+
     // partial: 4 floats of LDS
     __device__ __forceinline__ void publish(float eps, int k, u32x4 *xa, float *xsum, float *partial) const {
         float acc = 0.0f;
