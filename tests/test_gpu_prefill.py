@@ -117,7 +117,10 @@ def device_grouping(idx, wts_bits, T, top_k, E):
     return dict(sorted_pairs=sp, offsets=offs, counts=cnts, chunks=chunks, n_chunks=nch, cap=cap, keep=(d_idx, d_w))
 
 
-@pytest.mark.parametrize("T,top_k,E", [(4, 3, 6), (32, 8, 128), (300, 8, 128), (2048, 8, 128), (16, 8, 16)])
+# one 256-thread block up to 32 tokens, three launches over up to 64 token segments beyond (ragged last batches, an odd top-k,
+# more tokens than 64 segments of 32, the largest expert count)
+@pytest.mark.parametrize("T,top_k,E", [(4, 3, 6), (32, 8, 128), (33, 8, 128), (100, 5, 7), (300, 8, 128), (2048, 8, 128), (2049, 8, 200),
+                                       (4096, 8, 128), (4100, 8, 256), (16, 8, 16)])
 def test_device_grouping_equals_host_grouping(T, top_k, E):
     rng = np.random.default_rng(T + E)
     p = 1.0 / np.arange(1, E + 1) ** 1.1
