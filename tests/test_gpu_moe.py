@@ -489,13 +489,13 @@ def _decode_step_case(d, f, num_experts, seed):
                 residual_bits=refcases.normal_f16(d, seed + 9))
 
 
-def _decode_step_call(k, t, c, d, f, num_experts, outs):
+def _decode_step_call(k, t, c, d, f, num_experts, outs, scale_dtype=tfk.TF_BF16):
     idx, wts, acts, y = outs
     off = tfk.ExpertOffsets(*c["off"].as_tuple())
     return k.lib.tf_moe_decode_step(k.handle, None, t["rW"].data_ptr(), 0, t["rS"].data_ptr(), 0, t["rB"].data_ptr(), 0, t["x"].data_ptr(),
                                     t["eff"].data_ptr(), 0, t["gain"].data_ptr(), 0, t["pool"].data_ptr(), c["stride"], num_experts,
                                     off, t["x"].data_ptr(), acts.data_ptr(), t["res"].data_ptr(), y.data_ptr(), idx.data_ptr(),
-                                    wts.data_ptr(), d, f, 8, tfk.TF_BF16)
+                                    wts.data_ptr(), d, f, 8, scale_dtype)
 
 
 def _decode_step_tensors(c):
