@@ -377,3 +377,77 @@ def test_layer_tail_inside_the_next_qkv_launch_equals_the_two_calls(n, q_rows, k
         assert tfo.rel_error(tfo.from_f16_bits(got), tfo.from_f16_bits(want)) < TOL
     assert lib.tf_fused_layer_tail_norm_qkv_gemv(h, None, h2_ptr, d_sh.data_ptr(), hid.data_ptr(), None, d_w1.data_ptr(), 0, d_w2.data_ptr(), 0,
                                                  d_w3.data_ptr(), 0, EPS, LAYER_SCALAR, d_nw.data_ptr(), 0, EPS, *qkv, *out_args) == tfk.TF_ERR_INVALID_ARGUMENT
+
+
+def test_folded_stages_replayed_from_a_graph():
+    # the two launches that fold a stage into their prologue (post-attention setup + decode step with the shared expert, then the
+    # layer tail + input norm + q/k/v of the next layer), captured into a HIP graph and replayed three times with eager calls of
+    # the same entry points in between: every replay must leave what the eager sequence leaves
+    import torch
+    d, f, fs, q_rows, kv_rows = D, F_MOE, F_SHARED, NQ * HD, NKV * HD
+    c = M._decode_step_case(d, f, E, 0x6A11)
+    shared = dict(gate=refcases.synthetic_int4(fs, d, 0x71, "sg"), up=refcases.synthetic_int4(fs, d, 0x72, "su"),
+                  down=refcases.synthetic_int4(d, fs, 0x73, "sd"))
+    mats = [refcases.synthetic_int4(r, d, 0x97 + i, "qkv"[i]) for i, r in enumerate((q_rows, kv_rows, kv_rows))]
+    rng = np.random.default_rng(0x74)
+    norm = [dev(tfo.bf16_bits_array(1.0 + 0.1 * rng.standard_normal(d).astype(np.float32))) for _ in range(7)]
+    hidden_bits, attn_bits = refcases.normal_f16(d, 0x75), refcases.normal_f16(d, 0x76)
+    k = ctx()
+    lib, h = k.lib, k.handle
+    t = M._decode_step_tensors(c)
+    st = {n: [dev(a) for a in shared[n]] for n in shared}
+    gate, up, down = (tfk.projection(*st[n], r, cc) for n, r, cc in (("gate", fs, d), ("up", fs, d), ("down", d, fs)))
+    tq = [[dev(a) for a in m] for m in mats]
+    qkv = []
+    for m in tq:
+        qkv += [m[0].data_ptr(), 0, m[1].data_ptr(), 0, m[2].data_ptr(), 0]
+    off = tfk.ExpertOffsets(*c["off"].as_tuple())
+    d_attn, hidden = dev(attn_bits), dev(hidden_bits)
+    names = ("mid", "next_hidden", "dense_x", "routed_x", "router_x", "y", "sy")
+    sizes = dict(q=q_rows, kk=kv_rows, v=kv_rows, sg=fs, su=fs, sa=fs, acts=8 * f)
+
+    def fresh():
+        b = {n: dev(np.full(d, 0x7BFF, np.uint16)) for n in names}
+        b.update({n: dev(np.full(s_, 0x7BFF, np.uint16)) for n, s_ in sizes.items()})
+        b["idx"], b["wts"] = zeros_bytes(32), zeros_bytes(16)
+        return b
+
+    def run(b, stream):
+        p = lambda n: b[n].data_ptr()
+        k.check(lib.tf_moe_decode_step_shared_post_attn(h, stream, hidden.data_ptr(), d_attn.data_ptr(), p("mid"), norm[0].data_ptr(), 0, norm[1].data_ptr(), 0,
+                                                        norm[2].data_ptr(), 0, EPS, t["rW"].data_ptr(), 0, t["rS"].data_ptr(), 0, t["rB"].data_ptr(), 0,
+                                                        p("router_x"), t["eff"].data_ptr(), 0, t["gain"].data_ptr(), 0, t["pool"].data_ptr(), c["stride"], E, off,
+                                                        p("routed_x"), p("acts"), t["res"].data_ptr(), p("y"), p("idx"), p("wts"), d, f, 8, tfk.TF_BF16,
+                                                        p("dense_x"), C.byref(gate), C.byref(up), C.byref(down), p("sy"), p("sg"), p("su"), p("sa")))
+        k.check(lib.tf_fused_layer_tail_norm_qkv_gemv(h, stream, p("y"), p("sy"), p("mid"), p("next_hidden"), norm[3].data_ptr(), 0, norm[4].data_ptr(), 0,
+                                                      norm[5].data_ptr(), 0, EPS, LAYER_SCALAR, norm[6].data_ptr(), 0, EPS, *qkv, p("q"), 0, p("kk"), 0, p("v"), 0,
+                                                      q_rows, kv_rows, d, tfk.TF_BF16))
+
+    def read(b):
+        return {n: host(b[n], np.uint16) for n in list(names) + ["q", "kk", "v", "sa", "acts"]}
+
+    eager = fresh()
+    run(eager, None)
+    k.synchronize()
+    want = read(eager)
+    assert not np.all(want["q"] == 0x7BFF) and not np.all(want["next_hidden"] == 0x7BFF)
+    side = torch.cuda.Stream()
+    gb = fresh()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            run(gb, side.cuda_stream)
+    for replay in range(3):
+        for buf in gb.values():
+            buf.fill_(0x55) if buf.dtype == torch.uint8 else buf.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        got = read(gb)
+        for n in want:
+            assert np.array_equal(got[n], want[n]), (replay, n)
+        again = fresh()                   # eager work between the replays
+        run(again, None)
+        k.synchronize()
+        for n, v in read(again).items():
+            assert np.array_equal(v, want[n]), (replay, n)
