@@ -217,15 +217,20 @@ __global__ __launch_bounds__(256, 2) void qmm_dense_geglu_kernel(DenseGegluArgs 
 
 // Block number -> (chunk, column tile) for the grouped kernels.  Workgroups go to the 8 XCDs round-robin by linear id and
 // each XCD has its own L2; the column tiles of one chunk all read the same activation rows, so they are given ids that
-// are congruent modulo 8: a run of 8 * tiles consecutive ids serves 8 chunks, one per XCD, and a chunk's activations are
-// fetched into one L2 once instead of into all eight.
+// are congruent modulo 8: a run of 16 * tiles consecutive ids serves 16 chunks, two consecutive ones per XCD, and a chunk's
+// activations are fetched into one L2 once instead of into all eight.  Two consecutive chunks on one XCD, because the chunks
+// of a popular expert follow each other in the work list and read the same weights: side by side in one L2 the second finds
+// what the first fetched (2048 tokens, Zipf routing: 0.362 -> 0.355 ms on one box, 0.361 -> 0.347 on another; four a run
+// measured slower again, 0.361).
 constexpr uint32_t kXcds = 8;
+constexpr uint32_t kChunksPerXcdRun = 2;
 __device__ __forceinline__ void chunk_and_tile(uint32_t id, uint32_t tiles, uint32_t &chunk, uint32_t &tile) {
-    const uint32_t run = kXcds * tiles;
-    const uint32_t within = id % run;
-    chunk = (id / run) * kXcds + within % kXcds;
-    tile = within / kXcds;
+    const uint32_t run = kXcds * kChunksPerXcdRun * tiles;
+    const uint32_t within = id % run, xcd = within % kXcds, local = within / kXcds;   // local: 0 .. kChunksPerXcdRun * tiles - 1
+    chunk = (id / run) * (kXcds * kChunksPerXcdRun) + xcd * kChunksPerXcdRun + local / tiles;
+    tile = local % tiles;
 }
+constexpr uint32_t kChunkRun = kXcds * kChunksPerXcdRun;
 
 // ------------------------------------------------------------------------------------------------ grouped phase 1
 // Block = one chunk (<= 128 sorted pairs of one expert) x 32 NW intermediate columns.  A wave's first column tile is 32
@@ -432,7 +437,7 @@ int32_t launch_grouped_phase1_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTabl
                                    const ChunkList &cl, uint32_t n_chunks_upper, const tf_prefill_pair *pairs,
                                    const half_t *hidden, long hidden_stride, half_t *acts, uint32_t acts_pair_base, int d, int f,
                                    tf_dtype sd, const DenseRide *ride) {
-    const uint32_t grouped = (uint32_t)((f + kP1BN - 1) / kP1BN) * ((n_chunks_upper + kXcds - 1) / kXcds * kXcds);
+    const uint32_t grouped = (uint32_t)((f + kP1BN - 1) / kP1BN) * ((n_chunks_upper + kChunkRun - 1) / kChunkRun * kChunkRun);
     const GroupedP1Args a = {tab, off, cl, pairs, hidden, hidden_stride, acts, acts_pair_base, d, f};
     if (ride) {
         // the shared expert's gate / up / GeGLU tiles ahead of the grouped tiles (the full-height, longest tiles first), padded
@@ -451,7 +456,7 @@ int32_t launch_grouped_phase1_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTabl
 int32_t launch_grouped_down_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off,
                                  const ChunkList &cl, uint32_t n_chunks_upper, const tf_prefill_pair *pairs, const half_t *acts,
                                  uint32_t acts_pair_base, half_t *route_partials, int d, int f, int top_k, tf_dtype sd, const DenseRide *ride) {
-    const uint32_t grouped = (uint32_t)((d + kDownBN - 1) / kDownBN) * ((n_chunks_upper + kXcds - 1) / kXcds * kXcds);
+    const uint32_t grouped = (uint32_t)((d + kDownBN - 1) / kDownBN) * ((n_chunks_upper + kChunkRun - 1) / kChunkRun * kChunkRun);
     const GroupedDownArgs a = {tab, off, cl, pairs, acts, acts_pair_base, route_partials, d, f, top_k};
     if (ride) {
         const tf_projection *dn = ride->down;   // ride->y: 16-byte aligned rows of whole 16-byte pieces (dense_ride_ok)
