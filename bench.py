@@ -33,15 +33,21 @@ def int4_matrix_bytes(rows, cols):
 
 # per-unit algorithmic bytes (what one launch must move at least once)
 ROUTER_BYTES = E * D + 2 * E * (D // 64) * 2 + D * 2 + D * 2 + E * 2 + TOPK * 4 + TOPK * 2   # W + s/b + hidden + eff + gains + outputs
-# HBM bytes one phase-1 launch moves, from hardware counters (profiles/bench_hbm_traffic_counters.txt): FETCH_SIZE 8895.6 KiB
-# x 2.0 (the factor a plain 1 GiB copy calibrates) + WRITE_SIZE 22.1 KiB x 1.0.  Collected before the kernel's weight loads
-# became non-temporal; what it must fetch is the same.
-PHASE1_TRAFFIC_BYTES = int(8895.6 * 1024 * 1.9999 + 22.1 * 1024)
+# HBM bytes one fused phase-1 launch moves, from hardware counters of `bench.py --only-decode-step` (two rocprofv3 --pmc runs,
+# FETCH_SIZE then WRITE_SIZE; profiles/decode_step_counters.txt gives the commands, the raw KiB per dispatch and the factors a
+# plain copy of known size calibrates).  None until such a profile of the current kernels is on file.
+PHASE1_TRAFFIC_BYTES = None
+PHASE1_TRAFFIC_FROM = None
 PHASE1_BYTES = TOPK * 2 * int4_matrix_bytes(F_MOE, D) + D * 2 + TOPK * F_MOE * 2             # gate+up of 8 experts + x + acts out
 PHASE2_BYTES = TOPK * int4_matrix_bytes(D, F_MOE) + TOPK * F_MOE * 2 + TOPK * 2 + D * 2 + D * 2   # down of 8 + acts in + w + residual + y
 STEP_BYTES = ROUTER_BYTES + PHASE1_BYTES + PHASE2_BYTES
 SHARED_BYTES = 2 * int4_matrix_bytes(F_SHARED, D) + int4_matrix_bytes(D, F_SHARED) + D * 2 + 4 * F_SHARED * 2 + D * 2
 LM_HEAD_BYTES = int4_matrix_bytes(VOCAB, D) + D * 2 + 4
+
+
+# (blocks, threads per block) of the decode step's three launches at the production shape: one block per router row, one wave
+# per two-row gate/up tile, eight down rows per block of eight waves
+STEP_GRID_SHAPES = ((E, 256), (TOPK * (F_MOE // 2) // 4, 256), (D // 8, 512))
 
 
 def expert_layout():
@@ -61,22 +67,87 @@ def bf16_bits_cuda(t):
     return t.to(torch.bfloat16).view(torch.int16)
 
 
-def make_layer(torch, gen, offs, stride):
-    """One layer's resident weights on the device: expert pool [E, stride] + int8 router."""
-    pool = torch.randint(0, 256, (E, stride), dtype=torch.uint8, device="cuda", generator=gen)
+# ---- the reference's seeded streams (Sources/TurboFieldfareValidation/Support/PRNG/SplitMix64.swift:11-23, SeedTree.swift:12-19),
+# evaluated in counter form on the device: draw number i (from 1) of a stream with seed s is mix(s + i * GAMMA), so a whole
+# tensor is drawn at once and equals the sequential generator draw for draw.
+_M64 = (1 << 64) - 1
+
+
+def _s64(v):
+    """A 64-bit pattern as the signed value torch.int64 holds."""
+    v &= _M64
+    return v - (1 << 64) if v >= (1 << 63) else v
+
+
+def seed_tree_key(root, label):
+    """SeedTree(root).key(label): the SplitMix64 seed root ^ FNV-1a(label)."""
+    h = 0xCBF29CE484222325
+    for byte in label.encode("utf-8"):
+        h = ((h ^ byte) * 0x100000001B3) & _M64
+    return (root ^ h) & _M64
+
+
+def _lsr(z, k):
+    return (z >> k) & ((1 << (64 - k)) - 1)
+
+
+def splitmix64_draws(torch, seed, first, count, device="cuda"):
+    """Draws first+1 ... first+count of SplitMix64(seed) as the int64 bit patterns of the UInt64 values."""
+    i = torch.arange(first + 1, first + count + 1, dtype=torch.int64, device=device)
+    z = i * _s64(0x9E3779B97F4A7C15) + _s64(seed)                 # two's-complement wrap = the reference's &+ / &*
+    z = (z ^ _lsr(z, 30)) * _s64(0xBF58476D1CE4E5B9)
+    z = (z ^ _lsr(z, 27)) * _s64(0x94D049BB133111EB)
+    return z ^ _lsr(z, 31)
+
+
+def splitmix64_uniform(torch, seed, first, count, lo, hi, device="cuda"):
+    """SplitMix64.uniform(lo, hi) for draws first+1 ... first+count: lo + (hi - lo) * Float(next >> 40) / 2^24 in fp32."""
+    u = _lsr(splitmix64_draws(torch, seed, first, count, device), 40).to(torch.float32) / 16777216.0
+    lo32 = np.float32(lo)
+    return float(np.float32(hi) - lo32) * u + float(lo32)          # (hi - lo) formed in fp32, as the reference's Float arithmetic does
+
+
+def splitmix64_nibble_bytes(torch, seed, nbytes, device="cuda", chunk=1 << 25):
+    """nbytes packed int4 bytes: nibble j = next() & 0xF, low nibble first (byte b = draws 2b+1 and 2b+2)."""
+    out = torch.empty(nbytes, dtype=torch.uint8, device=device)
+    for b0 in range(0, nbytes, chunk):
+        n = min(chunk, nbytes - b0)
+        nib = (splitmix64_draws(torch, seed, 2 * b0, 2 * n, device) & 0xF).view(n, 2)
+        out[b0:b0 + n] = (nib[:, 0] | (nib[:, 1] << 4)).to(torch.uint8)
+    return out
+
+
+def splitmix64_normal_f16(torch, seed, count, device="cuda"):
+    """count N(0,1) values by Box-Muller on `uniform`: value j = sqrt(-2 ln(1 - u1)) cos(2 pi u2) with (u1, u2) = draws 2j+1, 2j+2
+    of uniform(0, 1); rounded to fp16."""
+    u = splitmix64_uniform(torch, seed, 0, 2 * count, 0.0, 1.0, device).view(count, 2)
+    r = torch.sqrt(-2.0 * torch.log1p(-u[:, 0]))
+    return (r * torch.cos(6.283185307179586 * u[:, 1])).to(torch.float16)
+
+
+BENCH_ROOT_SEED = 0x7F1E1DFA      # SeedTree root of every stream below
+
+
+def make_layer_seeded(torch, layer, offs, stride):
+    """One layer's resident weights drawn as the measurement plan of the reference-side survey states: uniform nibbles
+    (next() & 0xF, low nibble first), scale ~U(0.005, 0.02) and bias ~U(-0.1, 0.1) rounded to bf16, every tensor from a
+    SeedTree stream of its own label.  Router: 8-bit weights (next() & 0xFF), scale ~U(0.0002, 0.0008), bias ~U(-0.1, 0)."""
+    key = lambda what: seed_tree_key(BENCH_ROOT_SEED, f"bench-layer{layer}-{what}")
+    pool = splitmix64_nibble_bytes(torch, key("expert-nibbles"), E * stride).view(E, stride)
     shapes = ((F_MOE, D), (F_MOE, D), (D, F_MOE))
     for p, (rows, cols) in enumerate(shapes):
         n = rows * (cols // 64)
-        for j, (lo, hi) in ((1, (0.005, 0.02)), (2, (-0.1, 0.1))):
-            vals = torch.rand((E, n), device="cuda", generator=gen) * (hi - lo) + lo
+        for j, (what, lo, hi) in ((1, ("scales", 0.005, 0.02)), (2, ("biases", -0.1, 0.1))):
+            vals = splitmix64_uniform(torch, key(f"{('gate', 'up', 'down')[p]}-{what}"), 0, E * n, lo, hi).view(E, n)
             o = offs[3 * p + j]
             pool[:, o:o + 2 * n] = bf16_bits_cuda(vals).view(torch.uint8).view(E, 2 * n)
+    uni = lambda what, n, lo, hi: splitmix64_uniform(torch, key(what), 0, n, lo, hi)
     router = dict(
-        W=torch.randint(0, 256, (E, D), dtype=torch.uint8, device="cuda", generator=gen),
-        S=bf16_bits_cuda(torch.rand((E, D // 64), device="cuda", generator=gen) * 0.0006 + 0.0002),
-        B=bf16_bits_cuda(torch.rand((E, D // 64), device="cuda", generator=gen) * -0.1),
-        eff=bf16_bits_cuda((torch.rand(D, device="cuda", generator=gen) + 0.5) / (D ** 0.5)),
-        gain=bf16_bits_cuda(torch.rand(E, device="cuda", generator=gen) * 0.8 + 0.6),
+        W=(splitmix64_draws(torch, key("router-weights"), 0, E * D) & 0xFF).to(torch.uint8).view(E, D),
+        S=bf16_bits_cuda(uni("router-scales", E * (D // 64), 0.0002, 0.0008).view(E, D // 64)),
+        B=bf16_bits_cuda(uni("router-biases", E * (D // 64), -0.1, 0.0).view(E, D // 64)),
+        eff=bf16_bits_cuda(uni("router-effective-scale", D, 0.5, 1.5) / (D ** 0.5)),
+        gain=bf16_bits_cuda(uni("router-per-expert-scale", E, 0.6, 1.4)),
     )
     return pool, router
 
@@ -88,6 +159,18 @@ def make_int4(torch, gen, rows, cols):
     return W, S, B
 
 
+def profiler_attached():
+    """True when a rocprofiler tool library rides in this process (rocprofv3 preloads it and names it in the environment)."""
+    env = " ".join(os.environ.get(v, "") for v in ("LD_PRELOAD", "ROCP_TOOL_LIBRARIES", "ROCPROFILER_REGISTER_FORCE_LOAD", "ROCPROF_OUTPUT_PATH"))
+    if "rocprof" in env.lower():
+        return True
+    try:
+        with open("/proc/self/maps") as f:
+            return any("rocprofiler-sdk-tool" in line or "librocprofiler" in line for line in f)
+    except OSError:
+        return False
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -96,12 +179,17 @@ def main():
     ap.add_argument("--layers", type=int, default=4, help="layer replicas the steps rotate through")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip lm_head / GEMV / shared-expert side measurements")
-    ap.add_argument("--no-layer-chain", action="store_true", help="skip the whole-decoder-layer graph (long under a counter-collecting profiler)")
+    ap.add_argument("--no-layer-chain", action="store_true", help="skip the whole-decoder-layer graph")
     ap.add_argument("--layer-chain-fork", action="store_true",
                     help="also replay the layer chain with the shared expert on a second captured stream (a graph that forks and joins; "
-                         "not part of the default run, and not meant to run under a profiler)")
+                         "not part of the default run; refused under a profiler)")
     ap.add_argument("--calibration-copy", action="store_true",
                     help="also run one plain 1 GiB device copy (a known-size reference for hardware byte counters)")
+    ap.add_argument("--only-decode-step", action="store_true",
+                    help="run nothing but the headline decode-step measurement (graph-replayed steps and the one- and two-stage chains) and "
+                         "print its JSON: the short program a profiler attributes the step's three kernels with")
+    ap.add_argument("--only-lm-head", action="store_true",
+                    help="run nothing but the lm_head measurements (configs[2]) and print their JSON")
     ap.add_argument("--only-small-m", type=int, nargs="+", metavar="M",
                     help="run nothing but the few-token routed-MoE measurement at these token counts and print its JSON "
                          "(a short program whose launches a profiler can attribute to one size)")
@@ -114,20 +202,34 @@ def main():
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         sys.exit(2)
+    sub_command = bool(args.only_decode_step or args.only_lm_head or args.only_small_m or args.only_prefill_2048)
+    if profiler_attached() and (not sub_command or args.layer_chain_fork):
+        # The all-sections run ended the GPU box twice under `rocprofv3 --kernel-trace --stats` (no output came back either time)
+        # and the cause has not been shown; the --only-* sub-commands run the same measurements one at a time and profile fine.
+        print("bench.py: refusing to run every section (or --layer-chain-fork) with a profiler attached; profile one of "
+              "--only-decode-step, --only-lm-head, --only-small-m M, --only-prefill-2048 instead", file=sys.stderr)
+        sys.exit(2)
 
     import torch
     tfk = importlib.import_module("turbo-fieldfare_amd")
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     torch.cuda.set_device(0)
     k = tfk.Context(0)
-    gen = torch.Generator(device="cuda")
+    gen = torch.Generator(device="cuda")       # side measurements (extras) draw from torch's generator
     gen.manual_seed(0x7F1E1DFA)
     offs, payload, stride = expert_layout()
     off = tfk.ExpertOffsets(*offs)
-    layers = [make_layer(torch, gen, offs, stride) for _ in range(args.layers)]
     global TIMING_STREAM
     side = torch.cuda.Stream()            # default priority; everything timed is recorded on it
     TIMING_STREAM = side
+    lib, h = k.lib, k.handle
+    if args.only_lm_head:
+        note("lm_head only")
+        print(json.dumps(head_extras(torch, tfk, k, gen, lib, h, side.cuda_stream)))
+        return
+    note("resident weights: SplitMix64 / SeedTree streams")
+    n_layers = 1 if (args.only_small_m or args.only_prefill_2048) else args.layers
+    layers = [make_layer_seeded(torch, li, offs, stride) for li in range(n_layers)]
     if args.only_small_m or args.only_prefill_2048:
         only = multi_token_extras(torch, tfk, k, gen, k.lib, k.handle, side.cuda_stream, layers[0], offs, stride,
                                   small_sizes=tuple(args.only_small_m or ()), small_only=not args.only_prefill_2048,
@@ -135,27 +237,27 @@ def main():
         print(json.dumps(only))
         return
     n_hidden = 64
-    hidden = torch.randn((n_hidden, D), device="cuda", generator=gen).to(torch.float16)
+    hidden = splitmix64_normal_f16(torch, seed_tree_key(BENCH_ROOT_SEED, "bench-hidden-states"), n_hidden * D).view(n_hidden, D)
     idx = torch.zeros((n_hidden, TOPK), dtype=torch.int32, device="cuda")
     wts = torch.zeros((n_hidden, TOPK), dtype=torch.float16, device="cuda")
     acts = torch.zeros(TOPK * F_MOE, dtype=torch.float16, device="cuda")
     residual = torch.zeros(D, dtype=torch.float16, device="cuda")
     y = torch.zeros((n_hidden, D), dtype=torch.float16, device="cuda")
-    lib, h = k.lib, k.handle
 
     import ctypes as C
 
-    def step(i, stream):
+    def step_args(i, stream):
         li, hi = i % args.layers, i % n_hidden
         pool, r = layers[li]
         hp = hidden.data_ptr() + hi * D * 2
         ip, wp = idx.data_ptr() + hi * TOPK * 4, wts.data_ptr() + hi * TOPK * 2
+        return (h, stream, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, hp, r["eff"].data_ptr(), 0, r["gain"].data_ptr(), 0,
+                pool.data_ptr(), stride, E, C.byref(off), hp, acts.data_ptr(), residual.data_ptr(), y.data_ptr() + hi * D * 2, ip, wp, D, F_MOE,
+                TOPK, tfk.TF_BF16)
+
+    def step(i, stream):
         # one call = router logits -> (top-8 + gate/up/GeGLU of the 8 chosen experts) -> down + weighted sum + residual
-        rc = lib.tf_moe_decode_step(h, stream, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, hp,
-                                    r["eff"].data_ptr(), 0, r["gain"].data_ptr(), 0, pool.data_ptr(), stride, E, C.byref(off),
-                                    hp, acts.data_ptr(), residual.data_ptr(), y.data_ptr() + hi * D * 2, ip, wp, D, F_MOE, TOPK,
-                                    tfk.TF_BF16)
-        if rc != 0:
+        if lib.tf_moe_decode_step(*step_args(i, stream)) != 0:
             raise RuntimeError("kernel call failed: " + k.last_error())
 
     def run_steps(first, count, stream):
@@ -192,58 +294,20 @@ def main():
     value = STEP_BYTES / (ms_per_step * 1e-3) / 1e9
     stream = side.cuda_stream
 
-    # the same loop launched call by call (no graph): what a host that encodes every step itself would see
-    note("decode step: eager launches")
-    with torch.cuda.stream(side):
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        run_steps(args.warmup, max(args.steps, 256), stream)
-        torch.cuda.synchronize()
-        ms_per_step_eager = (time.perf_counter() - t0) * 1e3 / max(args.steps, 256)
+    # ---- each kernel's share of the step: the step's first launch alone and its first two launches, replayed as chains of 64
+    # like the step itself (same operands, same rotation).  Launches on one stream run one after the other, so
+    # router = chain of 1, phase 1 = chain of 2 - chain of 1, phase 2 = step - chain of 2; each share includes the boundary
+    # to the launch before it.  No events sit between the kernels.
+    note("decode step: one- and two-stage chains")
 
-    # ---- latency floor of the step: three dependent launches of the step's grid shapes that move no data, plus the step's
-    # bytes at the rate a plain streaming read reaches in this run.  The step cannot go below that with three launches.
-    note("latency floor: empty launch chain, streaming read")
-    words = torch.zeros(8, dtype=torch.int32, device="cuda")
-    wp0 = words.data_ptr()
-
-    def empty_chain(i):
-        rc = lib.tf_bench_empty_launch(h, stream, E, 256, wp0, wp0 + 4)                          # router: one block per expert row
-        rc |= lib.tf_bench_empty_launch(h, stream, TOPK * (F_MOE // 2) // 4, 256, wp0 + 4, wp0 + 8)   # phase 1: 704 blocks
-        rc |= lib.tf_bench_empty_launch(h, stream, D // 8, 512, wp0 + 8, wp0)                     # phase 2: 352 blocks
-        assert rc == 0, k.last_error()
-    empty_chain_us = time_loop(torch, empty_chain, 64)
-    read_bufs = [torch.randint(0, 256, (400 << 20,), dtype=torch.uint8, device="cuda", generator=gen) for _ in range(2)]
-
-    def stream_read(i):
-        assert lib.tf_bench_stream_read(h, stream, read_bufs[i % 2].data_ptr(), 400 << 20, wp0 + 16) == 0, k.last_error()
-    read_us = time_loop(torch, stream_read, 10)
-    read_gbps = (400 << 20) / (read_us * 1e-6) / 1e9
-    del read_bufs
-    latency_floor_us = empty_chain_us + STEP_BYTES / (read_gbps * 1e9) * 1e6
-
-    # ---- per-kernel durations: the library brackets the step's three launches with HIP events on the launch stream
-    # (eager launches; a spin kernel is queued first so that the host is ahead of the GPU and the events bracket
-    # back-to-back execution, not host gaps).
-    note("decode step: per-kernel event brackets")
-    n_ev = min(args.steps, 128)
-    k.set_step_timing(True)
-    times = []
-    for i0 in range(0, n_ev, 8):
-        torch.cuda._sleep(int(2.4e9 * 0.002))
-        for i in range(i0, min(i0 + 8, n_ev)):
-            step(args.warmup + i, torch.cuda.current_stream().cuda_stream)
-            times.append(None)
-        times[-1] = k.last_step_timing()      # only the last step of a burst keeps its events
-    k.set_step_timing(False)
-    burst_last = [t for t in times if t is not None]
-    raw = [float(np.mean([t[j] for t in burst_last])) for j in range(3)]
-    t_empty = float(np.median([t[3] for t in burst_last]))     # an empty bracket, for reference
-    # Every bracket carries the same constant cost of its event packets.  The three kernels of a step depend on one
-    # another and so run back to back: in the timed region (no events) their durations add up to the step time, which
-    # fixes that constant.
-    per_bracket = max((sum(raw) - ms_per_step * 1e3) / 3.0, 0.0)
-    t_router, t_p1, t_p2 = (max(t - per_bracket, 1e-3) for t in raw)
+    def stages(n_stages):
+        def fn(i):
+            if lib.tf_bench_moe_decode_step_stages(*step_args(i, stream), n_stages) != 0:
+                raise RuntimeError("kernel call failed: " + k.last_error())
+        return fn
+    us_chain = {n: time_loop(torch, stages(n), 64) for n in (1, 2, 3)}
+    t_router, t_p1 = us_chain[1], us_chain[2] - us_chain[1]
+    t_p2 = ms_per_step * 1e3 - us_chain[2]
     p1_gbps = PHASE1_BYTES / (t_p1 * 1e-6) / 1e9
 
     out = {
@@ -254,29 +318,69 @@ def main():
         "config": {"workload": "configs[1]: routed MoE FFN decode step, batch 1, hidden 2816, int8 router 128x2816 + top-8, "
                                "8 of 128 int4 g64 experts (gate/up 704x2816, down 2816x704), GeGLU, weighted sum",
                    "layer_replicas": args.layers, "resident_expert_bytes": args.layers * E * stride,
-                   "algorithmic_bytes_per_step": STEP_BYTES},
+                   "algorithmic_bytes_per_step": STEP_BYTES,
+                   "inputs": "every tensor of the headline workload (expert pools, routers, hidden states) from SplitMix64 streams keyed by "
+                             f"SeedTree({BENCH_ROOT_SEED:#x}) labels: nibbles next() & 0xF low first, scale ~U(0.005,0.02), bias ~U(-0.1,0.1) as bf16, "
+                             "activations N(0,1) by Box-Muller as fp16; the side measurements in `extras` draw from torch's generator"},
         "roofline": {"bound": "hbm", "kernel": "phase1_long_kernel<2,3,bf16,fused top-8> (expert selection + gate/up/GeGLU of 8 experts)",
                      "achieved": round(p1_gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(p1_gbps / HBM_PEAK_GBPS, 4), "traffic": PHASE1_TRAFFIC_BYTES,
-                     "traffic_from": "rocprofv3 FETCH_SIZE x 2.0 + WRITE_SIZE of this kernel before its loads became non-temporal (same bytes to fetch)",
+                     "traffic_from": PHASE1_TRAFFIC_FROM,
                      "algorithmic_bytes_per_launch": PHASE1_BYTES, "avg_launch_us": round(t_p1, 3),
-                     "latency_floor_us": round(latency_floor_us, 3),
-                     "latency_floor": {"what": "three dependent launches of the step's grid shapes that move no data + the step's "
-                                               "algorithmic bytes at the plain streaming-read rate, both measured in this run",
-                                       "empty_three_launch_chain_us": round(empty_chain_us, 3),
-                                       "stream_read_GBps": round(read_gbps, 1), "stream_read_frac_of_peak": round(read_gbps / HBM_PEAK_GBPS, 4),
-                                       "step_us": round(ms_per_step * 1e3, 3),
-                                       "step_over_floor": round(ms_per_step * 1e3 / latency_floor_us, 3)}},
+                     "duration_from": "HIP events around graph replays on the launch stream: (chain of the step's first two launches) - (chain of "
+                                      "its first launch), 64 launches per graph, >= 50 ms per figure; includes the boundary to the router launch, so "
+                                      "the kernel's own duration in a profiler's trace is shorter by about that boundary",
+                     },
         "launch": f"HIP graph replay, {graph_steps} steps per graph; {len(rounds_ms)} rounds of {args.steps} steps, median round reported",
         "ms_per_step_wallclock_all_rounds": round(ms_per_step_wall, 6),
         "step_per_s": round(1e3 / ms_per_step, 1),
-        "ms_per_step_eager_launch": round(ms_per_step_eager, 6),
         "pct_hbm_peak": round(100.0 * value / HBM_PEAK_GBPS, 2),
         "kernels_us": {"router": round(t_router, 3), "phase1": round(t_p1, 3), "phase2": round(t_p2, 3),
-                       "event_bracket_overhead_subtracted": round(per_bracket, 3), "empty_bracket": round(t_empty, 3),
-                       "raw_brackets": [round(t, 3) for t in raw],
-                       "phase2_GBps": round(PHASE2_BYTES / (t_p2 * 1e-6) / 1e9, 1)},
+                       "how": "chains of the step's first 1, 2 and 3 launches replayed from graphs; differences of their times",
+                       "chain_us": {str(n): round(v, 3) for n, v in us_chain.items()},
+                       "phase1_GBps": round(p1_gbps, 1), "phase2_GBps": round(PHASE2_BYTES / (t_p2 * 1e-6) / 1e9, 1)},
     }
+    if args.only_decode_step:
+        print(json.dumps(out))
+        return
+
+    # the same loop launched call by call (no graph): what a host that encodes every step itself would see
+    note("decode step: eager launches")
+    with torch.cuda.stream(side):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        run_steps(args.warmup, max(args.steps, 256), stream)
+        torch.cuda.synchronize()
+        out["ms_per_step_eager_launch"] = round((time.perf_counter() - t0) * 1e3 / max(args.steps, 256), 6)
+
+    # ---- latency floor of the step: three dependent launches of the step's grid shapes that move no data, plus the step's
+    # bytes at the rate a plain streaming read reaches in this run.  The step cannot go below that with three launches.
+    note("latency floor: empty launch chain, streaming read")
+    words = torch.zeros(8, dtype=torch.int32, device="cuda")
+    wp0 = words.data_ptr()
+    shapes = STEP_GRID_SHAPES
+
+    def empty_chain(i):
+        rc = 0
+        for j, (blocks, threads) in enumerate(shapes):
+            rc |= lib.tf_bench_empty_launch(h, stream, blocks, threads, wp0 + 4 * j, wp0 + 4 * ((j + 1) % 3))
+        assert rc == 0, k.last_error()
+    empty_chain_us = time_loop(torch, empty_chain, 64)
+    read_bufs = [torch.randint(0, 256, (400 << 20,), dtype=torch.uint8, device="cuda", generator=gen) for _ in range(2)]
+
+    def stream_read(i):
+        assert lib.tf_bench_stream_read(h, stream, read_bufs[i % 2].data_ptr(), 400 << 20, wp0 + 16) == 0, k.last_error()
+    read_us = time_loop(torch, stream_read, 10)
+    read_gbps = (400 << 20) / (read_us * 1e-6) / 1e9
+    del read_bufs
+    latency_floor_us = empty_chain_us + STEP_BYTES / (read_gbps * 1e9) * 1e6
+    out["roofline"]["latency_floor_us"] = round(latency_floor_us, 3)
+    out["roofline"]["latency_floor"] = {"what": "three dependent launches of the step's grid shapes that move no data + the step's "
+                                                "algorithmic bytes at the plain streaming-read rate, both measured in this run",
+                                        "empty_three_launch_chain_us": round(empty_chain_us, 3),
+                                        "stream_read_GBps": round(read_gbps, 1), "stream_read_frac_of_peak": round(read_gbps / HBM_PEAK_GBPS, 4),
+                                        "step_us": round(ms_per_step * 1e3, 3),
+                                        "step_over_floor": round(ms_per_step * 1e3 / latency_floor_us, 3)}
 
     if args.calibration_copy:
         src = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda")
@@ -286,7 +390,8 @@ def main():
         del src, dst
     if not args.no_extras:
         note("extras: lm_head, GEMV, attention, shared expert")
-        out["extras"] = extras(torch, tfk, k, gen, lib, h, stream)
+        out["extras"] = head_extras(torch, tfk, k, gen, lib, h, stream)
+        out["extras"].update(extras(torch, tfk, k, gen, lib, h, stream))
         note("extras: small-M verification sizes, 2048-token prefill")
         out["extras"].update(multi_token_extras(torch, tfk, k, gen, lib, h, stream, layers[0], offs, stride))
         if not args.no_layer_chain:
@@ -356,8 +461,8 @@ def time_loop(torch, fn, iters, warmup=3, side=None):
 TIMING_STREAM = None     # the side stream every measurement records on (set in main)
 
 
-def extras(torch, tfk, k, gen, lib, h, stream):
-    """Side measurements on the other single-GPU configurations (not the headline value)."""
+def head_extras(torch, tfk, k, gen, lib, h, stream):
+    """configs[2]: the int4 lm_head, greedy and with fp32 logits."""
     res = {}
     # configs[2]: int4 lm_head 262144 x 2816 -> greedy argmax; two replicas alternate (830 MB > Infinity Cache)
     heads = [make_int4(torch, gen, VOCAB, D) for _ in range(2)]
@@ -387,7 +492,12 @@ def extras(torch, tfk, k, gen, lib, h, stream):
     res["lm_head_logits_fp32"] = {"us_per_call": round(us, 2), "GBps": round(nbytes / (us * 1e-6) / 1e9, 1),
                                   "frac_hbm_peak": round(nbytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)}
     del heads
+    return res
 
+
+def extras(torch, tfk, k, gen, lib, h, stream):
+    """Side measurements on the other single-GPU configurations (not the headline value)."""
+    res = {}
     # configs[0]: int4 GEMV 2112 x 2816, rotating over 192 replicas (644 MB)
     reps = 192
     W, S, B = make_int4(torch, gen, reps * F_SHARED, D)
@@ -785,7 +895,7 @@ def cpu_baseline(torch, layers, hidden, idx, wts, y, offs, stride, payload, args
     steps; also checks the device results of those steps against it."""
     from oracle import tfo
     off = tfo.ExpertOffsets(*offs)
-    n_sample = 12
+    n_sample = 64
     total_1, total_n, worst_rel, idx_match = 0.0, 0.0, 0.0, 0
     cores = max(1, min(os.cpu_count() or 1, 16))
     for sidx in range(n_sample):

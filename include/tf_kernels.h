@@ -20,8 +20,9 @@
  *     vector path, anything else a slower path with identical results;
  *   - calls only enqueue work on `stream` (one in-order stream = the reference's
  *     command queue); nothing blocks or allocates except tf_ctx_create,
- *     tf_ctx_reserve, tf_stream_synchronize and the tf_upload_* loaders, so every
- *     other entry point may be recorded into a HIP graph;
+ *     tf_ctx_reserve, tf_stream_synchronize, the tf_upload_* loaders and
+ *     tf_ctx_last_step_timing (which waits for the timed step's last event), so
+ *     every other entry point may be recorded into a HIP graph;
  *   - the caller owns every buffer; the library never frees caller memory;
  *   - where the reference traps on a broken precondition or throws, the call
  *     returns a negative tf_status and enqueues nothing.
@@ -798,17 +799,6 @@ int32_t tf_upload_packed_experts_layer(tf_ctx *ctx, tf_stream stream, const char
  * says which tensor lives where inside the range is read on the host (tf::gturbo::loadResidentIndex). */
 int32_t tf_upload_file_region(tf_ctx *ctx, tf_stream stream, const char *file_path, uint64_t file_offset, uint64_t bytes,
                               void *device_dst);
-
-/* ---- measurement helpers (no counterpart in the reference) ----------------------------------------------------- */
-/* A launch of `blocks` x `threads_per_block` that reads in_word[0] in every block and writes out_word[0] from one thread:
- * chained on a stream, what dependent launches of those shapes cost when they move no data (the latency floor of a
- * multi-launch step). */
-int32_t tf_bench_empty_launch(tf_ctx *ctx, tf_stream stream, uint32_t blocks, uint32_t threads_per_block,
-                              const void *in_word, void *out_word);
-/* A plain streaming read of `bytes` (multiple of 4096, 16-byte aligned) with the access pattern and cache policy of the
- * row streamers and no arithmetic: the read rate this part sustains, to hold the GEMV kernels against beside the
- * published peak. */
-int32_t tf_bench_stream_read(tf_ctx *ctx, tf_stream stream, const void *data, uint64_t bytes, void *out_word);
 
 #ifdef __cplusplus
 }

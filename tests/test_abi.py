@@ -7,8 +7,8 @@ import re
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
-def declared_symbols():
-    text = open(os.path.join(ROOT, "include", "tf_kernels.h")).read()
+def declared_symbols(header="tf_kernels.h"):
+    text = open(os.path.join(ROOT, "include", header)).read()
     text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
     return sorted(set(re.findall(r"\b(tf_[a-z0-9_]+)\s*\(", text)))
 
@@ -21,6 +21,10 @@ def test_library_exports_every_declared_symbol():
     for name in names:
         assert hasattr(lib, name), f"{name} declared in tf_kernels.h but not exported"
     assert sorted(tfk.EXPORTS) == names, "python binding table and header disagree"
+    # the measurement helpers live in a header of their own: the drop-in surface holds nothing without a reference counterpart
+    assert not [n for n in names if n.startswith("tf_bench_")]
+    bench = declared_symbols("tf_bench.h")
+    assert bench == sorted(tfk.BENCH_EXPORTS) and all(hasattr(lib, n) for n in bench)
     assert lib.tf_abi_version() == 1
     assert lib.tf_status_string(0) == b"ok"
     assert lib.tf_status_string(tfk.TF_ERR_UNAVAILABLE).startswith(b"unavailable")

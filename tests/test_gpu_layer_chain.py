@@ -327,6 +327,56 @@ def test_post_attention_setup_inside_the_decode_step_equals_the_two_calls(d, f, 
         assert np.max(np.abs(tfo.from_f16_bits(got) - tfo.from_f16_bits(ref))) <= 2e-3 * max(1.0, float(np.max(np.abs(tfo.from_f16_bits(ref)))))
 
 
+@pytest.mark.parametrize("in_place,misalign", [(False, 0), (True, 0), (False, 2)])
+def test_a_refused_decode_step_with_setup_and_shared_expert_launches_nothing(in_place, misalign):
+    # A broken precondition of the ROUTED step (topK != 8, too many experts, a null pool, an odd activation pointer) is found before
+    # the post-attention setup or the shared expert are enqueued, also where those run as launches of their own (in place, or a
+    # misaligned attention row): every output keeps its sentinel and the residual row its input.
+    d, f, fs = D, F_MOE, F_SHARED
+    c = M._decode_step_case(d, f, E, 0xBAD + misalign)
+    shared = dict(gate=refcases.synthetic_int4(fs, d, 0x71, "sg"), up=refcases.synthetic_int4(fs, d, 0x72, "su"),
+                  down=refcases.synthetic_int4(d, fs, 0x73, "sd"))
+    rng = np.random.default_rng(0x74)
+    weights = [tfo.bf16_bits_array(1.0 + 0.1 * rng.standard_normal(d).astype(np.float32)) for _ in range(3)]
+    hidden_bits, attn_bits = refcases.normal_f16(d, 0x75), refcases.normal_f16(d, 0x76)
+    k = ctx()
+    lib, h = k.lib, k.handle
+    t = M._decode_step_tensors(c)
+    st = {n: [dev(a) for a in shared[n]] for n in shared}
+    gate, up, down = (tfk.projection(*st[n], r, cc) for n, r, cc in (("gate", fs, d), ("up", fs, d), ("down", d, fs)))
+    d_w = [dev(w) for w in weights]
+    d_attn = dev(np.concatenate([np.zeros(misalign // 2, np.uint16), attn_bits]))
+    off = tfk.ExpertOffsets(*c["off"].as_tuple())
+    sentinel = 0x7BFF
+    outs = M._fresh_outs(d, f)
+    idx, wts, acts, y = outs
+    before = M._read_outs(outs, d, f)
+    sy, sg, su, sa = (dev(np.full(n, sentinel, np.uint16)) for n in (d, fs, fs, fs))
+    hidden = dev(hidden_bits)
+    hidden_out = hidden if in_place else dev(np.full(d, sentinel, np.uint16))
+    dense_x, routed_x, router_x = (dev(np.full(d, sentinel, np.uint16)) for _ in range(3))
+
+    def call(top_k=8, experts=E, pool=None, routed_ptr=None):
+        step = (t["rW"].data_ptr(), 0, t["rS"].data_ptr(), 0, t["rB"].data_ptr(), 0, router_x.data_ptr(), t["eff"].data_ptr(), 0,
+                t["gain"].data_ptr(), 0, t["pool"].data_ptr() if pool is None else pool, c["stride"], experts, off,
+                routed_x.data_ptr() if routed_ptr is None else routed_ptr, acts.data_ptr(), t["res"].data_ptr(),
+                y.data_ptr(), idx.data_ptr(), wts.data_ptr(), d, f, top_k, tfk.TF_BF16, dense_x.data_ptr(), C.byref(gate), C.byref(up), C.byref(down),
+                sy.data_ptr(), sg.data_ptr(), su.data_ptr(), sa.data_ptr())
+        return lib.tf_moe_decode_step_shared_post_attn(h, None, hidden.data_ptr(), d_attn.data_ptr() + misalign, hidden_out.data_ptr(),
+                                                       d_w[0].data_ptr(), 0, d_w[1].data_ptr(), 0, d_w[2].data_ptr(), 0, EPS, *step)
+
+    for kwargs in (dict(top_k=4), dict(experts=257), dict(pool=0), dict(routed_ptr=routed_x.data_ptr() + 1)):
+        assert call(**kwargs) == tfk.TF_ERR_INVALID_ARGUMENT, kwargs
+        k.synchronize()
+        assert np.array_equal(host(hidden, np.uint16), hidden_bits), kwargs
+        for buf in (sy, sg, su, sa, dense_x, routed_x, router_x) + (() if in_place else (hidden_out,)):
+            assert np.all(host(buf, np.uint16) == sentinel), kwargs
+        for a, b_ in zip(M._read_outs(outs, d, f), before):
+            assert np.array_equal(a, b_), kwargs
+    assert call() == tfk.TF_OK      # and the same buffers are accepted when the arguments are right
+    k.synchronize()
+
+
 @pytest.mark.parametrize("n,q_rows,kv_rows,in_place,misalign,sd", [(D, NQ * HD, NKV * HD, False, 0, tfk.TF_BF16), (D, NQ * HD, NKV * HD, False, 0, tfk.TF_FP16),
                                                                   (D, NQ * HD, NKV * HD, True, 0, tfk.TF_BF16), (D, NQ * HD, NKV * HD, False, 2, tfk.TF_BF16),
                                                                   (512, 96, 64, False, 0, tfk.TF_BF16), (4096, 130, 66, False, 0, tfk.TF_BF16)])

@@ -201,14 +201,21 @@ EXPORTS = {
     "tf_logit_softcap_softmax": (i32, [vp, vp, vp, vp, u32, C.c_float, i32]),
     "tf_sample": (i32, [vp, vp, vp, vp, u32, C.c_float, u32, C.c_float, u64, u32]),
     "tf_sample_topk64": (i32, [vp, vp, vp, vp, u32, C.c_float, C.c_float, u64]),
-    "tf_bench_empty_launch": (i32, [vp, vp, u32, u32, vp, vp]),
-    "tf_bench_stream_read": (i32, [vp, vp, vp, u64, vp]),
     "tf_upload_packed_experts_layer": (i32, [vp, vp, C.c_char_p, u64, u32, C.POINTER(u32), vp]),
     "tf_upload_file_region": (i32, [vp, vp, C.c_char_p, u64, u64, vp]),
     "tf_lm_head_greedy_int4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u32, u32, C.c_float, i32]),
     "tf_lm_head_logits_int4": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, u32, u32, C.c_float,
                                      i32, i32]),
 }
+
+# measurement helpers of include/tf_bench.h: same library, not part of the drop-in surface
+BENCH_EXPORTS = {
+    "tf_bench_empty_launch": (i32, [vp, vp, u32, u32, vp, vp]),
+    "tf_bench_stream_read": (i32, [vp, vp, vp, u64, vp]),
+    "tf_bench_moe_decode_step_stages": None,     # the argument list of tf_moe_decode_step + stages, filled in below
+}
+
+BENCH_EXPORTS["tf_bench_moe_decode_step_stages"] = (i32, list(EXPORTS["tf_moe_decode_step"][1]) + [u32])
 
 _lib = None
 
@@ -229,7 +236,7 @@ def load() -> C.CDLL:
     except ImportError:
         pass
     lib = C.CDLL(LIB_PATH)
-    for name, (restype, argtypes) in EXPORTS.items():
+    for name, (restype, argtypes) in {**EXPORTS, **BENCH_EXPORTS}.items():
         fn = getattr(lib, name)      # AttributeError if the ABI and the library disagree
         fn.restype = restype
         fn.argtypes = argtypes

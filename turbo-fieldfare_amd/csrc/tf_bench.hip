@@ -1,6 +1,7 @@
 // Measurement helpers behind the C ABI: what a kernel boundary and a plain streaming read cost on the part the library runs
 // on, so that a benchmark can print the latency floor of a chain of dependent launches and the read rate a streaming kernel
 // can be held against, measured in the same run as the kernels themselves.
+#include "../../include/tf_bench.h"
 #include "tf_gemv_kernels.hpp"
 
 using namespace tfk;

@@ -703,6 +703,9 @@ static int32_t qkv_gemv_entry(tf_ctx *ctx, tf_stream stream, const char *who, co
     const LongPlan plan = plan_long_rows((int)n);
     bool fast = aligned16(x) && n > 1024 && n <= (uint32_t)XStage::kMaxK && plan.rt > 0 && (!nw || aligned16(nw));
     for (int i = 0; i < 3; ++i) fast = fast && aligned16(at(w[i], wo[i]));
+    // the one refusal left after the operand checks, ahead of the tail's launch: a refused call has launched nothing
+    TF_REQUIRE(ctx, fast || !nw || n <= kMaxHeadD, TF_ERR_SCRATCH_TOO_SMALL, "%s: rows of %u values exceed the context's one-row buffer (%u)", who, n,
+               kMaxHeadD);
     TailFuse tf = {};
     bool tail_fused = false;
     if (tail) {
@@ -712,9 +715,11 @@ static int32_t qkv_gemv_entry(tf_ctx *ctx, tf_stream stream, const char *who, co
               static_cast<half_t *>(tail->hidden_out), reinterpret_cast<const uint16_t *>(at(tail->w_postffn2, tail->w_postffn2_offset)),
               reinterpret_cast<const uint16_t *>(at(tail->w_postffn, tail->w_postffn_offset)),
               reinterpret_cast<const uint16_t *>(at(tail->w_postffn1, tail->w_postffn1_offset)), tail->eps, tail->layer_scalar};
+        // the output row (n halves) must not overlap any of the three input rows
         const void *ins[3] = {tf.h2, tf.h1, tf.hidden};
+        const uintptr_t row_bytes = (uintptr_t)n * 2, out_at = (uintptr_t)tf.hidden_out;
         bool distinct = true;
-        for (int i = 0; i < 3; ++i) distinct = distinct && ins[i] != (const void *)tf.hidden_out;
+        for (int i = 0; i < 3; ++i) distinct = distinct && ((uintptr_t)ins[i] + row_bytes <= out_at || out_at + row_bytes <= (uintptr_t)ins[i]);
         tail_fused = fast && nw && distinct && n <= kGlueMaxD && n % 8 == 0 && aligned16(tf.h2) && aligned16(tf.h1) && aligned16(tf.hidden) &&
                      aligned16(tf.hidden_out) && aligned16(tf.w_postffn2) && aligned16(tf.w_postffn) && aligned16(tf.w_postffn1);
         if (!tail_fused) {
@@ -761,7 +766,6 @@ static int32_t qkv_gemv_entry(tf_ctx *ctx, tf_stream stream, const char *who, co
     // any other shape or alignment: the three projections one after the other (same arithmetic per row), after the norm as
     // a launch of its own into the context's one-row buffer
     if (nw) {
-        TF_REQUIRE(ctx, n <= kMaxHeadD, TF_ERR_SCRATCH_TOO_SMALL, "%s: rows of %u values exceed the context's one-row buffer (%u)", who, n, kMaxHeadD);
         const int32_t rc = launch_rmsnorm_bf16w(ctx, st, x, nw, ctx->head_x_normed, n, eps);
         if (rc != TF_OK) return rc;
         x = ctx->head_x_normed;

@@ -1,4 +1,5 @@
 // Router (int8 GEMV + top-8 + softmax), routed expert phases 1 and 2, and the int4 shared expert, for gfx950.
+#include "../../include/tf_bench.h"
 #include "tf_gemv_kernels.hpp"
 #include "tf_router.hpp"
 #include "tf_rowslice.hpp"
@@ -21,7 +22,11 @@ static __device__ unsigned long long stamp_buf[3 * kStampWaves * 8];
     do {                                                                                                                  \
         if ((threadIdx.x & 63) == 0 && (wave_) < kStampWaves) stamp_buf[(((kernel_) * kStampWaves + (wave_)) << 3) + (slot_)] = wall_clock64(); \
     } while (0)
+#ifdef TF_STAMPS_NOWAIT
+#define TF_STAMP_WAIT() do {} while (0)
+#else
 #define TF_STAMP_WAIT() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
+#endif
 extern "C" unsigned long long *tf_debug_stamps(void) {
     void *ptr = nullptr;
     return hipGetSymbolAddress(&ptr, HIP_SYMBOL(stamp_buf)) == hipSuccess ? static_cast<unsigned long long *>(ptr) : nullptr;
@@ -976,6 +981,32 @@ int32_t router_select_entry(tf_ctx *ctx, tf_stream stream, const void *per_exper
     return check_launch(ctx, "router_gemma4 select");
 }
 
+// Every precondition of the step's three stages (router, phase 1, phase 2), checked without launching anything: a refused
+// step leaves every buffer as it was.  The stage entries repeat these checks when they are called on their own.
+int32_t decode_step_check(tf_ctx *ctx, const void *router_weights, uint64_t router_weights_offset, const void *router_scales,
+                          uint64_t router_scales_offset, const void *router_biases, uint64_t router_biases_offset, const void *router_x,
+                          const void *effective_scale, uint64_t effective_scale_offset, const void *per_expert_scale,
+                          uint64_t per_expert_scale_offset, const void *expert_pool, uint32_t num_experts, const tf_expert_offsets *routed_offsets,
+                          const void *x, const void *acts, const void *residual, const void *y, const void *out_indices, const void *out_weights,
+                          uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: null context");
+    TF_REQUIRE(ctx, router_weights && router_scales && router_biases && router_x && effective_scale && per_expert_scale && expert_pool &&
+                   routed_offsets && x && acts && residual && y && out_indices && out_weights,
+               TF_ERR_INVALID_ARGUMENT, "moe_decode_step: null argument");
+    TF_REQUIRE(ctx, d > 0 && d % TF_GROUP_SIZE == 0, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: d must be a multiple of 64, got %u", d);
+    TF_REQUIRE(ctx, f > 0 && f % TF_GROUP_SIZE == 0, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: f must be a multiple of 64, got %u", f);
+    TF_REQUIRE(ctx, num_experts > 0 && num_experts <= 256, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: numExperts must be in 1...256, got %u", num_experts);
+    TF_REQUIRE(ctx, top_k == TF_MAX_STREAMED_EXPERTS, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: topK must be 8, got %u", top_k);
+    TF_REQUIRE(ctx, scale_dtype == TF_BF16 || scale_dtype == TF_FP16, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: scale dtype must be bf16 or fp16");
+    (void)router_weights_offset;   // 8-bit weights: any byte offset
+    TF_REQUIRE(ctx, aligned(at(router_scales, router_scales_offset), 2) && aligned(at(router_biases, router_biases_offset), 2) &&
+                   aligned(at(effective_scale, effective_scale_offset), 2) && aligned(at(per_expert_scale, per_expert_scale_offset), 2) &&
+                   aligned(router_x, 2) && aligned(out_indices, 4) && aligned(out_weights, 2) && offsets_even(*routed_offsets) && aligned(x, 2) &&
+                   aligned(acts, 2) && aligned(residual, 2) && aligned(y, 2),
+               TF_ERR_INVALID_ARGUMENT, "moe_decode_step: misaligned operand");
+    return TF_OK;
+}
+
 // router logits -> (selection + phase 1) -> phase 2 on one stream; `logits` is the num_experts-float scratch between the launches
 // The shared expert riding along with the decode step's launches (see router_and_shared_gate_up_kernel).
 struct SharedRide {
@@ -990,8 +1021,12 @@ int32_t decode_step_impl(tf_ctx *ctx, tf_stream stream, const void *router_weigh
                            const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
                            const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
                            void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype, float *logits,
-                         bool may_time, const SharedRide *ride = nullptr, const PostAttnFuseArgs *post = nullptr) {
-    TF_REQUIRE(ctx, ctx && expert_pool && out_indices, TF_ERR_INVALID_ARGUMENT, "moe_decode_step: null argument");
+                         bool may_time, const SharedRide *ride = nullptr, const PostAttnFuseArgs *post = nullptr, uint32_t stages = 3) {
+    int32_t rc = decode_step_check(ctx, router_weights, router_weights_offset, router_scales, router_scales_offset, router_biases,
+                                   router_biases_offset, router_x, effective_scale, effective_scale_offset, per_expert_scale,
+                                   per_expert_scale_offset, expert_pool, num_experts, routed_offsets, x, acts, residual, y, out_indices,
+                                   out_weights, d, f, top_k, scale_dtype);
+    if (rc != TF_OK) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool timed = may_time && ctx->step_timing;
     auto mark = [&](int i) {
@@ -1000,11 +1035,11 @@ int32_t decode_step_impl(tf_ctx *ctx, tf_stream stream, const void *router_weigh
     mark(0);
     const int ride_sd = scale_dtype == TF_BF16 ? 0 : 1;
     bool rode = false;
-    int32_t rc = router_logits_entry(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset,
+    rc = router_logits_entry(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset,
                                      router_biases, router_biases_offset, router_x, effective_scale, effective_scale_offset,
                                      per_expert_scale, per_expert_scale_offset, out_indices, out_weights, num_experts, d, top_k, logits,
                                      ride ? &ride->gate_up : nullptr, ride_sd, &rode, post);
-    if (rc != TF_OK) return rc;
+    if (rc != TF_OK || stages < 2) return rc;
     if (ride && !rode) {   // the router took another kernel: the shared expert's gate / up rows get their own launch
         if (ride_sd == 0) hipLaunchKernelGGL((shared_gate_up_long_kernel<2, 3, 0>), dim3(((ride->gate_up.f + 1) / 2 + 3) / 4), dim3(256), 0, st, ride->gate_up);
         else hipLaunchKernelGGL((shared_gate_up_long_kernel<2, 3, 1>), dim3(((ride->gate_up.f + 1) / 2 + 3) / 4), dim3(256), 0, st, ride->gate_up);
@@ -1033,7 +1068,7 @@ int32_t decode_step_impl(tf_ctx *ctx, tf_stream stream, const void *router_weigh
         mark(1);
         rc = phase1_entry(ctx, stream, &routed, routed_offsets, x, acts, nullptr, 0, false, d, f, top_k, scale_dtype);
     }
-    if (rc != TF_OK) return rc;
+    if (rc != TF_OK || stages < 3) return rc;
     mark(2);
     rc = tf_moe_phase2_down_reduce(ctx, stream, &routed, routed_offsets, acts, out_weights, residual, y, d, f, top_k, scale_dtype);
     mark(3);
@@ -1161,6 +1196,23 @@ int32_t tf_moe_decode_step(tf_ctx *ctx, tf_stream stream, const void *router_wei
                             out_indices, out_weights, d, f, top_k, scale_dtype, ctx->router_logits, true);
 }
 
+// include/tf_bench.h: the first `stages` launches of tf_moe_decode_step (1: router logits, 2: + selection and phase 1, 3: the step)
+int32_t tf_bench_moe_decode_step_stages(tf_ctx *ctx, tf_stream stream, const void *router_weights, uint64_t router_weights_offset,
+                                        const void *router_scales, uint64_t router_scales_offset, const void *router_biases,
+                                        uint64_t router_biases_offset, const void *router_x, const void *effective_scale,
+                                        uint64_t effective_scale_offset, const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                                        const void *expert_pool, uint64_t expert_pool_stride, uint32_t num_experts,
+                                        const tf_expert_offsets *routed_offsets, const void *x, void *acts, const void *residual, void *y,
+                                        void *out_indices, void *out_weights, uint32_t d, uint32_t f, uint32_t top_k, tf_dtype scale_dtype,
+                                        uint32_t stages) {
+    TF_REQUIRE(ctx, ctx != nullptr, TF_ERR_INVALID_ARGUMENT, "bench_moe_decode_step_stages: null context");
+    TF_REQUIRE(ctx, stages >= 1 && stages <= 3, TF_ERR_INVALID_ARGUMENT, "bench_moe_decode_step_stages: stages must be 1, 2 or 3, got %u", stages);
+    return decode_step_impl(ctx, stream, router_weights, router_weights_offset, router_scales, router_scales_offset, router_biases,
+                            router_biases_offset, router_x, effective_scale, effective_scale_offset, per_expert_scale,
+                            per_expert_scale_offset, expert_pool, expert_pool_stride, num_experts, routed_offsets, x, acts, residual, y,
+                            out_indices, out_weights, d, f, top_k, scale_dtype, ctx->router_logits, false, nullptr, nullptr, stages);
+}
+
 int32_t tf_moe_decode_step_static(tf_ctx *ctx, tf_stream stream, const void *router_weights, uint64_t router_weights_offset,
                                   const void *router_scales, uint64_t router_scales_offset, const void *router_biases,
                                   uint64_t router_biases_offset, const void *router_x, const void *effective_scale,
@@ -1226,6 +1278,15 @@ int32_t decode_step_shared_impl(tf_ctx *ctx, tf_stream stream, const void *route
     const bool ride_ok = proj16 && aligned16(shared_x) && aligned16(shared_scratch_act) && aligned(shared_scratch_gate, 2) && aligned(shared_scratch_up, 2) &&
                          aligned(shared_y, 2) && sdim > 1024 && sdim <= (uint32_t)XStage::kMaxK && sf > 1024 && sf <= (uint32_t)XStage::kMaxK &&
                          plan_up.rt == 2 && plan_up.np == 3 && plan_down.rt == 2 && plan_down.np == 3;
+    // the routed step's own preconditions before anything is launched (the setup and the shared expert may run as launches
+    // of their own below): a refused call leaves the residual stream and every other buffer untouched
+    {
+        const int32_t rc = decode_step_check(ctx, router_weights, router_weights_offset, router_scales, router_scales_offset, router_biases,
+                                             router_biases_offset, router_x, effective_scale, effective_scale_offset, per_expert_scale,
+                                             per_expert_scale_offset, expert_pool, num_experts, routed_offsets, x, acts, residual, y, out_indices,
+                                             out_weights, d, f, top_k, scale_dtype);
+        if (rc != TF_OK) return rc;
+    }
     // the setup inside the first launch: that launch must be the block-per-expert router with the shared rows riding along,
     // every row and norm weight must move in 16-byte pieces, and nobody may write what other blocks still read
     PostAttnFuseArgs fuse = {};
@@ -1240,9 +1301,15 @@ int32_t decode_step_shared_impl(tf_ctx *ctx, tf_stream stream, const void *route
                 reinterpret_cast<const uint16_t *>(at(post->w_post_attn, post->w_post_attn_offset)),
                 reinterpret_cast<const uint16_t *>(at(post->w_pre_ffn, post->w_pre_ffn_offset)),
                 reinterpret_cast<const uint16_t *>(at(post->w_pre_ffn2, post->w_pre_ffn2_offset)), post->eps};
-        const void *outs[4] = {fuse.hidden_out, fuse.dense_x, fuse.routed_x, fuse.router_x};
+        // four output rows and two input rows of d halves each: no output may overlap an input or another output
+        const void *rows[6] = {fuse.hidden_out, fuse.dense_x, fuse.routed_x, fuse.router_x, fuse.hidden, fuse.attn};
+        const uintptr_t row_bytes = (uintptr_t)d * 2;
         bool distinct = true;
-        for (int i = 0; i < 4; ++i) distinct = distinct && outs[i] != (const void *)fuse.hidden && outs[i] != (const void *)fuse.attn;
+        for (int i = 0; i < 4; ++i)
+            for (int j = i + 1; j < 6; ++j) {
+                const uintptr_t a = (uintptr_t)rows[i], b = (uintptr_t)rows[j];
+                distinct = distinct && (a + row_bytes <= b || b + row_bytes <= a);
+            }
         const bool router_fast = router_weights && effective_scale && aligned16(at(router_weights, router_weights_offset)) &&
                                  aligned16(at(effective_scale, effective_scale_offset)) && d <= 4096 && d % TF_GROUP_SIZE == 0 && num_experts > 0 &&
                                  num_experts <= 256;

@@ -1532,7 +1532,7 @@ int32_t tf_prefill_grouped_routed_moe_resident_shared(tf_ctx *ctx, tf_stream str
                                                       uint32_t shared_x_stride_elements, uint32_t shared_y_stride_elements,
                                                       uint32_t shared_weight_bits) {
     // both calls' argument checks first, so that a refused call has launched nothing
-    DenseRide ride;
+    DenseRide ride = {};
     int32_t rc = shared_expert_block_plan(ctx, shared_x, shared_x_offset, shared_y, shared_y_offset, shared_gate, shared_up, shared_down,
                                           scratch_gate, scratch_gate_offset, scratch_gate_length, scratch_up, scratch_up_offset, scratch_up_length,
                                           scratch_act, scratch_act_offset, scratch_act_length, query_count, d, shared_intermediate,

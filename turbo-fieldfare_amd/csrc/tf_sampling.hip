@@ -213,47 +213,64 @@ __global__ __launch_bounds__(256) void topk_tile_kernel(const half_t *probs, con
     }
 }
 
-// Last tile: sort, then one thread walks the k best: drop unusable slots, cut at the top-p mass (probabilities still carry
-// their full-vocabulary normalisation), reweight by p^(1/T), draw by inverse CDF with the seeded xorshift64*.
+// Running sums of values[0..n) in index order, one fp32 add per element (thread 0; n <= 256), left in sums[] for the whole
+// block: sums[i] is what a sequential accumulation holds after element i, so a search over sums[] finds exactly the element a
+// sequential walk would stop at.  Ends with a barrier.
+__device__ __forceinline__ void running_sums(const float *values, uint32_t n, float *sums) {
+    if (threadIdx.x == 0) {
+        float acc = 0.0f;
+        for (uint32_t i = 0; i < n; ++i) {
+            acc += values[i];
+            sums[i] = acc;
+        }
+    }
+    __syncthreads();
+}
+
+// Smallest candidate any thread of the block offers (threads without one offer `none`), through one LDS word.  Two barriers.
+__device__ __forceinline__ uint32_t block_first(uint32_t candidate, uint32_t none, uint32_t *word) {
+    if (threadIdx.x == 0) *word = none;
+    __syncthreads();
+    if (candidate < none) atomicMin(word, candidate);
+    __syncthreads();
+    const uint32_t found = *word;
+    __syncthreads();
+    return found;
+}
+
+// Last tile: sort, then thread t looks after slot t of the k best (k <= 256 = the block).  Results follow the reference's
+// sampler (Metal/Sampling/logit.metal:564-606): the usable prefix ends at the first slot that is padding or not finite; the
+// top-p cut keeps the shortest prefix whose mass (probabilities still carry their full-vocabulary normalisation) reaches top_p;
+// survivors are reweighted by p^(1/T); the draw is the inverse CDF of the seeded xorshift64* uniform.  The sums that decide
+// the cut and the draw are accumulated in index order (running_sums); the slots are tested and reweighted side by side.
 __global__ __launch_bounds__(256) void topk_final_kernel(const half_t *probs, const float *in_values, const uint32_t *in_indices, uint32_t count,
                                                          uint32_t k, float temperature, float top_p, uint64_t seed, uint32_t *out_token) {
     __shared__ float values[kTile];
     __shared__ uint32_t indices[kTile];
+    __shared__ float sums[256];
+    __shared__ uint32_t word;
     load_tile(probs, in_values, in_indices, 0, count, values, indices);
     sort_tile(values, indices);
-    if (threadIdx.x != 0) return;
-    uint32_t kept = 0;
-    while (kept < k && indices[kept] != 0xFFFFFFFFu && __builtin_isfinite(values[kept])) ++kept;
+    const uint32_t t = threadIdx.x;
+    const bool unusable = t < k && (indices[t] == 0xFFFFFFFFu || !__builtin_isfinite(values[t]));
+    uint32_t n = block_first(unusable ? t : k, k, &word);
     if (top_p > 0.0f && top_p < 1.0f) {
-        float cumulative = 0.0f;
-        uint32_t cut = kept;
-        for (uint32_t i = 0; i < kept; ++i) {
-            cumulative += values[i];
-            if (cumulative >= top_p) {
-                cut = i + 1;
-                break;
-            }
-        }
-        kept = cut;
+        running_sums(values, n, sums);
+        n = block_first(t < n && sums[t] >= top_p ? t + 1 : n, n, &word);
     }
-    const float inv_temperature = 1.0f / temperature;
-    if (temperature != 1.0f)
-        for (uint32_t i = 0; i < kept; ++i) values[i] = powf(values[i], inv_temperature);
-    float surviving = 0.0f;
-    for (uint32_t i = 0; i < kept; ++i) surviving += values[i];
+    if (temperature != 1.0f) {
+        if (t < n) values[t] = powf(values[t], 1.0f / temperature);
+        __syncthreads();
+    }
+    running_sums(values, n, sums);
     uint64_t rng = seed;
     (void)xorshift64(rng);
-    const float u = uniform01(rng) * surviving;
-    float running = 0.0f;
-    uint32_t picked = indices[0];
-    for (uint32_t i = 0; i < kept; ++i) {
-        running += values[i];
-        if (u <= running) {
-            picked = indices[i];
-            break;
-        }
+    const float u = uniform01(rng) * (n > 0 ? sums[n - 1] : 0.0f);
+    const uint32_t slot = block_first(t < n && u <= sums[t] ? t : n, n, &word);
+    if (t == 0) {
+        const uint32_t token = indices[slot < n ? slot : 0];
+        out_token[0] = token == 0xFFFFFFFFu ? 0u : token;
     }
-    out_token[0] = picked == 0xFFFFFFFFu ? 0u : picked;
 }
 
 // Wrapper-owned scratch of the samplers: [argmax cells + ticket | softmax partials | two pair buffers].
