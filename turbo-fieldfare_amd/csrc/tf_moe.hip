@@ -328,6 +328,122 @@ __global__ __launch_bounds__(512) void phase2_short_kernel(RoutedArg routed, tf_
     TF_STAMP(2, blockIdx.x * 8 + slot, 4);
 }
 
+// The same projection with an even share of the rows for every block and every lane busy (F <= 1024, 16-byte aligned operands).
+// A block takes `rpb` consecutive rows; wave s reads those rows of slot s's matrix as ONE flat stream of 16-byte chunks
+// (rows are contiguous: pass p, lane l reads chunk 64 p + l of the block's rows, 1 KiB per load instruction), so at F = 704
+// eleven rows fill 242 of the 256 chunk positions of four passes where one row per half-wave fills 22 of 32, and 2816 rows make
+// exactly one block for each of 256 CUs.  A lane's chunk lies in row c / nch, column c % nch: the slot's activations are staged
+// once per wave in LDS in dot-product order and each pass picks its column there.  Row sums are sums over runs of nch
+// consecutive lanes that may cross a pass boundary: every pass is prefix-summed across the wave (six DPP adds), the running
+// sums go to LDS indexed by chunk, and lane r takes row r's sum as a difference of two of them.
+// The hot arguments lead the list as plain scalars (kernel-argument preloading takes leading scalars only).
+constexpr int kFlatMaxRows = 32;
+struct BlobPtrs {
+    const uint8_t *blob[TF_MAX_STREAMED_EXPERTS];
+};
+__device__ __forceinline__ float wave_inclusive_scan(float v) {
+    v += dpp_f32<0x111>(v);          // row_shr:1 (lanes without a source inside their row of 16 add 0)
+    v += dpp_f32<0x112>(v);          // row_shr:2
+    v += dpp_f32<0x114>(v);          // row_shr:4
+    v += dpp_f32<0x118>(v);          // row_shr:8
+    v += dpp_f32<0x142, 0xA>(v);     // row_bcast15 into rows 1 and 3
+    v += dpp_f32<0x143, 0xC>(v);     // row_bcast31 into rows 2 and 3
+    return v;
+}
+template <int NP, int SD>
+__global__ __launch_bounds__(512) void phase2_flat_kernel(const uint32_t *indices, const uint8_t *pool, uint64_t stride, const half_t *acts,
+                                                          const half_t *routing_w, const half_t *residual, half_t *y, uint32_t d, uint32_t f,
+                                                          uint32_t rpb, uint32_t inv_nch, uint32_t num_experts, tf_expert_offsets off,
+                                                          BlobPtrs blobs) {
+    __shared__ __align__(16) u32x4 xa[8][128];        // [slot][word d of column c at d * nch + c]
+    __shared__ float xsum[8][32];
+    __shared__ float running[8][NP * 64];             // [slot][chunk]: inclusive sums within each pass
+    __shared__ float partial[8][kFlatMaxRows];
+    const int lane = threadIdx.x & 63;
+    const uint32_t slot = uniform_u32(threadIdx.x >> 6);
+    const uint32_t row0 = blockIdx.x * rpb;
+    const uint32_t rows_here = min(rpb, d - row0);
+    const int nch = (int)(f >> 5), groups = (int)(f >> 6), pieces = (int)(f >> 3);
+    TF_STAMP(2, blockIdx.x * 8 + slot, 0);
+    // what does not depend on the expert lookup goes first: the slot's activations, its routing weight, the residual
+    const rsrc_t ra = make_rsrc(acts + (size_t)slot * f, f * 2u);
+    u32x4 xr[2];
+    xr[0] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, (uint32_t)lane * 16u, 0, 0));
+    xr[1] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(ra, (uint32_t)(lane + 64) * 16u, 0, 0));
+    const half_t w16 = routing_w[slot];
+    const bool writer = threadIdx.x < rows_here;
+    const half_t res16 = writer ? residual[row0 + threadIdx.x] : (half_t)0.0f;   // needed after the barrier
+    const uint8_t *base;
+    if (indices) {
+        uint32_t e = indices[slot];
+        e = e < num_experts ? e : num_experts - 1;
+        base = pool + (uint64_t)e * stride;
+    } else {
+        base = blobs.blob[slot];
+    }
+    base = uniform_ptr(base);
+    TF_STAMP(2, blockIdx.x * 8 + slot, 1);
+    const rsrc_t rw = make_rsrc(base + off.down_W_off + (size_t)row0 * (f >> 1), rows_here * (f >> 1));
+    const rsrc_t rs = make_rsrc(base + off.down_s_off + (size_t)row0 * groups * 2, rows_here * (uint32_t)groups * 2u);
+    const rsrc_t rb = make_rsrc(base + off.down_b_off + (size_t)row0 * groups * 2, rows_here * (uint32_t)groups * 2u);
+    u32x4 w[NP];
+    uint16_t sv[NP], bv[NP];
+    int col[NP];
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        const uint32_t c = 64u * p + (uint32_t)lane;
+        const uint32_t r = (c * inv_nch) >> 16;            // c / nch (the host checked the reciprocal for every c < 64 NP)
+        const uint32_t cc = c - r * (uint32_t)nch;
+        col[p] = (int)cc;
+        const uint32_t sboff = (r * (uint32_t)groups + (cc >> 1)) * 2u;   // past the block's rows: past the descriptor, reads zero
+        w[p] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rw, c * 16u, 0, kStreamOnce));
+        sv[p] = __builtin_amdgcn_raw_buffer_load_b16(rs, sboff, 0, 0);
+        bv[p] = __builtin_amdgcn_raw_buffer_load_b16(rb, sboff, 0, 0);
+    }
+    // the wave's own LDS image of its slot's activations (LDS serves one wave's requests in order: no barrier needed)
+    XStage::publish_piece(xr[0], lane, pieces, nch, xa[slot], xsum[slot]);
+    XStage::publish_piece(xr[1], lane + 64, pieces, nch, xa[slot], xsum[slot]);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const float wgt = (float)w16;
+    TF_STAMP_WAIT();
+    TF_STAMP(2, blockIdx.x * 8 + slot, 2);
+#pragma unroll
+    for (int p = 0; p < NP; ++p) {
+        half2_t xq[16];
+#pragma unroll
+        for (int dd = 0; dd < 4; ++dd) {
+            const u32x4 v = xa[slot][dd * nch + col[p]];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) xq[4 * dd + j] = as_half2(v[j]);
+        }
+        const float part = fmaf(sb_to_f32<SD>(sv[p]), chunk_dot(w[p], xq), sb_to_f32<SD>(bv[p]) * xsum[slot][col[p]]);
+        running[slot][64 * p + lane] = wave_inclusive_scan(part);
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    if ((uint32_t)lane < rows_here) {
+        // row `lane` = chunks first .. last of the stream
+        const uint32_t first = (uint32_t)lane * (uint32_t)nch, last = first + (uint32_t)nch - 1u;
+        const float *run = running[slot];
+        float sum = run[last];
+        if ((first >> 6) != (last >> 6)) sum += run[(first | 63u)];            // the row started in the pass before
+        if (first & 63u) sum -= run[first - 1u];
+        partial[slot][lane] = wgt * sum;
+    }
+    TF_STAMP(2, blockIdx.x * 8 + slot, 3);
+    __syncthreads();
+    if (writer) {
+        float acc = (float)res16;
+#pragma unroll
+        for (int s = 0; s < 8; ++s) acc += partial[s][threadIdx.x];
+        y[row0 + threadIdx.x] = (half_t)acc;
+    }
+    TF_STAMP(2, blockIdx.x * 8 + slot, 4);
+}
+
 template <int SD>
 __global__ __launch_bounds__(512) void phase2_generic_kernel(RoutedArg routed, tf_expert_offsets off, const half_t *acts,
                                                              const half_t *routing_w, const half_t *residual, half_t *y,
@@ -1171,6 +1287,42 @@ int32_t tf_moe_phase2_down_reduce(tf_ctx *ctx, tf_stream stream, const tf_routed
     // acts rows start at slot * f halves: 16-byte aligned when f % 8 == 0, which f % 64 == 0 guarantees
     const bool fast = all16 && aligned16(acts) && (routed_offsets->down_W_off % 16 == 0) && f <= 1024;
     if (fast) {
+        // rows per block and passes: fewest passes on the busiest CU (blocks are dealt out evenly), then fullest lanes
+        const uint32_t nch = f / 32;
+        int best_np = 0;
+        uint32_t best_rpb = 0;
+        double best_cost = 0.0;
+        for (int np = 1; np <= 4; ++np) {
+            const uint32_t rpb = std::min<uint32_t>((uint32_t)(64 * np) / nch, (uint32_t)kFlatMaxRows);
+            if (rpb == 0) continue;
+            const uint32_t blocks = (d + rpb - 1) / rpb;
+            const uint32_t rounds = (blocks + (uint32_t)ctx->num_cus - 1) / (uint32_t)std::max(ctx->num_cus, 1);
+            const double cost = (double)rounds * np + 1e-3 * (1.0 - (double)(rpb * nch) / (64.0 * np));
+            if (best_np == 0 || cost < best_cost) {
+                best_np = np;
+                best_rpb = rpb;
+                best_cost = cost;
+            }
+        }
+        // c / nch as a multiply and a shift, checked for every chunk position a lane can hold
+        const uint32_t inv_nch = (65536u + nch - 1) / nch;
+        bool inv_ok = best_np > 0;
+        for (uint32_t c = 0; inv_ok && c < 64u * (uint32_t)best_np; ++c) inv_ok = ((c * inv_nch) >> 16) == c / nch;
+        if (inv_ok) {
+            const dim3 grid((d + best_rpb - 1) / best_rpb);
+            BlobPtrs blobs;
+            for (uint32_t i = 0; i < TF_MAX_STREAMED_EXPERTS; ++i) blobs.blob[i] = arg.blob[i];
+#define TF_P2_FLAT(NP_, SD_)                                                                                                          \
+    hipLaunchKernelGGL((phase2_flat_kernel<NP_, SD_>), grid, dim3(512), 0, st, arg.indices, arg.pool, arg.stride, ah, wh, rh, yh, d, f, \
+                       best_rpb, inv_nch, arg.num_experts, *routed_offsets, blobs)
+            if (scale_dtype == TF_BF16) {
+                if (best_np == 1) TF_P2_FLAT(1, 0); else if (best_np == 2) TF_P2_FLAT(2, 0); else if (best_np == 3) TF_P2_FLAT(3, 0); else TF_P2_FLAT(4, 0);
+            } else {
+                if (best_np == 1) TF_P2_FLAT(1, 1); else if (best_np == 2) TF_P2_FLAT(2, 1); else if (best_np == 3) TF_P2_FLAT(3, 1); else TF_P2_FLAT(4, 1);
+            }
+#undef TF_P2_FLAT
+            return check_launch(ctx, "moe_phase2_flat");
+        }
         constexpr int NPASS = 4;
         const dim3 grid((d + 2 * NPASS - 1) / (2 * NPASS));
         if (scale_dtype == TF_BF16) hipLaunchKernelGGL((phase2_short_kernel<NPASS, 0>), grid, dim3(512), 0, st, arg, *routed_offsets, ah, wh, rh, yh, d, f);
