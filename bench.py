@@ -46,8 +46,8 @@ LM_HEAD_BYTES = int4_matrix_bytes(VOCAB, D) + D * 2 + 4
 
 
 # (blocks, threads per block) of the decode step's three launches at the production shape: one block per router row, one wave
-# per two-row gate/up tile, eight down rows per block of eight waves
-STEP_GRID_SHAPES = ((E, 256), (TOPK * (F_MOE // 2) // 4, 256), (D // 8, 512))
+# per two-row gate/up tile, eleven down rows per block of eight waves
+STEP_GRID_SHAPES = ((E, 256), (TOPK * (F_MOE // 2) // 4, 256), (D // 11, 512))
 
 
 def expert_layout():

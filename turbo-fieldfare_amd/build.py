@@ -16,6 +16,10 @@ OUT = os.path.join(HERE, "libtf_kernels.so")
 SOURCES = ["tf_context.hip", "tf_gemv.hip", "tf_moe.hip", "tf_lmhead.hip", "tf_prefill.hip", "tf_qmm.hip", "tf_glue.hip", "tf_sampling.hip", "tf_loader.hip", "tf_attention.hip", "tf_rope.hip", "tf_bench.hip"]
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+# Per-file additions.  The decode step's kernels are a launch and two or three memory round trips long, so the scalar loads of
+# their kernel arguments are on the critical path: gfx950 can hand the leading scalar arguments to a wave in registers at launch
+# (kernel-argument preloading; the code keeps a prologue that loads them itself where the firmware does not preload).
+EXTRA_FLAGS = {"tf_moe.hip": ["-mllvm", "-amdgpu-kernarg-preload-count=16"]}
 
 
 def _hipcc() -> str:
@@ -27,7 +31,7 @@ def _hipcc() -> str:
 
 def _compile(src: str) -> str:
     obj = os.path.join(CSRC, os.path.splitext(src)[0] + ".o")
-    cmd = [_hipcc(), *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [_hipcc(), *FLAGS, *EXTRA_FLAGS.get(src, []), "-c", os.path.join(CSRC, src), "-o", obj]
     res = subprocess.run(cmd, capture_output=True, text=True)
     # the host pass does not know the packed-fp32 feature and says so; that line is noise
     err = "\n".join(l for l in res.stderr.splitlines() if "packed-fp32-ops" not in l)
