@@ -35,9 +35,10 @@ def int4_matrix_bytes(rows, cols):
 ROUTER_BYTES = E * D + 2 * E * (D // 64) * 2 + D * 2 + D * 2 + E * 2 + TOPK * 4 + TOPK * 2   # W + s/b + hidden + eff + gains + outputs
 # HBM bytes one fused phase-1 launch moves, from hardware counters of `bench.py --only-decode-step` (two rocprofv3 --pmc runs,
 # FETCH_SIZE then WRITE_SIZE; profiles/decode_step_counters.txt gives the commands, the raw KiB per dispatch and the factors a
-# plain copy of known size calibrates).  None until such a profile of the current kernels is on file.
-PHASE1_TRAFFIC_BYTES = None
-PHASE1_TRAFFIC_FROM = None
+# plain copy of known size calibrates).  The literal below is that file's figure.
+PHASE1_TRAFFIC_BYTES = int(8908.2 * 1024 * 1.9999 + 22.1 * 1024)
+PHASE1_TRAFFIC_FROM = ("profiles/decode_step_counters.txt: FETCH_SIZE 8908.2 KiB x 1.9999 + WRITE_SIZE 22.1 KiB x 1.0000 per launch of the fused "
+                       "phase-1 kernel (factors from the 1 GiB copy of the same runs)")
 PHASE1_BYTES = TOPK * 2 * int4_matrix_bytes(F_MOE, D) + D * 2 + TOPK * F_MOE * 2             # gate+up of 8 experts + x + acts out
 PHASE2_BYTES = TOPK * int4_matrix_bytes(D, F_MOE) + TOPK * F_MOE * 2 + TOPK * 2 + D * 2 + D * 2   # down of 8 + acts in + w + residual + y
 STEP_BYTES = ROUTER_BYTES + PHASE1_BYTES + PHASE2_BYTES
@@ -159,6 +160,15 @@ def make_int4(torch, gen, rows, cols):
     return W, S, B
 
 
+def calibration_copy(torch):
+    """One plain 1 GiB device-to-device copy: a launch of known size to scale hardware byte counters by."""
+    src = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
+
 def profiler_attached():
     """True when a rocprofiler tool library rides in this process (rocprofv3 preloads it and names it in the environment)."""
     env = " ".join(os.environ.get(v, "") for v in ("LD_PRELOAD", "ROCP_TOOL_LIBRARIES", "ROCPROFILER_REGISTER_FORCE_LOAD", "ROCPROF_OUTPUT_PATH"))
@@ -188,6 +198,9 @@ def main():
     ap.add_argument("--only-decode-step", action="store_true",
                     help="run nothing but the headline decode-step measurement (graph-replayed steps and the one- and two-stage chains) and "
                          "print its JSON: the short program a profiler attributes the step's three kernels with")
+    ap.add_argument("--chain-launches", type=int, default=64,
+                    help="launches per graph of the one-, two- and three-stage chains (a counter-collecting profiler serialises every "
+                         "dispatch: give it short chains and few --steps)")
     ap.add_argument("--only-lm-head", action="store_true",
                     help="run nothing but the lm_head measurements (configs[2]) and print their JSON")
     ap.add_argument("--only-small-m", type=int, nargs="+", metavar="M",
@@ -305,7 +318,7 @@ def main():
             if lib.tf_bench_moe_decode_step_stages(*step_args(i, stream), n_stages) != 0:
                 raise RuntimeError("kernel call failed: " + k.last_error())
         return fn
-    us_chain = {n: time_loop(torch, stages(n), 64) for n in (1, 2, 3)}
+    us_chain = {n: time_loop(torch, stages(n), args.chain_launches) for n in (1, 2, 3)}
     t_router, t_p1 = us_chain[1], us_chain[2] - us_chain[1]
     t_p2 = ms_per_step * 1e3 - us_chain[2]
     p1_gbps = PHASE1_BYTES / (t_p1 * 1e-6) / 1e9
@@ -341,6 +354,8 @@ def main():
                        "phase1_GBps": round(p1_gbps, 1), "phase2_GBps": round(PHASE2_BYTES / (t_p2 * 1e-6) / 1e9, 1)},
     }
     if args.only_decode_step:
+        if args.calibration_copy:
+            calibration_copy(torch)
         print(json.dumps(out))
         return
 
@@ -383,11 +398,7 @@ def main():
                                         "step_over_floor": round(ms_per_step * 1e3 / latency_floor_us, 3)}
 
     if args.calibration_copy:
-        src = torch.zeros(1 << 30, dtype=torch.uint8, device="cuda")
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
+        calibration_copy(torch)
     if not args.no_extras:
         note("extras: lm_head, GEMV, attention, shared expert")
         out["extras"] = head_extras(torch, tfk, k, gen, lib, h, stream)
