@@ -800,12 +800,14 @@ def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, 
 
         def fn(i):
             rc = 0
-            if with_router:
-                rc |= lib.tf_prefill_router_gemma4_block(h, stream, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0,
-                                                         hid.data_ptr(), 0, r["eff"].data_ptr(), 0, r["gain"].data_ptr(), 0,
-                                                         idx.data_ptr(), 0, wts.data_ptr(), 0, T, E, D, TOPK, D)
-            rc |= lib.tf_prefill_group_pairs_device(h, stream, idx.data_ptr(), wts.data_ptr(), T, TOPK, E, sp.data_ptr(),
-                                                    offs_d.data_ptr(), cnts_d.data_ptr(), chunks.data_ptr(), nch.data_ptr())
+            if with_router:     # router block + device grouping as one call (one launch fewer up to 32 tokens)
+                rc |= lib.tf_prefill_router_group_block(h, stream, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0,
+                                                        hid.data_ptr(), 0, r["eff"].data_ptr(), 0, r["gain"].data_ptr(), 0,
+                                                        idx.data_ptr(), 0, wts.data_ptr(), 0, T, E, D, TOPK, D, sp.data_ptr(),
+                                                        offs_d.data_ptr(), cnts_d.data_ptr(), chunks.data_ptr(), nch.data_ptr())
+            else:
+                rc |= lib.tf_prefill_group_pairs_device(h, stream, idx.data_ptr(), wts.data_ptr(), T, TOPK, E, sp.data_ptr(),
+                                                        offs_d.data_ptr(), cnts_d.data_ptr(), chunks.data_ptr(), nch.data_ptr())
             routed = (h, stream, hid.data_ptr(), 0, D, sp.data_ptr(), chunks.data_ptr(), nch.data_ptr(), cap, n, pool.data_ptr(), stride, E,
                       C.byref(off), acts.data_ptr(), partials.data_ptr(), D, F_MOE, TOPK, tfk.TF_BF16)
             if shared is None:

@@ -681,6 +681,24 @@ int32_t tf_prefill_grouped_routed_moe_streamed(tf_ctx *ctx, tf_stream stream,
                                                const void *const *blobs, const tf_prefill_streamed_params *params,
                                                const tf_prefill_group *tile_groups, uint32_t tile_group_count,
                                                int32_t pair_microbatch_rows, int32_t *out_microbatches, tf_dtype scale_dtype);
+/* tf_prefill_router_gemma4_block followed by tf_prefill_group_pairs_device on its outputs, as one call with every output of
+ * both (PrefillRouter.encodeGemma4Block, PrefillRouter.swift:37-89, then makeTokenExpertPairs + groupTokenExpertPairs,
+ * PrefillRouter.swift:91-111 and PrefillMoEGrouping.swift:90-193, which the reference runs on the host between two command
+ * buffers).  For up to 32 token rows and top_k <= 8 the selection and the grouping share one launch; results are bit-identical
+ * to the two calls, which larger calls are forwarded to. */
+int32_t tf_prefill_router_group_block(tf_ctx *ctx, tf_stream stream,
+                                      const void *weights, uint64_t weights_offset,
+                                      const void *scales, uint64_t scales_offset,
+                                      const void *biases, uint64_t biases_offset,
+                                      const void *hidden, uint64_t hidden_offset,
+                                      const void *effective_scale, uint64_t effective_scale_offset,
+                                      const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                                      void *out_indices, uint64_t out_indices_offset,
+                                      void *out_weights, uint64_t out_weights_offset,
+                                      uint32_t query_count, uint32_t num_experts, uint32_t d, uint32_t top_k,
+                                      uint32_t hidden_stride_elements,
+                                      void *sorted_pairs, void *per_expert_offsets, void *per_expert_counts,
+                                      void *chunks, void *chunk_count);
 /* Resident-pool form of the same computation over ALL sorted pairs of a chunk of tokens in one go: experts are
  * pool + expert * pool_stride, the work list comes from tf_prefill_group_pairs_device, nothing is read by the host.  Groups
  * of a few pairs stream each expert row once and apply it to every routed token (weight-read bound, the small-M regime);

@@ -143,6 +143,56 @@ def test_device_grouping_equals_host_grouping(T, top_k, E):
     assert covered == list(range(T * top_k)) and nch <= g["cap"]
 
 
+@pytest.mark.parametrize("T,E,d,top_k", [(1, 128, 2816, 8), (2, 128, 2816, 8), (16, 128, 2816, 8), (32, 128, 2816, 8), (31, 200, 704, 8), (7, 16, 128, 3),
+                                         (33, 128, 2816, 8), (12, 64, 256, 12)])
+def test_router_block_and_grouping_in_one_call_equal_the_two_calls(T, E, d, top_k):
+    # tf_prefill_router_group_block = tf_prefill_router_gemma4_block + tf_prefill_group_pairs_device, every output of both bit
+    # for bit: up to 32 tokens (and top-k <= 8) the selection and the grouping share one launch; 33 tokens and a top-12 are
+    # forwarded to the two calls.  The two calls are the ones the oracle and the host grouping check above.
+    rng = np.random.default_rng(T * 31 + E)
+    W, S, B = refcases.synthetic_int8(E, d, 0x6A0 + T)
+    hidden = np.concatenate([refcases.normal_f16(d, 0x700 + r) for r in range(T)])
+    eff = tfo.bf16_bits_array(rng.uniform(0.5, 1.5, d).astype(np.float32) / np.float32(np.sqrt(d)))
+    pes = tfo.bf16_bits_array(rng.uniform(0.6, 1.4, E).astype(np.float32))
+    k = ctx()
+    dW, dS, dB, dh, de, dp = dev(W), dev(S), dev(B), dev(hidden), dev(eff), dev(pes)
+    n = T * top_k
+    cap = E + n // 64 + 1
+
+    def outputs():
+        return dict(idx=zeros_bytes(n * 4, 0xEE), wts=zeros_bytes(n * 2, 0xEE), sp=zeros_bytes(n * 16, 0xEE), offs=zeros_bytes(E * 4, 0xEE),
+                    cnts=zeros_bytes(E * 4, 0xEE), chunks=zeros_bytes(cap * 12, 0xEE), nch=zeros_bytes(4, 0xEE))
+
+    router = (k.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dh.data_ptr(), 0, de.data_ptr(), 0, dp.data_ptr(), 0)
+    two, one = outputs(), outputs()
+    k.check(k.lib.tf_prefill_router_gemma4_block(*router, two["idx"].data_ptr(), 0, two["wts"].data_ptr(), 0, T, E, d, top_k, d))
+    k.check(k.lib.tf_prefill_group_pairs_device(k.handle, None, two["idx"].data_ptr(), two["wts"].data_ptr(), T, top_k, E, two["sp"].data_ptr(),
+                                                two["offs"].data_ptr(), two["cnts"].data_ptr(), two["chunks"].data_ptr(), two["nch"].data_ptr()))
+    k.check(k.lib.tf_prefill_router_group_block(*router, one["idx"].data_ptr(), 0, one["wts"].data_ptr(), 0, T, E, d, top_k, d, one["sp"].data_ptr(),
+                                                one["offs"].data_ptr(), one["cnts"].data_ptr(), one["chunks"].data_ptr(), one["nch"].data_ptr()))
+    nch = int(host(two["nch"], np.uint32, 1)[0])
+    assert 1 <= nch <= cap and nch == int(host(one["nch"], np.uint32, 1)[0])
+    for name, count in (("idx", n * 4), ("wts", n * 2), ("sp", n * 16), ("offs", E * 4), ("cnts", E * 4), ("chunks", nch * 12)):
+        assert np.array_equal(host(one[name], np.uint8, count), host(two[name], np.uint8, count)), name
+    # every token's experts are the reference router's
+    got = host(one["idx"], np.uint32, n).reshape(T, top_k)
+    if top_k == 8:
+        for r in (0, T - 1):
+            ref_idx, _, _ = tfo.router_reference(W, S, B, tfo.from_f16_bits(hidden[r * d:(r + 1) * d]), tfo.bf16_array_to_float(eff),
+                                                 tfo.bf16_array_to_float(pes))
+            assert list(got[r]) == list(ref_idx)
+    # a refused call launches nothing
+    bad = outputs()
+    rc = k.lib.tf_prefill_router_group_block(*router, bad["idx"].data_ptr(), 0, bad["wts"].data_ptr(), 0, T, E, d, 65, d, bad["sp"].data_ptr(),
+                                             bad["offs"].data_ptr(), bad["cnts"].data_ptr(), bad["chunks"].data_ptr(), bad["nch"].data_ptr())
+    assert rc == tfk.TF_ERR_INVALID_ARGUMENT
+    rc = k.lib.tf_prefill_router_group_block(*router, bad["idx"].data_ptr(), 0, bad["wts"].data_ptr(), 0, T, E, d, top_k, d, bad["sp"].data_ptr(),
+                                             bad["offs"].data_ptr(), None, bad["chunks"].data_ptr(), bad["nch"].data_ptr())
+    assert rc == tfk.TF_ERR_INVALID_ARGUMENT
+    k.synchronize()
+    assert all(np.all(host(bad[name], np.uint8) == 0xEE) for name in bad)
+
+
 def test_streamed_batched_matches_reference_across_partial_microbatch():
     # PrefillGroupedRoutedMoETests+Execution.swift:8-103
     d = f = 64

@@ -367,45 +367,57 @@ __global__ __launch_bounds__(64) void group_place_kernel(const uint32_t *indices
     }
 }
 
-// A single segment (at most 32 tokens, the multi-token verification case): the three steps in one 256-thread block.
-__global__ __launch_bounds__(256) void group_small_kernel(const uint32_t *indices, const uint16_t *weights, uint32_t n_pairs,
-                                                          uint32_t top_k, uint32_t num_experts, tf_prefill_pair *sorted_pairs,
-                                                          uint32_t *per_expert_offsets, uint32_t *per_expert_counts,
-                                                          tf_prefill_group *chunks, uint32_t *chunk_count) {
-    __shared__ uint32_t cnt[256], scan_pairs[256], scan_chunks[256], next[256];
-    __shared__ unsigned long long mask[256];
+// A single segment (at most 32 tokens, the multi-token verification case): the three steps by the first 256 threads of one
+// block (every thread of the block must call: the barriers are block-wide).  indices / weights may live in LDS.
+struct GroupSmallLds {
+    uint32_t cnt[256], scan_pairs[256], scan_chunks[256], next[256];
+    unsigned long long mask[256];
+};
+__device__ __forceinline__ void group_small_body(GroupSmallLds &l, const uint32_t *indices, const uint16_t *weights, uint32_t n_pairs, uint32_t top_k,
+                                                 uint32_t num_experts, tf_prefill_pair *sorted_pairs, uint32_t *per_expert_offsets,
+                                                 uint32_t *per_expert_counts, tf_prefill_group *chunks, uint32_t *chunk_count) {
     const uint32_t e = threadIdx.x;
-    cnt[e] = 0;
-    mask[e] = 0ull;
+    const bool owner = e < 256;        // thread e owns expert e
+    if (owner) {
+        l.cnt[e] = 0;
+        l.mask[e] = 0ull;
+    }
     __syncthreads();
-    for (uint32_t i = e; i < n_pairs; i += 256) atomicAdd(&cnt[clamp_expert(indices[i], num_experts)], 1u);
+    if (owner)
+        for (uint32_t i = e; i < n_pairs; i += 256) atomicAdd(&l.cnt[clamp_expert(indices[i], num_experts)], 1u);
     __syncthreads();
-    const uint32_t total = cnt[e];
+    const uint32_t total = owner ? l.cnt[e] : 0u;
     const uint32_t nch = (total + kChunkPairs - 1) / kChunkPairs;
-    scan_pairs[e] = total;
-    scan_chunks[e] = nch;
+    if (owner) {
+        l.scan_pairs[e] = total;
+        l.scan_chunks[e] = nch;
+    }
     __syncthreads();
     for (uint32_t step = 1; step < 256; step <<= 1) {
-        const uint32_t a = e >= step ? scan_pairs[e - step] : 0u, c = e >= step ? scan_chunks[e - step] : 0u;
+        const uint32_t a = owner && e >= step ? l.scan_pairs[e - step] : 0u, c = owner && e >= step ? l.scan_chunks[e - step] : 0u;
         __syncthreads();
-        scan_pairs[e] += a;
-        scan_chunks[e] += c;
+        if (owner) {
+            l.scan_pairs[e] += a;
+            l.scan_chunks[e] += c;
+        }
         __syncthreads();
     }
-    const uint32_t start = scan_pairs[e] - total, chunk_start = scan_chunks[e] - nch;
-    if (e == 255) chunk_count[0] = scan_chunks[255];
-    if (e < num_experts) {
-        per_expert_offsets[e] = total ? start : 0xFFFFFFFFu;
-        per_expert_counts[e] = total;
+    if (owner) {
+        const uint32_t start = l.scan_pairs[e] - total, chunk_start = l.scan_chunks[e] - nch;
+        if (e == 255) chunk_count[0] = l.scan_chunks[255];
+        if (e < num_experts) {
+            per_expert_offsets[e] = total ? start : 0xFFFFFFFFu;
+            per_expert_counts[e] = total;
+        }
+        for (uint32_t c = 0; c < nch; ++c) {
+            tf_prefill_group g;
+            g.expert = e;
+            g.pair_start = start + c * kChunkPairs;
+            g.pair_count = min(kChunkPairs, total - c * kChunkPairs);
+            chunks[chunk_start + c] = g;
+        }
+        l.next[e] = start;
     }
-    for (uint32_t c = 0; c < nch; ++c) {
-        tf_prefill_group g;
-        g.expert = e;
-        g.pair_start = start + c * kChunkPairs;
-        g.pair_count = min(kChunkPairs, total - c * kChunkPairs);
-        chunks[chunk_start + c] = g;
-    }
-    next[e] = start;
     __syncthreads();
     if (threadIdx.x >= 64) return;
     const uint32_t lane = threadIdx.x;
@@ -414,7 +426,7 @@ __global__ __launch_bounds__(256) void group_small_kernel(const uint32_t *indice
         const bool valid = i < n_pairs;
         const uint32_t x = valid ? clamp_expert(indices[i], num_experts) : 0u;
         const uint16_t wbits = valid ? weights[i] : (uint16_t)0;
-        const uint32_t pos = place_batch(x, valid, lane, mask, next);
+        const uint32_t pos = place_batch(x, valid, lane, l.mask, l.next);
         if (valid) {
             tf_prefill_pair p;
             p.token = i / top_k;
@@ -424,6 +436,41 @@ __global__ __launch_bounds__(256) void group_small_kernel(const uint32_t *indice
             sorted_pairs[pos] = p;
         }
     }
+}
+__global__ __launch_bounds__(256) void group_small_kernel(const uint32_t *indices, const uint16_t *weights, uint32_t n_pairs,
+                                                          uint32_t top_k, uint32_t num_experts, tf_prefill_pair *sorted_pairs,
+                                                          uint32_t *per_expert_offsets, uint32_t *per_expert_counts,
+                                                          tf_prefill_group *chunks, uint32_t *chunk_count) {
+    __shared__ GroupSmallLds l;
+    group_small_body(l, indices, weights, n_pairs, top_k, num_experts, sorted_pairs, per_expert_offsets, per_expert_counts, chunks, chunk_count);
+}
+
+// The selection of up to kSelectGroupTokens token rows and the grouping of their pairs in ONE block of sixteen waves: wave w
+// selects for tokens w and w + 16 from the logits the launch before left in scratch (the arithmetic of prefill_select_kernel),
+// writes the router's outputs and keeps them in LDS, where the grouping above takes them from.  One launch where the
+// router block's selection and the device grouping were two.
+constexpr uint32_t kSelectGroupTokens = 32, kSelectGroupTopK = 8;
+__global__ __launch_bounds__(1024) void select_group_small_kernel(const float *logits, const uint16_t *per_expert_scale, uint32_t *out_indices,
+                                                                  half_t *out_weights, uint32_t tokens, uint32_t num_experts, uint32_t top_k,
+                                                                  tf_prefill_pair *sorted_pairs, uint32_t *per_expert_offsets,
+                                                                  uint32_t *per_expert_counts, tf_prefill_group *chunks, uint32_t *chunk_count) {
+    __shared__ GroupSmallLds l;
+    __shared__ uint32_t s_idx[kSelectGroupTokens * kSelectGroupTopK];
+    __shared__ uint16_t s_w[kSelectGroupTokens * kSelectGroupTopK];
+    const int lane = threadIdx.x & 63;
+    for (uint32_t tkn = threadIdx.x >> 6; tkn < tokens; tkn += 16) {
+        uint32_t idx;
+        half_t weight;
+        router_select_lanes(logits + (size_t)tkn * num_experts, per_expert_scale, num_experts, top_k, lane, idx, weight);
+        if ((uint32_t)lane < top_k) {
+            out_indices[(size_t)tkn * top_k + lane] = idx;
+            out_weights[(size_t)tkn * top_k + lane] = weight;
+            s_idx[tkn * top_k + lane] = idx;
+            s_w[tkn * top_k + lane] = f32_to_f16_bits((float)weight);
+        }
+    }
+    __syncthreads();
+    group_small_body(l, s_idx, s_w, tokens * top_k, top_k, num_experts, sorted_pairs, per_expert_offsets, per_expert_counts, chunks, chunk_count);
 }
 
 // ------------------------------------------------------------------------------------------------ grouped, row-streaming
@@ -565,11 +612,12 @@ __global__ __launch_bounds__(512) void grouped_phase1_stream_kernel(ExpertTable 
 // experts' bytes, not by arithmetic: every touched expert has to stream through once, at the rate of a plain read.
 //
 // v_mfma_f32_4x4x4_16b_f16 multiplies, in each group of four lanes, the lanes' four A rows with the lanes' four B columns.
-// Here the four lanes of a quad hold the SAME 32-element piece of FOUR DIFFERENT weight rows (A: nibbles isolated as fp16
-// subnormals, exact) and the activations of that piece for FOUR DIFFERENT pairs (B, from an LDS image of the chunk's
+// Here the four lanes of a quad hold the SAME 32-element piece of FOUR DIFFERENT weight rows (B: nibbles isolated as fp16
+// subnormals, exact) and the activations of that piece for FOUR DIFFERENT pairs (A, from an LDS image of the chunk's
 // activation rows): all sixteen products of the instruction are wanted, a 4-row x 4-pair x 32-element product costs eight
-// instructions, and the nibbles of a piece are isolated once however many pairs meet it.  Result register k of lane m of a
-// quad = row k x pair m, over the quad's piece; scale and bias of row k come from lane k of the quad through DPP.
+// instructions, and the nibbles of a piece are isolated once however many pairs meet it.  Result register i of lane j of a
+// quad = pair i x row j, over the quad's piece: a lane collects ITS OWN row against four pairs, so the row's scale and bias
+// are the ones the lane loaded itself (with the operands the other way round every pass paid eight cross-lane moves for them).
 // A wave's 16 quads take QC consecutive pieces of 16 / QC groups of four rows; pieces of a row are summed across quads at
 // the end of a tile.  A block takes one slice of one chunk's rows; the next tile's loads follow the current tile's use
 // pass by pass, so one tile buffer keeps the memory pipe full.
@@ -580,6 +628,8 @@ constexpr int kQuadMaxD = 3072, kQuadMaxF = 1024;   // widest rows the LDS image
 constexpr int kQuadRowPad = 4;   // in 16-byte pieces
 constexpr size_t quad_row_bytes(int k) { return (size_t)k * 2 + kQuadRowPad * 16; }
 constexpr size_t quad_lds_bytes(int k) { return (size_t)kQuadMaxPairs * (quad_row_bytes(k) + (size_t)(k >> 5) * 4 + 16); }
+// The sums of a column's 32 activations sit side by side for the kQuadMaxPairs pairs of the image (xsum[column][pair]): a lane
+// needs the sums of four pairs at once and takes them in one 16-byte read.
 
 template <int CTRL>
 __device__ __forceinline__ float quad_bcast(float v) {
@@ -657,24 +707,23 @@ __device__ __forceinline__ void quad_request(QuadPass &t, const QuadMap<QC, NPAS
     t.b = __builtin_amdgcn_raw_buffer_load_b16(blob, qm.sboff(p), (int)b_at, 0);
 }
 
-// acc[k] += (row k of the quad) . (this lane's pair), over one piece: eight matrix instructions, then scale and bias of
-// each row from the lane of the quad that holds them.  xs: sum of the lane's pair's activations over the piece.
+// acc[i] += (pair i of the group) . (this lane's row), over one piece: eight matrix instructions, then the row's scale and
+// bias.  o: this lane's row piece; xq: the piece's activations of the lane's pair (lane % 4 of the group); xs4: the sums of the
+// four pairs' activations over the piece.  The matrix pipe's subnormal units (2^-24) are folded into the scale: s * 2^24 is
+// exact, so fma(s 2^24, c, .) rounds exactly as fma(s, c 2^24, .) would.
 template <int SD>
-__device__ __forceinline__ void quad_piece(const ChunkOperands &o, uint16_t s_bits, uint16_t b_bits, const half2_t *xq, float xs, float acc[4]) {
+__device__ __forceinline__ void quad_piece(const ChunkOperands &o, uint16_t s_bits, uint16_t b_bits, const half2_t *xq, const f32x4 xs4, float acc[4]) {
     f32x4 c = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (int d = 0; d < 4; ++d) {
-        const half4_t b0 = __builtin_shufflevector(xq[4 * d + 0], xq[4 * d + 1], 0, 1, 2, 3);
-        const half4_t b1 = __builtin_shufflevector(xq[4 * d + 2], xq[4 * d + 3], 0, 1, 2, 3);
-        c = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, o.a[2 * d]), b0, c, 0, 0, 0);
-        c = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4_t, o.a[2 * d + 1]), b1, c, 0, 0, 0);
+        const half4_t a0 = __builtin_shufflevector(xq[4 * d + 0], xq[4 * d + 1], 0, 1, 2, 3);
+        const half4_t a1 = __builtin_shufflevector(xq[4 * d + 2], xq[4 * d + 3], 0, 1, 2, 3);
+        c = __builtin_amdgcn_mfma_f32_4x4x4f16(a0, __builtin_bit_cast(half4_t, o.a[2 * d]), c, 0, 0, 0);
+        c = __builtin_amdgcn_mfma_f32_4x4x4f16(a1, __builtin_bit_cast(half4_t, o.a[2 * d + 1]), c, 0, 0, 0);
     }
-    c = c * 16777216.0f;   // subnormal units -> integers (exact)
-    const float sf = sb_to_f32<SD>(s_bits), bf = sb_to_f32<SD>(b_bits);
-    acc[0] = fmaf(quad_bcast<0x00>(sf), c[0], fmaf(quad_bcast<0x00>(bf), xs, acc[0]));
-    acc[1] = fmaf(quad_bcast<0x55>(sf), c[1], fmaf(quad_bcast<0x55>(bf), xs, acc[1]));
-    acc[2] = fmaf(quad_bcast<0xAA>(sf), c[2], fmaf(quad_bcast<0xAA>(bf), xs, acc[2]));
-    acc[3] = fmaf(quad_bcast<0xFF>(sf), c[3], fmaf(quad_bcast<0xFF>(bf), xs, acc[3]));
+    const float s24 = sb_to_f32<SD>(s_bits) * 16777216.0f, bf = sb_to_f32<SD>(b_bits);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) acc[i] = fmaf(s24, c[i], fmaf(bf, xs4[i], acc[i]));
 }
 
 // sum over the QC quads that hold pieces of the same rows: lanes that agree in (lane & 3) and in the row group
@@ -706,12 +755,13 @@ __device__ __forceinline__ void quad_stage_rows(uint32_t nb, int k, u32x4 *xa, f
         for (int i = 0; i < 4; ++i) {
             const int q = q0 + 256 * i + (int)threadIdx.x;
             const int j = q < total ? q / pieces : 0, piece = q < total ? q - j * pieces : pieces;   // piece == pieces: nothing is written
-            XStage::publish_piece(raw[i], piece, pieces, nch, xa + (size_t)j * (pieces + kQuadRowPad), xsum + (size_t)j * nch);
+            XStage::publish_piece(raw[i], piece, pieces, nch, xa + (size_t)j * (pieces + kQuadRowPad), xsum + j, (int)kQuadMaxPairs);
         }
     }
 }
 
-// pieces of one pass x the LDS image of the batch's pairs -> acc[g][k] (row k of the lane's quad x pair 4 g + lane % 4)
+// pieces of one pass x the LDS image of the batch's pairs -> acc[g][i] (pair 4 g + i x the lane's row).  A group's pairs beyond
+// the batch repeat its last pair (their sums are not stored); the sums of their activations are whatever the image holds.
 template <int QC, int NPASS, int SD, int G>
 __device__ __forceinline__ void quad_pass(const ChunkOperands &o, uint16_t s_bits, uint16_t b_bits, int colp, const QuadMap<QC, NPASS> &qm, const u32x4 *xa,
                                           const float *xsum, int nch, int pieces, uint32_t nb, int groups_of_pairs, float (&acc)[G][4]) {
@@ -728,7 +778,7 @@ __device__ __forceinline__ void quad_pass(const ChunkOperands &o, uint16_t s_bit
 #pragma unroll
                 for (int q = 0; q < 4; ++q) xq[4 * dd + q] = as_half2(v[q]);
             }
-            quad_piece<SD>(o, s_bits, b_bits, xq, xsum[(size_t)j * nch + colp], acc[g]);
+            quad_piece<SD>(o, s_bits, b_bits, xq, *reinterpret_cast<const f32x4 *>(xsum + (size_t)colp * kQuadMaxPairs + 4 * g), acc[g]);
         }
     }
 }
@@ -815,15 +865,12 @@ __global__ __launch_bounds__(256, 2) void grouped_phase1_quad_kernel(ExpertTable
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 if (g < groups_of_pairs) {
-                    uint32_t packed[2];
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const uint32_t h = f32_to_f16_bits(ag[g][k] * quad_sum<QC>(au[g][k]));
-                        packed[k >> 1] = (k & 1) ? (packed[k >> 1] | (h << 16)) : h;
+                    for (int i = 0; i < 4; ++i) {
+                        const half_t h = (half_t)(ag[g][i] * quad_sum<QC>(au[g][i]));
+                        const uint32_t j = 4 * g + i;
+                        if (lane < 4 && j < nb) acts[(size_t)(first + j - acts_pair_base) * f + row0 + lane] = h;   // lanes 0..3: the tile's four rows
                     }
-                    const uint32_t j = 4 * g + lane;
-                    if (lane < 4 && j < nb)
-                        *reinterpret_cast<u32x2 *>(acts + (size_t)(first + j - acts_pair_base) * f + row0) = u32x2{packed[0], packed[1]};   // whole tiles: f % 4 == 0
                 }
             }
         }
@@ -898,19 +945,17 @@ __global__ __launch_bounds__(256, 4) void grouped_down_quad_kernel(ExpertTable t
                 request(next, tile + 4, p);
                 quad_pass<QC, NPASS, SD, G>(ow, ws, wb, qm.col(p), qm, xa, xsum, nch, pieces, nb, groups_of_pairs, acc);
             }
-            const long row0 = (long)tile * Map::kRows + qm.rg * 4;
+            const long row0 = (long)tile * Map::kRows + qm.rg * 4 + qm.m;   // this lane's row
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 if (g < groups_of_pairs) {
-                    uint32_t packed[2];
 #pragma unroll
-                    for (int k = 0; k < 4; ++k) {
-                        const uint32_t h = f32_to_f16_bits(quad_sum<QC>(acc[g][k]));
-                        packed[k >> 1] = (k & 1) ? (packed[k >> 1] | (h << 16)) : h;
+                    for (int i = 0; i < 4; ++i) {
+                        const half_t h = (half_t)quad_sum<QC>(acc[g][i]);
+                        const uint32_t j = 4 * g + i;
+                        if ((lane & 31) < 4 && j < nb)   // lanes 0..3: rows of group 0; lanes 32..35: rows of group 1
+                            route_partials[(size_t)out_row[j] * d + row0] = h;
                     }
-                    const uint32_t j = 4 * g + (lane & 3);
-                    if ((lane & 31) < 4 && j < nb)       // lanes 0..3: rows of group 0; lanes 32..35: rows of group 1
-                        *reinterpret_cast<u32x2 *>(route_partials + (size_t)out_row[j] * d + row0) = u32x2{packed[0], packed[1]};   // whole tiles: d % 8 == 0
                 }
             }
         }
@@ -1401,6 +1446,66 @@ int32_t tf_prefill_group_pairs_device(tf_ctx *ctx, tf_stream stream, const void 
     hipLaunchKernelGGL(group_place_kernel, dim3(n_segments), dim3(64), 0, st, idx, static_cast<const uint16_t *>(weights), n_pairs,
                        seg_pairs, top_k, num_experts, ctx->group_scratch, static_cast<tf_prefill_pair *>(sorted_pairs));
     return check_launch(ctx, "group_pairs_device");
+}
+
+int32_t tf_prefill_router_group_block(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t weights_offset, const void *scales,
+                                      uint64_t scales_offset, const void *biases, uint64_t biases_offset, const void *hidden,
+                                      uint64_t hidden_offset, const void *effective_scale, uint64_t effective_scale_offset,
+                                      const void *per_expert_scale, uint64_t per_expert_scale_offset, void *out_indices,
+                                      uint64_t out_indices_offset, void *out_weights, uint64_t out_weights_offset, uint32_t query_count,
+                                      uint32_t num_experts, uint32_t d, uint32_t top_k, uint32_t hidden_stride_elements, void *sorted_pairs,
+                                      void *per_expert_offsets, void *per_expert_counts, void *chunks, void *chunk_count) {
+    // both calls' argument checks first, so that a refused call has launched nothing
+    TF_REQUIRE(ctx, ctx && weights && scales && biases && hidden && effective_scale && per_expert_scale && out_indices && out_weights &&
+                        sorted_pairs && per_expert_offsets && per_expert_counts && chunks && chunk_count,
+               TF_ERR_INVALID_ARGUMENT, "prefill_router_group: null argument");
+    TF_REQUIRE(ctx, query_count > 0 && num_experts > 0 && num_experts <= 256 && top_k > 0 && top_k <= 64 && d > 0 && d % TF_GROUP_SIZE == 0 &&
+                        hidden_stride_elements >= d,
+               TF_ERR_INVALID_ARGUMENT, "prefill_router_group: need queryCount > 0, 1 <= numExperts <= 256, 1 <= topK <= 64, D a multiple of 64, hidden stride >= D");
+    const uint8_t *w = at(weights, weights_offset);
+    const uint8_t *s = at(scales, scales_offset), *b = at(biases, biases_offset);
+    const half_t *h = reinterpret_cast<const half_t *>(at(hidden, hidden_offset));
+    const uint16_t *eff = reinterpret_cast<const uint16_t *>(at(effective_scale, effective_scale_offset));
+    const uint16_t *pes = reinterpret_cast<const uint16_t *>(at(per_expert_scale, per_expert_scale_offset));
+    uint32_t *oi = reinterpret_cast<uint32_t *>(at(out_indices, out_indices_offset));
+    half_t *ow = reinterpret_cast<half_t *>(at(out_weights, out_weights_offset));
+    TF_REQUIRE(ctx, aligned(s, 2) && aligned(b, 2) && aligned(h, 2) && aligned(eff, 2) && aligned(pes, 2) && aligned(oi, 4) && aligned(ow, 2) &&
+                        aligned(sorted_pairs, 4) && aligned(chunks, 4) && aligned(per_expert_offsets, 4) && aligned(per_expert_counts, 4) &&
+                        aligned(chunk_count, 4),
+               TF_ERR_INVALID_ARGUMENT, "prefill_router_group: misaligned operand");
+    const size_t need = std::max<size_t>((size_t)kFewTokens * 256, (size_t)query_count * num_experts);
+    if (query_count <= kFewTokens && ctx->prefill_logits_count < need)
+        return scratch_too_small(ctx, "prefill_router", need * sizeof(float), ctx->prefill_logits_count * sizeof(float));
+    if (query_count <= kSelectGroupTokens && top_k <= kSelectGroupTopK) {
+        const bool fast = aligned16(w) && aligned16(h) && aligned16(eff) && hidden_stride_elements % 8 == 0 && d <= 4096;
+        const int npass = fast ? (int)((d / 16 + 63) / 64) : 0;
+        hipStream_t st = static_cast<hipStream_t>(stream);
+        const dim3 grid((num_experts + 3) / 4, query_count);
+#define TF_PL(NP_)                                                                                                           \
+    hipLaunchKernelGGL(prefill_logits_kernel<NP_>, grid, dim3(256), 0, st, w, s, b, h, (long)hidden_stride_elements, eff,    \
+                       ctx->prefill_logits, num_experts, (int)d)
+        switch (npass) {
+            case 1: TF_PL(1); break;
+            case 2: TF_PL(2); break;
+            case 3: TF_PL(3); break;
+            case 4: TF_PL(4); break;
+            default: TF_PL(0); break;
+        }
+#undef TF_PL
+        const int32_t rc = check_launch(ctx, "prefill_router logits");
+        if (rc != TF_OK) return rc;
+        hipLaunchKernelGGL(select_group_small_kernel, dim3(1), dim3(1024), 0, st, ctx->prefill_logits, pes, oi, ow, query_count, num_experts, top_k,
+                           static_cast<tf_prefill_pair *>(sorted_pairs), static_cast<uint32_t *>(per_expert_offsets),
+                           static_cast<uint32_t *>(per_expert_counts), static_cast<tf_prefill_group *>(chunks), static_cast<uint32_t *>(chunk_count));
+        return check_launch(ctx, "prefill_router select + group");
+    }
+    const int32_t rc = tf_prefill_router_gemma4_block(ctx, stream, weights, weights_offset, scales, scales_offset, biases, biases_offset, hidden,
+                                                      hidden_offset, effective_scale, effective_scale_offset, per_expert_scale,
+                                                      per_expert_scale_offset, out_indices, out_indices_offset, out_weights, out_weights_offset,
+                                                      query_count, num_experts, d, top_k, hidden_stride_elements);
+    if (rc != TF_OK) return rc;
+    return tf_prefill_group_pairs_device(ctx, stream, oi, ow, query_count, top_k, num_experts, sorted_pairs, per_expert_offsets, per_expert_counts,
+                                         chunks, chunk_count);
 }
 
 int32_t tf_prefill_grouped_routed_moe_streamed(tf_ctx *ctx, tf_stream stream, const void *hidden, uint64_t hidden_offset,

@@ -185,7 +185,10 @@ struct XStage {
     }
 
     // piece = 8 consecutive activations = word (piece & 3) of chunk column (piece >> 2)
-    static __device__ __forceinline__ void publish_piece(const u32x4 raw, int piece, int pieces, int nch, u32x4 *xa, float *xsum) {
+    // xsum_stride: distance between the sums of neighbouring columns (1: one vector's sums side by side; a caller that keeps
+    // several vectors' sums interleaved per column passes their count)
+    static __device__ __forceinline__ void publish_piece(const u32x4 raw, int piece, int pieces, int nch, u32x4 *xa, float *xsum,
+                                                         int xsum_stride = 1) {
         const half2_t sixteenth = {(half_t)0.0625f, (half_t)0.0625f};
         const uint32_t p01 = raw[0], p23 = raw[1], p45 = raw[2], p67 = raw[3];
         u32x4 o;
@@ -204,7 +207,7 @@ struct XStage {
         sum += dpp_f32<0x4E>(sum);
         if (piece < pieces) {
             xa[(piece & 3) * nch + (piece >> 2)] = o;
-            if ((piece & 3) == 0) xsum[piece >> 2] = sum;
+            if ((piece & 3) == 0) xsum[(piece >> 2) * xsum_stride] = sum;
         }
     }
 
