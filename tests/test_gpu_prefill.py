@@ -504,6 +504,38 @@ def test_int4_qmm_on_matrix_cores(m, n, k, adv):
     assert within_north_star(got, want)
 
 
+@pytest.mark.parametrize("m,n,k,lo,hi,mixed", [(64, 128, 2816, 2e-6, 5e-5, False), (40, 96, 704, 1e-7, 3e-6, False), (33, 64, 2112, 3e-5, 9e-5, False),
+                                                (48, 160, 1408, 1e-6, 4e-5, True)])
+def test_int4_qmm_on_matrix_cores_with_scales_below_fp16_normal_range(m, n, k, lo, hi, mixed):
+    # The reference's staged-affine path forms half(fma(float(q), scale, bias)) in fp32 (Metal/TensorCore/tensorops.metal:73-75), so a
+    # bf16 scale of any size keeps its mantissa.  Scales of 1e-7 ... 9e-5 lie below or across the bottom of fp16's normal range
+    # (6.1e-5): the matrix-core path carries every weight row times a power of two and must still meet the MPP tolerance.
+    rng = np.random.default_rng(int(k + m))
+    groups = k // 64
+    W = rng.integers(0, 256, (n, k // 2), dtype=np.uint8)
+    s = rng.uniform(lo, hi, (n, groups)).astype(np.float32)
+    if mixed:   # every third row has ordinary scales: rows of both kinds share a wave, each is carried at its own power of two
+        s[::3] = rng.uniform(0.004, 0.02, s[::3].shape).astype(np.float32)
+    S = tfo.bf16_bits_array(s).reshape(n, groups)
+    B = tfo.bf16_bits_array((-7.5 * s * rng.uniform(0.5, 1.5, (n, groups))).astype(np.float32)).reshape(n, groups)
+    x = tfo.to_f16_bits(rng.standard_normal(m * k).astype(np.float32) * 4.0)
+    kk = ctx()
+    y = zeros_bytes(m * n * 2)
+    dW, dS, dB, dx = dev(W), dev(S), dev(B), dev(x)
+    assert kk.lib.tf_int4_qmm(kk.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dx.data_ptr(), 0, y.data_ptr(), 0, m, n, k,
+                              tfk.TF_BF16) == tfk.TF_OK
+    got = tfo.from_f16_bits(host(y, np.uint16, m * n)).reshape(m, n).astype(np.float64)
+    # fp64 reference from the fp32 weights float(q) * s + b (what every path approximates), beside the reference's own fp32 loop
+    nib = np.stack([W & 0xF, W >> 4], axis=2).reshape(n, k).astype(np.float32)
+    wf = (nib * np.repeat(tfo.bf16_array_to_float(S.ravel()).reshape(n, groups), 64, axis=1)
+          + np.repeat(tfo.bf16_array_to_float(B.ravel()).reshape(n, groups), 64, axis=1)).astype(np.float64)
+    exact = tfo.from_f16_bits(x).reshape(m, k).astype(np.float64) @ wf.T
+    scale = np.max(np.abs(exact), axis=0)   # per weight row: a tiny row beside an ordinary one is held to its own size
+    assert np.all(np.abs(got - exact) <= 1e-3 * scale[None, :]), float(np.max(np.abs(got - exact) / scale[None, :]))
+    want = tfo.qmm_cpu_reference(W, S, B, x, m, n, k, threads=8)
+    assert tfo.rel_error(got.astype(np.float32), want) <= 1e-3
+
+
 def test_int4_qmm_unavailable_and_exact_variant():
     W, S, B, x = mpp_inputs(8, 64, 128)
     kk = ctx()

@@ -9,6 +9,7 @@ namespace {
 
 // The wave's weight rows: column tile j covers rows row0[j] .. row0[j] + 31 of a matrix of `limit[j]` rows that starts
 // at w / s / b.
+template <int SD>
 __device__ __forceinline__ QmmBRows make_b_rows(const uint8_t *const w[2], const uint8_t *const s[2], const uint8_t *const b[2],
                                                 const int row0[2], const int limit[2], int row_bytes, int groups, int lane) {
     QmmBRows rows;
@@ -25,6 +26,14 @@ __device__ __forceinline__ QmmBRows make_b_rows(const uint8_t *const w[2], const
         const int piece = (lane & 3) ^ ((r >> 2) & 3);
         rows.copy_off[t] = (uint32_t)(row0[t >> 1] + r) * (uint32_t)row_bytes + (uint32_t)piece * 16u;
     }
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        rows.pre[j] = 0u;
+        rows.post[j] = 1.0f;
+        const uint32_t array_bytes = (uint32_t)limit[j] * (uint32_t)groups * 2u;
+        rows.scan_off[j] = min(rows.sb_off[j], array_bytes - (uint32_t)groups * 2u);   // a column past the matrix: its last row (never stored)
+    }
+    rows.groups = groups;
     return rows;
 }
 
@@ -124,7 +133,7 @@ __device__ __forceinline__ void qmm_dense_body(const DenseArgs &a, uint32_t id, 
     for (int q = 0; q < QmmGeom<4>::kAChunks; ++q) qmm_a_rows_set(arow, q, (uint64_t)min(m0 + qmm_a_row_of<4>(q), M - 1) * (uint64_t)ldx * 2u);
     const uint8_t *w[2] = {W, W}, *s[2] = {S, S}, *b[2] = {B, B};
     const int row0[2] = {n0, n0 + 32}, limit[2] = {N, N};
-    const QmmBRows rows = make_b_rows(w, s, b, row0, limit, K >> 1, K >> 6, lane);
+    QmmBRows rows = make_b_rows<SD>(w, s, b, row0, limit, K >> 1, K >> 6, lane);
     const int row_tiles = min(4, (M - m0 + 31) >> 5);
     float16_t acc[4][2];
     zero_acc(acc);
@@ -137,7 +146,7 @@ __device__ __forceinline__ void qmm_dense_body(const DenseArgs &a, uint32_t id, 
             for (int mt = 0; mt < 4; ++mt)
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
-                    out_tile_put<kQmmBN>(lds, mt * 32 + acc_row(r, lane), wave * kQmmWaveN + j * 32 + acc_col(lane), acc[mt][j][r]);
+                    out_tile_put<kQmmBN>(lds, mt * 32 + acc_row(r, lane), wave * kQmmWaveN + j * 32 + acc_col(lane), acc[mt][j][r] * rows.post[j]);
         const int nb = (int)col_tile * kQmmBN;
         out_tile_store<kQmmBN>(lds, min(kQmmBM, M - m0), min(kQmmBN, N - nb), [&](int row) { return Y + (size_t)(m0 + row) * ldy + nb; });
         return;
@@ -150,7 +159,7 @@ __device__ __forceinline__ void qmm_dense_body(const DenseArgs &a, uint32_t id, 
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int m = m0 + mt * 32 + acc_row(r, lane);
-                if (m < M && n < N) Y[(size_t)m * ldy + n] = (half_t)acc[mt][j][r];
+                if (m < M && n < N) Y[(size_t)m * ldy + n] = (half_t)(acc[mt][j][r] * rows.post[j]);
             }
     }
 }
@@ -190,7 +199,7 @@ __device__ __forceinline__ void qmm_dense_geglu_body(const DenseGegluArgs &a, ui
     for (int q = 0; q < QmmGeom<4>::kAChunks; ++q) qmm_a_rows_set(arow, q, (uint64_t)min(m0 + qmm_a_row_of<4>(q), M - 1) * (uint64_t)ldx * 2u);
     const uint8_t *w[2] = {gW, uW}, *s[2] = {gS, uS}, *b[2] = {gB, uB};
     const int row0[2] = {n0, n0}, limit[2] = {F, F};
-    const QmmBRows rows = make_b_rows(w, s, b, row0, limit, K >> 1, K >> 6, lane);
+    QmmBRows rows = make_b_rows<SD>(w, s, b, row0, limit, K >> 1, K >> 6, lane);
     const int row_tiles = min(4, (M - m0 + 31) >> 5);
     float16_t acc[4][2];
     zero_acc(acc);
@@ -201,7 +210,7 @@ __device__ __forceinline__ void qmm_dense_geglu_body(const DenseGegluArgs &a, ui
         if (mt >= row_tiles) break;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float gate = (float)(half_t)acc[mt][0][r], up = (float)(half_t)acc[mt][1][r];
+            const float gate = (float)(half_t)(acc[mt][0][r] * rows.post[0]), up = (float)(half_t)(acc[mt][1][r] * rows.post[1]);
             out_tile_put<kGegluBN>(lds, mt * 32 + acc_row(r, lane), wave * 32 + acc_col(lane), gelu_tanh_fast(gate) * up);
         }
     }
@@ -290,7 +299,7 @@ __device__ __forceinline__ void grouped_phase1_body(const GroupedP1Args &a, uint
     const uint8_t *s[2] = {base + off.gate_s_off, base + off.up_s_off};
     const uint8_t *b[2] = {base + off.gate_b_off, base + off.up_b_off};
     const int row0[2] = {n0, n0}, limit[2] = {F, F};
-    const QmmBRows rows = make_b_rows(w, s, b, row0, limit, D >> 1, D >> 6, lane);
+    QmmBRows rows = make_b_rows<SD>(w, s, b, row0, limit, D >> 1, D >> 6, lane);
     const int row_tiles = (int)((ch.pair_count + 31) >> 5);
     float16_t acc[4][2];
     zero_acc(acc);
@@ -302,7 +311,8 @@ __device__ __forceinline__ void grouped_phase1_body(const GroupedP1Args &a, uint
         if (mt >= row_tiles) break;   // tiles without rows were not multiplied and are not stored
 #pragma unroll
         for (int r = 0; r < 16; ++r)
-            out_tile_put<kP1BN>(lds, mt * 32 + acc_row(r, lane), wave * 32 + acc_col(lane), gelu_tanh_fast(acc[mt][0][r]) * acc[mt][1][r]);
+            out_tile_put<kP1BN>(lds, mt * 32 + acc_row(r, lane), wave * 32 + acc_col(lane),
+                                gelu_tanh_fast(acc[mt][0][r] * rows.post[0]) * (acc[mt][1][r] * rows.post[1]));
     }
     const int nb = (int)col_tile * kP1BN;
     half_t *tile = acts + (size_t)(ch.pair_start - acts_pair_base) * F + nb;
@@ -373,7 +383,7 @@ __device__ __forceinline__ void grouped_down_body(const GroupedDownArgs &a, uint
     const uint8_t *s[2] = {base + off.down_s_off, base + off.down_s_off};
     const uint8_t *b[2] = {base + off.down_b_off, base + off.down_b_off};
     const int row0[2] = {n0, n0 + 32}, limit[2] = {D, D};
-    const QmmBRows rows = make_b_rows(w, s, b, row0, limit, F >> 1, F >> 6, lane);
+    QmmBRows rows = make_b_rows<SD>(w, s, b, row0, limit, F >> 1, F >> 6, lane);
     const int row_tiles = (int)((ch.pair_count + 31) >> 5);
     float16_t acc[4][2];
     zero_acc(acc);
@@ -391,7 +401,7 @@ __device__ __forceinline__ void grouped_down_body(const GroupedDownArgs &a, uint
         for (int j = 0; j < 2; ++j)
 #pragma unroll
             for (int r = 0; r < 16; ++r)
-                out_tile_put<kDownBN>(lds, mt * 32 + acc_row(r, lane), wave * kQmmWaveN + j * 32 + acc_col(lane), acc[mt][j][r]);
+                out_tile_put<kDownBN>(lds, mt * 32 + acc_row(r, lane), wave * kQmmWaveN + j * 32 + acc_col(lane), acc[mt][j][r] * rows.post[j]);
     const int nb = (int)col_tile * kDownBN;
     out_tile_store<kDownBN>(lds, (int)ch.pair_count, min(kDownBN, D - nb), [&](int row) { return route_partials + (size_t)row_slot[row] * D + nb; });
 }

@@ -70,9 +70,14 @@ __device__ __forceinline__ half8_t dequant_word(uint32_t v, half2_t s2, half2_t 
     return half8_t{w[0][0], w[0][1], w[1][0], w[1][1], w[2][0], w[2][1], w[3][0], w[3][1]};
 }
 
+// A bf16 scale or bias times the row's power of two, as an fp16 pair.  The power of two goes into the exponent field while the
+// value is widened to fp32 (one shift-and-add instead of a shift): exact for every normal value, since the row's largest value
+// bounds the sum of the fields; zeros and subnormals come out below 2^-26 and round to fp16 zero.
 template <int SD>
-__device__ __forceinline__ half2_t sb_to_half2(uint16_t v) {
-    const half_t h = (half_t)sb_to_f32<SD>(v);
+__device__ __forceinline__ half2_t sb_to_half2(uint16_t v, uint32_t pre) {
+    half_t h;
+    if constexpr (SD == 0) h = (half_t)__uint_as_float(((uint32_t)v << 16) + pre);
+    else h = (half_t)sb_to_f32<SD>(v);          // fp16 scales are what they are
     return half2_t{h, h};
 }
 
@@ -108,15 +113,80 @@ __device__ __forceinline__ void qmm_a_rows_set(QmmARows<NW> &a, int q, uint64_t 
 //                tile t / 2, 16-byte piece (lane & 3) ^ ((row / 4) & 3) of the row's 64 bytes (the XOR keeps the later
 //                reads free of bank conflicts);
 //   sb_off[j]:   the lane's own row (lane & 31) of tile j in the scale / bias arrays.
+//   pre[j] / post[j]: a power of two 2^e per weight row (as e << 23, added to a value's fp32 bits) and 2^-e.  The expansion
+//                computes half(q s + b) with fp16 copies of s and b; a bf16 scale below fp16's normal range (6.1e-5) would lose
+//                mantissa bits in that copy.  A wave whose first two groups show such a scale (qmm_normalise_small_rows) scans
+//                its rows' scales and biases once, multiplies them by 2^e on their way into the expansion, with e chosen from
+//                the largest of them over the whole row so that every |q s + b| 2^e stays below 2^15, and multiplies the rows'
+//                sums by 2^-e when they leave.  Both scalings are exact: half((q s + b) 2^e) = half(q s + b) 2^e wherever the
+//                right side is a normal fp16 number, and where it is not (weights below 6.1e-5) the scaled form keeps the
+//                mantissa the unscaled one drops.  Rows whose first groups have ordinary scales are left alone (e = 0): a later
+//                group with a tiny scale then carries at most 15 x 2^-25 of absolute error per weight, next to weights of at
+//                least 6.1e-5 in the same row.
+//   scan_off[j], groups: the lane's row in the scale / bias arrays (clamped into the matrix) and its length, for that scan.
 struct QmmBRows {
     qmm_rsrc_t w[2], s[2], b[2];
     uint32_t copy_off[4];
     uint32_t sb_off[2];
+    uint32_t pre[2];
+    float post[2];
+    uint32_t scan_off[2];
+    int groups;
 };
 // scales and biases of the lane's rows for two consecutive groups (low half: even group)
 struct QmmSB {
     uint32_t s[2], b[2];
 };
+// Largest biased exponent field among the bf16 values of a row of `row_bytes` bytes (>= 16) that starts `row_off` bytes into
+// `rsrc`; 0 when all are zero or subnormal.  The row is read in 16-byte pieces, all requested before the first is looked at;
+// the last piece ends with the row (it may overlap the one before: a maximum does not mind), so nothing outside the row is read
+// and nothing needs masking.  The exponent fields of a word's two values are compared in place with packed 16-bit maxima.
+typedef unsigned short u16x2 __attribute__((ext_vector_type(2)));
+template <int PIECES>
+__device__ __forceinline__ uint32_t row_max_exponent(qmm_rsrc_t rsrc, uint32_t row_off, uint32_t row_bytes) {
+    u32x4 v[PIECES];
+#pragma unroll
+    for (int p = 0; p < PIECES; ++p)
+        v[p] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(rsrc, row_off + min(16u * p, row_bytes - 16u), 0, 0));
+    u16x2 m = {0, 0};
+#pragma unroll
+    for (int p = 0; p < PIECES; ++p)
+#pragma unroll
+        for (int w = 0; w < 4; ++w) m = __builtin_elementwise_max(m, __builtin_bit_cast(u16x2, v[p][w] & 0x7F807F80u));
+    return (uint32_t)max(m[0], m[1]) >> 7;
+}
+__device__ __forceinline__ uint32_t row_max_exponent_any(qmm_rsrc_t rsrc, uint32_t row_off, int groups) {
+    const uint32_t row_bytes = (uint32_t)groups * 2u;
+    uint32_t e = 0;
+    if (groups < 8) {   // rows of fewer than 8 values: value by value
+        for (int g = 0; g < groups; ++g) e = max(e, ((uint32_t)__builtin_amdgcn_raw_buffer_load_b16(rsrc, row_off + 2u * g, 0, 0) >> 7) & 0xFFu);
+        return e;
+    }
+    for (uint32_t done = 0; done < row_bytes; done += 128u)      // 128 bytes (a row of 4096 columns) a round trip
+        e = max(e, row_max_exponent<8>(rsrc, row_off + min(done, row_bytes - 16u), min(128u, max(row_bytes - done, 16u))));
+    return e;
+}
+// sb: the scales of the wave's first two groups.  Wave-uniform decision; only bf16 scales need it.
+__device__ __forceinline__ void qmm_normalise_small_rows(QmmBRows &rows, const uint32_t first_scales[2]) {
+    bool small = false;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t lo = (first_scales[j] >> 7) & 0xFFu, hi = (first_scales[j] >> 23) & 0xFFu;   // exponent fields of the two bf16 values
+        small = small || (lo != 0u && lo < 113u) || (hi != 0u && hi < 113u);                        // 2^-14 = fp16's smallest normal number
+    }
+    if (__builtin_amdgcn_ballot_w64(small) == 0ull) return;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        // every |s| < 2^(es - 126) and every |b| < 2^(eb - 126): with top = max(es + 4, eb), 15 |s| and |b| lie below 2^(top - 126),
+        // and 2^(140 - top) brings them below 2^14, their sum below 2^15
+        const uint32_t es = row_max_exponent_any(rows.s[j], rows.scan_off[j], rows.groups), eb = row_max_exponent_any(rows.b[j], rows.scan_off[j], rows.groups);
+        const uint32_t top = max(es + 4u, eb);
+        const int shift = top == 0u ? 0 : min(max(140 - (int)top, -100), 100);
+        rows.pre[j] = (uint32_t)shift << 23;
+        rows.post[j] = __uint_as_float((uint32_t)(127 - shift) << 23);
+    }
+}
+
 // single (wave-uniform): the pair has only its first group (the last pair of an odd number of groups); a 32-bit load
 // would run past the end of the last row.  Both arms issue the same number of loads.
 __device__ __forceinline__ void qmm_sb_load(QmmSB &sb, const QmmBRows &rows, int pair, bool single) {
@@ -164,12 +234,13 @@ __device__ __forceinline__ u32x4 lds_read16(uint32_t addr) {
 // The fragments of MFMA group d + 1 are requested before group d is multiplied, and the weights of group d + 1 are
 // expanded between the MFMAs of group d.
 template <int SD, int RT, int STAGE, int HALF>
-__device__ __forceinline__ void qmm_group(const u32x4 w[2], const QmmSB &sb, const uint32_t frag[4], const NibbleConsts &nc, float16_t acc[4][2]) {
+__device__ __forceinline__ void qmm_group(const u32x4 w[2], const QmmSB &sb, const uint32_t pre[2], const uint32_t frag[4], const NibbleConsts &nc,
+                                          float16_t acc[4][2]) {
     half2_t s2[2], b2[2];
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        s2[j] = sb_to_half2<SD>((uint16_t)(HALF ? sb.s[j] >> 16 : sb.s[j] & 0xFFFFu));
-        b2[j] = sb_to_half2<SD>((uint16_t)(HALF ? sb.b[j] >> 16 : sb.b[j] & 0xFFFFu));
+        s2[j] = sb_to_half2<SD>((uint16_t)(HALF ? sb.s[j] >> 16 : sb.s[j] & 0xFFFFu), pre[j]);
+        b2[j] = sb_to_half2<SD>((uint16_t)(HALF ? sb.b[j] >> 16 : sb.b[j] & 0xFFFFu), pre[j]);
     }
     constexpr int base = STAGE * kQmmStageBytes;
     half8_t bf0 = dequant_word(w[0][0], s2[0], b2[0], nc);
@@ -232,7 +303,7 @@ struct QmmLoop {
     // of them (the others re-read valid rows out of L2): without them chunks of 32 to 128 tokens measured 5 % slower.
     static constexpr int AC = RT == 1 ? QmmGeom<NW>::kAChunks : (4 * RT + NW - 1) / NW;
     const QmmARows<NW> &a;
-    const QmmBRows &rows;
+    QmmBRows &rows;
     uint32_t lds;
     uint32_t frag[4];
     uint32_t wread;      // this lane's 16 bytes of column tile 0, first step of a pair, in the wave's W buffer 0
@@ -258,7 +329,7 @@ struct QmmLoop {
         __builtin_amdgcn_s_barrier();
         qmm_a_copy<NW, AC>(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
         qmm_w_copy(rows, min(pair + 1, last_pair), wbuf + (pb ^ kQmmWBytes));
-        qmm_group<SD, RT, U3, 0>(w[0], sb, frag, nc, acc);
+        qmm_group<SD, RT, U3, 0>(w[0], sb, rows.pre, frag, nc, acc);
         const int next_pair = min(pair + 1, last_pair);
         qmm_sb_load(sb_next, rows, next_pair, odd_count && next_pair == last_pair);
         // everything older than this step's AC + 4 + 4 requests (X, W, scales and biases) has landed
@@ -268,7 +339,7 @@ struct QmmLoop {
     __device__ __forceinline__ void odd_step(int kt, float16_t acc[4][2]) {
         __builtin_amdgcn_s_barrier();
         qmm_a_copy<NW, AC>(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
-        qmm_group<SD, RT, U3, 1>(w[1], sb, frag, nc, acc);
+        qmm_group<SD, RT, U3, 1>(w[1], sb, rows.pre, frag, nc, acc);
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AC) : "memory");   // only this step's X copies may still be on their way
         pb ^= kQmmWBytes;
         read_w(wread + pb);
@@ -292,6 +363,7 @@ struct QmmLoop {
         qmm_w_copy(rows, 0, wbuf);
         qmm_sb_load(sb, rows, 0, odd_count && last_pair == 0);
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if constexpr (SD == 0) qmm_normalise_small_rows(rows, sb.s);
         read_w(wread);
         int kt0 = 0;
         for (; kt0 + 6 <= kt_count; kt0 += 6) {
@@ -313,7 +385,7 @@ struct QmmLoop {
 };
 
 template <int SD, int RT, int NW>
-__device__ __forceinline__ void qmm_k_loop_rt(int kt_count, const QmmARows<NW> &a, const QmmBRows &rows, uint32_t lds, int lane,
+__device__ __forceinline__ void qmm_k_loop_rt(int kt_count, const QmmARows<NW> &a, QmmBRows &rows, uint32_t lds, int lane,
                                               float16_t acc[4][2]) {
     QmmLoop<SD, RT, NW> loop{a, rows, lds};
     loop.run(kt_count, lane, acc);
@@ -322,7 +394,7 @@ __device__ __forceinline__ void qmm_k_loop_rt(int kt_count, const QmmARows<NW> &
 // row_tiles (1..4, block-uniform): 32-row tiles that hold rows; the others are not multiplied.
 // lds: byte address of QmmGeom<NW>::kLoopLdsBytes of LDS, 128-byte aligned.
 template <int SD, int NW>
-__device__ __forceinline__ void qmm_k_loop(int kt_count, const QmmARows<NW> &a, const QmmBRows &rows, uint32_t lds, int lane,
+__device__ __forceinline__ void qmm_k_loop(int kt_count, const QmmARows<NW> &a, QmmBRows &rows, uint32_t lds, int lane,
                                            int row_tiles, float16_t acc[4][2]) {
     switch (row_tiles) {
         case 1: qmm_k_loop_rt<SD, 1, NW>(kt_count, a, rows, lds, lane, acc); break;
