@@ -4,8 +4,8 @@
 //
 //   W   In v_mfma_f32_32x32x16_f16 lane (i, kb) supplies, for output column i, the 8 weights of k-slots 8 kb .. 8 kb + 7.
 //       The lane reads 16 packed bytes of "its" row (32 nibbles: the kb-th half of the group) and expands one 32-bit
-//       word (8 nibbles) per MFMA straight into the operand registers as half(q * s + b), the rounding point of the
-//       reference's staged-affine path (tensorops.metal:57-94).  MFMA number d of the group then covers
+//       word (8 nibbles) per MFMA round straight into the operand registers as half(q * s + b), the rounding point of the
+//       reference's staged-affine path (tensorops.metal:57-94).  MFMA round d of the group then covers
 //       k = {8d .. 8d+7} u {32+8d .. 32+8d+7}.  Reading "its" row straight from global memory would touch 32 cache
 //       lines per load instruction; instead the load unit copies the packed rows into a wave-private LDS area two K
 //       steps at a time (64 contiguous bytes per row, four lanes per row), and the lanes pick their 16 bytes there.
@@ -14,9 +14,14 @@
 //       no vector instructions), two K steps ahead, into a ring of three stages shared by the four waves.  A stage is
 //       128 rows x 8 chunks of 16 bytes; chunk c of row r sits at position c ^ ((r >> 1) & 7) of its row, which keeps
 //       the fragment reads free of bank conflicts although the copies land contiguously.
-//   The fragment reads are software-pipelined by hand (the fragments of MFMA group d + 1 are requested before group d
-//   is multiplied) and written as inline assembly with explicit waits: the compiler would otherwise make every LDS read
-//   wait for all outstanding copies, the prefetched ones included.
+//   The instruction stream of a K step is placed by hand: every MFMA, fragment read, wait and expansion instruction is a
+//   volatile asm statement, in the order it is to issue.  Measured on this part, a wave's own vector instructions issue in
+//   the shadow of its MFMAs as long as there are at most about five of them per MFMA (an MFMA holds the issue port for some
+//   10 of its 32 cycles; with eight instructions per MFMA the pair takes 44 cycles instead of 32), and only when they are
+//   spread out: left to the compiler, the 16 instructions that expand a word clump together between runs of back-to-back
+//   MFMAs.  So a round (the 2 RT MFMAs of one 16-wide K slice) carries the expansion of the next round's two words in eight
+//   parts of four instructions, one or more behind each MFMA; the last round of a step expands the first words of the next
+//   step and reads that step's first fragments, after the block's one barrier of the step.
 //
 // Row indirection makes the same loop serve the grouped expert GEMMs: X rows can be gathered through a row table
 // (tokens routed to one expert) and Y rows scattered through another; row tiles beyond the rows present are skipped.
@@ -44,31 +49,6 @@ struct QmmGeom {
 };
 constexpr int kQmmBN = QmmGeom<4>::kBN;
 constexpr int kQmmLdsBytes = QmmGeom<4>::kLoopLdsBytes;
-
-// 8 nibbles of one word -> 8 fp16 weights half(q * s + b) in element order.  A byte holds two neighbouring elements:
-// v_perm_b32 copies it into both halves of a register, one v_and_or_b32 leaves the low nibble in the low half as
-// 1024 + q (0x6400 | q) and the high nibble in place in the high half as 64 + q (0x5400 | q << 4); both offsets are
-// removed exactly, and q * s + b is one fp16 fused multiply-add on fp16 copies of s and b: four instructions a pair.
-// v_and_or_b32 takes no literal operands, so mask and exponent bits live in registers (see nibble_consts()).
-struct NibbleConsts {
-    uint32_t mask, exponents;
-};
-__device__ __forceinline__ NibbleConsts nibble_consts() {
-    NibbleConsts c{0x00F0000Fu, 0x54006400u};
-    asm("" : "+v"(c.mask), "+v"(c.exponents));   // opaque: kept in registers instead of being re-materialised as literals
-    return c;
-}
-__device__ __forceinline__ half8_t dequant_word(uint32_t v, half2_t s2, half2_t b2, const NibbleConsts &c) {
-    const half2_t offs = {(half_t)1024.0f, (half_t)64.0f};
-    half2_t w[4];
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const uint32_t both = __builtin_amdgcn_perm(0u, v, 0x0c000c00u | ((uint32_t)p << 16) | (uint32_t)p);
-        const half2_t q = as_half2((both & c.mask) | c.exponents) - offs;
-        w[p] = __builtin_elementwise_fma(q, s2, b2);
-    }
-    return half8_t{w[0][0], w[0][1], w[1][0], w[1][1], w[2][0], w[2][1], w[3][0], w[3][1]};
-}
 
 // A bf16 scale or bias times the row's power of two, as an fp16 pair.  The power of two goes into the exponent field while the
 // value is widened to fp32 (one shift-and-add instead of a shift): exact for every normal value, since the row's largest value
@@ -229,121 +209,161 @@ __device__ __forceinline__ u32x4 lds_read16(uint32_t addr) {
     return v;
 }
 
-// One K group for this wave: acc[mt][j] += X[mt*32.., group] . W_j[.., group]^T for the row tiles mt < RT, out of LDS
-// stage STAGE.  frag[d]: LDS byte address of this lane's fragment for MFMA d in row tile 0 of stage 0.
-// The fragments of MFMA group d + 1 are requested before group d is multiplied, and the weights of group d + 1 are
-// expanded between the MFMAs of group d.
-template <int SD, int RT, int STAGE, int HALF>
-__device__ __forceinline__ void qmm_group(const u32x4 w[2], const QmmSB &sb, const uint32_t pre[2], const uint32_t frag[4], const NibbleConsts &nc,
-                                          float16_t acc[4][2]) {
-    half2_t s2[2], b2[2];
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        s2[j] = sb_to_half2<SD>((uint16_t)(HALF ? sb.s[j] >> 16 : sb.s[j] & 0xFFFFu), pre[j]);
-        b2[j] = sb_to_half2<SD>((uint16_t)(HALF ? sb.b[j] >> 16 : sb.b[j] & 0xFFFFu), pre[j]);
-    }
-    constexpr int base = STAGE * kQmmStageBytes;
-    half8_t bf0 = dequant_word(w[0][0], s2[0], b2[0], nc);
-    half8_t bf1 = dequant_word(w[1][0], s2[1], b2[1], nc);
-    u32x4 af[2][4];
-    af[0][0] = lds_read16<base>(frag[0]);
-    if constexpr (RT > 1) af[0][1] = lds_read16<base + 4096>(frag[0]);
-    if constexpr (RT > 2) af[0][2] = lds_read16<base + 8192>(frag[0]);
-    if constexpr (RT > 3) af[0][3] = lds_read16<base + 12288>(frag[0]);
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        // fragments of the next MFMA group first: they arrive while this group is multiplied
-        if (d < 3) {
-            af[(d + 1) & 1][0] = lds_read16<base>(frag[d + 1]);
-            if constexpr (RT > 1) af[(d + 1) & 1][1] = lds_read16<base + 4096>(frag[d + 1]);
-            if constexpr (RT > 2) af[(d + 1) & 1][2] = lds_read16<base + 8192>(frag[d + 1]);
-            if constexpr (RT > 3) af[(d + 1) & 1][3] = lds_read16<base + 12288>(frag[d + 1]);
-        }
-        // this group's RT reads are older than the RT just requested
-        constexpr int newer = RT;
-        if (d < 3) {
-            if constexpr (newer == 1) asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(af[d & 1][0]));
-            if constexpr (newer == 2) asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(af[d & 1][0]), "+v"(af[d & 1][1]));
-            if constexpr (newer == 3) asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(af[d & 1][0]), "+v"(af[d & 1][1]), "+v"(af[d & 1][2]));
-            if constexpr (newer == 4) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(af[d & 1][0]), "+v"(af[d & 1][1]), "+v"(af[d & 1][2]), "+v"(af[d & 1][3]));
-        } else {
-            if constexpr (RT == 1) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[d & 1][0]));
-            if constexpr (RT == 2) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[d & 1][0]), "+v"(af[d & 1][1]));
-            if constexpr (RT == 3) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[d & 1][0]), "+v"(af[d & 1][1]), "+v"(af[d & 1][2]));
-            if constexpr (RT == 4) asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(af[d & 1][0]), "+v"(af[d & 1][1]), "+v"(af[d & 1][2]), "+v"(af[d & 1][3]));
-        }
-        half8_t nf0 = bf0, nf1 = bf1;
-#pragma unroll
-        for (int mt = 0; mt < RT; ++mt) {
-            const half8_t a8 = __builtin_bit_cast(half8_t, af[d & 1][mt]);
-            acc[mt][0] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a8, bf0, acc[mt][0], 0, 0, 0);
-            acc[mt][1] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a8, bf1, acc[mt][1], 0, 0, 0);
-            // the next group's weights are expanded between the MFMAs
-            if (d < 3 && mt == 0) nf0 = dequant_word(w[0][d + 1], s2[0], b2[0], nc);
-            if (d < 3 && mt == (RT > 1 ? 1 : 0)) nf1 = dequant_word(w[1][d + 1], s2[1], b2[1], nc);
-        }
-        bf0 = nf0;
-        bf1 = nf1;
-    }
+// One MFMA; everything that must keep its place in the instruction stream is a volatile asm statement.
+__device__ __forceinline__ void mfma_slot(float16_t &acc, const u32x4 &a, const u32x4 &b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc) : "v"(a), "v"(b));
+}
+// Expansion of nibbles into fp16 weights half(q * s + b).  A byte holds two neighbouring elements: v_perm_b32 copies it into
+// both halves of a register, one v_and_or_b32 leaves the low nibble in the low half as 1024 + q (0x6400 | q) and the high
+// nibble in place in the high half as 64 + q (0x5400 | q << 4); a packed add removes both offsets exactly, and q * s + b is
+// one packed fp16 fused multiply-add on fp16 copies of s and b: four instructions a byte.  Two bytes of word `w` (P and
+// P + 1) are expanded together, in two halves of four instructions that go behind two consecutive MFMAs; the result of a
+// packed instruction is read two instructions later at the earliest (read in the very next one it needs a wait state).
+template <int P>
+__device__ __forceinline__ void expand_first(uint32_t w, uint32_t mask, uint32_t &t0, uint32_t &t1) {
+    asm volatile("v_perm_b32 %0, 0, %2, %3\n\tv_perm_b32 %1, 0, %2, %4\n\tv_and_or_b32 %0, %0, %5, %6\n\tv_and_or_b32 %1, %1, %5, %6"
+                 : "=&v"(t0), "=&v"(t1)
+                 : "v"(w), "s"(0x0c000c00u | ((uint32_t)P << 16) | (uint32_t)P), "s"(0x0c000c00u | ((uint32_t)(P + 1) << 16) | (uint32_t)(P + 1)), "v"(mask),
+                   "s"(0x54006400u));
+}
+__device__ __forceinline__ void expand_second(uint32_t t0, uint32_t t1, uint32_t s2, uint32_t b2, uint32_t &o0, uint32_t &o1) {
+    asm volatile("v_pk_add_f16 %0, %2, %4\n\tv_pk_add_f16 %1, %3, %4\n\tv_pk_fma_f16 %0, %0, %5, %6\n\tv_pk_fma_f16 %1, %1, %5, %6"
+                 : "=&v"(o0), "=&v"(o1)
+                 : "v"(t0), "v"(t1), "s"(0xD400E400u), "v"(s2), "v"(b2));   // (-64, -1024): the offsets of the two nibble positions
 }
 
-// The K loop.  The X tile of step kt lives in LDS stage kt % 3; the packed W rows of steps 2p, 2p + 1 in the wave's
-// buffer p & 1, the scales / biases of those two groups in register slot p & 1.
-// Even step kt = 2p:  barrier; request X(kt + 2), W(p + 1); multiply with the W words read from LDS at the end of the
-//                     previous step; request the scales of pair p + 1; wait for X(kt + 1) (the AC + 8 newer
-//                     requests stay in flight).
-// Odd step:           barrier; request X(kt + 2); multiply; wait for X(kt + 1), W(p + 1) and the scales (the AC
-//                     newer requests stay in flight); read the W words of both steps of pair p + 1 from LDS, switch
-//                     to its scales.
-// Requests are unconditional: past the end they repeat the last step or pair, which nobody reads, so that the number
-// of requests in flight is the same at every wait.
+struct BFrag {
+    uint32_t r[4];
+    __device__ __forceinline__ u32x4 tuple() const { return u32x4{r[0], r[1], r[2], r[3]}; }
+};
+
 template <int SD, int RT, int NW>
 struct QmmLoop {
-    // X copies per step and thread: those that carry rows of the RT row tiles.  A block with a single row tile keeps all
-    // of them (the others re-read valid rows out of L2): without them chunks of 32 to 128 tokens measured 5 % slower.
     static constexpr int AC = RT == 1 ? QmmGeom<NW>::kAChunks : (4 * RT + NW - 1) / NW;
     const QmmARows<NW> &a;
     QmmBRows &rows;
     uint32_t lds;
     uint32_t frag[4];
-    uint32_t wread;      // this lane's 16 bytes of column tile 0, first step of a pair, in the wave's W buffer 0
-    uint32_t wbuf;       // the wave's W buffer 0
+    uint32_t wread, wbuf;
     int last, last_pair;
-    bool odd_count;      // an odd number of K steps: the last pair has one group
+    bool odd_count;
     u32x4 w[2][2];       // [step of the pair][column tile]
     QmmSB sb, sb_next;
-    uint32_t pb;         // (current pair & 1) * kQmmWBytes: which W buffer holds the current pair
-    NibbleConsts nc;
+    uint32_t pb;
+    uint32_t mask;
+    u32x4 af[2][4];
+    BFrag bc[2], bn[2];
+    uint32_t s2c[2], b2c[2];   // this group's scale / bias pairs (fp16 x 2)
+    uint32_t tmp[4][2];
 
-    __device__ __forceinline__ void read_w(uint32_t at) {
-        w[0][0] = lds_read16<0>(at);
-        w[0][1] = lds_read16<2048>(at);
-        w[1][0] = lds_read16<0>(at ^ 32u);
-        w[1][1] = lds_read16<2048>(at ^ 32u);
-        asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]));
+    template <int OFF>
+    __device__ __forceinline__ void read_frags(int buf, uint32_t at) {
+        af[buf][0] = lds_read16<OFF>(at);
+        if constexpr (RT > 1) af[buf][1] = lds_read16<OFF + 4096>(at);
+        if constexpr (RT > 2) af[buf][2] = lds_read16<OFF + 8192>(at);
+        if constexpr (RT > 3) af[buf][3] = lds_read16<OFF + 12288>(at);
+    }
+    // waits until at most NEWER LDS reads are outstanding and ties the fragments of `buf` to the wait
+    template <int NEWER>
+    __device__ __forceinline__ void wait_frags(int buf) {
+        if constexpr (RT == 1) asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(af[buf][0]) : "n"(NEWER));
+        if constexpr (RT == 2) asm volatile("s_waitcnt lgkmcnt(%2)" : "+v"(af[buf][0]), "+v"(af[buf][1]) : "n"(NEWER));
+        if constexpr (RT == 3) asm volatile("s_waitcnt lgkmcnt(%3)" : "+v"(af[buf][0]), "+v"(af[buf][1]), "+v"(af[buf][2]) : "n"(NEWER));
+        if constexpr (RT == 4) asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(af[buf][0]), "+v"(af[buf][1]), "+v"(af[buf][2]), "+v"(af[buf][3]) : "n"(NEWER));
+    }
+    __device__ __forceinline__ void scales_of(uint32_t s, uint32_t b, int j, bool high, uint32_t &s2, uint32_t &b2) {
+        s2 = as_u32(sb_to_half2<SD>((uint16_t)(high ? s >> 16 : s & 0xFFFFu), rows.pre[j]));
+        b2 = as_u32(sb_to_half2<SD>((uint16_t)(high ? b >> 16 : b & 0xFFFFu), rows.pre[j]));
+    }
+    // part I of the eight expansion parts of one MFMA round: words wa (column tile 0), wb (tile 1) -> bn, with scales s2x / b2x
+    template <int I>
+    __device__ __forceinline__ void part(uint32_t wa, uint32_t wb, const uint32_t s2x[2], const uint32_t b2x[2]) {
+        constexpr int c = I >> 1, j = c >> 1, p = (c & 1) * 2;
+        if constexpr ((I & 1) == 0) expand_first<p>(j ? wb : wa, mask, tmp[c][0], tmp[c][1]);
+        else expand_second(tmp[c][0], tmp[c][1], s2x[j], b2x[j], bn[j].r[p], bn[j].r[p + 1]);
+    }
+    template <int FROM, int TO>
+    __device__ __forceinline__ void parts(uint32_t wa, uint32_t wb, const uint32_t s2x[2], const uint32_t b2x[2]) {
+        if constexpr (FROM < TO) {
+            part<FROM>(wa, wb, s2x, b2x);
+            parts<FROM + 1, TO>(wa, wb, s2x, b2x);
+        }
+    }
+    // the 2 RT MFMAs of one round with the eight parts spread behind them
+    template <int M>
+    __device__ __forceinline__ void round_slots(int buf, uint32_t wa, uint32_t wb, const uint32_t s2x[2], const uint32_t b2x[2], float16_t acc[4][2]) {
+        if constexpr (M < 2 * RT) {
+            const u32x4 b = bc[M & 1].tuple();
+            mfma_slot(acc[M >> 1][M & 1], af[buf][M >> 1], b);
+            parts<M * 8 / (2 * RT), (M + 1) * 8 / (2 * RT)>(wa, wb, s2x, b2x);
+            round_slots<M + 1>(buf, wa, wb, s2x, b2x, acc);
+        }
+    }
+    __device__ __forceinline__ void advance_b() {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) bc[j] = bn[j];
     }
 
-    template <int U3>
-    __device__ __forceinline__ void even_step(int kt, float16_t acc[4][2]) {
+    // One K step: rounds 0..2 expand this group's words 1..3; the last round expands word 0 of the next group, after the
+    // block has met (every wave has its last fragments of this stage, and the copies of the next stage have landed).
+    template <int U3, int HALF>
+    __device__ __forceinline__ void step(int kt, float16_t acc[4][2]) {
+        constexpr int base = U3 * kQmmStageBytes;
+#pragma unroll
+        for (int d = 0; d < 3; ++d) {
+            read_frags<base>((d + 1) & 1, frag[d + 1]);
+            wait_frags<RT>(d & 1);
+            round_slots<0>(d & 1, w[HALF][0][d + 1], w[HALF][1][d + 1], s2c, b2c, acc);
+            advance_b();
+        }
         const int pair = kt >> 1;
+        // the copies of X(kt + 1) [and, in the second step of a pair, W and scales of the next pair] have landed; the AC (+ 8) requests
+        // made after them may still be on their way
+        if constexpr (HALF == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AC + 8) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AC) : "memory");
+        wait_frags<0>(1);
         __builtin_amdgcn_s_barrier();
-        qmm_a_copy<NW, AC>(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
-        qmm_w_copy(rows, min(pair + 1, last_pair), wbuf + (pb ^ kQmmWBytes));
-        qmm_group<SD, RT, U3, 0>(w[0], sb, rows.pre, frag, nc, acc);
-        const int next_pair = min(pair + 1, last_pair);
-        qmm_sb_load(sb_next, rows, next_pair, odd_count && next_pair == last_pair);
-        // everything older than this step's AC + 4 + 4 requests (X, W, scales and biases) has landed
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AC + 8) : "memory");
-    }
-    template <int U3>
-    __device__ __forceinline__ void odd_step(int kt, float16_t acc[4][2]) {
-        __builtin_amdgcn_s_barrier();
-        qmm_a_copy<NW, AC>(a, min(kt + 2, last), lds + ((U3 + 2) % 3) * kQmmStageBytes);
-        qmm_group<SD, RT, U3, 1>(w[1], sb, rows.pre, frag, nc, acc);
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AC) : "memory");   // only this step's X copies may still be on their way
-        pb ^= kQmmWBytes;
-        read_w(wread + pb);
-        sb = sb_next;
+        qmm_a_copy<NW, AC>(a, min(kt + 3, last), lds + base);
+        uint32_t s2n[2], b2n[2];
+        uint32_t wa, wb;
+        if constexpr (HALF == 1) {
+            qmm_w_copy(rows, min(pair + 2, last_pair), wbuf + pb);     // the buffer of this pair: its words are in registers
+            pb ^= kQmmWBytes;
+            // the next pair's words
+            const uint32_t at = wread + pb;
+            w[0][0] = lds_read16<0>(at);
+            w[0][1] = lds_read16<2048>(at);
+            w[1][0] = lds_read16<0>(at ^ 32u);
+            w[1][1] = lds_read16<2048>(at ^ 32u);
+            read_frags<((U3 + 1) % 3) * kQmmStageBytes>(0, frag[0]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) scales_of(sb_next.s[j], sb_next.b[j], j, false, s2n[j], b2n[j]);
+            sb = sb_next;
+            const int next_pair = min(pair + 2, last_pair);
+            qmm_sb_load(sb_next, rows, next_pair, odd_count && next_pair == last_pair);
+            mfma_slot(acc[0][0], af[1][0], bc[0].tuple());
+            if constexpr (RT == 1) asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]));
+            if constexpr (RT == 2) asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]));
+            if constexpr (RT == 3) asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]));
+            if constexpr (RT == 4) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]));
+            wa = w[0][0][0];
+            wb = w[0][1][0];
+        } else {
+            read_frags<((U3 + 1) % 3) * kQmmStageBytes>(0, frag[0]);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) scales_of(sb.s[j], sb.b[j], j, true, s2n[j], b2n[j]);
+            wa = w[1][0][0];
+            wb = w[1][1][0];
+            mfma_slot(acc[0][0], af[1][0], bc[0].tuple());
+        }
+        parts<0, 8 / (2 * RT)>(wa, wb, s2n, b2n);
+        round_slots<1>(1, wa, wb, s2n, b2n, acc);
+        advance_b();
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            s2c[j] = s2n[j];
+            b2c[j] = b2n[j];
+        }
     }
 
     __device__ __forceinline__ void run(int kt_count, int lane, float16_t acc[4][2]) {
@@ -353,33 +373,49 @@ struct QmmLoop {
         const int i = lane & 31, kb = lane >> 5;
         const uint32_t frag0 = lds + (uint32_t)i * 128u + ((((uint32_t)kb * 4u) ^ (uint32_t)((i >> 1) & 7)) << 4);
 #pragma unroll
-        for (int d = 0; d < 4; ++d) frag[d] = frag0 ^ ((uint32_t)d << 4);   // lds is 128-byte aligned
-        wbuf = lds + 3 * kQmmStageBytes + (threadIdx.x >> 6) * (2 * kQmmWBytes);   // NW such pairs of buffers follow the X ring
+        for (int d = 0; d < 4; ++d) frag[d] = frag0 ^ ((uint32_t)d << 4);
+        wbuf = lds + 3 * kQmmStageBytes + (threadIdx.x >> 6) * (2 * kQmmWBytes);
         wread = wbuf + (uint32_t)i * 64u + ((((uint32_t)kb) ^ (uint32_t)((i >> 2) & 3)) << 4);
         pb = 0;
-        nc = nibble_consts();
+        mask = 0x00F0000Fu;
+        asm volatile("" : "+v"(mask));
         qmm_a_copy<NW, AC>(a, 0, lds);
-        qmm_a_copy<NW, AC>(a, min(1, last), lds + kQmmStageBytes);
         qmm_w_copy(rows, 0, wbuf);
         qmm_sb_load(sb, rows, 0, odd_count && last_pair == 0);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        qmm_a_copy<NW, AC>(a, min(1, last), lds + kQmmStageBytes);
+        qmm_w_copy(rows, min(1, last_pair), wbuf + kQmmWBytes);
+        qmm_sb_load(sb_next, rows, min(1, last_pair), odd_count && last_pair <= 1);
+        qmm_a_copy<NW, AC>(a, min(2, last), lds + 2 * kQmmStageBytes);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * AC + 8) : "memory");
         if constexpr (SD == 0) qmm_normalise_small_rows(rows, sb.s);
-        read_w(wread);
+        __builtin_amdgcn_s_barrier();
+        w[0][0] = lds_read16<0>(wread);
+        w[0][1] = lds_read16<2048>(wread);
+        w[1][0] = lds_read16<0>(wread ^ 32u);
+        w[1][1] = lds_read16<2048>(wread ^ 32u);
+        read_frags<0>(0, frag[0]);
+        asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]) : "n"(RT));
+#pragma unroll
+        for (int j = 0; j < 2; ++j) scales_of(sb.s[j], sb.b[j], j, false, s2c[j], b2c[j]);
+        parts<0, 8>(w[0][0][0], w[0][1][0], s2c, b2c);
+        advance_b();
         int kt0 = 0;
         for (; kt0 + 6 <= kt_count; kt0 += 6) {
-            even_step<0>(kt0, acc);
-            odd_step<1>(kt0 + 1, acc);
-            even_step<2>(kt0 + 2, acc);
-            odd_step<0>(kt0 + 3, acc);
-            even_step<1>(kt0 + 4, acc);
-            odd_step<2>(kt0 + 5, acc);
+            step<0, 0>(kt0, acc);
+            step<1, 1>(kt0 + 1, acc);
+            step<2, 0>(kt0 + 2, acc);
+            step<0, 1>(kt0 + 3, acc);
+            step<1, 0>(kt0 + 4, acc);
+            step<2, 1>(kt0 + 5, acc);
         }
-        if (kt0 < kt_count) even_step<0>(kt0, acc);
-        if (kt0 + 1 < kt_count) odd_step<1>(kt0 + 1, acc);
-        if (kt0 + 2 < kt_count) even_step<2>(kt0 + 2, acc);
-        if (kt0 + 3 < kt_count) odd_step<0>(kt0 + 3, acc);
-        if (kt0 + 4 < kt_count) even_step<1>(kt0 + 4, acc);
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // nothing may still be landing in LDS when the block moves on
+        if (kt0 < kt_count) step<0, 0>(kt0, acc);
+        if (kt0 + 1 < kt_count) step<1, 1>(kt0 + 1, acc);
+        if (kt0 + 2 < kt_count) step<2, 0>(kt0 + 2, acc);
+        if (kt0 + 3 < kt_count) step<0, 1>(kt0 + 3, acc);
+        if (kt0 + 4 < kt_count) step<1, 0>(kt0 + 4, acc);
+        // nothing may still be landing in LDS or in registers when the block moves on; the accumulators are read by ordinary
+        // instructions from here on
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
         __builtin_amdgcn_s_barrier();
     }
 };
