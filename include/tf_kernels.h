@@ -334,7 +334,8 @@ int32_t tf_shared_expert_int8_down(tf_ctx *ctx, tf_stream stream, const tf_proje
 /* PrefillSharedExpert.encodeBlock (Kernels/Prefill/MoE/PrefillSharedExpert.swift:11-58): the shared expert for
  * query_count rows of x (row stride x_stride_elements halves) into query_count rows of y.  The reference runs the
  * single-row chain once per row through the same one-row scratch buffers; so does this entry for fewer than 8 rows and
- * for operands the matrix-core path cannot take (weights or x rows not 16-byte aligned, intermediate % 64 != 0).
+ * for operands the matrix-core path cannot take (weights or x rows not 16-byte aligned, intermediate % 64 != 0, the scale
+ * or the bias arrays of gate and up more than 2 GiB apart).
  * Otherwise the rows go through the matrix cores: gate and up in one pass with both sums rounded to fp16 before GeGLU
  * (the chain's stage boundary), activations in a buffer the context owns, then the down projection; weights are
  * expanded to fp16 half(q*s+b) per group as in tf_int4_qmm, so results agree with the row chain within the shared
@@ -749,7 +750,8 @@ int32_t tf_prefill_moe_reduce_token_major(tf_ctx *ctx, tf_stream stream,
 /* MPPPrefillInt4QMM.encode (Kernels/TensorCore/MPPPrefillInt4QMM.swift:34-77) -> mpp_prefill_affine_threadgroup_f16
  * (Metal/TensorCore/tensorops.metal:13-105): y[m, n] fp16 [M, N] = x[M, K] . W[N, K]^T, weights expanded to fp16
  * half(q*s+b) per K group, fp32 accumulation on the matrix cores.  Returns TF_ERR_UNAVAILABLE (the reference's
- * Path.unavailable) when m, n, k <= 0, k % 64 != 0 or an operand is not 16-byte aligned; nothing is enqueued then. */
+ * Path.unavailable) when m, n, k <= 0, k % 64 != 0, an operand is not 16-byte aligned or the matrix has fewer than six
+ * groups in all (n * k / 64 < 6: the tiles stage scales six at a time); nothing is enqueued then. */
 int32_t tf_int4_qmm(tf_ctx *ctx, tf_stream stream,
                     const void *weights, uint64_t weights_offset,
                     const void *scales, uint64_t scales_offset,

@@ -1,6 +1,7 @@
 """GPU parity: router, routed experts (phase 1 / subset / phase 2), shared expert — through the C ABI, against the
 CPU oracle.  Cases restate RouterTopKTests, MoEFusedFFNTests and SharedExpertInt4Tests of the reference."""
 import numpy as np
+import torch
 import pytest
 
 import refcases
@@ -449,6 +450,29 @@ def test_prefill_shared_expert_block_on_matrix_cores(rows, d, f, x_stride, y_str
     chain = _repeated_rows(c, min(rows, 3))
     for r in range(min(rows, 3)):
         assert tfo.rel_error(tfo.from_f16_bits(y[r, :d]), tfo.from_f16_bits(chain[r])) < 6e-3
+
+
+def test_prefill_shared_expert_block_with_gate_and_up_scales_far_apart_takes_the_row_chain():
+    # the fused gate / up tiles address the scale arrays of both matrices through one 32-bit-offset descriptor; arrays more than
+    # 2 GiB apart are outside it, and the rows go one by one through the single-row chain instead (bit-identical to it)
+    rows, d, f = 16, 128, 64
+    c = _shared_block_case(rows, d, f, 0xFA2)
+    k = ctx()
+    spacer_bytes = (1 << 31) + (1 << 20)
+    arena = torch.empty(spacer_bytes + (1 << 16), dtype=torch.uint8, device="cuda")      # one allocation: gate scales at its start, up scales past 2 GiB
+    gate_s, up_s = c["gate"][1], c["up"][1]
+    arena[:gate_s.nbytes] = torch.from_numpy(np.ascontiguousarray(gate_s).view(np.uint8).ravel()).cuda()
+    arena[spacer_bytes:spacer_bytes + up_s.nbytes] = torch.from_numpy(np.ascontiguousarray(up_s).view(np.uint8).ravel()).cuda()
+    t = {n: [dev(a) for a in c[n]] for n in ("gate", "up", "down")}
+    pg, pu = _proj(*t["gate"], f, d), _proj(*t["up"], f, d)
+    pg.scales, pg.scales_offset = arena.data_ptr(), 0
+    pu.scales, pu.scales_offset = arena.data_ptr(), spacer_bytes
+    x, y = dev(c["x_bits"]), dev(np.full((rows, d), SENTINEL, np.uint16))
+    sg, su, sa = zeros_bytes(f * 2), zeros_bytes(f * 2), zeros_bytes(f * 2)
+    rc = k.prefill_shared_expert_block(x, pg, pu, _proj(*t["down"], d, f), y, sg, su, sa, rows, d, f, raise_on_error=False)
+    assert rc == tfk.TF_OK, k.last_error()
+    assert np.array_equal(host(y, np.uint16).reshape(rows, d), _repeated_rows(c, rows))
+    del arena
 
 
 def test_prefill_shared_expert_block_contract():

@@ -487,7 +487,9 @@ def mpp_inputs(m, n, k, adversarial=False):
 
 
 @pytest.mark.parametrize("m,n,k,adv", [(64, 32, 64, False), (128, 64, 128, False), (33, 70, 192, True), (5, 40, 128, False),
-                                       (32, 2112, 2816, False), (32, 2816, 2112, False), (100, 704, 2816, True), (32, 2816, 704, False)])
+                                       (32, 2112, 2816, False), (32, 2816, 2112, False), (100, 704, 2816, True), (32, 2816, 704, False),
+                                       # scales are staged six groups at a time: rows of 1, 5, 6, 7 and 13 groups, and the shortest arrays taken
+                                       (17, 8, 64, False), (40, 24, 320, True), (40, 33, 384, False), (70, 65, 448, True), (12, 31, 832, False), (9, 2, 192, False)])
 def test_int4_qmm_on_matrix_cores(m, n, k, adv):
     # MPPPrefillInt4QMMTests.swift:183-200 (rel <= 1e-3 vs the fp32-fma CPU reference rounded to fp16) + production shapes
     W, S, B, x = mpp_inputs(m, n, k, adv)
@@ -545,6 +547,8 @@ def test_int4_qmm_unavailable_and_exact_variant():
     assert kk.lib.tf_int4_qmm(kk.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dx.data_ptr(), 0, y.data_ptr(), 0, 8, 64, 96, tfk.TF_BF16) == tfk.TF_ERR_UNAVAILABLE
     assert kk.lib.tf_int4_qmm(kk.handle, None, dW.data_ptr(), 2, dS.data_ptr(), 0, dB.data_ptr(), 0, dx.data_ptr(), 0, y.data_ptr(), 0, 8, 64, 128, tfk.TF_BF16) == tfk.TF_ERR_UNAVAILABLE
     assert kk.lib.tf_int4_qmm(kk.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dx.data_ptr(), 0, y.data_ptr(), 0, 0, 64, 128, tfk.TF_BF16) == tfk.TF_ERR_UNAVAILABLE
+    # fewer than six scale values in the whole matrix: left to the exact kernel
+    assert kk.lib.tf_int4_qmm(kk.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dx.data_ptr(), 0, y.data_ptr(), 0, 8, 5, 64, tfk.TF_BF16) == tfk.TF_ERR_UNAVAILABLE
     torch.cuda.synchronize()
     assert np.all(host(y, np.uint8) == 0xEE)
     # the exact (fp32 weight) QMM equals repeated GEMV bit for bit, at the +2 weight offset too (PrefillAffineTests.swift:176-231)

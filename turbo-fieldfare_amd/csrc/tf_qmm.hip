@@ -8,31 +8,45 @@ using namespace tfk;
 namespace {
 
 // The wave's weight rows: column tile j covers rows row0[j] .. row0[j] + 31 of a matrix of `limit[j]` rows that starts
-// at w / s / b.
+// at w / s / b.  s[0] and s[1] (and b[0], b[1]) lie within 2 GiB of each other: the same array, or arrays of one expert.
 template <int SD>
 __device__ __forceinline__ QmmBRows make_b_rows(const uint8_t *const w[2], const uint8_t *const s[2], const uint8_t *const b[2],
                                                 const int row0[2], const int limit[2], int row_bytes, int groups, int lane) {
     QmmBRows rows;
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
-        rows.w[j] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w[j]), 0, limit[j] * row_bytes, 0x00020000);
-        rows.s[j] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(s[j]), 0, limit[j] * groups * 2, 0x00020000);
-        rows.b[j] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(b[j]), 0, limit[j] * groups * 2, 0x00020000);
-        rows.sb_off[j] = (uint32_t)(row0[j] + (lane & 31)) * (uint32_t)groups * 2u;
-    }
+    for (int j = 0; j < 2; ++j) rows.w[j] = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(w[j]), 0, limit[j] * row_bytes, 0x00020000);
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
         const int r = 16 * (t & 1) + (lane >> 2);                    // row inside the column tile
         const int piece = (lane & 3) ^ ((r >> 2) & 3);
         rows.copy_off[t] = (uint32_t)(row0[t >> 1] + r) * (uint32_t)row_bytes + (uint32_t)piece * 16u;
     }
+    // scales and biases: one descriptor per kind over the arrays of both tiles, from the lower of the two
+    const uint32_t sb_row_bytes = (uint32_t)groups * 2u;
+    const uint8_t *const sbase = s[0] <= s[1] ? s[0] : s[1], *const bbase = b[0] <= b[1] ? b[0] : b[1];
+    uint32_t srel[2], brel[2], send = 0, bend = 0;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
+        srel[j] = (uint32_t)(s[j] - sbase);
+        brel[j] = (uint32_t)(b[j] - bbase);
+        send = max(send, srel[j] + (uint32_t)limit[j] * sb_row_bytes);
+        bend = max(bend, brel[j] + (uint32_t)limit[j] * sb_row_bytes);
+    }
+    rows.sd = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(sbase), 0, (int)send, 0x00020000);
+    rows.bd = __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(bbase), 0, (int)bend, 0x00020000);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t row = (uint32_t)min(row0[j] + (lane & 31), limit[j] - 1);   // a column past the matrix: its last row (never stored)
+        rows.scan_s[j] = srel[j] + row * sb_row_bytes;
+        rows.scan_b[j] = brel[j] + row * sb_row_bytes;
         rows.pre[j] = 0u;
         rows.post[j] = 1.0f;
-        const uint32_t array_bytes = (uint32_t)limit[j] * (uint32_t)groups * 2u;
-        rows.scan_off[j] = min(rows.sb_off[j], array_bytes - (uint32_t)groups * 2u);   // a column past the matrix: its last row (never stored)
     }
+    // as a copier the lane serves row lane & 31 of tile lane >> 5: its own row of one of the tiles
+    rows.sb_copy_off[0] = lane < 32 ? rows.scan_s[0] : rows.scan_s[1];
+    rows.sb_copy_off[1] = lane < 32 ? rows.scan_b[0] : rows.scan_b[1];
+    rows.s_end = send;
+    rows.b_end = bend;
     rows.groups = groups;
     return rows;
 }
@@ -438,9 +452,21 @@ bool qmm_operands_ok(const void *w, const void *x, long ldx_halves, int k) {
     return aligned16(w) && aligned16(x) && (ldx_halves % 8 == 0) && k > 0 && (k % 64 == 0);
 }
 
+// The gate and the up matrix of a fused gate / up / GeGLU tile share one descriptor for their scales and one for their biases:
+// the two arrays of a kind must lie within 2 GiB of each other (they do wherever an expert is one blob).
+bool geglu_arrays_near(const tf_projection *gate, const tf_projection *up) {
+    const size_t bytes = (size_t)gate->rows * (size_t)(gate->cols / 64) * 2u;
+    auto near = [&](const uint8_t *a, const uint8_t *b) {
+        const uintptr_t lo = (uintptr_t)(a < b ? a : b), hi = (uintptr_t)(a < b ? b : a);
+        return hi - lo + bytes <= (size_t)0x7FFFFFFF;
+    };
+    return near(at(gate->scales, gate->scales_offset), at(up->scales, up->scales_offset)) &&
+           near(at(gate->biases, gate->biases_offset), at(up->biases, up->biases_offset));
+}
+
 // a shared expert's tiles may ride in the grouped launches: its output rows leave as whole 16-byte pieces
 bool dense_ride_ok(const DenseRide &ride) {
-    return aligned16(ride.y) && ride.down->rows % 8 == 0 && ride.ldy % 8 == 0;
+    return aligned16(ride.y) && ride.down->rows % 8 == 0 && ride.ldy % 8 == 0 && geglu_arrays_near(ride.gate, ride.up);
 }
 
 int32_t launch_grouped_phase1_mfma(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off,
@@ -503,7 +529,7 @@ int32_t launch_qmm_dense(tf_ctx *ctx, hipStream_t st, const uint8_t *w, const ui
     return check_launch(ctx, "int4_qmm");
 }
 
-// A[m, f] = GeGLU(half(X . gate^T), half(X . up^T)); a 16-byte aligned, lda % 8 == 0, f % 8 == 0
+// A[m, f] = GeGLU(half(X . gate^T), half(X . up^T)); a 16-byte aligned, lda % 8 == 0, f % 8 == 0, geglu_arrays_near(gate, up)
 int32_t launch_qmm_dense_geglu(tf_ctx *ctx, hipStream_t st, const tf_projection *gate, const tf_projection *up, const half_t *x, long ldx,
                                half_t *a_out, long lda, int m, tf_dtype sd) {
     const int f = (int)gate->rows;
@@ -681,7 +707,8 @@ int32_t tf_int4_qmm(tf_ctx *ctx, tf_stream stream, const void *weights, uint64_t
                     void *y, uint64_t y_offset, int32_t m, int32_t n, int32_t k, tf_dtype scale_dtype) {
     TF_REQUIRE(ctx, ctx && weights && scales && biases && x && y, TF_ERR_INVALID_ARGUMENT, "int4_qmm: null argument");
     // MPPPrefillInt4QMM.encode's guard list (MPPPrefillInt4QMM.swift:40-56): anything it refuses is "unavailable", not an error
-    const bool shape_ok = m > 0 && n > 0 && k > 0 && (k % (int32_t)TF_GROUP_SIZE == 0);
+    // (the tiles stage scales twelve bytes at a time: a matrix with fewer than six of them is left to the exact kernel)
+    const bool shape_ok = m > 0 && n > 0 && k > 0 && (k % (int32_t)TF_GROUP_SIZE == 0) && (int64_t)n * (k / (int32_t)TF_GROUP_SIZE) >= 6;
     const bool offs_ok = scales_offset % 2 == 0 && biases_offset % 2 == 0 && x_offset % 2 == 0 && y_offset % 2 == 0;
     if (!shape_ok || !offs_ok || !(scale_dtype == TF_BF16 || scale_dtype == TF_FP16)) return fail(ctx, TF_ERR_UNAVAILABLE, "int4_qmm: unsupported shape or offsets");
     const uint8_t *w = at(weights, weights_offset);
@@ -730,7 +757,7 @@ int32_t shared_expert_block_impl(tf_ctx *ctx, tf_stream stream, const void *x, u
                       up->scales_offset % 2 == 0 && up->biases_offset % 2 == 0 && down->scales_offset % 2 == 0 && down->biases_offset % 2 == 0;
     const bool block_path = weight_bits == 4 && pointers && even && query_count >= kSharedBlockMinRows && (scale_dtype == TF_BF16 || scale_dtype == TF_FP16) &&
                             qmm_operands_ok(gw, xp, x_stride_elements, (int)d) && aligned16(uw) && aligned16(dw) &&
-                            intermediate % TF_GROUP_SIZE == 0 && query_count <= (uint32_t)INT32_MAX;
+                            intermediate % TF_GROUP_SIZE == 0 && query_count <= (uint32_t)INT32_MAX && geglu_arrays_near(gate, up);
     if (plan && !block_path) return TF_OK;
     if (weight_bits == 8 && pointers && even && query_count >= 2) {
         // 8-bit projections.  Up to kShared8MfmaMinRows - 1 rows: rows in groups against each weight row, bit-identical to the

@@ -9,7 +9,11 @@
 //       k = {8d .. 8d+7} u {32+8d .. 32+8d+7}.  Reading "its" row straight from global memory would touch 32 cache
 //       lines per load instruction; instead the load unit copies the packed rows into a wave-private LDS area two K
 //       steps at a time (64 contiguous bytes per row, four lanes per row), and the lanes pick their 16 bytes there.
-//       Scales and biases are loaded two groups at a time (one 32-bit load per row and array).
+//       Scales and biases take the same road: a load of "its" rows' scales touches a cache line per lane, and the lines of a
+//       row come round again every two steps, long after the X and W streams have pushed them out of the CU's cache (without
+//       these loads the 2048-token prefill measured 10 % faster).  So every six steps the load unit copies twelve bytes - six
+//       groups - of each of the wave's 64 rows per array into the wave's LDS (two instructions instead of twelve), and the
+//       lanes read their two groups a pair from there.
 //   X   is copied by the load unit from global memory straight into LDS (global_load_lds_dwordx4: no staging registers,
 //       no vector instructions), two K steps ahead, into a ring of three stages shared by the four waves.  A stage is
 //       128 rows x 8 chunks of 16 bytes; chunk c of row r sits at position c ^ ((r >> 1) & 7) of its row, which keeps
@@ -38,6 +42,12 @@ constexpr int kQmmBM = 128;      // rows per block tile (4 MFMA row tiles)
 constexpr int kQmmWaveN = 64;    // columns per wave (2 MFMA column tiles)
 constexpr int kQmmStageBytes = kQmmBM * 8 * 16;  // one X stage
 constexpr int kQmmWBytes = 64 * 64;               // packed W rows of one wave for two K steps: 64 rows x 64 bytes
+constexpr int kQmmSBWindowSteps = 6;              // K steps (groups) per staged window of scales / biases
+constexpr int kQmmSBRowBytes = 2 * kQmmSBWindowSteps;   // per row and array, in memory
+constexpr int kQmmSBSlotBytes = 16;               // per row and array in LDS: a 12-byte LDS-direct copy puts lane l's bytes at 16 l
+constexpr int kQmmSBArrayBytes = 64 * kQmmSBSlotBytes;  // 64 rows (two column tiles) of one array
+constexpr int kQmmSBBufBytes = 2048;              // one window: scales at 0, biases at kQmmSBArrayBytes; two such buffers per wave
+static_assert(2 * kQmmSBArrayBytes <= kQmmSBBufBytes, "a window fits its buffer");
 // A block is NW waves (4 or 8) that share the X ring: with 8 waves the same activation rows serve twice as many output
 // columns, so a tile's activations are fetched half as often; such a block has a CU to itself.
 template <int NW>
@@ -45,7 +55,8 @@ struct QmmGeom {
     static constexpr int kThreads = NW * 64;
     static constexpr int kBN = NW * kQmmWaveN;                                     // columns per block tile
     static constexpr int kAChunks = kQmmBM * 8 / kThreads;                         // 16-byte X chunks copied per thread and K step
-    static constexpr int kLoopLdsBytes = 3 * kQmmStageBytes + NW * 2 * kQmmWBytes; // X ring + two W buffers per wave
+    static constexpr int kWaveLdsBytes = kQmmWBytes + 2 * kQmmSBBufBytes;          // per wave: one W buffer, two scale windows
+    static constexpr int kLoopLdsBytes = 3 * kQmmStageBytes + NW * kWaveLdsBytes;  // X ring + the waves' private areas
 };
 constexpr int kQmmBN = QmmGeom<4>::kBN;
 constexpr int kQmmLdsBytes = QmmGeom<4>::kLoopLdsBytes;
@@ -92,7 +103,6 @@ __device__ __forceinline__ void qmm_a_rows_set(QmmARows<NW> &a, int q, uint64_t 
 //   copy_off[t]: where copy number t of a two-step block starts for this lane: row 16 (t & 1) + lane / 4 of column
 //                tile t / 2, 16-byte piece (lane & 3) ^ ((row / 4) & 3) of the row's 64 bytes (the XOR keeps the later
 //                reads free of bank conflicts);
-//   sb_off[j]:   the lane's own row (lane & 31) of tile j in the scale / bias arrays.
 //   pre[j] / post[j]: a power of two 2^e per weight row (as e << 23, added to a value's fp32 bits) and 2^-e.  The expansion
 //                computes half(q s + b) with fp16 copies of s and b; a bf16 scale below fp16's normal range (6.1e-5) would lose
 //                mantissa bits in that copy.  A wave whose first two groups show such a scale (qmm_normalise_small_rows) scans
@@ -103,14 +113,22 @@ __device__ __forceinline__ void qmm_a_rows_set(QmmARows<NW> &a, int q, uint64_t 
 //                mantissa the unscaled one drops.  Rows whose first groups have ordinary scales are left alone (e = 0): a later
 //                group with a tiny scale then carries at most 15 x 2^-25 of absolute error per weight, next to weights of at
 //                least 6.1e-5 in the same row.
-//   scan_off[j], groups: the lane's row in the scale / bias arrays (clamped into the matrix) and its length, for that scan.
+//   sd / bd:     the scale and the bias arrays of BOTH column tiles under one descriptor each (the lower of the two arrays is
+//                the base; they lie within 2 GiB of each other: two row ranges of one matrix, or gate and up of one expert).
+//                Rows beyond a matrix are clamped to its last row (what such lanes compute is never stored).
+//   sb_copy_off: where this lane's row starts in sd / bd when the lane copies for the wave: row lane & 31 of tile lane >> 5.
+//   scan_s[j], scan_b[j], groups: the lane's own row (lane & 31) of tile j in sd / bd and its length, for the scan above.
+//   s_end, b_end: where sd / bd end.  A copy that would reach past that end comes back as zeros, all of it: the last window of
+//                the last row starts early enough to end with the array instead (qmm_sb_copy), and its readers allow for the
+//                displacement (qmm_sb_read_tail).
 struct QmmBRows {
-    qmm_rsrc_t w[2], s[2], b[2];
+    qmm_rsrc_t w[2], sd, bd;
     uint32_t copy_off[4];
-    uint32_t sb_off[2];
+    uint32_t sb_copy_off[2];   // [0]: in sd, [1]: in bd
     uint32_t pre[2];
     float post[2];
-    uint32_t scan_off[2];
+    uint32_t scan_s[2], scan_b[2];
+    uint32_t s_end, b_end;     // bytes sd / bd cover
     int groups;
 };
 // scales and biases of the lane's rows for two consecutive groups (low half: even group)
@@ -159,7 +177,7 @@ __device__ __forceinline__ void qmm_normalise_small_rows(QmmBRows &rows, const u
     for (int j = 0; j < 2; ++j) {
         // every |s| < 2^(es - 126) and every |b| < 2^(eb - 126): with top = max(es + 4, eb), 15 |s| and |b| lie below 2^(top - 126),
         // and 2^(140 - top) brings them below 2^14, their sum below 2^15
-        const uint32_t es = row_max_exponent_any(rows.s[j], rows.scan_off[j], rows.groups), eb = row_max_exponent_any(rows.b[j], rows.scan_off[j], rows.groups);
+        const uint32_t es = row_max_exponent_any(rows.sd, rows.scan_s[j], rows.groups), eb = row_max_exponent_any(rows.bd, rows.scan_b[j], rows.groups);
         const uint32_t top = max(es + 4u, eb);
         const int shift = top == 0u ? 0 : min(max(140 - (int)top, -100), 100);
         rows.pre[j] = (uint32_t)shift << 23;
@@ -167,22 +185,64 @@ __device__ __forceinline__ void qmm_normalise_small_rows(QmmBRows &rows, const u
     }
 }
 
-// single (wave-uniform): the pair has only its first group (the last pair of an odd number of groups); a 32-bit load
-// would run past the end of the last row.  Both arms issue the same number of loads.
-__device__ __forceinline__ void qmm_sb_load(QmmSB &sb, const QmmBRows &rows, int pair, bool single) {
-    if (single) {
+// Window `window` (groups 6 window .. 6 window + 5) of the wave's 64 rows: scales -> dst, biases -> dst + kQmmSBArrayBytes, twelve
+// bytes a lane (lane l's land at 16 l).  Past the end of a row the copy takes what follows it; no step uses those groups.  A
+// copy may not reach past the end of the arrays: where it would, it starts earlier by the excess.
+__device__ __forceinline__ void qmm_sb_copy(const QmmBRows &rows, int window, uint32_t dst) {
+    const uint32_t at = (uint32_t)window * kQmmSBRowBytes;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rows.sd, (__attribute__((address_space(3))) void *)(uintptr_t)dst, 12,
+                                             min(rows.sb_copy_off[0] + at, rows.s_end - kQmmSBRowBytes), 0, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rows.bd, (__attribute__((address_space(3))) void *)(uintptr_t)(dst + kQmmSBArrayBytes), 12,
+                                             min(rows.sb_copy_off[1] + at, rows.b_end - kQmmSBRowBytes), 0, 0, 0);
+}
+template <int OFFSET>
+__device__ __forceinline__ uint32_t lds_read4(uint32_t addr) {
+    uint32_t v;
+    asm volatile("ds_read_b32 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+template <int OFFSET>
+__device__ __forceinline__ uint32_t lds_read2(uint32_t addr) {
+    uint32_t v;
+    asm volatile("ds_read_u16 %0, %1 offset:%2" : "=v"(v) : "v"(addr), "n"(OFFSET));
+    return v;
+}
+// The lane's scales and biases of pair PAIR (0..2) of the window at `at` (the lane's row of tile 0 in the scale area): LDS
+// reads, to be waited for by the caller.
+template <int PAIR>
+__device__ __forceinline__ void qmm_sb_read(QmmSB &sb, uint32_t at) {
+    sb.s[0] = lds_read4<PAIR * 4>(at);
+    sb.s[1] = lds_read4<PAIR * 4 + 32 * kQmmSBSlotBytes>(at);
+    sb.b[0] = lds_read4<PAIR * 4 + kQmmSBArrayBytes>(at);
+    sb.b[1] = lds_read4<PAIR * 4 + kQmmSBArrayBytes + 32 * kQmmSBSlotBytes>(at);
+}
+// The same in a window that reaches past the end of the rows: the row that ends its array was copied from an earlier start, by a
+// number of bytes that need not be a multiple of four, so the two values of a pair are read one by one.  Rare (the last
+// window of a row): the reads are waited for on the spot.
+template <int PAIR>
+__device__ __forceinline__ void qmm_sb_read_tail(QmmSB &sb, const QmmBRows &rows, int window, uint32_t at) {
+    const uint32_t reach = (uint32_t)(window + 1) * kQmmSBRowBytes;
+    uint32_t lo[4], hi[4];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            sb.s[j] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rows.s[j], rows.sb_off[j], pair * 4, 0);
-            sb.b[j] = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(rows.b[j], rows.sb_off[j], pair * 4, 0);
-        }
-    } else {
-#pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            sb.s[j] = __builtin_amdgcn_raw_buffer_load_b32(rows.s[j], rows.sb_off[j], pair * 4, 0);
-            sb.b[j] = __builtin_amdgcn_raw_buffer_load_b32(rows.b[j], rows.sb_off[j], pair * 4, 0);
+    for (int j = 0; j < 2; ++j) {
+        const uint32_t ds = (uint32_t)max((int)(rows.scan_s[j] + reach) - (int)rows.s_end, 0), db = (uint32_t)max((int)(rows.scan_b[j] + reach) - (int)rows.b_end, 0);
+        if (j == 0) {
+            lo[0] = lds_read2<PAIR * 4>(at + ds);
+            hi[0] = lds_read2<PAIR * 4 + 2>(at + ds);
+            lo[2] = lds_read2<PAIR * 4 + kQmmSBArrayBytes>(at + db);
+            hi[2] = lds_read2<PAIR * 4 + kQmmSBArrayBytes + 2>(at + db);
+        } else {
+            lo[1] = lds_read2<PAIR * 4 + 32 * kQmmSBSlotBytes>(at + ds);
+            hi[1] = lds_read2<PAIR * 4 + 32 * kQmmSBSlotBytes + 2>(at + ds);
+            lo[3] = lds_read2<PAIR * 4 + kQmmSBArrayBytes + 32 * kQmmSBSlotBytes>(at + db);
+            hi[3] = lds_read2<PAIR * 4 + kQmmSBArrayBytes + 32 * kQmmSBSlotBytes + 2>(at + db);
         }
     }
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(lo[0]), "+v"(lo[1]), "+v"(lo[2]), "+v"(lo[3]), "+v"(hi[0]), "+v"(hi[1]), "+v"(hi[2]), "+v"(hi[3]));
+    sb.s[0] = lo[0] | (hi[0] << 16);
+    sb.s[1] = lo[1] | (hi[1] << 16);
+    sb.b[0] = lo[2] | (hi[2] << 16);
+    sb.b[1] = lo[3] | (hi[3] << 16);
 }
 // packed W rows of K steps 2 pair, 2 pair + 1 -> the wave's LDS buffer at byte address `dst` (wave-uniform)
 __device__ __forceinline__ void qmm_w_copy(const QmmBRows &rows, int pair, uint32_t dst) {
@@ -244,12 +304,12 @@ struct QmmLoop {
     QmmBRows &rows;
     uint32_t lds;
     uint32_t frag[4];
-    uint32_t wread, wbuf;
+    uint32_t wread, wbuf;      // the wave's W buffer and this lane's 16 bytes of column tile 0, first step of a pair, in it
+    uint32_t sbuf, sbread;     // the wave's two scale windows and this lane's row of tile 0 in the first
+    uint32_t sbp;              // which window is current: 0 or kQmmSBBufBytes
     int last, last_pair;
-    bool odd_count;
-    u32x4 w[2][2];       // [step of the pair][column tile]
-    QmmSB sb, sb_next;
-    uint32_t pb;
+    u32x4 w[2][2];             // [step of the pair][column tile]
+    QmmSB sb;                  // scales and biases of the current pair
     uint32_t mask;
     u32x4 af[2][4];
     BFrag bc[2], bn[2];
@@ -306,9 +366,17 @@ struct QmmLoop {
 
     // One K step: rounds 0..2 expand this group's words 1..3; the last round expands word 0 of the next group, after the
     // block has met (every wave has its last fragments of this stage, and the copies of the next stage have landed).
+    // Steps come in cycles of six, (U3, HALF) = (0,0) (1,1) (2,0) (0,1) (1,0) (2,1), one window of scales a cycle:
+    //   every step:          X(kt + 3) is requested at the meeting point (AC copies);
+    //   second steps (HALF): the next pair's W words and scales are read from LDS, then W of the pair after it is requested
+    //                        into the same buffer (4 copies);
+    //   step (0,1):          also the next cycle's window of scales and biases (2 copies), read from step (2,1) on.
+    // What a step waits for was requested two steps earlier; the counts below are what may still be on its way at each wait.
     template <int U3, int HALF>
     __device__ __forceinline__ void step(int kt, float16_t acc[4][2]) {
         constexpr int base = U3 * kQmmStageBytes;
+        constexpr bool kWindowStep = U3 == 0 && HALF == 1;            // requests the next window
+        constexpr bool kAfterWindowStep = U3 == 1 && HALF == 0;       // the step after it
 #pragma unroll
         for (int d = 0; d < 3; ++d) {
             read_frags<base>((d + 1) & 1, frag[d + 1]);
@@ -317,9 +385,9 @@ struct QmmLoop {
             advance_b();
         }
         const int pair = kt >> 1;
-        // the copies of X(kt + 1) [and, in the second step of a pair, W and scales of the next pair] have landed; the AC (+ 8) requests
-        // made after them may still be on their way
-        if constexpr (HALF == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AC + 8) : "memory");
+        // X(kt + 1) has landed [second steps: also W and, where due, the window requested two steps ago]; younger requests may be
+        // under way: after a second step its X, W (and window) copies, after a first step its X copies
+        if constexpr (HALF == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AC + 4 + (kAfterWindowStep ? 2 : 0)) : "memory");
         else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(AC) : "memory");
         wait_frags<0>(1);
         __builtin_amdgcn_s_barrier();
@@ -327,25 +395,30 @@ struct QmmLoop {
         uint32_t s2n[2], b2n[2];
         uint32_t wa, wb;
         if constexpr (HALF == 1) {
-            qmm_w_copy(rows, min(pair + 2, last_pair), wbuf + pb);     // the buffer of this pair: its words are in registers
-            pb ^= kQmmWBytes;
-            // the next pair's words
-            const uint32_t at = wread + pb;
-            w[0][0] = lds_read16<0>(at);
-            w[0][1] = lds_read16<2048>(at);
-            w[1][0] = lds_read16<0>(at ^ 32u);
-            w[1][1] = lds_read16<2048>(at ^ 32u);
+            if constexpr (kWindowStep) qmm_sb_copy(rows, kt / kQmmSBWindowSteps + 1, sbuf + (sbp ^ kQmmSBBufBytes));
+            // the next pair's words and scales
+            w[0][0] = lds_read16<0>(wread);
+            w[0][1] = lds_read16<2048>(wread);
+            w[1][0] = lds_read16<0>(wread ^ 32u);
+            w[1][1] = lds_read16<2048>(wread ^ 32u);
+            if constexpr (U3 == 2) sbp ^= kQmmSBBufBytes;            // (2,1): the next pair opens the next window
+            {
+                const int window = kt / kQmmSBWindowSteps + (U3 == 2 ? 1 : 0);
+                if ((window + 1) * kQmmSBWindowSteps <= rows.groups) qmm_sb_read<U3 == 1 ? 1 : U3 == 0 ? 2 : 0>(sb, sbread + sbp);
+                else qmm_sb_read_tail<U3 == 1 ? 1 : U3 == 0 ? 2 : 0>(sb, rows, window, sbread + sbp);
+            }
             read_frags<((U3 + 1) % 3) * kQmmStageBytes>(0, frag[0]);
-#pragma unroll
-            for (int j = 0; j < 2; ++j) scales_of(sb_next.s[j], sb_next.b[j], j, false, s2n[j], b2n[j]);
-            sb = sb_next;
-            const int next_pair = min(pair + 2, last_pair);
-            qmm_sb_load(sb_next, rows, next_pair, odd_count && next_pair == last_pair);
             mfma_slot(acc[0][0], af[1][0], bc[0].tuple());
-            if constexpr (RT == 1) asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]));
-            if constexpr (RT == 2) asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]));
-            if constexpr (RT == 3) asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]));
-            if constexpr (RT == 4) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]));
+            // the eight word and scale reads are older than the fragment reads; the wait is also a compiler barrier: the copy
+            // into the W buffer below must not be moved ahead of the reads of that buffer
+            if constexpr (RT == 1) asm volatile("s_waitcnt lgkmcnt(1)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]), "+v"(sb.s[0]), "+v"(sb.s[1]), "+v"(sb.b[0]), "+v"(sb.b[1]) : : "memory");
+            if constexpr (RT == 2) asm volatile("s_waitcnt lgkmcnt(2)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]), "+v"(sb.s[0]), "+v"(sb.s[1]), "+v"(sb.b[0]), "+v"(sb.b[1]) : : "memory");
+            if constexpr (RT == 3) asm volatile("s_waitcnt lgkmcnt(3)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]), "+v"(sb.s[0]), "+v"(sb.s[1]), "+v"(sb.b[0]), "+v"(sb.b[1]) : : "memory");
+            if constexpr (RT == 4) asm volatile("s_waitcnt lgkmcnt(4)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]), "+v"(sb.s[0]), "+v"(sb.s[1]), "+v"(sb.b[0]), "+v"(sb.b[1]) : : "memory");
+            // the W buffer has been read: the pair after the next goes into it
+            qmm_w_copy(rows, min(pair + 2, last_pair), wbuf);
+#pragma unroll
+            for (int j = 0; j < 2; ++j) scales_of(sb.s[j], sb.b[j], j, false, s2n[j], b2n[j]);
             wa = w[0][0][0];
             wb = w[0][1][0];
         } else {
@@ -369,32 +442,34 @@ struct QmmLoop {
     __device__ __forceinline__ void run(int kt_count, int lane, float16_t acc[4][2]) {
         last = kt_count - 1;
         last_pair = last >> 1;
-        odd_count = (kt_count & 1) != 0;
         const int i = lane & 31, kb = lane >> 5;
         const uint32_t frag0 = lds + (uint32_t)i * 128u + ((((uint32_t)kb * 4u) ^ (uint32_t)((i >> 1) & 7)) << 4);
 #pragma unroll
         for (int d = 0; d < 4; ++d) frag[d] = frag0 ^ ((uint32_t)d << 4);
-        wbuf = lds + 3 * kQmmStageBytes + (threadIdx.x >> 6) * (2 * kQmmWBytes);
+        wbuf = lds + 3 * kQmmStageBytes + (threadIdx.x >> 6) * QmmGeom<NW>::kWaveLdsBytes;   // NW such areas follow the X ring
         wread = wbuf + (uint32_t)i * 64u + ((((uint32_t)kb) ^ (uint32_t)((i >> 2) & 3)) << 4);
-        pb = 0;
+        sbuf = wbuf + kQmmWBytes;
+        sbread = sbuf + (uint32_t)i * kQmmSBSlotBytes;
+        sbp = 0;
         mask = 0x00F0000Fu;
         asm volatile("" : "+v"(mask));
         qmm_a_copy<NW, AC>(a, 0, lds);
         qmm_w_copy(rows, 0, wbuf);
-        qmm_sb_load(sb, rows, 0, odd_count && last_pair == 0);
+        qmm_sb_copy(rows, 0, sbuf);
         qmm_a_copy<NW, AC>(a, min(1, last), lds + kQmmStageBytes);
-        qmm_w_copy(rows, min(1, last_pair), wbuf + kQmmWBytes);
-        qmm_sb_load(sb_next, rows, min(1, last_pair), odd_count && last_pair <= 1);
         qmm_a_copy<NW, AC>(a, min(2, last), lds + 2 * kQmmStageBytes);
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * AC + 8) : "memory");
-        if constexpr (SD == 0) qmm_normalise_small_rows(rows, sb.s);
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * AC) : "memory");
         __builtin_amdgcn_s_barrier();
         w[0][0] = lds_read16<0>(wread);
         w[0][1] = lds_read16<2048>(wread);
         w[1][0] = lds_read16<0>(wread ^ 32u);
         w[1][1] = lds_read16<2048>(wread ^ 32u);
+        if (kQmmSBWindowSteps <= rows.groups) qmm_sb_read<0>(sb, sbread);
+        else qmm_sb_read_tail<0>(sb, rows, 0, sbread);
         read_frags<0>(0, frag[0]);
-        asm volatile("s_waitcnt lgkmcnt(%4)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]) : "n"(RT));
+        asm volatile("s_waitcnt lgkmcnt(%8)" : "+v"(w[0][0]), "+v"(w[0][1]), "+v"(w[1][0]), "+v"(w[1][1]), "+v"(sb.s[0]), "+v"(sb.s[1]), "+v"(sb.b[0]), "+v"(sb.b[1]) : "n"(RT) : "memory");
+        qmm_w_copy(rows, min(1, last_pair), wbuf);
+        if constexpr (SD == 0) qmm_normalise_small_rows(rows, sb.s);
 #pragma unroll
         for (int j = 0; j < 2; ++j) scales_of(sb.s[j], sb.b[j], j, false, s2c[j], b2c[j]);
         parts<0, 8>(w[0][0][0], w[0][1][0], s2c, b2c);
