@@ -771,6 +771,20 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=Fal
             side.synchronize()
             rounds, _ = replay_rounds(torch, side, g.replay)
             results[label] = (float(np.median(rounds)) * 1e3 / per_graph, b["hidden" if br is not None else "hidden_alt"].clone())
+        # four tokens' layers in one graph: a graph launch costs the device about 12 us before its first kernel, 0.4 us a layer of
+        # a one-token graph and 0.1 us here
+        tokens_per_graph = 4
+        g4 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g4, stream=side):
+            st = torch.cuda.current_stream().cuda_stream
+            for tkn in range(tokens_per_graph):
+                b["hidden"].copy_(hidden0)
+                for i in range(per_graph):
+                    layer_step(i, st, None, first=i == 0, last=i == per_graph - 1)
+        g4.replay()
+        side.synchronize()
+        rounds4, _ = replay_rounds(torch, side, g4.replay)
+        us4 = float(np.median(rounds4)) * 1e3 / (per_graph * tokens_per_graph)
     us = results["serial"][0]
     if fork:
         assert torch.equal(results["forked"][1], results["serial"][1]), "forked and serial layer chains disagree"
@@ -780,7 +794,8 @@ def layer_chain_extra(torch, tfk, k, gen, lib, h, layers, offs, stride, fork=Fal
                    + 2 * WINDOW * NKV * HD * 2)
     res = {"workload": "one token through one whole decoder layer (16q/8kv x 256, window 1024, shared 2112, 8 of 128 experts), 30 layers per graph replay",
            "us_per_layer": round(us, 2), "ms_per_30_layers": round(us * 30 / 1e3, 3), "algorithmic_bytes_per_layer": layer_bytes,
-           "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 8, "graph": "one in-order chain of launches"}
+           "GBps": round(layer_bytes / (us * 1e-6) / 1e9, 1), "launches_per_layer": 8, "graph": "one in-order chain of launches",
+           "us_per_layer_four_tokens_per_graph": round(us4, 2)}
     if fork:
         res["us_per_layer_shared_expert_on_forked_branch"] = round(results["forked"][0], 2)
         res["forked_branch_note"] = ("the shared expert + its norm on a second captured stream (event fork after the post-attention setup, join "
