@@ -813,10 +813,12 @@ def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, 
     expert_bytes = 3 * int4_matrix_bytes(F_MOE, D)
     res = {}
 
-    def run(T, idx_dev=None, wts_dev=None, iters=20, with_router=True, shared=None):
+    def run(T, idx_dev=None, wts_dev=None, iters=20, with_router=True, shared=None, one_call=False):
         n = T * TOPK
         cap = E + n // 64 + 1
-        hid = torch.randn((T, D), device="cuda", generator=gen).to(torch.float16)
+        rows_gen = torch.Generator(device="cuda")
+        rows_gen.manual_seed(0x51A0 + T)          # the same token rows for every way of running a size
+        hid = torch.randn((T, D), device="cuda", generator=rows_gen).to(torch.float16)
         idx = torch.zeros((T, TOPK), dtype=torch.int32, device="cuda") if idx_dev is None else idx_dev
         wts = torch.zeros((T, TOPK), dtype=torch.float16, device="cuda") if wts_dev is None else wts_dev
         sp = torch.zeros(n * 4, dtype=torch.int32, device="cuda")
@@ -828,6 +830,13 @@ def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, 
 
         def fn(i):
             rc = 0
+            if one_call:        # router, experts and reduce of a few token rows as one call of three launches
+                rc = lib.tf_prefill_routed_moe_few_tokens(h, stream, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0, hid.data_ptr(), 0,
+                                                          r["eff"].data_ptr(), 0, r["gain"].data_ptr(), 0, idx.data_ptr(), 0, wts.data_ptr(), 0, T, E, D,
+                                                          TOPK, D, hid.data_ptr(), 0, D, pool.data_ptr(), stride, C.byref(off), acts.data_ptr(),
+                                                          partials.data_ptr(), h2.data_ptr(), 0, F_MOE, tfk.TF_BF16)
+                assert rc == 0, k.last_error()
+                return
             if with_router:     # router block + device grouping as one call (one launch fewer up to 32 tokens)
                 rc |= lib.tf_prefill_router_group_block(h, stream, r["W"].data_ptr(), 0, r["S"].data_ptr(), 0, r["B"].data_ptr(), 0,
                                                         hid.data_ptr(), 0, r["eff"].data_ptr(), 0, r["gain"].data_ptr(), 0,
@@ -847,17 +856,24 @@ def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, 
             rc |= lib.tf_prefill_moe_reduce_token_major(h, stream, partials.data_ptr(), 0, wts.data_ptr(), 0, h2.data_ptr(), 0, T, TOPK, D)
             assert rc == 0, k.last_error()
         us = time_loop(torch, fn, iters, warmup=2)
-        unique = int((cnts_d > 0).sum().item())
+        unique = int(torch.unique(idx).numel()) if one_call else int((cnts_d > 0).sum().item())
         return us, unique
 
     small = {}
     for M in (() if prefill_only else small_sizes):      # by default: verification sizes, then the reference's prefill chunk sizes (RuntimeConfiguration.swift:24)
         us, unique = run(M, iters=50)
+        entry = {"us_grouped_calls": round(us, 2)}
+        if M <= 32:      # tf_prefill_routed_moe_few_tokens serves up to 32 token rows
+            us_one, unique_one = run(M, iters=50, one_call=True)
+            assert unique_one == unique, (unique_one, unique)
+            entry["us_one_call"] = round(us_one, 2)
+            us = min(us, us_one)
         nbytes = unique * expert_bytes + E * D + M * (2 * D * 2 + TOPK * F_MOE * 2 * 2 + TOPK * D * 2 * 2)
-        small[str(M)] = {"us": round(us, 2), "unique_experts": unique, "GBps_on_unique_expert_bytes": round(nbytes / (us * 1e-6) / 1e9, 1),
+        small[str(M)] = {"us": round(us, 2), **entry, "unique_experts": unique, "GBps_on_unique_expert_bytes": round(nbytes / (us * 1e-6) / 1e9, 1),
                          "tokens_per_s": round(M / (us * 1e-6), 1)}
     if small:
-        res["small_m"] = {"workload": "configs[3]: M tokens x top-8 over 128 resident experts (router block + grouping + grouped experts + reduce)",
+        res["small_m"] = {"workload": "configs[3]: M tokens x top-8 over 128 resident experts (router block + grouping + grouped experts + reduce; "
+                                      "us = the faster of the grouped calls, five launches, and the one-call form for up to 32 tokens, three launches)",
                           "per_M": small}
     if small_only:
         return res

@@ -700,6 +700,37 @@ int32_t tf_prefill_router_group_block(tf_ctx *ctx, tf_stream stream,
                                       uint32_t hidden_stride_elements,
                                       void *sorted_pairs, void *per_expert_offsets, void *per_expert_counts,
                                       void *chunks, void *chunk_count);
+/* A few token rows (multi-token verification: up to 32, top_k == 8, at most 128 experts in a resident pool) through the whole
+ * routed path as ONE call of three launches: tf_prefill_router_group_block, tf_prefill_grouped_routed_moe_resident and
+ * tf_prefill_moe_reduce_token_major (PrefillRouter.encodeGemma4Block, PrefillRouter.swift:37-89; the host grouping,
+ * PrefillMoEGrouping.swift:90-193; PrefillGroupedRoutedMoE.encodeStreamedBatched, PrefillGroupedRoutedMoE.swift:386-461;
+ * PrefillMoE.encodeReduceTokenMajor, PrefillMoE.swift:11-38; in RealForwardRunner.swift:922-1156 the router reads routerX and
+ * the experts routedX, hence the two hidden arguments).  Nothing is sorted: every block of the gate / up launch repeats its
+ * token's selection and finds the other tokens that chose its expert by counting, the first such token's blocks read the
+ * expert's rows once for all of them; the down launch reads each expert in use once and adds a token's eight partial results
+ * in rank order itself.  Outputs: out_indices uint32[T, 8], out_weights fp16[T, 8] (the router's), route_partials fp16[T, 8, d]
+ * (unweighted, as the grouped call leaves them), h2 fp16[T, d].  acts_scratch: T * 8 * f halves.  Same arithmetic as the three
+ * calls (fp16 activations and partials, fused multiply-adds in rank order); sums inside a dot product are taken in another order,
+ * so results agree to rounding, not bit for bit.  Returns TF_ERR_UNAVAILABLE, with nothing enqueued, for shapes it does not
+ * serve (more tokens, another top_k, num_experts > 128 or not a multiple of 4, d outside (1024, 4096], f > 1024, operands not
+ * 16-byte aligned, strides not multiples of 8): the caller makes the three calls. */
+int32_t tf_prefill_routed_moe_few_tokens(tf_ctx *ctx, tf_stream stream,
+                                         const void *weights, uint64_t weights_offset,
+                                         const void *scales, uint64_t scales_offset,
+                                         const void *biases, uint64_t biases_offset,
+                                         const void *hidden, uint64_t hidden_offset,
+                                         const void *effective_scale, uint64_t effective_scale_offset,
+                                         const void *per_expert_scale, uint64_t per_expert_scale_offset,
+                                         void *out_indices, uint64_t out_indices_offset,
+                                         void *out_weights, uint64_t out_weights_offset,
+                                         uint32_t query_count, uint32_t num_experts, uint32_t d, uint32_t top_k,
+                                         uint32_t hidden_stride_elements,
+                                         const void *routed_hidden, uint64_t routed_hidden_offset,
+                                         uint32_t routed_hidden_stride_elements,
+                                         const void *expert_pool, uint64_t expert_pool_stride,
+                                         const tf_expert_offsets *routed_offsets,
+                                         void *acts_scratch, void *route_partials, void *h2, uint64_t h2_offset,
+                                         uint32_t f, tf_dtype scale_dtype);
 /* Resident-pool form of the same computation over ALL sorted pairs of a chunk of tokens in one go: experts are
  * pool + expert * pool_stride, the work list comes from tf_prefill_group_pairs_device, nothing is read by the host.  Groups
  * of a few pairs stream each expert row once and apply it to every routed token (weight-read bound, the small-M regime);

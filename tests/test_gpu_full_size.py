@@ -224,6 +224,121 @@ def test_few_tokens_over_the_128_expert_pool(pool, M):
     assert np.max(np.abs(dec - r["h2"])) <= 4e-3 * max(1.0, float(np.max(np.abs(dec))))
 
 
+def few_tokens_inputs(M, seed, copy_of=None):
+    """Router operands of the production shape and M token rows; copy_of: {row: source row} duplicates (tokens that share all eight experts)."""
+    rng = np.random.default_rng(seed)
+    W, S, B = refcases.synthetic_int8(E, D, seed)
+    router_x = np.stack([refcases.normal_f16(D, seed * 64 + r) for r in range(M)])
+    routed_x = rng.standard_normal((M, D)).astype(np.float16).view(np.uint16)
+    for row, src in (copy_of or {}).items():
+        router_x[row] = router_x[src]
+    eff = tfo.bf16_bits_array(rng.uniform(0.5, 1.5, D).astype(np.float32) / np.float32(np.sqrt(D)))
+    pes = tfo.bf16_bits_array(rng.uniform(0.6, 1.4, E).astype(np.float32))
+    return W, S, B, router_x, routed_x, eff, pes
+
+
+def run_few_tokens(pool, W, S, B, router_x, routed_x, eff, pes, expect=tfk.TF_OK):
+    M = router_x.shape[0]
+    k = ctx()
+    n = M * TOPK
+    koff = tfk.ExpertOffsets(*pool["off"].as_tuple())
+    keep = [dev(a) for a in (W, S, B, router_x, eff, pes, routed_x)]
+    dW, dS, dB, dh, de, dp, dx = keep
+    idx, wts = zeros_bytes(n * 4, 0xEE), zeros_bytes(n * 2, 0xEE)
+    acts = zeros_bytes(n * F * 2)
+    partials = torch.full((n * D,), SENTINEL - 0x10000, dtype=torch.int16, device="cuda").view(torch.uint8)
+    h2 = torch.full((M * D,), SENTINEL - 0x10000, dtype=torch.int16, device="cuda").view(torch.uint8)
+    rc = k.lib.tf_prefill_routed_moe_few_tokens(k.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dh.data_ptr(), 0, de.data_ptr(), 0,
+                                                dp.data_ptr(), 0, idx.data_ptr(), 0, wts.data_ptr(), 0, M, E, D, TOPK, D, dx.data_ptr(), 0, D,
+                                                pool["dev"].data_ptr(), pool["stride"], C.byref(koff), acts.data_ptr(), partials.data_ptr(),
+                                                h2.data_ptr(), 0, F, tfk.TF_BF16)
+    assert rc == expect, k.last_error()
+    k.synchronize()
+    return dict(idx=host(idx, np.uint32, n).reshape(M, TOPK), w_bits=host(wts, np.uint16, n).reshape(M, TOPK),
+                partials=host(partials, np.uint16, n * D).reshape(M, TOPK, D), h2_bits=host(h2, np.uint16, M * D).reshape(M, D))
+
+
+def pairs_of(idx, w_bits):
+    """token-major pairs of a routing (every pair of a token, in rank order): the layout the oracle's grouped path takes"""
+    M = idx.shape[0]
+    pairs = np.zeros(M * TOPK, tfo.PAIR_DTYPE)
+    pairs["token"] = np.repeat(np.arange(M, dtype=np.uint32), TOPK)
+    pairs["rank"] = np.tile(np.arange(TOPK, dtype=np.uint32), M)
+    pairs["expert"] = np.minimum(idx.ravel(), E - 1)
+    pairs["weight_bits"] = w_bits.ravel().astype(np.uint32)
+    return pairs
+
+
+@pytest.mark.parametrize("M,copy_of", [(1, None), (2, None), (2, {1: 0}), (3, {2: 0}), (4, None), (8, {5: 1, 7: 1}), (16, None), (32, {31: 0})])
+def test_few_tokens_in_one_call_of_three_launches(pool, M, copy_of):
+    # tf_prefill_routed_moe_few_tokens against the calls it replaces (router block + grouping, grouped experts over the resident
+    # pool, token-major reduce) and against the oracle, production shape, 128 experts.  Rows copied from another row choose that
+    # row's eight experts: the owner of an expert then serves several tokens (and a first pair several followers in the down launch).
+    W, S, B, router_x, routed_x, eff, pes = few_tokens_inputs(M, 0x7E0 + M, copy_of)
+    got = run_few_tokens(pool, W, S, B, router_x, routed_x, eff, pes)
+    assert not np.any(np.all(got["partials"] == SENTINEL, axis=2))
+    assert not np.any(np.all(got["h2_bits"] == SENTINEL, axis=1))
+    # the router's outputs: the block router's (its logits are summed in another order: same experts away from near ties, weights to fp16 rounding)
+    k = ctx()
+    keep = [dev(a) for a in (W, S, B, router_x, eff, pes)]
+    idx2, wts2 = zeros_bytes(M * TOPK * 4), zeros_bytes(M * TOPK * 2)
+    k.check(k.lib.tf_prefill_router_gemma4_block(k.handle, None, keep[0].data_ptr(), 0, keep[1].data_ptr(), 0, keep[2].data_ptr(), 0, keep[3].data_ptr(), 0,
+                                                 keep[4].data_ptr(), 0, keep[5].data_ptr(), 0, idx2.data_ptr(), 0, wts2.data_ptr(), 0, M, E, D, TOPK, D))
+    ref_idx = host(idx2, np.uint32, M * TOPK).reshape(M, TOPK)
+    ref_w = tfo.from_f16_bits(host(wts2, np.uint16, M * TOPK)).reshape(M, TOPK)
+    assert np.array_equal(got["idx"], ref_idx)
+    assert np.max(np.abs(tfo.from_f16_bits(got["w_bits"]) - ref_w)) <= 2e-3
+    for row, src in (copy_of or {}).items():
+        assert np.array_equal(got["idx"][row], got["idx"][src])
+    if M >= 8 or copy_of:
+        assert len(np.unique(got["idx"])) < M * TOPK          # experts are shared between tokens
+    # the grouped path on the same routing
+    r = run_block(pool, routed_x, got["idx"], got["w_bits"])
+    scale = float(np.max(np.abs(tfo.from_f16_bits(r["partials"]))))
+    assert within_north_star(tfo.from_f16_bits(got["partials"]), tfo.from_f16_bits(r["partials"]), abs_=1e-3 * max(1.0, scale))
+    assert within_north_star(tfo.from_f16_bits(got["h2_bits"]), r["h2"], abs_=1e-3 * max(1.0, scale))
+    # the reduce is exact given the partials: fused multiply-adds in rank order
+    want_h2 = tfo.prefill_reduce_token_major(got["partials"].ravel(), got["w_bits"].ravel(), M, TOPK, D).reshape(M, D)
+    assert np.array_equal(got["h2_bits"], want_h2)
+    # the oracle, every pair (up to 16 tokens) or the pairs of four tokens
+    tokens = np.arange(M, dtype=np.uint32) if M <= 16 else np.array([0, 1, M // 2, M - 1], np.uint32)
+    pairs = pairs_of(got["idx"], got["w_bits"])
+    pairs = pairs[np.isin(pairs["token"], tokens)]
+    want = tfo.prefill_route_partials(pairs, M, routed_x.ravel(), D, pool["flat"], pool["stride"], pool["off"], TOPK, D, F, fill_bits=0,
+                                      threads=8).reshape(M, TOPK, D)
+    assert within_north_star(tfo.from_f16_bits(got["partials"][tokens]), tfo.from_f16_bits(want[tokens]), abs_=1e-3 * max(1.0, scale))
+
+
+def test_few_tokens_in_one_call_when_a_token_has_fewer_than_eight_finite_logits(pool):
+    # 123 of the 128 router rows carry a NaN scale: every token has five finite logits, the selection fills ranks 5..7 with
+    # expert 0 at weight zero (the reference's rule for unfilled places), and nothing is shared between blocks.  Every pair's
+    # partial result is still that pair's expert applied to its token.
+    M = 4
+    W, S, B, router_x, routed_x, eff, pes = few_tokens_inputs(M, 0x7F5)
+    S = S.copy()
+    live = [3, 17, 64, 90, 127]
+    for e in range(E):
+        if e not in live:
+            S.reshape(E, -1)[e, :] = 0x7FC0
+    got = run_few_tokens(pool, W, S, B, router_x, routed_x, eff, pes)
+    for t in range(M):
+        assert sorted(got["idx"][t][:5]) == live and list(got["idx"][t][5:]) == [0, 0, 0]
+        assert list(got["w_bits"][t][5:]) == [0, 0, 0]
+    pairs = pairs_of(got["idx"], got["w_bits"])
+    want = tfo.prefill_route_partials(pairs, M, routed_x.ravel(), D, pool["flat"], pool["stride"], pool["off"], TOPK, D, F, fill_bits=0,
+                                      threads=8).reshape(M, TOPK, D)
+    scale = float(np.max(np.abs(tfo.from_f16_bits(want))))
+    assert within_north_star(tfo.from_f16_bits(got["partials"]), tfo.from_f16_bits(want), abs_=1e-3 * max(1.0, scale))
+    want_h2 = tfo.prefill_reduce_token_major(got["partials"].ravel(), got["w_bits"].ravel(), M, TOPK, D).reshape(M, D)
+    assert np.array_equal(got["h2_bits"], want_h2)
+
+
+def test_few_tokens_in_one_call_refuses_what_it_does_not_serve(pool):
+    W, S, B, router_x, routed_x, eff, pes = few_tokens_inputs(33, 0x7F9)
+    got = run_few_tokens(pool, W, S, B, router_x, routed_x, eff, pes, expect=tfk.TF_ERR_UNAVAILABLE)
+    assert np.all(got["idx"] == 0xEEEEEEEE) and np.all(got["h2_bits"] == SENTINEL)       # nothing was enqueued
+
+
 # ------------------------------------------------------------------------------------------------ config 4, second half
 F_SHARED = 2112
 

@@ -183,6 +183,9 @@ EXPORTS = {
                                              u32, u32, u32, u32, u32]),
     "tf_prefill_router_group_block": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64,
                                             u32, u32, u32, u32, u32, vp, vp, vp, vp, vp]),
+    "tf_prefill_routed_moe_few_tokens": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64, vp, u64,
+                                               u32, u32, u32, u32, u32, vp, u64, u32, vp, u64, C.POINTER(ExpertOffsets), vp, vp, vp, u64,
+                                               u32, i32]),
     "tf_prefill_make_token_expert_pairs": (i32, [vp, vp, i32, i32, vp]),
     "tf_prefill_group_token_expert_pairs": (i32, [vp, u64, i32, i32, i32, i32, vp, u64, vp, vp, vp, vp, vp, vp, vp]),
     "tf_prefill_group_pairs_device": (i32, [vp, vp, vp, vp, u32, u32, u32, vp, vp, vp, vp, vp]),

@@ -13,7 +13,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libtf_kernels.so")
-SOURCES = ["tf_context.hip", "tf_gemv.hip", "tf_moe.hip", "tf_lmhead.hip", "tf_prefill.hip", "tf_qmm.hip", "tf_glue.hip", "tf_sampling.hip", "tf_loader.hip", "tf_attention.hip", "tf_rope.hip", "tf_bench.hip"]
+SOURCES = ["tf_context.hip", "tf_gemv.hip", "tf_moe.hip", "tf_lmhead.hip", "tf_prefill.hip", "tf_prefill_few.hip", "tf_qmm.hip", "tf_glue.hip", "tf_sampling.hip", "tf_loader.hip", "tf_attention.hip", "tf_rope.hip", "tf_bench.hip"]
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
 # Kernel-argument preloading: gfx950 can hand the leading scalar arguments to a wave in registers at launch instead of through
