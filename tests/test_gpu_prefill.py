@@ -357,6 +357,59 @@ def test_quad_kernels_long_chunks_and_row_widths(T, E, d, f):
     check_against_oracle(r, T, d, f, top_k, abs_tol=1e-3 * max(1.0, scale))
 
 
+@pytest.mark.parametrize("T,E,d,f,fp16_scales", [(3, 16, 1536, 128, False), (5, 64, 2048, 256, True), (2, 32, 4096, 64, False), (7, 128, 2304, 192, True),
+                                                 (4, 12, 2816, 1024, False)])
+def test_few_tokens_in_one_call_other_row_widths_and_fp16_scales(T, E, d, f, fp16_scales):
+    # tf_prefill_routed_moe_few_tokens away from the production shape: rows that take tiles of four rows in three passes (1536),
+    # one row in one or two passes (2048, 4096), two mirrored rows with a partly filled pass (2304, 2816); down rows of 2, 6, 8, 32
+    # chunks; 12 to 128 experts; scales as fp16.  Routing = the block router's, partials = the oracle's for those pairs, h2 = the
+    # reduce of the partials bit for bit.
+    top_k, seed = 8, 0x5F00 + T
+    rng = np.random.default_rng(seed)
+    blobs, off = [], None
+    for e in range(E):
+        blob, off = tfo.make_blob(refcases.synthetic_int4(f, d, seed + e, "g"), refcases.synthetic_int4(f, d, seed + e, "u"),
+                                  refcases.synthetic_int4(d, f, seed + e, "d"))
+        blobs.append(blob)
+    oracle_blobs = blobs
+    if fp16_scales:
+        blobs = [scales_as_fp16(b, off, d, f) for b in blobs]
+        oracle_blobs = [bf16_pool_matching(b, off, d, f) for b in blobs]
+    stride = (blobs[0].size + 255) // 256 * 256
+    pool_np, oracle_pool = np.zeros((E, stride), np.uint8), np.zeros((E, stride), np.uint8)
+    for e in range(E):
+        pool_np[e, :blobs[e].size] = blobs[e]
+        oracle_pool[e, :blobs[e].size] = oracle_blobs[e]
+    router_x = np.concatenate([refcases.normal_f16(d, seed * 8 + r) for r in range(T)])
+    router_x[(T - 1) * d:] = router_x[:d]                     # the last row chooses the first row's experts
+    routed_x = rng.standard_normal((T, d)).astype(np.float16).view(np.uint16)
+    rW, rS, rB = refcases.synthetic_int8(E, d, seed)
+    eff = tfo.bf16_bits_array((rng.uniform(0.5, 1.5, d) / np.sqrt(d)).astype(np.float32))
+    pes = tfo.bf16_bits_array(rng.uniform(0.6, 1.4, E).astype(np.float32))
+    k = ctx()
+    n = T * top_k
+    koff = tfk.ExpertOffsets(*off.as_tuple())
+    dW, dS, dB, dh, de, dp, dx, d_pool = (dev(a) for a in (rW, rS, rB, router_x, eff, pes, routed_x, pool_np))
+    idx, wts = zeros_bytes(n * 4, 0xEE), zeros_bytes(n * 2, 0xEE)
+    acts, partials, h2 = zeros_bytes(n * f * 2), zeros_bytes(n * d * 2, 0xEE), zeros_bytes(T * d * 2, 0xEE)
+    k.check(k.lib.tf_prefill_routed_moe_few_tokens(k.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dh.data_ptr(), 0, de.data_ptr(), 0,
+                                                   dp.data_ptr(), 0, idx.data_ptr(), 0, wts.data_ptr(), 0, T, E, d, top_k, d, dx.data_ptr(), 0, d,
+                                                   d_pool.data_ptr(), stride, C.byref(koff), acts.data_ptr(), partials.data_ptr(), h2.data_ptr(), 0, f,
+                                                   tfk.TF_FP16 if fp16_scales else tfk.TF_BF16))
+    got_idx, got_w = host(idx, np.uint32, n).reshape(T, top_k), host(wts, np.uint16, n).reshape(T, top_k)
+    ref_idx, ref_w = prefill_router(rW, rS, rB, router_x, d, eff, pes, T)
+    assert np.array_equal(got_idx, ref_idx) and np.array_equal(got_idx[T - 1], got_idx[0])
+    assert np.max(np.abs(tfo.from_f16_bits(got_w) - ref_w)) <= 2e-3
+    pairs = np.zeros(n, tfo.PAIR_DTYPE)
+    pairs["token"], pairs["rank"] = np.repeat(np.arange(T, dtype=np.uint32), top_k), np.tile(np.arange(top_k, dtype=np.uint32), T)
+    pairs["expert"], pairs["weight_bits"] = got_idx.ravel(), got_w.ravel().astype(np.uint32)
+    want = tfo.prefill_route_partials(pairs, T, routed_x.ravel(), d, oracle_pool.ravel(), stride, off, top_k, d, f, fill_bits=0, threads=8)
+    got_p = host(partials, np.uint16, n * d)
+    scale = float(np.max(np.abs(tfo.from_f16_bits(want))))
+    assert within_north_star(tfo.from_f16_bits(got_p), tfo.from_f16_bits(want), abs_=1e-3 * max(1.0, scale))
+    assert np.array_equal(host(h2, np.uint16, T * d), tfo.prefill_reduce_token_major(got_p, got_w.ravel(), T, top_k, d))
+
+
 @pytest.mark.parametrize("T", [6, 12, 24])
 def test_grouped_experts_fp16_scales_equal_bf16_scales(T):
     # the reference's expert blobs carry bf16 scales, and so does the oracle; the fp16 variant of the grouped kernels is pinned
