@@ -69,6 +69,19 @@ __global__ __launch_bounds__(256) void prefill_logits_kernel(const uint8_t *W, c
     if (lane == 0) logits[(size_t)t * num_experts + e] = v;
 }
 
+// The same logits with one 256-thread block per (expert, token) where every operand is 16-byte aligned and d <= 4096: thread c
+// takes chunk c of 16 weights, so a row is one memory round trip and a sixteenth of a wave's arithmetic (the decode router's
+// row, router_row_block).
+__global__ __launch_bounds__(256) void prefill_logits_block_kernel(const uint8_t *W, const uint8_t *S, const uint8_t *B, const half_t *hidden,
+                                                                   long hidden_stride, const uint16_t *eff, float *logits, uint32_t num_experts, int d) {
+    __shared__ float partial[4];
+    const uint32_t e = blockIdx.x, t = blockIdx.y;
+    const int groups = d >> 6;
+    const float v = router_row_block<0>(W + (size_t)e * d, S + (size_t)e * groups * 2, B + (size_t)e * groups * 2,
+                                        hidden + (size_t)t * hidden_stride, eff, d, partial);
+    if (threadIdx.x == 0) logits[(size_t)t * num_experts + e] = v;
+}
+
 // planes > 0: the token's logits are first summed, in plane order, from `planes` partial planes that follow the
 // [tokens, experts] logits array (each lane sums the entries it will read back), then selected from.
 __global__ __launch_bounds__(64) void prefill_select_kernel(float *logits, const uint16_t *per_expert_scale,
@@ -369,8 +382,20 @@ __global__ __launch_bounds__(64) void group_place_kernel(const uint32_t *indices
 
 // A single segment (at most 32 tokens, the multi-token verification case): the three steps by the first 256 threads of one
 // block (every thread of the block must call: the barriers are block-wide).  indices / weights may live in LDS.
+__device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v) {
+    auto shifted = [](uint32_t x, auto ctrl, auto rows) {
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, decltype(ctrl)::value, decltype(rows)::value, 0xF, false);
+    };
+    v += shifted(v, std::integral_constant<int, 0x111>{}, std::integral_constant<int, 0xF>{});      // row_shr:1 (no source inside the row of 16: adds 0)
+    v += shifted(v, std::integral_constant<int, 0x112>{}, std::integral_constant<int, 0xF>{});      // row_shr:2
+    v += shifted(v, std::integral_constant<int, 0x114>{}, std::integral_constant<int, 0xF>{});      // row_shr:4
+    v += shifted(v, std::integral_constant<int, 0x118>{}, std::integral_constant<int, 0xF>{});      // row_shr:8
+    v += shifted(v, std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xA>{});      // row_bcast15 into rows 1 and 3
+    v += shifted(v, std::integral_constant<int, 0x143>{}, std::integral_constant<int, 0xC>{});      // row_bcast31 into rows 2 and 3
+    return v;
+}
 struct GroupSmallLds {
-    uint32_t cnt[256], scan_pairs[256], scan_chunks[256], next[256];
+    uint32_t cnt[256], scan_pairs[4], scan_chunks[4], next[256];      // scan_*: the four owner waves' totals
     unsigned long long mask[256];
 };
 __device__ __forceinline__ void group_small_body(GroupSmallLds &l, const uint32_t *indices, const uint16_t *weights, uint32_t n_pairs, uint32_t top_k,
@@ -388,23 +413,23 @@ __device__ __forceinline__ void group_small_body(GroupSmallLds &l, const uint32_
     __syncthreads();
     const uint32_t total = owner ? l.cnt[e] : 0u;
     const uint32_t nch = (total + kChunkPairs - 1) / kChunkPairs;
-    if (owner) {
-        l.scan_pairs[e] = total;
-        l.scan_chunks[e] = nch;
+    // running sums over the experts: inside each of the four owner waves across lanes, then the waves before added on
+    uint32_t sum_pairs = wave_inclusive_scan_u32(total), sum_chunks = wave_inclusive_scan_u32(nch);
+    const uint32_t wave = threadIdx.x >> 6;
+    if (owner && (threadIdx.x & 63) == 63) {
+        l.scan_pairs[wave] = sum_pairs;
+        l.scan_chunks[wave] = sum_chunks;
     }
     __syncthreads();
-    for (uint32_t step = 1; step < 256; step <<= 1) {
-        const uint32_t a = owner && e >= step ? l.scan_pairs[e - step] : 0u, c = owner && e >= step ? l.scan_chunks[e - step] : 0u;
-        __syncthreads();
-        if (owner) {
-            l.scan_pairs[e] += a;
-            l.scan_chunks[e] += c;
+    if (owner) {
+        for (uint32_t w = 0; w < wave; ++w) {
+            sum_pairs += l.scan_pairs[w];
+            sum_chunks += l.scan_chunks[w];
         }
-        __syncthreads();
     }
     if (owner) {
-        const uint32_t start = l.scan_pairs[e] - total, chunk_start = l.scan_chunks[e] - nch;
-        if (e == 255) chunk_count[0] = l.scan_chunks[255];
+        const uint32_t start = sum_pairs - total, chunk_start = sum_chunks - nch;
+        if (e == 255) chunk_count[0] = sum_chunks;
         if (e < num_experts) {
             per_expert_offsets[e] = total ? start : 0xFFFFFFFFu;
             per_expert_counts[e] = total;
@@ -1297,6 +1322,22 @@ int32_t run_grouped(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const t
 
 }  // namespace
 
+namespace {
+
+// The router logits of up to kFewTokens token rows into `logits` [tokens, experts]: a block per (expert, token) for aligned
+// operands (fast), else a wave per (expert, token) with byte loads.
+void launch_few_token_logits(hipStream_t st, const uint8_t *w, const uint8_t *s, const uint8_t *b, const half_t *h, uint32_t hidden_stride_elements,
+                             const uint16_t *eff, float *logits, uint32_t query_count, uint32_t num_experts, uint32_t d, bool fast) {
+    if (fast)
+        hipLaunchKernelGGL(prefill_logits_block_kernel, dim3(num_experts, query_count), dim3(256), 0, st, w, s, b, h, (long)hidden_stride_elements, eff,
+                           logits, num_experts, (int)d);
+    else
+        hipLaunchKernelGGL(prefill_logits_kernel<0>, dim3((num_experts + 3) / 4, query_count), dim3(256), 0, st, w, s, b, h,
+                           (long)hidden_stride_elements, eff, logits, num_experts, (int)d);
+}
+
+}  // namespace
+
 namespace tfk {
 
 // logits [tokens, experts] plus up to four partial planes of the split reduction, never less than the few-token router needs
@@ -1355,18 +1396,7 @@ int32_t tf_prefill_router_gemma4_block(tf_ctx *ctx, tf_stream stream, const void
                                (long)hidden_stride_elements, eff, ctx->prefill_logits + (planes ? plane : 0), query_count, num_experts, (int)d,
                                groups_per_split);
         } else {
-            const dim3 grid((num_experts + 3) / 4, query_count);
-#define TF_PL(NP_)                                                                                                           \
-    hipLaunchKernelGGL(prefill_logits_kernel<NP_>, grid, dim3(256), 0, st, w, s, b, h, (long)hidden_stride_elements, eff,    \
-                       ctx->prefill_logits, num_experts, (int)d)
-            switch (npass) {
-                case 1: TF_PL(1); break;
-                case 2: TF_PL(2); break;
-                case 3: TF_PL(3); break;
-                case 4: TF_PL(4); break;
-                default: TF_PL(0); break;
-            }
-#undef TF_PL
+            launch_few_token_logits(st, w, s, b, h, hidden_stride_elements, eff, ctx->prefill_logits, query_count, num_experts, d, fast);
         }
         const int32_t rc = check_launch(ctx, "prefill_router logits");
         if (rc != TF_OK) return rc;
@@ -1529,20 +1559,8 @@ int32_t tf_prefill_router_group_block(tf_ctx *ctx, tf_stream stream, const void 
         return scratch_too_small(ctx, "prefill_router", need * sizeof(float), ctx->prefill_logits_count * sizeof(float));
     if (query_count <= kSelectGroupTokens && top_k <= kSelectGroupTopK) {
         const bool fast = aligned16(w) && aligned16(h) && aligned16(eff) && hidden_stride_elements % 8 == 0 && d <= 4096;
-        const int npass = fast ? (int)((d / 16 + 63) / 64) : 0;
         hipStream_t st = static_cast<hipStream_t>(stream);
-        const dim3 grid((num_experts + 3) / 4, query_count);
-#define TF_PL(NP_)                                                                                                           \
-    hipLaunchKernelGGL(prefill_logits_kernel<NP_>, grid, dim3(256), 0, st, w, s, b, h, (long)hidden_stride_elements, eff,    \
-                       ctx->prefill_logits, num_experts, (int)d)
-        switch (npass) {
-            case 1: TF_PL(1); break;
-            case 2: TF_PL(2); break;
-            case 3: TF_PL(3); break;
-            case 4: TF_PL(4); break;
-            default: TF_PL(0); break;
-        }
-#undef TF_PL
+        launch_few_token_logits(st, w, s, b, h, hidden_stride_elements, eff, ctx->prefill_logits, query_count, num_experts, d, fast);
         const int32_t rc = check_launch(ctx, "prefill_router logits");
         if (rc != TF_OK) return rc;
         hipLaunchKernelGGL(select_group_small_kernel, dim3(1), dim3(1024), 0, st, ctx->prefill_logits, pes, oi, ow, query_count, num_experts, top_k,
