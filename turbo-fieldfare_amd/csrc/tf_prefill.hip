@@ -380,8 +380,12 @@ __global__ __launch_bounds__(64) void group_place_kernel(const uint32_t *indices
     }
 }
 
-// A single segment (at most 32 tokens, the multi-token verification case): the three steps by the first 256 threads of one
-// block (every thread of the block must call: the barriers are block-wide).  indices / weights may live in LDS.
+// Up to kGroupBlockPairs pairs (256 tokens at top-8) in ONE block: the three steps above with the segments (64 pairs each, one
+// wave's worth) kept in LDS.  A wave counts its segments' pairs per expert; thread e runs over expert e's segment counts and the
+// experts are scanned across lanes; then every wave places its segments' pairs, each lane ranking itself among the lanes of the
+// same expert (the lanes whose expert number agrees in every bit: eight ballots).  Every thread of the block must call (block-wide
+// barriers); the block has at least 256 threads.  indices / weights may live in LDS.
+constexpr uint32_t kGroupBlockPairs = 2048, kGroupBlockSegments = kGroupBlockPairs / 64;
 __device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v) {
     auto shifted = [](uint32_t x, auto ctrl, auto rows) {
         return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, decltype(ctrl)::value, decltype(rows)::value, 0xF, false);
@@ -394,40 +398,43 @@ __device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v) {
     v += shifted(v, std::integral_constant<int, 0x143>{}, std::integral_constant<int, 0xC>{});      // row_bcast31 into rows 2 and 3
     return v;
 }
-struct GroupSmallLds {
-    uint32_t cnt[256], scan_pairs[4], scan_chunks[4], next[256];      // scan_*: the four owner waves' totals
-    unsigned long long mask[256];
+struct GroupBlockLds {
+    uint32_t seg[kGroupBlockSegments][256];      // [segment][expert]: pair counts, then the position of the segment's first pair of the expert
+    uint32_t wave_pairs[4], wave_chunks[4];      // totals of the four waves that own the experts
 };
-__device__ __forceinline__ void group_small_body(GroupSmallLds &l, const uint32_t *indices, const uint16_t *weights, uint32_t n_pairs, uint32_t top_k,
+__device__ __forceinline__ void group_block_body(GroupBlockLds &l, const uint32_t *indices, const uint16_t *weights, uint32_t n_pairs, uint32_t top_k,
                                                  uint32_t num_experts, tf_prefill_pair *sorted_pairs, uint32_t *per_expert_offsets,
                                                  uint32_t *per_expert_counts, tf_prefill_group *chunks, uint32_t *chunk_count) {
-    const uint32_t e = threadIdx.x;
+    const uint32_t e = threadIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, waves = blockDim.x >> 6;
     const bool owner = e < 256;        // thread e owns expert e
-    if (owner) {
-        l.cnt[e] = 0;
-        l.mask[e] = 0ull;
+    const uint32_t n_seg = (n_pairs + 63) / 64;
+    for (uint32_t i = threadIdx.x; i < n_seg * 256; i += blockDim.x) (&l.seg[0][0])[i] = 0u;
+    __syncthreads();
+    for (uint32_t s = wave; s < n_seg; s += waves) {
+        const uint32_t i = s * 64 + lane;
+        if (i < n_pairs) atomicAdd(&l.seg[s][clamp_expert(indices[i], num_experts)], 1u);
     }
     __syncthreads();
+    uint32_t total = 0;
     if (owner)
-        for (uint32_t i = e; i < n_pairs; i += 256) atomicAdd(&l.cnt[clamp_expert(indices[i], num_experts)], 1u);
-    __syncthreads();
-    const uint32_t total = owner ? l.cnt[e] : 0u;
+        for (uint32_t s = 0; s < n_seg; ++s) {
+            const uint32_t c = l.seg[s][e];
+            l.seg[s][e] = total;      // exclusive prefix inside expert e
+            total += c;
+        }
     const uint32_t nch = (total + kChunkPairs - 1) / kChunkPairs;
     // running sums over the experts: inside each of the four owner waves across lanes, then the waves before added on
     uint32_t sum_pairs = wave_inclusive_scan_u32(total), sum_chunks = wave_inclusive_scan_u32(nch);
-    const uint32_t wave = threadIdx.x >> 6;
-    if (owner && (threadIdx.x & 63) == 63) {
-        l.scan_pairs[wave] = sum_pairs;
-        l.scan_chunks[wave] = sum_chunks;
+    if (owner && lane == 63) {
+        l.wave_pairs[wave] = sum_pairs;
+        l.wave_chunks[wave] = sum_chunks;
     }
     __syncthreads();
     if (owner) {
         for (uint32_t w = 0; w < wave; ++w) {
-            sum_pairs += l.scan_pairs[w];
-            sum_chunks += l.scan_chunks[w];
+            sum_pairs += l.wave_pairs[w];
+            sum_chunks += l.wave_chunks[w];
         }
-    }
-    if (owner) {
         const uint32_t start = sum_pairs - total, chunk_start = sum_chunks - nch;
         if (e == 255) chunk_count[0] = sum_chunks;
         if (e < num_experts) {
@@ -441,33 +448,36 @@ __device__ __forceinline__ void group_small_body(GroupSmallLds &l, const uint32_
             g.pair_count = min(kChunkPairs, total - c * kChunkPairs);
             chunks[chunk_start + c] = g;
         }
-        l.next[e] = start;
+        for (uint32_t s = 0; s < n_seg; ++s) l.seg[s][e] += start;
     }
     __syncthreads();
-    if (threadIdx.x >= 64) return;
-    const uint32_t lane = threadIdx.x;
-    for (uint32_t i0 = 0; i0 < n_pairs; i0 += 64) {
-        const uint32_t i = i0 + lane;
+    for (uint32_t s = wave; s < n_seg; s += waves) {
+        const uint32_t i = s * 64 + lane;
         const bool valid = i < n_pairs;
-        const uint32_t x = valid ? clamp_expert(indices[i], num_experts) : 0u;
+        const uint32_t x = valid ? clamp_expert(indices[i], num_experts) : 0x100u;      // bit 8: no pair
         const uint16_t wbits = valid ? weights[i] : (uint16_t)0;
-        const uint32_t pos = place_batch(x, valid, lane, l.mask, l.next);
+        unsigned long long same = ~0ull;      // the lanes whose expert number equals this lane's
+#pragma unroll
+        for (uint32_t bit = 0; bit < 9; ++bit) {
+            const unsigned long long set = __ballot((x >> bit) & 1u);
+            same &= ((x >> bit) & 1u) ? set : ~set;
+        }
         if (valid) {
             tf_prefill_pair p;
             p.token = i / top_k;
             p.expert = x;
             p.rank = i - p.token * top_k;
             p.weight_bits_and_reserved = (uint32_t)wbits;
-            sorted_pairs[pos] = p;
+            sorted_pairs[l.seg[s][x] + (uint32_t)__builtin_popcountll(same & ((1ull << lane) - 1ull))] = p;
         }
     }
 }
-__global__ __launch_bounds__(256) void group_small_kernel(const uint32_t *indices, const uint16_t *weights, uint32_t n_pairs,
-                                                          uint32_t top_k, uint32_t num_experts, tf_prefill_pair *sorted_pairs,
-                                                          uint32_t *per_expert_offsets, uint32_t *per_expert_counts,
-                                                          tf_prefill_group *chunks, uint32_t *chunk_count) {
-    __shared__ GroupSmallLds l;
-    group_small_body(l, indices, weights, n_pairs, top_k, num_experts, sorted_pairs, per_expert_offsets, per_expert_counts, chunks, chunk_count);
+__global__ __launch_bounds__(1024) void group_block_kernel(const uint32_t *indices, const uint16_t *weights, uint32_t n_pairs,
+                                                           uint32_t top_k, uint32_t num_experts, tf_prefill_pair *sorted_pairs,
+                                                           uint32_t *per_expert_offsets, uint32_t *per_expert_counts,
+                                                           tf_prefill_group *chunks, uint32_t *chunk_count) {
+    __shared__ GroupBlockLds l;
+    group_block_body(l, indices, weights, n_pairs, top_k, num_experts, sorted_pairs, per_expert_offsets, per_expert_counts, chunks, chunk_count);
 }
 
 // The selection of up to kSelectGroupTokens token rows and the grouping of their pairs in ONE block of sixteen waves: wave w
@@ -479,7 +489,7 @@ __global__ __launch_bounds__(1024) void select_group_small_kernel(const float *l
                                                                   half_t *out_weights, uint32_t tokens, uint32_t num_experts, uint32_t top_k,
                                                                   tf_prefill_pair *sorted_pairs, uint32_t *per_expert_offsets,
                                                                   uint32_t *per_expert_counts, tf_prefill_group *chunks, uint32_t *chunk_count) {
-    __shared__ GroupSmallLds l;
+    __shared__ GroupBlockLds l;
     __shared__ uint32_t s_idx[kSelectGroupTokens * kSelectGroupTopK];
     __shared__ uint16_t s_w[kSelectGroupTokens * kSelectGroupTopK];
     const int lane = threadIdx.x & 63;
@@ -495,7 +505,7 @@ __global__ __launch_bounds__(1024) void select_group_small_kernel(const float *l
         }
     }
     __syncthreads();
-    group_small_body(l, s_idx, s_w, tokens * top_k, top_k, num_experts, sorted_pairs, per_expert_offsets, per_expert_counts, chunks, chunk_count);
+    group_block_body(l, s_idx, s_w, tokens * top_k, top_k, num_experts, sorted_pairs, per_expert_offsets, per_expert_counts, chunks, chunk_count);
 }
 
 // ------------------------------------------------------------------------------------------------ grouped, row-streaming
@@ -1513,8 +1523,9 @@ int32_t tf_prefill_group_pairs_device(tf_ctx *ctx, tf_stream stream, const void 
     const uint32_t n_segments = (query_count + seg_tokens - 1) / seg_tokens;
     const uint32_t seg_pairs = seg_tokens * top_k;
     const uint32_t *idx = static_cast<const uint32_t *>(indices);
-    if (n_segments == 1) {
-        hipLaunchKernelGGL(group_small_kernel, dim3(1), dim3(256), 0, st, idx, static_cast<const uint16_t *>(weights), n_pairs, top_k,
+    if (n_pairs <= kGroupBlockPairs) {
+        const uint32_t threads = n_pairs <= 256 ? 256u : n_pairs <= 512 ? 512u : 1024u;      // a wave per 64 pairs, at least the 256 expert owners
+        hipLaunchKernelGGL(group_block_kernel, dim3(1), dim3(threads), 0, st, idx, static_cast<const uint16_t *>(weights), n_pairs, top_k,
                            num_experts, static_cast<tf_prefill_pair *>(sorted_pairs), static_cast<uint32_t *>(per_expert_offsets),
                            static_cast<uint32_t *>(per_expert_counts), static_cast<tf_prefill_group *>(chunks),
                            static_cast<uint32_t *>(chunk_count));
