@@ -357,13 +357,14 @@ def test_quad_kernels_long_chunks_and_row_widths(T, E, d, f):
     check_against_oracle(r, T, d, f, top_k, abs_tol=1e-3 * max(1.0, scale))
 
 
-@pytest.mark.parametrize("T,E,d,f,fp16_scales", [(3, 16, 1536, 128, False), (5, 64, 2048, 256, True), (2, 32, 4096, 64, False), (7, 128, 2304, 192, True),
-                                                 (4, 12, 2816, 1024, False)])
-def test_few_tokens_in_one_call_other_row_widths_and_fp16_scales(T, E, d, f, fp16_scales):
+@pytest.mark.parametrize("T,E,d,f,fp16_scales,pad", [(3, 16, 1536, 128, False, 0), (5, 64, 2048, 256, True, 8), (2, 32, 4096, 64, False, 0),
+                                                     (7, 128, 2304, 192, True, 24), (4, 12, 2816, 1024, False, 16)])
+def test_few_tokens_in_one_call_other_row_widths_and_fp16_scales(T, E, d, f, fp16_scales, pad):
     # tf_prefill_routed_moe_few_tokens away from the production shape: rows that take tiles of four rows in three passes (1536),
     # one row in one or two passes (2048, 4096), two mirrored rows with a partly filled pass (2304, 2816); down rows of 2, 6, 8, 32
-    # chunks; 12 to 128 experts; scales as fp16.  Routing = the block router's, partials = the oracle's for those pairs, h2 = the
-    # reduce of the partials bit for bit.
+    # chunks; 12 to 128 experts; scales as fp16; token rows `pad` halves apart beyond their length (the router's rows and the
+    # experts' rows with different strides, both buffers entered at a byte offset).  Routing = the block router's, partials = the
+    # oracle's for those pairs, h2 = the reduce of the partials bit for bit.
     top_k, seed = 8, 0x5F00 + T
     rng = np.random.default_rng(seed)
     blobs, off = [], None
@@ -389,11 +390,18 @@ def test_few_tokens_in_one_call_other_row_widths_and_fp16_scales(T, E, d, f, fp1
     k = ctx()
     n = T * top_k
     koff = tfk.ExpertOffsets(*off.as_tuple())
-    dW, dS, dB, dh, de, dp, dx, d_pool = (dev(a) for a in (rW, rS, rB, router_x, eff, pes, routed_x, pool_np))
+    # strided copies of the two activation blocks, filled with a value no row holds
+    rs_, xs_, r_off, x_off = d + pad, d + 2 * pad, 32 if pad else 0, 64 if pad else 0
+    router_buf = np.full(r_off // 2 + T * rs_, tfo.f16_bits(-31.0), np.uint16)
+    routed_buf = np.full(x_off // 2 + T * xs_, tfo.f16_bits(-31.0), np.uint16)
+    for r in range(T):
+        router_buf[r_off // 2 + r * rs_:r_off // 2 + r * rs_ + d] = router_x[r * d:(r + 1) * d]
+        routed_buf[x_off // 2 + r * xs_:x_off // 2 + r * xs_ + d] = routed_x[r]
+    dW, dS, dB, dh, de, dp, dx, d_pool = (dev(a) for a in (rW, rS, rB, router_buf, eff, pes, routed_buf, pool_np))
     idx, wts = zeros_bytes(n * 4, 0xEE), zeros_bytes(n * 2, 0xEE)
     acts, partials, h2 = zeros_bytes(n * f * 2), zeros_bytes(n * d * 2, 0xEE), zeros_bytes(T * d * 2, 0xEE)
-    k.check(k.lib.tf_prefill_routed_moe_few_tokens(k.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dh.data_ptr(), 0, de.data_ptr(), 0,
-                                                   dp.data_ptr(), 0, idx.data_ptr(), 0, wts.data_ptr(), 0, T, E, d, top_k, d, dx.data_ptr(), 0, d,
+    k.check(k.lib.tf_prefill_routed_moe_few_tokens(k.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dh.data_ptr(), r_off, de.data_ptr(), 0,
+                                                   dp.data_ptr(), 0, idx.data_ptr(), 0, wts.data_ptr(), 0, T, E, d, top_k, rs_, dx.data_ptr(), x_off, xs_,
                                                    d_pool.data_ptr(), stride, C.byref(koff), acts.data_ptr(), partials.data_ptr(), h2.data_ptr(), 0, f,
                                                    tfk.TF_FP16 if fp16_scales else tfk.TF_BF16))
     got_idx, got_w = host(idx, np.uint32, n).reshape(T, top_k), host(wts, np.uint16, n).reshape(T, top_k)
