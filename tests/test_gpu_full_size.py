@@ -333,6 +333,67 @@ def test_few_tokens_in_one_call_when_a_token_has_fewer_than_eight_finite_logits(
     assert np.array_equal(got["h2_bits"], want_h2)
 
 
+def test_few_tokens_in_one_call_back_to_back_and_replayed_from_a_graph(pool):
+    # Calls of different sizes in a row on one stream without a host wait (the context's logits scratch and the outputs pass
+    # from launch to launch through device memory), then the same calls captured into a graph on a side stream and replayed three
+    # times with an eager call between the replays: every output bit for bit what the call gives when it runs alone.
+    sizes = [3, 1, 4, 2]
+    k = ctx()
+    koff = tfk.ExpertOffsets(*pool["off"].as_tuple())
+    cases = []
+    for i, M in enumerate(sizes):
+        W, S, B, router_x, routed_x, eff, pes = few_tokens_inputs(M, 0x7A00 + i, {M - 1: 0} if M > 1 else None)
+        alone = run_few_tokens(pool, W, S, B, router_x, routed_x, eff, pes)
+        cases.append(dict(M=M, alone=alone, ins=[dev(a) for a in (W, S, B, router_x, eff, pes, routed_x)]))
+
+    def outputs(M):
+        n = M * TOPK
+        return dict(idx=zeros_bytes(n * 4, 0xEE), wts=zeros_bytes(n * 2, 0xEE), acts=zeros_bytes(n * F * 2), partials=zeros_bytes(n * D * 2, 0xEE),
+                    h2=zeros_bytes(M * D * 2, 0xEE))
+
+    def call(c, o, stream):
+        dW, dS, dB, dh, de, dp, dx = c["ins"]
+        k.check(k.lib.tf_prefill_routed_moe_few_tokens(k.handle, stream, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dh.data_ptr(), 0,
+                                                       de.data_ptr(), 0, dp.data_ptr(), 0, o["idx"].data_ptr(), 0, o["wts"].data_ptr(), 0, c["M"], E, D, TOPK,
+                                                       D, dx.data_ptr(), 0, D, pool["dev"].data_ptr(), pool["stride"], C.byref(koff), o["acts"].data_ptr(),
+                                                       o["partials"].data_ptr(), o["h2"].data_ptr(), 0, F, tfk.TF_BF16))
+
+    def check(c, o, what):
+        M, a = c["M"], c["alone"]
+        n = M * TOPK
+        assert np.array_equal(host(o["idx"], np.uint32, n).reshape(M, TOPK), a["idx"]), what
+        assert np.array_equal(host(o["wts"], np.uint16, n).reshape(M, TOPK), a["w_bits"]), what
+        assert np.array_equal(host(o["partials"], np.uint16, n * D).reshape(M, TOPK, D), a["partials"]), what
+        assert np.array_equal(host(o["h2"], np.uint16, M * D).reshape(M, D), a["h2_bits"]), what
+
+    outs = [outputs(c["M"]) for c in cases]
+    for c, o in zip(cases, outs):
+        call(c, o, None)
+    k.synchronize()
+    for i, (c, o) in enumerate(zip(cases, outs)):
+        check(c, o, ("in a row", i))
+    side = torch.cuda.Stream()
+    gouts = [outputs(c["M"]) for c in cases]
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(g, stream=side):
+            for c, o in zip(cases, gouts):
+                call(c, o, side.cuda_stream)
+    for replay in range(3):
+        for o in gouts:
+            for name in ("idx", "wts", "partials", "h2"):
+                o[name].fill_(0xEE)
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        for i, (c, o) in enumerate(zip(cases, gouts)):
+            check(c, o, ("replay", replay, i))
+        o = outputs(cases[replay]["M"])               # an eager call between the replays
+        call(cases[replay], o, None)
+        k.synchronize()
+        check(cases[replay], o, ("eager after replay", replay))
+
+
 def test_few_tokens_in_one_call_refuses_what_it_does_not_serve(pool):
     W, S, B, router_x, routed_x, eff, pes = few_tokens_inputs(33, 0x7F9)
     got = run_few_tokens(pool, W, S, B, router_x, routed_x, eff, pes, expect=tfk.TF_ERR_UNAVAILABLE)
