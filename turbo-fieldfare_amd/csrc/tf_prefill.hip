@@ -269,6 +269,19 @@ __global__ __launch_bounds__(256) void prefill_logits_mfma_kernel(const uint8_t 
 // lane ranking itself among the lanes of the same expert with ballots.  Deterministic: no order depends on timing.
 __device__ __forceinline__ uint32_t clamp_expert(uint32_t e, uint32_t num_experts) { return e < num_experts ? e : num_experts - 1; }
 
+__device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v) {
+    auto shifted = [](uint32_t x, auto ctrl, auto rows) {
+        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, decltype(ctrl)::value, decltype(rows)::value, 0xF, false);
+    };
+    v += shifted(v, std::integral_constant<int, 0x111>{}, std::integral_constant<int, 0xF>{});      // row_shr:1 (no source inside the row of 16: adds 0)
+    v += shifted(v, std::integral_constant<int, 0x112>{}, std::integral_constant<int, 0xF>{});      // row_shr:2
+    v += shifted(v, std::integral_constant<int, 0x114>{}, std::integral_constant<int, 0xF>{});      // row_shr:4
+    v += shifted(v, std::integral_constant<int, 0x118>{}, std::integral_constant<int, 0xF>{});      // row_shr:8
+    v += shifted(v, std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xA>{});      // row_bcast15 into rows 1 and 3
+    v += shifted(v, std::integral_constant<int, 0x143>{}, std::integral_constant<int, 0xC>{});      // row_bcast31 into rows 2 and 3
+    return v;
+}
+
 __global__ __launch_bounds__(64) void group_count_kernel(const uint32_t *indices, uint32_t n_pairs, uint32_t seg_pairs,
                                                          uint32_t num_experts, uint32_t *seg_counts) {
     __shared__ uint32_t cnt[256];
@@ -285,7 +298,7 @@ __global__ __launch_bounds__(64) void group_count_kernel(const uint32_t *indices
 __global__ __launch_bounds__(256) void group_scan_kernel(uint32_t *seg_counts, uint32_t n_segments, uint32_t num_experts,
                                                          uint32_t *per_expert_offsets, uint32_t *per_expert_counts,
                                                          tf_prefill_group *chunks, uint32_t *chunk_count) {
-    __shared__ uint32_t scan_pairs[256], scan_chunks[256];
+    __shared__ uint32_t scan_pairs[4], scan_chunks[4];      // the four waves' totals
     const uint32_t e = threadIdx.x;
     // all of this expert's segment counts are requested at once (one memory round trip), then summed in registers
     uint32_t v[kGroupSegments];
@@ -299,18 +312,20 @@ __global__ __launch_bounds__(256) void group_scan_kernel(uint32_t *seg_counts, u
         total += c;
     }
     const uint32_t nch = (total + kChunkPairs - 1) / kChunkPairs;
-    scan_pairs[e] = total;
-    scan_chunks[e] = nch;
-    __syncthreads();
-    for (uint32_t step = 1; step < 256; step <<= 1) {   // inclusive scans over the experts
-        const uint32_t a = e >= step ? scan_pairs[e - step] : 0u, c = e >= step ? scan_chunks[e - step] : 0u;
-        __syncthreads();
-        scan_pairs[e] += a;
-        scan_chunks[e] += c;
-        __syncthreads();
+    // inclusive scans over the experts: across the lanes of each wave, then the waves before added on
+    uint32_t sum_pairs = wave_inclusive_scan_u32(total), sum_chunks = wave_inclusive_scan_u32(nch);
+    const uint32_t wave = e >> 6;
+    if ((e & 63) == 63) {
+        scan_pairs[wave] = sum_pairs;
+        scan_chunks[wave] = sum_chunks;
     }
-    const uint32_t start = scan_pairs[e] - total, chunk_start = scan_chunks[e] - nch;
-    if (e == 255) chunk_count[0] = scan_chunks[255];
+    __syncthreads();
+    for (uint32_t w = 0; w < wave; ++w) {
+        sum_pairs += scan_pairs[w];
+        sum_chunks += scan_chunks[w];
+    }
+    const uint32_t start = sum_pairs - total, chunk_start = sum_chunks - nch;
+    if (e == 255) chunk_count[0] = sum_chunks;
     if (e < num_experts) {
         per_expert_offsets[e] = total ? start : 0xFFFFFFFFu;
         per_expert_counts[e] = total;
@@ -386,18 +401,6 @@ __global__ __launch_bounds__(64) void group_place_kernel(const uint32_t *indices
 // same expert (the lanes whose expert number agrees in every bit: eight ballots).  Every thread of the block must call (block-wide
 // barriers); the block has at least 256 threads.  indices / weights may live in LDS.
 constexpr uint32_t kGroupBlockPairs = 2048, kGroupBlockSegments = kGroupBlockPairs / 64;
-__device__ __forceinline__ uint32_t wave_inclusive_scan_u32(uint32_t v) {
-    auto shifted = [](uint32_t x, auto ctrl, auto rows) {
-        return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)x, decltype(ctrl)::value, decltype(rows)::value, 0xF, false);
-    };
-    v += shifted(v, std::integral_constant<int, 0x111>{}, std::integral_constant<int, 0xF>{});      // row_shr:1 (no source inside the row of 16: adds 0)
-    v += shifted(v, std::integral_constant<int, 0x112>{}, std::integral_constant<int, 0xF>{});      // row_shr:2
-    v += shifted(v, std::integral_constant<int, 0x114>{}, std::integral_constant<int, 0xF>{});      // row_shr:4
-    v += shifted(v, std::integral_constant<int, 0x118>{}, std::integral_constant<int, 0xF>{});      // row_shr:8
-    v += shifted(v, std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xA>{});      // row_bcast15 into rows 1 and 3
-    v += shifted(v, std::integral_constant<int, 0x143>{}, std::integral_constant<int, 0xC>{});      // row_bcast31 into rows 2 and 3
-    return v;
-}
 struct GroupBlockLds {
     uint32_t seg[kGroupBlockSegments][256];      // [segment][expert]: pair counts, then the position of the segment's first pair of the expert
     uint32_t wave_pairs[4], wave_chunks[4];      // totals of the four waves that own the experts
