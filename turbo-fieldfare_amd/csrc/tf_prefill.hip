@@ -1163,17 +1163,18 @@ __global__ __launch_bounds__(256) void reduce_token_major_kernel(const half_t *p
 constexpr uint32_t kReduceRanksInFlight = 8;
 __global__ __launch_bounds__(256) void reduce_token_major_vec_kernel(const half_t *partials, const half_t *weights, half_t *h2,
                                                                      uint32_t T, uint32_t top_k, uint32_t D) {
-    const uint32_t c = (blockIdx.x * blockDim.x + threadIdx.x) * 8;
-    const uint32_t t = blockIdx.y;
-    if (c >= D || t >= T) return;
+    // threads are numbered through all (token, eight columns) pieces: every block is full whatever D is
+    const uint32_t per_token = D / 8, piece = blockIdx.x * blockDim.x + threadIdx.x;
+    const uint32_t t = piece / per_token, c = (piece - t * per_token) * 8;
+    if (t >= T) return;
     float acc[8] = {};
     for (uint32_t r0 = 0; r0 < top_k; r0 += kReduceRanksInFlight) {
-        uint4 raw[kReduceRanksInFlight];
+        u32x4 raw[kReduceRanksInFlight];
         float w[kReduceRanksInFlight];
 #pragma unroll
         for (uint32_t j = 0; j < kReduceRanksInFlight; ++j) {
             const uint32_t r = min(r0 + j, top_k - 1);
-            raw[j] = *reinterpret_cast<const uint4 *>(partials + ((size_t)t * top_k + r) * D + c);
+            raw[j] = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(partials + ((size_t)t * top_k + r) * D + c));   // read once
             w[j] = (float)weights[t * top_k + r];
         }
 #pragma unroll
@@ -1751,7 +1752,9 @@ int32_t tf_prefill_moe_reduce_token_major(tf_ctx *ctx, tf_stream stream, const v
     const half_t *weights_at = reinterpret_cast<const half_t *>(at(route_weights, route_weights_offset));
     half_t *h2_at = reinterpret_cast<half_t *>(at(h2, h2_offset));
     if (d % 8 == 0 && aligned16(partials_at) && aligned16(h2_at)) {
-        const dim3 grid((d / 8 + 255) / 256, query_count);
+        const uint64_t pieces = (uint64_t)query_count * (d / 8);
+        TF_REQUIRE(ctx, pieces <= 0xFFFFFFFFull - 255, TF_ERR_INVALID_ARGUMENT, "moe_reduce_token_major: queryCount * D / 8 must fit 32 bits");
+        const dim3 grid((uint32_t)((pieces + 255) / 256));
         hipLaunchKernelGGL(reduce_token_major_vec_kernel, grid, dim3(256), 0, static_cast<hipStream_t>(stream), partials_at, weights_at,
                            h2_at, query_count, top_k, d);
     } else {
