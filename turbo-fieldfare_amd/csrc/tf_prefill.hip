@@ -659,13 +659,13 @@ __global__ __launch_bounds__(512) void grouped_phase1_stream_kernel(ExpertTable 
 // A wave's 16 quads take QC consecutive pieces of 16 / QC groups of four rows; pieces of a row are summed across quads at
 // the end of a tile.  A block takes one slice of one chunk's rows; the next tile's loads follow the current tile's use
 // pass by pass, so one tile buffer keeps the memory pipe full.
-constexpr uint32_t kQuadMaxPairs = 8;    // pairs whose activations a block holds in LDS: 2 MFMA pair groups (3 blocks a CU at d = 2816)
+constexpr uint32_t kQuadMaxPairs = 8;    // most pairs whose activations a block holds in LDS: 2 MFMA pair groups (the gate / up kernel's MAXP is 8 or 4)
 constexpr int kQuadMaxD = 3072, kQuadMaxF = 1024;   // widest rows the LDS images are sized for
 // A pair's row in the LDS image is followed by 64 bytes of padding: the four lanes of a quad read the same pieces of four
 // different pairs at once, and rows a multiple of 256 bytes apart would put them on the same banks.
 constexpr int kQuadRowPad = 4;   // in 16-byte pieces
 constexpr size_t quad_row_bytes(int k) { return (size_t)k * 2 + kQuadRowPad * 16; }
-constexpr size_t quad_lds_bytes(int k) { return (size_t)kQuadMaxPairs * (quad_row_bytes(k) + (size_t)(k >> 5) * 4 + 16); }
+constexpr size_t quad_lds_bytes(int k, uint32_t max_pairs = kQuadMaxPairs) { return (size_t)max_pairs * (quad_row_bytes(k) + (size_t)(k >> 5) * 4 + 16); }
 // Behind the image: per wave, the scales and the biases of the tile it is working on (512 bytes each at most: 4 rows of 48
 // groups or 8 rows of 16).  A tile's scales are consecutive bytes of the matrix, so the wave fetches them with ONE load per
 // array (4 or 8 bytes a lane), puts them down here and every pass picks its 16-bit value with an LDS read: two memory
@@ -673,7 +673,7 @@ constexpr size_t quad_lds_bytes(int k) { return (size_t)kQuadMaxPairs * (quad_ro
 // the down kernel ran 16 % faster, the gate / up kernel 7 %).
 constexpr size_t kQuadSBArrayBytes = 512;
 constexpr size_t kQuadSBWaveBytes = 2 * kQuadSBArrayBytes;
-constexpr size_t quad_lds_total(int k) { return (quad_lds_bytes(k) + 15) / 16 * 16 + 4 * kQuadSBWaveBytes; }
+constexpr size_t quad_lds_total(int k, uint32_t max_pairs = kQuadMaxPairs) { return (quad_lds_bytes(k, max_pairs) + 15) / 16 * 16 + 4 * kQuadSBWaveBytes; }
 // The sums of a column's 32 activations sit side by side for the kQuadMaxPairs pairs of the image (xsum[column][pair]): a lane
 // needs the sums of four pairs at once and takes them in one 16-byte read.
 
@@ -816,7 +816,7 @@ __device__ __forceinline__ float quad_sum(float v) {
 
 // activation rows -> LDS image in dot-product order; `row_of(j)` gives the row of batch pair j; all threads call
 template <typename RowOf>
-__device__ __forceinline__ void quad_stage_rows(uint32_t nb, int k, u32x4 *xa, float *xsum, RowOf row_of) {
+__device__ __forceinline__ void quad_stage_rows(uint32_t nb, int k, u32x4 *xa, float *xsum, RowOf row_of, int max_pairs = (int)kQuadMaxPairs) {
     const int nch = k >> 5, pieces = k >> 3, total = (int)nb * pieces;
     for (int q0 = 0; q0 < total; q0 += 1024) {
         u32x4 raw[4];
@@ -833,7 +833,7 @@ __device__ __forceinline__ void quad_stage_rows(uint32_t nb, int k, u32x4 *xa, f
         for (int i = 0; i < 4; ++i) {
             const int q = q0 + 256 * i + (int)threadIdx.x;
             const int j = q < total ? q / pieces : 0, piece = q < total ? q - j * pieces : pieces;   // piece == pieces: nothing is written
-            XStage::publish_piece(raw[i], piece, pieces, nch, xa + (size_t)j * (pieces + kQuadRowPad), xsum + j, (int)kQuadMaxPairs);
+            XStage::publish_piece(raw[i], piece, pieces, nch, xa + (size_t)j * (pieces + kQuadRowPad), xsum + j, max_pairs);
         }
     }
 }
@@ -856,23 +856,27 @@ __device__ __forceinline__ void quad_pass(const ChunkOperands &o, uint16_t s_bit
 #pragma unroll
                 for (int q = 0; q < 4; ++q) xq[4 * dd + q] = as_half2(v[q]);
             }
-            quad_piece<SD>(o, s_bits, b_bits, xq, *reinterpret_cast<const f32x4 *>(xsum + (size_t)colp * kQuadMaxPairs + 4 * g), acc[g]);
+            quad_piece<SD>(o, s_bits, b_bits, xq, *reinterpret_cast<const f32x4 *>(xsum + (size_t)colp * (4 * G) + 4 * g), acc[g]);
         }
     }
 }
 
-template <int NPASS, int SD>
-__global__ __launch_bounds__(256, 2) void grouped_phase1_quad_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl, uint32_t n_chunks_upper,
+// MAXP: pairs in the LDS image, 8 or 4.  With four the kernel needs 143 registers and 30 KB instead of 177 and 57 KB, and three
+// blocks fit a CU instead of two; chunks of more than four pairs then go through in two batches, which pays as long as they
+// are rare (calls of up to 64 pairs: 8 tokens 56.5 -> 55.1 us, 5 tokens 46.6 -> 45.4 us; the same image in the down kernel, five
+// blocks a CU instead of four, changed nothing).
+template <int NPASS, int SD, int MAXP>
+__global__ __launch_bounds__(256, MAXP == 4 ? 3 : 2) void grouped_phase1_quad_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl, uint32_t n_chunks_upper,
                                                                      const tf_prefill_pair *pairs, const half_t *hidden, long hidden_stride,
                                                                      half_t *acts, uint32_t acts_pair_base, int d, int f) {
-    constexpr int QC = 16, G = (int)kQuadMaxPairs / 4;
+    constexpr int QC = 16, G = MAXP / 4;
     typedef QuadMap<QC, NPASS> Map;
-    __shared__ __align__(16) uint8_t quad_lds[quad_lds_total(kQuadMaxD)];
+    __shared__ __align__(16) uint8_t quad_lds[quad_lds_total(kQuadMaxD, MAXP)];
     const int lane = threadIdx.x & 63, wave = uniform_int((int)(threadIdx.x >> 6));
     const int nch = d >> 5, pieces = d >> 3;
     u32x4 *xa = reinterpret_cast<u32x4 *>(quad_lds);
-    float *xsum = reinterpret_cast<float *>(quad_lds + (size_t)kQuadMaxPairs * quad_row_bytes(d));
-    uint8_t *sb_area = quad_lds + (quad_lds_bytes(kQuadMaxD) + 15) / 16 * 16 + (size_t)wave * kQuadSBWaveBytes;
+    float *xsum = reinterpret_cast<float *>(quad_lds + (size_t)MAXP * quad_row_bytes(d));
+    uint8_t *sb_area = quad_lds + (quad_lds_bytes(kQuadMaxD, MAXP) + 15) / 16 * 16 + (size_t)wave * kQuadSBWaveBytes;
     Map qm;
     qm.init(d, lane);
     QuadTileSB<8> tsb;                                    // 4 rows of up to 48 groups: 8 bytes a lane
@@ -907,15 +911,15 @@ __global__ __launch_bounds__(256, 2) void grouped_phase1_quad_kernel(ExpertTable
         quad_request(t[p], qm, p, from, (up ? off.up_W_off : off.gate_W_off) + w_byte);
     };
     // a chunk longer than the LDS image goes through in batches, its weights once a batch
-    for (uint32_t p0 = 0; p0 < ch.pair_count; p0 += kQuadMaxPairs) {
-        const uint32_t nb = min(kQuadMaxPairs, ch.pair_count - p0), first = ch.pair_start + p0;
+    for (uint32_t p0 = 0; p0 < ch.pair_count; p0 += (uint32_t)MAXP) {
+        const uint32_t nb = min((uint32_t)MAXP, ch.pair_count - p0), first = ch.pair_start + p0;
         const int groups_of_pairs = (int)((nb + 3) >> 2);
         int tile = t_lo + wave;
         if (tile < t_hi) {
 #pragma unroll
             for (int p = 0; p < NPASS; ++p) request(blob, false, tile, p);   // the weights do not wait for the activations
         }
-        quad_stage_rows(nb, d, xa, xsum, [&](uint32_t j) { return hidden + (size_t)pairs[first + j].token * hidden_stride; });
+        quad_stage_rows(nb, d, xa, xsum, [&](uint32_t j) { return hidden + (size_t)pairs[first + j].token * hidden_stride; }, MAXP);
         __syncthreads();
         for (; tile < t_hi; tile += 4) {
             float ag[G][4], au[G][4];
@@ -1232,19 +1236,24 @@ int32_t run_grouped(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const t
                          g.f % 4 == 0 && aligned(g.route_partials, 8) && aligned(g.acts, 8) && tab.pool != nullptr;
     const bool quad_pays = !use_mfma || (stream_pairs != 0 && (uint64_t)stream_pairs < (uint64_t)tab.num_experts * 4);
     if (quad_ok && quad_pays) {
-        // as many blocks as the compute units hold at once: two of the gate / up kernel, four of the down kernel
-        const dim3 grid(2u * (uint32_t)ctx->num_cus), grid_down(4u * (uint32_t)ctx->num_cus);
+        // as many blocks as the compute units hold at once: two of the gate / up kernel (three with the 4-pair image, for calls of
+        // up to 64 pairs), four of the down kernel
+        const bool few_pairs = stream_pairs != 0 && stream_pairs <= 64;
+        const dim3 grid((few_pairs ? 3u : 2u) * (uint32_t)ctx->num_cus), grid_down(4u * (uint32_t)ctx->num_cus);
+#define TF_GP1Q_LAUNCH(NP_, SD_, MAXP_)                                                                                   \
+    hipLaunchKernelGGL((grouped_phase1_quad_kernel<NP_, SD_, MAXP_>), grid, dim3(256), 0, st, tab, off, cl, n_chunks_upper, g.pairs, g.hidden, \
+                       g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f)
 #define TF_GP1Q(NP_)                                                                                                       \
     if (p1_passes == NP_) {                                                                                                \
-        if (sd == TF_BF16)                                                                                                 \
-            hipLaunchKernelGGL((grouped_phase1_quad_kernel<NP_, 0>), grid, dim3(256), 0, st, tab, off, cl, n_chunks_upper, g.pairs, g.hidden,        \
-                               g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f);                                       \
-        else                                                                                                               \
-            hipLaunchKernelGGL((grouped_phase1_quad_kernel<NP_, 1>), grid, dim3(256), 0, st, tab, off, cl, n_chunks_upper, g.pairs, g.hidden,        \
-                               g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f);                                       \
+        if (sd == TF_BF16) {                                                                                               \
+            if (few_pairs) TF_GP1Q_LAUNCH(NP_, 0, 4); else TF_GP1Q_LAUNCH(NP_, 0, 8);                                       \
+        } else {                                                                                                           \
+            if (few_pairs) TF_GP1Q_LAUNCH(NP_, 1, 4); else TF_GP1Q_LAUNCH(NP_, 1, 8);                                       \
+        }                                                                                                                  \
     }
         TF_GP1Q(1) TF_GP1Q(2) TF_GP1Q(3) TF_GP1Q(4) TF_GP1Q(5) TF_GP1Q(6)
 #undef TF_GP1Q
+#undef TF_GP1Q_LAUNCH
         rc = check_launch(ctx, "grouped phase 1 quad");
         if (rc != TF_OK) return rc;
 #define TF_GDQ(NP_)                                                                                                        \
