@@ -62,4 +62,21 @@ struct DenseRide {
     int rows;
 };
 
+// Operands of the grouped expert stages, as the launch helpers pass them on.
+struct GroupedGeom {
+    const tf_prefill_pair *pairs;
+    const half_t *hidden;
+    long hidden_stride;
+    half_t *acts;
+    uint32_t acts_pair_base;
+    half_t *route_partials;
+    int d, f, top_k;
+};
+
+// The quad kernels (tf_prefill_quad.hip): grouped gate / up / GeGLU and down for chunks of a few pairs, weights streamed once per
+// expert.  kQuadMaxD / kQuadMaxF: the widest rows they take; the caller checks alignment and shape (run_grouped).
+constexpr int kQuadMaxD = 3072, kQuadMaxF = 1024;
+int32_t launch_grouped_quad(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const tf_expert_offsets &off, const ChunkList &cl,
+                            uint32_t n_chunks_upper, const GroupedGeom &g, tf_dtype sd, uint32_t stream_pairs);
+
 }  // namespace tfk
