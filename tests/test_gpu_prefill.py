@@ -320,8 +320,8 @@ def check_against_oracle(r, T, d, f, top_k, abs_tol, rel_tol=1e-2):
 
 @pytest.mark.parametrize("M", [2, 4, 8, 12, 16, 24])
 def test_small_m_resident_pipeline_matches_oracle(M):
-    # BASELINE config 3: M tokens, top-8 over the production expert shape; below four pairs per expert on average (M = 2, 4,
-    # 8, 12 here) the quad kernels serve the call, from there on the matrix-core tiles
+    # BASELINE config 3: M tokens, top-8 over the production expert shape; below five pairs per expert on average (M = 2, 4,
+    # 8, 12, 16 here) the quad kernels serve the call, from there on the matrix-core tiles
     E, d, f, top_k = 32, 2816, 704, 8
     r = resident_pipeline(M, E, d, f, top_k, 0x300 + M)
     scale = float(np.max(np.abs(tfo.from_f16_bits(r["partials"]))))

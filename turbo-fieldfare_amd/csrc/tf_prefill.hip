@@ -806,14 +806,14 @@ int32_t run_grouped(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab, const t
     const bool p1_fast = blobs16 && hidden16 && off.gate_W_off % 16 == 0 && off.up_W_off % 16 == 0;
     const bool dn_fast = blobs16 && acts16 && off.down_W_off % 16 == 0;
     int32_t rc;
-    // Fewer than four pairs per expert on average: the quad kernels serve the call (chunks longer than their LDS image, if any,
-    // in batches).  From there on so few chunks are short that the matrix-core tile kernels are faster (64 tokens: 193 us
-    // either way; 80 - 128 tokens: 198 - 200 us on the tiles against 224 - 281 us; running both families in one call, each on
-    // its chunks, was never better than the better of the two).
+    // Fewer than five pairs per expert on average: the quad kernels serve the call (chunks longer than their LDS image, if any,
+    // in batches).  From there on so few chunks are short that the matrix-core tile kernels are faster (128 experts: 64 tokens
+    // 151 us on the quad kernels against 164 us on the tiles; 80 tokens 178 against 173 us; 96 tokens 187 against 173 us; running
+    // both families in one call, each on its chunks, was never better than the better of the two).
     const int p1_passes = ((g.d >> 5) + 15) / 16, dn_passes = ((g.f >> 5) + 7) / 8;
     const bool quad_ok = p1_fast && dn_fast && acts16 && g.d <= kQuadMaxD && p1_passes <= 6 && g.f <= kQuadMaxF && dn_passes <= 4 && g.d % 8 == 0 &&
                          g.f % 4 == 0 && aligned(g.route_partials, 8) && aligned(g.acts, 8) && tab.pool != nullptr;
-    const bool quad_pays = !use_mfma || (stream_pairs != 0 && (uint64_t)stream_pairs < (uint64_t)tab.num_experts * 4);
+    const bool quad_pays = !use_mfma || (stream_pairs != 0 && (uint64_t)stream_pairs < (uint64_t)tab.num_experts * 5);
     if (quad_ok && quad_pays) return launch_grouped_quad(ctx, st, tab, off, cl, n_chunks_upper, g, sd, stream_pairs);
     const bool p1_tiles = use_mfma && p1_fast && acts16, dn_tiles = use_mfma && dn_fast && aligned16(g.route_partials);
     if (!(p1_tiles && dn_tiles) || (ride && !dense_ride_ok(*ride))) ride = nullptr;

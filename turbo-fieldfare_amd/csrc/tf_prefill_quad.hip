@@ -228,7 +228,7 @@ __device__ __forceinline__ void quad_pass(const ChunkOperands &o, uint16_t s_bit
 // and a kernel that touches scratch memory dispatches several times slower).  LDS: the image is sized for the rows in use, 52.6 KB at
 // 2816 columns; wider rows (up to kQuadMaxD) leave room for two blocks.
 // MAXP: pairs in the LDS image, 8 or 4.  With four the kernel needs 143 registers and 30 KB; chunks of more than four pairs then
-// go through in two batches, which pays as long as they are rare (calls of up to 64 pairs).
+// go through in two batches, which pays as long as they are rare (calls of up to 96 pairs: 8 / 12 tokens 55.4 / 59.8 -> 54.4 / 58.9 us).
 template <int NPASS, int SD, int MAXP>
 __global__ __launch_bounds__(256, 3) void grouped_phase1_quad_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl, uint32_t n_chunks_upper,
                                                                      const tf_prefill_pair *pairs, const half_t *hidden, long hidden_stride,
@@ -431,8 +431,8 @@ int32_t launch_grouped_quad(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab,
     int32_t rc;
     {
         // as many blocks as the compute units hold at once: three of the gate / up kernel where its LDS image leaves room (rows of up
-        // to 2816 columns; the 4-pair image for calls of up to 64 pairs), four of the down kernel
-        const bool few_pairs = stream_pairs != 0 && stream_pairs <= 64;
+        // to 2816 columns; the 4-pair image for calls of up to 96 pairs), four of the down kernel
+        const bool few_pairs = stream_pairs != 0 && stream_pairs <= 96;
         const size_t lds1 = quad_lds_total(g.d, few_pairs ? 4u : 8u);
         const uint32_t per_cu = (uint32_t)std::min<size_t>(3, std::max<size_t>(1, (size_t)160 * 1024 / (lds1 + 256)));
         const dim3 grid(per_cu * (uint32_t)ctx->num_cus), grid_down(4u * (uint32_t)ctx->num_cus);
