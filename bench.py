@@ -873,7 +873,7 @@ def multi_token_extras(torch, tfk, k, gen, lib, h, stream, layer, offs, stride, 
                          "tokens_per_s": round(M / (us * 1e-6), 1)}
     if small:
         res["small_m"] = {"workload": "configs[3]: M tokens x top-8 over 128 resident experts (router block + grouping + grouped experts + reduce; "
-                                      "us = the faster of the grouped calls, five launches, and the one-call form for up to 32 tokens, three launches)",
+                                      "us = the faster of the grouped calls, five launches, and the one-call form for up to 32 tokens: three launches of its own up to five tokens, the grouped calls made inside beyond)",
                           "per_M": small}
     if small_only:
         return res

@@ -700,20 +700,22 @@ int32_t tf_prefill_router_group_block(tf_ctx *ctx, tf_stream stream,
                                       uint32_t hidden_stride_elements,
                                       void *sorted_pairs, void *per_expert_offsets, void *per_expert_counts,
                                       void *chunks, void *chunk_count);
-/* A few token rows (multi-token verification: up to 32, top_k == 8, at most 128 experts in a resident pool) through the whole
- * routed path as ONE call of three launches: tf_prefill_router_group_block, tf_prefill_grouped_routed_moe_resident and
- * tf_prefill_moe_reduce_token_major (PrefillRouter.encodeGemma4Block, PrefillRouter.swift:37-89; the host grouping,
- * PrefillMoEGrouping.swift:90-193; PrefillGroupedRoutedMoE.encodeStreamedBatched, PrefillGroupedRoutedMoE.swift:386-461;
- * PrefillMoE.encodeReduceTokenMajor, PrefillMoE.swift:11-38; in RealForwardRunner.swift:922-1156 the router reads routerX and
- * the experts routedX, hence the two hidden arguments).  Nothing is sorted: every block of the gate / up launch repeats its
- * token's selection and finds the other tokens that chose its expert by counting, the first such token's blocks read the
+/* A few token rows (multi-token verification: up to 32, top_k == 8, experts in a resident pool) through the whole routed path
+ * as ONE call: tf_prefill_router_group_block, tf_prefill_grouped_routed_moe_resident and tf_prefill_moe_reduce_token_major
+ * (PrefillRouter.encodeGemma4Block, PrefillRouter.swift:37-89; the host grouping, PrefillMoEGrouping.swift:90-193;
+ * PrefillGroupedRoutedMoE.encodeStreamedBatched, PrefillGroupedRoutedMoE.swift:386-461; PrefillMoE.encodeReduceTokenMajor,
+ * PrefillMoE.swift:11-38; in RealForwardRunner.swift:922-1156 the router reads routerX and the experts routedX, hence the two
+ * hidden arguments).  Outputs: out_indices uint32[T, 8], out_weights fp16[T, 8] (the router's), route_partials fp16[T, 8, d]
+ * (unweighted, as the grouped call leaves them), h2 fp16[T, d].  acts_scratch: T * 8 * f halves.
+ * Up to five rows (at most 128 experts, a multiple of 4; d in (1024, 4096]; f <= 1024; 16-byte aligned operands, strides
+ * multiples of 8) take three launches of their own, in which nothing is sorted: every block of the gate / up launch repeats
+ * its token's selection and finds the other tokens that chose its expert by counting, the first such token's blocks read the
  * expert's rows once for all of them; the down launch reads each expert in use once and adds a token's eight partial results
- * in rank order itself.  Outputs: out_indices uint32[T, 8], out_weights fp16[T, 8] (the router's), route_partials fp16[T, 8, d]
- * (unweighted, as the grouped call leaves them), h2 fp16[T, d].  acts_scratch: T * 8 * f halves.  Same arithmetic as the three
- * calls (fp16 activations and partials, fused multiply-adds in rank order); sums inside a dot product are taken in another order,
- * so results agree to rounding, not bit for bit.  Returns TF_ERR_UNAVAILABLE, with nothing enqueued, for shapes it does not
- * serve (more tokens, another top_k, num_experts > 128 or not a multiple of 4, d outside (1024, 4096], f > 1024, operands not
- * 16-byte aligned, strides not multiples of 8): the caller makes the three calls. */
+ * in rank order itself.  Same arithmetic as the three calls (fp16 activations and partials, fused multiply-adds in rank order);
+ * sums inside a dot product are taken in another order, so these rows agree with the three calls to rounding, not bit for bit.
+ * More rows, and shapes the three launches do not take, go through the three calls themselves (from six rows on their
+ * persistent kernels are faster), with the grouping's outputs kept in the context: bit-identical to making the calls.
+ * Returns TF_ERR_UNAVAILABLE, with nothing enqueued, for more than 32 rows or another top_k. */
 int32_t tf_prefill_routed_moe_few_tokens(tf_ctx *ctx, tf_stream stream,
                                          const void *weights, uint64_t weights_offset,
                                          const void *scales, uint64_t scales_offset,

@@ -269,11 +269,13 @@ def pairs_of(idx, w_bits):
     return pairs
 
 
-@pytest.mark.parametrize("M,copy_of", [(1, None), (2, None), (2, {1: 0}), (3, {2: 0}), (4, None), (8, {5: 1, 7: 1}), (16, None), (32, {31: 0})])
+@pytest.mark.parametrize("M,copy_of", [(1, None), (2, None), (2, {1: 0}), (3, {2: 0}), (4, None), (5, {1: 0, 3: 0, 4: 0}), (8, {5: 1, 7: 1}), (16, None),
+                                       (32, {31: 0})])
 def test_few_tokens_in_one_call_of_three_launches(pool, M, copy_of):
     # tf_prefill_routed_moe_few_tokens against the calls it replaces (router block + grouping, grouped experts over the resident
     # pool, token-major reduce) and against the oracle, production shape, 128 experts.  Rows copied from another row choose that
     # row's eight experts: the owner of an expert then serves several tokens (and a first pair several followers in the down launch).
+    # Up to five rows run the three launches of their own; more rows are the three calls made inside (bit-identical to them).
     W, S, B, router_x, routed_x, eff, pes = few_tokens_inputs(M, 0x7E0 + M, copy_of)
     got = run_few_tokens(pool, W, S, B, router_x, routed_x, eff, pes)
     assert not np.any(np.all(got["partials"] == SENTINEL, axis=2))

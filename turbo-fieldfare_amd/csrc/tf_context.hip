@@ -48,6 +48,7 @@ int32_t tf_ctx_create(int32_t device, tf_ctx **out_ctx) {
     ok = ok && hipMalloc(&ctx->head_summaries, summary_bytes) == hipSuccess;
     ok = ok && hipMemset(ctx->head_summaries, 0, summary_bytes) == hipSuccess;
     ok = ok && hipMalloc(&ctx->group_scratch, (size_t)kGroupSegments * 256 * sizeof(uint32_t)) == hipSuccess;
+    ok = ok && hipMalloc(&ctx->few_scratch, kFewScratchBytes) == hipSuccess;
     // the reference's model (Infrastructure/ModelIO/ModelTypes.swift:78-100) at the largest block sizes this library is run at
     const tf_scratch_limits defaults = {262144u, 2048u, 256u, 2112u, 16u, 512u, 128u};
     ok = ok && tf_ctx_reserve(ctx, &defaults) == TF_OK;
@@ -71,6 +72,7 @@ void tf_ctx_destroy(tf_ctx *ctx) {
     if (ctx->head_summaries) (void)hipFree(ctx->head_summaries);
     if (ctx->head_logits) (void)hipFree(ctx->head_logits);
     if (ctx->group_scratch) (void)hipFree(ctx->group_scratch);
+    if (ctx->few_scratch) (void)hipFree(ctx->few_scratch);
     if (ctx->prefill_logits) (void)hipFree(ctx->prefill_logits);
     if (ctx->sample_scratch) (void)hipFree(ctx->sample_scratch);
     if (ctx->shared_block_acts) (void)hipFree(ctx->shared_block_acts);

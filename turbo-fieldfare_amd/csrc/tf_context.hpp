@@ -20,6 +20,7 @@ struct tf_ctx {
     float *head_logits = nullptr;       // fp32 logits of the unaligned lm_head path, limits.max_vocab of them
     size_t head_logits_count = 0;
     uint32_t *group_scratch = nullptr;  // kGroupSegments x 256 per-segment expert counts of the device pair grouping
+    uint8_t *few_scratch = nullptr;     // kFewScratchBytes: sorted pairs, per-expert tables and work list of tf_prefill_routed_moe_few_tokens
     float *prefill_logits = nullptr;    // [tokens, experts] router logits (+ partial planes) of the multi-token router
     size_t prefill_logits_count = 0;
     void *sample_scratch = nullptr;     // argmax cells, softmax partials, top-k pair buffers of the samplers
@@ -42,6 +43,10 @@ namespace tfk {
 constexpr uint32_t kMaxHeadD = 16384;
 constexpr uint32_t kMaxHeadWaves = 16384;
 constexpr uint32_t kGroupSegments = 64;   // token segments the device pair grouping counts and places independently
+// what tf_prefill_routed_moe_few_tokens keeps between its launches when it runs the grouped kernels: up to 256 sorted pairs
+// (16 bytes each), per-expert offsets and counts (256 x 4 bytes each), a work list of up to 264 chunks (12 bytes each), its length
+constexpr uint32_t kFewScratchPairs = 256, kFewScratchChunks = 264;
+constexpr size_t kFewScratchBytes = (size_t)kFewScratchPairs * 16 + 2 * 256 * 4 + (size_t)kFewScratchChunks * 12 + 16;
 
 inline int32_t fail(tf_ctx *ctx, int32_t status, const char *fmt, ...) {
     if (ctx) {

@@ -26,6 +26,7 @@ constexpr uint32_t kFewMaxTokens = 32;      // 256 pairs: four lanes' worth of p
 constexpr uint32_t kFewMaxExperts = 128;
 constexpr uint32_t kFewTopK = 8;
 constexpr uint32_t kNoSlot = 0xFFu;
+constexpr uint32_t kFewCrossoverTokens = 5;      // up to here the three launches of this file, beyond the grouped path's five
 
 // ------------------------------------------------------------------------------------------------ router logits
 // One 256-thread block per (expert, token): a row is one memory round trip and a sixteenth of a wave's arithmetic.
@@ -457,7 +458,26 @@ extern "C" int32_t tf_prefill_routed_moe_few_tokens(tf_ctx *ctx, tf_stream strea
         ok = best_np > 0;
         for (uint32_t c = 0; ok && c < 64u * (uint32_t)best_np; ++c) ok = ((c * inv_nch) >> 16) == c / nch;
     }
-    if (!ok) return TF_ERR_UNAVAILABLE;
+    // From six token rows on the grouped path's persistent kernels are faster (every block here pays for its own selection): the
+    // call then makes the three calls it stands for itself, with the grouping's outputs in the context's scratch.
+    if (!ok || query_count > kFewCrossoverTokens) {
+        if (query_count > kFewMaxTokens || top_k != kFewTopK || query_count * top_k > kFewScratchPairs ||
+            num_experts + query_count * top_k / 64 + 1 > kFewScratchChunks)
+            return TF_ERR_UNAVAILABLE;
+        uint8_t *scratch = ctx->few_scratch;
+        void *sorted_pairs = scratch, *offsets = scratch + (size_t)kFewScratchPairs * 16, *counts = scratch + (size_t)kFewScratchPairs * 16 + 1024;
+        void *chunks = scratch + (size_t)kFewScratchPairs * 16 + 2048, *chunk_count = scratch + (size_t)kFewScratchPairs * 16 + 2048 + (size_t)kFewScratchChunks * 12;
+        int32_t rc = tf_prefill_router_group_block(ctx, stream, weights, weights_offset, scales, scales_offset, biases, biases_offset, hidden, hidden_offset,
+                                                   effective_scale, effective_scale_offset, per_expert_scale, per_expert_scale_offset, out_indices,
+                                                   out_indices_offset, out_weights, out_weights_offset, query_count, num_experts, d, top_k,
+                                                   hidden_stride_elements, sorted_pairs, offsets, counts, chunks, chunk_count);
+        if (rc != TF_OK) return rc;
+        rc = tf_prefill_grouped_routed_moe_resident(ctx, stream, routed_hidden, routed_hidden_offset, routed_hidden_stride_elements, sorted_pairs, chunks,
+                                                    chunk_count, kFewScratchChunks, query_count * top_k, expert_pool, expert_pool_stride, num_experts,
+                                                    routed_offsets, acts_scratch, route_partials, d, f, top_k, scale_dtype);
+        if (rc != TF_OK) return rc;
+        return tf_prefill_moe_reduce_token_major(ctx, stream, route_partials, 0, out_weights, out_weights_offset, h2, h2_offset, query_count, top_k, d);
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
     float *logits = ctx->prefill_logits;
     hipLaunchKernelGGL(few_logits_kernel<0>, dim3(num_experts, query_count), dim3(256), 0, st, w, s, b, h, hidden_stride_elements, eff, logits,
