@@ -332,9 +332,10 @@ __global__ __launch_bounds__(256, 3) void grouped_phase1_quad_kernel(ExpertTable
     }
 }
 
-// down rows for such chunks: rows of 22 pieces (f = 704): eight quads along the row, two groups of four rows a wave.
+// down rows for such chunks: rows of 22 pieces (f = 704): eight quads along the row, two groups of four rows a wave.  95 registers
+// and 22 KB: five blocks a CU (48 / 64 tokens 116.6 / 150.6 -> 114.4 / 148.6 us against four).
 template <int NPASS, int SD>
-__global__ __launch_bounds__(256, 4) void grouped_down_quad_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl, uint32_t n_chunks_upper,
+__global__ __launch_bounds__(256, 5) void grouped_down_quad_kernel(ExpertTable tab, tf_expert_offsets off, ChunkList cl, uint32_t n_chunks_upper,
                                                                    const tf_prefill_pair *pairs, const half_t *acts, uint32_t acts_pair_base,
                                                                    half_t *route_partials, int d, int f, int top_k) {
     constexpr int QC = 8, G = (int)kQuadMaxPairs / 4;
@@ -402,7 +403,7 @@ __global__ __launch_bounds__(256, 4) void grouped_down_quad_kernel(ExpertTable t
                 request(next, tile + 4, p);
                 quad_pass<QC, NPASS, SD, G>(ow, ws, wb, qm.col(p), qm, xa, xsum, nch, pieces, nb, groups_of_pairs, acc);
             }
-            const long row0 = (long)tile * Map::kRows + qm.rg * 4 + qm.m;   // this lane's row
+            const uint32_t row0 = (uint32_t)tile * Map::kRows + (uint32_t)(qm.rg * 4 + qm.m);   // this lane's row
 #pragma unroll
             for (int g = 0; g < G; ++g) {
                 if (g < groups_of_pairs) {
@@ -431,11 +432,11 @@ int32_t launch_grouped_quad(tf_ctx *ctx, hipStream_t st, const ExpertTable &tab,
     int32_t rc;
     {
         // as many blocks as the compute units hold at once: three of the gate / up kernel where its LDS image leaves room (rows of up
-        // to 2816 columns; the 4-pair image for calls of up to 96 pairs), four of the down kernel
+        // to 2816 columns; the 4-pair image for calls of up to 96 pairs), five of the down kernel
         const bool few_pairs = stream_pairs != 0 && stream_pairs <= 96;
         const size_t lds1 = quad_lds_total(g.d, few_pairs ? 4u : 8u);
         const uint32_t per_cu = (uint32_t)std::min<size_t>(3, std::max<size_t>(1, (size_t)160 * 1024 / (lds1 + 256)));
-        const dim3 grid(per_cu * (uint32_t)ctx->num_cus), grid_down(4u * (uint32_t)ctx->num_cus);
+        const dim3 grid(per_cu * (uint32_t)ctx->num_cus), grid_down(5u * (uint32_t)ctx->num_cus);
 #define TF_GP1Q_LAUNCH(NP_, SD_, MAXP_)                                                                                   \
     hipLaunchKernelGGL((grouped_phase1_quad_kernel<NP_, SD_, MAXP_>), grid, dim3(256), lds1, st, tab, off, cl, n_chunks_upper, g.pairs, g.hidden, \
                        g.hidden_stride, g.acts, g.acts_pair_base, g.d, g.f)
