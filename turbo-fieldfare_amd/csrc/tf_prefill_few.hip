@@ -1,9 +1,10 @@
 // A few token rows (multi-token verification) through the router and the routed experts in THREE launches: router logits;
 // gate / up / GeGLU with the selection repeated inside every block; down projection with the token-major reduce inside the
 // block.  The grouped path spends five launches on the same work (logits, selection + grouping, gate / up, down, reduce), and at
-// two to four tokens the launches' boundaries and their first memory round trips are most of the call: 21.6 / 28.1 / 33.7 us for
-// 2 / 3 / 4 tokens of the production shape against 33.0 / 35.2 / 40.7 us.  From about six tokens on the grouped path's
-// persistent kernels win (every block here pays for its own selection, and the arithmetic per pair is the same).
+// two to four tokens the launches' boundaries and their first memory round trips are most of the call: 21.3 / 28.1 / 35.0 us for
+// 2 / 3 / 4 tokens of the production shape against 30.8 / 35.2 / 40.1 us.  From six tokens on the grouped path's persistent
+// kernels win (every block here pays for its own selection, and the arithmetic per pair is the same), so the entry point at the
+// end of this file gives batches of more than five rows to the grouped calls and the kernels here hold at most eight rows.
 //
 // Experts are still read once however many tokens chose them:
 //   * gate / up: the grid has one set of blocks per (token, rank) pair.  Every block ranks its own token's logits (by counting, as
@@ -22,11 +23,13 @@ using namespace tfk;
 
 namespace {
 
-constexpr uint32_t kFewMaxTokens = 32;      // 256 pairs: four lanes' worth of pair masks, 16 KiB of logits in LDS
+constexpr uint32_t kFewMaxTokens = 8;       // the kernels' capacity: 64 pairs (one lane each of a wave), 4 KiB of logits in LDS
+constexpr uint32_t kFewEntryMaxTokens = 32; // what the entry point takes (beyond kFewCrossoverTokens through the grouped calls)
 constexpr uint32_t kFewMaxExperts = 128;
 constexpr uint32_t kFewTopK = 8;
 constexpr uint32_t kNoSlot = 0xFFu;
 constexpr uint32_t kFewCrossoverTokens = 5;      // up to here the three launches of this file, beyond the grouped path's five
+static_assert(kFewCrossoverTokens <= kFewMaxTokens, "the kernels hold every batch they are given");
 
 // ------------------------------------------------------------------------------------------------ router logits
 // One 256-thread block per (expert, token): a row is one memory round trip and a sixteenth of a wave's arithmetic.
@@ -71,13 +74,8 @@ __global__ __launch_bounds__(256, NP <= 3 ? 4 : 3) void few_phase1_kernel(const 
     // requests first: the token's logits for the ranking, every token's logits, the token's activations
     const float my_logit = rank_select_load(my_row, num_experts);
     const uint32_t n4 = tokens * num_experts / 4;
-    f32x4 lg[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t i = threadIdx.x + 256u * j;
-        lg[j] = f32x4{-INFINITY, -INFINITY, -INFINITY, -INFINITY};
-        if (i < n4) lg[j] = reinterpret_cast<const f32x4 *>(logits)[i];
-    }
+    f32x4 lg = {-INFINITY, -INFINITY, -INFINITY, -INFINITY};      // at most 8 x 128 logits: one 16-byte piece a thread
+    if (threadIdx.x < n4) lg = reinterpret_cast<const f32x4 *>(logits)[threadIdx.x];
     XStage stage;
     stage.request(hidden + (size_t)t * hidden_stride, (int)d);
     RowStream<RT, NP> rs;
@@ -98,15 +96,10 @@ __global__ __launch_bounds__(256, NP <= 3 ? 4 : 3) void few_phase1_kernel(const 
             }
         }
     }
+    if (threadIdx.x < n4) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const uint32_t i = threadIdx.x + 256u * j;
-        if (i < n4) {
-            f32x4 v = lg[j];
-#pragma unroll
-            for (int c = 0; c < 4; ++c) v[c] = (v[c] != v[c]) ? -INFINITY : v[c];
-            reinterpret_cast<f32x4 *>(all_logits)[i] = v;
-        }
+        for (int c = 0; c < 4; ++c) lg[c] = (lg[c] != lg[c]) ? -INFINITY : lg[c];
+        reinterpret_cast<f32x4 *>(all_logits)[threadIdx.x] = lg;
     }
     stage.publish((int)d, xa, xsum);            // ends with a block barrier: chosen and all_logits are visible after it
     const uint32_t e = uniform_u32(chosen[s]);
@@ -213,7 +206,7 @@ __global__ __launch_bounds__(64 * kFewDownWaves) void few_down_kernel(const uint
     __shared__ half_t part[kFewMaxTokens * kFewTopK][kFewDownMaxRows];    // the partial results of the block's rows
     __shared__ uint32_t s_idx[kFewMaxTokens * kFewTopK];
     __shared__ half_t s_w[kFewMaxTokens * kFewTopK];
-    __shared__ uint32_t first[kFewMaxExperts], uniq[kFewMaxExperts], wave_count[4];
+    __shared__ uint32_t first[kFewMaxExperts], uniq[kFewMaxTokens * kFewTopK], n_uniq_lds;
 
     const int lane = threadIdx.x & 63;
     const uint32_t wave = uniform_u32(threadIdx.x >> 6);
@@ -234,17 +227,14 @@ __global__ __launch_bounds__(64 * kFewDownWaves) void few_down_kernel(const uint
     __syncthreads();
     if (threadIdx.x < pairs) atomicMin(&first[my_e], threadIdx.x);
     __syncthreads();
-    const bool leads = threadIdx.x < pairs && first[my_e] == threadIdx.x;
-    const uint64_t lead_mask = __ballot(leads);
-    if (wave < 4 && lane == 0) wave_count[wave] = (uint32_t)__builtin_popcountll(lead_mask);
-    __syncthreads();
-    if (leads) {
-        uint32_t pos = (uint32_t)__builtin_popcountll(lead_mask & ((1ull << lane) - 1ull));
-        for (uint32_t w = 0; w < wave; ++w) pos += wave_count[w];
-        uniq[pos] = threadIdx.x;
+    if (wave == 0) {      // the pairs are the first wave's lanes
+        const bool leads = (uint32_t)lane < pairs && first[my_e] == (uint32_t)lane;
+        const uint64_t lead_mask = __ballot(leads);
+        if (leads) uniq[__builtin_popcountll(lead_mask & ((1ull << lane) - 1ull))] = (uint32_t)lane;
+        if (lane == 0) n_uniq_lds = (uint32_t)__builtin_popcountll(lead_mask);
     }
     __syncthreads();
-    const uint32_t n_uniq = wave_count[0] + wave_count[1] + wave_count[2] + wave_count[3];
+    const uint32_t n_uniq = n_uniq_lds;
 
     // this lane's chunk positions: the same for every expert
     uint32_t sboff[NP];
@@ -257,32 +247,19 @@ __global__ __launch_bounds__(64 * kFewDownWaves) void few_down_kernel(const uint
         col[p] = (int)cc;
         sboff[p] = (r * (uint32_t)groups + (cc >> 1)) * 2u;   // past the block's rows: past the descriptor, reads zero
     }
-    // the pairs that chose expert e, as four 64-bit masks over the pair numbers
+    // the pairs that chose expert e, as a 64-bit mask over the pair numbers
     struct Pairs {
-        uint64_t m[4];
-        __device__ __forceinline__ bool any() const { return (m[0] | m[1] | m[2] | m[3]) != 0ull; }
+        uint64_t m;
+        __device__ __forceinline__ bool any() const { return m != 0ull; }
         __device__ __forceinline__ uint32_t pop() {      // the lowest pair, removed; call only if any()
-            int sel_j = 3;
-            uint64_t v = m[3];
-#pragma unroll
-            for (int j = 2; j >= 0; --j)
-                if (m[j] != 0ull) {
-                    sel_j = j;
-                    v = m[j];
-                }
-#pragma unroll
-            for (int j = 0; j < 4; ++j)
-                if (sel_j == j) m[j] = v & (v - 1ull);
-            return 64u * (uint32_t)sel_j + (uint32_t)__builtin_ctzll(v);
+            const uint32_t q = (uint32_t)__builtin_ctzll(m);
+            m &= m - 1ull;
+            return q;
         }
     };
     auto pairs_of = [&](uint32_t e) {
         Pairs ps;
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t i = (uint32_t)lane + 64u * j;
-            ps.m[j] = __ballot(i < pairs && s_idx[i < pairs ? i : 0] == e);
-        }
+        ps.m = __ballot((uint32_t)lane < pairs && s_idx[(uint32_t)lane < pairs ? lane : 0] == e);
         return ps;
     };
     auto request_acts = [&](u32x4 (&xr)[2], uint32_t q) {
@@ -432,7 +409,7 @@ extern "C" int32_t tf_prefill_routed_moe_few_tokens(tf_ctx *ctx, tf_stream strea
     const uint32_t nch = f / 32;
     const bool plan_ok = (plan.rt == 1 && (plan.np == 1 || plan.np == 2)) || (plan.rt == 2 && plan.np >= 2 && plan.np <= 4) ||
                          (plan.rt == 4 && (plan.np == 3 || plan.np == 4));
-    bool ok = plan_ok && query_count <= kFewMaxTokens && top_k == kFewTopK && num_experts <= kFewMaxExperts && num_experts % 4 == 0 && d > 1024 && d <= 4096 &&
+    bool ok = plan_ok && query_count <= kFewCrossoverTokens && top_k == kFewTopK && num_experts <= kFewMaxExperts && num_experts % 4 == 0 && d > 1024 && d <= 4096 &&
               plan.rt > 0 && f <= 1024 && aligned16(w) && aligned16(h) && aligned16(eff) && hidden_stride_elements % 8 == 0 && aligned16(x) &&
               routed_hidden_stride_elements % 8 == 0 && aligned16(pool) &&
               expert_pool_stride % 16 == 0 && offsets_fit(*routed_offsets) && aligned16(acts_scratch) &&
@@ -460,8 +437,8 @@ extern "C" int32_t tf_prefill_routed_moe_few_tokens(tf_ctx *ctx, tf_stream strea
     }
     // From six token rows on the grouped path's persistent kernels are faster (every block here pays for its own selection): the
     // call then makes the three calls it stands for itself, with the grouping's outputs in the context's scratch.
-    if (!ok || query_count > kFewCrossoverTokens) {
-        if (query_count > kFewMaxTokens || top_k != kFewTopK || query_count * top_k > kFewScratchPairs ||
+    if (!ok) {
+        if (query_count > kFewEntryMaxTokens || top_k != kFewTopK || query_count * top_k > kFewScratchPairs ||
             num_experts + query_count * top_k / 64 + 1 > kFewScratchChunks)
             return TF_ERR_UNAVAILABLE;
         uint8_t *scratch = ctx->few_scratch;
