@@ -193,6 +193,42 @@ def test_router_block_and_grouping_in_one_call_equal_the_two_calls(T, E, d, top_
     assert all(np.all(host(bad[name], np.uint8) == 0xEE) for name in bad)
 
 
+def test_router_block_and_grouping_in_one_call_with_equal_logits():
+    # Three router rows are byte-for-byte the same: a token that picks one of them has three equal scores among its best eight.
+    # Ties go to the lower index in both forms of the call, and the one-launch form equals the two calls bit for bit.
+    T, E, d, top_k = 16, 128, 2816, 8
+    rng = np.random.default_rng(0x71E5)
+    W, S, B = refcases.synthetic_int8(E, d, 0x71E)
+    W, S, B = W.copy(), S.copy(), B.copy()
+    for dup in (40, 77):
+        W[dup], S[dup], B[dup] = W[3], S[3], B[3]
+    hidden = np.concatenate([refcases.normal_f16(d, 0x7100 + r) for r in range(T)])
+    eff = tfo.bf16_bits_array(rng.uniform(0.5, 1.5, d).astype(np.float32) / np.float32(np.sqrt(d)))
+    pes = tfo.bf16_bits_array(rng.uniform(0.6, 1.4, E).astype(np.float32))
+    k = ctx()
+    dW, dS, dB, dh, de, dp = dev(W), dev(S), dev(B), dev(hidden), dev(eff), dev(pes)
+    n = T * top_k
+    cap = E + n // 64 + 1
+    outs = [dict(idx=zeros_bytes(n * 4, 0xEE), wts=zeros_bytes(n * 2, 0xEE), sp=zeros_bytes(n * 16, 0xEE), offs=zeros_bytes(E * 4, 0xEE),
+                 cnts=zeros_bytes(E * 4, 0xEE), chunks=zeros_bytes(cap * 12, 0xEE), nch=zeros_bytes(4, 0xEE)) for _ in range(2)]
+    two, one = outs
+    router = (k.handle, None, dW.data_ptr(), 0, dS.data_ptr(), 0, dB.data_ptr(), 0, dh.data_ptr(), 0, de.data_ptr(), 0, dp.data_ptr(), 0)
+    k.check(k.lib.tf_prefill_router_gemma4_block(*router, two["idx"].data_ptr(), 0, two["wts"].data_ptr(), 0, T, E, d, top_k, d))
+    k.check(k.lib.tf_prefill_group_pairs_device(k.handle, None, two["idx"].data_ptr(), two["wts"].data_ptr(), T, top_k, E, two["sp"].data_ptr(),
+                                                two["offs"].data_ptr(), two["cnts"].data_ptr(), two["chunks"].data_ptr(), two["nch"].data_ptr()))
+    k.check(k.lib.tf_prefill_router_group_block(*router, one["idx"].data_ptr(), 0, one["wts"].data_ptr(), 0, T, E, d, top_k, d, one["sp"].data_ptr(),
+                                                one["offs"].data_ptr(), one["cnts"].data_ptr(), one["chunks"].data_ptr(), one["nch"].data_ptr()))
+    idx = host(two["idx"], np.uint32, n).reshape(T, top_k)
+    tied = [t_ for t_ in range(T) if {3, 40, 77} <= set(idx[t_].tolist())]
+    assert len(tied) >= 1, "no token picked the three equal rows: the case tests nothing"
+    for t_ in tied:      # ties go to the lower index, in this order
+        pos = [list(idx[t_]).index(e) for e in (3, 40, 77)]
+        assert pos == sorted(pos) and pos[2] - pos[0] == 2
+    nch = int(host(two["nch"], np.uint32, 1)[0])
+    for name, count in (("idx", n * 4), ("wts", n * 2), ("sp", n * 16), ("offs", E * 4), ("cnts", E * 4), ("chunks", nch * 12)):
+        assert np.array_equal(host(one[name], np.uint8, count), host(two[name], np.uint8, count)), name
+
+
 def test_streamed_batched_matches_reference_across_partial_microbatch():
     # PrefillGroupedRoutedMoETests+Execution.swift:8-103
     d = f = 64
