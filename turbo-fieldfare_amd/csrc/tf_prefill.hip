@@ -946,16 +946,21 @@ int32_t tf_prefill_router_gemma4_block(tf_ctx *ctx, tf_stream stream, const void
     hipStream_t st = static_cast<hipStream_t>(stream);
     const bool mfma_ok = fast && num_experts <= 128 && d <= 4096 && aligned16(w) && d % 64 == 0;
     if (query_count <= kFewTokens || mfma_ok) {
-        // many tokens: enough blocks to fill the chip, by cutting the reduction dimension into up to four runs of groups
+        // many tokens: enough blocks to fill the chip, by cutting the reduction dimension into up to sixteen runs of groups
         // whose partial logits the selection kernel adds up in a fixed order
         const uint32_t token_blocks = (query_count + 31) / 32;
         const uint32_t groups = d / 64;
+        const size_t plane = (size_t)query_count * num_experts;
         uint32_t splits = 1;
         if (query_count > kFewTokens) {
-            while (splits < 4 && token_blocks * splits < (uint32_t)ctx->num_cus && groups / (splits * 2) >= 8) splits *= 2;
+            // a block's time is a fixed part plus its run of groups (12.5 us for 11 groups at 128 tokens): runs of at least three
+            // groups, as many as the scratch holds planes for (it is sized for four at the largest call), every run non-empty
+            while (splits < 16 && token_blocks * splits < (uint32_t)ctx->num_cus && groups / (splits * 2) >= 3) splits *= 2;
+            while (splits > 1 && plane * (1 + splits) > ctx->prefill_logits_count) splits /= 2;
+            const uint32_t run = (groups + splits - 1) / splits;
+            splits = (groups + run - 1) / run;
         }
         const uint32_t planes = splits > 1 ? splits : 0;   // partial planes behind the logits
-        const size_t plane = (size_t)query_count * num_experts;
         const size_t need = std::max<size_t>((size_t)kFewTokens * 256, plane * (1 + planes));
         if (ctx->prefill_logits_count < need)
             return scratch_too_small(ctx, "prefill_router", need * sizeof(float), ctx->prefill_logits_count * sizeof(float));
